@@ -1,0 +1,232 @@
+/*
+ * lightseq_hip.h -- C ABI of the MI355X (gfx950) int8 transformer-layer forward path.
+ *
+ * Every entry point replaces one launcher / helper of the reference
+ * (bytedance/lightseq v3.0.1; paths below are relative to lightseq/inference/
+ * unless noted).  Argument names, order and meaning follow the reference
+ * launcher, with three systematic changes:
+ *   - the template parameter T in {float, __half} becomes a _f32 / _f16 suffix and
+ *     T-typed pointers become void*;
+ *   - cudaStream_t becomes lsh_stream_t (a hipStream_t);
+ *   - every function returns an int status (LSH_OK == 0) instead of void, and a
+ *     description of the last failure on the calling thread is available from
+ *     lsh_last_error().  Where the reference throws (bad sampling k, hidden % 8,
+ *     batch > max_batch ...) the status is LSH_ERR_INVALID with the same message.
+ * The cuBLASLt-specific COL32 layouts do not exist here: a call with an
+ * in_col32 / out_col32 flag set returns LSH_ERR_UNSUPPORTED.
+ *
+ * All pointers are device pointers unless a parameter is documented as host.
+ * Launchers are asynchronous on `stream`, allocate nothing and never synchronise.
+ */
+#ifndef LIGHTSEQ_HIP_H_
+#define LIGHTSEQ_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* lsh_stream_t;
+
+enum {
+  LSH_OK = 0,
+  LSH_ERR_INVALID = 1,     /* violated precondition (the reference throws or misbehaves) */
+  LSH_ERR_UNSUPPORTED = 2, /* valid in the reference, not provided here (COL32 layouts ...) */
+  LSH_ERR_HIP = 3,         /* a HIP runtime call failed */
+  LSH_ERR_IO = 4           /* model file could not be read / parsed */
+};
+
+/* Message of the last non-OK status returned on this thread ("" if none). */
+const char* lsh_last_error(void);
+/* Library version string and the gfx architecture the kernels were built for. */
+const char* lsh_version(void);
+
+/* ---- quantise / dequantise --------------------------------------------------- */
+/* kernels/transformerKernels_int8.h:11-14 */
+int lsh_launch_quantize_tensor_f16(const void* input, int8_t* output, int batch_tokens,
+                                   int hidden_size, float quant_scale, lsh_stream_t stream,
+                                   int out_col32);
+int lsh_launch_quantize_tensor_f32(const void* input, int8_t* output, int batch_tokens,
+                                   int hidden_size, float quant_scale, lsh_stream_t stream,
+                                   int out_col32);
+/* kernels/transformerKernels_int8.h:16-19 */
+int lsh_launch_dequantize_tensor_f16(const int32_t* input, void* output, int batch_tokens,
+                                     int hidden_size, float dequant_scale, lsh_stream_t stream,
+                                     int in_col32);
+int lsh_launch_dequantize_tensor_f32(const int32_t* input, void* output, int batch_tokens,
+                                     int hidden_size, float dequant_scale, lsh_stream_t stream,
+                                     int in_col32);
+
+/* ---- LayerNorm family ---------------------------------------------------------- */
+/* kernels/transformerKernels_int8.h:21-26 */
+int lsh_ker_norm_layer_resual_i8O_f16(int token_num, int hidden_size, lsh_stream_t stream,
+                                      void* input, int8_t* output, const void* scale,
+                                      const void* bias, const void* residual_bias,
+                                      int max_thread_per_block, float quant_scale, int is_post_ln,
+                                      int out_col32);
+int lsh_ker_norm_layer_resual_i8O_f32(int token_num, int hidden_size, lsh_stream_t stream,
+                                      void* input, int8_t* output, const void* scale,
+                                      const void* bias, const void* residual_bias,
+                                      int max_thread_per_block, float quant_scale, int is_post_ln,
+                                      int out_col32);
+/* kernels/transformerKernels_int8.h:47-53 */
+int lsh_ker_residual_bias_ln_i32I_i8O_f16(const int32_t* input, const void* scale,
+                                          const void* bias, const void* residual_bias,
+                                          int8_t* output, void* residual, int batch_tokens,
+                                          int hidden_size, float dequant_scale, float quant_scale,
+                                          int max_thread_per_block, lsh_stream_t stream,
+                                          int is_post_ln, int in_col32, int out_col32,
+                                          const void* colsum);
+int lsh_ker_residual_bias_ln_i32I_i8O_f32(const int32_t* input, const void* scale,
+                                          const void* bias, const void* residual_bias,
+                                          int8_t* output, void* residual, int batch_tokens,
+                                          int hidden_size, float dequant_scale, float quant_scale,
+                                          int max_thread_per_block, lsh_stream_t stream,
+                                          int is_post_ln, int in_col32, int out_col32,
+                                          const void* colsum);
+/* kernels/transformerKernels_int8.h:55-61 */
+int lsh_ker_residual_bias_ln_i8I_i8O_f16(const int8_t* input, const void* scale, const void* bias,
+                                         const void* residual_bias, int8_t* output, void* residual,
+                                         int batch_tokens, int hidden_size, float dequant_scale,
+                                         float quant_scale, int max_thread_per_block,
+                                         lsh_stream_t stream, int is_post_ln, int in_col32,
+                                         int out_col32, const void* colsum);
+int lsh_ker_residual_bias_ln_i8I_i8O_f32(const int8_t* input, const void* scale, const void* bias,
+                                         const void* residual_bias, int8_t* output, void* residual,
+                                         int batch_tokens, int hidden_size, float dequant_scale,
+                                         float quant_scale, int max_thread_per_block,
+                                         lsh_stream_t stream, int is_post_ln, int in_col32,
+                                         int out_col32, const void* colsum);
+/* kernels/transformerKernels_int8.h:63-68 (output may alias residual) */
+int lsh_ker_residual_bias_ln_i32I_f16(const int32_t* input, const void* scale, const void* bias,
+                                      const void* residual, void* output, int batch_tokens,
+                                      int hidden_size, float dequant_scale,
+                                      int max_thread_per_block, lsh_stream_t stream, int in_col32,
+                                      const void* colsum);
+int lsh_ker_residual_bias_ln_i32I_f32(const int32_t* input, const void* scale, const void* bias,
+                                      const void* residual, void* output, int batch_tokens,
+                                      int hidden_size, float dequant_scale,
+                                      int max_thread_per_block, lsh_stream_t stream, int in_col32,
+                                      const void* colsum);
+
+/* ---- bias + activation + requant ------------------------------------------------ */
+/* kernels/transformerKernels_int8.h:29-35 */
+int lsh_ker_bias_gelu_i8I_i8O_f16(int batch_token_num, lsh_stream_t stream, const int8_t* input,
+                                  int8_t* output, const void* bias, int feature_dim,
+                                  float dequant_scale, float quant_scale, int in_col32,
+                                  int out_col32);
+int lsh_ker_bias_gelu_i8I_i8O_f32(int batch_token_num, lsh_stream_t stream, const int8_t* input,
+                                  int8_t* output, const void* bias, int feature_dim,
+                                  float dequant_scale, float quant_scale, int in_col32,
+                                  int out_col32);
+/* kernels/transformerKernels_int8.h:38-45 */
+int lsh_ker_bias_relu_i8I_i8O_f16(int batch_token_num, lsh_stream_t stream, const int8_t* input,
+                                  int8_t* output, const void* bias, int feature_dim,
+                                  float dequant_scale, float quant_scale, float clip_max,
+                                  int in_col32, int out_col32, int narrow_clip);
+int lsh_ker_bias_relu_i8I_i8O_f32(int batch_token_num, lsh_stream_t stream, const int8_t* input,
+                                  int8_t* output, const void* bias, int feature_dim,
+                                  float dequant_scale, float quant_scale, float clip_max,
+                                  int in_col32, int out_col32, int narrow_clip);
+
+/* ---- head split / merge ----------------------------------------------------------- */
+/* kernels/transformerKernels_int8.h:70-75 */
+int lsh_ker_arrange_encself_qkv_i8I_f16(int batch_token_num, int hidden_size, lsh_stream_t stream,
+                                        const int8_t* ori_qkv, const void* qkv_bias, void* new_qkv,
+                                        int max_batch_dim, int batch_seq_len, int dim_per_head,
+                                        int head_num, int max_thread_per_block,
+                                        float dequant_scale, int in_col32);
+int lsh_ker_arrange_encself_qkv_i8I_f32(int batch_token_num, int hidden_size, lsh_stream_t stream,
+                                        const int8_t* ori_qkv, const void* qkv_bias, void* new_qkv,
+                                        int max_batch_dim, int batch_seq_len, int dim_per_head,
+                                        int head_num, int max_thread_per_block,
+                                        float dequant_scale, int in_col32);
+/* kernels/transformerKernels_int8.h:77-83 */
+int lsh_ker_arrange_encself_qkv_i8I_i8O_f16(int batch_token_num, int hidden_size,
+                                            lsh_stream_t stream, const int8_t* ori_qkv,
+                                            const void* qkv_bias, int8_t* new_q, int8_t* new_k,
+                                            int8_t* new_v, void* d_v, int batch_seq_len,
+                                            int dim_per_head, int head_num,
+                                            int max_thread_per_block, float dequant_scale,
+                                            float quant_scale, int in_col32);
+int lsh_ker_arrange_encself_qkv_i8I_i8O_f32(int batch_token_num, int hidden_size,
+                                            lsh_stream_t stream, const int8_t* ori_qkv,
+                                            const void* qkv_bias, int8_t* new_q, int8_t* new_k,
+                                            int8_t* new_v, void* d_v, int batch_seq_len,
+                                            int dim_per_head, int head_num,
+                                            int max_thread_per_block, float dequant_scale,
+                                            float quant_scale, int in_col32);
+/* kernels/transformerKernels_int8.h:85-89 */
+int lsh_ker_arrange_atten_output_i8O_f16(int batch_token_num, int hidden_size, lsh_stream_t stream,
+                                         const void* ori_q, int8_t* new_q, int beam_size,
+                                         int dim_per_head, int head_num, int max_thread_per_block,
+                                         float quant_scale, int out_col32);
+int lsh_ker_arrange_atten_output_i8O_f32(int batch_token_num, int hidden_size, lsh_stream_t stream,
+                                         const void* ori_q, int8_t* new_q, int beam_size,
+                                         int dim_per_head, int head_num, int max_thread_per_block,
+                                         float quant_scale, int out_col32);
+
+/* ---- encoder attention core --------------------------------------------------------- */
+/* kernels/transformerKernels.h (ker_correlation_softmax_encself_launcher),
+ * kernels/transformerKernels.cc.cu:1119-1172 */
+int lsh_ker_correlation_softmax_encself_f16(int batch_size, int batch_seq_len, int head_num,
+                                            lsh_stream_t stream, void* correlation,
+                                            const int* src_padding_mask);
+int lsh_ker_correlation_softmax_encself_f32(int batch_size, int batch_seq_len, int head_num,
+                                            lsh_stream_t stream, void* correlation,
+                                            const int* src_padding_mask);
+/* Fused replacement of the sequence at model/quant_bert_encoder.cc.cu:321-347
+ * (cublasGemmStridedBatchedEx K^T Q, ker_correlation_softmax_encself,
+ * cublasGemmStridedBatchedEx V P, ker_arrange_atten_output_i8O).  q, k, v are
+ * [batch, head_num, seq_len, dim_per_head] fp16.  ctx ([batch, head_num, seq_len,
+ * dim_per_head] fp16) and ctx_q ([batch*seq_len, head_num*dim_per_head] int8,
+ * quantised with quant_scale) are each optional (NULL), not both. */
+int lsh_encself_attention_f16(const void* q, const void* k, const void* v,
+                              const int* src_padding_mask, void* ctx, int8_t* ctx_q,
+                              float quant_scale, int batch_size, int batch_seq_len, int head_num,
+                              int dim_per_head, lsh_stream_t stream);
+
+/* ---- embedding ------------------------------------------------------------------------ */
+/* kernels/embKernels_int8.h:7-13 */
+int lsh_launch_enc_emb_i8I_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,
+                               void* output, int* pad_mask, int pad_id, int batch_size,
+                               int seq_len, int hidden_dim, lsh_stream_t stream,
+                               const void* lang_emb, const int* lang_id, int multilg_type,
+                               float dequant_scale, int scaled);
+int lsh_launch_enc_emb_i8I_f32(const int8_t* token_emb, const void* pos_emb, const int* tokens,
+                               void* output, int* pad_mask, int pad_id, int batch_size,
+                               int seq_len, int hidden_dim, lsh_stream_t stream,
+                               const void* lang_emb, const int* lang_id, int multilg_type,
+                               float dequant_scale, int scaled);
+/* kernels/transformerKernels.h:15-17 */
+int lsh_launch_scaled_colsum_f16(const void* inp, void* out, int rows, int cols, float scale,
+                                 lsh_stream_t stream);
+int lsh_launch_scaled_colsum_f32(const void* inp, void* out, int rows, int cols, float scale,
+                                 lsh_stream_t stream);
+
+/* ---- int8 GEMM (replaces cuBLASLt + the tuned-algorithm map) ---------------------------- */
+/* C[m,n] = A[m,k] * W[n,k]^T with A (activations) and W (weights) K-contiguous.
+ * model/cublas_helper.h:21-34 cublasLtMM_withAlgo (int32 out) and
+ * model/cublas_helper.h:50-58 cublaslt_gemm<int32_t,int32_t>. */
+int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n, int k,
+                     lsh_stream_t stream);
+/* int8 out: C = clamp(floor(float(acc) * alpha + 0.5), -127, 127).
+ * model/cublas_helper.h:36-48 cublasLtMM_withAlgo_i8IO and
+ * model/cublas_helper.h:50-58 cublaslt_gemm<int8_t,float>. */
+int lsh_gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int m, int n, int k, float alpha,
+                    lsh_stream_t stream);
+/* model/cublas_helper.h:60 quantize_weight: `origin_weight` is a HOST pointer to a
+ * row-major [rows, cols] T matrix; it is uploaded, quantised with quant_scale and
+ * stored at device pointer quantized_weight as [rows, cols] (layout 0, kRowMajor)
+ * or transposed [cols, rows] (layout 1, kColMajor: the K-contiguous form the GEMMs
+ * take).  Layout 2 (kColMajor32) is unsupported.  Synchronises `stream`. */
+int lsh_quantize_weight_f16(const void* origin_weight, int8_t* quantized_weight, int rows,
+                            int cols, float quant_scale, lsh_stream_t stream, int layout);
+int lsh_quantize_weight_f32(const void* origin_weight, int8_t* quantized_weight, int rows,
+                            int cols, float quant_scale, lsh_stream_t stream, int layout);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LIGHTSEQ_HIP_H_ */

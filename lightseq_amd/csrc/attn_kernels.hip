@@ -1,0 +1,286 @@
+// Encoder self-attention core for the int8 layer path (fp16 attention, as in the
+// reference): a stand-alone masked softmax with the reference's launcher
+// signature, and a fused QK^T -> mask -> softmax -> PV kernel on fp16 MFMA that
+// keeps the reference's rounding points (scores and probabilities are rounded to
+// fp16 exactly where the reference stores them) without materialising the
+// [B,h,S,S] score tensor in HBM.
+//
+// Replaces inference/model/quant_bert_encoder.cc.cu:321-347 (two cuBLAS strided
+// batched GEMMs + ker_correlation_softmax_encself + ker_arrange_atten_output_i8O)
+// and inference/kernels/transformerKernels.cc.cu:1119-1172.
+#include "ls_device.cuh"
+#include "ls_launch.h"
+
+namespace lsh {
+
+// ---------------------------------------------------------------------------------
+// masked softmax over the last dim of [B, h, S, S]; one wavefront per row.
+template <typename T, int ITER>
+__global__ void __launch_bounds__(256)
+softmax_encself_kernel(T* corr, const int* __restrict__ pad_mask, long rows, int seq_len,
+                       int head_num) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int b = (int)(row / ((long)head_num * seq_len));
+  const int qpos = (int)(row % seq_len);
+  const int* mask = pad_mask + (long)b * seq_len;
+  T* p = corr + row * seq_len;
+  if (mask[qpos]) {  // padded query: the whole row is zeroed
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+      int j = it * 64 + lane;
+      if (j < seq_len) TT<T>::st(p, j, 0.f);
+    }
+    return;
+  }
+  float val[ITER];
+  bool dead[ITER];
+  float mx = kFloatInfNeg;
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    int j = it * 64 + lane;
+    dead[it] = j >= seq_len || mask[j] != 0;
+    val[it] = j < seq_len ? TT<T>::ld(p, j) : kFloatInfNeg;
+    mx = fmaxf(mx, dead[it] ? kFloatInfNeg : val[it]);
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    val[it] = dead[it] ? 0.f : __expf(val[it] - mx);
+    sum += val[it];
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    int j = it * 64 + lane;
+    if (j < seq_len) TT<T>::st(p, j, val[it] / sum);
+  }
+}
+
+template <typename T>
+int correlation_softmax_encself(int batch_size, int batch_seq_len, int head_num, hipStream_t s,
+                                T* correlation, const int* src_padding_mask) {
+  if (batch_size <= 0 || batch_seq_len <= 0 || head_num <= 0 || !correlation ||
+      !src_padding_mask)
+    return lsh_fail(LSH_ERR_INVALID, "ker_correlation_softmax_encself: bad arguments");
+  if (batch_seq_len > 1024)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "ker_correlation_softmax_encself: seq_len > 1024");
+  const long rows = (long)batch_size * head_num * batch_seq_len;
+  const int grid = (int)((rows + 3) / 4);
+#define LSH_SM_CASE(IT)                                               \
+  softmax_encself_kernel<T, IT><<<grid, 256, 0, s>>>(correlation, src_padding_mask, rows, \
+                                                     batch_seq_len, head_num)
+  const int iters = (batch_seq_len + 63) / 64;
+  if (iters <= 1) LSH_SM_CASE(1);
+  else if (iters <= 2) LSH_SM_CASE(2);
+  else if (iters <= 4) LSH_SM_CASE(4);
+  else if (iters <= 8) LSH_SM_CASE(8);
+  else LSH_SM_CASE(16);
+#undef LSH_SM_CASE
+  return lsh_check_launch("softmax_encself_kernel");
+}
+
+template int correlation_softmax_encself<float>(int, int, int, hipStream_t, float*, const int*);
+template int correlation_softmax_encself<__half>(int, int, int, hipStream_t, __half*, const int*);
+
+// ---------------------------------------------------------------------------------
+// Fused encoder attention.
+//
+// Grid (ceil(S/64), B*h), 128 threads = 2 wavefronts, 32 queries per wavefront.
+// Keys are processed in blocks of 128: K block row-major and V block transposed
+// are staged in LDS.  Scores are computed transposed (S^T = K Q^T) with
+// v_mfma_f32_32x32x16_f16 so that one lane owns one query: the row max / sum need
+// a single cross-lane exchange, and the probability registers feed the P V MFMA
+// directly as its B operand (the MFMA contraction slots are mapped onto the keys a
+// lane already holds).  Two passes over the key blocks (max+sum, then P V); with a
+// single key block (S <= 128) the scores stay in registers between the passes.
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float round_h(float x) { return (float)(_Float16)x; }
+
+template <int D>
+__global__ void __launch_bounds__(128)
+encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
+                    const __half* __restrict__ v, const int* __restrict__ pad_mask,
+                    __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale, int S,
+                    int head_num, float alpha) {
+  constexpr int KSTR = D + 8;    // halfs per K row in LDS (pad kills bank conflicts)
+  constexpr int VSTR = 128 + 4;  // halfs per V^T row in LDS
+  constexpr int CH = D / 8;      // 16-byte chunks per row
+  __shared__ _Float16 Ks[128 * KSTR];
+  __shared__ _Float16 Vt[D * VSTR];
+  __shared__ int msk[128];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int bh = blockIdx.y;
+  const int b = bh / head_num, head = bh % head_num;
+  const int qi = blockIdx.x * 64 + wave * 32 + l32;
+  const _Float16* qb = reinterpret_cast<const _Float16*>(q) + (long)bh * S * D;
+  const _Float16* kbase = reinterpret_cast<const _Float16*>(k) + (long)bh * S * D;
+  const _Float16* vbase = reinterpret_cast<const _Float16*>(v) + (long)bh * S * D;
+
+  v8h qreg[D / 16];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) {
+    if (qi < S)
+      qreg[ks] = *reinterpret_cast<const v8h*>(qb + (long)qi * D + ks * 16 + g * 8);
+    else
+      qreg[ks] = (v8h)(_Float16)0;
+  }
+  const bool q_pad = qi >= S || pad_mask[(long)b * S + qi] != 0;
+
+  float m = kFloatInfNeg, sum = 0.f;
+  v16f sc[4];
+  v16f acc[D / 32];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+
+  const int nkb = (S + 127) / 128;
+  for (int phase = 0; phase < 2; ++phase) {
+    for (int kb = 0; kb < nkb; ++kb) {
+      const int key0 = kb * 128;
+      const bool fresh = !(nkb == 1 && phase == 1);
+      if (fresh) {
+        __syncthreads();
+        const bool want_v = phase == 1 || nkb == 1;
+        for (int c = tid; c < 128 * CH; c += 128) {
+          const int row = c / CH, ch = c % CH;
+          const int key = key0 + row;
+          v8h kv = (v8h)(_Float16)0, vv = (v8h)(_Float16)0;
+          if (key < S) {
+            kv = *reinterpret_cast<const v8h*>(kbase + (long)key * D + ch * 8);
+            if (want_v) vv = *reinterpret_cast<const v8h*>(vbase + (long)key * D + ch * 8);
+          }
+          *reinterpret_cast<v8h*>(&Ks[row * KSTR + ch * 8]) = kv;
+          if (want_v) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) Vt[(ch * 8 + i) * VSTR + row] = vv[i];
+          }
+        }
+        msk[tid] = (key0 + tid < S) ? pad_mask[(long)b * S + key0 + tid] : 1;
+        __syncthreads();
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb) {
+          v16f c;
+#pragma unroll
+          for (int i = 0; i < 16; ++i) c[i] = 0.f;
+#pragma unroll
+          for (int ks = 0; ks < D / 16; ++ks) {
+            v8h a = *reinterpret_cast<const v8h*>(&Ks[(sb * 32 + l32) * KSTR + ks * 16 + g * 8]);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[ks], c, 0, 0, 0);
+          }
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key_local = sb * 32 + 8 * (i / 4) + 4 * g + (i % 4);
+            sc[sb][i] = msk[key_local] ? kFloatInfNeg : round_h(alpha * c[i]);
+          }
+        }
+      }
+      if (phase == 0) {
+        float bm = kFloatInfNeg;
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) bm = fmaxf(bm, sc[sb][i]);
+        bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+        const float m_new = fmaxf(m, bm);
+        float part = 0.f;
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i)
+            part += sc[sb][i] == kFloatInfNeg ? 0.f : __expf(sc[sb][i] - m_new);
+        part += __shfl_xor(part, 32, 64);
+        sum = sum * __expf(m - m_new) + part;
+        m = m_new;
+      } else {
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) {
+            v8h pb;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float s = sc[sb][8 * t + j];
+              pb[j] = (_Float16)(s == kFloatInfNeg ? 0.f : __expf(s - m) / sum);
+            }
+#pragma unroll
+            for (int db = 0; db < D / 32; ++db) {
+              const _Float16* vrow = &Vt[(db * 32 + l32) * VSTR + sb * 32 + 16 * t + 4 * g];
+              v4h lo = *reinterpret_cast<const v4h*>(vrow);
+              v4h hi = *reinterpret_cast<const v4h*>(vrow + 8);
+              v8h a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+              acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, acc[db], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+  }
+
+  if (qi >= S) return;
+  const long tok = (long)b * S + qi;
+  const int hidden = head_num * D;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db) {
+#pragma unroll
+    for (int vg = 0; vg < 4; ++vg) {
+      const int dd = db * 32 + 8 * vg + 4 * g;
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = q_pad ? 0.f : round_h(acc[db][4 * vg + j]);
+      if (ctx != nullptr) {
+        half4_t t;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t.v[j] = __float2half_rn(o[j]);
+        *reinterpret_cast<half4_t*>(ctx + ((long)bh * S + qi) * D + dd) = t;
+      }
+      if (ctx_q != nullptr) {
+        *reinterpret_cast<uint32_t*>(ctx_q + tok * hidden + head * D + dd) =
+            pack4_i8(float2int8(o[0], quant_scale), float2int8(o[1], quant_scale),
+                     float2int8(o[2], quant_scale), float2int8(o[3], quant_scale));
+      }
+    }
+  }
+}
+
+int encself_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,
+                          __half* ctx, int8_t* ctx_q, float quant_scale, int batch, int seq_len,
+                          int head_num, int dim_per_head, hipStream_t s) {
+  if (batch <= 0 || seq_len <= 0 || head_num <= 0 || !q || !k || !v || !pad_mask ||
+      (!ctx && !ctx_q))
+    return lsh_fail(LSH_ERR_INVALID, "encself_attention: bad arguments");
+  if (seq_len > 1024) return lsh_fail(LSH_ERR_UNSUPPORTED, "encself_attention: seq_len > 1024");
+  if (((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
+        reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(ctx) |
+        reinterpret_cast<uintptr_t>(ctx_q)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_INVALID, "encself_attention: pointers must be 16-byte aligned");
+  const float alpha = __half2float(__float2half_rn(sqrtf(1.f / (float)dim_per_head)));
+  dim3 grid((seq_len + 63) / 64, batch * head_num);
+  switch (dim_per_head) {
+    case 32:
+      encself_attn_kernel<32><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q, quant_scale,
+                                                   seq_len, head_num, alpha);
+      break;
+    case 64:
+      encself_attn_kernel<64><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q, quant_scale,
+                                                   seq_len, head_num, alpha);
+      break;
+    case 128:
+      encself_attn_kernel<128><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q, quant_scale,
+                                                    seq_len, head_num, alpha);
+      break;
+    default:
+      return lsh_fail(LSH_ERR_UNSUPPORTED, "encself_attention: dim_per_head must be 32, 64 or 128");
+  }
+  return lsh_check_launch("encself_attn_kernel");
+}
+
+}  // namespace lsh

@@ -1,0 +1,138 @@
+// Device-side helpers shared by every gfx950 kernel of the int8 layer path.
+// Wavefronts are 64 lanes wide; all reductions below are written for that.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace lsh {
+
+constexpr int kWave = 64;
+constexpr float kLnEpsilon = 1e-12f;      // inference/kernels/transformerKernels.h:13
+constexpr float kFloatInfNeg = -1.0e8f;   // inference/kernels/common.h:12
+
+// ---- storage-type traits ---------------------------------------------------
+template <typename T>
+struct TT;
+template <>
+struct TT<float> {
+  static constexpr bool is_half = false;
+  __device__ static float ld(const float* p, long i) { return p[i]; }
+  __device__ static void st(float* p, long i, float v) { p[i] = v; }
+  // value as it would read back after a store
+  __device__ static float rnd(float v) { return v; }
+  // kernels/common.h:217-227 clamps half loads only
+  __device__ static float safe(float v) { return v; }
+};
+template <>
+struct TT<__half> {
+  static constexpr bool is_half = true;
+  __device__ static float ld(const __half* p, long i) { return __half2float(p[i]); }
+  __device__ static void st(__half* p, long i, float v) { p[i] = __float2half_rn(v); }
+  __device__ static float rnd(float v) { return __half2float(__float2half_rn(v)); }
+  __device__ static float safe(float v) { return fmaxf(fminf(100000.f, v), -100000.f); }
+};
+
+// ---- scalar quantisers: inference/kernels/transformerKernels_int8.cc.cu:14-27
+// (no FMA contraction in the three quantisers: the product is rounded before the
+// +0.5, as written, so results do not depend on the compiler's fusing choices)
+__device__ __forceinline__ int float2int8(float x, float quant_scale) {
+#pragma clang fp contract(off)
+  float i8_f = x * quant_scale;
+  int i8 = (int)floorf(i8_f + 0.5f);
+  return max(-127, min(127, i8));
+}
+__device__ __forceinline__ int posfloat2int8(float x, float quant_scale, float clip_max) {
+#pragma clang fp contract(off)
+  float i8_f = x * 2 * quant_scale - quant_scale * clip_max;
+  int i8 = (int)floorf(i8_f + 0.5f);
+  return max(-127, min(127, i8));
+}
+// int32 accumulator -> int8 code: the requantising GEMM epilogue.
+__device__ __forceinline__ int requant_acc(int acc, float alpha) {
+#pragma clang fp contract(off)
+  float f = (float)acc * alpha;
+  int q = (int)floorf(f + 0.5f);
+  return max(-127, min(127, q));
+}
+// inference/kernels/common.h:17-23
+__device__ __forceinline__ float gelu_tanh(float x) {
+  float cdf = 0.5f * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+  return x * cdf;
+}
+
+__device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
+  return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
+         ((uint32_t)(d & 0xff) << 24);
+}
+__device__ __forceinline__ int unpack_i8(uint32_t w, int i) {
+  return (int)(int8_t)((w >> (8 * i)) & 0xff);
+}
+
+// ---- vector views ------------------------------------------------------------
+struct __align__(8) half4_t {
+  __half v[4];
+};
+struct __align__(16) half8_t {
+  __half v[8];
+};
+
+// load/store 4 consecutive T as floats
+__device__ __forceinline__ void ld4(const float* p, long i, float (&o)[4]) {
+  float4 t = *reinterpret_cast<const float4*>(p + i);
+  o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+}
+__device__ __forceinline__ void ld4(const __half* p, long i, float (&o)[4]) {
+  half4_t t = *reinterpret_cast<const half4_t*>(p + i);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) o[k] = __half2float(t.v[k]);
+}
+__device__ __forceinline__ void st4(float* p, long i, const float (&o)[4]) {
+  *reinterpret_cast<float4*>(p + i) = make_float4(o[0], o[1], o[2], o[3]);
+}
+__device__ __forceinline__ void st4(__half* p, long i, const float (&o)[4]) {
+  half4_t t;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) t.v[k] = __float2half_rn(o[k]);
+  *reinterpret_cast<half4_t*>(p + i) = t;
+}
+
+// ---- wavefront reductions ------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = kWave / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = kWave / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
+  return v;
+}
+
+// Block-wide reductions for blocks of up to 1024 threads (16 wavefronts).
+// `red` must point to at least 16 floats of LDS.  All threads get the result.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x >> 6;
+  const int nw = (blockDim.x + kWave - 1) >> 6;
+  __syncthreads();  // protect `red` from a previous use
+  if (lane == 0) red[wid] = v;
+  __syncthreads();
+  float r = 0.f;
+  for (int i = 0; i < nw; ++i) r += red[i];
+  return r;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x >> 6;
+  const int nw = (blockDim.x + kWave - 1) >> 6;
+  __syncthreads();
+  if (lane == 0) red[wid] = v;
+  __syncthreads();
+  float r = red[0];
+  for (int i = 1; i < nw; ++i) r = fmaxf(r, red[i]);
+  return r;
+}
+
+}  // namespace lsh

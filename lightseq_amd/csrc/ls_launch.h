@@ -1,0 +1,96 @@
+// Host-side internal interface between the kernel translation units and the
+// C ABI (capi.cpp).  Every function returns an LSH_* status and records a message
+// retrievable through lsh_last_error().
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/lightseq_hip.h"
+
+namespace lsh {
+
+// Records `msg` as the calling thread's last error and returns `code`.
+int lsh_fail(int code, const char* msg);
+// hipGetLastError() after a launch -> status.
+int lsh_check_launch(const char* what);
+int lsh_check_hip(hipError_t e, const char* what);
+
+// ---- quantise / dequantise (quant_kernels.hip) -------------------------------
+template <typename T>
+int quantize_tensor(const T* input, int8_t* output, long n, float quant_scale, hipStream_t s);
+template <typename T>
+int dequantize_tensor(const int32_t* input, T* output, long n, float dequant_scale,
+                      hipStream_t s);
+// rows x cols T (row-major) -> int8 codes, optionally transposed to cols x rows
+template <typename T>
+int quantize_transpose(const T* input, int8_t* output, int rows, int cols, float quant_scale,
+                       bool transpose, hipStream_t s);
+template <typename T>
+int scaled_colsum(const T* inp, T* out, int rows, int cols, float scale, hipStream_t s);
+
+// ---- bias + activation + requant (act_kernels.hip) -----------------------------
+template <typename T>
+int bias_gelu_i8I_i8O(int tokens, hipStream_t s, const int8_t* input, int8_t* output,
+                      const T* bias, int feature_dim, float dequant_scale, float quant_scale);
+template <typename T>
+int bias_relu_i8I_i8O(int tokens, hipStream_t s, const int8_t* input, int8_t* output,
+                      const T* bias, int feature_dim, float dequant_scale, float quant_scale,
+                      float clip_max, bool narrow_clip);
+
+// ---- LayerNorm family (ln_kernels.hip) ------------------------------------------
+template <typename T>
+int norm_layer_resual_i8O(int token_num, int hidden_size, hipStream_t stream, T* input,
+                          int8_t* output, const T* scale, const T* bias, const T* residual_bias,
+                          float quant_scale, bool is_post_ln);
+template <typename T, typename AccT>
+int residual_bias_ln_i8O(const AccT* input, const T* scale, const T* bias, const T* residual_bias,
+                         int8_t* output, T* residual, int batch_tokens, int hidden_size,
+                         float dequant_scale, float quant_scale, hipStream_t stream,
+                         bool is_post_ln, const T* colsum);
+template <typename T>
+int residual_bias_ln_i32I(const int32_t* input, const T* scale, const T* bias, const T* residual,
+                          T* output, int batch_tokens, int hidden_size, float dequant_scale,
+                          hipStream_t stream, const T* colsum);
+
+// ---- head split / merge, embedding (arrange_kernels.hip) -------------------------
+template <typename T>
+int arrange_encself_qkv_i8I(int batch_token_num, int hidden_size, hipStream_t s,
+                            const int8_t* ori_qkv, const T* qkv_bias, T* new_qkv,
+                            long max_batch_dim, int batch_seq_len, int dim_per_head, int head_num,
+                            float dequant_scale);
+template <typename T>
+int arrange_encself_qkv_i8I_i8O(int batch_token_num, int hidden_size, hipStream_t s,
+                                const int8_t* ori_qkv, const T* qkv_bias, int8_t* new_q,
+                                int8_t* new_k, int8_t* new_v, T* d_v, int batch_seq_len,
+                                int dim_per_head, int head_num, float dequant_scale,
+                                float quant_scale);
+template <typename T>
+int arrange_atten_output_i8O(int batch_token_num, int hidden_size, hipStream_t s, const T* ori_q,
+                             int8_t* new_q, int beam_size, int dim_per_head, int head_num,
+                             float quant_scale);
+template <typename T>
+int enc_emb_i8I(const int8_t* token_emb, const T* pos_emb, const int* tokens, T* output,
+                int* pad_mask, int pad_id, int batch_size, int seq_len, int hidden_dim,
+                hipStream_t s, float dequant_scale, bool scaled);
+
+// ---- encoder attention (attn_kernels.hip) ------------------------------------------
+template <typename T>
+int correlation_softmax_encself(int batch_size, int batch_seq_len, int head_num, hipStream_t s,
+                                T* correlation, const int* src_padding_mask);
+// Fused (1/sqrt(d)) Q K^T -> mask -> softmax -> P V for the encoder, with the
+// reference's rounding points (scores and probabilities rounded to fp16).
+// ctx ([B,h,S,d] fp16) and ctx_q ([B*S, h*d] int8) are both optional.
+int encself_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,
+                          __half* ctx, int8_t* ctx_q, float quant_scale, int batch, int seq_len,
+                          int head_num, int dim_per_head, hipStream_t s);
+
+// ---- int8 MFMA GEMM (gemm_i8.hip) -----------------------------------------------------
+// C[M,N] = A[M,K] * W[N,K]^T, both operands K-contiguous.
+int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int K,
+                 hipStream_t s);
+int gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K, float alpha,
+                hipStream_t s);
+
+}  // namespace lsh

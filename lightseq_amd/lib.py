@@ -1,0 +1,114 @@
+"""ctypes binding of ``liblightseq_hip.so``.
+
+``import torch`` happens first on purpose: PyTorch-ROCm ships its own HIP runtime
+(SONAME ``libamdhip64.so.7``) and the library must resolve its HIP symbols against
+that already-loaded copy so that device pointers and streams are shared.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (must be loaded before the library, see module docstring)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "liblightseq_hip.so")
+
+LSH_OK, LSH_ERR_INVALID, LSH_ERR_UNSUPPORTED, LSH_ERR_HIP, LSH_ERR_IO = range(5)
+
+
+class LSHError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+    def __init__(self, code, message, func):
+        super().__init__("%s failed (status %d): %s" % (func, code, message))
+        self.code = code
+        self.func = func
+
+
+_P, _I, _F, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
+_CODES = {"p": _P, "s": _P, "i": _I, "f": _F, "l": _L}
+
+# name -> (has _f16/_f32 variants, argument codes).  p pointer, s stream, i int, f float
+_SIGNATURES = {
+    "lsh_launch_quantize_tensor": (True, "ppiifsi"),
+    "lsh_launch_dequantize_tensor": (True, "ppiifsi"),
+    "lsh_ker_norm_layer_resual_i8O": (True, "iispppppifii"),
+    "lsh_ker_residual_bias_ln_i32I_i8O": (True, "ppppppiiffisiiip"),
+    "lsh_ker_residual_bias_ln_i8I_i8O": (True, "ppppppiiffisiiip"),
+    "lsh_ker_residual_bias_ln_i32I": (True, "pppppiifisip"),
+    "lsh_ker_bias_gelu_i8I_i8O": (True, "isppp" + "iffii"),
+    "lsh_ker_bias_relu_i8I_i8O": (True, "isppp" + "ifffiii"),
+    "lsh_ker_arrange_encself_qkv_i8I": (True, "iisppp" + "iiiiifi"),
+    "lsh_ker_arrange_encself_qkv_i8I_i8O": (True, "iispppppp" + "iiiiffi"),
+    "lsh_ker_arrange_atten_output_i8O": (True, "iispp" + "iiiifi"),
+    "lsh_ker_correlation_softmax_encself": (True, "iiispp"),
+    "lsh_encself_attention_f16": (False, "pppppp" + "fiiiis"),
+    "lsh_launch_enc_emb_i8I": (True, "ppppp" + "iiiispp" + "ifi"),
+    "lsh_launch_scaled_colsum": (True, "ppiifs"),
+    "lsh_gemm_i8_i32o": (False, "pppiiis"),
+    "lsh_gemm_i8_i8o": (False, "pppiiifs"),
+    "lsh_quantize_weight": (True, "ppiifsi"),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "%s is missing: build it with `python -m lightseq_amd.build` "
+            "(there is no CPU fallback)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.lsh_last_error.restype = ctypes.c_char_p
+    lib.lsh_last_error.argtypes = []
+    lib.lsh_version.restype = ctypes.c_char_p
+    lib.lsh_version.argtypes = []
+    for name, (typed, codes) in _SIGNATURES.items():
+        for suffix in (("_f16", "_f32") if typed else ("",)):
+            fn = getattr(lib, name + suffix)
+            fn.restype = ctypes.c_int
+            fn.argtypes = [_CODES[c] for c in codes]
+    _lib = lib
+    return lib
+
+
+def bind(name, codes, restype=ctypes.c_int):
+    """Declare one more entry point (used by modules that add their own)."""
+    fn = getattr(load(), name)
+    fn.restype = restype
+    fn.argtypes = [_CODES[c] for c in codes]
+    return fn
+
+
+def last_error():
+    return load().lsh_last_error().decode()
+
+
+def version():
+    return load().lsh_version().decode()
+
+
+def ptr(x):
+    """Device pointer of a torch tensor (None -> NULL); ints pass through."""
+    if x is None:
+        return None
+    if isinstance(x, torch.Tensor):
+        if not x.is_contiguous():
+            raise ValueError("tensor must be contiguous")
+        return x.data_ptr()
+    return int(x)
+
+
+def current_stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def call(name, *args):
+    """Call ``name`` and raise :class:`LSHError` on a non-zero status."""
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise LSHError(rc, lib.lsh_last_error().decode(), name)
