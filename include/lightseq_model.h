@@ -1,0 +1,83 @@
+/*
+ * lightseq_model.h -- C ABI of the model entry points (one MI355X, one stream).
+ *
+ * Replaces the C++ interface lightseq::cuda::LSModel / LSModelFactory of the
+ * reference (lightseq/inference/pywrapper/model_base.h:59-148), which is what its
+ * pybind module (pywrapper/wrapper.cc), C++ examples and Triton backend bind.
+ * Every LSModel method has one function here with the same meaning; C++ exceptions
+ * become a non-zero status and the message is available from lsh_last_error()
+ * (include/lightseq_hip.h).  Device buffers for inputs and outputs are owned by the
+ * caller (the model also owns a default set, used until a pointer is set), exactly
+ * as in the reference; ls_model_infer() is synchronous.
+ *
+ * Model classes: "QuantBert" (quant_bert.proto file; input 0 "token_ids" int32
+ * [batch, seq_len]; output 0 "encoder_output" fp16 [batch, seq_len, hidden]),
+ * pywrapper/quant_bert.cc:6-149.
+ */
+#ifndef LIGHTSEQ_MODEL_H_
+#define LIGHTSEQ_MODEL_H_
+
+#include "lightseq_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ls_model ls_model;
+
+/* values of lightseq::cuda::DataType, model_base.h:12-26 */
+enum {
+  LS_DTYPE_NOT_SUPPORTED = 0, LS_DTYPE_FLOAT32 = 1, LS_DTYPE_INT32 = 2, LS_DTYPE_INT64 = 3,
+  LS_DTYPE_FLOAT16 = 4, LS_DTYPE_INT8 = 5
+};
+#define LS_MAX_DIMS 8
+
+/* LSModelFactory::GetInstance().CreateModel(class_name, weight_path, max_batch_size),
+ * model_base.h:126-135 */
+int ls_model_create(const char* class_name, const char* weight_path, int max_batch_size,
+                    ls_model** model);
+int ls_model_destroy(ls_model* model);
+/* LSModel::Infer, model_base.h:69 */
+int ls_model_infer(ls_model* model);
+/* model_base.h:72-79 */
+int ls_model_set_input_ptr(ls_model* model, int index, void* input_ptr);
+int ls_model_set_input_shape(ls_model* model, int index, const int* shape, int ndim);
+int ls_model_get_input_max_shape(ls_model* model, int index, int* shape /*[LS_MAX_DIMS]*/,
+                                 int* ndim);
+int ls_model_get_input_size(ls_model* model, int* count);
+int ls_model_get_input_name(ls_model* model, int index, const char** name);
+int ls_model_get_input_dtype(ls_model* model, int index, int* dtype);
+/* model_base.h:82-89 */
+int ls_model_set_output_ptr(ls_model* model, int index, void* output_ptr);
+int ls_model_get_output_ptr(ls_model* model, int index, const void** output_ptr);
+int ls_model_get_output_size(ls_model* model, int* count);
+int ls_model_get_output_name(ls_model* model, int index, const char** name);
+int ls_model_get_output_shape(ls_model* model, int index, int* shape /*[LS_MAX_DIMS]*/, int* ndim);
+int ls_model_get_output_max_shape(ls_model* model, int index, int* shape /*[LS_MAX_DIMS]*/,
+                                  int* ndim);
+int ls_model_get_output_dtype(ls_model* model, int index, int* dtype);
+/* model_base.h:91 */
+int ls_model_benchmark_mode(ls_model* model, int is_benchmark);
+
+/* No counterpart in the reference: the HIP stream the model launches on, so that a
+ * caller can bracket ls_model_infer() with events on that stream. */
+int ls_model_get_stream(ls_model* model, lsh_stream_t* stream);
+/* No counterpart in the reference (it times whole Infer() calls on the host): when
+ * enabled, a QuantBert model brackets every int8 GEMM launch with HIP events on its
+ * stream; ls_model_get_profile() writes a JSON array with, per GEMM site (qkv,
+ * attn_out, ffn1, ffn2): kernel instantiation, m, n, k, launches and total_ms
+ * accumulated since profiling was switched on.  Enabling resets the counters. */
+int ls_model_set_profiling(ls_model* model, int on);
+int ls_model_get_profile(ls_model* model, char* buf, int capacity);
+/* No counterpart in the reference (its DEBUG_RESULT build prints tensors instead):
+ * asks a QuantBert model to copy the named intermediate of encoder layer
+ * `layer` into `dst` (device memory, caller-sized) during the next ls_model_infer().
+ * Names: ln1_q qkv_q ctx_q out_q ln2_q ffn1_q act_q (int8), ffn2_acc (int32),
+ * res_attn res_ffn (fp16 [tokens, hidden]: the residual stream as the LayerNorm kernel
+ * after the attention out-projection / after FFN2 reads it).  dst NULL clears. */
+int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LIGHTSEQ_MODEL_H_ */

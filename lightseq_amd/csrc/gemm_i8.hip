@@ -17,6 +17,8 @@
 #include "ls_device.cuh"
 #include "ls_launch.h"
 
+#include <string>
+
 namespace lsh {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -230,7 +232,23 @@ static int launch_tile(const int8_t* A, const int8_t* W, Epi epi, int M, int N, 
 
 // Picks the tile that wastes the fewest matrix-core cycles on 256 compute units:
 // cost = (#rounds of 256 workgroups) x (work per tile), penalising small tiles for
-// their higher LDS traffic per MAC.
+// their higher LDS traffic per MAC.  Returns an index into kTiles.
+struct TileCand { int bm, bn; double eff; };
+static const TileCand kTiles[3] = {{256, 256, 1.0}, {256, 128, 0.92}, {128, 128, 0.80}};
+
+static int select_tile(int M, int N) {
+  int best = 2;
+  double best_cost = 1e300;
+  for (int c = 0; c < 3; ++c) {
+    const long tiles =
+        (long)((M + kTiles[c].bm - 1) / kTiles[c].bm) * ((N + kTiles[c].bn - 1) / kTiles[c].bn);
+    const long rounds = (tiles + 255) / 256;
+    const double cost = (double)rounds * kTiles[c].bm * kTiles[c].bn / kTiles[c].eff;
+    if (cost < best_cost) { best_cost = cost; best = c; }
+  }
+  return best;
+}
+
 template <typename Epi>
 static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int K,
                     const void* Cptr, hipStream_t s) {
@@ -240,21 +258,18 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   if (((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) & 15u) != 0)
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: operands must be 16-byte aligned");
   const bool vec_store = Epi::vec_ok(N, Cptr);
-  struct Cand { int bm, bn; double eff; };
-  const Cand cands[3] = {{256, 256, 1.0}, {256, 128, 0.92}, {128, 128, 0.80}};
-  int best = 2;
-  double best_cost = 1e300;
-  for (int c = 0; c < 3; ++c) {
-    const long tiles = (long)((M + cands[c].bm - 1) / cands[c].bm) * ((N + cands[c].bn - 1) / cands[c].bn);
-    const long rounds = (tiles + 255) / 256;
-    const double cost = (double)rounds * cands[c].bm * cands[c].bn / cands[c].eff;
-    if (cost < best_cost) { best_cost = cost; best = c; }
-  }
-  switch (best) {
+  switch (select_tile(M, N)) {
     case 0: return launch_tile<256, 256, Epi>(A, W, epi, M, N, K, vec_store, s);
     case 1: return launch_tile<256, 128, Epi>(A, W, epi, M, N, K, vec_store, s);
     default: return launch_tile<128, 128, Epi>(A, W, epi, M, N, K, vec_store, s);
   }
+}
+
+std::string gemm_i8_kernel_name(int M, int N, int K, bool int8_out) {
+  (void)K;
+  const TileCand& t = kTiles[select_tile(M, N)];
+  return "gemm_i8_kernel<" + std::to_string(t.bm) + "," + std::to_string(t.bn) + "," +
+         (int8_out ? "EpiI8" : "EpiI32") + ">";
 }
 
 int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int K,

@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <string>
+
 #include "../../include/lightseq_hip.h"
 
 namespace lsh {
@@ -27,6 +29,11 @@ int dequantize_tensor(const int32_t* input, T* output, long n, float dequant_sca
 template <typename T>
 int quantize_transpose(const T* input, int8_t* output, int rows, int cols, float quant_scale,
                        bool transpose, hipStream_t s);
+// stored uint8 (= code + 127) kernels -> int8 codes (optionally transposed) / T values
+int stored_u8_to_i8(const uint8_t* input, int8_t* output, int rows, int cols, bool transpose,
+                    hipStream_t s);
+template <typename T>
+int stored_u8_dequant(const uint8_t* input, T* output, long n, float clip_max, hipStream_t s);
 template <typename T>
 int scaled_colsum(const T* inp, T* out, int rows, int cols, float scale, hipStream_t s);
 
@@ -92,5 +99,7 @@ int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int
                  hipStream_t s);
 int gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K, float alpha,
                 hipStream_t s);
+// Name of the kernel instantiation the dispatcher picks for a shape (for profiles).
+std::string gemm_i8_kernel_name(int M, int N, int K, bool int8_out);
 
 }  // namespace lsh

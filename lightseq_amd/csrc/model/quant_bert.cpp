@@ -1,0 +1,84 @@
+#include "quant_bert.h"
+
+namespace lightseq {
+namespace hip {
+
+QuantBert::QuantBert(const std::string weight_path, const int max_batch_size)
+    : LSModel({"token_ids"}, {"encoder_output"}), _max_batch_size(max_batch_size) {
+  if (max_batch_size <= 0) throw std::runtime_error("max_batch_size must be positive");
+  CHECK_GPU_ERROR(hipSetDevice(0));
+  CHECK_GPU_ERROR(hipStreamCreate(&stream_));
+
+  std::string res = tw_.initializing(weight_path);
+  if (!res.empty()) throw std::runtime_error(res);
+
+  const size_t tokens = (size_t)_max_batch_size * tw_._max_step;
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_input_), tokens * sizeof(int)));
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_padding_mask_), tokens * sizeof(int)));
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_encoder_output_),
+                            tokens * tw_._hidden_size * sizeof(__half)));
+
+  encoder_ = std::make_shared<QuantBertEncoder>(max_batch_size, d_input_, d_padding_mask_,
+                                                d_encoder_output_, tw_, stream_);
+  res = encoder_->check();
+  if (!res.empty()) throw std::runtime_error(res);
+  encoder_->init_buffer();
+  CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+}
+
+QuantBert::~QuantBert() {
+  encoder_.reset();
+  if (d_input_) (void)hipFree(d_input_);
+  if (d_padding_mask_) (void)hipFree(d_padding_mask_);
+  if (d_encoder_output_) (void)hipFree(d_encoder_output_);
+  if (stream_) (void)hipStreamDestroy(stream_);
+}
+
+void QuantBert::Infer() {
+  if (input_shapes_[0].size() != 2) throw std::runtime_error("token_ids must be 2-D");
+  int batch_size = input_shapes_[0][0], seq_len = input_shapes_[0][1];
+  encoder_->run_one_infer(batch_size, seq_len);
+  CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+  encoder_->collect_profile();
+  set_output_shape(0, {batch_size, seq_len, tw_._hidden_size});
+}
+
+void QuantBert::set_input_ptr(int index, void* input_ptr) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  encoder_->_p_d_token_id = static_cast<int*>(input_ptr);
+}
+
+void QuantBert::set_output_ptr(int index, void* output_ptr) {
+  if (index != 0) throw std::runtime_error("invalid output index");
+  encoder_->_p_d_output = static_cast<__half*>(output_ptr);
+}
+
+const void* QuantBert::get_output_ptr(int index) {
+  if (index != 0) throw std::runtime_error("invalid output index");
+  return static_cast<void*>(encoder_->_p_d_output);
+}
+
+std::vector<int> QuantBert::get_input_max_shape(int index) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  return {_max_batch_size, tw_._max_step};
+}
+
+std::vector<int> QuantBert::get_output_max_shape(int index) {
+  if (index != 0) throw std::runtime_error("invalid output index");
+  return {_max_batch_size, tw_._max_step, tw_._hidden_size};
+}
+
+DataType QuantBert::get_input_dtype(int index) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  return DataType::kInt32;
+}
+
+DataType QuantBert::get_output_dtype(int index) {
+  if (index != 0) throw std::runtime_error("invalid output index");
+  return DataType::kFloat16;
+}
+
+LSMODEL_REGISTER(QuantBert)
+
+}  // namespace hip
+}  // namespace lightseq

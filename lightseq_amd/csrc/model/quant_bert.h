@@ -1,0 +1,44 @@
+// "QuantBert" model: the int8 BERT encoder behind the LSModel interface.
+// Mirrors lightseq/inference/pywrapper/quant_bert.{h,cc}: input 0 "token_ids"
+// int32 [batch, seq_len]; output 0 "encoder_output" fp16 [batch, seq_len, hidden].
+#pragma once
+
+#include <memory>
+
+#include "ls_model.h"
+#include "quant_bert_encoder.h"
+
+namespace lightseq {
+namespace hip {
+
+class QuantBert : public LSModel {
+ public:
+  QuantBert(const std::string weight_path, const int max_batch_size);
+  ~QuantBert();
+
+  void Infer() override;
+  void set_input_ptr(int index, void* input_ptr) override;
+  void set_output_ptr(int index, void* output_ptr) override;
+  const void* get_output_ptr(int index) override;
+  std::vector<int> get_input_max_shape(int index) override;
+  std::vector<int> get_output_max_shape(int index) override;
+  DataType get_input_dtype(int index) override;
+  DataType get_output_dtype(int index) override;
+  void benchmark_mode(bool) override {}
+  void* get_stream() override { return stream_; }
+
+  QuantBertEncoder* encoder() { return encoder_.get(); }
+  const QuantBertWeight& weight() const { return tw_; }
+
+ private:
+  std::shared_ptr<QuantBertEncoder> encoder_;
+  int* d_input_ = nullptr;
+  int* d_padding_mask_ = nullptr;
+  __half* d_encoder_output_ = nullptr;
+  int _max_batch_size;
+  hipStream_t stream_ = nullptr;
+  QuantBertWeight tw_;
+};
+
+}  // namespace hip
+}  // namespace lightseq

@@ -1,0 +1,280 @@
+#include "quant_bert_encoder.h"
+
+#include <algorithm>
+
+namespace lightseq {
+namespace hip {
+
+using namespace lsh;
+
+QuantBertEncoder::QuantBertEncoder(int max_batch_size, const int* p_d_token_id,
+                                   int* p_d_padding_mask, __half* p_d_output,
+                                   const QuantBertWeight& tw, hipStream_t stream)
+    : _p_d_token_id(p_d_token_id),
+      _p_d_padding_mask(p_d_padding_mask),
+      _p_d_output(p_d_output),
+      _max_batch_size(max_batch_size),
+      _tw(tw),
+      _stream(stream),
+      _src_emb_clip_max(tw._src_emb_clip_max),
+      _enc_clip_max(tw._enc_clip_max),
+      _max_batch_dim((long)max_batch_size * tw._max_step * tw._hidden_size) {}
+
+std::string QuantBertEncoder::check() {
+  if (_tw._inner_size & 1) return "violate inner_size % 2 = 0";
+  if (_tw._dim_per_head & 1) return "violate dim_per_head % 2 = 0";
+  if (_tw._multilg_type != 0) return "multilingual models are not supported";
+  if ((int)_tw.layers.size() != _tw._n_enc_layer)
+    return "violate p_d_enc_wei.size() = weight_per_enc_layer * n_enc_layer";
+  if ((int)_enc_clip_max.size() != 11 * _tw._n_enc_layer) return "wrong clip_max table size";
+  if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)
+    return "violate hidden_size % 16 = 0 and inner_size % 16 = 0 (int8 MFMA GEMM)";
+  if (_tw._dim_per_head != 32 && _tw._dim_per_head != 64)
+    return "violate dim_per_head in {32, 64} (fused attention kernel)";
+  if (_tw._max_step > 1024) return "violate max_step <= 1024";
+  return "";
+}
+
+static DeviceBuffer<__half> upload_half(const std::vector<float>& v, hipStream_t s) {
+  std::vector<__half> h = to_half(v);
+  DeviceBuffer<__half> d(h.size());
+  d.upload(h.data(), h.size(), s);
+  CHECK_GPU_ERROR(hipStreamSynchronize(s));  // `h` dies at return
+  return d;
+}
+
+// stored uint8 [rows(in), cols(out)] -> int8 [cols, rows] (K-contiguous for the GEMM)
+static DeviceBuffer<int8_t> upload_kernel(const std::vector<uint8_t>& w, int rows, int cols,
+                                          bool transpose, hipStream_t s) {
+  DeviceBuffer<uint8_t> raw(w.size());
+  raw.upload(w.data(), w.size(), s);
+  DeviceBuffer<int8_t> q(w.size());
+  LSH_CALL(stored_u8_to_i8(raw.get(), q.get(), rows, cols, transpose, s));
+  CHECK_GPU_ERROR(hipStreamSynchronize(s));
+  return q;
+}
+
+void QuantBertEncoder::init_buffer() {
+  const int H = _tw._hidden_size, I = _tw._inner_size;
+  const long tokens = (long)_max_batch_size * _tw._max_step;
+  _qkv_buf.alloc((size_t)(3 * _max_batch_dim));
+  const size_t wide = (size_t)tokens * std::max(I, 3 * H);
+  _int8_ffn_in_buf.alloc(wide);
+  _int8_ffn_out_buf.alloc(wide);
+  _int32_ffn_out_buf.alloc((size_t)tokens * H);
+
+  _int8_emb = upload_kernel(_tw.token_embedding, _tw._src_vocab_size, H, false, _stream);
+  _pos_emb = upload_half(_tw.position_embedding, _stream);
+  _final_ln_scale = upload_half(_tw.norm_scale, _stream);
+  _final_ln_bias = upload_half(_tw.norm_bias, _stream);
+
+  _layers.clear();
+  _layers.resize(_tw._n_enc_layer);
+  for (int l = 0; l < _tw._n_enc_layer; ++l) {
+    const QuantBertLayerWeight& w = _tw.layers[l];
+    Layer& d = _layers[l];
+    d.ln1_scale = upload_half(w.multihead_norm_scale, _stream);
+    d.ln1_bias = upload_half(w.multihead_norm_bias, _stream);
+    d.b_qkv = upload_half(w.multihead_project_bias_qkv, _stream);
+    d.b_out = upload_half(w.multihead_project_bias_output, _stream);
+    d.ln2_scale = upload_half(w.ffn_norm_scale, _stream);
+    d.ln2_bias = upload_half(w.ffn_norm_bias, _stream);
+    d.b_ffn1 = upload_half(w.ffn_first_bias, _stream);
+    d.b_ffn2 = upload_half(w.ffn_second_bias, _stream);
+    d.w_qkv = upload_kernel(w.multihead_project_kernel_qkv, H, 3 * H, true, _stream);
+    d.w_out = upload_kernel(w.multihead_project_kernel_output, H, H, true, _stream);
+    d.w_ffn1 = upload_kernel(w.ffn_first_kernel, H, I, true, _stream);
+    d.w_ffn2 = upload_kernel(w.ffn_second_kernel, I, H, true, _stream);
+    if (!_tw._use_gelu) {
+      // ReLU offset trick: colsum of the fp16-rounded dequantised FFN2 weight times
+      // clip/2 (quant_bert_encoder.cc.cu:156-175)
+      const size_t n = w.ffn_second_kernel.size();
+      DeviceBuffer<uint8_t> raw(n);
+      raw.upload(w.ffn_second_kernel.data(), n, _stream);
+      DeviceBuffer<__half> deq(n);
+      LSH_CALL(stored_u8_dequant<__half>(raw.get(), deq.get(), (long)n, _enc_clip_max[l * 11 + 3],
+                                         _stream));
+      d.ffn2_colsum.alloc(H);
+      LSH_CALL(scaled_colsum<__half>(deq.get(), d.ffn2_colsum.get(), I, H,
+                                     _enc_clip_max[l * 11 + 7] / 2, _stream));
+      CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+    }
+  }
+}
+
+void QuantBertEncoder::set_profiling(bool on) {
+  _profiling = on;
+  if (on && _profile.empty()) {
+    _profile.resize(4);
+    const char* names[4] = {"qkv", "attn_out", "ffn1", "ffn2"};
+    for (int i = 0; i < 4; ++i) _profile[i].site = names[i];
+  }
+}
+
+void QuantBertEncoder::reset_profile() {
+  for (auto& p : _profile) { p.launches = 0; p.total_ms = 0.0; }
+}
+
+void QuantBertEncoder::prof_begin(int site, int m, int n, int k, bool int8_out) {
+  if (!_profiling) return;
+  SiteProfile& p = _profile[site];
+  if (p.m != m || p.n != n || p.k != k) {
+    p.m = m; p.n = n; p.k = k;
+    p.kernel = gemm_i8_kernel_name(m, n, k, int8_out);
+  }
+  Pending pe;
+  pe.site = site;
+  for (hipEvent_t* e : {&pe.e0, &pe.e1}) {
+    if (_event_pool.empty()) {
+      CHECK_GPU_ERROR(hipEventCreate(e));
+    } else {
+      *e = _event_pool.back();
+      _event_pool.pop_back();
+    }
+  }
+  CHECK_GPU_ERROR(hipEventRecord(pe.e0, _stream));
+  _pending.push_back(pe);
+}
+
+void QuantBertEncoder::prof_end() {
+  if (!_profiling) return;
+  CHECK_GPU_ERROR(hipEventRecord(_pending.back().e1, _stream));
+}
+
+void QuantBertEncoder::collect_profile() {
+  for (Pending& pe : _pending) {
+    float ms = 0.f;
+    CHECK_GPU_ERROR(hipEventElapsedTime(&ms, pe.e0, pe.e1));
+    _profile[pe.site].launches += 1;
+    _profile[pe.site].total_ms += ms;
+    _event_pool.push_back(pe.e0);
+    _event_pool.push_back(pe.e1);
+  }
+  _pending.clear();
+}
+
+void QuantBertEncoder::tap(int8_t* dst, const int8_t* src, size_t n) {
+  if (dst && taps.tap_layer == _layer_id)
+    CHECK_GPU_ERROR(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, _stream));
+}
+
+void QuantBertEncoder::run_one_infer(int batch_size, int batch_seq_len) {
+  if (batch_size > _max_batch_size)
+    throw std::runtime_error("batch size of input greater than max_batch_size");
+  if (batch_seq_len > _tw._max_step)
+    throw std::runtime_error("seq len of input greater than max_step");
+  if (batch_size <= 0 || batch_seq_len <= 0) throw std::runtime_error("empty input");
+  _batch_size = batch_size;
+  _batch_seq_len = batch_seq_len;
+  _batch_token_num = batch_size * batch_seq_len;
+
+  LSH_CALL(enc_emb_i8I<__half>(_int8_emb.get(), _pos_emb.get(), _p_d_token_id, _p_d_output,
+                               _p_d_padding_mask, _tw._padding_id, batch_size, batch_seq_len,
+                               _tw._hidden_size, _stream, _src_emb_clip_max / _quant_range, false));
+  for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
+    self_attention();
+    ffn_add_norm();
+  }
+}
+
+void QuantBertEncoder::self_attention() {
+  const int H = _tw._hidden_size, M = _batch_token_num;
+  const Layer& w = _layers[_layer_id];
+  const float* c = &_enc_clip_max[_layer_id * 11];
+  const float Q = _quant_range;
+
+  if (_layer_id == 0) {
+    LSH_CALL(norm_layer_resual_i8O<__half>(M, H, _stream, _p_d_output, _int8_ffn_in_buf.get(),
+                                           w.ln1_scale.get(), w.ln1_bias.get(), w.b_out.get(),
+                                           Q / c[4], _tw._is_post_ln));
+  }
+  tap(taps.ln1_q, _int8_ffn_in_buf.get(), (size_t)M * H);
+
+  // qkv = ori_q * qkv_wei, int8 out
+  prof_begin(0, M, 3 * H, H, true);
+  LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_qkv.get(), _int8_ffn_out_buf.get(), M, 3 * H, H,
+                       c[0] * c[4] / (c[8] * Q), _stream));
+  prof_end();
+  tap(taps.qkv_q, _int8_ffn_out_buf.get(), (size_t)M * 3 * H);
+
+  // dequant + bias, split heads -> fp16 q, k, v [B, h, S, d]
+  const long mbd = (long)M * H;
+  LSH_CALL(arrange_encself_qkv_i8I<__half>(M, H, _stream, _int8_ffn_out_buf.get(), w.b_qkv.get(),
+                                           _qkv_buf.get(), mbd, _batch_seq_len, _tw._dim_per_head,
+                                           _tw._head_num, c[8] / Q));
+
+  // scores -> masked softmax -> context -> merge heads + quantise, one kernel
+  LSH_CALL(encself_attention_f16(_qkv_buf.get(), _qkv_buf.get() + mbd, _qkv_buf.get() + 2 * mbd,
+                                 _p_d_padding_mask, nullptr, _int8_ffn_in_buf.get(), Q / c[5],
+                                 _batch_size, _batch_seq_len, _tw._head_num, _tw._dim_per_head,
+                                 _stream));
+  tap(taps.ctx_q, _int8_ffn_in_buf.get(), (size_t)M * H);
+
+  prof_begin(1, M, H, H, true);
+  LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_out.get(), _int8_ffn_out_buf.get(), M, H, H,
+                       c[1] * c[5] / (c[9] * Q), _stream));
+  prof_end();
+  tap(taps.out_q, _int8_ffn_out_buf.get(), (size_t)M * H);
+
+  if (taps.res_attn && taps.tap_layer == _layer_id)
+    CHECK_GPU_ERROR(hipMemcpyAsync(taps.res_attn, _p_d_output, (size_t)M * H * sizeof(__half),
+                                   hipMemcpyDeviceToDevice, _stream));
+  LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(
+      _int8_ffn_out_buf.get(), w.ln2_scale.get(), w.ln2_bias.get(), w.b_ffn2.get(),
+      _int8_ffn_in_buf.get(), _p_d_output, M, H, c[9] / Q, Q / c[6], _stream, _tw._is_post_ln,
+      nullptr)));
+  tap(taps.ln2_q, _int8_ffn_in_buf.get(), (size_t)M * H);
+}
+
+void QuantBertEncoder::ffn_add_norm() {
+  const int H = _tw._hidden_size, I = _tw._inner_size, M = _batch_token_num;
+  const Layer& w = _layers[_layer_id];
+  const float* c = &_enc_clip_max[_layer_id * 11];
+  const float Q = _quant_range;
+
+  prof_begin(2, M, I, H, true);
+  LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_ffn1.get(), _int8_ffn_out_buf.get(), M, I, H,
+                       c[2] * c[6] / (c[10] * Q), _stream));
+  prof_end();
+  tap(taps.ffn1_q, _int8_ffn_out_buf.get(), (size_t)M * I);
+
+  if (_tw._use_gelu) {
+    LSH_CALL(bias_gelu_i8I_i8O<__half>(M, _stream, _int8_ffn_out_buf.get(), _int8_ffn_in_buf.get(),
+                                       w.b_ffn1.get(), I, c[10] / Q, Q / c[7]));
+  } else {
+    LSH_CALL(bias_relu_i8I_i8O<__half>(M, _stream, _int8_ffn_out_buf.get(), _int8_ffn_in_buf.get(),
+                                       w.b_ffn1.get(), I, c[10] / Q, Q / c[7], c[7], true));
+  }
+  tap(taps.act_q, _int8_ffn_in_buf.get(), (size_t)M * I);
+
+  prof_begin(3, M, H, I, false);
+  LSH_CALL(gemm_i8_i32o(_int8_ffn_in_buf.get(), w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I,
+                        _stream));
+  prof_end();
+  if (taps.ffn2_acc && taps.tap_layer == _layer_id)
+    CHECK_GPU_ERROR(hipMemcpyAsync(taps.ffn2_acc, _int32_ffn_out_buf.get(),
+                                   (size_t)M * H * sizeof(int32_t), hipMemcpyDeviceToDevice,
+                                   _stream));
+
+  if (taps.res_ffn && taps.tap_layer == _layer_id)
+    CHECK_GPU_ERROR(hipMemcpyAsync(taps.res_ffn, _p_d_output, (size_t)M * H * sizeof(__half),
+                                   hipMemcpyDeviceToDevice, _stream));
+  const float dequant_scale =
+      _tw._use_gelu ? c[3] * c[7] / (Q * Q) : c[3] * c[7] / (2 * Q * Q);
+  const __half* colsum = w.ffn2_colsum.get();  // nullptr for GELU models
+  if (_layer_id == _tw._n_enc_layer - 1) {
+    LSH_CALL(residual_bias_ln_i32I<__half>(_int32_ffn_out_buf.get(), _final_ln_scale.get(),
+                                           _final_ln_bias.get(), _p_d_output, _p_d_output, M, H,
+                                           dequant_scale, _stream, colsum));
+  } else {
+    const Layer& nx = _layers[_layer_id + 1];
+    const float clip_next = _enc_clip_max[(_layer_id + 1) * 11 + 4];
+    LSH_CALL((residual_bias_ln_i8O<__half, int32_t>(
+        _int32_ffn_out_buf.get(), nx.ln1_scale.get(), nx.ln1_bias.get(), nx.b_out.get(),
+        _int8_ffn_in_buf.get(), _p_d_output, M, H, dequant_scale, Q / clip_next, _stream,
+        _tw._is_post_ln, colsum)));
+  }
+}
+
+}  // namespace hip
+}  // namespace lightseq

@@ -158,6 +158,68 @@ int scaled_colsum(const T* inp, T* out, int rows, int cols, float scale, hipStre
   return lsh_check_launch("scaled_colsum_kernel");
 }
 
+// Stored model kernels are uint8 = code + 127 (training/ops/pytorch/export_quant.py:12-20).
+// rows x cols bytes -> int8 codes clamped to [-127, 127], optionally transposed.
+template <bool TRANSPOSE>
+__global__ void __launch_bounds__(256)
+stored_u8_to_i8_kernel(const uint8_t* __restrict__ in, int8_t* __restrict__ out, int rows,
+                       int cols) {
+  __shared__ int8_t tile[64][65];
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int r = ty; r < 64; r += 4) {
+    int rr = r0 + r, cc = c0 + tx;
+    if (rr < rows && cc < cols) {
+      int q = (int)in[(long)rr * cols + cc] - 127;
+      tile[r][tx] = (int8_t)max(-127, min(127, q));
+    }
+  }
+  __syncthreads();
+  if (TRANSPOSE) {
+    for (int c = ty; c < 64; c += 4) {
+      int cc = c0 + c, rr = r0 + tx;
+      if (rr < rows && cc < cols) out[(long)cc * rows + rr] = tile[tx][c];
+    }
+  } else {
+    for (int r = ty; r < 64; r += 4) {
+      int rr = r0 + r, cc = c0 + tx;
+      if (rr < rows && cc < cols) out[(long)rr * cols + cc] = tile[r][tx];
+    }
+  }
+}
+
+int stored_u8_to_i8(const uint8_t* input, int8_t* output, int rows, int cols, bool transpose,
+                    hipStream_t s) {
+  if (rows <= 0 || cols <= 0 || !input || !output)
+    return lsh_fail(LSH_ERR_INVALID, "stored_u8_to_i8: bad arguments");
+  dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+  if (transpose)
+    stored_u8_to_i8_kernel<true><<<grid, 256, 0, s>>>(input, output, rows, cols);
+  else
+    stored_u8_to_i8_kernel<false><<<grid, 256, 0, s>>>(input, output, rows, cols);
+  return lsh_check_launch("stored_u8_to_i8_kernel");
+}
+
+// T((uint8 - 127) * clip_max / 127): the loader's dequantize() followed by its cast
+// to T (inference/tools/util.cc.cu:346-348, proto/quant_bert_weight.cc:28-30).
+template <typename T>
+__global__ void stored_u8_dequant_kernel(const uint8_t* __restrict__ in, T* __restrict__ out,
+                                         long n, float clip_max) {
+  long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long stride = (long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) TT<T>::st(out, i, ((float)in[i] - 127.f) * clip_max / 127.f);
+}
+
+template <typename T>
+int stored_u8_dequant(const uint8_t* input, T* output, long n, float clip_max, hipStream_t s) {
+  if (n <= 0 || !input || !output)
+    return lsh_fail(LSH_ERR_INVALID, "stored_u8_dequant: bad arguments");
+  stored_u8_dequant_kernel<T><<<stream_grid(n, 256), 256, 0, s>>>(input, output, n, clip_max);
+  return lsh_check_launch("stored_u8_dequant_kernel");
+}
+template int stored_u8_dequant<float>(const uint8_t*, float*, long, float, hipStream_t);
+template int stored_u8_dequant<__half>(const uint8_t*, __half*, long, float, hipStream_t);
+
 #define LSH_INST(T)                                                                          \
   template int quantize_tensor<T>(const T*, int8_t*, long, float, hipStream_t);              \
   template int dequantize_tensor<T>(const int32_t*, T*, long, float, hipStream_t);           \

@@ -16,3 +16,6 @@ def to_np(t):
 
 def torch_dtype(np_dtype):
     return {np.dtype(np.float16): torch.float16, np.dtype(np.float32): torch.float32}[np.dtype(np_dtype)]
+
+
+from oracle.model_io import oracle_weights_from_message  # noqa: E402,F401

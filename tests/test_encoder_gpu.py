@@ -1,0 +1,225 @@
+"""GPU parity of the whole int8 encoder stack (QuantBert) against the CPU oracle,
+through the model C ABI, on synthetic model files in the reference's format.
+
+Bars: int32 FFN2 accumulators bit-exact wherever their int8 inputs agree, int8
+activations within +-1 code on <= 0.1 % of elements, fp16 layer outputs within
+2e-2 absolute at valid (non-padded) positions.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_codes_close
+from helpers import DEV, oracle_weights_from_message
+
+pytestmark = pytest.mark.gpu
+
+
+def _build(tmp_path, cfg_name, seed, **over):
+    from lightseq_amd import synthetic
+    cfg = synthetic.bert_config(cfg_name)
+    cfg.update(over)
+    path = str(tmp_path / ("%s_%d.pb" % (cfg_name, seed)))
+    msg = synthetic.write_quant_bert(path, cfg, seed=seed)
+    return cfg, msg, path
+
+
+def _valid(ids, cfg):
+    return ids != cfg["padding_id"]
+
+
+@pytest.mark.parametrize("cfg_name,batch,seq,over", [
+    ("tiny", 3, 20, {}),
+    ("tiny", 2, 33, {"use_gelu": False}),
+    ("tiny", 2, 16, {"is_post_ln": False}),
+    ("tiny", 1, 64, {"is_post_ln": False, "use_gelu": False}),
+])
+def test_tiny_stack_with_taps(tmp_path, oracle, cfg_name, batch, seq, over):
+    from lightseq_amd import inference, synthetic
+    cfg, msg, path = _build(tmp_path, cfg_name, 3, **over)
+    ids, _ = synthetic.make_token_ids(cfg, batch, seq, seed=5)
+    w = oracle_weights_from_message(msg, cfg)
+    M, H, I = batch * seq, cfg["hidden"], cfg["inner"]
+    model = inference.QuantBert(path, batch)
+    for layer in range(cfg["n_layer"]):
+        want, want_mask, taps = oracle.quant_bert_encoder(w, ids, tap_layer=layer)
+        bufs = {}
+        for name, shape, dt in [("ln1_q", (M, H), torch.int8), ("qkv_q", (M, 3 * H), torch.int8),
+                                ("ctx_q", (M, H), torch.int8), ("out_q", (M, H), torch.int8),
+                                ("ln2_q", (M, H), torch.int8), ("ffn1_q", (M, I), torch.int8),
+                                ("act_q", (M, I), torch.int8), ("ffn2_acc", (M, H), torch.int32)]:
+            bufs[name] = torch.zeros(shape, dtype=dt, device=DEV)
+            model.set_tap(layer, name, bufs[name])
+        got = model.infer_fp16(ids)
+        valid = _valid(ids, cfg).reshape(-1)
+        for name in ("ln1_q", "qkv_q", "ctx_q", "out_q", "ln2_q", "ffn1_q", "act_q"):
+            g = bufs[name].cpu().numpy()
+            # padded query rows of the attention context are don't-care downstream
+            assert_codes_close(g[valid], taps[name][valid], max_frac=3e-3, what="%s layer %d" % (name, layer))
+        # int32 accumulators: exact given the kernel's own int8 inputs
+        act = bufs["act_q"].cpu().numpy()
+        w2 = w["w_ffn2"][layer]
+        exact = np.rint(act.astype(np.float64) @ w2.astype(np.float64).T).astype(np.int64)
+        np.testing.assert_array_equal(bufs["ffn2_acc"].cpu().numpy().astype(np.int64), exact)
+        for name in bufs:
+            model.set_tap(layer, name, None)
+    v = _valid(ids, cfg)
+    np.testing.assert_allclose(got.astype(np.float32)[v], want.astype(np.float32)[v], atol=2e-2, rtol=0)
+    model.close()
+
+
+def test_transformer_base_layer_config(tmp_path, oracle):
+    """One Transformer-base-shaped int8 encoder layer: batch 8, seq 64, hidden 512,
+    8 heads, FFN 2048 ReLU, post-LN, all-ones mask, seed 0."""
+    from lightseq_amd import inference, synthetic
+    cfg, msg, path = _build(tmp_path, "transformer_base_layer", 0)
+    ids, _ = synthetic.make_token_ids(cfg, 8, 64, seed=0, min_len=64)  # no padding
+    w = oracle_weights_from_message(msg, cfg)
+    want, _, _ = oracle.quant_bert_encoder(w, ids)
+    model = inference.QuantBert(path, 8)
+    got = model.infer(ids)
+    assert got.dtype == np.float32 and got.shape == (8, 64, 512)
+    np.testing.assert_allclose(got, want.astype(np.float32), atol=2e-2, rtol=0)
+    model.close()
+
+
+TAP_SPECS = [("ln1_q", "H", "i8"), ("qkv_q", "3H", "i8"), ("ctx_q", "H", "i8"), ("out_q", "H", "i8"),
+             ("ln2_q", "H", "i8"), ("ffn1_q", "I", "i8"), ("act_q", "I", "i8"), ("ffn2_acc", "H", "i32"),
+             ("res_attn", "H", "f16"), ("res_ffn", "H", "f16")]
+
+
+def _run_with_taps(model, ids, layer, M, H, I):
+    width = {"H": H, "3H": 3 * H, "I": I}
+    dts = {"i8": torch.int8, "i32": torch.int32, "f16": torch.float16}
+    bufs = {}
+    for name, wd, dt in TAP_SPECS:
+        bufs[name] = torch.zeros((M, width[wd]), dtype=dts[dt], device=DEV)
+        model.set_tap(layer, name, bufs[name])
+    out = model.infer_fp16(ids)
+    taps = {k: v.cpu().numpy() for k, v in bufs.items()}
+    for name, _, _ in TAP_SPECS:
+        model.set_tap(layer, name, None)
+    return out, taps
+
+
+def test_bert_base_two_layers_full_width(tmp_path, oracle):
+    """BERT-base width (hidden 768, 12 heads, FFN 3072 GELU), batch 32 x seq 128 with
+    ragged valid lengths, cut to 2 layers so the oracle finishes in seconds.
+
+    A +-1 code difference in one int8 activation perturbs every accumulator of its row
+    in the next GEMM and flips further codes there, so two correct implementations
+    drift apart layer by layer.  Parity is therefore checked per stage, each stage of
+    the oracle being fed the GPU's own input of that stage; the end-to-end output is
+    checked statistically."""
+    from lightseq_amd import inference, synthetic
+    cfg, msg, path = _build(tmp_path, "bert_base", 1, n_layer=2, vocab=2000, max_step=128)
+    B, S, H, I, h = 32, 128, cfg["hidden"], cfg["inner"], cfg["head_num"]
+    M, Q = B * S, np.float32(127)
+    ids, lens = synthetic.make_token_ids(cfg, B, S, seed=2, min_len=32)
+    w = oracle_weights_from_message(msg, cfg)
+    want, want_mask, _ = oracle.quant_bert_encoder(w, ids)
+    model = inference.QuantBert(path, B)
+    valid = _valid(ids, cfg).reshape(-1)
+    for layer in range(2):
+        got, t = _run_with_taps(model, ids, layer, M, H, I)
+        c = w["clip_max"][layer * 11:(layer + 1) * 11]
+        # int8 GEMMs with requantising epilogue: bit exact given the same int8 input
+        np.testing.assert_array_equal(
+            t["qkv_q"], oracle.gemm_i8_i8(t["ln1_q"], w["w_qkv"][layer], c[0] * c[4] / (c[8] * Q)))
+        np.testing.assert_array_equal(
+            t["out_q"], oracle.gemm_i8_i8(t["ctx_q"], w["w_out"][layer], c[1] * c[5] / (c[9] * Q)))
+        np.testing.assert_array_equal(
+            t["ffn1_q"], oracle.gemm_i8_i8(t["ln2_q"], w["w_ffn1"][layer], c[2] * c[6] / (c[10] * Q)))
+        # FFN2: int32 accumulators bit exact
+        np.testing.assert_array_equal(t["ffn2_acc"], oracle.gemm_i8_i32(t["act_q"], w["w_ffn2"][layer]))
+        # attention block from the GPU's own qkv codes
+        qkv = oracle.arrange_encself_qkv_i8I(t["qkv_q"], w["b_qkv"][layer], B, S, h, c[8] / Q)
+        probs = oracle.correlation_softmax_encself(
+            oracle.attn_scores(qkv[0], qkv[1], np.sqrt(1.0 / (H // h))), want_mask)
+        ctx_q = oracle.arrange_atten_output_i8O(oracle.attn_context(probs, qkv[2]), Q / c[5])
+        assert_codes_close(t["ctx_q"][valid], ctx_q[valid], what="ctx_q layer %d" % layer)
+        # LayerNorm after attention, from the GPU's own GEMM output and residual stream
+        ln2_q, _ = oracle.residual_bias_ln_i8O(t["out_q"], w["ln2_scale"][layer], w["ln2_bias"][layer],
+                                               w["b_ffn2"][layer], t["res_attn"], c[9] / Q, Q / c[6],
+                                               cfg["is_post_ln"])
+        assert_codes_close(t["ln2_q"], ln2_q, what="ln2_q layer %d" % layer)
+        act_q = oracle.bias_gelu_i8I_i8O(t["ffn1_q"], w["b_ffn1"][layer], c[10] / Q, Q / c[7])
+        assert_codes_close(t["act_q"], act_q, what="act_q layer %d" % layer)
+        dq = c[3] * c[7] / (Q * Q)
+        if layer == 0:
+            cn = w["clip_max"][11:22]
+            ln1_next, _ = oracle.residual_bias_ln_i8O(t["ffn2_acc"], w["ln1_scale"][1], w["ln1_bias"][1],
+                                                      w["b_out"][1], t["res_ffn"], dq, Q / cn[4],
+                                                      cfg["is_post_ln"])
+            _, t_next = _run_with_taps(model, ids, 1, M, H, I)
+            assert_codes_close(t_next["ln1_q"], ln1_next, what="ln1_q layer 1")
+        else:
+            final = oracle.residual_bias_ln_i32I(t["ffn2_acc"], w["final_ln_scale"], w["final_ln_bias"],
+                                                 t["res_ffn"], dq)
+            np.testing.assert_allclose(got.reshape(M, H).astype(np.float32), final.astype(np.float32),
+                                       atol=8e-3, rtol=0)
+    # end to end against the oracle's own run: drift from code flips stays small
+    v = _valid(ids, cfg)
+    diff = np.abs(got.astype(np.float32)[v] - want.astype(np.float32)[v])
+    assert diff.mean() <= 5e-3, diff.mean()
+    assert np.quantile(diff, 0.999) <= 3e-2, np.quantile(diff, 0.999)
+    assert diff.max() <= 0.1, diff.max()
+    model.close()
+
+
+def test_bert_base_full_stack_properties(tmp_path):
+    """The benchmark workload itself (12 layers, b32 x s128): size-independent
+    properties.  A sequence's output does not depend on what else is in the batch
+    (every kernel is row- or sequence-independent), runs are deterministic, and the
+    final LayerNorm leaves every valid row with the statistics of its scale/bias."""
+    from lightseq_amd import inference, synthetic
+    cfg, msg, path = _build(tmp_path, "bert_base", 0, vocab=3000)
+    ids, lens = synthetic.make_token_ids(cfg, 32, 128, seed=0, min_len=32)
+    model = inference.QuantBert(path, 32)
+    out = model.infer_fp16(ids)
+    assert np.isfinite(out.astype(np.float32)).all()
+    np.testing.assert_array_equal(out, model.infer_fp16(ids))
+    for b in (0, 7, 31):
+        alone = model.infer_fp16(ids[b:b + 1])
+        np.testing.assert_array_equal(alone[0], out[b])
+    perm = np.random.default_rng(0).permutation(32)
+    np.testing.assert_array_equal(model.infer_fp16(ids[perm]), out[perm])
+    g = np.asarray(msg["src_embedding"]["norm_scale"], np.float32)
+    beta = np.asarray(msg["src_embedding"]["norm_bias"], np.float32)
+    z = (out.astype(np.float32) - beta) / g
+    v = ids != cfg["padding_id"]
+    np.testing.assert_allclose(z[v].mean(-1), 0.0, atol=2e-2)
+    np.testing.assert_allclose(z[v].std(-1), 1.0, atol=2e-2)
+    model.close()
+
+
+def test_model_interface_and_errors(tmp_path):
+    from lightseq_amd import inference, synthetic
+    from lightseq_amd.lib import LSHError
+    cfg, msg, path = _build(tmp_path, "tiny", 0)
+    model = inference.QuantBert(path, 4)
+    assert model.get_input_size() == 1 and model.get_output_size() == 1
+    assert model.get_input_name(0) == "token_ids" and model.get_output_name(0) == "encoder_output"
+    assert model.get_input_max_shape(0) == [4, cfg["max_step"]]
+    assert model.get_output_max_shape(0) == [4, cfg["max_step"], cfg["hidden"]]
+    assert model.get_input_dtype(0) == 2 and model.get_output_dtype(0) == 4
+    ids, _ = synthetic.make_token_ids(cfg, 2, 10)
+    out = model.infer(ids)
+    assert out.shape == (2, 10, cfg["hidden"]) and np.isfinite(out).all()
+    assert model.get_output_shape(0) == [2, 10, cfg["hidden"]]
+    # same input twice -> identical output (no state leaks between calls)
+    np.testing.assert_array_equal(out, model.infer(ids))
+    with pytest.raises(LSHError, match="batch size of input greater than max_batch_size"):
+        model.infer(np.ones((5, 4), np.int32))
+    big = np.ones((1, cfg["max_step"] + 1), np.int32)
+    with pytest.raises(LSHError, match="seq len of input greater than max_step"):
+        model.infer(big)
+    model.close()
+    with pytest.raises(LSHError, match="not found"):
+        inference.QuantBert(str(tmp_path / "missing.pb"), 1)
+    with pytest.raises(LSHError, match="Model not supported"):
+        inference.LSModel("NoSuchModel", path, 1)
+    bad = tmp_path / "bad.pb"
+    bad.write_bytes(b"\x0a\x03abc")
+    with pytest.raises(LSHError):
+        inference.QuantBert(str(bad), 1)
