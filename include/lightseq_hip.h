@@ -216,6 +216,29 @@ int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n,
  * model/cublas_helper.h:50-58 cublaslt_gemm<int8_t,float>. */
 int lsh_gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int m, int n, int k, float alpha,
                     lsh_stream_t stream);
+/* Fused GEMM epilogues (fp16 storage).  No single counterpart in the reference: each is
+ * the int8-output GEMM above followed, in the same kernel, by the launcher named below,
+ * and produces exactly the bytes that pair produces (the intermediate int8 code is
+ * formed in registers and never written to HBM).
+ *  - lsh_gemm_i8_bias_gelu_i8o_f16 / lsh_gemm_i8_bias_relu_i8o_f16: FFN1 GEMM
+ *    (model/quant_bert_encoder.cc.cu:415-431) + ker_bias_gelu_i8I_i8O_launcher /
+ *    ker_bias_relu_i8I_i8O_launcher (:433-447); alpha as for lsh_gemm_i8_i8o, the
+ *    remaining arguments as for the launcher.
+ *  - lsh_gemm_i8_qkv_arrange_f16: QKV GEMM (:296-311) +
+ *    ker_arrange_encself_qkv_i8I_launcher (:314-318); writes q, k, v as fp16
+ *    [batch, head_num, seq_len, dim_per_head] at new_qkv + {0,1,2} * max_batch_dim.
+ *    Needs dim_per_head % 16 == 0. */
+int lsh_gemm_i8_bias_gelu_i8o_f16(const int8_t* A, const int8_t* W, int8_t* C, const void* bias,
+                                  int m, int n, int k, float alpha, float dequant_scale,
+                                  float quant_scale, lsh_stream_t stream);
+int lsh_gemm_i8_bias_relu_i8o_f16(const int8_t* A, const int8_t* W, int8_t* C, const void* bias,
+                                  int m, int n, int k, float alpha, float dequant_scale,
+                                  float quant_scale, float clip_max, int narrow_clip,
+                                  lsh_stream_t stream);
+int lsh_gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, void* new_qkv,
+                                const void* qkv_bias, int max_batch_dim, int batch_token_num,
+                                int hidden_size, int k, int batch_seq_len, int head_num,
+                                float alpha, float dequant_scale, lsh_stream_t stream);
 /* model/cublas_helper.h:60 quantize_weight: `origin_weight` is a HOST pointer to a
  * row-major [rows, cols] T matrix; it is uploaded, quantised with quant_scale and
  * stored at device pointer quantized_weight as [rows, cols] (layout 0, kRowMajor)

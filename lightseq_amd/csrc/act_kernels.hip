@@ -7,23 +7,6 @@
 
 namespace lsh {
 
-enum ActKind { kGelu = 0, kRelu = 1, kReluNarrow = 2 };
-
-// tanh-form GELU (inference/kernels/common.h:17-23) written as x * sigmoid(2u):
-// 0.5 * (1 + tanh(u)) == 1 / (1 + exp(-2u)); one hardware exp and one reciprocal.
-__device__ __forceinline__ float gelu_sigmoid_form(float x) {
-  float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-  return x * __frcp_rn(1.0f + __expf(-2.0f * u));
-}
-
-template <int ACT>
-__device__ __forceinline__ int act_requant(float x, float qs, float clip_max) {
-  if (ACT == kGelu) return float2int8(gelu_sigmoid_form(x), qs);
-  float r = fmaxf(x, 0.f);
-  if (ACT == kReluNarrow) return posfloat2int8(r, qs, clip_max);
-  return float2int8(r, qs);
-}
-
 template <typename T, int ACT>
 __global__ void __launch_bounds__(256)
 bias_act16_kernel(const int8_t* __restrict__ in, int8_t* __restrict__ out,
@@ -44,7 +27,7 @@ bias_act16_kernel(const int8_t* __restrict__ in, int8_t* __restrict__ out,
       int q[4];
 #pragma unroll
       for (int k = 0; k < 4; ++k)
-        q[k] = act_requant<ACT>((float)unpack_i8(wi[g], k) * ds + b[k], qs, clip_max);
+        q[k] = dequant_bias_act_requant<ACT>(unpack_i8(wi[g], k), ds, b[k], qs, clip_max);
       wo[g] = pack4_i8(q[0], q[1], q[2], q[3]);
     }
     *reinterpret_cast<uint4*>(out + e) = make_uint4(wo[0], wo[1], wo[2], wo[3]);
@@ -58,8 +41,8 @@ __global__ void bias_act1_kernel(const int8_t* __restrict__ in, int8_t* __restri
   long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const long stride = (long)gridDim.x * blockDim.x;
   for (; i < n; i += stride) {
-    float x = (float)in[i] * ds + TT<T>::ld(bias, i % feat);
-    out[i] = (int8_t)act_requant<ACT>(x, qs, clip_max);
+    out[i] = (int8_t)dequant_bias_act_requant<ACT>((int)in[i], ds, TT<T>::ld(bias, i % feat), qs,
+                                                   clip_max);
   }
 }
 
@@ -90,7 +73,7 @@ static int launch_bias_act(int tokens, hipStream_t s, const int8_t* input, int8_
 template <typename T>
 int bias_gelu_i8I_i8O(int tokens, hipStream_t s, const int8_t* input, int8_t* output,
                       const T* bias, int feature_dim, float dequant_scale, float quant_scale) {
-  return launch_bias_act<T, kGelu>(tokens, s, input, output, bias, feature_dim, dequant_scale,
+  return launch_bias_act<T, kActGelu>(tokens, s, input, output, bias, feature_dim, dequant_scale,
                                    quant_scale, 0.f);
 }
 
@@ -99,9 +82,9 @@ int bias_relu_i8I_i8O(int tokens, hipStream_t s, const int8_t* input, int8_t* ou
                       const T* bias, int feature_dim, float dequant_scale, float quant_scale,
                       float clip_max, bool narrow_clip) {
   if (narrow_clip)
-    return launch_bias_act<T, kReluNarrow>(tokens, s, input, output, bias, feature_dim,
+    return launch_bias_act<T, kActReluNarrow>(tokens, s, input, output, bias, feature_dim,
                                            dequant_scale, quant_scale, clip_max);
-  return launch_bias_act<T, kRelu>(tokens, s, input, output, bias, feature_dim, dequant_scale,
+  return launch_bias_act<T, kActRelu>(tokens, s, input, output, bias, feature_dim, dequant_scale,
                                    quant_scale, clip_max);
 }
 

@@ -75,7 +75,8 @@ arrange_qkv_kernel(const int8_t* __restrict__ ori, const T* __restrict__ bias,
       if (!I8OUT) {
         // fp16: T(x * ds) + bias as a half add; fp32: float add (rnd is the identity)
 #pragma unroll
-        for (int k = 0; k < 8; ++k) x[k] = TT<T>::rnd(x[k] * ds) + bv[k];
+        for (int k = 0; k < 8; ++k)
+          x[k] = TT<T>::is_half ? dequant_add_bias_h((int)x[k], ds, bv[k]) : x[k] * ds + bv[k];
         st8(new_qkv, max_batch_dim * which + target, x);
       } else {
 #pragma unroll

@@ -2,6 +2,7 @@
 // dispatch on the storage type.  No kernel code lives here.
 #include <string>
 
+#include "ls_device.cuh"
 #include "ls_launch.h"
 
 namespace lsh {
@@ -324,6 +325,27 @@ int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n,
 int lsh_gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int m, int n, int k, float alpha,
                     lsh_stream_t stream) {
   return gemm_i8_i8o(A, W, C, m, n, k, alpha, HS(stream));
+}
+int lsh_gemm_i8_bias_gelu_i8o_f16(const int8_t* A, const int8_t* W, int8_t* C, const void* bias,
+                                  int m, int n, int k, float alpha, float dequant_scale,
+                                  float quant_scale, lsh_stream_t stream) {
+  return gemm_i8_bias_act_i8o(A, W, C, H(bias), m, n, k, alpha, dequant_scale, quant_scale, 0.f,
+                              kActGelu, HS(stream));
+}
+int lsh_gemm_i8_bias_relu_i8o_f16(const int8_t* A, const int8_t* W, int8_t* C, const void* bias,
+                                  int m, int n, int k, float alpha, float dequant_scale,
+                                  float quant_scale, float clip_max, int narrow_clip,
+                                  lsh_stream_t stream) {
+  return gemm_i8_bias_act_i8o(A, W, C, H(bias), m, n, k, alpha, dequant_scale, quant_scale,
+                              clip_max, narrow_clip ? kActReluNarrow : kActRelu, HS(stream));
+}
+int lsh_gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, void* new_qkv,
+                                const void* qkv_bias, int max_batch_dim, int batch_token_num,
+                                int hidden_size, int k, int batch_seq_len, int head_num,
+                                float alpha, float dequant_scale, lsh_stream_t stream) {
+  return gemm_i8_qkv_arrange_f16(A, W, HM(new_qkv), H(qkv_bias), max_batch_dim, batch_token_num,
+                                 hidden_size, k, batch_seq_len, head_num, alpha, dequant_scale,
+                                 HS(stream));
 }
 int lsh_quantize_weight_f16(const void* origin_weight, int8_t* quantized_weight, int rows,
                             int cols, float quant_scale, lsh_stream_t stream, int layout) {

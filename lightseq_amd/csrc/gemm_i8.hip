@@ -1,21 +1,33 @@
 // int8 x int8 -> int32 GEMM on the gfx950 matrix cores (v_mfma_i32_32x32x32_i8),
-// with optional requantising epilogue.
+// with requantising and fused epilogues.
 //
 //   C[M,N] = epilogue( sum_k A[M,k] * W[N,k] )        A, W: K-contiguous int8
 //
 // Replaces the cuBLASLt int8 GEMMs and their tuned-algorithm table
 // (inference/model/cublas_helper.cc:31-225,361-489, cublas_algo_map.cc).
 //
-// Tiling.  A workgroup of 256 threads (4 wavefronts, 2x2) owns a BM x BN tile of C
-// and walks K in steps of 128 bytes.  Both operand tiles are staged in LDS,
-// double buffered, as rows of 128 bytes whose eight 16-byte chunks are XOR
-// swizzled so that the 16-byte per-lane MFMA operand reads are bank-conflict free.
-// The W tile is the MFMA "A" operand and the activation tile the "B" operand, so
-// that consecutive accumulator registers of a lane run along N; the W rows fed to
-// the MFMA are permuted so that the 16 accumulators of a lane are 16 *adjacent*
-// columns of C (one 16-byte store for int8 output).
+// Two kernels share the tile geometry and the epilogues:
+//
+//  * gemm_i8_stream_kernel -- the fast path (K % 128 == 0).  Persistent: 2 workgroups
+//    per compute unit walk a list of 128x128 tiles; operand stages (128 rows x 128 B
+//    each for A and W) are brought from L2 straight into LDS with
+//    global_load_lds_dwordx4 (no VGPR staging) into a 2-stage ring, and the prefetch
+//    cursor runs ahead of the compute cursor across tile boundaries, so a tile's first
+//    loads are in flight while the previous tile is still in its K loop / epilogue.
+//  * gemm_i8_generic_kernel -- any K % 16 == 0, any alignment of M and N: register
+//    staged, zero-filled tails, one tile per workgroup.
+//
+// Common geometry.  256 threads = 4 wavefronts (2x2), 64x64 accumulators per wavefront
+// as 2x2 MFMA blocks.  LDS rows are 128 B = eight 16-byte chunks, XOR swizzled for the
+// 64-bank LDS (a ds_read_b128 is served 16 lanes per clock; the 16 lanes must hit 16
+// distinct 16-byte slots of a 256-byte window).  The W tile is the MFMA "A" operand so
+// that consecutive accumulator registers of a lane run along N, and the W rows fed to
+// the MFMA are permuted (sigma) so that the 16 accumulators of a lane are 16 adjacent
+// columns of C: one 16-byte store for int8 output, two for fp16.
 #include "ls_device.cuh"
 #include "ls_launch.h"
+
+#include <hip/hip_ext.h>
 
 #include <string>
 
@@ -25,14 +37,20 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kBK = 128;  // bytes of K per LDS stage
+constexpr int kBM = 128, kBN = 128;
 
-// swizzle keys (3 bits) of a tile row
-__device__ __forceinline__ int key_act(int row) { return row & 7; }
-__device__ __forceinline__ int key_wgt(int row) { return (row & 3) | (((row >> 4) & 1) << 2); }
+// swizzle keys (3 bits) of a tile row, for the activation tile (rows read in natural
+// order) and the weight tile (rows read in sigma order)
+__device__ __forceinline__ int key_act(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int key_wgt(int row) { return ((row >> 1) & 3) | (((row >> 4) & 1) << 2); }
 // MFMA row r (0..31) of the weight operand -> local column of C, chosen so that the
 // accumulators c[0..15] of lane (l%32, g=l/32) are columns 16g .. 16g+15.
 __device__ __forceinline__ int sigma(int r) { return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3); }
 
+// ---------------------------------------------------------------------------------
+// Epilogues.  store16(m, n, N, c, full): c[0..15] are C[m, n .. n+15]; `full` means all
+// 16 columns exist and the vector path may be used.
+// ---------------------------------------------------------------------------------
 struct EpiI32 {
   int32_t* C;
   __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
@@ -48,40 +66,269 @@ struct EpiI32 {
         if (n + i < N) p[i] = c[i];
     }
   }
-  __host__ __device__ static bool vec_ok(int N, const void* C) {
-    return N % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
-  }
+  bool vec_ok(int N) const { return N % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
+  static const char* name() { return "EpiI32"; }
 };
+
+__device__ __forceinline__ void store16_i8(int8_t* p, int n, int N, const int (&q)[16], bool full) {
+  if (full) {
+    uint4 o;
+    o.x = pack4_i8(q[0], q[1], q[2], q[3]);
+    o.y = pack4_i8(q[4], q[5], q[6], q[7]);
+    o.z = pack4_i8(q[8], q[9], q[10], q[11]);
+    o.w = pack4_i8(q[12], q[13], q[14], q[15]);
+    *reinterpret_cast<uint4*>(p) = o;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (n + i < N) p[i] = (int8_t)q[i];
+  }
+}
 
 struct EpiI8 {
   int8_t* C;
   float alpha;
   __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
-    int8_t* p = C + m * N + n;
-    if (full) {
-      uint4 o;
-      o.x = pack4_i8(requant_acc(c[0], alpha), requant_acc(c[1], alpha), requant_acc(c[2], alpha),
-                     requant_acc(c[3], alpha));
-      o.y = pack4_i8(requant_acc(c[4], alpha), requant_acc(c[5], alpha), requant_acc(c[6], alpha),
-                     requant_acc(c[7], alpha));
-      o.z = pack4_i8(requant_acc(c[8], alpha), requant_acc(c[9], alpha),
-                     requant_acc(c[10], alpha), requant_acc(c[11], alpha));
-      o.w = pack4_i8(requant_acc(c[12], alpha), requant_acc(c[13], alpha),
-                     requant_acc(c[14], alpha), requant_acc(c[15], alpha));
-      *reinterpret_cast<uint4*>(p) = o;
-    } else {
+    int q[16];
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (n + i < N) p[i] = (int8_t)requant_acc(c[i], alpha);
-    }
+    for (int i = 0; i < 16; ++i) q[i] = requant_acc(c[i], alpha);
+    store16_i8(C + m * N + n, n, N, q, full);
   }
-  __host__ __device__ static bool vec_ok(int N, const void* C) {
-    return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0;
-  }
+  bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
+  static const char* name() { return "EpiI8"; }
 };
 
-// Load one BK-wide stage of a ROWS-row tile (row stride K bytes in HBM) into
-// registers: ROWS*8 chunks of 16 B spread over 256 threads.
+// requantise to the GEMM's int8 output code, then dequant + bias + activation +
+// requant exactly as the stand-alone bias/activation kernel would on that code.
+template <int ACT>
+struct EpiActI8 {
+  int8_t* C;
+  const __half* bias;
+  float alpha, dequant_scale, quant_scale, clip_max;
+  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
+    float b[16];
+    if (full) {  // n % 16 == 0 here, so the two 16-byte bias loads are aligned when bias is
+      const half8_t b0 = *reinterpret_cast<const half8_t*>(bias + n);
+      const half8_t b1 = *reinterpret_cast<const half8_t*>(bias + n + 8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        b[i] = __half2float(b0.v[i]);
+        b[8 + i] = __half2float(b1.v[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) b[i] = n + i < N ? __half2float(bias[n + i]) : 0.f;
+    }
+    int q[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      q[i] = dequant_bias_act_requant<ACT>(requant_acc(c[i], alpha), dequant_scale, b[i],
+                                           quant_scale, clip_max);
+    store16_i8(C + m * N + n, n, N, q, full);
+  }
+  bool vec_ok(int N) const {
+    return N % 16 == 0 &&
+           ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(bias)) & 15u) == 0;
+  }
+  static const char* name() { return ACT == kActGelu ? "EpiGeluI8" : "EpiReluI8"; }
+};
+
+// requantise to the GEMM's int8 output code, then dequant + bias and scatter into the
+// three [B, h, S, d] fp16 tensors exactly as the QKV arrange kernel would.
+// Requires N == 3*h*d, d % 16 == 0.
+struct EpiQkvF16 {
+  __half* qkv;
+  const __half* bias;
+  long max_batch_dim;
+  float alpha, dequant_scale;
+  int seq_len, head_num, dim_per_head;
+  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool) const {
+    const int hidden = head_num * dim_per_head;
+    const int which = n / hidden, i = n - which * hidden;
+    const int head = i / dim_per_head, dim = i - head * dim_per_head;
+    const int b = (int)(m / seq_len), s = (int)(m - (long)b * seq_len);
+    __half* dst = qkv + max_batch_dim * which +
+                  (((long)b * head_num + head) * seq_len + s) * dim_per_head + dim;
+    const half8_t b0 = *reinterpret_cast<const half8_t*>(bias + n);
+    const half8_t b1 = *reinterpret_cast<const half8_t*>(bias + n + 8);
+    half8_t lo, hi;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      lo.v[k] = __float2half_rn(dequant_add_bias_h(requant_acc(c[k], alpha), dequant_scale,
+                                                   __half2float(b0.v[k])));
+      hi.v[k] = __float2half_rn(dequant_add_bias_h(requant_acc(c[8 + k], alpha), dequant_scale,
+                                                   __half2float(b1.v[k])));
+    }
+    *reinterpret_cast<half8_t*>(dst) = lo;
+    *reinterpret_cast<half8_t*>(dst + 8) = hi;
+    (void)N;
+  }
+  bool vec_ok(int) const { return true; }
+  static const char* name() { return "EpiQkvF16"; }
+};
+
+template <typename Epi, int MB, int NB>
+__device__ __forceinline__ void store_tile_acc(const Epi& epi, const v16i (&acc)[MB][NB], int m0,
+                                               int n0, int wm, int wn, int l32, int g, int M, int N,
+                                               bool vec_store) {
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const long m = m0 + wm * (MB * 32) + i * 32 + l32;
+    if (m < M) {
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int n = n0 + wn * (NB * 32) + j * 32 + 16 * g;
+        if (n < N) epi.store16(m, n, N, acc[i][j], vec_store && n + 16 <= N);
+      }
+    }
+  }
+}
+
+// linear work index -> tile.  Workgroups (and the persistent kernel's work items) are
+// dealt round-robin to the 8 XCDs; renumber so that each XCD (own L2) works on a
+// contiguous run of tiles, walked in column-major order of 8-tile-tall groups so that a
+// run shares W columns and A rows.
+__device__ __forceinline__ void tile_of(int t, int nblk, int tiles_m, int tiles_n, int& tile_m,
+                                        int& tile_n) {
+  const int per = nblk / 8, rem = nblk % 8;
+  const int xcd = t % 8, loc = t / 8;
+  const int pid = xcd * per + (xcd < rem ? xcd : rem) + loc;
+  constexpr int GROUP = 8;
+  const int group_sz = GROUP * tiles_n;
+  const int first_m = (pid / group_sz) * GROUP;
+  const int gm = min(tiles_m - first_m, GROUP);
+  tile_m = first_m + (pid % group_sz) % gm;
+  tile_n = (pid % group_sz) / gm;
+}
+
+// ---------------------------------------------------------------------------------
+// Fast path: persistent, direct-to-LDS, 2-stage ring, cross-tile prefetch.
+// Preconditions (checked by the dispatcher): K % 128 == 0, (rows-1)*K + 128 < 2^32 for
+// both operands, operands 16-byte aligned.
+// ---------------------------------------------------------------------------------
+template <typename Epi>
+__global__ void __launch_bounds__(256)
+gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
+                      int N, int K, int tiles_m, int tiles_n, bool vec_store) {
+  constexpr int NST = 2;
+  constexpr int STAGE = (kBM + kBN) * kBK;  // 32 KB: A tile then W tile
+  constexpr int NA = kBM / 32, NW = kBN / 32;  // 1-KB DMA instructions per wavefront per stage
+  extern __shared__ __align__(16) int8_t smem[];
+  const int nblk = tiles_m * tiles_n;
+  const int G = gridDim.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, g = lane >> 5;
+  const int my_tiles = (nblk - (int)blockIdx.x + G - 1) / G;
+  const int nk = K / kBK;
+
+  // DMA sources: each instruction moves 8 rows x 128 B; lane i lands in LDS slot i of that
+  // 1-KB block, so it fetches the chunk the swizzle puts there.  Row clamping keeps the
+  // reads of partial tiles in bounds (the clamped rows are never stored).
+  uint32_t a_src[NA], w_src[NW];
+  auto set_src = [&](int j) {
+    int tm, tn;
+    tile_of(blockIdx.x + j * G, nblk, tiles_m, tiles_n, tm, tn);
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int row = (wave + 4 * i) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ key_act(row);
+      a_src[i] = (uint32_t)min(tm * kBM + row, M - 1) * (uint32_t)K + c * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int row = (wave + 4 * i) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ key_wgt(row);
+      w_src[i] = (uint32_t)min(tn * kBN + row, N - 1) * (uint32_t)K + c * 16;
+    }
+  };
+  const uint32_t lds0 =
+      (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+  // Issued through inline asm so that the compiler's wait-count insertion does not see an
+  // outstanding LDS write and drain vmcnt before every ds_read; the waits are explicit.
+  auto dma1 = [&](const int8_t* base, uint32_t voff, uint32_t lds) {
+    lds = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff),
+                 "s"(base)
+                 : "memory");
+  };
+  int p_j = 0, p_kt = 0, p_st = 0;  // prefetch cursor: tile, K step, ring slot
+  auto issue_next = [&]() {
+    if (p_j < my_tiles) {
+      const uint32_t base = lds0 + p_st * STAGE;
+#pragma unroll
+      for (int i = 0; i < NA; ++i) dma1(A + p_kt * kBK, a_src[i], base + (wave + 4 * i) * 1024);
+#pragma unroll
+      for (int i = 0; i < NW; ++i)
+        dma1(W + p_kt * kBK, w_src[i], base + kBM * kBK + (wave + 4 * i) * 1024);
+      if (++p_kt == nk) {
+        p_kt = 0;
+        if (++p_j < my_tiles) set_src(p_j);
+      }
+      p_st ^= 1;
+    }
+  };
+
+  int a_off[2], w_off[2], a_key[2], w_key[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = wm * 64 + i * 32 + l32;
+    a_off[i] = row * kBK;
+    a_key[i] = key_act(row);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int row = wn * 64 + j * 32 + sigma(l32);
+    w_off[j] = kBM * kBK + row * kBK;
+    w_key[j] = key_wgt(row);
+  }
+
+  if (my_tiles > 0) set_src(0);
+  issue_next();
+  int st = 0;
+  for (int j = 0; j < my_tiles; ++j) {
+    int tm, tn;
+    tile_of(blockIdx.x + j * G, nblk, tiles_m, tiles_n, tm, tn);
+    v16i acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj) acc[i][jj] = (v16i)0;
+    for (int kt = 0; kt < nk; ++kt) {
+      // stage `st` has landed for this wavefront ...
+      __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0)
+      // ... and for everyone; everyone is also done reading the other stage
+      __builtin_amdgcn_s_barrier();
+      issue_next();
+      const int8_t* stage = smem + st * STAGE;
+      v4i bv[kBK / 32][2], av[kBK / 32][2];
+#pragma unroll
+      for (int ks = 0; ks < kBK / 32; ++ks) {
+        const int chunk = 2 * ks + g;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          bv[ks][i] = *reinterpret_cast<const v4i*>(stage + a_off[i] + ((chunk ^ a_key[i]) << 4));
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj)
+          av[ks][jj] = *reinterpret_cast<const v4i*>(stage + w_off[jj] + ((chunk ^ w_key[jj]) << 4));
+      }
+#pragma unroll
+      for (int ks = 0; ks < kBK / 32; ++ks)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj)
+            acc[i][jj] =
+                __builtin_amdgcn_mfma_i32_32x32x32_i8(av[ks][jj], bv[ks][i], acc[i][jj], 0, 0, 0);
+      st ^= 1;
+    }
+    store_tile_acc<Epi, 2, 2>(epi, acc, tm * kBM, tn * kBN, wm, wn, l32, g, M, N, vec_store);
+  }
+  __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
+}
+
+// ---------------------------------------------------------------------------------
+// Generic path: register-staged double buffering, zero-filled tails.
+// ---------------------------------------------------------------------------------
 template <int ROWS>
 __device__ __forceinline__ void load_tile(const int8_t* __restrict__ base, int row0, int nrows,
                                           int K, int k0, int tid, v4i (&regs)[ROWS / 32]) {
@@ -107,63 +354,43 @@ __device__ __forceinline__ void store_tile(int8_t* lds, int tid, const v4i (&reg
   }
 }
 
-template <int BM, int BN, typename Epi>
+template <typename Epi>
 __global__ void __launch_bounds__(256)
-gemm_i8_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M, int N,
-               int K, int tiles_m, int tiles_n, bool vec_store) {
-  constexpr int TM = BM / 2, TN = BN / 2;      // wavefront tile
-  constexpr int MB = TM / 32, NB = TN / 32;    // MFMA blocks per wavefront tile
+gemm_i8_generic_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
+                       int N, int K, int tiles_m, int tiles_n, bool vec_store) {
+  constexpr int kStage = (kBM + kBN) * kBK;
   extern __shared__ __align__(16) int8_t smem[];
-  constexpr int kStage = (BM + BN) * kBK;  // bytes per LDS stage: A tile then W tile
-
-  // Workgroups are dealt round-robin to the 8 XCDs; renumber them so that each XCD
-  // (own L2) works on a contiguous run of tiles, and walk tiles in column-major
-  // order of 8-tile-tall groups so a run shares W columns and A rows.
-  const int nblk = tiles_m * tiles_n;
-  int pid = blockIdx.x;
-  {
-    const int per = nblk / 8, rem = nblk % 8;
-    const int xcd = pid % 8, loc = pid / 8;
-    pid = xcd * per + (xcd < rem ? xcd : rem) + loc;
-  }
-  constexpr int GROUP = 8;
-  const int group_sz = GROUP * tiles_n;
-  const int gid = pid / group_sz;
-  const int first_m = gid * GROUP;
-  const int gm = min(tiles_m - first_m, GROUP);
-  const int tile_m = first_m + (pid % group_sz) % gm;
-  const int tile_n = (pid % group_sz) / gm;
-
+  int tile_m, tile_n;
+  tile_of(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tile_m, tile_n);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int l32 = lane & 31, g = lane >> 5;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int m0 = tile_m * kBM, n0 = tile_n * kBN;
 
-  v16i acc[MB][NB];
+  v16i acc[2][2];
 #pragma unroll
-  for (int i = 0; i < MB; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < NB; ++j) acc[i][j] = (v16i)0;
+    for (int j = 0; j < 2; ++j) acc[i][j] = (v16i)0;
 
-  v4i ra[BM / 32], rw[BN / 32];
+  v4i ra[kBM / 32], rw[kBN / 32];
   const int nk = (K + kBK - 1) / kBK;
-  load_tile<BM>(A, m0, M, K, 0, tid, ra);
-  load_tile<BN>(W, n0, N, K, 0, tid, rw);
-  store_tile<BM, false>(smem, tid, ra);
-  store_tile<BN, true>(smem + BM * kBK, tid, rw);
+  load_tile<kBM>(A, m0, M, K, 0, tid, ra);
+  load_tile<kBN>(W, n0, N, K, 0, tid, rw);
+  store_tile<kBM, false>(smem, tid, ra);
+  store_tile<kBN, true>(smem + kBM * kBK, tid, rw);
   __syncthreads();
 
-  // per-lane LDS row offsets of the MFMA operands
-  int a_off[MB], w_off[NB], a_key[MB], w_key[NB];
+  int a_off[2], w_off[2], a_key[2], w_key[2];
 #pragma unroll
-  for (int i = 0; i < MB; ++i) {
-    const int row = wm * TM + i * 32 + l32;
+  for (int i = 0; i < 2; ++i) {
+    const int row = wm * 64 + i * 32 + l32;
     a_off[i] = row * kBK;
     a_key[i] = key_act(row);
   }
 #pragma unroll
-  for (int j = 0; j < NB; ++j) {
-    const int row = wn * TN + j * 32 + sigma(l32);
+  for (int j = 0; j < 2; ++j) {
+    const int row = wn * 64 + j * 32 + sigma(l32);
     w_off[j] = row * kBK;
     w_key[j] = key_wgt(row);
   }
@@ -171,115 +398,153 @@ gemm_i8_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi e
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
     if (kt + 1 < nk) {
-      load_tile<BM>(A, m0, M, K, (kt + 1) * kBK, tid, ra);
-      load_tile<BN>(W, n0, N, K, (kt + 1) * kBK, tid, rw);
+      load_tile<kBM>(A, m0, M, K, (kt + 1) * kBK, tid, ra);
+      load_tile<kBN>(W, n0, N, K, (kt + 1) * kBK, tid, rw);
     }
     const int8_t* pa = smem + cur * kStage;
-    const int8_t* pw = pa + BM * kBK;
+    const int8_t* pw = pa + kBM * kBK;
 #pragma unroll
     for (int ks = 0; ks < kBK / 32; ++ks) {
       const int chunk = 2 * ks + g;
-      v4i bv[MB], av[NB];
+      v4i bv[2], av[2];
 #pragma unroll
-      for (int i = 0; i < MB; ++i)
+      for (int i = 0; i < 2; ++i)
         bv[i] = *reinterpret_cast<const v4i*>(pa + a_off[i] + ((chunk ^ a_key[i]) << 4));
 #pragma unroll
-      for (int j = 0; j < NB; ++j)
+      for (int j = 0; j < 2; ++j)
         av[j] = *reinterpret_cast<const v4i*>(pw + w_off[j] + ((chunk ^ w_key[j]) << 4));
 #pragma unroll
-      for (int i = 0; i < MB; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
+        for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[j], bv[i], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < nk) {
       int8_t* nxt = smem + (cur ^ 1) * kStage;
-      store_tile<BM, false>(nxt, tid, ra);
-      store_tile<BN, true>(nxt + BM * kBK, tid, rw);
+      store_tile<kBM, false>(nxt, tid, ra);
+      store_tile<kBN, true>(nxt + kBM * kBK, tid, rw);
     }
     __syncthreads();
   }
-
-#pragma unroll
-  for (int i = 0; i < MB; ++i) {
-    const long m = m0 + wm * TM + i * 32 + l32;
-    if (m < M) {
-#pragma unroll
-      for (int j = 0; j < NB; ++j) {
-        const int n = n0 + wn * TN + j * 32 + 16 * g;
-        if (n < N) epi.store16(m, n, N, acc[i][j], vec_store && n + 16 <= N);
-      }
-    }
-  }
+  store_tile_acc<Epi, 2, 2>(epi, acc, m0, n0, wm, wn, l32, g, M, N, vec_store);
 }
 
-template <int BM, int BN, typename Epi>
-static int launch_tile(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int K,
-                       bool vec_store, hipStream_t s) {
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  const size_t smem = 2 * (size_t)(BM + BN) * kBK;
-  auto kern = gemm_i8_kernel<BM, BN, Epi>;
-  static bool attr_set = false;  // per instantiation
-  if (!attr_set) {
+// ---------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------
+static thread_local hipEvent_t g_ev_start = nullptr, g_ev_stop = nullptr;
+
+void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop) {
+  g_ev_start = start;
+  g_ev_stop = stop;
+}
+
+static bool stream_ok(int M, int N, int K) {
+  if (K % kBK != 0) return false;
+  const unsigned long long lim = 0xffffffffull;
+  return (unsigned long long)(M - 1) * K + kBK < lim && (unsigned long long)(N - 1) * K + kBK < lim;
+}
+
+template <typename Kern, typename Epi>
+static int launch(Kern kern, int grid, size_t smem, const int8_t* A, const int8_t* W, Epi epi,
+                  int M, int N, int K, int tiles_m, int tiles_n, bool vec_store, hipStream_t s,
+                  bool* attr_set) {
+  if (!*attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return lsh_check_hip(e, "hipFuncSetAttribute(gemm_i8_kernel)");
-    attr_set = true;
+    if (e != hipSuccess) return lsh_check_hip(e, "hipFuncSetAttribute(gemm_i8)");
+    *attr_set = true;
   }
-  kern<<<tiles_m * tiles_n, 256, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store);
+  if (g_ev_start != nullptr) {
+    // kernel-exact begin/end timestamps on the launch stream
+    hipEvent_t e0 = g_ev_start, e1 = g_ev_stop;
+    g_ev_start = g_ev_stop = nullptr;
+    hipExtLaunchKernelGGL(kern, dim3(grid), dim3(256), (unsigned)smem, s, e0, e1, 0, A, W, epi, M,
+                          N, K, tiles_m, tiles_n, vec_store);
+  } else {
+    kern<<<grid, 256, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store);
+  }
   return lsh_check_launch("gemm_i8_kernel");
-}
-
-// Picks the tile that wastes the fewest matrix-core cycles on 256 compute units:
-// cost = (#rounds of 256 workgroups) x (work per tile), penalising small tiles for
-// their higher LDS traffic per MAC.  Returns an index into kTiles.
-struct TileCand { int bm, bn; double eff; };
-static const TileCand kTiles[3] = {{256, 256, 1.0}, {256, 128, 0.92}, {128, 128, 0.80}};
-
-static int select_tile(int M, int N) {
-  int best = 2;
-  double best_cost = 1e300;
-  for (int c = 0; c < 3; ++c) {
-    const long tiles =
-        (long)((M + kTiles[c].bm - 1) / kTiles[c].bm) * ((N + kTiles[c].bn - 1) / kTiles[c].bn);
-    const long rounds = (tiles + 255) / 256;
-    const double cost = (double)rounds * kTiles[c].bm * kTiles[c].bn / kTiles[c].eff;
-    if (cost < best_cost) { best_cost = cost; best = c; }
-  }
-  return best;
 }
 
 template <typename Epi>
 static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int K,
-                    const void* Cptr, hipStream_t s) {
-  if (M <= 0 || N <= 0 || K <= 0 || !A || !W || !Cptr)
+                    hipStream_t s) {
+  if (M <= 0 || N <= 0 || K <= 0 || !A || !W)
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: bad arguments");
   if (K % 16 != 0) return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: K must be a multiple of 16");
   if (((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) & 15u) != 0)
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: operands must be 16-byte aligned");
-  const bool vec_store = Epi::vec_ok(N, Cptr);
-  switch (select_tile(M, N)) {
-    case 0: return launch_tile<256, 256, Epi>(A, W, epi, M, N, K, vec_store, s);
-    case 1: return launch_tile<256, 128, Epi>(A, W, epi, M, N, K, vec_store, s);
-    default: return launch_tile<128, 128, Epi>(A, W, epi, M, N, K, vec_store, s);
+  const bool vec_store = epi.vec_ok(N);
+  const int tiles_m = (M + kBM - 1) / kBM, tiles_n = (N + kBN - 1) / kBN;
+  const int tiles = tiles_m * tiles_n;
+  const size_t smem = 2 * (size_t)(kBM + kBN) * kBK;
+  static bool attr_stream = false, attr_generic = false;  // per Epi instantiation
+  if (stream_ok(M, N, K)) {
+    const int grid = tiles < 512 ? tiles : 512;  // 2 resident workgroups per compute unit
+    return launch(gemm_i8_stream_kernel<Epi>, grid, smem, A, W, epi, M, N, K, tiles_m, tiles_n,
+                  vec_store, s, &attr_stream);
   }
+  return launch(gemm_i8_generic_kernel<Epi>, tiles, smem, A, W, epi, M, N, K, tiles_m, tiles_n,
+                vec_store, s, &attr_generic);
 }
 
-std::string gemm_i8_kernel_name(int M, int N, int K, bool int8_out) {
-  (void)K;
-  const TileCand& t = kTiles[select_tile(M, N)];
-  return "gemm_i8_kernel<" + std::to_string(t.bm) + "," + std::to_string(t.bn) + "," +
-         (int8_out ? "EpiI8" : "EpiI32") + ">";
+std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
+  return std::string(stream_ok(M, N, K) ? "gemm_i8_stream_kernel<" : "gemm_i8_generic_kernel<") +
+         epilogue + ">";
 }
 
 int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int K,
                  hipStream_t s) {
-  return dispatch(A, W, EpiI32{C}, M, N, K, C, s);
+  if (!C) return lsh_fail(LSH_ERR_INVALID, "int8 gemm: null output");
+  return dispatch(A, W, EpiI32{C}, M, N, K, s);
 }
 
 int gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K, float alpha,
                 hipStream_t s) {
-  return dispatch(A, W, EpiI8{C, alpha}, M, N, K, C, s);
+  if (!C) return lsh_fail(LSH_ERR_INVALID, "int8 gemm: null output");
+  return dispatch(A, W, EpiI8{C, alpha}, M, N, K, s);
+}
+
+int gemm_i8_bias_act_i8o(const int8_t* A, const int8_t* W, int8_t* C, const __half* bias, int M,
+                         int N, int K, float alpha, float dequant_scale, float quant_scale,
+                         float clip_max, int act, hipStream_t s) {
+  if (!C || !bias) return lsh_fail(LSH_ERR_INVALID, "int8 gemm (bias+act): null pointer");
+  switch (act) {
+    case kActGelu:
+      return dispatch(A, W, EpiActI8<kActGelu>{C, bias, alpha, dequant_scale, quant_scale, clip_max},
+                      M, N, K, s);
+    case kActRelu:
+      return dispatch(A, W, EpiActI8<kActRelu>{C, bias, alpha, dequant_scale, quant_scale, clip_max},
+                      M, N, K, s);
+    case kActReluNarrow:
+      return dispatch(A, W,
+                      EpiActI8<kActReluNarrow>{C, bias, alpha, dequant_scale, quant_scale, clip_max},
+                      M, N, K, s);
+    default:
+      return lsh_fail(LSH_ERR_INVALID, "int8 gemm (bias+act): unknown activation");
+  }
+}
+
+int gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, __half* new_qkv, const __half* qkv_bias,
+                            long max_batch_dim, int batch_tokens, int hidden, int K, int seq_len,
+                            int head_num, float alpha, float dequant_scale, hipStream_t s) {
+  if (!new_qkv || !qkv_bias || seq_len <= 0 || head_num <= 0 || hidden % head_num != 0 ||
+      batch_tokens % seq_len != 0 || max_batch_dim < (long)batch_tokens * hidden)
+    return lsh_fail(LSH_ERR_INVALID, "int8 gemm (qkv arrange): bad arguments");
+  const int d = hidden / head_num;
+  if (d % 16 != 0 || max_batch_dim % 8 != 0 ||
+      ((reinterpret_cast<uintptr_t>(new_qkv) | reinterpret_cast<uintptr_t>(qkv_bias)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "int8 gemm (qkv arrange): needs dim_per_head % 16 == 0 and aligned output");
+  return dispatch(A, W,
+                  EpiQkvF16{new_qkv, qkv_bias, max_batch_dim, alpha, dequant_scale, seq_len,
+                            head_num, d},
+                  batch_tokens, 3 * hidden, K, s);
+}
+
+const char* gemm_i8_act_epilogue_name(int act) {
+  return act == kActGelu ? EpiActI8<kActGelu>::name() : EpiActI8<kActRelu>::name();
 }
 
 }  // namespace lsh

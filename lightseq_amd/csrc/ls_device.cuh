@@ -62,6 +62,39 @@ __device__ __forceinline__ float gelu_tanh(float x) {
   return x * cdf;
 }
 
+// tanh-form GELU written as x * sigmoid(2u): 0.5 * (1 + tanh(u)) == 1 / (1 + exp(-2u));
+// one hardware exp and one reciprocal instead of a tanhf call.
+__device__ __forceinline__ float gelu_sigmoid_form(float x) {
+  float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return x * __frcp_rn(1.0f + __expf(-2.0f * u));
+}
+
+enum ActKind { kActGelu = 0, kActRelu = 1, kActReluNarrow = 2 };
+
+// int8 code -> dequant + bias -> activation -> int8 code
+// (inference/kernels/transformerKernels_int8.cc.cu:865-1078).  Shared by the stand-alone
+// kernel and the fused GEMM epilogue so both produce the same bits.
+template <int ACT>
+__device__ __forceinline__ int dequant_bias_act_requant(int q, float dequant_scale, float bias,
+                                                        float quant_scale, float clip_max) {
+  float x;
+  {
+#pragma clang fp contract(off)
+    x = (float)q * dequant_scale + bias;
+  }
+  if (ACT == kActGelu) return float2int8(gelu_sigmoid_form(x), quant_scale);
+  float r = fmaxf(x, 0.f);
+  if (ACT == kActReluNarrow) return posfloat2int8(r, quant_scale, clip_max);
+  return float2int8(r, quant_scale);
+}
+
+// fp16 head-split value: T(q * dequant_scale) + bias as a half add
+// (inference/kernels/transformerKernels_int8.cc.cu:1140-1145); the caller rounds the
+// returned float to fp16.
+__device__ __forceinline__ float dequant_add_bias_h(int q, float dequant_scale, float bias) {
+  return __half2float(__float2half_rn((float)q * dequant_scale)) + bias;
+}
+
 __device__ __forceinline__ uint32_t pack4_i8(int a, int b, int c, int d) {
   return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
          ((uint32_t)(d & 0xff) << 24);

@@ -99,7 +99,23 @@ int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int
                  hipStream_t s);
 int gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K, float alpha,
                 hipStream_t s);
-// Name of the kernel instantiation the dispatcher picks for a shape (for profiles).
-std::string gemm_i8_kernel_name(int M, int N, int K, bool int8_out);
+// Fused epilogues (fp16 models).  Each produces exactly the bits of the int8-output GEMM
+// followed by the stand-alone kernel it absorbs.
+//   act: ActKind (0 GELU, 1 ReLU, 2 ReLU with the narrow unsigned clip)
+int gemm_i8_bias_act_i8o(const int8_t* A, const int8_t* W, int8_t* C, const __half* bias, int M,
+                         int N, int K, float alpha, float dequant_scale, float quant_scale,
+                         float clip_max, int act, hipStream_t s);
+//   writes q, k, v as fp16 [B, h, S, d] at new_qkv + {0, 1, 2} * max_batch_dim
+int gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, __half* new_qkv,
+                            const __half* qkv_bias, long max_batch_dim, int batch_tokens,
+                            int hidden, int K, int seq_len, int head_num, float alpha,
+                            float dequant_scale, hipStream_t s);
+// Name of the kernel instantiation the dispatcher picks for a shape (for profiles);
+// epilogue is "EpiI8", "EpiI32", "EpiGeluI8", "EpiReluI8" or "EpiQkvF16".
+std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue);
+const char* gemm_i8_act_epilogue_name(int act);
+// The next int8 GEMM launched from this thread records kernel-exact begin / end
+// timestamps into the two events (hipExtLaunchKernelGGL), then the hook clears itself.
+void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop);
 
 }  // namespace lsh

@@ -1,5 +1,7 @@
 #include "quant_bert_encoder.h"
 
+#include "../ls_device.cuh"
+
 #include <algorithm>
 
 namespace lightseq {
@@ -115,12 +117,12 @@ void QuantBertEncoder::reset_profile() {
   for (auto& p : _profile) { p.launches = 0; p.total_ms = 0.0; }
 }
 
-void QuantBertEncoder::prof_begin(int site, int m, int n, int k, bool int8_out) {
+void QuantBertEncoder::prof_begin(int site, int m, int n, int k, const char* epilogue) {
   if (!_profiling) return;
   SiteProfile& p = _profile[site];
   if (p.m != m || p.n != n || p.k != k) {
     p.m = m; p.n = n; p.k = k;
-    p.kernel = gemm_i8_kernel_name(m, n, k, int8_out);
+    p.kernel = gemm_i8_kernel_name(m, n, k, epilogue);
   }
   Pending pe;
   pe.site = site;
@@ -132,13 +134,9 @@ void QuantBertEncoder::prof_begin(int site, int m, int n, int k, bool int8_out) 
       _event_pool.pop_back();
     }
   }
-  CHECK_GPU_ERROR(hipEventRecord(pe.e0, _stream));
+  // the GEMM launcher records the kernel's own begin / end timestamps into the events
+  gemm_i8_time_next_launch(pe.e0, pe.e1);
   _pending.push_back(pe);
-}
-
-void QuantBertEncoder::prof_end() {
-  if (!_profiling) return;
-  CHECK_GPU_ERROR(hipEventRecord(_pending.back().e1, _stream));
 }
 
 void QuantBertEncoder::collect_profile() {
@@ -191,17 +189,25 @@ void QuantBertEncoder::self_attention() {
   tap(taps.ln1_q, _int8_ffn_in_buf.get(), (size_t)M * H);
 
   // qkv = ori_q * qkv_wei, int8 out
-  prof_begin(0, M, 3 * H, H, true);
-  LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_qkv.get(), _int8_ffn_out_buf.get(), M, 3 * H, H,
-                       c[0] * c[4] / (c[8] * Q), _stream));
-  prof_end();
-  tap(taps.qkv_q, _int8_ffn_out_buf.get(), (size_t)M * 3 * H);
-
-  // dequant + bias, split heads -> fp16 q, k, v [B, h, S, d]
+  // qkv = ori_q * qkv_wei -> int8 code -> dequant + bias, split heads -> fp16 q, k, v
+  // [B, h, S, d].  Fused into the GEMM epilogue unless the int8 GEMM output is tapped
+  // (or the head size does not allow it); both routes give the same bits.
   const long mbd = (long)M * H;
-  LSH_CALL(arrange_encself_qkv_i8I<__half>(M, H, _stream, _int8_ffn_out_buf.get(), w.b_qkv.get(),
-                                           _qkv_buf.get(), mbd, _batch_seq_len, _tw._dim_per_head,
-                                           _tw._head_num, c[8] / Q));
+  const bool tap_qkv = taps.qkv_q && taps.tap_layer == _layer_id;
+  if (_fuse && !tap_qkv && _tw._dim_per_head % 16 == 0) {
+    prof_begin(0, M, 3 * H, H, "EpiQkvF16");
+    LSH_CALL(gemm_i8_qkv_arrange_f16(_int8_ffn_in_buf.get(), w.w_qkv.get(), _qkv_buf.get(),
+                                     w.b_qkv.get(), mbd, M, H, H, _batch_seq_len, _tw._head_num,
+                                     c[0] * c[4] / (c[8] * Q), c[8] / Q, _stream));
+  } else {
+    prof_begin(0, M, 3 * H, H, "EpiI8");
+    LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_qkv.get(), _int8_ffn_out_buf.get(), M, 3 * H,
+                         H, c[0] * c[4] / (c[8] * Q), _stream));
+    tap(taps.qkv_q, _int8_ffn_out_buf.get(), (size_t)M * 3 * H);
+    LSH_CALL(arrange_encself_qkv_i8I<__half>(M, H, _stream, _int8_ffn_out_buf.get(),
+                                             w.b_qkv.get(), _qkv_buf.get(), mbd, _batch_seq_len,
+                                             _tw._dim_per_head, _tw._head_num, c[8] / Q));
+  }
 
   // scores -> masked softmax -> context -> merge heads + quantise, one kernel
   LSH_CALL(encself_attention_f16(_qkv_buf.get(), _qkv_buf.get() + mbd, _qkv_buf.get() + 2 * mbd,
@@ -210,10 +216,9 @@ void QuantBertEncoder::self_attention() {
                                  _stream));
   tap(taps.ctx_q, _int8_ffn_in_buf.get(), (size_t)M * H);
 
-  prof_begin(1, M, H, H, true);
+  prof_begin(1, M, H, H, "EpiI8");
   LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_out.get(), _int8_ffn_out_buf.get(), M, H, H,
                        c[1] * c[5] / (c[9] * Q), _stream));
-  prof_end();
   tap(taps.out_q, _int8_ffn_out_buf.get(), (size_t)M * H);
 
   if (taps.res_attn && taps.tap_layer == _layer_id)
@@ -232,25 +237,38 @@ void QuantBertEncoder::ffn_add_norm() {
   const float* c = &_enc_clip_max[_layer_id * 11];
   const float Q = _quant_range;
 
-  prof_begin(2, M, I, H, true);
-  LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_ffn1.get(), _int8_ffn_out_buf.get(), M, I, H,
-                       c[2] * c[6] / (c[10] * Q), _stream));
-  prof_end();
-  tap(taps.ffn1_q, _int8_ffn_out_buf.get(), (size_t)M * I);
-
-  if (_tw._use_gelu) {
-    LSH_CALL(bias_gelu_i8I_i8O<__half>(M, _stream, _int8_ffn_out_buf.get(), _int8_ffn_in_buf.get(),
-                                       w.b_ffn1.get(), I, c[10] / Q, Q / c[7]));
+  // FFN1 -> int8 code -> dequant + bias + activation + requant.  Fused into the GEMM
+  // epilogue unless the int8 GEMM output is tapped; both routes give the same bits.
+  // The fused GEMM reads _int8_ffn_in_buf and must not overwrite it: it writes to
+  // _int8_ffn_out_buf and the two buffers swap roles for the rest of the layer.
+  const bool tap_ffn1 = taps.ffn1_q && taps.tap_layer == _layer_id;
+  const int act = _tw._use_gelu ? kActGelu : kActReluNarrow;
+  int8_t* act_buf = _int8_ffn_in_buf.get();
+  if (_fuse && !tap_ffn1) {
+    prof_begin(2, M, I, H, gemm_i8_act_epilogue_name(act));
+    LSH_CALL(gemm_i8_bias_act_i8o(_int8_ffn_in_buf.get(), w.w_ffn1.get(), _int8_ffn_out_buf.get(),
+                                  w.b_ffn1.get(), M, I, H, c[2] * c[6] / (c[10] * Q), c[10] / Q,
+                                  Q / c[7], c[7], act, _stream));
+    act_buf = _int8_ffn_out_buf.get();
   } else {
-    LSH_CALL(bias_relu_i8I_i8O<__half>(M, _stream, _int8_ffn_out_buf.get(), _int8_ffn_in_buf.get(),
-                                       w.b_ffn1.get(), I, c[10] / Q, Q / c[7], c[7], true));
+    prof_begin(2, M, I, H, "EpiI8");
+    LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_ffn1.get(), _int8_ffn_out_buf.get(), M, I, H,
+                         c[2] * c[6] / (c[10] * Q), _stream));
+    tap(taps.ffn1_q, _int8_ffn_out_buf.get(), (size_t)M * I);
+    if (_tw._use_gelu) {
+      LSH_CALL(bias_gelu_i8I_i8O<__half>(M, _stream, _int8_ffn_out_buf.get(),
+                                         _int8_ffn_in_buf.get(), w.b_ffn1.get(), I, c[10] / Q,
+                                         Q / c[7]));
+    } else {
+      LSH_CALL(bias_relu_i8I_i8O<__half>(M, _stream, _int8_ffn_out_buf.get(),
+                                         _int8_ffn_in_buf.get(), w.b_ffn1.get(), I, c[10] / Q,
+                                         Q / c[7], c[7], true));
+    }
   }
-  tap(taps.act_q, _int8_ffn_in_buf.get(), (size_t)M * I);
+  tap(taps.act_q, act_buf, (size_t)M * I);
 
-  prof_begin(3, M, H, I, false);
-  LSH_CALL(gemm_i8_i32o(_int8_ffn_in_buf.get(), w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I,
-                        _stream));
-  prof_end();
+  prof_begin(3, M, H, I, "EpiI32");
+  LSH_CALL(gemm_i8_i32o(act_buf, w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I, _stream));
   if (taps.ffn2_acc && taps.tap_layer == _layer_id)
     CHECK_GPU_ERROR(hipMemcpyAsync(taps.ffn2_acc, _int32_ffn_out_buf.get(),
                                    (size_t)M * H * sizeof(int32_t), hipMemcpyDeviceToDevice,

@@ -46,6 +46,7 @@ class QuantBertEncoder {
     double total_ms = 0.0;
   };
   void set_profiling(bool on);
+  void set_fusion(bool on) { _fuse = on; }
   void collect_profile();
   void reset_profile();
   const std::vector<SiteProfile>& profile() const { return _profile; }
@@ -59,9 +60,9 @@ class QuantBertEncoder {
   void ffn_add_norm();
   void tap(int8_t* dst, const int8_t* src, size_t n);
   // event bracket around one GEMM launch of `site` (0 qkv, 1 out, 2 ffn1, 3 ffn2)
-  void prof_begin(int site, int m, int n, int k, bool int8_out);
-  void prof_end();
+  void prof_begin(int site, int m, int n, int k, const char* epilogue);
   bool _profiling = false;
+  bool _fuse = true;  // use the fused GEMM epilogues (QKV arrange, FFN1 bias+activation)
   std::vector<SiteProfile> _profile;
   struct Pending { int site; hipEvent_t e0, e1; };
   std::vector<Pending> _pending;

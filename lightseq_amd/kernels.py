@@ -169,6 +169,30 @@ def gemm_i8_i8o(a, w, c, m, n, k, alpha):
     call("lsh_gemm_i8_i8o", ptr(a), ptr(w), ptr(c), m, n, k, alpha, current_stream())
 
 
+def gemm_i8_bias_gelu_i8o(a, w, c, bias, m, n, k, alpha, dequant_scale, quant_scale):
+    """int8-output GEMM fused with ker_bias_gelu_i8I_i8O (fp16 bias)."""
+    _dev(a, w, c, bias)
+    call("lsh_gemm_i8_bias_gelu_i8o_f16", ptr(a), ptr(w), ptr(c), ptr(bias), m, n, k, alpha,
+         dequant_scale, quant_scale, current_stream())
+
+
+def gemm_i8_bias_relu_i8o(a, w, c, bias, m, n, k, alpha, dequant_scale, quant_scale, clip_max,
+                          narrow_clip):
+    """int8-output GEMM fused with ker_bias_relu_i8I_i8O (fp16 bias)."""
+    _dev(a, w, c, bias)
+    call("lsh_gemm_i8_bias_relu_i8o_f16", ptr(a), ptr(w), ptr(c), ptr(bias), m, n, k, alpha,
+         dequant_scale, quant_scale, clip_max, int(narrow_clip), current_stream())
+
+
+def gemm_i8_qkv_arrange(a, w, new_qkv, qkv_bias, max_batch_dim, batch_token_num, hidden_size, k,
+                        batch_seq_len, head_num, alpha, dequant_scale):
+    """QKV int8-output GEMM fused with ker_arrange_encself_qkv_i8I (fp16)."""
+    _dev(a, w, new_qkv, qkv_bias)
+    call("lsh_gemm_i8_qkv_arrange_f16", ptr(a), ptr(w), ptr(new_qkv), ptr(qkv_bias), max_batch_dim,
+         batch_token_num, hidden_size, k, batch_seq_len, head_num, alpha, dequant_scale,
+         current_stream())
+
+
 def quantize_weight(host_weight, dev_q, rows, cols, quant_scale, layout):
     """``host_weight``: CPU tensor [rows, cols]; layout 0 = kRowMajor, 1 = kColMajor."""
     if host_weight.is_cuda:

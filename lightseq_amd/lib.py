@@ -46,6 +46,9 @@ _SIGNATURES = {
     "lsh_launch_scaled_colsum": (True, "ppiifs"),
     "lsh_gemm_i8_i32o": (False, "pppiiis"),
     "lsh_gemm_i8_i8o": (False, "pppiiifs"),
+    "lsh_gemm_i8_bias_gelu_i8o_f16": (False, "pppp" + "iiifffs"),
+    "lsh_gemm_i8_bias_relu_i8o_f16": (False, "pppp" + "iiiffffis"),
+    "lsh_gemm_i8_qkv_arrange_f16": (False, "pppp" + "iiiiiiffs"),
     "lsh_quantize_weight": (True, "ppiifsi"),
 }
 

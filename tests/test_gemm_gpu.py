@@ -98,3 +98,55 @@ def test_gemm_rejects_bad_k():
     c = torch.zeros((4, 4), dtype=torch.int32, device=DEV)
     with pytest.raises(LSHError):
         _k().gemm_i8_i32o(a, a, c, 4, 4, 8)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 3072, 768), (4096, 3072, 768), (77, 160, 48)])
+@pytest.mark.parametrize("act", ["gelu", "relu", "relu_narrow"])
+def test_fused_bias_act_epilogue_equals_unfused_pair(rng, M, N, K, act):
+    """GEMM + bias/activation/requant in one kernel == int8-output GEMM followed by the
+    stand-alone kernel, byte for byte."""
+    k = _k()
+    a = to_dev(rng.integers(-127, 128, size=(M, K), dtype=np.int8))
+    w = to_dev(rng.integers(-127, 128, size=(N, K), dtype=np.int8))
+    bias = to_dev((0.3 * rng.standard_normal(N)).astype(np.float16))
+    alpha, ds, qs, clip = 3.0 / (np.sqrt(K) * 127), 2.2 / 127, 127 / 1.65, 1.65
+    tmp = torch.zeros((M, N), dtype=torch.int8, device=DEV)
+    want = torch.zeros_like(tmp)
+    got = torch.zeros_like(tmp)
+    k.gemm_i8_i8o(a, w, tmp, M, N, K, alpha)
+    if act == "gelu":
+        k.ker_bias_gelu_i8I_i8O_launcher(M, tmp, want, bias, N, ds, qs)
+        k.gemm_i8_bias_gelu_i8o(a, w, got, bias, M, N, K, alpha, ds, qs)
+    else:
+        narrow = act == "relu_narrow"
+        k.ker_bias_relu_i8I_i8O_launcher(M, tmp, want, bias, N, ds, qs, clip, False, False, narrow)
+        k.gemm_i8_bias_relu_i8o(a, w, got, bias, M, N, K, alpha, ds, qs, clip, narrow)
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("B,S,h,d,K", [(2, 16, 2, 64, 128), (32, 128, 12, 64, 768), (3, 10, 4, 16, 64)])
+def test_fused_qkv_arrange_epilogue_equals_unfused_pair(rng, B, S, h, d, K):
+    k = _k()
+    H, M = h * d, B * S
+    a = to_dev(rng.integers(-127, 128, size=(M, K), dtype=np.int8))
+    w = to_dev(rng.integers(-127, 128, size=(3 * H, K), dtype=np.int8))
+    bias = to_dev((0.3 * rng.standard_normal(3 * H)).astype(np.float16))
+    alpha, ds = 3.0 / (np.sqrt(K) * 127), 2.2 / 127
+    tmp = torch.zeros((M, 3 * H), dtype=torch.int8, device=DEV)
+    want = torch.zeros((3, B, h, S, d), dtype=torch.float16, device=DEV)
+    got = torch.zeros_like(want)
+    k.gemm_i8_i8o(a, w, tmp, M, 3 * H, K, alpha)
+    k.ker_arrange_encself_qkv_i8I_launcher(M, H, tmp, bias, want, M * H, S, d, h, 1024, ds)
+    k.gemm_i8_qkv_arrange(a, w, got, bias, M * H, M, H, K, S, h, alpha, ds)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_fused_qkv_arrange_rejects_small_heads(rng):
+    from lightseq_amd.lib import LSHError
+    k = _k()
+    a = torch.zeros((8, 16), dtype=torch.int8, device=DEV)
+    w = torch.zeros((3 * 8, 16), dtype=torch.int8, device=DEV)
+    out = torch.zeros((3, 8, 8), dtype=torch.float16, device=DEV)
+    bias = torch.zeros(24, dtype=torch.float16, device=DEV)
+    with pytest.raises(LSHError):
+        k.gemm_i8_qkv_arrange(a, w, out, bias, 64, 8, 8, 16, 8, 1, 1.0, 1.0)
