@@ -249,6 +249,218 @@ int lsh_quantize_weight_f16(const void* origin_weight, int8_t* quantized_weight,
 int lsh_quantize_weight_f32(const void* origin_weight, int8_t* quantized_weight, int rows,
                             int cols, float quant_scale, lsh_stream_t stream, int layout);
 
+/* ======================================================================== */
+/* decoder step                                                               */
+/* ======================================================================== */
+
+/* kernels/embKernels_int8.h launch_dec_emb_i8I (embKernels_int8.cc.cu:181-200).
+ * tokens [batch*beam, max_step]; token_emb [hidden_dim, vocab_size] int8 codes;
+ * output [batch*beam, hidden_dim] T.  multilg_type != 0 -> LSH_ERR_UNSUPPORTED
+ * ("multilingle not supported", as the reference throws); step >= max_step ->
+ * LSH_ERR_INVALID ("violate step < max_step").  The _vocab_major variants take the
+ * table as [vocab_size, hidden_dim] -- the layout of the logits GEMM weight -- so one
+ * copy of the shared embedding serves both uses and a row lookup is contiguous. */
+int lsh_launch_dec_emb_i8I_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,
+                               const void* lang_emb, const int* lang_id, void* output,
+                               int batch_size, int beam_size, int hidden_dim, int vocab_size,
+                               int step, int max_step, int multilg_type, lsh_stream_t stream,
+                               float dequant_scale, int scaled);
+int lsh_launch_dec_emb_i8I_f32(const int8_t* token_emb, const void* pos_emb, const int* tokens,
+                               const void* lang_emb, const int* lang_id, void* output,
+                               int batch_size, int beam_size, int hidden_dim, int vocab_size,
+                               int step, int max_step, int multilg_type, lsh_stream_t stream,
+                               float dequant_scale, int scaled);
+int lsh_launch_dec_emb_i8I_vocab_major_f16(const int8_t* token_emb, const void* pos_emb,
+                                           const int* tokens, const void* lang_emb,
+                                           const int* lang_id, void* output, int batch_size,
+                                           int beam_size, int hidden_dim, int vocab_size, int step,
+                                           int max_step, int multilg_type, lsh_stream_t stream,
+                                           float dequant_scale, int scaled);
+int lsh_launch_dec_emb_i8I_vocab_major_f32(const int8_t* token_emb, const void* pos_emb,
+                                           const int* tokens, const void* lang_emb,
+                                           const int* lang_id, void* output, int batch_size,
+                                           int beam_size, int hidden_dim, int vocab_size, int step,
+                                           int max_step, int multilg_type, lsh_stream_t stream,
+                                           float dequant_scale, int scaled);
+
+/* kernels/transformerKernels_int8.h ker_arrange_decself_qkv_i8I_i8O_launcher
+ * (transformerKernels_int8.cc.cu:1475-1486).  ori_qkv [step_token_num, 3*hidden] int8;
+ * new_q [step_token_num, hidden]; new_k / new_v: slot step_id of the caches
+ * [step_token_num, head_num, max_step, dim_per_head] int8. */
+int lsh_ker_arrange_decself_qkv_i8I_i8O_f16(int step_token_num, int hidden_size,
+                                            lsh_stream_t stream, const int8_t* ori_qkv,
+                                            const void* qkv_bias, int8_t* new_q, int8_t* new_k,
+                                            int8_t* new_v, int head_num, int dim_per_head,
+                                            int max_step, int step_id, int max_thread_per_block,
+                                            float dequant_scale, float quant_scale, int in_col32);
+int lsh_ker_arrange_decself_qkv_i8I_i8O_f32(int step_token_num, int hidden_size,
+                                            lsh_stream_t stream, const int8_t* ori_qkv,
+                                            const void* qkv_bias, int8_t* new_q, int8_t* new_k,
+                                            int8_t* new_v, int head_num, int dim_per_head,
+                                            int max_step, int step_id, int max_thread_per_block,
+                                            float dequant_scale, float quant_scale, int in_col32);
+
+/* The strided-batched int8 GEMM of model/quant_decoder.cc.cu:676-683:
+ * scores[bh, j] = sum_d q[bh, d] * k_cache[bh, j, d] for j < step_num, int32, row
+ * stride max_step.  q [batch_head_num, dim_per_head], k_cache [batch_head_num,
+ * max_step, dim_per_head]. */
+int lsh_decself_scores_i8_i32o(const int8_t* k_cache, const int8_t* q, int32_t* scores,
+                               int batch_head_num, int step_num, int max_step, int dim_per_head,
+                               lsh_stream_t stream);
+/* kernels/transformerKernels_int8.h ker_fuse_softmax_new_value_i32I_i8O_launcher
+ * (transformerKernels_int8.cc.cu:1579-1594).  The value sum runs in ascending step
+ * order (the reference accumulates with float atomics in no fixed order). */
+int lsh_ker_fuse_softmax_new_value_i32I_i8O(const int32_t* correlation, const int8_t* v,
+                                            int8_t* new_v, int batch_head_num, int step_num,
+                                            int max_step, int head_num, int dim_per_head,
+                                            float attn_scale, float dequant_scale,
+                                            float quant_scale, int out_col32, lsh_stream_t stream);
+/* The two calls above in one kernel (the int32 scores never reach HBM); produces the
+ * bytes the pair produces.  No single counterpart in the reference. */
+int lsh_decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v_cache,
+                             int8_t* new_v, int batch_head_num, int step_num, int max_step,
+                             int head_num, int dim_per_head, float attn_scale,
+                             float dequant_scale, float quant_scale, lsh_stream_t stream);
+
+/* kernels/transformerKernels_int8.h ker_arrange_encdec_q_i8I_launcher
+ * (transformerKernels_int8.cc.cu:1653-1676).  new_q [batch, head_num, beam_size,
+ * dim_per_head] T. */
+int lsh_ker_arrange_encdec_q_i8I_f16(int step_token_num, int hidden_size, lsh_stream_t stream,
+                                     const int8_t* ori_q, const void* q_bias, void* new_q,
+                                     int beam_size, int dim_per_head, int head_num,
+                                     int max_thread_per_block, float dequant_scale, int in_col32);
+int lsh_ker_arrange_encdec_q_i8I_f32(int step_token_num, int hidden_size, lsh_stream_t stream,
+                                     const int8_t* ori_q, const void* q_bias, void* new_q,
+                                     int beam_size, int dim_per_head, int head_num,
+                                     int max_thread_per_block, float dequant_scale, int in_col32);
+/* kernels/transformerKernels.h ker_arrange_encdec_kv_launcher
+ * (transformerKernels.cc.cu:985-1007).  ori_kv [batch_token_num, dec_layer_num, 2,
+ * hidden] T; layer l of new_k / new_v starts l*offset_per_layer elements in and is
+ * [batch, head_num, batch_seq_len, dim_per_head]. */
+int lsh_ker_arrange_encdec_kv_f16(int batch_token_num, int dec_layer_num, int hidden_size,
+                                  lsh_stream_t stream, const void* ori_kv, const void* kv_bias,
+                                  void* new_k, void* new_v, int64_t offset_per_layer,
+                                  int batch_seq_len, int dim_per_head, int head_num,
+                                  int max_thread_per_block);
+int lsh_ker_arrange_encdec_kv_f32(int batch_token_num, int dec_layer_num, int hidden_size,
+                                  lsh_stream_t stream, const void* ori_kv, const void* kv_bias,
+                                  void* new_k, void* new_v, int64_t offset_per_layer,
+                                  int batch_seq_len, int dim_per_head, int head_num,
+                                  int max_thread_per_block);
+/* kernels/transformerKernels.h ker_correlation_softmax_encdec_launcher
+ * (transformerKernels.cc.cu:1264-1276).  correlation [batch_size, head_num_per_seq,
+ * batch_seq_len] T, in place; head_num_per_seq = head_num * beam_size. */
+int lsh_ker_correlation_softmax_encdec_f16(int batch_size, int head_num_per_seq,
+                                           int batch_seq_len, lsh_stream_t stream,
+                                           void* correlation, const int* src_padding_mask);
+int lsh_ker_correlation_softmax_encdec_f32(int batch_size, int head_num_per_seq,
+                                           int batch_seq_len, lsh_stream_t stream,
+                                           void* correlation, const int* src_padding_mask);
+/* Fused encoder-decoder attention of one decoder layer (fp16): the two strided-batched
+ * GEMMs, the softmax above and ker_arrange_atten_output_i8O of
+ * model/quant_decoder.cc.cu:765-800 in one kernel, with the reference's fp16 rounding
+ * points.  q [batch, head, beam, d]; k, v [batch, head, batch_seq_len, d]; ctx (same
+ * layout as q) and ctx_q ([batch*beam, head*d] int8) are each optional. */
+int lsh_encdec_attention_f16(const void* q, const void* k, const void* v, const int* pad_mask,
+                             void* ctx, int8_t* ctx_q, float quant_scale, int batch_size,
+                             int beam_size, int head_num, int batch_seq_len, int dim_per_head,
+                             lsh_stream_t stream);
+/* The cublasGemmEx of model/quant_decoder.cc.cu:497-501 in K-contiguous form:
+ * C[m,n] = A[m,k] * W[n,k]^T, fp16 with fp32 accumulation.  k % 16 == 0. */
+int lsh_gemm_f16_nt(const void* A, const void* W, void* C, int m, int n, int k,
+                    lsh_stream_t stream);
+
+/* ======================================================================== */
+/* beam search                                                                */
+/* ======================================================================== */
+
+/* kernels/transformerKernels.h:137-140 length_norm (host). */
+float lsh_length_norm(int length, float alpha);
+
+/* kernels/transformerKernels_int8.h select_beam_rough_topk_i8I_launcher
+ * (transformerKernels_int8.cc.cu:1846-1890).  Same buffers and candidate set as the
+ * reference; candidates are written row by row in ascending vocabulary order (the
+ * reference's order depends on atomics).  num_beam_can[0] = total,
+ * num_beam_can[1 + row] = candidates of that row (not yet scanned).
+ * max_thread_per_block defines the rough top-k threshold exactly as the reference's
+ * block size does and must be a power of two in [32, 1024].  diverse_lambda != 0 ->
+ * LSH_ERR_UNSUPPORTED. */
+int lsh_select_beam_rough_topk_i8I_f16(const int8_t* logits, const void* logit_bias,
+                                       const float* seq_probs, const float* seq_score,
+                                       const int* alive_seq, float dequant_scale, int* can_idx,
+                                       float* can_score, int* num_beam_can, int vocab_size,
+                                       int max_step, float length_norm, int cur_step,
+                                       int step_token_num, int max_thread_per_block,
+                                       lsh_stream_t stream, int beam_size, float diverse_lambda,
+                                       int end_id, int in_col32);
+int lsh_select_beam_rough_topk_i8I_f32(const int8_t* logits, const void* logit_bias,
+                                       const float* seq_probs, const float* seq_score,
+                                       const int* alive_seq, float dequant_scale, int* can_idx,
+                                       float* can_score, int* num_beam_can, int vocab_size,
+                                       int max_step, float length_norm, int cur_step,
+                                       int step_token_num, int max_thread_per_block,
+                                       lsh_stream_t stream, int beam_size, float diverse_lambda,
+                                       int end_id, int in_col32);
+/* kernels/transformerKernels.h ker_refresh_result (transformerKernels.cc.cu:1398-1463;
+ * launched at model/quant_decoder.cc.cu:1022-1027 with grid (batch_size, beam_size) and
+ * max_step threads, given here as arguments).  Consumes candidates sorted by score,
+ * descending, and the exclusively scanned per-row counts. */
+int lsh_ker_refresh_result(const int* can_idx, const float* can_score,
+                           const int* num_can_per_beam, const int* old_alive_seq,
+                           int* new_alive_seq, float* seq_probs, float* seq_score,
+                           int* num_finish_beam, int vocab_size, int cur_step, float length_norm,
+                           float diverse_lambda, int end_id, int batch_size, int beam_size,
+                           int max_step, lsh_stream_t stream);
+/* kernels/transformerKernels.h ker_refresh_cache_launcher<int8_t>
+ * (transformerKernels.cc.cu:1657-1681): grid_dim_x = decoder layers, grid_dim_y =
+ * 2 * batch * beam, block_dim ignored.  self_k_bgeem_offset = bytes between layers. */
+int lsh_ker_refresh_cache_i8(int grid_dim_x, int grid_dim_y, int block_dim, lsh_stream_t stream,
+                             const int* num_can_per_beam, const int* can_idx,
+                             const int8_t* self_k_bgeem, const int8_t* self_v_bgeem,
+                             int8_t* new_self_k_bgeem, int8_t* new_self_v_bgeem,
+                             int64_t self_k_bgeem_offset, int beam_size, int dim_per_head,
+                             int head_num, int vocab_size, int cur_step, int max_step,
+                             int diverse, int end_id);
+/* kernels/transformerKernels.h ker_write_trg_tokenid_pos_penalty / _neg_penalty /
+ * ker_write_topk_result (transformerKernels.cc.cu:1722-1815; launched at
+ * model/quant_decoder.cc.cu:454-476 with out_len = cur_step + 1 threads). */
+int lsh_ker_write_trg_tokenid_pos_penalty(const int* alive_seq, float* seq_score, int* output,
+                                          int max_step, int beam_size, int batch_size,
+                                          int out_len, lsh_stream_t stream);
+int lsh_ker_write_trg_tokenid_neg_penalty(const int* alive_seq, const float* seq_score,
+                                          int* output, int max_step, int beam_size,
+                                          int vocab_size, int end_id, int batch_size, int out_len,
+                                          lsh_stream_t stream);
+int lsh_ker_write_topk_result(const int* alive_seq, float* seq_score, int* res_seq,
+                              int vocab_size, int max_step, int beam_size, int end_id,
+                              int batch_beam_num, int out_len, lsh_stream_t stream);
+
+/* One whole search step without a sort, a scan or a host round trip: replaces
+ * update_new_seq_probs + thrust::sort_by_key + ker_refresh_result of
+ * model/quant_decoder.cc.cu:988-1057 (diverse_lambda == 0) and selects the same
+ * beams; ties go to the lower candidate id (thrust leaves them unspecified).
+ * Workspace: top_score / top_idx [batch*beam, beam_size].  Outputs: new_alive_seq,
+ * seq_probs / seq_score (in place), parent [batch*beam] (source beam of each new beam
+ * inside its sentence, -1 for a finished beam) and *num_finished. */
+int lsh_beam_search_step_i8I_f16(const int8_t* logits, const void* logit_bias, float* seq_probs,
+                                 float* seq_score, const int* old_alive_seq, int* new_alive_seq,
+                                 float* top_score, int* top_idx, int* parent, int* num_finished,
+                                 float dequant_scale, int vocab_size, int max_step,
+                                 float length_norm, int cur_step, int batch_size, int beam_size,
+                                 int end_id, lsh_stream_t stream);
+int lsh_beam_search_step_i8I_f32(const int8_t* logits, const void* logit_bias, float* seq_probs,
+                                 float* seq_score, const int* old_alive_seq, int* new_alive_seq,
+                                 float* top_score, int* top_idx, int* parent, int* num_finished,
+                                 float dequant_scale, int vocab_size, int max_step,
+                                 float length_norm, int cur_step, int batch_size, int beam_size,
+                                 int end_id, lsh_stream_t stream);
+/* Cache reorder driven by the parent table of lsh_beam_search_step_i8I (same copy as
+ * lsh_ker_refresh_cache_i8).  rows = batch * beam. */
+int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, const int* parent,
+                                   const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
+                                   int8_t* v_new, int64_t layer_offset, int beam_size,
+                                   int dim_per_head, int head_num, int cur_step, int max_step);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,666 @@
+// Beam search over int8 logits.
+//
+// Two families live here.
+//  * The kernels behind the launchers of the reference, with their buffers and
+//    meaning: candidate selection with the "rough top-k" threshold, the result and
+//    cache refresh that consume globally sorted candidates, and the output writers.
+//    The candidate set is exactly the reference's; candidates are emitted row by row
+//    in ascending vocabulary order instead of in an order decided by atomics.
+//  * The search step the decoder itself runs: an exact per-row top-k followed by a
+//    per-sentence merge that also refreshes the sequences and scores.  It selects
+//    the same beams as sorting the reference's candidates (any candidate among a
+//    sentence's best `beam_size` is among its row's best `beam_size`, and the rough
+//    threshold never cuts into a row's best `beam_size`), without a global sort, a
+//    prefix scan or a device-to-host round trip.  Ties go to the lower candidate id.
+#include "ls_device.cuh"
+#include "ls_launch.h"
+
+namespace lsh {
+
+constexpr float kMinLogProb = -2000.f;      // inference/kernels/transformerKernels.h:12
+constexpr float kLogitThreshMin = -64.f;    // inference/kernels/transformerKernels.h:11
+constexpr float kSeqLenEpsilon = 1e-12f;    // inference/kernels/transformerKernels.h:13
+
+template <typename T>
+__device__ __forceinline__ float logit_of(const int8_t* __restrict__ lr,
+                                          const T* __restrict__ bias, int v, float dq) {
+#pragma clang fp contract(off)
+  return (float)lr[v] * dq + TT<T>::ld(bias, v);
+}
+
+__device__ __forceinline__ float cand_score(float lgt, float base, float length_norm,
+                                            int batch_id) {
+#pragma clang fp contract(off)
+  return fmaxf((lgt + base) * length_norm, kMinLogProb + 1.f) + (float)batch_id * kMinLogProb;
+}
+
+// Row statistics shared by every selection kernel: max logit, sum of exp and (when
+// `threads` > 0) the rough top-k threshold of inference/kernels/common.h:118-137 as a
+// block of `threads` threads would compute it -- thread t of that block sees the
+// vocabulary ids congruent to t modulo `threads`; `threads` is a power of two <= 1024
+// so a lane of this 1024-thread block always stays inside one such class.
+struct RowStats {
+  float max_logit, sum_exp, topk;
+};
+
+// integer block sum for blocks of up to 1024 threads; `red` holds >= 16 ints
+__device__ __forceinline__ int block_sum_i(int v, int* red) {
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m, 64);
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if (lane == 0) red[wid] = v;
+  __syncthreads();
+  int r = 0;
+  for (int i = 0; i < nw; ++i) r += red[i];
+  return r;
+}
+
+template <typename T>
+__device__ RowStats row_stats(const int8_t* __restrict__ lr, const T* __restrict__ bias,
+                              int vocab, float dq, int threads, int K, float* red /*[1024+32]*/) {
+  const int t = threadIdx.x;
+  float tmax = kFloatInfNeg;
+  for (int v = t; v < vocab; v += 1024) tmax = fmaxf(tmax, logit_of(lr, bias, v, dq));
+  RowStats st;
+  st.max_logit = block_max(tmax, red);
+  float se = 0.f;
+  for (int v = t; v < vocab; v += 1024)
+    se += __expf(fmaxf(logit_of(lr, bias, v, dq) - st.max_logit, kLogitThreshMin));
+  st.sum_exp = block_sum(se, red);
+  st.topk = 0.f;
+  if (threads > 0) {
+    float* tm = red + 32;
+    __syncthreads();
+    tm[t] = tmax;
+    __syncthreads();
+    if (t < 32) {  // maximum of warp t of the emulated block
+      float g = 0.f;
+      if (t < (threads >> 5)) {
+        g = kFloatInfNeg;
+        for (int u = 0; u < 1024; ++u)
+          if (((u & (threads - 1)) >> 5) == t) g = fmaxf(g, tm[u]);
+      }
+      red[t] = g;
+    }
+    __syncthreads();
+    float best = 0.f;
+    for (int r = 0; r < K; ++r) {
+      float m = red[r];
+      for (int j = r + K; j < 32; j += K) m = fmaxf(m, red[j]);
+      best = r == 0 ? m : fminf(best, m);
+    }
+    st.topk = best;
+    __syncthreads();
+  }
+  return st;
+}
+
+// ---------------------------------------------------------------------------------
+// select_beam_rough_topk_i8I (inference/kernels/transformerKernels_int8.cc.cu:1690-1890)
+// pass 1: candidates per row -> num_beam_can[1 + row]
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(1024)
+beam_select_count_kernel(const int8_t* __restrict__ logits, const T* __restrict__ logit_bias,
+                         const int* __restrict__ alive_seq, float dq, int* __restrict__ num_beam_can,
+                         int vocab, int max_step, int cur_step, int threads, int beam_size,
+                         int end_id) {
+  __shared__ float red[1024 + 32];
+  const int row = blockIdx.x;
+  if (cur_step != 0 && alive_seq[(long)row * max_step + cur_step] == end_id) {
+    if (threadIdx.x == 0) num_beam_can[row + 1] = 1;
+    return;
+  }
+  const int8_t* lr = logits + (long)row * vocab;
+  const RowStats st = row_stats(lr, logit_bias, vocab, dq, threads, beam_size, red);
+  int n = 0;
+  for (int v = threadIdx.x; v < vocab; v += 1024)
+    n += logit_of(lr, logit_bias, v, dq) >= st.topk ? 1 : 0;
+  n = block_sum_i(n, reinterpret_cast<int*>(red));
+  if (threadIdx.x == 0) num_beam_can[row + 1] = n;
+}
+
+// pass 2: emit at the row's offset (sum of the preceding counts), ascending vocab id
+template <typename T>
+__global__ void __launch_bounds__(1024)
+beam_select_emit_kernel(const int8_t* __restrict__ logits, const T* __restrict__ logit_bias,
+                        const float* __restrict__ seq_probs, const float* __restrict__ seq_score,
+                        const int* __restrict__ alive_seq, float dq, int* __restrict__ can_idx,
+                        float* __restrict__ can_score, int* __restrict__ num_beam_can, int vocab,
+                        int max_step, float length_norm, int cur_step, int rows, int threads,
+                        int beam_size, int end_id) {
+#pragma clang fp contract(off)
+  __shared__ float red[1024 + 32];
+  __shared__ int wave_cnt[16];
+  __shared__ int s_base;
+  const int row = blockIdx.x, t = threadIdx.x;
+  const int lane = t & 63, wid = t >> 6;
+  // offset of this row = candidates of the rows before it
+  int ahead = 0, all = 0;
+  for (int r = t; r < rows; r += 1024) {
+    const int c = num_beam_can[r + 1];
+    all += c;
+    if (r < row) ahead += c;
+  }
+  const int pos = block_sum_i(ahead, reinterpret_cast<int*>(red));
+  if (row == 0) {
+    all = block_sum_i(all, reinterpret_cast<int*>(red));
+    if (t == 0) num_beam_can[0] = all;
+  }
+  const int batch_id = row / beam_size;
+  if (cur_step != 0 && alive_seq[(long)row * max_step + cur_step] == end_id) {
+    if (t == 0) {  // a finished beam keeps its score and proposes <eos> once
+      can_score[pos] = seq_score[row];
+      can_idx[pos] = end_id + (row % beam_size) * vocab;
+    }
+    return;
+  }
+  const int8_t* lr = logits + (long)row * vocab;
+  const RowStats st = row_stats(lr, logit_bias, vocab, dq, threads, beam_size, red);
+  const float base = seq_probs[row] - logf(st.sum_exp) - st.max_logit;
+  if (t == 0) s_base = pos;
+  __syncthreads();
+  for (int v0 = 0; v0 < vocab; v0 += 1024) {
+    const int v = v0 + t;
+    float lgt = 0.f;
+    bool take = false;
+    if (v < vocab) {
+      lgt = logit_of(lr, logit_bias, v, dq);
+      take = lgt >= st.topk;
+    }
+    const unsigned long long ballot = __ballot(take);
+    if (lane == 0) wave_cnt[wid] = __popcll(ballot);
+    __syncthreads();
+    int off = s_base;
+    for (int w2 = 0; w2 < wid; ++w2) off += wave_cnt[w2];
+    off += __popcll(ballot & ((1ull << lane) - 1ull));
+    if (take) {
+      can_score[off] = cand_score(lgt, base, length_norm, batch_id);
+      can_idx[off] = (row - batch_id * beam_size) * vocab + v;
+    }
+    __syncthreads();
+    if (t == 0) {
+      int tot = 0;
+      for (int w2 = 0; w2 < 16; ++w2) tot += wave_cnt[w2];
+      s_base += tot;
+    }
+    __syncthreads();
+  }
+}
+
+template <typename T>
+int select_beam_rough_topk_i8I(const int8_t* logits, const T* logit_bias, const float* seq_probs,
+                               const float* seq_score, const int* alive_seq, float dequant_scale,
+                               int* can_idx, float* can_score, int* num_beam_can, int vocab_size,
+                               int max_step, float length_norm, int cur_step, int step_token_num,
+                               int max_thread_per_block, hipStream_t s, int beam_size,
+                               float diverse_lambda, int end_id) {
+  if (!logits || !logit_bias || !seq_probs || !seq_score || !alive_seq || !can_idx ||
+      !can_score || !num_beam_can || vocab_size <= 0 || step_token_num <= 0 || max_step <= 0 ||
+      cur_step < 0 || cur_step >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "select_beam_rough_topk_i8I: bad arguments");
+  if (diverse_lambda != 0.f)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "select_beam_rough_topk_i8I: diverse beam search");
+  if (beam_size < 1 || beam_size > 32 || (beam_size & (beam_size - 1)) ||
+      step_token_num % beam_size != 0)
+    return lsh_fail(LSH_ERR_INVALID, "wrong beam_size, should be 1, 2, 4, 8, 16 or 32");
+  const int th = max_thread_per_block;
+  if (th < 32 || th > 1024 || (th & (th - 1)))
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "select_beam_rough_topk_i8I: max_thread_per_block must be a power of two in "
+                    "[32, 1024]");
+  beam_select_count_kernel<T><<<step_token_num, 1024, 0, s>>>(
+      logits, logit_bias, alive_seq, dequant_scale, num_beam_can, vocab_size, max_step, cur_step,
+      th, beam_size, end_id);
+  if (int rc = lsh_check_launch("beam_select_count_kernel")) return rc;
+  beam_select_emit_kernel<T><<<step_token_num, 1024, 0, s>>>(
+      logits, logit_bias, seq_probs, seq_score, alive_seq, dequant_scale, can_idx, can_score,
+      num_beam_can, vocab_size, max_step, length_norm, cur_step, step_token_num, th, beam_size,
+      end_id);
+  return lsh_check_launch("beam_select_emit_kernel");
+}
+template int select_beam_rough_topk_i8I<float>(const int8_t*, const float*, const float*,
+                                               const float*, const int*, float, int*, float*, int*,
+                                               int, int, float, int, int, int, hipStream_t, int,
+                                               float, int);
+template int select_beam_rough_topk_i8I<__half>(const int8_t*, const __half*, const float*,
+                                                const float*, const int*, float, int*, float*,
+                                                int*, int, int, float, int, int, int, hipStream_t,
+                                                int, float, int);
+
+// ---------------------------------------------------------------------------------
+// ker_refresh_result (inference/kernels/transformerKernels.cc.cu:1398-1463),
+// diverse_lambda == 0.  Grid (batch, beam), one thread per position.
+// ---------------------------------------------------------------------------------
+__global__ void refresh_result_kernel(const int* __restrict__ can_idx,
+                                      const float* __restrict__ can_score,
+                                      const int* __restrict__ num_can_per_beam,
+                                      const int* __restrict__ old_alive_seq,
+                                      int* __restrict__ new_alive_seq, float* seq_probs,
+                                      float* seq_score, int* num_finish_beam, int vocab_size,
+                                      int cur_step, float length_norm, int end_id, int max_step) {
+#pragma clang fp contract(off)
+  const int b = blockIdx.x, j = blockIdx.y, beam = gridDim.y;
+  const int can_pos = num_can_per_beam[b * beam] + j;
+  const int ori = can_idx[can_pos];
+  const int can_beam_id = ori / vocab_size, can_vocab_id = ori % vocab_size;
+  for (int t = threadIdx.x; t < max_step; t += blockDim.x) {
+    int tok;
+    if (t > cur_step + 1)
+      tok = end_id;
+    else if (t == cur_step + 1)
+      tok = can_vocab_id;
+    else
+      tok = old_alive_seq[((long)b * beam + can_beam_id) * max_step + t];
+    new_alive_seq[((long)b * beam + j) * max_step + t] = tok;
+  }
+  if (threadIdx.x == 0) {
+    if (can_vocab_id != end_id) {
+      seq_probs[b * beam + j] = (can_score[can_pos] - (float)b * kMinLogProb) / length_norm;
+    } else {
+      atomicAdd(num_finish_beam, 1);
+      seq_score[b * beam + j] = can_score[can_pos];
+    }
+  }
+}
+
+int refresh_result(const int* can_idx, const float* can_score, const int* num_can_per_beam,
+                   const int* old_alive_seq, int* new_alive_seq, float* seq_probs,
+                   float* seq_score, int* num_finish_beam, int vocab_size, int cur_step,
+                   float length_norm, float diverse_lambda, int end_id, int batch_size,
+                   int beam_size, int max_step, hipStream_t s) {
+  if (!can_idx || !can_score || !num_can_per_beam || !old_alive_seq || !new_alive_seq ||
+      !seq_probs || !seq_score || !num_finish_beam || batch_size <= 0 || beam_size <= 0 ||
+      vocab_size <= 0 || max_step <= 0 || cur_step < 0 || cur_step + 1 >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "ker_refresh_result: bad arguments");
+  if (diverse_lambda != 0.f)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "ker_refresh_result: diverse beam search");
+  if (old_alive_seq == new_alive_seq)
+    return lsh_fail(LSH_ERR_INVALID, "ker_refresh_result: the sequence buffers must differ");
+  refresh_result_kernel<<<dim3(batch_size, beam_size), 256, 0, s>>>(
+      can_idx, can_score, num_can_per_beam, old_alive_seq, new_alive_seq, seq_probs, seq_score,
+      num_finish_beam, vocab_size, cur_step, length_norm, end_id, max_step);
+  return lsh_check_launch("refresh_result_kernel");
+}
+
+// ---------------------------------------------------------------------------------
+// K/V cache reorder after a search step
+// (inference/kernels/transformerKernels.cc.cu:1579-1627 and its launcher :1657-1681).
+// Grid (layer, 2 * rows).  The parent beam comes either from the sorted candidates
+// (reference launcher) or from a parent table (-1 = finished beam, nothing copied).
+// ---------------------------------------------------------------------------------
+template <bool PARENT_TABLE>
+__global__ void __launch_bounds__(256)
+refresh_cache_kernel(const int* __restrict__ num_can_per_beam, const int* __restrict__ can_idx,
+                     const int* __restrict__ parent, const int8_t* __restrict__ k_old,
+                     const int8_t* __restrict__ v_old, int8_t* __restrict__ k_new,
+                     int8_t* __restrict__ v_new, long layer_offset, int beam_size, int d,
+                     int head_num, int vocab_size, int cur_step, int max_step, int end_id) {
+  const int layer = blockIdx.x, kv = blockIdx.y & 1, row = blockIdx.y >> 1;
+  const int b = row / beam_size, j = row % beam_size;
+  int src;
+  if (PARENT_TABLE) {
+    src = parent[row];
+    if (src < 0) return;
+  } else {
+    const int c = can_idx[num_can_per_beam[b * beam_size] + j];
+    if (c % vocab_size == end_id) return;
+    src = c / vocab_size;
+  }
+  if (src < 0 || src >= beam_size) return;  // never read outside the sentence's beams
+  const long beam_bytes = (long)head_num * max_step * d;
+  const long o = layer * layer_offset + ((long)b * beam_size + src) * beam_bytes;
+  const long n = layer * layer_offset + ((long)b * beam_size + j) * beam_bytes;
+  const int8_t* from = (kv ? v_old : k_old) + o;
+  int8_t* to = (kv ? v_new : k_new) + n;
+  const int chunk = (cur_step + 1) * d;  // contiguous bytes per head
+  const long head_stride = (long)max_step * d;
+  const bool vec = (d % 16 == 0) && (layer_offset % 16 == 0) &&
+                   ((reinterpret_cast<uintptr_t>(from) | reinterpret_cast<uintptr_t>(to)) & 15u) == 0;
+  if (vec) {
+    const int per_head = chunk >> 4;
+    for (int i = threadIdx.x; i < per_head * head_num; i += blockDim.x) {
+      const int h = i / per_head, c16 = i % per_head;
+      const long p = h * head_stride + (long)c16 * 16;
+      *reinterpret_cast<uint4*>(to + p) = *reinterpret_cast<const uint4*>(from + p);
+    }
+  } else {
+    for (int i = threadIdx.x; i < chunk * head_num; i += blockDim.x) {
+      const long p = (i / chunk) * head_stride + (i % chunk);
+      to[p] = from[p];
+    }
+  }
+}
+
+static int refresh_cache_check(const void* a, const void* b, const void* c, const void* d2,
+                               int n_layer, int rows, int beam_size, int d, int head_num,
+                               int cur_step, int max_step) {
+  if (!a || !b || !c || !d2 || n_layer <= 0 || rows <= 0 || beam_size <= 0 ||
+      rows % beam_size != 0 || d <= 0 || head_num <= 0 || cur_step < 0 || cur_step >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "ker_refresh_cache: bad arguments");
+  if (a == c || b == d2)
+    return lsh_fail(LSH_ERR_INVALID, "ker_refresh_cache: old and new cache must differ");
+  if (rows * 2 > 65535) return lsh_fail(LSH_ERR_UNSUPPORTED, "ker_refresh_cache: too many rows");
+  return LSH_OK;
+}
+
+int refresh_cache_i8(int n_layer, int rows_x2, hipStream_t s, const int* num_can_per_beam,
+                     const int* can_idx, const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
+                     int8_t* v_new, long layer_offset, int beam_size, int dim_per_head,
+                     int head_num, int vocab_size, int cur_step, int max_step, bool diverse,
+                     int end_id) {
+  if (diverse) return lsh_fail(LSH_ERR_UNSUPPORTED, "ker_refresh_cache: diverse beam search");
+  if (!num_can_per_beam || !can_idx || vocab_size <= 0 || (rows_x2 & 1))
+    return lsh_fail(LSH_ERR_INVALID, "ker_refresh_cache: bad arguments");
+  if (int rc = refresh_cache_check(k_old, v_old, k_new, v_new, n_layer, rows_x2 / 2, beam_size,
+                                   dim_per_head, head_num, cur_step, max_step))
+    return rc;
+  refresh_cache_kernel<false><<<dim3(n_layer, rows_x2), 256, 0, s>>>(
+      num_can_per_beam, can_idx, nullptr, k_old, v_old, k_new, v_new, layer_offset, beam_size,
+      dim_per_head, head_num, vocab_size, cur_step, max_step, end_id);
+  return lsh_check_launch("refresh_cache_kernel<false>");
+}
+
+int refresh_cache_by_parent_i8(int n_layer, int rows, hipStream_t s, const int* parent,
+                               const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
+                               int8_t* v_new, long layer_offset, int beam_size, int dim_per_head,
+                               int head_num, int cur_step, int max_step) {
+  if (!parent) return lsh_fail(LSH_ERR_INVALID, "refresh_cache_by_parent: null parent table");
+  if (int rc = refresh_cache_check(k_old, v_old, k_new, v_new, n_layer, rows, beam_size,
+                                   dim_per_head, head_num, cur_step, max_step))
+    return rc;
+  refresh_cache_kernel<true><<<dim3(n_layer, rows * 2), 256, 0, s>>>(
+      nullptr, nullptr, parent, k_old, v_old, k_new, v_new, layer_offset, beam_size,
+      dim_per_head, head_num, 1, cur_step, max_step, 0);
+  return lsh_check_launch("refresh_cache_kernel<true>");
+}
+
+// ---------------------------------------------------------------------------------
+// output writers (inference/kernels/transformerKernels.cc.cu:1707-1815)
+// ---------------------------------------------------------------------------------
+__global__ void write_trg_tokenid_pos_penalty_kernel(const int* __restrict__ alive_seq,
+                                                     float* seq_score, int* __restrict__ output,
+                                                     int max_step, int beam_size, int batch,
+                                                     int out_len) {
+  const int b = blockIdx.x;
+  for (int t = threadIdx.x; t < out_len; t += blockDim.x)
+    output[(long)b * out_len + t] = alive_seq[(long)b * beam_size * max_step + t + 1];
+  if (b == 0) {
+    // slot b <- score of sentence b's first beam, every read taken before the slot it
+    // targets can be overwritten (chunks in ascending order, reads before writes)
+    for (int c0 = 0; c0 < batch; c0 += blockDim.x) {
+      const int i = c0 + threadIdx.x;
+      float v = 0.f;
+      if (i < batch) v = seq_score[(long)i * beam_size] - (float)i * kMinLogProb;
+      __syncthreads();
+      if (i < batch) seq_score[i] = v;
+      __syncthreads();
+    }
+  }
+}
+
+__global__ void write_trg_tokenid_neg_penalty_kernel(const int* __restrict__ alive_seq,
+                                                     const float* __restrict__ seq_score,
+                                                     int* __restrict__ output, int max_step,
+                                                     int beam_size, int end_id, int out_len) {
+#pragma clang fp contract(off)
+  __shared__ float red[16];
+  const int b = blockIdx.x;
+  float best = kFloatInfNeg;
+  int res = 0;
+  for (int j = 0; j < beam_size; ++j) {
+    float n = 0.f;
+    for (int t = threadIdx.x; t < out_len; t += blockDim.x)
+      n += alive_seq[((long)b * beam_size + j) * max_step + t + 1] != end_id ? 1.f : 0.f;
+    n = block_sum(n, red);
+    float sc = seq_score[b * beam_size + j] - (float)b * kMinLogProb;
+    sc /= (n + kSeqLenEpsilon);
+    if (sc > best) {
+      best = sc;
+      res = j;
+    }
+  }
+  for (int t = threadIdx.x; t < out_len; t += blockDim.x)
+    output[(long)b * out_len + t] = alive_seq[((long)b * beam_size + res) * max_step + t + 1];
+}
+
+__global__ void write_topk_result_kernel(const int* __restrict__ alive_seq, float* seq_score,
+                                         int* __restrict__ res_seq, int max_step, int beam_size,
+                                         int end_id, int out_len) {
+#pragma clang fp contract(off)
+  const int r = blockIdx.x;
+  for (int t = threadIdx.x; t < out_len; t += blockDim.x)
+    res_seq[(long)r * out_len + t] =
+        t == out_len - 1 ? end_id : alive_seq[(long)r * max_step + t + 1];
+  if (threadIdx.x == 0) seq_score[r] -= (float)(r / beam_size) * kMinLogProb;
+}
+
+static int write_check(const void* a, const void* b, const void* c, int rows, int max_step,
+                       int beam_size, int out_len, const char* who) {
+  if (!a || !b || !c || rows <= 0 || beam_size <= 0 || out_len <= 0 || out_len + 1 > max_step) {
+    lsh_fail(LSH_ERR_INVALID, who);
+    return LSH_ERR_INVALID;
+  }
+  return LSH_OK;
+}
+
+int write_trg_tokenid_pos_penalty(const int* alive_seq, float* seq_score, int* output,
+                                  int max_step, int beam_size, int batch_size, int out_len,
+                                  hipStream_t s) {
+  if (int rc = write_check(alive_seq, seq_score, output, batch_size, max_step, beam_size, out_len,
+                           "ker_write_trg_tokenid_pos_penalty: bad arguments"))
+    return rc;
+  write_trg_tokenid_pos_penalty_kernel<<<batch_size, 256, 0, s>>>(
+      alive_seq, seq_score, output, max_step, beam_size, batch_size, out_len);
+  return lsh_check_launch("write_trg_tokenid_pos_penalty_kernel");
+}
+
+int write_trg_tokenid_neg_penalty(const int* alive_seq, const float* seq_score, int* output,
+                                  int max_step, int beam_size, int vocab_size, int end_id,
+                                  int batch_size, int out_len, hipStream_t s) {
+  (void)vocab_size;
+  if (int rc = write_check(alive_seq, seq_score, output, batch_size, max_step, beam_size, out_len,
+                           "ker_write_trg_tokenid_neg_penalty: bad arguments"))
+    return rc;
+  write_trg_tokenid_neg_penalty_kernel<<<batch_size, 256, 0, s>>>(
+      alive_seq, seq_score, output, max_step, beam_size, end_id, out_len);
+  return lsh_check_launch("write_trg_tokenid_neg_penalty_kernel");
+}
+
+int write_topk_result(const int* alive_seq, float* seq_score, int* res_seq, int vocab_size,
+                      int max_step, int beam_size, int end_id, int rows, int out_len,
+                      hipStream_t s) {
+  (void)vocab_size;
+  if (int rc = write_check(alive_seq, seq_score, res_seq, rows, max_step, beam_size, out_len,
+                           "ker_write_topk_result: bad arguments"))
+    return rc;
+  write_topk_result_kernel<<<rows, 256, 0, s>>>(alive_seq, seq_score, res_seq, max_step,
+                                                beam_size, end_id, out_len);
+  return lsh_check_launch("write_topk_result_kernel");
+}
+
+// ---------------------------------------------------------------------------------
+// The decoder's own search step.
+//
+// beam_topk_kernel: one 1024-thread block per row; `beam_size` rounds of a block-wide
+// arg-max over (score descending, vocabulary id ascending), each round restricted to
+// the keys after the previous pick.  Output [rows, beam_size] (score, candidate id);
+// a finished row proposes <eos> with its own score in slot 0 and nothing else.
+// ---------------------------------------------------------------------------------
+struct ScoreIdx {
+  float s;
+  int i;
+};
+// true when a comes before b: higher score, then lower id
+__device__ __forceinline__ bool before(const ScoreIdx& a, const ScoreIdx& b) {
+  return a.s > b.s || (a.s == b.s && a.i < b.i);
+}
+__device__ __forceinline__ ScoreIdx wave_first(ScoreIdx v) {
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) {
+    ScoreIdx o;
+    o.s = __shfl_xor(v.s, m, 64);
+    o.i = __shfl_xor(v.i, m, 64);
+    if (before(o, v)) v = o;
+  }
+  return v;
+}
+
+constexpr int kNoCand = 0x7fffffff;
+
+template <typename T>
+__global__ void __launch_bounds__(1024)
+beam_topk_kernel(const int8_t* __restrict__ logits, const T* __restrict__ logit_bias,
+                 const float* __restrict__ seq_probs, const float* __restrict__ seq_score,
+                 const int* __restrict__ alive_seq, float dq, float* __restrict__ top_score,
+                 int* __restrict__ top_idx, int vocab, int max_step, float length_norm,
+                 int cur_step, int beam_size, int end_id) {
+#pragma clang fp contract(off)
+  __shared__ float red[1024 + 32];
+  __shared__ ScoreIdx wbest[16];
+  const int row = blockIdx.x, t = threadIdx.x;
+  const int lane = t & 63, wid = t >> 6;
+  const int batch_id = row / beam_size, beam_id = row % beam_size;
+  float* os = top_score + (long)row * beam_size;
+  int* oi = top_idx + (long)row * beam_size;
+  if (cur_step != 0 && alive_seq[(long)row * max_step + cur_step] == end_id) {
+    if (t < beam_size) {
+      os[t] = t == 0 ? seq_score[row] : -INFINITY;
+      oi[t] = t == 0 ? end_id + beam_id * vocab : kNoCand;
+    }
+    return;
+  }
+  const int8_t* lr = logits + (long)row * vocab;
+  const RowStats st = row_stats(lr, logit_bias, vocab, dq, 0, 0, red);
+  const float base = seq_probs[row] - logf(st.sum_exp) - st.max_logit;
+  ScoreIdx prev;
+  prev.s = INFINITY;
+  prev.i = -1;
+  for (int k = 0; k < beam_size; ++k) {
+    ScoreIdx best;
+    best.s = -INFINITY;
+    best.i = kNoCand;
+    for (int v = t; v < vocab; v += 1024) {
+      ScoreIdx c;
+      c.s = cand_score(logit_of(lr, logit_bias, v, dq), base, length_norm, batch_id);
+      c.i = v;
+      if (before(prev, c) && before(c, best)) best = c;
+    }
+    best = wave_first(best);
+    __syncthreads();
+    if (lane == 0) wbest[wid] = best;
+    __syncthreads();
+    best = wbest[0];
+    for (int w2 = 1; w2 < 16; ++w2)
+      if (before(wbest[w2], best)) best = wbest[w2];
+    if (t == 0) {
+      os[k] = best.i == kNoCand ? -INFINITY : best.s;
+      oi[k] = best.i == kNoCand ? kNoCand : beam_id * vocab + best.i;
+    }
+    prev = best;
+  }
+}
+
+// beam_merge_kernel: one block, one wavefront per sentence (sentences are dealt to the
+// wavefronts round-robin).  Picks the sentence's best `beam_size` of its
+// beam_size * beam_size proposals in (score descending, candidate id ascending) order
+// and applies ker_refresh_result to them (inference/kernels/transformerKernels.cc.cu:
+// 1398-1463): new sequences, summed log-probabilities of live beams, scores of
+// finished ones, the finished count, plus the parent table for the cache reorder.
+__global__ void __launch_bounds__(1024)
+beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ top_idx,
+                  const int* __restrict__ old_alive_seq, int* __restrict__ new_alive_seq,
+                  float* __restrict__ seq_probs, float* __restrict__ seq_score,
+                  int* __restrict__ parent, int* __restrict__ num_finished, int batch,
+                  int beam_size, int vocab, int max_step, int cur_step, float length_norm,
+                  int end_id) {
+#pragma clang fp contract(off)
+  __shared__ int fin_cnt[16];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int ncand = beam_size * beam_size;  // <= 1024
+  int finished = 0;
+  for (int b = wid; b < batch; b += nw) {
+    const float* cs = top_score + (long)b * ncand;
+    const int* ci = top_idx + (long)b * ncand;
+    ScoreIdx prev;
+    prev.s = INFINITY;
+    prev.i = -1;
+    for (int j = 0; j < beam_size; ++j) {
+      ScoreIdx best;
+      best.s = -INFINITY;
+      best.i = kNoCand;
+      for (int c = lane; c < ncand; c += 64) {
+        ScoreIdx x;
+        x.s = cs[c];
+        x.i = ci[c];
+        if (x.i != kNoCand && before(prev, x) && before(x, best)) best = x;
+      }
+      best = wave_first(best);
+      prev = best;
+      // a sentence always has at least beam_size proposals; guard the indices anyway
+      const int ori = best.i == kNoCand ? end_id : best.i;
+      int can_beam = ori / vocab;
+      const int can_vocab = ori % vocab;
+      if (can_beam >= beam_size) can_beam = 0;
+      const int* from = old_alive_seq + ((long)b * beam_size + can_beam) * max_step;
+      int* to = new_alive_seq + ((long)b * beam_size + j) * max_step;
+      for (int t = lane; t < max_step; t += 64)
+        to[t] = t > cur_step + 1 ? end_id : (t == cur_step + 1 ? can_vocab : from[t]);
+      if (lane == 0) {
+        if (can_vocab != end_id) {
+          seq_probs[b * beam_size + j] = (best.s - (float)b * kMinLogProb) / length_norm;
+          parent[b * beam_size + j] = can_beam;
+        } else {
+          seq_score[b * beam_size + j] = best.s;
+          parent[b * beam_size + j] = -1;
+          ++finished;
+        }
+      }
+    }
+  }
+  if (lane == 0) fin_cnt[wid] = finished;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int tot = 0;
+    for (int w2 = 0; w2 < nw; ++w2) tot += fin_cnt[w2];
+    *num_finished = tot;
+  }
+}
+
+template <typename T>
+int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_probs,
+                         float* seq_score, const int* old_alive_seq, int* new_alive_seq,
+                         float* top_score, int* top_idx, int* parent, int* num_finished,
+                         float dequant_scale, int vocab_size, int max_step, float length_norm,
+                         int cur_step, int batch_size, int beam_size, int end_id, hipStream_t s) {
+  if (!logits || !logit_bias || !seq_probs || !seq_score || !old_alive_seq || !new_alive_seq ||
+      !top_score || !top_idx || !parent || !num_finished || vocab_size <= 0 || batch_size <= 0 ||
+      max_step <= 0 || cur_step < 0 || cur_step + 1 >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "beam_search_step: bad arguments");
+  if (beam_size < 1 || beam_size > 32 || (beam_size & (beam_size - 1)))
+    return lsh_fail(LSH_ERR_INVALID, "wrong beam_size, should be 1, 2, 4, 8, 16 or 32");
+  if (old_alive_seq == new_alive_seq)
+    return lsh_fail(LSH_ERR_INVALID, "beam_search_step: the sequence buffers must differ");
+  if ((long)beam_size * vocab_size > 0x7ffffffe)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "beam_search_step: beam_size * vocab_size overflows");
+  beam_topk_kernel<T><<<batch_size * beam_size, 1024, 0, s>>>(
+      logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score, top_idx,
+      vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+  if (int rc = lsh_check_launch("beam_topk_kernel")) return rc;
+  beam_merge_kernel<<<1, 1024, 0, s>>>(top_score, top_idx, old_alive_seq, new_alive_seq,
+                                       seq_probs, seq_score, parent, num_finished, batch_size,
+                                       beam_size, vocab_size, max_step, cur_step, length_norm,
+                                       end_id);
+  return lsh_check_launch("beam_merge_kernel");
+}
+template int beam_search_step_i8I<float>(const int8_t*, const float*, float*, float*, const int*,
+                                         int*, float*, int*, int*, int*, float, int, int, float,
+                                         int, int, int, int, hipStream_t);
+template int beam_search_step_i8I<__half>(const int8_t*, const __half*, float*, float*, const int*,
+                                          int*, float*, int*, int*, int*, float, int, int, float,
+                                          int, int, int, int, hipStream_t);
+
+}  // namespace lsh

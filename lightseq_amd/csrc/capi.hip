@@ -358,4 +358,208 @@ int lsh_quantize_weight_f32(const void* origin_weight, int8_t* quantized_weight,
                                      HS(stream), layout);
 }
 
+// ---- decoder step ------------------------------------------------------------------
+#define LSH_DEC_EMB(NAME, TY, CAST_C, CAST_M, VM)                                              \
+  int NAME(const int8_t* token_emb, const void* pos_emb, const int* tokens,                    \
+           const void* lang_emb, const int* lang_id, void* output, int batch_size,             \
+           int beam_size, int hidden_dim, int vocab_size, int step, int max_step,              \
+           int multilg_type, lsh_stream_t stream, float dequant_scale, int scaled) {           \
+    (void)lang_emb;                                                                            \
+    (void)lang_id;                                                                             \
+    if (multilg_type != 0) return lsh_fail(LSH_ERR_UNSUPPORTED, "multilingle not supported");  \
+    return dec_emb_i8I<TY>(token_emb, CAST_C(pos_emb), tokens, CAST_M(output), batch_size,     \
+                           beam_size, hidden_dim, vocab_size, step, max_step, HS(stream),      \
+                           dequant_scale, scaled != 0, VM);                                    \
+  }
+LSH_DEC_EMB(lsh_launch_dec_emb_i8I_f16, __half, H, HM, false)
+LSH_DEC_EMB(lsh_launch_dec_emb_i8I_f32, float, F, FM, false)
+LSH_DEC_EMB(lsh_launch_dec_emb_i8I_vocab_major_f16, __half, H, HM, true)
+LSH_DEC_EMB(lsh_launch_dec_emb_i8I_vocab_major_f32, float, F, FM, true)
+#undef LSH_DEC_EMB
+
+#define LSH_DECSELF_QKV(NAME, TY, CAST_C)                                                      \
+  int NAME(int step_token_num, int hidden_size, lsh_stream_t stream, const int8_t* ori_qkv,    \
+           const void* qkv_bias, int8_t* new_q, int8_t* new_k, int8_t* new_v, int head_num,    \
+           int dim_per_head, int max_step, int step_id, int max_thread_per_block,              \
+           float dequant_scale, float quant_scale, int in_col32) {                             \
+    (void)max_thread_per_block;                                                                \
+    if (int rc = no_col32(in_col32, 0, "ker_arrange_decself_qkv_i8I_i8O")) return rc;          \
+    return arrange_decself_qkv_i8I_i8O<TY>(step_token_num, hidden_size, HS(stream), ori_qkv,   \
+                                           CAST_C(qkv_bias), new_q, new_k, new_v, head_num,    \
+                                           dim_per_head, max_step, step_id, dequant_scale,     \
+                                           quant_scale);                                       \
+  }
+LSH_DECSELF_QKV(lsh_ker_arrange_decself_qkv_i8I_i8O_f16, __half, H)
+LSH_DECSELF_QKV(lsh_ker_arrange_decself_qkv_i8I_i8O_f32, float, F)
+#undef LSH_DECSELF_QKV
+
+int lsh_decself_scores_i8_i32o(const int8_t* k_cache, const int8_t* q, int32_t* scores,
+                               int batch_head_num, int step_num, int max_step, int dim_per_head,
+                               lsh_stream_t stream) {
+  return decself_scores_i8(q, k_cache, scores, batch_head_num, step_num, max_step, dim_per_head,
+                           HS(stream));
+}
+int lsh_ker_fuse_softmax_new_value_i32I_i8O(const int32_t* correlation, const int8_t* v,
+                                            int8_t* new_v, int batch_head_num, int step_num,
+                                            int max_step, int head_num, int dim_per_head,
+                                            float attn_scale, float dequant_scale,
+                                            float quant_scale, int out_col32,
+                                            lsh_stream_t stream) {
+  if (int rc = no_col32(out_col32, 0, "ker_fuse_softmax_new_value_i32I_i8O")) return rc;
+  return fuse_softmax_new_value_i32I_i8O(correlation, v, new_v, batch_head_num, step_num,
+                                         max_step, head_num, dim_per_head, attn_scale,
+                                         dequant_scale, quant_scale, HS(stream));
+}
+int lsh_decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v_cache,
+                             int8_t* new_v, int batch_head_num, int step_num, int max_step,
+                             int head_num, int dim_per_head, float attn_scale,
+                             float dequant_scale, float quant_scale, lsh_stream_t stream) {
+  return decself_attention_i8(q, k_cache, v_cache, new_v, batch_head_num, step_num, max_step,
+                              head_num, dim_per_head, attn_scale, dequant_scale, quant_scale,
+                              HS(stream));
+}
+
+#define LSH_ENCDEC_Q(NAME, TY, CAST_C, CAST_M)                                                 \
+  int NAME(int step_token_num, int hidden_size, lsh_stream_t stream, const int8_t* ori_q,      \
+           const void* q_bias, void* new_q, int beam_size, int dim_per_head, int head_num,     \
+           int max_thread_per_block, float dequant_scale, int in_col32) {                      \
+    (void)max_thread_per_block;                                                                \
+    if (int rc = no_col32(in_col32, 0, "ker_arrange_encdec_q_i8I")) return rc;                 \
+    return arrange_encdec_q_i8I<TY>(step_token_num, hidden_size, HS(stream), ori_q,            \
+                                    CAST_C(q_bias), CAST_M(new_q), beam_size, dim_per_head,    \
+                                    head_num, dequant_scale);                                  \
+  }
+LSH_ENCDEC_Q(lsh_ker_arrange_encdec_q_i8I_f16, __half, H, HM)
+LSH_ENCDEC_Q(lsh_ker_arrange_encdec_q_i8I_f32, float, F, FM)
+#undef LSH_ENCDEC_Q
+
+#define LSH_ENCDEC_KV(NAME, TY, CAST_C, CAST_M)                                                \
+  int NAME(int batch_token_num, int dec_layer_num, int hidden_size, lsh_stream_t stream,       \
+           const void* ori_kv, const void* kv_bias, void* new_k, void* new_v,                  \
+           int64_t offset_per_layer, int batch_seq_len, int dim_per_head, int head_num,        \
+           int max_thread_per_block) {                                                         \
+    (void)max_thread_per_block;                                                                \
+    return arrange_encdec_kv<TY>(batch_token_num, dec_layer_num, hidden_size, HS(stream),      \
+                                 CAST_C(ori_kv), CAST_C(kv_bias), CAST_M(new_k), CAST_M(new_v), \
+                                 (long)offset_per_layer, batch_seq_len, dim_per_head,          \
+                                 head_num);                                                    \
+  }
+LSH_ENCDEC_KV(lsh_ker_arrange_encdec_kv_f16, __half, H, HM)
+LSH_ENCDEC_KV(lsh_ker_arrange_encdec_kv_f32, float, F, FM)
+#undef LSH_ENCDEC_KV
+
+int lsh_ker_correlation_softmax_encdec_f16(int batch_size, int head_num_per_seq,
+                                           int batch_seq_len, lsh_stream_t stream,
+                                           void* correlation, const int* src_padding_mask) {
+  return correlation_softmax_encdec<__half>(batch_size, head_num_per_seq, batch_seq_len,
+                                            HS(stream), HM(correlation), src_padding_mask);
+}
+int lsh_ker_correlation_softmax_encdec_f32(int batch_size, int head_num_per_seq,
+                                           int batch_seq_len, lsh_stream_t stream,
+                                           void* correlation, const int* src_padding_mask) {
+  return correlation_softmax_encdec<float>(batch_size, head_num_per_seq, batch_seq_len,
+                                           HS(stream), FM(correlation), src_padding_mask);
+}
+int lsh_encdec_attention_f16(const void* q, const void* k, const void* v, const int* pad_mask,
+                             void* ctx, int8_t* ctx_q, float quant_scale, int batch_size,
+                             int beam_size, int head_num, int batch_seq_len, int dim_per_head,
+                             lsh_stream_t stream) {
+  return encdec_attention_f16(H(q), H(k), H(v), pad_mask, HM(ctx), ctx_q, quant_scale, batch_size,
+                              beam_size, head_num, batch_seq_len, dim_per_head, HS(stream));
+}
+int lsh_gemm_f16_nt(const void* A, const void* W, void* C, int m, int n, int k,
+                    lsh_stream_t stream) {
+  return gemm_f16_nt(H(A), H(W), HM(C), m, n, k, HS(stream));
+}
+
+// ---- beam search -------------------------------------------------------------------
+float lsh_length_norm(int length, float alpha) { return length_norm(length, alpha); }
+
+#define LSH_SELECT_BEAM(NAME, TY, CAST_C)                                                      \
+  int NAME(const int8_t* logits, const void* logit_bias, const float* seq_probs,               \
+           const float* seq_score, const int* alive_seq, float dequant_scale, int* can_idx,    \
+           float* can_score, int* num_beam_can, int vocab_size, int max_step,                  \
+           float length_norm_v, int cur_step, int step_token_num, int max_thread_per_block,    \
+           lsh_stream_t stream, int beam_size, float diverse_lambda, int end_id,               \
+           int in_col32) {                                                                     \
+    if (int rc = no_col32(in_col32, 0, "select_beam_rough_topk_i8I")) return rc;               \
+    return select_beam_rough_topk_i8I<TY>(logits, CAST_C(logit_bias), seq_probs, seq_score,    \
+                                          alive_seq, dequant_scale, can_idx, can_score,        \
+                                          num_beam_can, vocab_size, max_step, length_norm_v,   \
+                                          cur_step, step_token_num, max_thread_per_block,      \
+                                          HS(stream), beam_size, diverse_lambda, end_id);      \
+  }
+LSH_SELECT_BEAM(lsh_select_beam_rough_topk_i8I_f16, __half, H)
+LSH_SELECT_BEAM(lsh_select_beam_rough_topk_i8I_f32, float, F)
+#undef LSH_SELECT_BEAM
+
+int lsh_ker_refresh_result(const int* can_idx, const float* can_score,
+                           const int* num_can_per_beam, const int* old_alive_seq,
+                           int* new_alive_seq, float* seq_probs, float* seq_score,
+                           int* num_finish_beam, int vocab_size, int cur_step,
+                           float length_norm_v, float diverse_lambda, int end_id, int batch_size,
+                           int beam_size, int max_step, lsh_stream_t stream) {
+  return refresh_result(can_idx, can_score, num_can_per_beam, old_alive_seq, new_alive_seq,
+                        seq_probs, seq_score, num_finish_beam, vocab_size, cur_step,
+                        length_norm_v, diverse_lambda, end_id, batch_size, beam_size, max_step,
+                        HS(stream));
+}
+int lsh_ker_refresh_cache_i8(int grid_dim_x, int grid_dim_y, int block_dim, lsh_stream_t stream,
+                             const int* num_can_per_beam, const int* can_idx,
+                             const int8_t* self_k_bgeem, const int8_t* self_v_bgeem,
+                             int8_t* new_self_k_bgeem, int8_t* new_self_v_bgeem,
+                             int64_t self_k_bgeem_offset, int beam_size, int dim_per_head,
+                             int head_num, int vocab_size, int cur_step, int max_step,
+                             int diverse, int end_id) {
+  (void)block_dim;
+  return refresh_cache_i8(grid_dim_x, grid_dim_y, HS(stream), num_can_per_beam, can_idx,
+                          self_k_bgeem, self_v_bgeem, new_self_k_bgeem, new_self_v_bgeem,
+                          (long)self_k_bgeem_offset, beam_size, dim_per_head, head_num,
+                          vocab_size, cur_step, max_step, diverse != 0, end_id);
+}
+int lsh_ker_write_trg_tokenid_pos_penalty(const int* alive_seq, float* seq_score, int* output,
+                                          int max_step, int beam_size, int batch_size,
+                                          int out_len, lsh_stream_t stream) {
+  return write_trg_tokenid_pos_penalty(alive_seq, seq_score, output, max_step, beam_size,
+                                       batch_size, out_len, HS(stream));
+}
+int lsh_ker_write_trg_tokenid_neg_penalty(const int* alive_seq, const float* seq_score,
+                                          int* output, int max_step, int beam_size,
+                                          int vocab_size, int end_id, int batch_size, int out_len,
+                                          lsh_stream_t stream) {
+  return write_trg_tokenid_neg_penalty(alive_seq, seq_score, output, max_step, beam_size,
+                                       vocab_size, end_id, batch_size, out_len, HS(stream));
+}
+int lsh_ker_write_topk_result(const int* alive_seq, float* seq_score, int* res_seq,
+                              int vocab_size, int max_step, int beam_size, int end_id,
+                              int batch_beam_num, int out_len, lsh_stream_t stream) {
+  return write_topk_result(alive_seq, seq_score, res_seq, vocab_size, max_step, beam_size, end_id,
+                           batch_beam_num, out_len, HS(stream));
+}
+
+#define LSH_BEAM_STEP(NAME, TY, CAST_C)                                                        \
+  int NAME(const int8_t* logits, const void* logit_bias, float* seq_probs, float* seq_score,   \
+           const int* old_alive_seq, int* new_alive_seq, float* top_score, int* top_idx,       \
+           int* parent, int* num_finished, float dequant_scale, int vocab_size, int max_step,  \
+           float length_norm_v, int cur_step, int batch_size, int beam_size, int end_id,       \
+           lsh_stream_t stream) {                                                              \
+    return beam_search_step_i8I<TY>(logits, CAST_C(logit_bias), seq_probs, seq_score,          \
+                                    old_alive_seq, new_alive_seq, top_score, top_idx, parent,  \
+                                    num_finished, dequant_scale, vocab_size, max_step,         \
+                                    length_norm_v, cur_step, batch_size, beam_size, end_id,    \
+                                    HS(stream));                                               \
+  }
+LSH_BEAM_STEP(lsh_beam_search_step_i8I_f16, __half, H)
+LSH_BEAM_STEP(lsh_beam_search_step_i8I_f32, float, F)
+#undef LSH_BEAM_STEP
+
+int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, const int* parent,
+                                   const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
+                                   int8_t* v_new, int64_t layer_offset, int beam_size,
+                                   int dim_per_head, int head_num, int cur_step, int max_step) {
+  return refresh_cache_by_parent_i8(n_layer, rows, HS(stream), parent, k_old, v_old, k_new, v_new,
+                                    (long)layer_offset, beam_size, dim_per_head, head_num,
+                                    cur_step, max_step);
+}
+
 }  // extern "C"

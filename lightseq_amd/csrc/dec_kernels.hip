@@ -1,0 +1,452 @@
+// Decoder-step kernels: target embedding, the int8 self-attention against the
+// K/V cache, and the fp16 attention over the projected encoder output.
+//
+// One decoding step handles rows = batch * beam_size query vectors, so every kernel
+// here is small and latency-bound: the layout goal is few launches and coalesced
+// rows, not tiling.  A wavefront owns one (row, head) pair in the attention kernels;
+// all cross-lane traffic is wave reductions, and sums run in a fixed order so that a
+// step is reproducible bit for bit.
+#include "ls_device.cuh"
+#include "ls_launch.h"
+
+namespace lsh {
+
+// ---------------------------------------------------------------------------------
+// target embedding (inference/kernels/embKernels_int8.cc.cu:158-200)
+// ---------------------------------------------------------------------------------
+template <typename T, bool VOCAB_MAJOR>
+__global__ void __launch_bounds__(256)
+dec_emb_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__ pos_emb,
+               const int* __restrict__ tokens, T* __restrict__ out, int rows, int hidden,
+               int vocab, int step, int max_step, float scale) {
+#pragma clang fp contract(off)
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)rows * hidden) return;
+  const int r = (int)(idx / hidden), i = (int)(idx % hidden);
+  int token = tokens[(long)r * max_step + step];
+  token = min(max(token, 0), vocab - 1);  // never index outside the table
+  const int8_t e =
+      VOCAB_MAJOR ? token_emb[(long)token * hidden + i] : token_emb[(long)i * vocab + token];
+  const float v = (float)e * scale + TT<T>::ld(pos_emb, (long)step * hidden + i);
+  TT<T>::st(out, idx, v);
+}
+
+template <typename T>
+int dec_emb_i8I(const int8_t* token_emb, const T* pos_emb, const int* tokens, T* output,
+                int batch_size, int beam_size, int hidden_dim, int vocab_size, int step,
+                int max_step, hipStream_t s, float dequant_scale, bool scaled, bool vocab_major) {
+  if (!token_emb || !pos_emb || !tokens || !output || batch_size <= 0 || beam_size <= 0 ||
+      hidden_dim <= 0 || vocab_size <= 0 || max_step <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "launch_dec_emb_i8I: bad arguments");
+  if (step < 0 || step >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "violate step < max_step");
+  const int rows = batch_size * beam_size;
+  float scale = dequant_scale;
+  if (scaled) scale *= sqrtf((float)hidden_dim);
+  const long n = (long)rows * hidden_dim;
+  const int grid = (int)((n + 255) / 256);
+  if (vocab_major)
+    dec_emb_kernel<T, true><<<grid, 256, 0, s>>>(token_emb, pos_emb, tokens, output, rows,
+                                                 hidden_dim, vocab_size, step, max_step, scale);
+  else
+    dec_emb_kernel<T, false><<<grid, 256, 0, s>>>(token_emb, pos_emb, tokens, output, rows,
+                                                  hidden_dim, vocab_size, step, max_step, scale);
+  return lsh_check_launch("dec_emb_kernel");
+}
+template int dec_emb_i8I<float>(const int8_t*, const float*, const int*, float*, int, int, int,
+                                int, int, int, hipStream_t, float, bool, bool);
+template int dec_emb_i8I<__half>(const int8_t*, const __half*, const int*, __half*, int, int, int,
+                                 int, int, int, hipStream_t, float, bool, bool);
+
+// ---------------------------------------------------------------------------------
+// split QKV of the current step: q -> [rows, H] int8, k / v -> cache slot `step_id`
+// (inference/kernels/transformerKernels_int8.cc.cu:1395-1499).  The bias is added
+// in float for both storage types, as the reference does here.
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+arrange_decself_qkv_kernel(const int8_t* __restrict__ ori_qkv, const T* __restrict__ qkv_bias,
+                           int8_t* __restrict__ new_q, int8_t* __restrict__ new_k,
+                           int8_t* __restrict__ new_v, int head_num, int dim_per_head,
+                           int max_step, int step_id, float dequant_scale, float quant_scale) {
+#pragma clang fp contract(off)
+  const int H = head_num * dim_per_head;
+  const int row = blockIdx.x, part = blockIdx.y;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float val = (float)ori_qkv[((long)row * 3 + part) * H + i] * dequant_scale +
+                      TT<T>::ld(qkv_bias, (long)part * H + i);
+    const int8_t qv = (int8_t)float2int8(val, quant_scale);
+    if (part == 0) {
+      new_q[(long)row * H + i] = qv;
+    } else {
+      const int head = i / dim_per_head, dim = i % dim_per_head;
+      const long t = (((long)row * head_num + head) * max_step + step_id) * dim_per_head + dim;
+      (part == 1 ? new_k : new_v)[t] = qv;
+    }
+  }
+}
+
+template <typename T>
+int arrange_decself_qkv_i8I_i8O(int step_token_num, int hidden_size, hipStream_t s,
+                                const int8_t* ori_qkv, const T* qkv_bias, int8_t* new_q,
+                                int8_t* new_k, int8_t* new_v, int head_num, int dim_per_head,
+                                int max_step, int step_id, float dequant_scale,
+                                float quant_scale) {
+  if (!ori_qkv || !qkv_bias || !new_q || !new_k || !new_v || step_token_num <= 0 ||
+      head_num <= 0 || dim_per_head <= 0 || hidden_size != head_num * dim_per_head)
+    return lsh_fail(LSH_ERR_INVALID, "ker_arrange_decself_qkv_i8I_i8O: bad arguments");
+  if (step_id < 0 || step_id >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "ker_arrange_decself_qkv_i8I_i8O: step_id outside the cache");
+  arrange_decself_qkv_kernel<T><<<dim3(step_token_num, 3), 256, 0, s>>>(
+      ori_qkv, qkv_bias, new_q, new_k, new_v, head_num, dim_per_head, max_step, step_id,
+      dequant_scale, quant_scale);
+  return lsh_check_launch("arrange_decself_qkv_kernel");
+}
+template int arrange_decself_qkv_i8I_i8O<float>(int, int, hipStream_t, const int8_t*, const float*,
+                                                int8_t*, int8_t*, int8_t*, int, int, int, int,
+                                                float, float);
+template int arrange_decself_qkv_i8I_i8O<__half>(int, int, hipStream_t, const int8_t*,
+                                                 const __half*, int8_t*, int8_t*, int8_t*, int,
+                                                 int, int, int, float, float);
+
+// ---------------------------------------------------------------------------------
+// decoder self attention over the int8 cache
+//   scores[j]  = sum_d q[d] * K[j][d]                      (int32, exact)
+//   val[j]     = float(scores[j]) * dq * dq * attn_scale
+//   p[j]       = exp(val[j] - max) / sum
+//   out[d]     = float2int8(sum_j float(V[j][d]) * p[j] * dq, quant_scale)
+// (inference/model/quant_decoder.cc.cu:676-700 and
+//  inference/kernels/transformerKernels_int8.cc.cu:1515-1594).
+// One wavefront per (row, head); the value sum runs over j in ascending order.
+// MODE 0: write the int32 scores only; 1: read scores, write new value; 2: fused.
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ int dot_i8_row(const int8_t* __restrict__ a,
+                                          const int8_t* __restrict__ b, int d) {
+  int acc = 0;
+  if ((d & 3) == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 3) == 0) {
+    const uint32_t* aw = reinterpret_cast<const uint32_t*>(a);
+    const uint32_t* bw = reinterpret_cast<const uint32_t*>(b);
+    for (int w = 0; w < (d >> 2); ++w) {
+      const uint32_t x = aw[w], y = bw[w];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) acc += unpack_i8(x, k) * unpack_i8(y, k);
+    }
+  } else {
+    for (int k = 0; k < d; ++k) acc += (int)a[k] * (int)b[k];
+  }
+  return acc;
+}
+
+template <int MODE>
+__global__ void __launch_bounds__(256)
+decself_attn_kernel(int32_t* __restrict__ scores, const int8_t* __restrict__ q,
+                    const int8_t* __restrict__ k_cache, const int8_t* __restrict__ v_cache,
+                    int8_t* __restrict__ new_v, long bh_total, int step_num, int max_step,
+                    int head_num, int d, float attn_scale, float dq, float quant_scale) {
+#pragma clang fp contract(off)
+  extern __shared__ float probs_all[];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const long bh = (long)blockIdx.x * 4 + wid;
+  if (bh >= bh_total) return;  // whole wavefronts leave; no block barrier below
+  const int padded = (step_num + 63) & ~63;
+  float* probs = probs_all + (long)wid * padded;
+  const int8_t* kb = k_cache + bh * (long)max_step * d;
+  const int8_t* vb = v_cache + bh * (long)max_step * d;
+
+  float mx = kFloatInfNeg;
+  for (int j = lane; j < padded; j += 64) {
+    float val = kFloatInfNeg;
+    if (j < step_num) {
+      int sc;
+      if (MODE == 1) {
+        sc = scores[bh * max_step + j];
+      } else {
+        sc = dot_i8_row(q + bh * d, kb + (long)j * d, d);
+        if (MODE == 0) scores[bh * max_step + j] = sc;
+      }
+      val = (float)sc * dq * dq * attn_scale;
+    }
+    if (MODE != 0) probs[j] = val;
+    mx = fmaxf(mx, val);
+  }
+  if (MODE == 0) return;
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int j = lane; j < padded; j += 64) {
+    const float e = j < step_num ? __expf(probs[j] - mx) : 0.f;
+    probs[j] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  for (int j = lane; j < padded; j += 64) probs[j] = probs[j] / sum;
+  // each lane re-reads values written by other lanes of its own wavefront
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const long row = bh / head_num;
+  const int head = (int)(bh % head_num);
+  for (int dd = lane; dd < d; dd += 64) {
+    float acc = 0.f;
+    for (int j = 0; j < step_num; ++j) acc += (float)vb[(long)j * d + dd] * probs[j] * dq;
+    new_v[row * ((long)head_num * d) + (long)head * d + dd] = (int8_t)float2int8(acc, quant_scale);
+  }
+}
+
+static int decself_check(long bh_total, int step_num, int max_step, int head_num, int d) {
+  if (bh_total <= 0 || head_num <= 0 || d <= 0 || max_step <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "decoder self attention: bad shape");
+  if (step_num <= 0 || step_num > max_step)
+    return lsh_fail(LSH_ERR_INVALID, "decoder self attention: step_num outside the cache");
+  if (max_step > 4096)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "decoder self attention: max_step above 4096");
+  return LSH_OK;
+}
+
+static size_t decself_lds(int step_num) { return (size_t)4 * ((step_num + 63) & ~63) * sizeof(float); }
+
+int decself_scores_i8(const int8_t* q, const int8_t* k_cache, int32_t* scores, int batch_head_num,
+                      int step_num, int max_step, int dim_per_head, hipStream_t s) {
+  if (!q || !k_cache || !scores) return lsh_fail(LSH_ERR_INVALID, "decself_scores: null pointer");
+  if (int rc = decself_check(batch_head_num, step_num, max_step, 1, dim_per_head)) return rc;
+  decself_attn_kernel<0><<<(batch_head_num + 3) / 4, 256, 0, s>>>(
+      scores, q, k_cache, nullptr, nullptr, batch_head_num, step_num, max_step, 1, dim_per_head,
+      0.f, 0.f, 0.f);
+  return lsh_check_launch("decself_attn_kernel<0>");
+}
+
+int fuse_softmax_new_value_i32I_i8O(const int32_t* correlation, const int8_t* v, int8_t* new_v,
+                                    int batch_head_num, int step_num, int max_step, int head_num,
+                                    int dim_per_head, float attn_scale, float dequant_scale,
+                                    float quant_scale, hipStream_t s) {
+  if (!correlation || !v || !new_v)
+    return lsh_fail(LSH_ERR_INVALID, "ker_fuse_softmax_new_value_i32I_i8O: null pointer");
+  if (int rc = decself_check(batch_head_num, step_num, max_step, head_num, dim_per_head)) return rc;
+  decself_attn_kernel<1><<<(batch_head_num + 3) / 4, 256, decself_lds(step_num), s>>>(
+      const_cast<int32_t*>(correlation), nullptr, nullptr, v, new_v, batch_head_num, step_num,
+      max_step, head_num, dim_per_head, attn_scale, dequant_scale, quant_scale);
+  return lsh_check_launch("decself_attn_kernel<1>");
+}
+
+int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v_cache,
+                         int8_t* new_v, int batch_head_num, int step_num, int max_step,
+                         int head_num, int dim_per_head, float attn_scale, float dequant_scale,
+                         float quant_scale, hipStream_t s) {
+  if (!q || !k_cache || !v_cache || !new_v)
+    return lsh_fail(LSH_ERR_INVALID, "decself_attention: null pointer");
+  if (int rc = decself_check(batch_head_num, step_num, max_step, head_num, dim_per_head)) return rc;
+  decself_attn_kernel<2><<<(batch_head_num + 3) / 4, 256, decself_lds(step_num), s>>>(
+      nullptr, q, k_cache, v_cache, new_v, batch_head_num, step_num, max_step, head_num,
+      dim_per_head, attn_scale, dequant_scale, quant_scale);
+  return lsh_check_launch("decself_attn_kernel<2>");
+}
+
+// ---------------------------------------------------------------------------------
+// encoder-decoder attention: query re-layout
+// (inference/kernels/transformerKernels_int8.cc.cu:1596-1688)
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+arrange_encdec_q_kernel(const int8_t* __restrict__ ori_q, const T* __restrict__ q_bias,
+                        T* __restrict__ new_q, int beam_size, int dim_per_head, int head_num,
+                        float dequant_scale) {
+#pragma clang fp contract(off)
+  const int H = dim_per_head * head_num;
+  const int row = blockIdx.x;
+  const int batch_id = row / beam_size, beam_id = row % beam_size;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    // fp16: half(code * dq) + bias as a half add; fp32: plain float arithmetic
+    const int code = ori_q[(long)row * H + i];
+    const float bias = TT<T>::ld(q_bias, i);
+    const float val = TT<T>::is_half ? dequant_add_bias_h(code, dequant_scale, bias)
+                                     : (float)code * dequant_scale + bias;
+    const int head = i / dim_per_head, dim = i % dim_per_head;
+    TT<T>::st(new_q,
+              (((long)batch_id * head_num + head) * beam_size + beam_id) * dim_per_head + dim, val);
+  }
+}
+
+template <typename T>
+int arrange_encdec_q_i8I(int step_token_num, int hidden_size, hipStream_t s, const int8_t* ori_q,
+                         const T* q_bias, T* new_q, int beam_size, int dim_per_head, int head_num,
+                         float dequant_scale) {
+  if (!ori_q || !q_bias || !new_q || step_token_num <= 0 || beam_size <= 0 ||
+      step_token_num % beam_size != 0 || hidden_size != dim_per_head * head_num)
+    return lsh_fail(LSH_ERR_INVALID, "ker_arrange_encdec_q_i8I: bad arguments");
+  arrange_encdec_q_kernel<T><<<step_token_num, 256, 0, s>>>(ori_q, q_bias, new_q, beam_size,
+                                                            dim_per_head, head_num, dequant_scale);
+  return lsh_check_launch("arrange_encdec_q_kernel");
+}
+template int arrange_encdec_q_i8I<float>(int, int, hipStream_t, const int8_t*, const float*, float*,
+                                         int, int, int, float);
+template int arrange_encdec_q_i8I<__half>(int, int, hipStream_t, const int8_t*, const __half*,
+                                          __half*, int, int, int, float);
+
+// ---------------------------------------------------------------------------------
+// projected encoder output -> per-layer K and V in [batch, head, seq, dim]
+// (inference/kernels/transformerKernels.cc.cu:903-1020)
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+arrange_encdec_kv_kernel(const T* __restrict__ ori_kv, const T* __restrict__ kv_bias,
+                         T* __restrict__ new_k, T* __restrict__ new_v, long offset_per_layer,
+                         int batch_seq_len, int dim_per_head, int head_num) {
+  const int H = dim_per_head * head_num;
+  const long tok = blockIdx.x;
+  const int y = blockIdx.y;
+  const long seq_id = tok / batch_seq_len, token_id = tok % batch_seq_len;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float val = TT<T>::ld(ori_kv, (tok * gridDim.y + y) * H + i) +
+                      TT<T>::ld(kv_bias, (long)y * H + i);  // rounded to T by the store
+    const int head = i / dim_per_head, dim = i % dim_per_head;
+    const long t = ((seq_id * head_num + head) * batch_seq_len + token_id) * dim_per_head + dim +
+                   (long)(y >> 1) * offset_per_layer;
+    TT<T>::st((y & 1) ? new_v : new_k, t, val);
+  }
+}
+
+template <typename T>
+int arrange_encdec_kv(int batch_token_num, int dec_layer_num, int hidden_size, hipStream_t s,
+                      const T* ori_kv, const T* kv_bias, T* new_k, T* new_v,
+                      long offset_per_layer, int batch_seq_len, int dim_per_head, int head_num) {
+  if (!ori_kv || !kv_bias || !new_k || !new_v || batch_token_num <= 0 || dec_layer_num <= 0 ||
+      batch_seq_len <= 0 || batch_token_num % batch_seq_len != 0 ||
+      hidden_size != dim_per_head * head_num)
+    return lsh_fail(LSH_ERR_INVALID, "ker_arrange_encdec_kv: bad arguments");
+  if (dec_layer_num * 2 > 65535)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "ker_arrange_encdec_kv: too many layers");
+  if (offset_per_layer < (long)batch_token_num * hidden_size)
+    return lsh_fail(LSH_ERR_INVALID, "ker_arrange_encdec_kv: layers would overlap");
+  arrange_encdec_kv_kernel<T><<<dim3(batch_token_num, dec_layer_num * 2), 256, 0, s>>>(
+      ori_kv, kv_bias, new_k, new_v, offset_per_layer, batch_seq_len, dim_per_head, head_num);
+  return lsh_check_launch("arrange_encdec_kv_kernel");
+}
+template int arrange_encdec_kv<float>(int, int, int, hipStream_t, const float*, const float*,
+                                      float*, float*, long, int, int, int);
+template int arrange_encdec_kv<__half>(int, int, int, hipStream_t, const __half*, const __half*,
+                                       __half*, __half*, long, int, int, int);
+
+// ---------------------------------------------------------------------------------
+// softmax of the encoder-decoder correlation, keys masked by the source padding
+// (inference/kernels/transformerKernels.cc.cu:1226-1284); one wavefront per row
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+softmax_encdec_kernel(T* corr, const int* __restrict__ pad_mask, long rows, int rows_per_batch,
+                      int seq_len) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int* mask = pad_mask + (row / rows_per_batch) * seq_len;
+  T* p = corr + row * seq_len;
+  float mx = kFloatInfNeg;
+  for (int j = lane; j < seq_len; j += 64)
+    if (!mask[j]) mx = fmaxf(mx, TT<T>::ld(p, j));
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int j = lane; j < seq_len; j += 64)
+    if (!mask[j]) sum += __expf(TT<T>::ld(p, j) - mx);
+  sum = wave_sum(sum);
+  for (int j = lane; j < seq_len; j += 64) {
+    const float e = mask[j] ? 0.f : __expf(TT<T>::ld(p, j) - mx);
+    TT<T>::st(p, j, e / sum);
+  }
+}
+
+template <typename T>
+int correlation_softmax_encdec(int batch_size, int head_num_per_seq, int batch_seq_len,
+                               hipStream_t s, T* correlation, const int* src_padding_mask) {
+  if (!correlation || !src_padding_mask || batch_size <= 0 || head_num_per_seq <= 0 ||
+      batch_seq_len <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "ker_correlation_softmax_encdec: bad arguments");
+  const long rows = (long)batch_size * head_num_per_seq;
+  softmax_encdec_kernel<T><<<(int)((rows + 3) / 4), 256, 0, s>>>(
+      correlation, src_padding_mask, rows, head_num_per_seq, batch_seq_len);
+  return lsh_check_launch("softmax_encdec_kernel");
+}
+template int correlation_softmax_encdec<float>(int, int, int, hipStream_t, float*, const int*);
+template int correlation_softmax_encdec<__half>(int, int, int, hipStream_t, __half*, const int*);
+
+// ---------------------------------------------------------------------------------
+// Fused encoder-decoder attention (fp16), one wavefront per (batch, head, beam):
+//   s[j] = half(half(1/sqrt(d)) * sum_d q[d] k[j][d]);  p = half(masked softmax(s));
+//   c[d] = half(sum_j p[j] v[j][d]);  out = float2int8(c, quant_scale) in [rows, H]
+// i.e. the two strided-batched GEMMs, ker_correlation_softmax_encdec and
+// ker_arrange_atten_output_i8O of inference/model/quant_decoder.cc.cu:765-800 with
+// their fp16 rounding points kept.
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+encdec_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
+                   const __half* __restrict__ v, const int* __restrict__ pad_mask,
+                   __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale,
+                   long waves_total, int beam_size, int head_num, int seq_len, int d,
+                   float alpha_h) {
+#pragma clang fp contract(off)
+  extern __shared__ float probs_all[];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const long w = (long)blockIdx.x * 4 + wid;
+  if (w >= waves_total) return;
+  const int padded = (seq_len + 63) & ~63;
+  float* probs = probs_all + (long)wid * padded;
+  const long bh = w / beam_size;
+  const int beam = (int)(w % beam_size);
+  const long b = bh / head_num;
+  const int head = (int)(bh % head_num);
+  const int* mask = pad_mask + b * seq_len;
+  const __half* qp = q + w * d;  // [B, h, beam, d]
+  const __half* kb = k + bh * (long)seq_len * d;
+  const __half* vb = v + bh * (long)seq_len * d;
+
+  float mx = kFloatInfNeg;
+  for (int j = lane; j < padded; j += 64) {
+    float sc = kFloatInfNeg;
+    if (j < seq_len) {
+      float acc = 0.f;
+      const __half* kr = kb + (long)j * d;
+      for (int dd = 0; dd < d; ++dd) acc += __half2float(qp[dd]) * __half2float(kr[dd]);
+      sc = TT<__half>::rnd(alpha_h * acc);
+      if (!mask[j]) mx = fmaxf(mx, sc);
+    }
+    probs[j] = sc;
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int j = lane; j < padded; j += 64) {
+    const float e = (j < seq_len && !mask[j]) ? __expf(probs[j] - mx) : 0.f;
+    probs[j] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  for (int j = lane; j < padded; j += 64) probs[j] = TT<__half>::rnd(probs[j] / sum);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const long row = b * beam_size + beam;
+  for (int dd = lane; dd < d; dd += 64) {
+    float acc = 0.f;
+    for (int j = 0; j < seq_len; ++j) acc += probs[j] * __half2float(vb[(long)j * d + dd]);
+    const float c = TT<__half>::rnd(acc);
+    if (ctx) ctx[w * d + dd] = __float2half_rn(c);
+    if (ctx_q)
+      ctx_q[row * ((long)head_num * d) + (long)head * d + dd] = (int8_t)float2int8(c, quant_scale);
+  }
+}
+
+int encdec_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,
+                         __half* ctx, int8_t* ctx_q, float quant_scale, int batch_size,
+                         int beam_size, int head_num, int batch_seq_len, int dim_per_head,
+                         hipStream_t s) {
+  if (!q || !k || !v || !pad_mask || (!ctx && !ctx_q) || batch_size <= 0 || beam_size <= 0 ||
+      head_num <= 0 || batch_seq_len <= 0 || dim_per_head <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "encdec_attention: bad arguments");
+  if (batch_seq_len > 4096)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "encdec_attention: source length above 4096");
+  const long waves = (long)batch_size * head_num * beam_size;
+  const float alpha_h = __half2float(__float2half_rn(sqrtf(1.f / (float)dim_per_head)));
+  const size_t lds = (size_t)4 * ((batch_seq_len + 63) & ~63) * sizeof(float);
+  encdec_attn_kernel<<<(int)((waves + 3) / 4), 256, lds, s>>>(
+      q, k, v, pad_mask, ctx, ctx_q, quant_scale, waves, beam_size, head_num, batch_seq_len,
+      dim_per_head, alpha_h);
+  return lsh_check_launch("encdec_attn_kernel");
+}
+
+}  // namespace lsh

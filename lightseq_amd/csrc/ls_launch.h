@@ -7,6 +7,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cmath>
 #include <string>
 
 #include "../../include/lightseq_hip.h"
@@ -117,5 +118,88 @@ const char* gemm_i8_act_epilogue_name(int act);
 // The next int8 GEMM launched from this thread records kernel-exact begin / end
 // timestamps into the two events (hipExtLaunchKernelGGL), then the hook clears itself.
 void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop);
+
+// ---- fp16 MFMA GEMM (gemm_f16.hip) ------------------------------------------------------
+int gemm_f16_nt(const __half* A, const __half* W, __half* C, int M, int N, int K, hipStream_t s);
+
+// ---- decoder step (dec_kernels.hip) -----------------------------------------------------
+template <typename T>
+int dec_emb_i8I(const int8_t* token_emb, const T* pos_emb, const int* tokens, T* output,
+                int batch_size, int beam_size, int hidden_dim, int vocab_size, int step,
+                int max_step, hipStream_t s, float dequant_scale, bool scaled, bool vocab_major);
+template <typename T>
+int arrange_decself_qkv_i8I_i8O(int step_token_num, int hidden_size, hipStream_t s,
+                                const int8_t* ori_qkv, const T* qkv_bias, int8_t* new_q,
+                                int8_t* new_k, int8_t* new_v, int head_num, int dim_per_head,
+                                int max_step, int step_id, float dequant_scale,
+                                float quant_scale);
+int decself_scores_i8(const int8_t* q, const int8_t* k_cache, int32_t* scores, int batch_head_num,
+                      int step_num, int max_step, int dim_per_head, hipStream_t s);
+int fuse_softmax_new_value_i32I_i8O(const int32_t* correlation, const int8_t* v, int8_t* new_v,
+                                    int batch_head_num, int step_num, int max_step, int head_num,
+                                    int dim_per_head, float attn_scale, float dequant_scale,
+                                    float quant_scale, hipStream_t s);
+int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v_cache,
+                         int8_t* new_v, int batch_head_num, int step_num, int max_step,
+                         int head_num, int dim_per_head, float attn_scale, float dequant_scale,
+                         float quant_scale, hipStream_t s);
+template <typename T>
+int arrange_encdec_q_i8I(int step_token_num, int hidden_size, hipStream_t s, const int8_t* ori_q,
+                         const T* q_bias, T* new_q, int beam_size, int dim_per_head, int head_num,
+                         float dequant_scale);
+template <typename T>
+int arrange_encdec_kv(int batch_token_num, int dec_layer_num, int hidden_size, hipStream_t s,
+                      const T* ori_kv, const T* kv_bias, T* new_k, T* new_v,
+                      long offset_per_layer, int batch_seq_len, int dim_per_head, int head_num);
+template <typename T>
+int correlation_softmax_encdec(int batch_size, int head_num_per_seq, int batch_seq_len,
+                               hipStream_t s, T* correlation, const int* src_padding_mask);
+int encdec_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,
+                         __half* ctx, int8_t* ctx_q, float quant_scale, int batch_size,
+                         int beam_size, int head_num, int batch_seq_len, int dim_per_head,
+                         hipStream_t s);
+
+// ---- beam search (beam_kernels.hip) -------------------------------------------------------
+template <typename T>
+int select_beam_rough_topk_i8I(const int8_t* logits, const T* logit_bias, const float* seq_probs,
+                               const float* seq_score, const int* alive_seq, float dequant_scale,
+                               int* can_idx, float* can_score, int* num_beam_can, int vocab_size,
+                               int max_step, float length_norm, int cur_step, int step_token_num,
+                               int max_thread_per_block, hipStream_t s, int beam_size,
+                               float diverse_lambda, int end_id);
+int refresh_result(const int* can_idx, const float* can_score, const int* num_can_per_beam,
+                   const int* old_alive_seq, int* new_alive_seq, float* seq_probs,
+                   float* seq_score, int* num_finish_beam, int vocab_size, int cur_step,
+                   float length_norm, float diverse_lambda, int end_id, int batch_size,
+                   int beam_size, int max_step, hipStream_t s);
+int refresh_cache_i8(int n_layer, int rows_x2, hipStream_t s, const int* num_can_per_beam,
+                     const int* can_idx, const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
+                     int8_t* v_new, long layer_offset, int beam_size, int dim_per_head,
+                     int head_num, int vocab_size, int cur_step, int max_step, bool diverse,
+                     int end_id);
+int refresh_cache_by_parent_i8(int n_layer, int rows, hipStream_t s, const int* parent,
+                               const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
+                               int8_t* v_new, long layer_offset, int beam_size, int dim_per_head,
+                               int head_num, int cur_step, int max_step);
+int write_trg_tokenid_pos_penalty(const int* alive_seq, float* seq_score, int* output,
+                                  int max_step, int beam_size, int batch_size, int out_len,
+                                  hipStream_t s);
+int write_trg_tokenid_neg_penalty(const int* alive_seq, const float* seq_score, int* output,
+                                  int max_step, int beam_size, int vocab_size, int end_id,
+                                  int batch_size, int out_len, hipStream_t s);
+int write_topk_result(const int* alive_seq, float* seq_score, int* res_seq, int vocab_size,
+                      int max_step, int beam_size, int end_id, int rows, int out_len,
+                      hipStream_t s);
+template <typename T>
+int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_probs,
+                         float* seq_score, const int* old_alive_seq, int* new_alive_seq,
+                         float* top_score, int* top_idx, int* parent, int* num_finished,
+                         float dequant_scale, int vocab_size, int max_step, float length_norm,
+                         int cur_step, int batch_size, int beam_size, int end_id, hipStream_t s);
+// inference/kernels/transformerKernels.h:137-140
+inline float length_norm(int length, float alpha) {
+  if (alpha < 0.f) return 1.f / length;
+  return std::pow((5.f + length) / 6.f, -alpha);
+}
 
 }  // namespace lsh

@@ -202,5 +202,184 @@ def quantize_weight(host_weight, dev_q, rows, cols, quant_scale, layout):
          quant_scale, current_stream(), layout)
 
 
-__all__ = [n for n in dir() if n.startswith(("launch_", "ker_", "gemm_", "encself_", "quantize_"))]
+# --------------------------------------------------------------------------- #
+# decoder step
+# --------------------------------------------------------------------------- #
+def launch_dec_emb_i8I(token_emb, pos_emb, tokens, lang_emb, lang_id, output, batch_size,
+                       beam_size, hidden_dim, vocab_size, step, max_step, multilg_type,
+                       dequant_scale, scaled, vocab_major=False):
+    """``vocab_major``: ``token_emb`` is [vocab, hidden] instead of the reference's
+    [hidden, vocab]."""
+    _dev(token_emb, pos_emb, tokens, output)
+    name = "lsh_launch_dec_emb_i8I_vocab_major" if vocab_major else "lsh_launch_dec_emb_i8I"
+    call(name + _suffix(output), ptr(token_emb), ptr(pos_emb), ptr(tokens), ptr(lang_emb),
+         ptr(lang_id), ptr(output), batch_size, beam_size, hidden_dim, vocab_size, step, max_step,
+         multilg_type, current_stream(), dequant_scale, int(scaled))
+
+
+def ker_arrange_decself_qkv_i8I_i8O_launcher(step_token_num, hidden_size, ori_qkv, qkv_bias, new_q,
+                                             new_k, new_v, head_num, dim_per_head, max_step,
+                                             step_id, max_thread_per_block, dequant_scale,
+                                             quant_scale, in_col32=False):
+    _dev(ori_qkv, qkv_bias, new_q, new_k, new_v)
+    call("lsh_ker_arrange_decself_qkv_i8I_i8O" + _suffix(qkv_bias), step_token_num, hidden_size,
+         current_stream(), ptr(ori_qkv), ptr(qkv_bias), ptr(new_q), ptr(new_k), ptr(new_v),
+         head_num, dim_per_head, max_step, step_id, max_thread_per_block, dequant_scale,
+         quant_scale, int(in_col32))
+
+
+def decself_scores_i8_i32o(k_cache, q, scores, batch_head_num, step_num, max_step, dim_per_head):
+    _dev(k_cache, q, scores)
+    call("lsh_decself_scores_i8_i32o", ptr(k_cache), ptr(q), ptr(scores), batch_head_num, step_num,
+         max_step, dim_per_head, current_stream())
+
+
+def ker_fuse_softmax_new_value_i32I_i8O_launcher(correlation, v, new_v, batch_head_num, step_num,
+                                                 max_step, head_num, dim_per_head, attn_scale,
+                                                 dequant_scale, quant_scale, out_col32=False):
+    _dev(correlation, v, new_v)
+    call("lsh_ker_fuse_softmax_new_value_i32I_i8O", ptr(correlation), ptr(v), ptr(new_v),
+         batch_head_num, step_num, max_step, head_num, dim_per_head, attn_scale, dequant_scale,
+         quant_scale, int(out_col32), current_stream())
+
+
+def decself_attention_i8(q, k_cache, v_cache, new_v, batch_head_num, step_num, max_step, head_num,
+                         dim_per_head, attn_scale, dequant_scale, quant_scale):
+    """Scores + softmax + new value of the decoder self attention in one kernel."""
+    _dev(q, k_cache, v_cache, new_v)
+    call("lsh_decself_attention_i8", ptr(q), ptr(k_cache), ptr(v_cache), ptr(new_v),
+         batch_head_num, step_num, max_step, head_num, dim_per_head, attn_scale, dequant_scale,
+         quant_scale, current_stream())
+
+
+def ker_arrange_encdec_q_i8I_launcher(step_token_num, hidden_size, ori_q, q_bias, new_q, beam_size,
+                                      dim_per_head, head_num, max_thread_per_block, dequant_scale,
+                                      in_col32=False):
+    _dev(ori_q, q_bias, new_q)
+    call("lsh_ker_arrange_encdec_q_i8I" + _suffix(new_q), step_token_num, hidden_size,
+         current_stream(), ptr(ori_q), ptr(q_bias), ptr(new_q), beam_size, dim_per_head, head_num,
+         max_thread_per_block, dequant_scale, int(in_col32))
+
+
+def ker_arrange_encdec_kv_launcher(batch_token_num, dec_layer_num, hidden_size, ori_kv, kv_bias,
+                                   new_k, new_v, offset_per_layer, batch_seq_len, dim_per_head,
+                                   head_num, max_thread_per_block):
+    _dev(ori_kv, kv_bias, new_k, new_v)
+    call("lsh_ker_arrange_encdec_kv" + _suffix(ori_kv), batch_token_num, dec_layer_num,
+         hidden_size, current_stream(), ptr(ori_kv), ptr(kv_bias), ptr(new_k), ptr(new_v),
+         offset_per_layer, batch_seq_len, dim_per_head, head_num, max_thread_per_block)
+
+
+def ker_correlation_softmax_encdec_launcher(batch_size, head_num_per_seq, batch_seq_len,
+                                            correlation, src_padding_mask):
+    _dev(correlation, src_padding_mask)
+    call("lsh_ker_correlation_softmax_encdec" + _suffix(correlation), batch_size, head_num_per_seq,
+         batch_seq_len, current_stream(), ptr(correlation), ptr(src_padding_mask))
+
+
+def encdec_attention(q, k, v, pad_mask, ctx, ctx_q, quant_scale, batch_size, beam_size, head_num,
+                     batch_seq_len, dim_per_head):
+    """Fused encoder-decoder attention of one decoder layer (fp16 only)."""
+    _dev(q, k, v, pad_mask, ctx, ctx_q)
+    if q.dtype != torch.float16:
+        raise TypeError("encdec_attention is fp16 only")
+    call("lsh_encdec_attention_f16", ptr(q), ptr(k), ptr(v), ptr(pad_mask), ptr(ctx), ptr(ctx_q),
+         quant_scale, batch_size, beam_size, head_num, batch_seq_len, dim_per_head,
+         current_stream())
+
+
+def gemm_f16_nt(a, w, c, m, n, k):
+    """c[m,n] (fp16) = a[m,k] @ w[n,k]^T with fp32 accumulation."""
+    _dev(a, w, c)
+    call("lsh_gemm_f16_nt", ptr(a), ptr(w), ptr(c), m, n, k, current_stream())
+
+
+# --------------------------------------------------------------------------- #
+# beam search
+# --------------------------------------------------------------------------- #
+def length_norm(length, alpha):
+    return lib.load().lsh_length_norm(int(length), float(alpha))
+
+
+def select_beam_rough_topk_i8I_launcher(logits, logit_bias, seq_probs, seq_score, alive_seq,
+                                        dequant_scale, can_idx, can_score, num_beam_can,
+                                        vocab_size, max_step, length_norm_value, cur_step,
+                                        step_token_num, max_thread_per_block, beam_size,
+                                        diverse_lambda, end_id, in_col32=False):
+    _dev(logits, logit_bias, seq_probs, seq_score, alive_seq, can_idx, can_score, num_beam_can)
+    call("lsh_select_beam_rough_topk_i8I" + _suffix(logit_bias), ptr(logits), ptr(logit_bias),
+         ptr(seq_probs), ptr(seq_score), ptr(alive_seq), dequant_scale, ptr(can_idx),
+         ptr(can_score), ptr(num_beam_can), vocab_size, max_step, length_norm_value, cur_step,
+         step_token_num, max_thread_per_block, current_stream(), beam_size, diverse_lambda, end_id,
+         int(in_col32))
+
+
+def ker_refresh_result(can_idx, can_score, num_can_per_beam, old_alive_seq, new_alive_seq,
+                       seq_probs, seq_score, num_finish_beam, vocab_size, cur_step,
+                       length_norm_value, diverse_lambda, end_id, batch_size, beam_size, max_step):
+    """``num_can_per_beam`` may be an int (device address) to pass ``can_num + 1``."""
+    _dev(can_idx, can_score, old_alive_seq, new_alive_seq, seq_probs, seq_score, num_finish_beam)
+    ncp = num_can_per_beam if isinstance(num_can_per_beam, int) else ptr(num_can_per_beam)
+    call("lsh_ker_refresh_result", ptr(can_idx), ptr(can_score), ncp, ptr(old_alive_seq),
+         ptr(new_alive_seq), ptr(seq_probs), ptr(seq_score), ptr(num_finish_beam), vocab_size,
+         cur_step, length_norm_value, diverse_lambda, end_id, batch_size, beam_size, max_step,
+         current_stream())
+
+
+def ker_refresh_cache_launcher_i8(grid_dim_x, grid_dim_y, block_dim, num_can_per_beam, can_idx,
+                                  self_k_bgeem, self_v_bgeem, new_self_k_bgeem, new_self_v_bgeem,
+                                  self_k_bgeem_offset, beam_size, dim_per_head, head_num,
+                                  vocab_size, cur_step, max_step, diverse, end_id):
+    _dev(can_idx, self_k_bgeem, self_v_bgeem, new_self_k_bgeem, new_self_v_bgeem)
+    ncp = num_can_per_beam if isinstance(num_can_per_beam, int) else ptr(num_can_per_beam)
+    call("lsh_ker_refresh_cache_i8", grid_dim_x, grid_dim_y, block_dim, current_stream(), ncp,
+         ptr(can_idx), ptr(self_k_bgeem), ptr(self_v_bgeem), ptr(new_self_k_bgeem),
+         ptr(new_self_v_bgeem), self_k_bgeem_offset, beam_size, dim_per_head, head_num, vocab_size,
+         cur_step, max_step, int(diverse), end_id)
+
+
+def ker_write_trg_tokenid_pos_penalty(alive_seq, seq_score, output, max_step, beam_size,
+                                      batch_size, out_len):
+    _dev(alive_seq, seq_score, output)
+    call("lsh_ker_write_trg_tokenid_pos_penalty", ptr(alive_seq), ptr(seq_score), ptr(output),
+         max_step, beam_size, batch_size, out_len, current_stream())
+
+
+def ker_write_trg_tokenid_neg_penalty(alive_seq, seq_score, output, max_step, beam_size,
+                                      vocab_size, end_id, batch_size, out_len):
+    _dev(alive_seq, seq_score, output)
+    call("lsh_ker_write_trg_tokenid_neg_penalty", ptr(alive_seq), ptr(seq_score), ptr(output),
+         max_step, beam_size, vocab_size, end_id, batch_size, out_len, current_stream())
+
+
+def ker_write_topk_result(alive_seq, seq_score, res_seq, vocab_size, max_step, beam_size, end_id,
+                          batch_beam_num, out_len):
+    _dev(alive_seq, seq_score, res_seq)
+    call("lsh_ker_write_topk_result", ptr(alive_seq), ptr(seq_score), ptr(res_seq), vocab_size,
+         max_step, beam_size, end_id, batch_beam_num, out_len, current_stream())
+
+
+def beam_search_step_i8I(logits, logit_bias, seq_probs, seq_score, old_alive_seq, new_alive_seq,
+                         top_score, top_idx, parent, num_finished, dequant_scale, vocab_size,
+                         max_step, length_norm_value, cur_step, batch_size, beam_size, end_id):
+    """Exact top-k per row + per-sentence merge + result refresh, all on the device."""
+    _dev(logits, logit_bias, seq_probs, seq_score, old_alive_seq, new_alive_seq, top_score,
+         top_idx, parent, num_finished)
+    call("lsh_beam_search_step_i8I" + _suffix(logit_bias), ptr(logits), ptr(logit_bias),
+         ptr(seq_probs), ptr(seq_score), ptr(old_alive_seq), ptr(new_alive_seq), ptr(top_score),
+         ptr(top_idx), ptr(parent), ptr(num_finished), dequant_scale, vocab_size, max_step,
+         length_norm_value, cur_step, batch_size, beam_size, end_id, current_stream())
+
+
+def refresh_cache_by_parent_i8(n_layer, rows, parent, k_old, v_old, k_new, v_new, layer_offset,
+                               beam_size, dim_per_head, head_num, cur_step, max_step):
+    _dev(parent, k_old, v_old, k_new, v_new)
+    call("lsh_refresh_cache_by_parent_i8", n_layer, rows, current_stream(), ptr(parent),
+         ptr(k_old), ptr(v_old), ptr(k_new), ptr(v_new), layer_offset, beam_size, dim_per_head,
+         head_num, cur_step, max_step)
+
+
+__all__ = [n for n in dir() if n.startswith(("launch_", "ker_", "gemm_", "encself_", "quantize_",
+                                             "decself_", "encdec_", "select_beam_", "beam_",
+                                             "refresh_", "length_norm"))]
 _ = lib  # re-exported for callers that want lib.LSHError

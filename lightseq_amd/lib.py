@@ -50,6 +50,28 @@ _SIGNATURES = {
     "lsh_gemm_i8_bias_relu_i8o_f16": (False, "pppp" + "iiiffffis"),
     "lsh_gemm_i8_qkv_arrange_f16": (False, "pppp" + "iiiiiiffs"),
     "lsh_quantize_weight": (True, "ppiifsi"),
+    # decoder step
+    "lsh_launch_dec_emb_i8I": (True, "pppppp" + "iiiiiii" + "sfi"),
+    "lsh_launch_dec_emb_i8I_vocab_major": (True, "pppppp" + "iiiiiii" + "sfi"),
+    "lsh_ker_arrange_decself_qkv_i8I_i8O": (True, "iisppppp" + "iiiii" + "ffi"),
+    "lsh_decself_scores_i8_i32o": (False, "ppp" + "iiii" + "s"),
+    "lsh_ker_fuse_softmax_new_value_i32I_i8O": (False, "ppp" + "iiiii" + "fff" + "is"),
+    "lsh_decself_attention_i8": (False, "pppp" + "iiiii" + "fff" + "s"),
+    "lsh_ker_arrange_encdec_q_i8I": (True, "iisppp" + "iiii" + "fi"),
+    "lsh_ker_arrange_encdec_kv": (True, "iiispppp" + "l" + "iiii"),
+    "lsh_ker_correlation_softmax_encdec": (True, "iiispp"),
+    "lsh_encdec_attention_f16": (False, "pppppp" + "f" + "iiiii" + "s"),
+    "lsh_gemm_f16_nt": (False, "ppp" + "iii" + "s"),
+    # beam search
+    "lsh_select_beam_rough_topk_i8I": (True, "ppppp" + "f" + "ppp" + "ii" + "f" + "iii" + "s" +
+                                       "i" + "f" + "ii"),
+    "lsh_ker_refresh_result": (False, "pppppppp" + "ii" + "ff" + "iiii" + "s"),
+    "lsh_ker_refresh_cache_i8": (False, "iiis" + "pppppp" + "l" + "iiiiiiii"),
+    "lsh_ker_write_trg_tokenid_pos_penalty": (False, "ppp" + "iiii" + "s"),
+    "lsh_ker_write_trg_tokenid_neg_penalty": (False, "ppp" + "iiiiii" + "s"),
+    "lsh_ker_write_topk_result": (False, "ppp" + "iiiiii" + "s"),
+    "lsh_beam_search_step_i8I": (True, "pppppppppp" + "f" + "ii" + "f" + "iiii" + "s"),
+    "lsh_refresh_cache_by_parent_i8": (False, "iis" + "ppppp" + "l" + "iiiii"),
 }
 
 _lib = None
@@ -69,6 +91,8 @@ def load():
     lib.lsh_last_error.argtypes = []
     lib.lsh_version.restype = ctypes.c_char_p
     lib.lsh_version.argtypes = []
+    lib.lsh_length_norm.restype = ctypes.c_float
+    lib.lsh_length_norm.argtypes = [_I, _F]
     for name, (typed, codes) in _SIGNATURES.items():
         for suffix in (("_f16", "_f32") if typed else ("",)):
             fn = getattr(lib, name + suffix)

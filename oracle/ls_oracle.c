@@ -484,6 +484,7 @@ int lso_quant_bert_encoder(const lso_bert_weights* w, const int* token_ids,
   const long M = (long)batch * seq_len;
   const size_t tsz = f16 ? 2 : 4;
   const float Q = 127.f;
+  const int cs = w->clip_stride > 0 ? w->clip_stride : 11;
   long wide = I > 3 * H ? I : 3 * H;
 
   int8_t* i8_in = (int8_t*)malloc((size_t)(M * wide));
@@ -496,10 +497,10 @@ int lso_quant_bert_encoder(const lso_bert_weights* w, const int* token_ids,
 
   /* model/quant_bert_encoder.cc.cu:233-237 */
   lso_enc_emb_i8I(w->tok_emb_q, w->pos_emb, token_ids, output, pad_mask,
-                  w->padding_id, batch, seq_len, H, w->emb_clip_max / Q, 0, f16);
+                  w->padding_id, batch, seq_len, H, w->emb_clip_max / Q, w->emb_scaled, f16);
 
   for (int l = 0; l < w->n_layer; ++l) {
-    const float* c = w->clip_max + (long)l * 11;
+    const float* c = w->clip_max + (long)l * cs;
     const int tap = taps && taps->tap_layer == l;
     /* ---- self attention (:271-399) ---- */
     if (l == 0) {
@@ -544,7 +545,7 @@ int lso_quant_bert_encoder(const lso_bert_weights* w, const int* token_ids,
       lso_residual_bias_ln_i32I(i32_out, w->final_ln_scale, w->final_ln_bias, output,
                                 output, (int)M, H, dq, colsum, f16);
     } else {
-      const float* cn = w->clip_max + (long)(l + 1) * 11;
+      const float* cn = w->clip_max + (long)(l + 1) * cs;
       lso_residual_bias_ln_i8O(i32_out, 1, w->ln1_scale[l + 1], w->ln1_bias[l + 1],
                                w->b_out[l + 1], i8_in, output, (int)M, H, dq,
                                Q / cn[4], w->is_post_ln, colsum, f16);

@@ -150,7 +150,11 @@ typedef struct {
   const int8_t* const* w_ffn2; /* [H, I] */
   const void* const* b_ffn2;
   const void* const* ffn2_colsum; /* [H] or NULL entries (GELU) */
-  const float* clip_max;          /* [n_layer * 11], proto/quant_bert_weight.cc:194-205 */
+  const float* clip_max;          /* [n_layer * clip_stride], proto/quant_bert_weight.cc:194-205 */
+  /* 11 / 0 for QuantBert; 12 / 1 for the encoder of QuantTransformer
+   * (model/quant_encoder.cc.cu:140, :242; proto/quant_transformer_weight.cc:316-328) */
+  int clip_stride;
+  int emb_scaled;
 } lso_bert_weights;
 
 /* Optional taps: when non-NULL, receive a copy of the named intermediate of
@@ -172,6 +176,187 @@ typedef struct {
 int lso_quant_bert_encoder(const lso_bert_weights* w, const int* token_ids,
                            int batch, int seq_len, void* output /*[M,H] T*/,
                            int* pad_mask /*[M]*/, const lso_bert_taps* taps);
+
+/* ========================================================================= */
+/* decoder half                                                                */
+/* ========================================================================= */
+
+/* kernels/embKernels_int8.cc.cu:158-200.  tokens [rows, max_step]; token_emb is
+ * [hidden, vocab] as the reference stores it (vocab_major = 0) or [vocab, hidden]
+ * (vocab_major = 1, the table of the logits GEMM); output [rows, hidden] T. */
+void lso_dec_emb_i8I(const int8_t* token_emb, const void* pos_emb,
+                     const int* tokens, void* output, int rows, int hidden,
+                     int vocab, int step, int max_step, float dequant_scale,
+                     int scaled, int vocab_major, int f16);
+
+/* kernels/transformerKernels_int8.cc.cu:1395-1499.  ori_qkv [rows, 3H] int8;
+ * new_q [rows, H]; caches [rows, head_num, max_step, dim_per_head] int8. */
+void lso_arrange_decself_qkv_i8I_i8O(const int8_t* ori_qkv, const void* qkv_bias,
+                                     int8_t* new_q, int8_t* k_cache,
+                                     int8_t* v_cache, int rows, int head_num,
+                                     int dim_per_head, int max_step, int step_id,
+                                     float dequant_scale, float quant_scale,
+                                     int f16);
+
+/* model/quant_decoder.cc.cu:676-683 (strided-batched int8 GEMM):
+ * scores[r*head_num+h, j] = sum_d q[r,h,d] * k_cache[r,h,j,d], j < step_num;
+ * row stride of scores is max_step. */
+void lso_decself_scores(const int8_t* q, const int8_t* k_cache, int32_t* scores,
+                        int rows, int head_num, int dim_per_head, int max_step,
+                        int step_num);
+
+/* kernels/transformerKernels_int8.cc.cu:1515-1594 */
+void lso_fuse_softmax_new_value_i32I_i8O(const int32_t* logits, const int8_t* v,
+                                         int8_t* new_v, int batch_head_num,
+                                         int step_num, int max_step, int head_num,
+                                         int dim_per_head, float attn_scale,
+                                         float dequant_scale, float quant_scale);
+
+/* kernels/transformerKernels_int8.cc.cu:1596-1688.  new_q [batch, head_num,
+ * beam_size, dim_per_head] T. */
+void lso_arrange_encdec_q_i8I(const int8_t* ori_q, const void* q_bias, void* new_q,
+                              int rows, int beam_size, int dim_per_head,
+                              int head_num, float dequant_scale, int f16);
+
+/* kernels/transformerKernels.cc.cu:903-1020.  ori_kv [tokens, n_layer, 2, H] T;
+ * new_k / new_v: layer l at element offset l*offset_per_layer, laid out
+ * [batch, head_num, seq_len, dim_per_head]. */
+void lso_arrange_encdec_kv(const void* ori_kv, const void* kv_bias, void* new_k,
+                           void* new_v, long offset_per_layer, int batch,
+                           int seq_len, int n_layer, int dim_per_head,
+                           int head_num, int f16);
+
+/* kernels/transformerKernels.cc.cu:1226-1284.  correlation [batch,
+ * head_num*beam_size, seq_len] T, in place. */
+void lso_correlation_softmax_encdec(void* correlation, const int* pad_mask,
+                                    int batch, int heads_x_beams, int seq_len,
+                                    int f16);
+
+/* model/quant_decoder.cc.cu:767-790: rectangular versions of the two attention
+ * GEMMs (n_q queries against n_k keys per batch-head). */
+void lso_attn_scores_rect(const void* q, const void* k, void* scores,
+                          int batch_heads, int n_q, int n_k, int dim_per_head,
+                          float alpha, int f16);
+void lso_attn_context_rect(const void* probs, const void* v, void* ctx,
+                           int batch_heads, int n_q, int n_k, int dim_per_head,
+                           int f16);
+
+/* model/quant_decoder.cc.cu:497-501: C[M,N] = T(A[M,K] @ B[K,N]), T operands. */
+void lso_gemm_T(const void* A, const void* B, void* C, int M, int N, int K, int f16);
+
+/* kernels/transformerKernels.h:137-140 */
+float lso_length_norm(int length, float alpha);
+
+/* kernels/transformerKernels_int8.cc.cu:1690-1890 with diverse_lambda == 0.
+ * Candidates are emitted row by row in ascending vocabulary order (the reference
+ * emits the same set in an order decided by atomics).  num_beam_can[0] = total,
+ * num_beam_can[1 + row] = candidates of that row.  Returns the total. */
+int lso_select_beam_rough_topk_i8I(const int8_t* logits, const void* logit_bias,
+                                   const float* seq_probs, const float* seq_score,
+                                   const int* alive_seq, float dequant_scale,
+                                   int* can_idx, float* can_score,
+                                   int* num_beam_can, int vocab_size, int max_step,
+                                   float length_norm, int cur_step,
+                                   int step_token_num, int max_thread_per_block,
+                                   int beam_size, int end_id, int f16);
+
+/* thrust::exclusive_scan + thrust::sort_by_key(greater) of
+ * model/quant_decoder.cc.cu:1002-1003 and :1095-1096; ties keep emission order
+ * (thrust leaves them unspecified). */
+void lso_scan_sort_candidates(int* can_idx, float* can_score, int* num_beam_can,
+                              int step_token_num);
+
+/* kernels/transformerKernels.cc.cu:1398-1463 with diverse_lambda == 0.
+ * num_can_per_beam is the scanned array (num_beam_can + 1). */
+void lso_refresh_result(const int* can_idx, const float* can_score,
+                        const int* num_can_per_beam, const int* old_alive_seq,
+                        int* new_alive_seq, float* seq_probs, float* seq_score,
+                        int* num_finish_beam, int vocab_size, int cur_step,
+                        float length_norm, int end_id, int batch, int beam_size,
+                        int max_step);
+
+/* kernels/transformerKernels.cc.cu:1579-1627 (int8 cache).  Caches hold n_layer
+ * blocks of cache_offset bytes, each [rows, head_num, max_step, dim_per_head]. */
+void lso_refresh_cache_i8(const int* num_can_per_beam, const int* can_idx,
+                          const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
+                          int8_t* v_new, long cache_offset, int n_layer, int batch,
+                          int beam_size, int dim_per_head, int head_num,
+                          int vocab_size, int cur_step, int max_step, int end_id);
+
+/* kernels/transformerKernels.cc.cu:1707-1815.  out_len = cur_step + 1. */
+void lso_write_trg_tokenid_pos_penalty(const int* alive_seq, float* seq_score,
+                                       int* output, int max_step, int beam_size,
+                                       int batch, int out_len);
+void lso_write_trg_tokenid_neg_penalty(const int* alive_seq, const float* seq_score,
+                                       int* output, int max_step, int beam_size,
+                                       int end_id, int batch, int out_len);
+void lso_write_topk_result(const int* alive_seq, float* seq_score, int* res_seq,
+                           int max_step, int beam_size, int end_id, int rows,
+                           int out_len);
+
+/* ---- whole decoder: model/quant_decoder.cc.cu:413-1075 -------------------- */
+typedef struct {
+  int n_layer, hidden, inner, head_num, max_step, vocab;
+  int beam_size, extra_decode_length, start_id, end_id;
+  int is_post_ln, use_gelu, f16;
+  float length_penalty;
+  const int8_t* tok_emb_q;      /* [vocab, hidden] int8 codes */
+  const void* pos_emb;          /* [max_step, hidden] */
+  const void* out_ln_scale;     /* trg_embedding.norm_scale */
+  const void* out_ln_bias;
+  const void* encdec_kv_kernel; /* [hidden, n_layer*2*hidden] T (dequantised) */
+  const void* encdec_kv_bias;   /* [n_layer, 2, hidden] */
+  const void* logit_bias;       /* [vocab] */
+  float emb_clip_max, output_ln_clip_max, logits_clip_max;
+  /* per layer (arrays of n_layer pointers); int8 kernels are [N, K] codes */
+  const void* const* self_ln_scale;
+  const void* const* self_ln_bias;
+  const int8_t* const* w_self_qkv;
+  const void* const* b_self_qkv;
+  const int8_t* const* w_self_out;
+  const void* const* b_self_out;
+  const void* const* encdec_ln_scale;
+  const void* const* encdec_ln_bias;
+  const int8_t* const* w_encdec_q;
+  const void* const* b_encdec_q;
+  const int8_t* const* w_encdec_out;
+  const void* const* b_encdec_out;
+  const void* const* ffn_ln_scale;
+  const void* const* ffn_ln_bias;
+  const int8_t* const* w_ffn1;
+  const void* const* b_ffn1;
+  const int8_t* const* w_ffn2;
+  const void* const* b_ffn2;
+  const void* const* ffn2_colsum; /* NULL (GELU) or n_layer [H] arrays */
+  const float* clip_max;          /* [n_layer * 19], proto/quant_transformer_weight.cc:490-508 */
+} lso_dec_weights;
+
+typedef struct {
+  /* forced_logits: when non-NULL, step t's search consumes
+   * forced_logits[t] ([rows, vocab] int8) instead of the oracle's own logits, so
+   * the token history follows the run that produced them. */
+  const int8_t* forced_logits;
+  int forced_steps;
+  int8_t* logits_record;  /* NULL or [max_step, rows, vocab]: the oracle's own logits */
+  int* alive_seq_record;  /* NULL or [max_step, rows, max_step]: alive_seq after each step */
+  float* seq_probs_record; /* NULL or [max_step, rows] */
+  int steps_run;          /* out: number of run_step calls */
+  int early_stopped;      /* out */
+} lso_dec_trace;
+
+/* Beam search (sampling_method "beam_search", diverse_lambda 0).  enc_out
+ * [batch, seq_len, hidden] T, pad_mask [batch, seq_len].
+ * output_topk = 0: result [batch, *out_len], scores [batch] (first `batch` slots
+ * of the score array, as the reference leaves them);
+ * output_topk = 1 (what pywrapper/quant_transformer.cc:51-53 passes): result
+ * [batch*beam, *out_len], scores [batch*beam]; the score of a beam that never
+ * finished is whatever the score buffer held (0 here).
+ * `is_benchmark` reproduces benchmark_mode(true): no early stop.
+ * Returns 0 on success. */
+int lso_quant_decoder(const lso_dec_weights* w, const void* enc_out,
+                      const int* pad_mask, int batch, int seq_len, int is_benchmark,
+                      int output_topk, int* result, int* out_len, float* scores,
+                      lso_dec_trace* trace);
 
 #ifdef __cplusplus
 }

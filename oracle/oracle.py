@@ -284,7 +284,8 @@ class _BertWeights(_c.Structure):
         ("ln2_scale", _c.POINTER(_vp)), ("ln2_bias", _c.POINTER(_vp)),
         ("w_ffn1", _c.POINTER(_vp)), ("b_ffn1", _c.POINTER(_vp)),
         ("w_ffn2", _c.POINTER(_vp)), ("b_ffn2", _c.POINTER(_vp)),
-        ("ffn2_colsum", _c.POINTER(_vp)), ("clip_max", _c.POINTER(_c.c_float))]
+        ("ffn2_colsum", _c.POINTER(_vp)), ("clip_max", _c.POINTER(_c.c_float)),
+        ("clip_stride", _c.c_int), ("emb_scaled", _c.c_int)]
 
 
 class _BertTaps(_c.Structure):
@@ -339,7 +340,9 @@ def quant_bert_encoder(weights, token_ids, tap_layer=None):
     cs = weights.get("ffn2_colsum")
     w.ffn2_colsum = ptr_array(cs) if cs is not None else _c.cast(None, _c.POINTER(_vp))
     clip = np.ascontiguousarray(weights["clip_max"], np.float32)
-    assert clip.size == L * 11
+    w.clip_stride = int(weights.get("clip_stride", 11))
+    w.emb_scaled = int(weights.get("emb_scaled", 0))
+    assert clip.size == L * w.clip_stride
     w.clip_max = clip.ctypes.data_as(_c.POINTER(_c.c_float))
 
     out = np.empty((b, s, H), T)
@@ -364,3 +367,342 @@ def quant_bert_encoder(weights, token_ids, tap_layer=None):
     if rc != 0:
         raise RuntimeError("lso_quant_bert_encoder failed with code %d" % rc)
     return out, mask, taps_out
+
+
+# --------------------------------------------------------------------------- #
+# decoder half
+# --------------------------------------------------------------------------- #
+_lib.lso_length_norm.restype = _c.c_float
+_lib.lso_length_norm.argtypes = [_c.c_int, _c.c_float]
+_lib.lso_select_beam_rough_topk_i8I.restype = _c.c_int
+
+
+def _fl(x):
+    return _c.c_float(float(x))
+
+
+def length_norm(length, alpha):
+    return _lib.lso_length_norm(int(length), float(alpha))
+
+
+def dec_emb_i8I(token_emb, pos_emb, tokens, step, dequant_scale, scaled, vocab_major=False):
+    """tokens [rows, max_step] int32; token_emb [hidden, vocab] (or [vocab, hidden] when
+    ``vocab_major``) -> [rows, hidden] T."""
+    token_emb = _c_arr(token_emb, np.int8)
+    pos_emb = _c_arr(pos_emb)
+    tokens = _c_arr(tokens, np.int32)
+    rows, max_step = tokens.shape
+    vocab, hidden = token_emb.shape if vocab_major else token_emb.shape[::-1]
+    out = np.empty((rows, hidden), pos_emb.dtype)
+    _lib.lso_dec_emb_i8I(_p(token_emb), _p(pos_emb), _p(tokens), _p(out), rows, hidden, vocab,
+                         int(step), max_step, _fl(dequant_scale), int(scaled), int(vocab_major),
+                         _f16(pos_emb))
+    return out
+
+
+def arrange_decself_qkv_i8I_i8O(ori_qkv, qkv_bias, k_cache, v_cache, step_id, dequant_scale,
+                                quant_scale):
+    """Writes step ``step_id`` of the caches [rows, head, max_step, d] in place; returns new_q."""
+    ori_qkv = _c_arr(ori_qkv, np.int8)
+    qkv_bias = _c_arr(qkv_bias)
+    assert k_cache.flags.c_contiguous and v_cache.flags.c_contiguous
+    rows, head_num, max_step, d = k_cache.shape
+    new_q = np.empty((rows, head_num * d), np.int8)
+    _lib.lso_arrange_decself_qkv_i8I_i8O(_p(ori_qkv), _p(qkv_bias), _p(new_q), _p(k_cache),
+                                         _p(v_cache), rows, head_num, d, max_step, int(step_id),
+                                         _fl(dequant_scale), _fl(quant_scale), _f16(qkv_bias))
+    return new_q
+
+
+def decself_scores(q, k_cache, step_num):
+    q = _c_arr(q, np.int8)
+    k_cache = _c_arr(k_cache, np.int8)
+    rows, head_num, max_step, d = k_cache.shape
+    out = np.zeros((rows * head_num, max_step), np.int32)
+    _lib.lso_decself_scores(_p(q), _p(k_cache), _p(out), rows, head_num, d, max_step,
+                            int(step_num))
+    return out
+
+
+def fuse_softmax_new_value_i32I_i8O(logits, v_cache, step_num, attn_scale, dequant_scale,
+                                    quant_scale):
+    logits = _c_arr(logits, np.int32)
+    v_cache = _c_arr(v_cache, np.int8)
+    rows, head_num, max_step, d = v_cache.shape
+    out = np.empty((rows, head_num * d), np.int8)
+    _lib.lso_fuse_softmax_new_value_i32I_i8O(_p(logits), _p(v_cache), _p(out), rows * head_num,
+                                             int(step_num), max_step, head_num, d,
+                                             _fl(attn_scale), _fl(dequant_scale),
+                                             _fl(quant_scale))
+    return out
+
+
+def arrange_encdec_q_i8I(ori_q, q_bias, beam_size, head_num, dequant_scale):
+    ori_q = _c_arr(ori_q, np.int8)
+    q_bias = _c_arr(q_bias)
+    rows, hidden = ori_q.shape
+    d = hidden // head_num
+    out = np.empty((rows // beam_size, head_num, beam_size, d), q_bias.dtype)
+    _lib.lso_arrange_encdec_q_i8I(_p(ori_q), _p(q_bias), _p(out), rows, beam_size, d, head_num,
+                                  _fl(dequant_scale), _f16(q_bias))
+    return out
+
+
+def arrange_encdec_kv(ori_kv, kv_bias, batch, seq_len, n_layer, head_num):
+    """ori_kv [batch*seq_len, n_layer, 2, H] -> (k, v) each [n_layer, batch, head, seq_len, d]."""
+    ori_kv = _c_arr(ori_kv)
+    kv_bias = _c_arr(kv_bias)
+    hidden = ori_kv.shape[-1]
+    d = hidden // head_num
+    k = np.empty((n_layer, batch, head_num, seq_len, d), ori_kv.dtype)
+    v = np.empty_like(k)
+    _lib.lso_arrange_encdec_kv(_p(ori_kv), _p(kv_bias), _p(k), _p(v),
+                               _c.c_long(batch * seq_len * hidden), batch, seq_len, n_layer, d,
+                               head_num, _f16(ori_kv))
+    return k, v
+
+
+def correlation_softmax_encdec(correlation, pad_mask):
+    """correlation [batch, head*beam, seq_len] T -> probabilities (copy)."""
+    out = np.array(correlation, copy=True, order="C")
+    pad_mask = _c_arr(pad_mask, np.int32)
+    batch, hb, seq_len = out.shape
+    _lib.lso_correlation_softmax_encdec(_p(out), _p(pad_mask), batch, hb, seq_len, _f16(out))
+    return out
+
+
+def attn_scores_rect(q, k, alpha):
+    """q [BH, n_q, d], k [BH, n_k, d] -> [BH, n_q, n_k]."""
+    q = _c_arr(q)
+    k = _c_arr(k)
+    bh, n_q, d = q.shape
+    n_k = k.shape[1]
+    out = np.empty((bh, n_q, n_k), q.dtype)
+    _lib.lso_attn_scores_rect(_p(q), _p(k), _p(out), bh, n_q, n_k, d, _fl(alpha), _f16(q))
+    return out
+
+
+def attn_context_rect(probs, v):
+    probs = _c_arr(probs)
+    v = _c_arr(v)
+    bh, n_q, n_k = probs.shape
+    d = v.shape[2]
+    out = np.empty((bh, n_q, d), probs.dtype)
+    _lib.lso_attn_context_rect(_p(probs), _p(v), _p(out), bh, n_q, n_k, d, _f16(probs))
+    return out
+
+
+def gemm_T(a, b):
+    """[M,K] @ [K,N] in T with wide accumulation."""
+    a = _c_arr(a)
+    b = _c_arr(b)
+    m, k = a.shape
+    n = b.shape[1]
+    out = np.empty((m, n), a.dtype)
+    _lib.lso_gemm_T(_p(a), _p(b), _p(out), m, n, k, _f16(a))
+    return out
+
+
+def select_beam_rough_topk_i8I(logits, logit_bias, seq_probs, seq_score, alive_seq, dequant_scale,
+                               length_norm_value, cur_step, max_thread_per_block, beam_size,
+                               end_id):
+    """Returns (can_idx[:total], can_score[:total], num_beam_can [rows+1])."""
+    logits = _c_arr(logits, np.int8)
+    logit_bias = _c_arr(logit_bias)
+    seq_probs = _c_arr(seq_probs, np.float32)
+    seq_score = _c_arr(seq_score, np.float32)
+    alive_seq = _c_arr(alive_seq, np.int32)
+    rows, vocab = logits.shape
+    max_step = alive_seq.shape[1]
+    can_idx = np.empty(rows * vocab, np.int32)
+    can_score = np.empty(rows * vocab, np.float32)
+    num = np.zeros(rows + 1, np.int32)
+    total = _lib.lso_select_beam_rough_topk_i8I(
+        _p(logits), _p(logit_bias), _p(seq_probs), _p(seq_score), _p(alive_seq),
+        _fl(dequant_scale), _p(can_idx), _p(can_score), _p(num), vocab, max_step,
+        _fl(length_norm_value), int(cur_step), rows, int(max_thread_per_block), int(beam_size),
+        int(end_id), _f16(logit_bias))
+    return can_idx[:total].copy(), can_score[:total].copy(), num
+
+
+def scan_sort_candidates(can_idx, can_score, num_beam_can):
+    """Returns sorted copies and the scanned count array."""
+    can_idx = np.array(can_idx, np.int32, copy=True)
+    can_score = np.array(can_score, np.float32, copy=True)
+    num = np.array(num_beam_can, np.int32, copy=True)
+    _lib.lso_scan_sort_candidates(_p(can_idx), _p(can_score), _p(num), num.size - 1)
+    return can_idx, can_score, num
+
+
+def refresh_result(can_idx, can_score, num_scanned, alive_seq, seq_probs, seq_score, vocab_size,
+                   cur_step, length_norm_value, end_id, beam_size):
+    """``num_scanned``: the scanned array including slot 0.  Returns (new_alive_seq,
+    seq_probs, seq_score, num_finished) -- copies."""
+    can_idx = _c_arr(can_idx, np.int32)
+    can_score = _c_arr(can_score, np.float32)
+    num = _c_arr(num_scanned, np.int32)
+    alive_seq = _c_arr(alive_seq, np.int32)
+    rows, max_step = alive_seq.shape
+    new_alive = np.array(alive_seq, copy=True)
+    probs = np.array(seq_probs, np.float32, copy=True)
+    score = np.array(seq_score, np.float32, copy=True)
+    fin = _c.c_int(0)
+    _lib.lso_refresh_result(_p(can_idx), _p(can_score), _c.c_void_p(num.ctypes.data + 4),
+                            _p(alive_seq), _p(new_alive), _p(probs), _p(score), _c.byref(fin),
+                            int(vocab_size), int(cur_step), _fl(length_norm_value), int(end_id),
+                            rows // beam_size, int(beam_size), max_step)
+    return new_alive, probs, score, fin.value
+
+
+def refresh_cache_i8(num_scanned, can_idx, k_old, v_old, k_new, v_new, beam_size, vocab_size,
+                     cur_step, end_id):
+    """Caches [n_layer, rows, head, max_step, d]; k_new / v_new updated in place."""
+    num = _c_arr(num_scanned, np.int32)
+    can_idx = _c_arr(can_idx, np.int32)
+    n_layer, rows, head_num, max_step, d = k_old.shape
+    for a in (k_old, v_old, k_new, v_new):
+        assert a.flags.c_contiguous and a.dtype == np.int8
+    _lib.lso_refresh_cache_i8(_c.c_void_p(num.ctypes.data + 4), _p(can_idx), _p(k_old), _p(v_old),
+                              _p(k_new), _p(v_new), _c.c_long(rows * head_num * max_step * d),
+                              n_layer, rows // beam_size, int(beam_size), d, head_num,
+                              int(vocab_size), int(cur_step), max_step, int(end_id))
+
+
+def write_trg_tokenid_pos_penalty(alive_seq, seq_score, beam_size, out_len):
+    alive_seq = _c_arr(alive_seq, np.int32)
+    rows, max_step = alive_seq.shape
+    score = np.array(seq_score, np.float32, copy=True)
+    out = np.empty((rows // beam_size, out_len), np.int32)
+    _lib.lso_write_trg_tokenid_pos_penalty(_p(alive_seq), _p(score), _p(out), max_step,
+                                           int(beam_size), rows // beam_size, int(out_len))
+    return out, score
+
+
+def write_trg_tokenid_neg_penalty(alive_seq, seq_score, beam_size, end_id, out_len):
+    alive_seq = _c_arr(alive_seq, np.int32)
+    seq_score = _c_arr(seq_score, np.float32)
+    rows, max_step = alive_seq.shape
+    out = np.empty((rows // beam_size, out_len), np.int32)
+    _lib.lso_write_trg_tokenid_neg_penalty(_p(alive_seq), _p(seq_score), _p(out), max_step,
+                                           int(beam_size), int(end_id), rows // beam_size,
+                                           int(out_len))
+    return out
+
+
+def write_topk_result(alive_seq, seq_score, beam_size, end_id, out_len):
+    alive_seq = _c_arr(alive_seq, np.int32)
+    rows, max_step = alive_seq.shape
+    score = np.array(seq_score, np.float32, copy=True)
+    out = np.empty((rows, out_len), np.int32)
+    _lib.lso_write_topk_result(_p(alive_seq), _p(score), _p(out), max_step, int(beam_size),
+                               int(end_id), rows, int(out_len))
+    return out, score
+
+
+_DEC_INTS = ("n_layer", "hidden", "inner", "head_num", "max_step", "vocab", "beam_size",
+             "extra_decode_length", "start_id", "end_id", "is_post_ln", "use_gelu", "f16")
+_DEC_GLOBAL = ("tok_emb_q", "pos_emb", "out_ln_scale", "out_ln_bias", "encdec_kv_kernel",
+               "encdec_kv_bias", "logit_bias")
+_DEC_PER_LAYER = ("self_ln_scale", "self_ln_bias", "w_self_qkv", "b_self_qkv", "w_self_out",
+                  "b_self_out", "encdec_ln_scale", "encdec_ln_bias", "w_encdec_q", "b_encdec_q",
+                  "w_encdec_out", "b_encdec_out", "ffn_ln_scale", "ffn_ln_bias", "w_ffn1",
+                  "b_ffn1", "w_ffn2", "b_ffn2", "ffn2_colsum")
+
+
+class _DecWeights(_c.Structure):
+    _fields_ = ([(n, _c.c_int) for n in _DEC_INTS] + [("length_penalty", _c.c_float)] +
+                [(n, _vp) for n in _DEC_GLOBAL] +
+                [(n, _c.c_float) for n in ("emb_clip_max", "output_ln_clip_max",
+                                           "logits_clip_max")] +
+                [(n, _c.POINTER(_vp)) for n in _DEC_PER_LAYER] +
+                [("clip_max", _c.POINTER(_c.c_float))])
+
+
+class _DecTrace(_c.Structure):
+    _fields_ = [("forced_logits", _vp), ("forced_steps", _c.c_int), ("logits_record", _vp),
+                ("alive_seq_record", _vp), ("seq_probs_record", _vp), ("steps_run", _c.c_int),
+                ("early_stopped", _c.c_int)]
+
+
+def quant_decoder(weights, enc_out, pad_mask, is_benchmark=False, output_topk=True,
+                  forced_logits=None, record=False):
+    """Beam-search decode.  ``weights``: dict with the ints of ``_DEC_INTS`` (f16 is
+    derived), ``length_penalty``, the arrays of ``_DEC_GLOBAL``, the three clip floats,
+    per-layer lists named in ``_DEC_PER_LAYER`` (``ffn2_colsum`` None for GELU) and
+    ``clip_max`` float32 [n_layer*19].
+
+    Returns a dict: ``ids`` [batch, k, out_len] (k = beam_size when ``output_topk`` else 1),
+    ``scores`` [batch, k], ``steps_run``, ``early_stopped`` and, with ``record``, the
+    per-step ``logits`` [steps, rows, vocab], ``alive_seq`` [steps, rows, max_step] and
+    ``seq_probs`` [steps, rows].
+    """
+    enc_out = _c_arr(enc_out)
+    pad_mask = _c_arr(pad_mask, np.int32)
+    batch, seq_len, H = enc_out.shape
+    L, beam, V, max_step = (weights["n_layer"], weights["beam_size"], weights["vocab"],
+                            weights["max_step"])
+    rows = batch * beam
+    T = enc_out.dtype
+    keep = []
+
+    def ptr_array(arrs):
+        arr = (_vp * L)()
+        for i, a in enumerate(arrs):
+            if a is not None:
+                a = np.ascontiguousarray(a)
+                keep.append(a)
+                arr[i] = a.ctypes.data
+        keep.append(arr)
+        return _c.cast(arr, _c.POINTER(_vp))
+
+    w = _DecWeights()
+    for n in _DEC_INTS:
+        if n != "f16":
+            setattr(w, n, int(weights[n]))
+    w.f16 = 1 if T == np.float16 else 0
+    w.length_penalty = float(weights["length_penalty"])
+    for n in _DEC_GLOBAL:
+        a = np.ascontiguousarray(weights[n])
+        if n != "tok_emb_q" and a.dtype != T:
+            raise TypeError("%s must be %s" % (n, T))
+        keep.append(a)
+        setattr(w, n, a.ctypes.data)
+    for n in ("emb_clip_max", "output_ln_clip_max", "logits_clip_max"):
+        setattr(w, n, float(weights[n]))
+    for n in _DEC_PER_LAYER:
+        v = weights.get(n)
+        setattr(w, n, ptr_array(v) if v is not None else _c.cast(None, _c.POINTER(_vp)))
+    clip = np.ascontiguousarray(weights["clip_max"], np.float32)
+    assert clip.size == L * 19
+    w.clip_max = clip.ctypes.data_as(_c.POINTER(_c.c_float))
+
+    tr = _DecTrace()
+    rec = {}
+    if forced_logits is not None:
+        forced_logits = _c_arr(forced_logits, np.int8)
+        assert forced_logits.shape[1:] == (rows, V)
+        tr.forced_logits = forced_logits.ctypes.data
+        tr.forced_steps = forced_logits.shape[0]
+    if record:
+        rec["logits"] = np.zeros((max_step, rows, V), np.int8)
+        rec["alive_seq"] = np.zeros((max_step, rows, max_step), np.int32)
+        rec["seq_probs"] = np.zeros((max_step, rows), np.float32)
+        tr.logits_record = rec["logits"].ctypes.data
+        tr.alive_seq_record = rec["alive_seq"].ctypes.data
+        tr.seq_probs_record = rec["seq_probs"].ctypes.data
+    k = beam if output_topk else 1
+    result = np.zeros((batch * k * max_step,), np.int32)
+    scores = np.zeros((rows,), np.float32)
+    out_len = _c.c_int(0)
+    rc = _lib.lso_quant_decoder(_c.byref(w), _p(enc_out), _p(pad_mask), batch, seq_len,
+                                int(is_benchmark), int(output_topk), _p(result),
+                                _c.byref(out_len), _p(scores), _c.byref(tr))
+    if rc != 0:
+        raise RuntimeError("lso_quant_decoder failed with code %d" % rc)
+    n = out_len.value
+    out = {"ids": result[:batch * k * n].reshape(batch, k, n).copy(),
+           "scores": scores[:batch * k].reshape(batch, k).copy(),
+           "steps_run": tr.steps_run, "early_stopped": bool(tr.early_stopped)}
+    for name, a in rec.items():
+        out[name] = a[:tr.steps_run]
+    return out
