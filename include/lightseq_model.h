@@ -76,6 +76,15 @@ int ls_model_get_profile(ls_model* model, char* buf, int capacity);
  * res_attn res_ffn (fp16 [tokens, hidden]: the residual stream as the LayerNorm kernel
  * after the attention out-projection / after FFN2 reads it).  dst NULL clears. */
 int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst);
+/* QuantTransformer only: the tap "enc_out" (layer ignored) receives the encoder output
+ * [batch, seq_len, hidden] fp16 of every Infer().
+ *
+ * Debug aid without counterpart in the reference, QuantTransformer only: record, for the
+ * first max_steps decoding steps of every Infer(), the int8 logits [step, batch*beam,
+ * vocab] and the sequences after the step [step, batch*beam, max_step] (either may be
+ * NULL).  ls_model_get_steps_run gives the number of steps the last Infer() ran. */
+int ls_model_set_step_record(ls_model* model, int8_t* logits, int* alive_seq, int max_steps);
+int ls_model_get_steps_run(ls_model* model, int* steps);
 
 #ifdef __cplusplus
 }

@@ -7,10 +7,13 @@
 #include "../ls_launch.h"
 #include "ls_model.h"
 #include "quant_bert.h"
+#include "quant_transformer.h"
 
 using lightseq::hip::LSModel;
 using lightseq::hip::LSModelFactory;
 using lightseq::hip::QuantBert;
+using lightseq::hip::QuantBertEncoder;
+using lightseq::hip::QuantTransformer;
 
 struct ls_model {
   std::unique_ptr<LSModel> impl;
@@ -167,24 +170,32 @@ int ls_model_get_stream(ls_model* model, lsh_stream_t* stream) {
   return LSH_OK;
 }
 
+// the encoder stack of either model class, or nullptr
+static QuantBertEncoder* encoder_of(ls_model* model) {
+  if (QuantBert* qb = dynamic_cast<QuantBert*>(model->impl.get())) return qb->encoder();
+  if (QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get()))
+    return qt->encoder();
+  return nullptr;
+}
+
 int ls_model_set_profiling(ls_model* model, int on) {
   NEED_MODEL(model);
-  QuantBert* qb = dynamic_cast<QuantBert*>(model->impl.get());
-  if (!qb) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "profiling is only provided by QuantBert");
+  QuantBertEncoder* enc = encoder_of(model);
+  if (!enc) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "this model has no profiled encoder stack");
   return guarded([&] {
-    qb->encoder()->set_profiling(on != 0);
-    qb->encoder()->reset_profile();
+    enc->set_profiling(on != 0);
+    enc->reset_profile();
   });
 }
 
 int ls_model_get_profile(ls_model* model, char* buf, int capacity) {
   NEED_MODEL(model);
-  QuantBert* qb = dynamic_cast<QuantBert*>(model->impl.get());
-  if (!qb) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "profiling is only provided by QuantBert");
+  QuantBertEncoder* enc = encoder_of(model);
+  if (!enc) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "this model has no profiled encoder stack");
   if (!buf || capacity <= 0) return lsh::lsh_fail(LSH_ERR_INVALID, "null buffer");
   std::string out = "[";
   bool first = true;
-  for (const auto& p : qb->encoder()->profile()) {
+  for (const auto& p : enc->profile()) {
     if (!first) out += ",";
     first = false;
     out += "{\"site\":\"" + p.site + "\",\"kernel\":\"" + p.kernel + "\",\"m\":" +
@@ -201,9 +212,15 @@ int ls_model_get_profile(ls_model* model, char* buf, int capacity) {
 int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst) {
   NEED_MODEL(model);
   if (!name) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");
-  QuantBert* qb = dynamic_cast<QuantBert*>(model->impl.get());
-  if (!qb) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "taps are only provided by QuantBert");
-  auto& t = qb->encoder()->taps;
+  if (!strcmp(name, "enc_out")) {
+    QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get());
+    if (!qt) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "enc_out is a QuantTransformer tap");
+    qt->set_encoder_output_tap(static_cast<__half*>(dst));
+    return LSH_OK;
+  }
+  QuantBertEncoder* enc = encoder_of(model);
+  if (!enc) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "this model has no tapped encoder stack");
+  auto& t = enc->taps;
   t.tap_layer = layer;
   int8_t* p = static_cast<int8_t*>(dst);
   if (!strcmp(name, "ln1_q")) t.ln1_q = p;
@@ -217,6 +234,24 @@ int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst) {
   else if (!strcmp(name, "res_attn")) t.res_attn = static_cast<__half*>(dst);
   else if (!strcmp(name, "res_ffn")) t.res_ffn = static_cast<__half*>(dst);
   else return lsh::lsh_fail(LSH_ERR_INVALID, "unknown tap name");
+  return LSH_OK;
+}
+
+int ls_model_set_step_record(ls_model* model, int8_t* logits, int* alive_seq, int max_steps) {
+  NEED_MODEL(model);
+  QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get());
+  if (!qt) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "step records are a QuantTransformer debug aid");
+  if (max_steps < 0) return lsh::lsh_fail(LSH_ERR_INVALID, "negative max_steps");
+  qt->decoder()->set_step_record(logits, alive_seq, max_steps);
+  return LSH_OK;
+}
+
+int ls_model_get_steps_run(ls_model* model, int* steps) {
+  NEED_MODEL(model);
+  QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get());
+  if (!qt) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "step records are a QuantTransformer debug aid");
+  if (!steps) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");
+  *steps = qt->decoder()->steps_run();
   return LSH_OK;
 }
 

@@ -71,5 +71,25 @@ inline std::vector<__half> to_half(const std::vector<float>& v) {
   return out;
 }
 
+// float vector -> fp16 on the device
+inline DeviceBuffer<__half> upload_half(const std::vector<float>& v, hipStream_t s) {
+  std::vector<__half> h = to_half(v);
+  DeviceBuffer<__half> d(h.size());
+  d.upload(h.data(), h.size(), s);
+  CHECK_GPU_ERROR(hipStreamSynchronize(s));  // `h` dies at return
+  return d;
+}
+
+// stored uint8 [rows(in), cols(out)] -> int8 [cols, rows] (K-contiguous for the GEMM)
+inline DeviceBuffer<int8_t> upload_kernel(const std::vector<uint8_t>& w, int rows, int cols,
+                                          bool transpose, hipStream_t s) {
+  DeviceBuffer<uint8_t> raw(w.size());
+  raw.upload(w.data(), w.size(), s);
+  DeviceBuffer<int8_t> q(w.size());
+  LSH_CALL(lsh::stored_u8_to_i8(raw.get(), q.get(), rows, cols, transpose, s));
+  CHECK_GPU_ERROR(hipStreamSynchronize(s));
+  return q;
+}
+
 }  // namespace hip
 }  // namespace lightseq

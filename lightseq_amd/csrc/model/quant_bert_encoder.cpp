@@ -28,32 +28,14 @@ std::string QuantBertEncoder::check() {
   if (_tw._multilg_type != 0) return "multilingual models are not supported";
   if ((int)_tw.layers.size() != _tw._n_enc_layer)
     return "violate p_d_enc_wei.size() = weight_per_enc_layer * n_enc_layer";
-  if ((int)_enc_clip_max.size() != 11 * _tw._n_enc_layer) return "wrong clip_max table size";
+  if ((int)_enc_clip_max.size() != _tw._clip_stride * _tw._n_enc_layer)
+    return "wrong clip_max table size";
   if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)
     return "violate hidden_size % 16 = 0 and inner_size % 16 = 0 (int8 MFMA GEMM)";
   if (_tw._dim_per_head != 32 && _tw._dim_per_head != 64)
     return "violate dim_per_head in {32, 64} (fused attention kernel)";
   if (_tw._max_step > 1024) return "violate max_step <= 1024";
   return "";
-}
-
-static DeviceBuffer<__half> upload_half(const std::vector<float>& v, hipStream_t s) {
-  std::vector<__half> h = to_half(v);
-  DeviceBuffer<__half> d(h.size());
-  d.upload(h.data(), h.size(), s);
-  CHECK_GPU_ERROR(hipStreamSynchronize(s));  // `h` dies at return
-  return d;
-}
-
-// stored uint8 [rows(in), cols(out)] -> int8 [cols, rows] (K-contiguous for the GEMM)
-static DeviceBuffer<int8_t> upload_kernel(const std::vector<uint8_t>& w, int rows, int cols,
-                                          bool transpose, hipStream_t s) {
-  DeviceBuffer<uint8_t> raw(w.size());
-  raw.upload(w.data(), w.size(), s);
-  DeviceBuffer<int8_t> q(w.size());
-  LSH_CALL(stored_u8_to_i8(raw.get(), q.get(), rows, cols, transpose, s));
-  CHECK_GPU_ERROR(hipStreamSynchronize(s));
-  return q;
 }
 
 void QuantBertEncoder::init_buffer() {
@@ -94,11 +76,11 @@ void QuantBertEncoder::init_buffer() {
       DeviceBuffer<uint8_t> raw(n);
       raw.upload(w.ffn_second_kernel.data(), n, _stream);
       DeviceBuffer<__half> deq(n);
-      LSH_CALL(stored_u8_dequant<__half>(raw.get(), deq.get(), (long)n, _enc_clip_max[l * 11 + 3],
+      LSH_CALL(stored_u8_dequant<__half>(raw.get(), deq.get(), (long)n, _enc_clip_max[l * _tw._clip_stride + 3],
                                          _stream));
       d.ffn2_colsum.alloc(H);
       LSH_CALL(scaled_colsum<__half>(deq.get(), d.ffn2_colsum.get(), I, H,
-                                     _enc_clip_max[l * 11 + 7] / 2, _stream));
+                                     _enc_clip_max[l * _tw._clip_stride + 7] / 2, _stream));
       CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
     }
   }
@@ -168,7 +150,8 @@ void QuantBertEncoder::run_one_infer(int batch_size, int batch_seq_len) {
 
   LSH_CALL(enc_emb_i8I<__half>(_int8_emb.get(), _pos_emb.get(), _p_d_token_id, _p_d_output,
                                _p_d_padding_mask, _tw._padding_id, batch_size, batch_seq_len,
-                               _tw._hidden_size, _stream, _src_emb_clip_max / _quant_range, false));
+                               _tw._hidden_size, _stream, _src_emb_clip_max / _quant_range,
+                               _tw._scale_embedding));
   for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
     self_attention();
     ffn_add_norm();
@@ -178,7 +161,7 @@ void QuantBertEncoder::run_one_infer(int batch_size, int batch_seq_len) {
 void QuantBertEncoder::self_attention() {
   const int H = _tw._hidden_size, M = _batch_token_num;
   const Layer& w = _layers[_layer_id];
-  const float* c = &_enc_clip_max[_layer_id * 11];
+  const float* c = &_enc_clip_max[_layer_id * _tw._clip_stride];
   const float Q = _quant_range;
 
   if (_layer_id == 0) {
@@ -234,7 +217,7 @@ void QuantBertEncoder::self_attention() {
 void QuantBertEncoder::ffn_add_norm() {
   const int H = _tw._hidden_size, I = _tw._inner_size, M = _batch_token_num;
   const Layer& w = _layers[_layer_id];
-  const float* c = &_enc_clip_max[_layer_id * 11];
+  const float* c = &_enc_clip_max[_layer_id * _tw._clip_stride];
   const float Q = _quant_range;
 
   // FFN1 -> int8 code -> dequant + bias + activation + requant.  Fused into the GEMM
@@ -286,7 +269,7 @@ void QuantBertEncoder::ffn_add_norm() {
                                            dequant_scale, _stream, colsum));
   } else {
     const Layer& nx = _layers[_layer_id + 1];
-    const float clip_next = _enc_clip_max[(_layer_id + 1) * 11 + 4];
+    const float clip_next = _enc_clip_max[(_layer_id + 1) * _tw._clip_stride + 4];
     LSH_CALL((residual_bias_ln_i8O<__half, int32_t>(
         _int32_ffn_out_buf.get(), nx.ln1_scale.get(), nx.ln1_bias.get(), nx.b_out.get(),
         _int8_ffn_in_buf.get(), _p_d_output, M, H, dequant_scale, Q / clip_next, _stream,

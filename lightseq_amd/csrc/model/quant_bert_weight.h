@@ -43,6 +43,11 @@ class QuantBertWeight {
   // 11 per layer: w_qkv, w_out, w_ffn1, w_ffn2, ln1_out, attn_ctx, ln2_out, ffn_act,
   // qkv_gemm_out, outproj_gemm_out, ffn1_gemm_out
   std::vector<float> _enc_clip_max;
+  // Entries per layer in _enc_clip_max and whether the token embedding is scaled by
+  // sqrt(hidden): 11 / false for QuantBert; the encoder of QuantTransformer carries a
+  // twelfth (unused) clip and scales (inference/model/quant_encoder.cc.cu:140, :242).
+  int _clip_stride = 11;
+  bool _scale_embedding = false;
 
   int _hidden_size = 0, _inner_size = 0, _max_step = 0, _src_vocab_size = 0, _n_enc_layer = 0;
   int _dim_per_head = 0, _head_num = 0, _padding_id = 0, _multilg_type = 0;

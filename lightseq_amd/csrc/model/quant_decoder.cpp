@@ -1,0 +1,395 @@
+#include "quant_decoder.h"
+
+#include "../ls_device.cuh"
+
+#include <algorithm>
+
+namespace lightseq {
+namespace hip {
+
+using namespace lsh;
+
+static const float kMinLogProbability = -2000.f;  // inference/kernels/transformerKernels.h:12
+
+QuantDecoder::QuantDecoder(int max_batch_size, const int* p_d_padding_mask,
+                           const __half* p_d_encoder_output, int* p_d_result,
+                           QuantTransformerWeight& tw, hipStream_t stream, bool output_topk)
+    : _p_d_padding_mask(p_d_padding_mask),
+      _p_d_encoder_output(p_d_encoder_output),
+      _p_d_result(p_d_result),
+      _output_topk(output_topk),
+      _max_batch_size(max_batch_size),
+      _tw(tw),
+      _stream(stream),
+      _trg_emb_clip_max(tw._trg_emb_clip_max),
+      _output_ln_clip_max(tw._output_ln_clip_max),
+      _logits_clip_max(tw._logits_clip_max),
+      _dec_clip_max(tw._dec_clip_max),
+      _layer_size_encdec_k((long)max_batch_size * tw._max_step * tw._hidden_size),
+      _layer_size_self_k((long)max_batch_size * tw._max_step * tw._hidden_size * tw._beam_size),
+      _h_alive_seq_probs((size_t)max_batch_size * std::max(tw._beam_size, 1),
+                         kMinLogProbability / 2),
+      _h_length_norm((size_t)std::max(tw._max_step, 1), 1.f) {
+  // only the first beam of a sentence is alive before the first step (:64-66)
+  for (size_t i = 0; i < _h_alive_seq_probs.size(); i += std::max(tw._beam_size, 1))
+    _h_alive_seq_probs[i] = 0.f;
+  if (tw._length_penalty >= 0)
+    for (size_t i = 0; i < _h_length_norm.size(); i++)
+      _h_length_norm[i] = length_norm((int)i + 1, tw._length_penalty);
+}
+
+QuantDecoder::~QuantDecoder() {
+  if (_h_num_finished) (void)hipHostFree(_h_num_finished);
+}
+
+std::string QuantDecoder::check() {
+  if (_tw._inner_size & 1) return "violate inner_size % 2 = 0";
+  if (_tw._dim_per_head & 1) return "violate dim_per_head % 2 = 0";
+  if (_tw._multilg_type != 0) return "multilingual models are not supported";
+  if ((int)_tw.dec_layers.size() != _tw._n_dec_layer)
+    return "violate p_d_dec_wei.size() = weight_per_dec_layer * n_dec_layer";
+  if ((int)_dec_clip_max.size() != 19 * _tw._n_dec_layer) return "wrong clip_max table size";
+  bool btmp = false;
+  for (int i = 1; i < 64; i *= 2)
+    if (i == _tw._beam_size) btmp = true;
+  if (!btmp) return "wrong beam_size, should be 1, 2, 4, 8, 16 or 32";
+  const std::string& m = _tw._sampling_method;
+  if (m != "beam_search" && m != "topk" && m != "topp" && m != "topk_greedy")
+    return std::string("unsupported sampling_method: ") + m;
+  if (m != "beam_search")
+    return "sampling_method " + m + " is not available in this build (beam_search only)";
+  if (_tw._diverse_lambda != 0.f) return "diverse beam search is not available in this build";
+  if (_tw._max_step > 1024) return "max_step should not greater than 1024";
+  if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)
+    return "violate hidden_size % 16 = 0 and inner_size % 16 = 0 (int8 MFMA GEMM)";
+  if (_tw._end_id < 0 || _tw._end_id >= _tw._trg_vocab_size || _tw._start_id < 0 ||
+      _tw._start_id >= _tw._trg_vocab_size)
+    return "start_id / end_id outside the target vocabulary";
+  return "";
+}
+
+void QuantDecoder::init_buffer() {
+  const int H = _tw._hidden_size, I = _tw._inner_size, L = _tw._n_dec_layer;
+  const int V = _tw._trg_vocab_size, beam = _tw._beam_size;
+  const size_t rows = (size_t)_max_batch_size * beam;
+  const size_t tokens = (size_t)_max_batch_size * _tw._max_step;
+
+  _encdec_k.alloc((size_t)L * _layer_size_encdec_k);
+  _encdec_v.alloc((size_t)L * _layer_size_encdec_k);
+  _encoder_out_buf.alloc(tokens * (size_t)L * 2 * H);
+  _cur_step_query.alloc(rows * H);
+  _query_buf1.alloc(rows * H);
+  const size_t wide = rows * (size_t)std::max(I, 3 * H);
+  _buf_a.alloc(wide);
+  _buf_b.alloc(wide);
+  _logits.alloc(rows * (size_t)V);
+  _int32_ffn_out_buf.alloc(rows * H);
+  for (int i = 0; i < 2; ++i) {
+    _self_k_cache[i].alloc((size_t)L * _layer_size_self_k);
+    _self_v_cache[i].alloc((size_t)L * _layer_size_self_k);
+    CHECK_GPU_ERROR(hipMemsetAsync(_self_k_cache[i].get(), 0, _self_k_cache[i].size(), _stream));
+    CHECK_GPU_ERROR(hipMemsetAsync(_self_v_cache[i].get(), 0, _self_v_cache[i].size(), _stream));
+  }
+  std::vector<int> start_id_vec(rows * _tw._max_step, _tw._start_id);
+  for (int i = 0; i < 2; ++i) {
+    _alive_seq[i].alloc(start_id_vec.size());
+    _alive_seq[i].upload(start_id_vec.data(), start_id_vec.size(), _stream);
+  }
+  _alive_seq_probs.alloc(rows);
+  _alive_seq_score_own.alloc(rows);
+  CHECK_GPU_ERROR(hipMemsetAsync(_alive_seq_score_own.get(), 0, rows * sizeof(float), _stream));
+  if (!_p_d_alive_seq_score) _p_d_alive_seq_score = _alive_seq_score_own.get();
+  _top_score.alloc(rows * beam);
+  _top_idx.alloc(rows * beam);
+  _parent.alloc(rows);
+  _num_finished.alloc(1);
+  CHECK_GPU_ERROR(hipHostMalloc(reinterpret_cast<void**>(&_h_num_finished), sizeof(int)));
+  *_h_num_finished = 0;
+  CHECK_GPU_ERROR(hipStreamSynchronize(_stream));  // start_id_vec dies below
+
+  // ---- embedding block ----
+  // stored [H, vocab]; one [vocab, H] copy serves the row lookup and the logits GEMM
+  _int8_trg_emb = upload_kernel(_tw.trg_token_embedding, H, V, true, _stream);
+  _pos_emb = upload_half(_tw.trg_position_embedding, _stream);
+  _out_ln_scale = upload_half(_tw.trg_norm_scale, _stream);
+  _out_ln_bias = upload_half(_tw.trg_norm_bias, _stream);
+  _kv_bias = upload_half(_tw.encode_output_project_bias_kv, _stream);
+  _logit_bias = upload_half(_tw.shared_bias, _stream);
+  {
+    // The K/V projection stays an fp16 GEMM (:497-501).  File layout [H, n_layer*2*H],
+    // dequantised in flat chunks of 2*H*H with one clip each
+    // (inference/proto/quant_transformer_weight.cc:144-160), then transposed to the
+    // K-contiguous [n_layer*2*H, H] form of the GEMM here.
+    const size_t kv_dim = (size_t)L * 2 * H, chunk = (size_t)2 * H * H;
+    const std::vector<uint8_t>& src = _tw.encode_output_project_kernel_kv;
+    std::vector<__half> t(kv_dim * H);
+    for (size_t k = 0; k < (size_t)H; ++k)
+      for (size_t n = 0; n < kv_dim; ++n) {
+        const size_t flat = k * kv_dim + n;
+        const float clip = _tw._encode_output_project_kernel_kv_clip_max[flat / chunk];
+        // inference/tools/util.cc.cu:346-348
+        const float v = ((float)src[flat] - _quant_range) * clip / _quant_range;
+        t[n * H + k] = __float2half_rn(v);
+      }
+    _kv_kernel.alloc(t.size());
+    _kv_kernel.upload(t.data(), t.size(), _stream);
+    CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+  }
+
+  // ---- layers ----
+  _layers.clear();
+  _layers.resize(L);
+  for (int l = 0; l < L; ++l) {
+    const QuantDecoderLayerWeight& w = _tw.dec_layers[l];
+    Layer& d = _layers[l];
+    d.self_ln_scale = upload_half(w.self_norm_scale, _stream);
+    d.self_ln_bias = upload_half(w.self_norm_bias, _stream);
+    d.b_self_qkv = upload_half(w.self_project_bias_qkv, _stream);
+    d.b_self_out = upload_half(w.self_project_bias_output, _stream);
+    d.encdec_ln_scale = upload_half(w.encdec_norm_scale, _stream);
+    d.encdec_ln_bias = upload_half(w.encdec_norm_bias, _stream);
+    d.b_encdec_q = upload_half(w.encdec_project_bias_q, _stream);
+    d.b_encdec_out = upload_half(w.encdec_project_bias_output, _stream);
+    d.ffn_ln_scale = upload_half(w.ffn_norm_scale, _stream);
+    d.ffn_ln_bias = upload_half(w.ffn_norm_bias, _stream);
+    d.b_ffn1 = upload_half(w.ffn_first_bias, _stream);
+    d.b_ffn2 = upload_half(w.ffn_second_bias, _stream);
+    d.w_self_qkv = upload_kernel(w.self_project_kernel_qkv, H, 3 * H, true, _stream);
+    d.w_self_out = upload_kernel(w.self_project_kernel_output, H, H, true, _stream);
+    d.w_encdec_q = upload_kernel(w.encdec_project_kernel_q, H, H, true, _stream);
+    d.w_encdec_out = upload_kernel(w.encdec_project_kernel_output, H, H, true, _stream);
+    d.w_ffn1 = upload_kernel(w.ffn_first_kernel, H, I, true, _stream);
+    d.w_ffn2 = upload_kernel(w.ffn_second_kernel, I, H, true, _stream);
+    if (!_tw._use_gelu) {
+      // ReLU offset trick (:332-354): column sums of the fp16-rounded dequantised FFN2
+      // kernel times clip/2
+      const size_t n = w.ffn_second_kernel.size();
+      DeviceBuffer<uint8_t> raw(n);
+      raw.upload(w.ffn_second_kernel.data(), n, _stream);
+      DeviceBuffer<__half> deq(n);
+      LSH_CALL(stored_u8_dequant<__half>(raw.get(), deq.get(), (long)n, _dec_clip_max[l * 19 + 5],
+                                         _stream));
+      d.ffn2_colsum.alloc(H);
+      LSH_CALL(scaled_colsum<__half>(deq.get(), d.ffn2_colsum.get(), I, H,
+                                     _dec_clip_max[l * 19 + 11] / 2, _stream));
+      CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+    }
+  }
+}
+
+void QuantDecoder::run_one_infer(int batch_size, int batch_seq_len) {
+  if (batch_size > _max_batch_size)
+    throw std::runtime_error("batch size of input greater than max_batch_size");
+  if (batch_seq_len > _tw._max_step)
+    throw std::runtime_error("seq len of input greater than max_step");
+  if (batch_size <= 0 || batch_seq_len <= 0) throw std::runtime_error("empty input");
+
+  /* ---step1. init--- */
+  _batch_size = batch_size;
+  _batch_seq_len = batch_seq_len;
+  _batch_token_num = batch_size * batch_seq_len;
+  _step_token_num = batch_size * _tw._beam_size;
+  _batch_max_decode_length =
+      std::min(_tw._max_step, batch_seq_len + _tw._extra_decode_length) - 1;
+  _steps_run = 0;
+
+  project_encoder_output();
+  CHECK_GPU_ERROR(hipMemcpyAsync(_alive_seq_probs.get(), _h_alive_seq_probs.data(),
+                                 sizeof(float) * _step_token_num, hipMemcpyHostToDevice,
+                                 _stream));
+
+  /* ---step2. autoregressive decoding--- */
+  for (_cur_step = 0; _cur_step < _batch_max_decode_length - 1; _cur_step++) {
+    bool early_stop = run_step();
+    if (!_is_benchmark && early_stop) break;
+  }
+
+  /* ---step3. output the decoding result--- */
+  int* alive = _alive_seq[_alive_cur].get();
+  if (_output_topk) {
+    if (_cur_step == _batch_max_decode_length) _cur_step -= 1;
+    LSH_CALL(write_topk_result(alive, _p_d_alive_seq_score, _p_d_result, _tw._trg_vocab_size,
+                               _tw._max_step, _tw._beam_size, _tw._end_id, _step_token_num,
+                               _cur_step + 1, _stream));
+    return;
+  }
+  if (_tw._length_penalty >= 0.f || _cur_step == _batch_max_decode_length) {
+    LSH_CALL(write_trg_tokenid_pos_penalty(alive, _p_d_alive_seq_score, _p_d_result,
+                                           _tw._max_step, _tw._beam_size, _batch_size,
+                                           _cur_step + 1, _stream));
+  } else {
+    LSH_CALL(write_trg_tokenid_neg_penalty(alive, _p_d_alive_seq_score, _p_d_result,
+                                           _tw._max_step, _tw._beam_size, _tw._trg_vocab_size,
+                                           _tw._end_id, _batch_size, _cur_step + 1, _stream));
+  }
+}
+
+void QuantDecoder::project_encoder_output() {
+  const int H = _tw._hidden_size, L = _tw._n_dec_layer;
+  const int kv_dim = H * 2 * L;
+  LSH_CALL(gemm_f16_nt(_p_d_encoder_output, _kv_kernel.get(), _encoder_out_buf.get(),
+                       _batch_token_num, kv_dim, H, _stream));
+  // _encoder_out_buf: [batch_size, batch_seq_len, layer_num, 2, hidden_size]
+  LSH_CALL(arrange_encdec_kv<__half>(_batch_token_num, L, H, _stream, _encoder_out_buf.get(),
+                                     _kv_bias.get(), _encdec_k.get(), _encdec_v.get(),
+                                     _layer_size_encdec_k, _batch_seq_len, _tw._dim_per_head,
+                                     _tw._head_num));
+}
+
+bool QuantDecoder::run_step() {
+  embedding();
+  for (_layer_id = 0; _layer_id < _tw._n_dec_layer; _layer_id++) {
+    self_attention();
+    encdec_attention();
+    ffn_add_norm();
+  }
+  /* --- Project hidden states to vocab logits (:527-532) --- */
+  LSH_CALL(gemm_i8_i8o(_buf_a.get(), _int8_trg_emb.get(), _logits.get(), _step_token_num,
+                       _tw._trg_vocab_size, _tw._hidden_size,
+                       _output_ln_clip_max * _trg_emb_clip_max / (_logits_clip_max * _quant_range),
+                       _stream));
+  if (_rec_logits && _cur_step < _rec_max_steps)
+    CHECK_GPU_ERROR(hipMemcpyAsync(
+        _rec_logits + (size_t)_cur_step * _step_token_num * _tw._trg_vocab_size, _logits.get(),
+        (size_t)_step_token_num * _tw._trg_vocab_size, hipMemcpyDeviceToDevice, _stream));
+  ++_steps_run;
+  return beam_search();
+}
+
+void QuantDecoder::embedding() {
+  LSH_CALL(dec_emb_i8I<__half>(_int8_trg_emb.get(), _pos_emb.get(), _alive_seq[_alive_cur].get(),
+                               _cur_step_query.get(), _batch_size, _tw._beam_size,
+                               _tw._hidden_size, _tw._trg_vocab_size, _cur_step, _tw._max_step,
+                               _stream, _trg_emb_clip_max / _quant_range, true, true));
+}
+
+void QuantDecoder::self_attention() {
+  const int H = _tw._hidden_size, M = _step_token_num;
+  const Layer& w = _layers[_layer_id];
+  const float* c = &_dec_clip_max[_layer_id * 19];
+  const float Q = _quant_range;
+  int8_t* k_cache = _self_k_cache[_cache_cur].get() + (size_t)_layer_id * _layer_size_self_k;
+  int8_t* v_cache = _self_v_cache[_cache_cur].get() + (size_t)_layer_id * _layer_size_self_k;
+
+  if (_layer_id == 0) {
+    LSH_CALL(norm_layer_resual_i8O<__half>(M, H, _stream, _cur_step_query.get(), _buf_a.get(),
+                                           w.self_ln_scale.get(), w.self_ln_bias.get(),
+                                           w.b_self_out.get(), Q / c[6], _tw._is_post_ln));
+  }
+  LSH_CALL(gemm_i8_i8o(_buf_a.get(), w.w_self_qkv.get(), _buf_b.get(), M, 3 * H, H,
+                       c[0] * c[6] / (c[12] * Q), _stream));
+  // q -> _buf_a, k / v -> slot _cur_step of the caches (all three with the cache clip)
+  LSH_CALL(arrange_decself_qkv_i8I_i8O<__half>(M, H, _stream, _buf_b.get(), w.b_self_qkv.get(),
+                                               _buf_a.get(), k_cache, v_cache, _tw._head_num,
+                                               _tw._dim_per_head, _tw._max_step, _cur_step,
+                                               c[12] / Q, Q / c[18]));
+  // int8 q.K -> softmax -> new value, one kernel
+  const float attn_scale =
+      __half2float(__float2half_rn(sqrtf(1.f / (float)_tw._dim_per_head)));
+  LSH_CALL(decself_attention_i8(_buf_a.get(), k_cache, v_cache, _buf_b.get(), M * _tw._head_num,
+                                _cur_step + 1, _tw._max_step, _tw._head_num, _tw._dim_per_head,
+                                attn_scale, c[18] / Q, Q / c[7], _stream));
+  LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_self_out.get(), _buf_a.get(), M, H, H,
+                       c[1] * c[7] / (c[13] * Q), _stream));
+  LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(
+      _buf_a.get(), w.encdec_ln_scale.get(), w.encdec_ln_bias.get(), w.b_encdec_out.get(),
+      _buf_b.get(), _cur_step_query.get(), M, H, c[13] / Q, Q / c[8], _stream, _tw._is_post_ln,
+      nullptr)));
+}
+
+void QuantDecoder::encdec_attention() {
+  const int H = _tw._hidden_size, M = _step_token_num;
+  const Layer& w = _layers[_layer_id];
+  const float* c = &_dec_clip_max[_layer_id * 19];
+  const float Q = _quant_range;
+
+  LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_encdec_q.get(), _buf_a.get(), M, H, H,
+                       c[2] * c[8] / (c[14] * Q), _stream));
+  LSH_CALL(arrange_encdec_q_i8I<__half>(M, H, _stream, _buf_a.get(), w.b_encdec_q.get(),
+                                        _query_buf1.get(), _tw._beam_size, _tw._dim_per_head,
+                                        _tw._head_num, c[14] / Q));
+  // scores -> masked softmax -> context -> merge heads + quantise, one kernel
+  LSH_CALL(encdec_attention_f16(
+      _query_buf1.get(), _encdec_k.get() + (size_t)_layer_id * _layer_size_encdec_k,
+      _encdec_v.get() + (size_t)_layer_id * _layer_size_encdec_k, _p_d_padding_mask, nullptr,
+      _buf_b.get(), Q / c[9], _batch_size, _tw._beam_size, _tw._head_num, _batch_seq_len,
+      _tw._dim_per_head, _stream));
+  LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_encdec_out.get(), _buf_a.get(), M, H, H,
+                       c[3] * c[9] / (c[15] * Q), _stream));
+  LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(
+      _buf_a.get(), w.ffn_ln_scale.get(), w.ffn_ln_bias.get(), w.b_ffn2.get(), _buf_b.get(),
+      _cur_step_query.get(), M, H, c[15] / Q, Q / c[10], _stream, _tw._is_post_ln, nullptr)));
+}
+
+void QuantDecoder::ffn_add_norm() {
+  const int H = _tw._hidden_size, I = _tw._inner_size, M = _step_token_num;
+  const Layer& w = _layers[_layer_id];
+  const float* c = &_dec_clip_max[_layer_id * 19];
+  const float Q = _quant_range;
+
+  // FFN1 GEMM with the bias + activation + requantisation in its epilogue
+  const int act = _tw._use_gelu ? kActGelu : kActReluNarrow;
+  LSH_CALL(gemm_i8_bias_act_i8o(_buf_b.get(), w.w_ffn1.get(), _buf_a.get(), w.b_ffn1.get(), M, I,
+                                H, c[4] * c[10] / (c[16] * Q), c[16] / Q, Q / c[11], c[11], act,
+                                _stream));
+  LSH_CALL(gemm_i8_i32o(_buf_a.get(), w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I, _stream));
+
+  const float dequant_scale =
+      _tw._use_gelu ? c[5] * c[11] / (Q * Q) : c[5] * c[11] / (2 * Q * Q);
+  const __half *scale_ptr, *bias_ptr, *res_bias_ptr;
+  float clip_max;
+  if (_layer_id == _tw._n_dec_layer - 1) {
+    scale_ptr = _out_ln_scale.get();
+    bias_ptr = _out_ln_bias.get();
+    res_bias_ptr = nullptr;
+    clip_max = _output_ln_clip_max;
+  } else {
+    const Layer& nx = _layers[_layer_id + 1];
+    scale_ptr = nx.self_ln_scale.get();
+    bias_ptr = nx.self_ln_bias.get();
+    res_bias_ptr = nx.b_self_out.get();
+    clip_max = _dec_clip_max[(_layer_id + 1) * 19 + 6];
+  }
+  LSH_CALL((residual_bias_ln_i8O<__half, int32_t>(
+      _int32_ffn_out_buf.get(), scale_ptr, bias_ptr, res_bias_ptr, _buf_a.get(),
+      _cur_step_query.get(), M, H, dequant_scale, Q / clip_max, _stream, _tw._is_post_ln,
+      w.ffn2_colsum.get())));
+}
+
+bool QuantDecoder::beam_search() {
+  int* alive = _alive_seq[_alive_cur].get();
+  int* alive_new = _alive_seq[_alive_cur ^ 1].get();
+  LSH_CALL(beam_search_step_i8I<__half>(
+      _logits.get(), _logit_bias.get(), _alive_seq_probs.get(), _p_d_alive_seq_score, alive,
+      alive_new, _top_score.get(), _top_idx.get(), _parent.get(), _num_finished.get(),
+      _logits_clip_max / _quant_range, _tw._trg_vocab_size, _tw._max_step,
+      _h_length_norm[_cur_step], _cur_step, _batch_size, _tw._beam_size, _tw._end_id, _stream));
+  _alive_cur ^= 1;
+  if (_rec_alive && _cur_step < _rec_max_steps)
+    CHECK_GPU_ERROR(hipMemcpyAsync(
+        _rec_alive + (size_t)_cur_step * _step_token_num * _tw._max_step, alive_new,
+        (size_t)_step_token_num * _tw._max_step * sizeof(int), hipMemcpyDeviceToDevice, _stream));
+
+  if (!_is_benchmark) {
+    // the one device-to-host word of a step: all beams finished -> stop early
+    CHECK_GPU_ERROR(hipMemcpyAsync(_h_num_finished, _num_finished.get(), sizeof(int),
+                                   hipMemcpyDeviceToHost, _stream));
+    CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+    if (*_h_num_finished == _step_token_num) return true;
+  }
+
+  /* ---refresh cache: k, v for decoder self attention--- */
+  if (_cur_step > 0) {
+    LSH_CALL(refresh_cache_by_parent_i8(
+        _tw._n_dec_layer, _step_token_num, _stream, _parent.get(),
+        _self_k_cache[_cache_cur].get(), _self_v_cache[_cache_cur].get(),
+        _self_k_cache[_cache_cur ^ 1].get(), _self_v_cache[_cache_cur ^ 1].get(),
+        _layer_size_self_k, _tw._beam_size, _tw._dim_per_head, _tw._head_num, _cur_step,
+        _tw._max_step));
+    _cache_cur ^= 1;
+  }
+  return false;
+}
+
+}  // namespace hip
+}  // namespace lightseq

@@ -1,0 +1,119 @@
+#include "quant_transformer.h"
+
+namespace lightseq {
+namespace hip {
+
+QuantTransformer::QuantTransformer(const std::string weight_path, const int max_batch_size)
+    : LSModel({"source_ids"}, {"target_ids", "target_scores"}), _max_batch_size(max_batch_size) {
+  if (max_batch_size <= 0) throw std::runtime_error("max_batch_size must be positive");
+  CHECK_GPU_ERROR(hipSetDevice(0));
+  CHECK_GPU_ERROR(hipStreamCreate(&stream_));
+
+  std::string res = tw_.initializing(weight_path);
+  if (!res.empty()) throw std::runtime_error(res);
+  if (tw_._sampling_method == "topk" || tw_._sampling_method == "topp") tw_._beam_size = 1;
+
+  const size_t tokens = (size_t)_max_batch_size * tw_._max_step;
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_input_), tokens * sizeof(int)));
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_padding_mask_), tokens * sizeof(int)));
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_encoder_output_),
+                            tokens * tw_._hidden_size * sizeof(__half)));
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_output_),
+                            tokens * std::max(tw_._beam_size, 1) * sizeof(int)));
+
+  encoder_ = std::make_shared<QuantBertEncoder>(max_batch_size, d_input_, d_padding_mask_,
+                                                d_encoder_output_, tw_.enc, stream_);
+  res = encoder_->check();
+  if (!res.empty()) throw std::runtime_error(res);
+  decoder_ = std::make_shared<QuantDecoder>(max_batch_size, d_padding_mask_, d_encoder_output_,
+                                            d_output_, tw_, stream_, true);
+  res = decoder_->check();
+  if (!res.empty()) throw std::runtime_error(res);
+  encoder_->init_buffer();
+  decoder_->init_buffer();
+  CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+}
+
+QuantTransformer::~QuantTransformer() {
+  decoder_.reset();
+  encoder_.reset();
+  if (d_input_) (void)hipFree(d_input_);
+  if (d_padding_mask_) (void)hipFree(d_padding_mask_);
+  if (d_encoder_output_) (void)hipFree(d_encoder_output_);
+  if (d_output_) (void)hipFree(d_output_);
+  if (stream_) (void)hipStreamDestroy(stream_);
+}
+
+void QuantTransformer::Infer() {
+  if (input_shapes_[0].size() != 2) throw std::runtime_error("source_ids must be 2-D");
+  int batch_size = input_shapes_[0][0], seq_len = input_shapes_[0][1];
+  if (tw_._multilg_type != 0) throw std::runtime_error("multilingle not supported");
+  encoder_->run_one_infer(batch_size, seq_len);
+  if (enc_out_tap_)
+    CHECK_GPU_ERROR(hipMemcpyAsync(enc_out_tap_, d_encoder_output_,
+                                   (size_t)batch_size * seq_len * tw_._hidden_size * sizeof(__half),
+                                   hipMemcpyDeviceToDevice, stream_));
+  decoder_->run_one_infer(batch_size, seq_len);
+  CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+  encoder_->collect_profile();
+  int output_seq_len = decoder_->_cur_step + 1;
+  int output_k = decoder_->_output_topk ? tw_._beam_size : 1;
+  set_output_shape(0, {batch_size, output_k, output_seq_len});
+  set_output_shape(1, {batch_size, output_k});
+}
+
+void QuantTransformer::set_input_ptr(int index, void* input_ptr) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  encoder_->_p_d_token_id = static_cast<int*>(input_ptr);
+}
+
+void QuantTransformer::set_output_ptr(int index, void* output_ptr) {
+  switch (index) {
+    case 0: decoder_->_p_d_result = static_cast<int*>(output_ptr); break;
+    case 1: decoder_->_p_d_alive_seq_score = static_cast<float*>(output_ptr); break;
+    default: throw std::runtime_error("invalid input index");
+  }
+}
+
+const void* QuantTransformer::get_output_ptr(int index) {
+  switch (index) {
+    case 0: return static_cast<void*>(decoder_->_p_d_result);
+    case 1: return static_cast<void*>(decoder_->_p_d_alive_seq_score);
+    default: throw std::runtime_error("invalid output index");
+  }
+}
+
+std::vector<int> QuantTransformer::get_input_max_shape(int index) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  return {_max_batch_size, tw_._max_step};
+}
+
+std::vector<int> QuantTransformer::get_output_max_shape(int index) {
+  switch (index) {
+    case 0: return {_max_batch_size, tw_._beam_size, tw_._max_step};
+    case 1: return {_max_batch_size, tw_._beam_size};
+    default: throw std::runtime_error("invalid output index");
+  }
+}
+
+DataType QuantTransformer::get_input_dtype(int index) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  return DataType::kInt32;
+}
+
+DataType QuantTransformer::get_output_dtype(int index) {
+  switch (index) {
+    case 0: return DataType::kInt32;
+    case 1: return DataType::kFloat32;
+    default: throw std::runtime_error("invalid output index");
+  }
+}
+
+void QuantTransformer::benchmark_mode(bool is_benchmark) {
+  decoder_->benchmark_mode(is_benchmark);
+}
+
+LSMODEL_REGISTER(QuantTransformer)
+
+}  // namespace hip
+}  // namespace lightseq

@@ -1,7 +1,8 @@
 """``lightseq.inference``-style model classes over the model C ABI.
 
 Mirrors the pybind classes of the reference
-(lightseq/inference/pywrapper/wrapper.cc:240-320 ``PyQuantBert``): the constructor
+(lightseq/inference/pywrapper/wrapper.cc:85-156 ``PyQuantTransformer``, :240-320
+``PyQuantBert``): the constructor
 takes ``(weight_path, max_batch_size)``, ``infer`` takes a C-contiguous int32
 ``[batch, seq_len]`` numpy array, copies it to the device, runs the model and
 returns the output as a float32 numpy array.  Device buffers are allocated once at
@@ -53,6 +54,8 @@ def _bind():
         "ls_model_set_tap": [_P, _I, ctypes.c_char_p, _P],
         "ls_model_set_profiling": [_P, _I],
         "ls_model_get_profile": [_P, ctypes.c_char_p, _I],
+        "ls_model_set_step_record": [_P, _P, _P, _I],
+        "ls_model_get_steps_run": [_P, ip],
     }
     for name, argtypes in sigs.items():
         fn = getattr(L, name)
@@ -223,3 +226,27 @@ class QuantBert(_HostIOModel):
         self._upload(input_seq)
         self.infer_device()
         return self._download(0).cpu().numpy()
+
+
+class QuantTransformer(_HostIOModel):
+    """int8 encoder-decoder with beam search:
+    ``infer(source_ids) -> (tokens int32 [batch, beam, out_len], scores float32 [batch, beam])``.
+    """
+
+    def __init__(self, weight_path, max_batch_size):
+        super().__init__("QuantTransformer", weight_path, max_batch_size)
+
+    def infer(self, input_seq):
+        self._upload(input_seq)
+        self.infer_device()
+        return self._download(0).cpu().numpy(), self._download(1).cpu().numpy()
+
+    def set_step_record(self, logits, alive_seq, max_steps):
+        """Debug aid: device tensors that receive the per-step int8 logits
+        [max_steps, batch*beam, vocab] and sequences [max_steps, batch*beam, max_step]."""
+        self._call("ls_model_set_step_record", self._h,
+                   _P(None if logits is None else logits.data_ptr()),
+                   _P(None if alive_seq is None else alive_seq.data_ptr()), int(max_steps))
+
+    def steps_run(self):
+        return self._int("ls_model_get_steps_run")

@@ -9,7 +9,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADERS = [os.path.join(ROOT, "include", h) for h in ("lightseq_hip.h", "lightseq_model.h")]
-PROTO_RE = re.compile(r"^\s*(?:const\s+char\s*\*|int)\s+((?:lsh|ls_model)_\w+)\s*\(([^;]*?)\)\s*;",
+PROTO_RE = re.compile(r"^\s*(?:const\s+char\s*\*|int|float)\s+((?:lsh|ls_model)_\w+)\s*\(([^;]*?)\)\s*;",
                       re.M | re.S)
 
 
@@ -32,6 +32,8 @@ def _code(arg):
         return "s"
     if arg.startswith("float"):
         return "f"
+    if arg.startswith("int64_t"):
+        return "l"
     if arg.startswith("int"):
         return "i"
     raise AssertionError("unhandled parameter type: %r" % arg)
@@ -64,7 +66,8 @@ def test_ctypes_table_matches_header():
     # and nothing in lightseq_hip.h is left unbound
     bound = {n + s for n, (t, _) in lib._SIGNATURES.items() for s in (("_f16", "_f32") if t else ("",))}
     kernels_header = re.sub(r"/\*.*?\*/", "", open(HEADERS[0]).read(), flags=re.S)
-    declared = {n for n, _ in PROTO_RE.findall(kernels_header)} - {"lsh_last_error", "lsh_version"}
+    declared = {n for n, _ in PROTO_RE.findall(kernels_header)} - {"lsh_last_error", "lsh_version",
+                                                                         "lsh_length_norm"}
     assert declared == bound, declared ^ bound
 
 

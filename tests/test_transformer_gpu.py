@@ -1,0 +1,241 @@
+"""GPU parity of the QuantTransformer model (int8 encoder + int8 decoder with beam search)
+through the model C ABI, against the CPU oracle.
+
+One flipped int8 code can change a token and every token after it, so whole-run equality
+of token ids is only asserted where it is the bar that holds by construction:
+
+ * stage-conditional: the oracle decodes from the GPU's encoder output and consumes the
+   GPU's own logits in its search, so both follow the same token history; then
+   (a) the token ids and sequences are identical at every step -- the search, the
+   sequence / cache refresh and the output writer are bit-exact given equal logits --
+   and (b) the oracle's own logits are equal at step 0 (to the +-1 code / 0.1 % bar) and
+   stay within a few codes of the GPU's at every later step (see the comment at the
+   assertion for why not closer);
+ * free-running oracle vs GPU on small models: identical ids are expected and asserted
+   for the seeds used here (they are deterministic on both sides).
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def _make(tmp_path, cfg, seed, **kw):
+    from lightseq_amd import synthetic
+    path = os.path.join(str(tmp_path), "qt_%d.pb" % seed)
+    msg = synthetic.write_quant_transformer(path, cfg, seed=seed, **kw)
+    return path, msg
+
+
+def _src_ids(cfg, batch, seq, seed):
+    from lightseq_amd import synthetic
+    ids, _ = synthetic.make_token_ids(dict(vocab=cfg["src_vocab"], padding_id=cfg["padding_id"]),
+                                      batch, seq, seed=seed)
+    return ids
+
+
+def _run_gpu(path, cfg, ids, max_batch, record=True, benchmark=False):
+    from lightseq_amd.inference import QuantTransformer
+    model = QuantTransformer(path, max_batch)
+    batch, seq = ids.shape
+    rows = batch * cfg["beam_size"]
+    rec = {}
+    if record:
+        rec["logits"] = torch.zeros(cfg["max_step"], rows, cfg["trg_vocab"], dtype=torch.int8,
+                                    device=DEV)
+        rec["alive"] = torch.zeros(cfg["max_step"], rows, cfg["max_step"], dtype=torch.int32,
+                                   device=DEV)
+        rec["enc_out"] = torch.zeros(batch, seq, cfg["hidden"], dtype=torch.float16, device=DEV)
+        model.set_step_record(rec["logits"], rec["alive"], cfg["max_step"])
+        model.set_tap(-1, "enc_out", rec["enc_out"])
+    model.benchmark_mode(benchmark)
+    tokens, scores = model.infer(ids)
+    steps = model.steps_run()
+    out = {"tokens": tokens, "scores": scores, "steps": steps}
+    for k, v in rec.items():
+        out[k] = v.cpu().numpy()
+    if record:
+        out["logits"] = out["logits"][:steps]
+        out["alive"] = out["alive"][:steps]
+    model.close()
+    return out
+
+
+def _oracle_weights(msg, cfg):
+    from oracle import model_io
+    return model_io.oracle_transformer_weights_from_message(msg, cfg, np.float16)
+
+
+def _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch):
+    enc_w, dec_w = _oracle_weights(msg, cfg)
+    # encoder stage: the fp16 hidden states (layer outputs, tolerance of the path: 2e-2)
+    want_enc, mask, _ = oracle.quant_bert_encoder(enc_w, ids)
+    valid = mask == 0
+    err = np.abs(gpu["enc_out"].astype(np.float32) - want_enc.astype(np.float32))[valid]
+    assert err.max() <= 2e-2 or np.mean(err > 2e-2) < 2e-3, err.max()
+
+    # decoder, conditioned on the GPU's encoder output and logits
+    r = oracle.quant_decoder(dec_w, gpu["enc_out"], mask, forced_logits=gpu["logits"], record=True)
+    assert r["steps_run"] == gpu["steps"]
+    np.testing.assert_array_equal(r["alive_seq"], gpu["alive"])
+    np.testing.assert_array_equal(r["ids"], gpu["tokens"])
+    # scores of finished beams (the others hold whatever the buffer held)
+    end_id = dec_w["end_id"]
+    finished = (gpu["alive"][-1][:, 1:gpu["steps"] + 1] == end_id).any(axis=1)
+    g_sc, w_sc = gpu["scores"].reshape(-1), r["scores"].reshape(-1)
+    np.testing.assert_allclose(g_sc[finished], w_sc[finished], rtol=2e-6, atol=2e-4)
+
+    # the oracle's own logits, step by step, on the same token history
+    diff = np.abs(r["logits"].astype(np.int32) - gpu["logits"].astype(np.int32))
+    frac = float((diff != 0).mean())
+    frac2 = float((diff > 1).mean())
+    print("steps %d: %.3f%% of logit codes differ, %.4f%% by more than one code, max %d" %
+          (gpu["steps"], 100 * frac, 100 * frac2, diff.max()))
+    # Step 0 has no history (one key, softmax == 1): everything up to the logits must agree
+    # to the kernel-level bar.  Later steps: each side reads its own K/V cache, and every
+    # int8-output GEMM turns one flipped input code into a +-1 flip on a few percent of its
+    # outputs, so a row that has seen one flip anywhere upstream is decorrelated at the
+    # rounding level (still within a few codes) -- the bound below is on magnitude, plus a
+    # loose one on the fraction.
+    d0 = diff[0]
+    assert d0.max() <= 1 and (d0 != 0).mean() <= 1e-3, "step 0 logits differ"
+    assert diff.max() <= 6, "logit codes differ by %d" % diff.max()
+    assert frac2 <= 2e-2, "%.3f%% of logit codes differ by more than one code" % (100 * frac2)
+    assert frac <= max_logit_mismatch, "%.3f%% of logit codes differ" % (100 * frac)
+    return r, frac
+
+
+TINY_CASES = [  # seed, eos_bias (in sigma of the logits), batch, seq
+    (1, 1.0, 3, 10),
+    (2, 4.0, 2, 7),
+    (3, 2.5, 4, 12),
+    (4, 3.0, 1, 5),
+]
+
+
+@pytest.mark.parametrize("seed,eos,batch,seq", TINY_CASES)
+def test_tiny_transformer(oracle, tmp_path, seed, eos, batch, seq):
+    from lightseq_amd import synthetic
+    cfg = synthetic.transformer_config("tiny")
+    sigma = 0.02 * np.sqrt(cfg["hidden"])
+    path, msg = _make(tmp_path, cfg, seed, eos_bias=eos * sigma, w_std=0.2)
+    ids = _src_ids(cfg, batch, seq, seed)
+    gpu = _run_gpu(path, cfg, ids, max_batch=4)
+    assert gpu["tokens"].shape[:2] == (batch, cfg["beam_size"])
+    assert gpu["scores"].shape == (batch, cfg["beam_size"])
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
+
+    # free-running oracle (its own encoder output and logits): identical ids
+    enc_w, dec_w = _oracle_weights(msg, cfg)
+    enc_out, mask, _ = oracle.quant_bert_encoder(enc_w, ids)
+    free = oracle.quant_decoder(dec_w, enc_out, mask)
+    assert free["ids"].shape == gpu["tokens"].shape
+    same = float((free["ids"] == gpu["tokens"]).all(axis=-1).mean())
+    assert same == 1.0, "only %.0f%% of the beams agree with the free-running oracle" % (100 * same)
+
+
+def test_early_stop_and_benchmark_mode(oracle, tmp_path):
+    """A model that ends every beam early: early stop shortens the output; benchmark mode
+    runs to the length limit and pads with <eos>, as the reference does."""
+    from lightseq_amd import synthetic
+    cfg = synthetic.transformer_config("tiny")
+    sigma = 0.02 * np.sqrt(cfg["hidden"])
+    path, msg = _make(tmp_path, cfg, 1, eos_bias=4.0 * sigma, w_std=0.2)
+    ids = _src_ids(cfg, 3, 10, 0)
+    gpu = _run_gpu(path, cfg, ids, max_batch=3)
+    limit = min(cfg["max_step"], ids.shape[1] + cfg["extra_decode_length"]) - 1
+    assert gpu["steps"] < limit - 1, "expected an early stop"
+    assert gpu["tokens"].shape[2] == gpu["steps"]
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
+
+    bench = _run_gpu(path, cfg, ids, max_batch=3, benchmark=True)
+    assert bench["steps"] == limit - 1
+    n = gpu["tokens"].shape[2]
+    np.testing.assert_array_equal(bench["tokens"][:, :, :n], gpu["tokens"])
+    assert (bench["tokens"][:, :, n:] == cfg["end_id"]).all()
+    enc_w, dec_w = _oracle_weights(msg, cfg)
+    enc_out, mask, _ = oracle.quant_bert_encoder(enc_w, ids)
+    want = oracle.quant_decoder(dec_w, bench["enc_out"], mask, is_benchmark=True,
+                                forced_logits=bench["logits"])
+    np.testing.assert_array_equal(want["ids"], bench["tokens"])
+
+
+def test_gelu_post_ln_variant(oracle, tmp_path):
+    from lightseq_amd import synthetic
+    cfg = synthetic.transformer_config("tiny")
+    cfg.update(use_gelu=True, is_post_ln=True, beam_size=2, length_penalty=-1.0)
+    sigma = 0.02 * np.sqrt(cfg["hidden"])
+    path, msg = _make(tmp_path, cfg, 5, eos_bias=2.0 * sigma, w_std=0.2)
+    ids = _src_ids(cfg, 2, 9, 5)
+    gpu = _run_gpu(path, cfg, ids, max_batch=2)
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
+
+
+def test_repeated_infer_is_deterministic(tmp_path):
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import QuantTransformer
+    cfg = synthetic.transformer_config("tiny")
+    path, _ = _make(tmp_path, cfg, 7, w_std=0.2)
+    model = QuantTransformer(path, 4)
+    a = _src_ids(cfg, 4, 11, 1)
+    b = _src_ids(cfg, 2, 6, 2)
+    ta, sa = model.infer(a)
+    tb, _ = model.infer(b)
+    ta2, sa2 = model.infer(a)
+    np.testing.assert_array_equal(ta, ta2)
+    assert tb.shape[0] == 2
+    # sentences are decoded independently: a sub-batch gives the same beams
+    ts, _ = model.infer(a[:2])
+    n = min(ts.shape[2], ta.shape[2])
+    np.testing.assert_array_equal(ts[:, :, :n], ta[:2, :, :n])
+    model.close()
+
+
+def test_interface_and_errors(tmp_path):
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import LSModel, QuantTransformer
+    from lightseq_amd.lib import LSHError
+    cfg = synthetic.transformer_config("tiny")
+    path, _ = _make(tmp_path, cfg, 8, w_std=0.2)
+    model = QuantTransformer(path, 2)
+    assert model.get_input_size() == 1 and model.get_output_size() == 2
+    assert model.get_input_name(0) == "source_ids"
+    assert [model.get_output_name(i) for i in range(2)] == ["target_ids", "target_scores"]
+    assert model.get_input_max_shape(0) == [2, cfg["max_step"]]
+    assert model.get_output_max_shape(0) == [2, cfg["beam_size"], cfg["max_step"]]
+    assert model.get_output_max_shape(1) == [2, cfg["beam_size"]]
+    assert model.get_input_dtype(0) == 2 and model.get_output_dtype(0) == 2
+    assert model.get_output_dtype(1) == 1
+    with pytest.raises(LSHError, match="max_batch_size"):
+        model.infer(_src_ids(cfg, 3, 5, 0))
+    with pytest.raises(LSHError, match="max_step"):
+        model._d_input = torch.zeros(2 * (cfg["max_step"] + 1), dtype=torch.int32, device=DEV)
+        model.infer(_src_ids(cfg, 1, cfg["max_step"] + 1, 0))
+    model.close()
+    with pytest.raises(LSHError, match="failed"):
+        LSModel("QuantTransformer", os.path.join(str(tmp_path), "missing.pb"), 2)
+    bad = dict(cfg, sampling_method="topp")
+    path2 = os.path.join(str(tmp_path), "topp.pb")
+    synthetic.write_quant_transformer(path2, bad, seed=1)
+    with pytest.raises(LSHError, match="sampling_method"):
+        LSModel("QuantTransformer", path2, 2)
+
+
+def test_transformer_big_shape(oracle, tmp_path):
+    """Transformer-big-shaped model (hidden 1024, 16 heads, inner 4096, vocabulary 32000,
+    beam 4) with fewer layers so that the oracle finishes in seconds: stage-conditional
+    parity of every decoding step."""
+    from lightseq_amd import synthetic
+    cfg = synthetic.transformer_config("transformer_big")
+    cfg.update(n_enc_layer=2, n_dec_layer=2, max_step=32, extra_decode_length=12)
+    sigma = 0.02 * np.sqrt(cfg["hidden"])
+    path, msg = _make(tmp_path, cfg, 11, eos_bias=2.5 * sigma, w_std=0.05)
+    ids = _src_ids(cfg, 4, 16, 3)
+    gpu = _run_gpu(path, cfg, ids, max_batch=4)
+    _, frac = _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
+    print("transformer-big shape: %d steps, %.3f%% logit codes differ" % (gpu["steps"], 100 * frac))
