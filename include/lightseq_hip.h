@@ -461,6 +461,102 @@ int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, c
                                    int8_t* v_new, int64_t layer_offset, int beam_size,
                                    int dim_per_head, int head_num, int cur_step, int max_step);
 
+/* ======================================================================== */
+/* GPT path                                                                   */
+/* ======================================================================== */
+
+/* kernels/gptKernels_int8.h ker_gpt_embedding_i8I_launcher
+ * (gptKernels_int8.cc.cu:71-94).  token_emb [vocab, hidden] int8 codes; token_id
+ * [batch_size, batch_seq_len]; output [batch_size, batch_seq_len, hidden] T (zeros at
+ * padding); real_seq_len[b] += non-padding tokens of row b.  Token ids must lie inside
+ * the table, as for the reference. */
+int lsh_ker_gpt_embedding_i8I_f16(int batch_size, int batch_seq_len, int hidden_size,
+                                  lsh_stream_t stream, const int8_t* token_emb,
+                                  const void* pos_emb, const int* token_id, void* output,
+                                  int* real_seq_len, int padding_id, int pos_offset,
+                                  float dequant_scale);
+int lsh_ker_gpt_embedding_i8I_f32(int batch_size, int batch_seq_len, int hidden_size,
+                                  lsh_stream_t stream, const int8_t* token_emb,
+                                  const void* pos_emb, const int* token_id, void* output,
+                                  int* real_seq_len, int padding_id, int pos_offset,
+                                  float dequant_scale);
+/* The strided-batched int8 GEMM of model/quant_gpt_encoder.cc.cu:498-505:
+ * scores[bh, i, j] = sum_d q[bh, i, d] * k[bh, j, d], all [batch*head, seq, ...]. */
+int lsh_gpt_scores_i8_i32o(const int8_t* k, const int8_t* q, int32_t* scores, int batch_head_num,
+                           int batch_seq_len, int dim_per_head, lsh_stream_t stream);
+/* kernels/gptKernels_int8.h ker_correlation_softmax_gpt_i32I_launcher
+ * (gptKernels_int8.cc.cu:225-240).  Rows of padded queries (position >= real_seq_len)
+ * are written as zeros; the reference leaves them untouched. */
+int lsh_ker_correlation_softmax_gpt_i32I_f16(int batch_size, int batch_seq_len, int head_num,
+                                             lsh_stream_t stream, const int32_t* correlation,
+                                             void* output, const int* real_seq_len,
+                                             float attn_scale, float dequant_scale);
+int lsh_ker_correlation_softmax_gpt_i32I_f32(int batch_size, int batch_seq_len, int head_num,
+                                             lsh_stream_t stream, const int32_t* correlation,
+                                             void* output, const int* real_seq_len,
+                                             float attn_scale, float dequant_scale);
+/* kernels/gptKernels_int8.h ker_arrange_qkv_with_cache_i8I_i8O_launcher
+ * (gptKernels_int8.cc.cu:772-798): batch_token_num = batch * batch_seq_len; caches are
+ * re-laid out from [batch, head, batch_seq_len-1, d] (k_cache, v_cache) to
+ * [batch, head, batch_seq_len, d] (new_k, new_v) with the new token appended. */
+int lsh_ker_arrange_qkv_with_cache_i8I_i8O_f16(int batch_token_num, int hidden_size,
+                                               lsh_stream_t stream, const int8_t* ori_qkv,
+                                               const void* qkv_bias, int8_t* new_q, int8_t* new_k,
+                                               const int8_t* k_cache, int8_t* new_v,
+                                               const int8_t* v_cache, int batch_seq_len,
+                                               int dim_per_head, int head_num,
+                                               float dequant_scale, float quant_scale,
+                                               int in_col32);
+int lsh_ker_arrange_qkv_with_cache_i8I_i8O_f32(int batch_token_num, int hidden_size,
+                                               lsh_stream_t stream, const int8_t* ori_qkv,
+                                               const void* qkv_bias, int8_t* new_q, int8_t* new_k,
+                                               const int8_t* k_cache, int8_t* new_v,
+                                               const int8_t* v_cache, int batch_seq_len,
+                                               int dim_per_head, int head_num,
+                                               float dequant_scale, float quant_scale,
+                                               int in_col32);
+/* kernels/gptKernels_int8.h ker_topk_sample_i8I_launcher (gptKernels_int8.cc.cu:422-463).
+ * k == 1 (greedy) only: k in {2,..,32} -> LSH_ERR_UNSUPPORTED (random sampling needs the
+ * reference's curand state, passed here as an ignored pointer), other k ->
+ * LSH_ERR_INVALID with the reference's message.  Ties at the maximum go to the lowest
+ * token id (racing stores decide in the reference).  real_seq_len is unused, as in the
+ * reference. */
+int lsh_ker_topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len,
+                            int max_thread_per_block, lsh_stream_t stream, const int8_t* logits,
+                            int* old_input_ids, int* new_input_ids, const int* real_seq_len,
+                            int vocab_size, int k, int* unfinished, void* curandstate, int eos_id,
+                            float dequant_scale, int in_col32);
+/* kernels/gptKernels_int8.h ker_ppl_i8I_launcher (gptKernels_int8.cc.cu:182-190). */
+int lsh_ker_ppl_i8I(int batch_size, int batch_seq_len, int max_thread_per_block,
+                    lsh_stream_t stream, const int8_t* logits, const int* input_ids,
+                    const int* real_seq_len, float* ppl, int vocab_size, float dequant_scale,
+                    int in_col32);
+
+/* Prompt pass of the model, no single counterpart in the reference:
+ *  - lsh_gpt_arrange_qkv_prefill_f16 = ker_arrange_encself_qkv_i8I_i8O_launcher
+ *    (model/quant_gpt_encoder.cc.cu:489-496) writing q / k as fp16 code values and v
+ *    dequantised, each [batch, head, seq, d], plus k / v codes into caches of fixed
+ *    stride [batch, head, max_step, d];
+ *  - lsh_gpt_prefill_attention_f16 = the int8 q.K^T GEMM, ker_correlation_softmax_gpt_i32I,
+ *    the P.V GEMM and ker_arrange_atten_output_i8O (:498-530) in one causal kernel: the
+ *    fp32 MFMA accumulators over code values are the exact int32 scores.  ctx
+ *    ([batch, head, seq, d] fp16) and ctx_q ([batch*seq, hidden] int8) are each optional;
+ *  - lsh_gpt_greedy_step = ker_topk_sample_i8I<1> on ids kept in place as
+ *    [batch, max_step]: writes column cur_len, last_ids[batch] and the unfinished flag. */
+int lsh_gpt_arrange_qkv_prefill_f16(int batch_token_num, int hidden_size, lsh_stream_t stream,
+                                    const int8_t* ori_qkv, const void* qkv_bias, void* q_codes,
+                                    void* k_codes, void* v_deq, int8_t* k_cache, int8_t* v_cache,
+                                    int batch_seq_len, int dim_per_head, int head_num,
+                                    int max_step, float dequant_scale, float quant_scale);
+int lsh_gpt_prefill_attention_f16(const void* q_codes, const void* k_codes, const void* v,
+                                  const int* real_seq_len, void* ctx, int8_t* ctx_q,
+                                  float quant_scale, float dequant_scale, int batch_size,
+                                  int batch_seq_len, int head_num, int dim_per_head,
+                                  lsh_stream_t stream);
+int lsh_gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size,
+                        int max_step, int cur_len, int batch_size, int* unfinished, int eos_id,
+                        lsh_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -102,12 +102,19 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ float round_h(float x) { return (float)(_Float16)x; }
 
-template <int D>
+// GPT = true turns the kernel into the causal prompt attention of the int8 GPT path
+// (inference/model/quant_gpt_encoder.cc.cu:498-523 with
+// inference/kernels/gptKernels_int8.cc.cu:192-222): q and k hold int8 codes as fp16
+// values, so the fp32 MFMA accumulators are the exact int32 scores; a score becomes
+// float(acc) * alpha * dq * dq without fp16 rounding, key j is visible to query i when
+// j <= i, `pad_mask` is the per-sequence real length and queries at or beyond it give
+// zeros.  Key blocks entirely to the right of the query block are skipped.
+template <int D, bool GPT>
 __global__ void __launch_bounds__(128)
 encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
                     const __half* __restrict__ v, const int* __restrict__ pad_mask,
                     __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale, int S,
-                    int head_num, float alpha) {
+                    int head_num, float alpha, float dq) {
   constexpr int KSTR = D + 8;    // halfs per K row in LDS (pad kills bank conflicts)
   constexpr int VSTR = 128 + 4;  // halfs per V^T row in LDS
   constexpr int CH = D / 8;      // 16-byte chunks per row
@@ -132,7 +139,7 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
     else
       qreg[ks] = (v8h)(_Float16)0;
   }
-  const bool q_pad = qi >= S || pad_mask[(long)b * S + qi] != 0;
+  const bool q_pad = qi >= S || (GPT ? qi >= pad_mask[b] : pad_mask[(long)b * S + qi] != 0);
 
   float m = kFloatInfNeg, sum = 0.f;
   v16f sc[4];
@@ -142,7 +149,8 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
-  const int nkb = (S + 127) / 128;
+  int nkb = (S + 127) / 128;
+  if (GPT) nkb = min(nkb, min((int)blockIdx.x * 64 + 63, S - 1) / 128 + 1);
   for (int phase = 0; phase < 2; ++phase) {
     for (int kb = 0; kb < nkb; ++kb) {
       const int key0 = kb * 128;
@@ -164,7 +172,10 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
             for (int i = 0; i < 8; ++i) Vt[(ch * 8 + i) * VSTR + row] = vv[i];
           }
         }
-        msk[tid] = (key0 + tid < S) ? pad_mask[(long)b * S + key0 + tid] : 1;
+        if (GPT)
+          msk[tid] = (key0 + tid < S) ? 0 : 1;
+        else
+          msk[tid] = (key0 + tid < S) ? pad_mask[(long)b * S + key0 + tid] : 1;
         __syncthreads();
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb) {
@@ -179,7 +190,11 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             const int key_local = sb * 32 + 8 * (i / 4) + 4 * g + (i % 4);
-            sc[sb][i] = msk[key_local] ? kFloatInfNeg : round_h(alpha * c[i]);
+            if (GPT)
+              sc[sb][i] = (msk[key_local] || key0 + key_local > qi) ? kFloatInfNeg
+                                                                    : c[i] * alpha * dq * dq;
+            else
+              sc[sb][i] = msk[key_local] ? kFloatInfNeg : round_h(alpha * c[i]);
           }
         }
       }
@@ -266,21 +281,62 @@ int encself_attention_f16(const __half* q, const __half* k, const __half* v, con
   dim3 grid((seq_len + 63) / 64, batch * head_num);
   switch (dim_per_head) {
     case 32:
-      encself_attn_kernel<32><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q, quant_scale,
-                                                   seq_len, head_num, alpha);
+      encself_attn_kernel<32, false><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
+                                                          quant_scale, seq_len, head_num, alpha,
+                                                          0.f);
       break;
     case 64:
-      encself_attn_kernel<64><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q, quant_scale,
-                                                   seq_len, head_num, alpha);
+      encself_attn_kernel<64, false><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
+                                                          quant_scale, seq_len, head_num, alpha,
+                                                          0.f);
       break;
     case 128:
-      encself_attn_kernel<128><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q, quant_scale,
-                                                    seq_len, head_num, alpha);
+      encself_attn_kernel<128, false><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
+                                                           quant_scale, seq_len, head_num, alpha,
+                                                           0.f);
       break;
     default:
       return lsh_fail(LSH_ERR_UNSUPPORTED, "encself_attention: dim_per_head must be 32, 64 or 128");
   }
   return lsh_check_launch("encself_attn_kernel");
+}
+
+int gpt_prefill_attention_f16(const __half* q_codes, const __half* k_codes, const __half* v,
+                              const int* real_seq_len, __half* ctx, int8_t* ctx_q,
+                              float quant_scale, float dequant_scale, int batch, int seq_len,
+                              int head_num, int dim_per_head, hipStream_t s) {
+  if (batch <= 0 || seq_len <= 0 || head_num <= 0 || !q_codes || !k_codes || !v ||
+      !real_seq_len || (!ctx && !ctx_q))
+    return lsh_fail(LSH_ERR_INVALID, "gpt_prefill_attention: bad arguments");
+  if (seq_len > 4096)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "gpt_prefill_attention: seq_len > 4096");
+  if (((reinterpret_cast<uintptr_t>(q_codes) | reinterpret_cast<uintptr_t>(k_codes) |
+        reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(ctx) |
+        reinterpret_cast<uintptr_t>(ctx_q)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_INVALID, "gpt_prefill_attention: pointers must be 16-byte aligned");
+  const float alpha = __half2float(__float2half_rn(sqrtf(1.f / (float)dim_per_head)));
+  dim3 grid((seq_len + 63) / 64, batch * head_num);
+  switch (dim_per_head) {
+    case 32:
+      encself_attn_kernel<32, true><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
+                                                         ctx_q, quant_scale, seq_len, head_num,
+                                                         alpha, dequant_scale);
+      break;
+    case 64:
+      encself_attn_kernel<64, true><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
+                                                         ctx_q, quant_scale, seq_len, head_num,
+                                                         alpha, dequant_scale);
+      break;
+    case 128:
+      encself_attn_kernel<128, true><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
+                                                          ctx_q, quant_scale, seq_len, head_num,
+                                                          alpha, dequant_scale);
+      break;
+    default:
+      return lsh_fail(LSH_ERR_UNSUPPORTED,
+                      "gpt_prefill_attention: dim_per_head must be 32, 64 or 128");
+  }
+  return lsh_check_launch("encself_attn_kernel<GPT>");
 }
 
 }  // namespace lsh

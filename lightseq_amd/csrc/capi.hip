@@ -562,4 +562,107 @@ int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, c
                                     cur_step, max_step);
 }
 
+// ---- GPT path ------------------------------------------------------------------------
+int lsh_ker_gpt_embedding_i8I_f16(int batch_size, int batch_seq_len, int hidden_size,
+                                  lsh_stream_t stream, const int8_t* token_emb,
+                                  const void* pos_emb, const int* token_id, void* output,
+                                  int* real_seq_len, int padding_id, int pos_offset,
+                                  float dequant_scale) {
+  return gpt_embedding_i8I<__half>(batch_size, batch_seq_len, hidden_size, HS(stream), token_emb,
+                                   H(pos_emb), token_id, HM(output), real_seq_len, padding_id,
+                                   pos_offset, dequant_scale, 0, 0);
+}
+int lsh_ker_gpt_embedding_i8I_f32(int batch_size, int batch_seq_len, int hidden_size,
+                                  lsh_stream_t stream, const int8_t* token_emb,
+                                  const void* pos_emb, const int* token_id, void* output,
+                                  int* real_seq_len, int padding_id, int pos_offset,
+                                  float dequant_scale) {
+  return gpt_embedding_i8I<float>(batch_size, batch_seq_len, hidden_size, HS(stream), token_emb,
+                                  F(pos_emb), token_id, FM(output), real_seq_len, padding_id,
+                                  pos_offset, dequant_scale, 0, 0);
+}
+int lsh_gpt_scores_i8_i32o(const int8_t* k, const int8_t* q, int32_t* scores, int batch_head_num,
+                           int batch_seq_len, int dim_per_head, lsh_stream_t stream) {
+  return gpt_scores_i8(q, k, scores, batch_head_num, batch_seq_len, dim_per_head, HS(stream));
+}
+int lsh_ker_correlation_softmax_gpt_i32I_f16(int batch_size, int batch_seq_len, int head_num,
+                                             lsh_stream_t stream, const int32_t* correlation,
+                                             void* output, const int* real_seq_len,
+                                             float attn_scale, float dequant_scale) {
+  return correlation_softmax_gpt_i32I<__half>(batch_size, batch_seq_len, head_num, HS(stream),
+                                              correlation, HM(output), real_seq_len, attn_scale,
+                                              dequant_scale);
+}
+int lsh_ker_correlation_softmax_gpt_i32I_f32(int batch_size, int batch_seq_len, int head_num,
+                                             lsh_stream_t stream, const int32_t* correlation,
+                                             void* output, const int* real_seq_len,
+                                             float attn_scale, float dequant_scale) {
+  return correlation_softmax_gpt_i32I<float>(batch_size, batch_seq_len, head_num, HS(stream),
+                                             correlation, FM(output), real_seq_len, attn_scale,
+                                             dequant_scale);
+}
+#define LSH_QKV_CACHE(NAME, TY, CAST_C)                                                        \
+  int NAME(int batch_token_num, int hidden_size, lsh_stream_t stream, const int8_t* ori_qkv,   \
+           const void* qkv_bias, int8_t* new_q, int8_t* new_k, const int8_t* k_cache,          \
+           int8_t* new_v, const int8_t* v_cache, int batch_seq_len, int dim_per_head,          \
+           int head_num, float dequant_scale, float quant_scale, int in_col32) {               \
+    if (int rc = no_col32(in_col32, 0, "ker_arrange_qkv_with_cache_i8I_i8O")) return rc;       \
+    return arrange_qkv_with_cache_i8I_i8O<TY>(batch_token_num, hidden_size, HS(stream),        \
+                                              ori_qkv, CAST_C(qkv_bias), new_q, new_k, k_cache, \
+                                              new_v, v_cache, batch_seq_len, dim_per_head,     \
+                                              head_num, dequant_scale, quant_scale);           \
+  }
+LSH_QKV_CACHE(lsh_ker_arrange_qkv_with_cache_i8I_i8O_f16, __half, H)
+LSH_QKV_CACHE(lsh_ker_arrange_qkv_with_cache_i8I_i8O_f32, float, F)
+#undef LSH_QKV_CACHE
+
+int lsh_ker_topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len,
+                            int max_thread_per_block, lsh_stream_t stream, const int8_t* logits,
+                            int* old_input_ids, int* new_input_ids, const int* real_seq_len,
+                            int vocab_size, int k, int* unfinished, void* curandstate, int eos_id,
+                            float dequant_scale, int in_col32) {
+  (void)max_thread_per_block;
+  (void)real_seq_len;
+  (void)curandstate;
+  if (int rc = no_col32(in_col32, 0, "ker_topk_sample_i8I")) return rc;
+  if (!(dequant_scale > 0.f))
+    return lsh_fail(LSH_ERR_INVALID, "ker_topk_sample_i8I: dequant_scale must be positive");
+  return topk_sample_i8I(batch_size, batch_seq_len, logits_seq_len, HS(stream), logits,
+                         old_input_ids, new_input_ids, vocab_size, k, unfinished, eos_id);
+}
+int lsh_ker_ppl_i8I(int batch_size, int batch_seq_len, int max_thread_per_block,
+                    lsh_stream_t stream, const int8_t* logits, const int* input_ids,
+                    const int* real_seq_len, float* ppl, int vocab_size, float dequant_scale,
+                    int in_col32) {
+  (void)max_thread_per_block;
+  if (int rc = no_col32(in_col32, 0, "ker_ppl_i8I")) return rc;
+  return ppl_i8I(batch_size, batch_seq_len, HS(stream), logits, input_ids, real_seq_len, ppl,
+                 vocab_size, dequant_scale);
+}
+int lsh_gpt_arrange_qkv_prefill_f16(int batch_token_num, int hidden_size, lsh_stream_t stream,
+                                    const int8_t* ori_qkv, const void* qkv_bias, void* q_codes,
+                                    void* k_codes, void* v_deq, int8_t* k_cache, int8_t* v_cache,
+                                    int batch_seq_len, int dim_per_head, int head_num,
+                                    int max_step, float dequant_scale, float quant_scale) {
+  return gpt_arrange_qkv_prefill_f16(batch_token_num, hidden_size, HS(stream), ori_qkv,
+                                     H(qkv_bias), HM(q_codes), HM(k_codes), HM(v_deq), k_cache,
+                                     v_cache, batch_seq_len, dim_per_head, head_num, max_step,
+                                     dequant_scale, quant_scale);
+}
+int lsh_gpt_prefill_attention_f16(const void* q_codes, const void* k_codes, const void* v,
+                                  const int* real_seq_len, void* ctx, int8_t* ctx_q,
+                                  float quant_scale, float dequant_scale, int batch_size,
+                                  int batch_seq_len, int head_num, int dim_per_head,
+                                  lsh_stream_t stream) {
+  return gpt_prefill_attention_f16(H(q_codes), H(k_codes), H(v), real_seq_len, HM(ctx), ctx_q,
+                                   quant_scale, dequant_scale, batch_size, batch_seq_len,
+                                   head_num, dim_per_head, HS(stream));
+}
+int lsh_gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size,
+                        int max_step, int cur_len, int batch_size, int* unfinished, int eos_id,
+                        lsh_stream_t stream) {
+  return gpt_greedy_step(logits, ids, last_ids, vocab_size, max_step, cur_len, batch_size,
+                         unfinished, eos_id, HS(stream));
+}
+
 }  // extern "C"

@@ -1,0 +1,434 @@
+// Kernels of the int8 GPT path: embedding, prompt-pass QKV split, the launchers of
+// the reference's GPT kernel header (causal softmax over int32 scores, cache re-layout,
+// greedy sampling, perplexity) and the fixed-stride greedy step the model itself runs.
+//
+// The model keeps keys and values in caches of fixed stride [batch, head, max_step, d]
+// and token ids in [batch, max_step]: a generation step appends one column in place,
+// where the reference re-lays out (copies) every cache and the whole id matrix per step.
+#include "ls_device.cuh"
+#include "ls_launch.h"
+
+namespace lsh {
+
+constexpr float kLogitThreshMin = -64.f;  // inference/kernels/transformerKernels.h:11
+
+// ---------------------------------------------------------------------------------
+// embedding (inference/kernels/gptKernels_int8.cc.cu:21-106); token_emb [vocab, hidden]
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+gpt_embedding_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__ pos_emb,
+                     const int* __restrict__ token_id, T* __restrict__ output, int padding_id,
+                     int pos_offset, float dequant_scale, int seq_len, int hidden, int vocab) {
+#pragma clang fp contract(off)
+  const long pos = blockIdx.x;  // batch * seq_len + s
+  const int s = (int)(pos % seq_len);
+  int tid = token_id[pos];
+  if (tid == padding_id) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) TT<T>::st(output, pos * hidden + i, 0.f);
+    return;
+  }
+  if (vocab > 0) tid = min(max(tid, 0), vocab - 1);  // never index outside the table
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = (float)token_emb[(long)tid * hidden + i] * dequant_scale +
+                    TT<T>::ld(pos_emb, (long)(s + pos_offset) * hidden + i);
+    TT<T>::st(output, pos * hidden + i, v);
+  }
+}
+
+// real_seq_len[b] += non-padding tokens of row b (the reference counts with atomics)
+__global__ void __launch_bounds__(256)
+gpt_count_tokens_kernel(const int* __restrict__ token_id, int* real_seq_len, int padding_id,
+                        int seq_len) {
+  __shared__ float red[16];
+  const int b = blockIdx.x;
+  float n = 0.f;
+  for (int s = threadIdx.x; s < seq_len; s += blockDim.x)
+    n += token_id[(long)b * seq_len + s] != padding_id ? 1.f : 0.f;
+  n = block_sum(n, red);  // exact: seq_len is far below 2^24
+  if (threadIdx.x == 0) real_seq_len[b] += (int)n;
+}
+
+template <typename T>
+int gpt_embedding_i8I(int batch_size, int batch_seq_len, int hidden_size, hipStream_t s,
+                      const int8_t* token_emb, const T* pos_emb, const int* token_id, T* output,
+                      int* real_seq_len, int padding_id, int pos_offset, float dequant_scale,
+                      int vocab_size, int max_step) {
+  if (!token_emb || !pos_emb || !token_id || !output || !real_seq_len || batch_size <= 0 ||
+      batch_seq_len <= 0 || hidden_size <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "ker_gpt_embedding_i8I: bad arguments");
+  if (pos_offset < 0 || (max_step > 0 && pos_offset + batch_seq_len > max_step))
+    return lsh_fail(LSH_ERR_INVALID, "ker_gpt_embedding_i8I: position outside the table");
+  gpt_embedding_kernel<T><<<batch_size * batch_seq_len, 256, 0, s>>>(
+      token_emb, pos_emb, token_id, output, padding_id, pos_offset, dequant_scale, batch_seq_len,
+      hidden_size, vocab_size);
+  if (int rc = lsh_check_launch("gpt_embedding_kernel")) return rc;
+  gpt_count_tokens_kernel<<<batch_size, 256, 0, s>>>(token_id, real_seq_len, padding_id,
+                                                     batch_seq_len);
+  return lsh_check_launch("gpt_count_tokens_kernel");
+}
+template int gpt_embedding_i8I<float>(int, int, int, hipStream_t, const int8_t*, const float*,
+                                      const int*, float*, int*, int, int, float, int, int);
+template int gpt_embedding_i8I<__half>(int, int, int, hipStream_t, const int8_t*, const __half*,
+                                       const int*, __half*, int*, int, int, float, int, int);
+
+// ---------------------------------------------------------------------------------
+// prompt pass: int8 QKV GEMM output [tokens, 3H] + bias -> requantised with the cache
+// clip and written four ways in one pass:
+//   q, k as fp16 *code values* [B, h, S, d]   (operands of the MFMA score product)
+//   v dequantised to fp16      [B, h, S, d]   (code / quant_scale, the reference's d_v)
+//   k, v int8 codes into the caches [B, h, max_step, d]
+// Same arithmetic as ker_arrange_encself_qkv_i8I_i8O
+// (inference/kernels/transformerKernels_int8.cc.cu:1185-1299).
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+gpt_arrange_qkv_prefill_kernel(const int8_t* __restrict__ ori_qkv,
+                               const __half* __restrict__ qkv_bias, __half* __restrict__ q_codes,
+                               __half* __restrict__ k_codes, __half* __restrict__ v_deq,
+                               int8_t* __restrict__ k_cache, int8_t* __restrict__ v_cache,
+                               int seq_len, int head_num, int d, int max_step,
+                               float dequant_scale, float quant_scale) {
+#pragma clang fp contract(off)
+  const int H = head_num * d;
+  const long tok = blockIdx.x;
+  const int part = blockIdx.y;
+  const long b = tok / seq_len;
+  const int s = (int)(tok % seq_len);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float val = (float)ori_qkv[(tok * 3 + part) * H + i] * dequant_scale +
+                      __half2float(qkv_bias[(long)part * H + i]);
+    const int code = float2int8(val, quant_scale);
+    const int head = i / d, dim = i % d;
+    const long t = ((b * head_num + head) * seq_len + s) * d + dim;
+    const long c = ((b * head_num + head) * max_step + s) * d + dim;
+    if (part == 0) {
+      q_codes[t] = __float2half_rn((float)code);
+    } else if (part == 1) {
+      k_codes[t] = __float2half_rn((float)code);
+      k_cache[c] = (int8_t)code;
+    } else {
+      v_deq[t] = __float2half_rn((float)code / quant_scale);
+      v_cache[c] = (int8_t)code;
+    }
+  }
+}
+
+int gpt_arrange_qkv_prefill_f16(int batch_token_num, int hidden_size, hipStream_t s,
+                                const int8_t* ori_qkv, const __half* qkv_bias, __half* q_codes,
+                                __half* k_codes, __half* v_deq, int8_t* k_cache, int8_t* v_cache,
+                                int batch_seq_len, int dim_per_head, int head_num, int max_step,
+                                float dequant_scale, float quant_scale) {
+  if (!ori_qkv || !qkv_bias || !q_codes || !k_codes || !v_deq || !k_cache || !v_cache ||
+      batch_token_num <= 0 || batch_seq_len <= 0 || batch_token_num % batch_seq_len != 0 ||
+      hidden_size != dim_per_head * head_num || batch_seq_len > max_step)
+    return lsh_fail(LSH_ERR_INVALID, "gpt_arrange_qkv_prefill: bad arguments");
+  gpt_arrange_qkv_prefill_kernel<<<dim3(batch_token_num, 3), 256, 0, s>>>(
+      ori_qkv, qkv_bias, q_codes, k_codes, v_deq, k_cache, v_cache, batch_seq_len, head_num,
+      dim_per_head, max_step, dequant_scale, quant_scale);
+  return lsh_check_launch("gpt_arrange_qkv_prefill_kernel");
+}
+
+// ---------------------------------------------------------------------------------
+// causal softmax over int32 scores (inference/kernels/gptKernels_int8.cc.cu:192-250);
+// one wavefront per (batch, head, query) row.  Rows of padded queries are written as
+// zeros (the reference leaves them untouched).
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+softmax_gpt_i32I_kernel(const int32_t* __restrict__ corr, T* __restrict__ out,
+                        const int* __restrict__ real_seq_len, long rows, int seq_len, int head_num,
+                        float attn_scale, float dq) {
+#pragma clang fp contract(off)
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int b = (int)(row / ((long)head_num * seq_len));
+  const int qpos = (int)(row % seq_len);
+  const int32_t* c = corr + row * seq_len;
+  T* o = out + row * seq_len;
+  if (qpos >= real_seq_len[b]) {
+    for (int j = lane; j < seq_len; j += 64) TT<T>::st(o, j, 0.f);
+    return;
+  }
+  float mx = kFloatInfNeg;
+  for (int j = lane; j <= qpos; j += 64) mx = fmaxf(mx, (float)c[j] * attn_scale * dq * dq);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int j = lane; j <= qpos; j += 64) sum += __expf((float)c[j] * attn_scale * dq * dq - mx);
+  sum = wave_sum(sum);
+  for (int j = lane; j < seq_len; j += 64) {
+    const float e = j <= qpos ? __expf((float)c[j] * attn_scale * dq * dq - mx) : 0.f;
+    TT<T>::st(o, j, e / sum);
+  }
+}
+
+template <typename T>
+int correlation_softmax_gpt_i32I(int batch_size, int batch_seq_len, int head_num, hipStream_t s,
+                                 const int32_t* correlation, T* output, const int* real_seq_len,
+                                 float attn_scale, float dequant_scale) {
+  if (!correlation || !output || !real_seq_len || batch_size <= 0 || batch_seq_len <= 0 ||
+      head_num <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "ker_correlation_softmax_gpt_i32I: bad arguments");
+  const long rows = (long)batch_size * head_num * batch_seq_len;
+  softmax_gpt_i32I_kernel<T><<<(int)((rows + 3) / 4), 256, 0, s>>>(
+      correlation, output, real_seq_len, rows, batch_seq_len, head_num, attn_scale,
+      dequant_scale);
+  return lsh_check_launch("softmax_gpt_i32I_kernel");
+}
+template int correlation_softmax_gpt_i32I<float>(int, int, int, hipStream_t, const int32_t*,
+                                                 float*, const int*, float, float);
+template int correlation_softmax_gpt_i32I<__half>(int, int, int, hipStream_t, const int32_t*,
+                                                  __half*, const int*, float, float);
+
+// batched int8 q.K^T of the prompt pass (inference/model/quant_gpt_encoder.cc.cu:498-505)
+// for callers of the unfused launchers: scores[bh, i, j] = sum_d q[bh,i,d] * k[bh,j,d]
+__global__ void __launch_bounds__(256)
+gpt_scores_i8_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k,
+                     int32_t* __restrict__ scores, long rows, int seq_len, int d) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const long bh = row / seq_len;
+  const int8_t* qp = q + row * d;
+  for (int j = lane; j < seq_len; j += 64) {
+    const int8_t* kp = k + (bh * seq_len + j) * d;
+    int acc = 0;
+    for (int t = 0; t < d; ++t) acc += (int)qp[t] * (int)kp[t];
+    scores[row * seq_len + j] = acc;
+  }
+}
+
+int gpt_scores_i8(const int8_t* q, const int8_t* k, int32_t* scores, int batch_head_num,
+                  int batch_seq_len, int dim_per_head, hipStream_t s) {
+  if (!q || !k || !scores || batch_head_num <= 0 || batch_seq_len <= 0 || dim_per_head <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "gpt_scores_i8: bad arguments");
+  const long rows = (long)batch_head_num * batch_seq_len;
+  gpt_scores_i8_kernel<<<(int)((rows + 3) / 4), 256, 0, s>>>(q, k, scores, rows, batch_seq_len,
+                                                             dim_per_head);
+  return lsh_check_launch("gpt_scores_i8_kernel");
+}
+
+// ---------------------------------------------------------------------------------
+// ker_arrange_qkv_with_cache_i8I_i8O (inference/kernels/gptKernels_int8.cc.cu:658-812):
+// one new token per sequence; caches re-laid out from [B, h, S-1, d] to [B, h, S, d]
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+arrange_qkv_with_cache_kernel(const int8_t* __restrict__ ori_qkv, const T* __restrict__ qkv_bias,
+                              int8_t* __restrict__ new_q, int8_t* __restrict__ new_k,
+                              const int8_t* __restrict__ k_cache, int8_t* __restrict__ new_v,
+                              const int8_t* __restrict__ v_cache, int seq_len, int d, int head_num,
+                              float dequant_scale, float quant_scale) {
+#pragma clang fp contract(off)
+  const int H = head_num * d;
+  const long b = blockIdx.x / seq_len;
+  const int t = blockIdx.x % seq_len;
+  const int part = blockIdx.y;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const int head = i / d, dim = i % d;
+    const long target = ((b * head_num + head) * seq_len + t) * d + dim;
+    if (t < seq_len - 1) {
+      if (part == 0) return;
+      const long old = ((b * head_num + head) * (seq_len - 1) + t) * d + dim;
+      if (part == 1) new_k[target] = k_cache[old];
+      else new_v[target] = v_cache[old];
+    } else {
+      const float val = (float)ori_qkv[(b * 3 + part) * H + i] * dequant_scale +
+                        TT<T>::ld(qkv_bias, (long)part * H + i);
+      const int8_t qv = (int8_t)float2int8(val, quant_scale);
+      if (part == 0) new_q[(b * head_num + head) * d + dim] = qv;
+      else if (part == 1) new_k[target] = qv;
+      else new_v[target] = qv;
+    }
+  }
+}
+
+template <typename T>
+int arrange_qkv_with_cache_i8I_i8O(int batch_token_num, int hidden_size, hipStream_t s,
+                                   const int8_t* ori_qkv, const T* qkv_bias, int8_t* new_q,
+                                   int8_t* new_k, const int8_t* k_cache, int8_t* new_v,
+                                   const int8_t* v_cache, int batch_seq_len, int dim_per_head,
+                                   int head_num, float dequant_scale, float quant_scale) {
+  if (!ori_qkv || !qkv_bias || !new_q || !new_k || !new_v || batch_token_num <= 0 ||
+      batch_seq_len <= 0 || batch_token_num % batch_seq_len != 0 ||
+      hidden_size != dim_per_head * head_num || (batch_seq_len > 1 && (!k_cache || !v_cache)))
+    return lsh_fail(LSH_ERR_INVALID, "ker_arrange_qkv_with_cache_i8I_i8O: bad arguments");
+  if (new_k == k_cache || new_v == v_cache)
+    return lsh_fail(LSH_ERR_INVALID,
+                    "ker_arrange_qkv_with_cache_i8I_i8O: old and new cache must differ");
+  arrange_qkv_with_cache_kernel<T><<<dim3(batch_token_num, 3), 256, 0, s>>>(
+      ori_qkv, qkv_bias, new_q, new_k, k_cache, new_v, v_cache, batch_seq_len, dim_per_head,
+      head_num, dequant_scale, quant_scale);
+  return lsh_check_launch("arrange_qkv_with_cache_kernel");
+}
+template int arrange_qkv_with_cache_i8I_i8O<float>(int, int, hipStream_t, const int8_t*,
+                                                   const float*, int8_t*, int8_t*, const int8_t*,
+                                                   int8_t*, const int8_t*, int, int, int, float,
+                                                   float);
+template int arrange_qkv_with_cache_i8I_i8O<__half>(int, int, hipStream_t, const int8_t*,
+                                                    const __half*, int8_t*, int8_t*,
+                                                    const int8_t*, int8_t*, const int8_t*, int, int,
+                                                    int, float, float);
+
+// ---------------------------------------------------------------------------------
+// greedy sampling.  The dequantisation code * scale (scale > 0) is monotone, so the
+// arg-max runs on the int8 codes; ties go to the lowest token id (the reference lets
+// racing stores decide).
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ int block_argmax_i8(const int8_t* __restrict__ lr, int vocab,
+                                               int* red /*[32]*/) {
+  int best_c = -129, best_i = 0x7fffffff;
+  for (int v = threadIdx.x; v < vocab; v += blockDim.x) {
+    const int c = lr[v];
+    if (c > best_c) {  // ascending v per thread: the first maximum is kept
+      best_c = c;
+      best_i = v;
+    }
+  }
+#pragma unroll
+  for (int m = 32; m > 0; m >>= 1) {
+    const int oc = __shfl_xor(best_c, m, 64), oi = __shfl_xor(best_i, m, 64);
+    if (oc > best_c || (oc == best_c && oi < best_i)) {
+      best_c = oc;
+      best_i = oi;
+    }
+  }
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if (lane == 0) {
+    red[wid] = best_c;
+    red[16 + wid] = best_i;
+  }
+  __syncthreads();
+  best_c = red[0];
+  best_i = red[16];
+  for (int w2 = 1; w2 < nw; ++w2)
+    if (red[w2] > best_c || (red[w2] == best_c && red[16 + w2] < best_i)) {
+      best_c = red[w2];
+      best_i = red[16 + w2];
+    }
+  return best_i;
+}
+
+// ker_topk_sample_i8I<1> (inference/kernels/gptKernels_int8.cc.cu:252-463): ids re-laid
+// out from [batch, seq_len] to [batch, seq_len + 1], sampled ids also behind the old array
+__global__ void __launch_bounds__(1024)
+topk_sample_greedy_kernel(const int8_t* __restrict__ logits, int* old_input_ids,
+                          int* __restrict__ new_input_ids, int vocab, int seq_len,
+                          int logits_seq_len, int* unfinished, int eos_id) {
+  __shared__ int red[32];
+  const int b = blockIdx.x;
+  const bool ended = old_input_ids[(long)b * seq_len + seq_len - 1] == eos_id;
+  for (int t = threadIdx.x; t < seq_len; t += blockDim.x)
+    new_input_ids[(long)b * (seq_len + 1) + t] = old_input_ids[(long)b * seq_len + t];
+  int tok = eos_id;
+  if (!ended) {
+    const int8_t* lr = logits + ((long)b * logits_seq_len + logits_seq_len - 1) * vocab;
+    tok = block_argmax_i8(lr, vocab, red);
+  }
+  if (threadIdx.x == 0) {
+    if (!ended && tok != eos_id) unfinished[0] = 1;  // every writer stores the same value
+    new_input_ids[(long)b * (seq_len + 1) + seq_len] = tok;
+  }
+}
+
+// second pass: sampled ids behind the old array, after every block has read its old row
+__global__ void topk_sample_tail_kernel(int* old_input_ids, const int* __restrict__ new_input_ids,
+                                        int batch, int seq_len) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b < batch)
+    old_input_ids[(long)batch * seq_len + b] = new_input_ids[(long)b * (seq_len + 1) + seq_len];
+}
+
+int topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len, hipStream_t s,
+                    const int8_t* logits, int* old_input_ids, int* new_input_ids,
+                    int vocab_size, int k, int* unfinished, int eos_id) {
+  if (!logits || !old_input_ids || !new_input_ids || !unfinished || batch_size <= 0 ||
+      batch_seq_len <= 0 || logits_seq_len <= 0 || vocab_size <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "ker_topk_sample_i8I: bad arguments");
+  if (k != 1) {
+    if (k == 2 || k == 4 || k == 8 || k == 16 || k == 32)
+      return lsh_fail(LSH_ERR_UNSUPPORTED,
+                      "ker_topk_sample_i8I: only topk = 1 (greedy) is provided; random sampling "
+                      "needs the reference's generator state");
+    return lsh_fail(LSH_ERR_INVALID, "topk argument should be in [1,2,4,8,16,32]");
+  }
+  topk_sample_greedy_kernel<<<batch_size, 1024, 0, s>>>(logits, old_input_ids, new_input_ids,
+                                                        vocab_size, batch_seq_len, logits_seq_len,
+                                                        unfinished, eos_id);
+  if (int rc = lsh_check_launch("topk_sample_greedy_kernel")) return rc;
+  topk_sample_tail_kernel<<<(batch_size + 255) / 256, 256, 0, s>>>(old_input_ids, new_input_ids,
+                                                                   batch_size, batch_seq_len);
+  return lsh_check_launch("topk_sample_tail_kernel");
+}
+
+// the model's step: ids [batch, max_step] in place, logits [batch, vocab] of the last
+// position; writes column cur_len, the step's input ids and the unfinished flag
+__global__ void __launch_bounds__(1024)
+gpt_greedy_step_kernel(const int8_t* __restrict__ logits, int* ids, int* __restrict__ last_ids,
+                       int vocab, int max_step, int cur_len, int* unfinished, int eos_id) {
+  __shared__ int red[32];
+  const int b = blockIdx.x;
+  const bool ended = ids[(long)b * max_step + cur_len - 1] == eos_id;
+  int tok = eos_id;
+  if (!ended) tok = block_argmax_i8(logits + (long)b * vocab, vocab, red);
+  if (threadIdx.x == 0) {
+    if (!ended && tok != eos_id) unfinished[0] = 1;
+    ids[(long)b * max_step + cur_len] = tok;
+    last_ids[b] = tok;
+  }
+}
+
+int gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size, int max_step,
+                    int cur_len, int batch_size, int* unfinished, int eos_id, hipStream_t s) {
+  if (!logits || !ids || !last_ids || !unfinished || batch_size <= 0 || vocab_size <= 0 ||
+      cur_len <= 0 || cur_len >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "gpt_greedy_step: bad arguments");
+  gpt_greedy_step_kernel<<<batch_size, 1024, 0, s>>>(logits, ids, last_ids, vocab_size, max_step,
+                                                     cur_len, unfinished, eos_id);
+  return lsh_check_launch("gpt_greedy_step_kernel");
+}
+
+// ---------------------------------------------------------------------------------
+// perplexity (inference/kernels/gptKernels_int8.cc.cu:108-190).  One block per sequence
+// walks its positions in order, so the sum has a fixed order (the reference adds the
+// per-position terms with float atomics).
+// ---------------------------------------------------------------------------------
+__global__ void __launch_bounds__(1024)
+ppl_kernel(const int8_t* __restrict__ logits, const int* __restrict__ input_ids,
+           const int* __restrict__ real_seq_len, float* ppl, int vocab, int seq_len, float dq) {
+#pragma clang fp contract(off)
+  __shared__ float red[16];
+  const int b = blockIdx.x;
+  const int len = real_seq_len[b];
+  float total = 0.f;
+  for (int s = 0; s < seq_len && s < len - 1; ++s) {
+    const long tok = (long)b * seq_len + s;
+    const int8_t* lr = logits + tok * vocab;
+    float mx = kFloatInfNeg;
+    for (int v = threadIdx.x; v < vocab; v += blockDim.x) mx = fmaxf(mx, (float)lr[v] * dq);
+    mx = block_max(mx, red);
+    float se = 0.f;
+    for (int v = threadIdx.x; v < vocab; v += blockDim.x)
+      se += __expf(fmaxf((float)lr[v] * dq - mx, kLogitThreshMin));
+    se = block_sum(se, red);
+    int target = input_ids[tok + 1];
+    target = min(max(target, 0), vocab - 1);
+    const float log_prob = ((float)lr[target] * dq - mx - logf(se)) / (float)(len - 1);
+    total += -log_prob;
+  }
+  if (threadIdx.x == 0) ppl[b] += total;
+}
+
+int ppl_i8I(int batch_size, int batch_seq_len, hipStream_t s, const int8_t* logits,
+            const int* input_ids, const int* real_seq_len, float* ppl, int vocab_size,
+            float dequant_scale) {
+  if (!logits || !input_ids || !real_seq_len || !ppl || batch_size <= 0 || batch_seq_len <= 0 ||
+      vocab_size <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "ker_ppl_i8I: bad arguments");
+  ppl_kernel<<<batch_size, 1024, 0, s>>>(logits, input_ids, real_seq_len, ppl, vocab_size,
+                                         batch_seq_len, dequant_scale);
+  return lsh_check_launch("ppl_kernel");
+}
+
+}  // namespace lsh

@@ -196,6 +196,43 @@ int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_p
                          float* top_score, int* top_idx, int* parent, int* num_finished,
                          float dequant_scale, int vocab_size, int max_step, float length_norm,
                          int cur_step, int batch_size, int beam_size, int end_id, hipStream_t s);
+// ---- GPT path (gpt_kernels.hip, attn_kernels.hip) ------------------------------------------
+// vocab_size <= 0 disables the token-id clamp, max_step <= 0 the position check
+template <typename T>
+int gpt_embedding_i8I(int batch_size, int batch_seq_len, int hidden_size, hipStream_t s,
+                      const int8_t* token_emb, const T* pos_emb, const int* token_id, T* output,
+                      int* real_seq_len, int padding_id, int pos_offset, float dequant_scale,
+                      int vocab_size, int max_step);
+int gpt_arrange_qkv_prefill_f16(int batch_token_num, int hidden_size, hipStream_t s,
+                                const int8_t* ori_qkv, const __half* qkv_bias, __half* q_codes,
+                                __half* k_codes, __half* v_deq, int8_t* k_cache, int8_t* v_cache,
+                                int batch_seq_len, int dim_per_head, int head_num, int max_step,
+                                float dequant_scale, float quant_scale);
+int gpt_prefill_attention_f16(const __half* q_codes, const __half* k_codes, const __half* v,
+                              const int* real_seq_len, __half* ctx, int8_t* ctx_q,
+                              float quant_scale, float dequant_scale, int batch, int seq_len,
+                              int head_num, int dim_per_head, hipStream_t s);
+template <typename T>
+int correlation_softmax_gpt_i32I(int batch_size, int batch_seq_len, int head_num, hipStream_t s,
+                                 const int32_t* correlation, T* output, const int* real_seq_len,
+                                 float attn_scale, float dequant_scale);
+int gpt_scores_i8(const int8_t* q, const int8_t* k, int32_t* scores, int batch_head_num,
+                  int batch_seq_len, int dim_per_head, hipStream_t s);
+template <typename T>
+int arrange_qkv_with_cache_i8I_i8O(int batch_token_num, int hidden_size, hipStream_t s,
+                                   const int8_t* ori_qkv, const T* qkv_bias, int8_t* new_q,
+                                   int8_t* new_k, const int8_t* k_cache, int8_t* new_v,
+                                   const int8_t* v_cache, int batch_seq_len, int dim_per_head,
+                                   int head_num, float dequant_scale, float quant_scale);
+int topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len, hipStream_t s,
+                    const int8_t* logits, int* old_input_ids, int* new_input_ids,
+                    int vocab_size, int k, int* unfinished, int eos_id);
+int gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size, int max_step,
+                    int cur_len, int batch_size, int* unfinished, int eos_id, hipStream_t s);
+int ppl_i8I(int batch_size, int batch_seq_len, hipStream_t s, const int8_t* logits,
+            const int* input_ids, const int* real_seq_len, float* ppl, int vocab_size,
+            float dequant_scale);
+
 // inference/kernels/transformerKernels.h:137-140
 inline float length_norm(int length, float alpha) {
   if (alpha < 0.f) return 1.f / length;

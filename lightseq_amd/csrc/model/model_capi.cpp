@@ -7,12 +7,14 @@
 #include "../ls_launch.h"
 #include "ls_model.h"
 #include "quant_bert.h"
+#include "quant_gpt.h"
 #include "quant_transformer.h"
 
 using lightseq::hip::LSModel;
 using lightseq::hip::LSModelFactory;
 using lightseq::hip::QuantBert;
 using lightseq::hip::QuantBertEncoder;
+using lightseq::hip::QuantGpt;
 using lightseq::hip::QuantTransformer;
 
 struct ls_model {
@@ -239,18 +241,30 @@ int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst) {
 
 int ls_model_set_step_record(ls_model* model, int8_t* logits, int* alive_seq, int max_steps) {
   NEED_MODEL(model);
-  QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get());
-  if (!qt) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "step records are a QuantTransformer debug aid");
   if (max_steps < 0) return lsh::lsh_fail(LSH_ERR_INVALID, "negative max_steps");
+  if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get())) {
+    qg->encoder()->set_step_record(logits, max_steps);
+    return LSH_OK;
+  }
+  QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get());
+  if (!qt)
+    return lsh::lsh_fail(LSH_ERR_UNSUPPORTED,
+                         "step records are a debug aid of QuantTransformer and QuantGpt");
   qt->decoder()->set_step_record(logits, alive_seq, max_steps);
   return LSH_OK;
 }
 
 int ls_model_get_steps_run(ls_model* model, int* steps) {
   NEED_MODEL(model);
-  QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get());
-  if (!qt) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "step records are a QuantTransformer debug aid");
   if (!steps) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");
+  if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get())) {
+    *steps = qg->encoder()->steps_run();
+    return LSH_OK;
+  }
+  QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get());
+  if (!qt)
+    return lsh::lsh_fail(LSH_ERR_UNSUPPORTED,
+                         "step records are a debug aid of QuantTransformer and QuantGpt");
   *steps = qt->decoder()->steps_run();
   return LSH_OK;
 }

@@ -1,0 +1,95 @@
+#include "quant_gpt.h"
+
+namespace lightseq {
+namespace hip {
+
+QuantGpt::QuantGpt(const std::string weight_path, const int max_batch_size)
+    : LSModel({"token_ids"}, {"result"}), _max_batch_size(max_batch_size) {
+  if (max_batch_size <= 0) throw std::runtime_error("max_batch_size must be positive");
+  CHECK_GPU_ERROR(hipSetDevice(0));
+  CHECK_GPU_ERROR(hipStreamCreate(&stream_));
+
+  std::string res = tw_.initializing(weight_path);
+  if (!res.empty()) throw std::runtime_error(res);
+
+  const size_t tokens = (size_t)_max_batch_size * tw_._max_step;
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_input_), tokens * sizeof(int)));
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_sample_id), tokens * sizeof(int)));
+  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_ppl), _max_batch_size * sizeof(float)));
+
+  encoder_ = std::make_shared<QuantGptEncoder>(max_batch_size, d_input_, d_ppl, d_sample_id, tw_,
+                                               stream_);
+  res = encoder_->check();
+  if (!res.empty()) throw std::runtime_error(res);
+  encoder_->init_buffer();
+  CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+}
+
+QuantGpt::~QuantGpt() {
+  encoder_.reset();
+  if (d_input_) (void)hipFree(d_input_);
+  if (d_sample_id) (void)hipFree(d_sample_id);
+  if (d_ppl) (void)hipFree(d_ppl);
+  if (stream_) (void)hipStreamDestroy(stream_);
+}
+
+void QuantGpt::Infer() {
+  if (input_shapes_[0].size() != 2) throw std::runtime_error("token_ids must be 2-D");
+  int batch_size = input_shapes_[0][0], seq_len = input_shapes_[0][1];
+  if (is_ppl()) {
+    encoder_->run_one_infer(batch_size, seq_len);
+    CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+    set_output_shape(0, {batch_size});
+  } else if (tw_._sampling_method == "topk" || tw_._sampling_method == "topp") {
+    int sampled_seq_len = encoder_->run_one_sample(batch_size, seq_len);
+    CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+    set_output_shape(0, {batch_size, sampled_seq_len});
+  } else {
+    throw std::runtime_error("Unsupported sampling_method");
+  }
+}
+
+void QuantGpt::set_input_ptr(int index, void* input_ptr) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  encoder_->_p_d_token_id = static_cast<int*>(input_ptr);
+}
+
+void QuantGpt::set_output_ptr(int index, void* output_ptr) {
+  if (index != 0) throw std::runtime_error("invalid output index");
+  if (is_ppl())
+    encoder_->_p_d_ppl = static_cast<float*>(output_ptr);
+  else
+    encoder_->_p_d_sample_id = static_cast<int*>(output_ptr);
+}
+
+const void* QuantGpt::get_output_ptr(int index) {
+  if (index != 0) throw std::runtime_error("invalid output index");
+  if (is_ppl()) return static_cast<void*>(encoder_->_p_d_ppl);
+  return static_cast<void*>(encoder_->_p_d_sample_id);
+}
+
+std::vector<int> QuantGpt::get_input_max_shape(int index) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  return {_max_batch_size, tw_._max_step};
+}
+
+std::vector<int> QuantGpt::get_output_max_shape(int index) {
+  if (index != 0) throw std::runtime_error("invalid output index");
+  if (is_ppl()) return {_max_batch_size};
+  return {_max_batch_size, tw_._max_step};
+}
+
+DataType QuantGpt::get_input_dtype(int index) {
+  if (index != 0) throw std::runtime_error("invalid input index");
+  return DataType::kInt32;
+}
+
+DataType QuantGpt::get_output_dtype(int index) {
+  if (index != 0) throw std::runtime_error("invalid output index");
+  return is_ppl() ? DataType::kFloat32 : DataType::kInt32;
+}
+
+LSMODEL_REGISTER(QuantGpt)
+
+}  // namespace hip
+}  // namespace lightseq

@@ -1,0 +1,296 @@
+#include "quant_gpt_encoder.h"
+
+#include "../ls_device.cuh"
+
+#include <algorithm>
+
+namespace lightseq {
+namespace hip {
+
+using namespace lsh;
+
+QuantGptEncoder::QuantGptEncoder(int max_batch_size, const int* p_d_token_id, float* p_d_ppl,
+                                 int* p_d_sample_id, const QuantGptWeight& tw, hipStream_t stream)
+    : _p_d_token_id(p_d_token_id),
+      _p_d_ppl(p_d_ppl),
+      _p_d_sample_id(p_d_sample_id),
+      _max_batch_size(max_batch_size),
+      _tw(tw),
+      _stream(stream),
+      _src_emb_clip_max(tw._src_emb_clip_max),
+      _output_ln_clip_max(tw._output_ln_clip_max),
+      _logits_clip_max(tw._logits_clip_max),
+      _enc_clip_max(tw._enc_clip_max),
+      _atten_scaler(__half2float(__float2half_rn(sqrtf(1.f / (float)std::max(tw._dim_per_head, 1))))),
+      _max_batch_dim((long)max_batch_size * tw._max_step * tw._hidden_size) {}
+
+QuantGptEncoder::~QuantGptEncoder() {
+  if (_h_unfinished) (void)hipHostFree(_h_unfinished);
+}
+
+std::string QuantGptEncoder::check() {
+  if (_tw._inner_size & 1) return "violate inner_size % 2 = 0";
+  if (_tw._dim_per_head & 1) return "violate dim_per_head % 2 = 0";
+  if ((int)_tw.layers.size() != _tw._n_enc_layer)
+    return "violate p_d_enc_wei.size() = weight_per_enc_layer * n_enc_layer";
+  if ((int)_enc_clip_max.size() != 12 * _tw._n_enc_layer) return "wrong clip_max table size";
+  const std::string& m = _tw._sampling_method;
+  if (m != "topk" && m != "topp" && m != "ppl")
+    return std::string("unsupported sampling_method: ") + m;
+  if (_tw._topk <= 0) return "topk must be positive";
+  if (m == "topp" || (m == "topk" && _tw._topk != 1))
+    return "random sampling (topp, topk > 1) is not available in this build: use topk = 1 or ppl";
+  if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)
+    return "violate hidden_size % 16 = 0 and inner_size % 16 = 0 (int8 MFMA GEMM)";
+  if (_tw._dim_per_head != 32 && _tw._dim_per_head != 64 && _tw._dim_per_head != 128)
+    return "violate dim_per_head in {32, 64, 128} (fused attention kernel)";
+  if (_tw._max_step > 4096) return "violate max_step <= 4096";
+  if (_tw._eos_id < 0 || _tw._eos_id >= _tw._src_vocab_size)
+    return "eos_id outside the vocabulary";
+  return "";
+}
+
+void QuantGptEncoder::init_buffer() {
+  const int H = _tw._hidden_size, I = _tw._inner_size, L = _tw._n_enc_layer;
+  const int V = _tw._src_vocab_size;
+  const size_t tokens = (size_t)_max_batch_size * _tw._max_step;
+  _real_seq_len.alloc(_max_batch_size);
+  _ids.alloc(tokens);
+  _last_ids.alloc(_max_batch_size);
+  _unfinished.alloc(1);
+  CHECK_GPU_ERROR(hipHostMalloc(reinterpret_cast<void**>(&_h_unfinished), sizeof(int)));
+  *_h_unfinished = 0;
+  _query.alloc((size_t)_max_batch_dim);
+  _qkv_buf.alloc((size_t)(3 * _max_batch_dim));
+  const size_t wide = tokens * (size_t)std::max(I, 3 * H);
+  _buf_a.alloc(wide);
+  _buf_b.alloc(wide);
+  _hid_last.alloc((size_t)_max_batch_size * H);
+  // perplexity needs the logits of every position, sampling only of the last one
+  _logits.alloc((_tw._sampling_method == "ppl" ? tokens : (size_t)_max_batch_size) * V);
+  _int32_ffn_out_buf.alloc(tokens * H);
+  _self_k_cache.alloc((size_t)L * _max_batch_dim);
+  _self_v_cache.alloc((size_t)L * _max_batch_dim);
+  CHECK_GPU_ERROR(hipMemsetAsync(_self_k_cache.get(), 0, _self_k_cache.size(), _stream));
+  CHECK_GPU_ERROR(hipMemsetAsync(_self_v_cache.get(), 0, _self_v_cache.size(), _stream));
+
+  // stored [H, vocab]; one [vocab, H] copy serves the row lookup and the logits GEMM
+  _int8_emb = upload_kernel(_tw.token_embedding, H, V, true, _stream);
+  _pos_emb = upload_half(_tw.position_embedding, _stream);
+  _out_ln_scale = upload_half(_tw.norm_scale, _stream);
+  _out_ln_bias = upload_half(_tw.norm_bias, _stream);
+  _layers.clear();
+  _layers.resize(L);
+  for (int l = 0; l < L; ++l) {
+    const QuantBertLayerWeight& w = _tw.layers[l];
+    Layer& d = _layers[l];
+    d.ln1_scale = upload_half(w.multihead_norm_scale, _stream);
+    d.ln1_bias = upload_half(w.multihead_norm_bias, _stream);
+    d.b_qkv = upload_half(w.multihead_project_bias_qkv, _stream);
+    d.b_out = upload_half(w.multihead_project_bias_output, _stream);
+    d.ln2_scale = upload_half(w.ffn_norm_scale, _stream);
+    d.ln2_bias = upload_half(w.ffn_norm_bias, _stream);
+    d.b_ffn1 = upload_half(w.ffn_first_bias, _stream);
+    d.b_ffn2 = upload_half(w.ffn_second_bias, _stream);
+    d.w_qkv = upload_kernel(w.multihead_project_kernel_qkv, H, 3 * H, true, _stream);
+    d.w_out = upload_kernel(w.multihead_project_kernel_output, H, H, true, _stream);
+    d.w_ffn1 = upload_kernel(w.ffn_first_kernel, H, I, true, _stream);
+    d.w_ffn2 = upload_kernel(w.ffn_second_kernel, I, H, true, _stream);
+  }
+  CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+}
+
+// FFN block and the LayerNorm that follows it (:646-776).  `in` holds the int8
+// LayerNorm output and receives the next one; `tmp` is scratch of the same size.
+void QuantGptEncoder::ffn_add_norm(int rows, int8_t* in, int8_t* tmp) {
+  const int H = _tw._hidden_size, I = _tw._inner_size;
+  const Layer& w = _layers[_layer_id];
+  const float* c = &_enc_clip_max[_layer_id * 12];
+  const float Q = _quant_range;
+  LSH_CALL(gemm_i8_bias_act_i8o(in, w.w_ffn1.get(), tmp, w.b_ffn1.get(), rows, I, H,
+                                c[2] * c[6] / (c[10] * Q), c[10] / Q, Q / c[7], c[7], kActGelu,
+                                _stream));
+  LSH_CALL(gemm_i8_i32o(tmp, w.w_ffn2.get(), _int32_ffn_out_buf.get(), rows, H, I, _stream));
+  const float dequant_scale = c[3] * c[7] / (Q * Q);
+  const __half *scale_ptr, *bias_ptr, *res_bias_ptr;
+  float clip_max;
+  if (_layer_id == _tw._n_enc_layer - 1) {
+    scale_ptr = _out_ln_scale.get();
+    bias_ptr = _out_ln_bias.get();
+    res_bias_ptr = nullptr;
+    clip_max = _output_ln_clip_max;
+  } else {
+    const Layer& nx = _layers[_layer_id + 1];
+    scale_ptr = nx.ln1_scale.get();
+    bias_ptr = nx.ln1_bias.get();
+    res_bias_ptr = nx.b_out.get();
+    clip_max = _enc_clip_max[(_layer_id + 1) * 12 + 4];
+  }
+  LSH_CALL((residual_bias_ln_i8O<__half, int32_t>(
+      _int32_ffn_out_buf.get(), scale_ptr, bias_ptr, res_bias_ptr, in, _query.get(), rows, H,
+      dequant_scale, Q / clip_max, _stream, false, nullptr)));
+}
+
+// all prompt positions at once (:253-291 / :299-341); leaves the int8 LayerNorm output of
+// the last layer in _buf_a
+void QuantGptEncoder::prompt_pass(const int* ids) {
+  const int H = _tw._hidden_size, M = _batch_token_num;
+  const float Q = _quant_range;
+  CHECK_GPU_ERROR(hipMemsetAsync(_real_seq_len.get(), 0, sizeof(int) * _batch_size, _stream));
+  LSH_CALL(gpt_embedding_i8I<__half>(_batch_size, _batch_seq_len, H, _stream, _int8_emb.get(),
+                                     _pos_emb.get(), ids, _query.get(), _real_seq_len.get(),
+                                     _tw._padding_id, 0, _src_emb_clip_max / Q,
+                                     _tw._src_vocab_size, _tw._max_step));
+  int8_t *a = _buf_a.get(), *b = _buf_b.get();
+  __half* qc = _qkv_buf.get();
+  __half* kc = qc + _max_batch_dim;
+  __half* vd = kc + _max_batch_dim;
+  for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
+    const Layer& w = _layers[_layer_id];
+    const float* c = &_enc_clip_max[_layer_id * 12];
+    if (_layer_id == 0)
+      LSH_CALL(norm_layer_resual_i8O<__half>(M, H, _stream, _query.get(), a, w.ln1_scale.get(),
+                                             w.ln1_bias.get(), w.b_out.get(), Q / c[4], false));
+    LSH_CALL(gemm_i8_i8o(a, w.w_qkv.get(), b, M, 3 * H, H, c[0] * c[4] / (c[8] * Q), _stream));
+    LSH_CALL(gpt_arrange_qkv_prefill_f16(
+        M, H, _stream, b, w.b_qkv.get(), qc, kc, vd,
+        _self_k_cache.get() + (size_t)_layer_id * _max_batch_dim,
+        _self_v_cache.get() + (size_t)_layer_id * _max_batch_dim, _batch_seq_len,
+        _tw._dim_per_head, _tw._head_num, _tw._max_step, c[8] / Q, Q / c[11]));
+    LSH_CALL(gpt_prefill_attention_f16(qc, kc, vd, _real_seq_len.get(), nullptr, a, Q / c[5],
+                                       c[11] / Q, _batch_size, _batch_seq_len, _tw._head_num,
+                                       _tw._dim_per_head, _stream));
+    LSH_CALL(gemm_i8_i8o(a, w.w_out.get(), b, M, H, H, c[1] * c[5] / (c[9] * Q), _stream));
+    LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(b, w.ln2_scale.get(), w.ln2_bias.get(),
+                                                   w.b_ffn2.get(), a, _query.get(), M, H,
+                                                   c[9] / Q, Q / c[6], _stream, false, nullptr)));
+    ffn_add_norm(M, a, b);
+  }
+}
+
+// one cached step for the tokens in _last_ids at position _batch_seq_len - 1 (:363-377)
+void QuantGptEncoder::step_pass() {
+  const int H = _tw._hidden_size, B = _batch_size;
+  const float Q = _quant_range;
+  LSH_CALL(gpt_embedding_i8I<__half>(B, 1, H, _stream, _int8_emb.get(), _pos_emb.get(),
+                                     _last_ids.get(), _query.get(), _real_seq_len.get(),
+                                     _tw._padding_id, _batch_seq_len - 1, _src_emb_clip_max / Q,
+                                     _tw._src_vocab_size, _tw._max_step));
+  int8_t *a = _buf_a.get(), *b = _buf_b.get();
+  for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
+    const Layer& w = _layers[_layer_id];
+    const float* c = &_enc_clip_max[_layer_id * 12];
+    int8_t* k_cache = _self_k_cache.get() + (size_t)_layer_id * _max_batch_dim;
+    int8_t* v_cache = _self_v_cache.get() + (size_t)_layer_id * _max_batch_dim;
+    if (_layer_id == 0)
+      LSH_CALL(norm_layer_resual_i8O<__half>(B, H, _stream, _query.get(), a, w.ln1_scale.get(),
+                                             w.ln1_bias.get(), w.b_out.get(), Q / c[4], false));
+    LSH_CALL(gemm_i8_i8o(a, w.w_qkv.get(), b, B, 3 * H, H, c[0] * c[4] / (c[8] * Q), _stream));
+    // q -> a, k / v appended to the caches at the token's position
+    LSH_CALL(arrange_decself_qkv_i8I_i8O<__half>(B, H, _stream, b, w.b_qkv.get(), a, k_cache,
+                                                 v_cache, _tw._head_num, _tw._dim_per_head,
+                                                 _tw._max_step, _batch_seq_len - 1, c[8] / Q,
+                                                 Q / c[11]));
+    LSH_CALL(decself_attention_i8(a, k_cache, v_cache, b, B * _tw._head_num, _batch_seq_len,
+                                  _tw._max_step, _tw._head_num, _tw._dim_per_head, _atten_scaler,
+                                  c[11] / Q, Q / c[5], _stream));
+    LSH_CALL(gemm_i8_i8o(b, w.w_out.get(), a, B, H, H, c[1] * c[5] / (c[9] * Q), _stream));
+    LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(a, w.ln2_scale.get(), w.ln2_bias.get(),
+                                                   w.b_ffn2.get(), b, _query.get(), B, H,
+                                                   c[9] / Q, Q / c[6], _stream, false, nullptr)));
+    ffn_add_norm(B, b, a);
+    std::swap(a, b);  // `a` names the buffer holding the layer's int8 LayerNorm output
+  }
+  CHECK_GPU_ERROR(hipMemcpyAsync(_hid_last.get(), a, (size_t)B * H, hipMemcpyDeviceToDevice,
+                                 _stream));
+}
+
+// logits of the last position + greedy choice; returns the unfinished flag (:399-487)
+int QuantGptEncoder::sample_one_token() {
+  const int H = _tw._hidden_size, V = _tw._src_vocab_size, B = _batch_size;
+  LSH_CALL(gemm_i8_i8o(_hid_last.get(), _int8_emb.get(), _logits.get(), B, V, H,
+                       _output_ln_clip_max * _src_emb_clip_max / (_logits_clip_max * _quant_range),
+                       _stream));
+  if (_rec_logits && _steps_run < _rec_max_steps)
+    CHECK_GPU_ERROR(hipMemcpyAsync(_rec_logits + (size_t)_steps_run * B * V, _logits.get(),
+                                   (size_t)B * V, hipMemcpyDeviceToDevice, _stream));
+  CHECK_GPU_ERROR(hipMemsetAsync(_unfinished.get(), 0, sizeof(int), _stream));
+  LSH_CALL(gpt_greedy_step(_logits.get(), _ids.get(), _last_ids.get(), V, _tw._max_step,
+                           _batch_seq_len, B, _unfinished.get(), _tw._eos_id, _stream));
+  const bool first = _steps_run == 0;
+  ++_steps_run;
+  _batch_seq_len++;
+  _batch_token_num += B;
+  if (_is_benchmark && !first) return 1;  // nothing stops a benchmark run but the length
+  CHECK_GPU_ERROR(hipMemcpyAsync(_h_unfinished, _unfinished.get(), sizeof(int),
+                                 hipMemcpyDeviceToHost, _stream));
+  CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+  return *_h_unfinished;
+}
+
+int QuantGptEncoder::run_one_sample(int batch_size, int batch_seq_len) {
+  if (batch_size > _max_batch_size)
+    throw std::runtime_error("batch size of input greater than max_batch_size");
+  if (batch_seq_len > _tw._max_step)
+    throw std::runtime_error("seq len of input greater than max_step");
+  if (batch_size <= 0 || batch_seq_len <= 0) throw std::runtime_error("empty input");
+  if (_tw._sampling_method == "ppl")
+    throw std::runtime_error("this model file is configured for perplexity, not sampling");
+  _batch_size = batch_size;
+  _batch_seq_len = batch_seq_len;
+  _batch_token_num = batch_size * batch_seq_len;
+  _batch_max_seq_len = std::min(_tw._max_step, batch_seq_len + _tw._extra_decode_length);
+  _steps_run = 0;
+  const int H = _tw._hidden_size;
+
+  // ids [batch, max_step] <- prompt
+  CHECK_GPU_ERROR(hipMemcpy2DAsync(_ids.get(), sizeof(int) * _tw._max_step, _p_d_token_id,
+                                   sizeof(int) * batch_seq_len, sizeof(int) * batch_seq_len,
+                                   batch_size, hipMemcpyDeviceToDevice, _stream));
+  prompt_pass(_p_d_token_id);
+  // hidden states of the last prompt position of every sequence
+  CHECK_GPU_ERROR(hipMemcpy2DAsync(_hid_last.get(), H,
+                                   _buf_a.get() + (size_t)(batch_seq_len - 1) * H,
+                                   (size_t)batch_seq_len * H, H, batch_size,
+                                   hipMemcpyDeviceToDevice, _stream));
+  if (_batch_seq_len < _tw._max_step) {
+    // (:347-353) after the prompt pass the run ends when nothing is unfinished
+    if (!(sample_one_token() == 0 || _batch_seq_len >= _batch_max_seq_len)) {
+      while (_batch_seq_len < _batch_max_seq_len) {
+        step_pass();
+        int unfinished = sample_one_token();
+        if (!unfinished && !_is_benchmark) break;
+      }
+    }
+  }
+  CHECK_GPU_ERROR(hipMemcpy2DAsync(_p_d_sample_id, sizeof(int) * _batch_seq_len, _ids.get(),
+                                   sizeof(int) * _tw._max_step, sizeof(int) * _batch_seq_len,
+                                   batch_size, hipMemcpyDeviceToDevice, _stream));
+  CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+  return _batch_seq_len;
+}
+
+void QuantGptEncoder::run_one_infer(int batch_size, int batch_seq_len) {
+  if (batch_size > _max_batch_size)
+    throw std::runtime_error("batch size of input greater than max_batch_size");
+  if (batch_seq_len > _tw._max_step)
+    throw std::runtime_error("seq len of input greater than max_step");
+  if (batch_size <= 0 || batch_seq_len <= 0) throw std::runtime_error("empty input");
+  if (_tw._sampling_method != "ppl")
+    throw std::runtime_error("this model file is configured for sampling, not perplexity");
+  _batch_size = batch_size;
+  _batch_seq_len = batch_seq_len;
+  _batch_token_num = batch_size * batch_seq_len;
+  const int H = _tw._hidden_size, V = _tw._src_vocab_size;
+  CHECK_GPU_ERROR(hipMemsetAsync(_p_d_ppl, 0, sizeof(float) * batch_size, _stream));
+  prompt_pass(_p_d_token_id);
+  /* compute_ppl (:781-797) */
+  LSH_CALL(gemm_i8_i8o(_buf_a.get(), _int8_emb.get(), _logits.get(), _batch_token_num, V, H,
+                       _output_ln_clip_max * _src_emb_clip_max / (_logits_clip_max * _quant_range),
+                       _stream));
+  LSH_CALL(ppl_i8I(batch_size, batch_seq_len, _stream, _logits.get(), _p_d_token_id,
+                   _real_seq_len.get(), _p_d_ppl, V, _logits_clip_max / _quant_range));
+}
+
+}  // namespace hip
+}  // namespace lightseq

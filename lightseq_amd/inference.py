@@ -250,3 +250,29 @@ class QuantTransformer(_HostIOModel):
 
     def steps_run(self):
         return self._int("ls_model_get_steps_run")
+
+
+class QuantGpt(_HostIOModel):
+    """int8 GPT (wrapper.cc ``PyQuantGpt``): ``sample(token_ids) -> int32 [batch, sampled_len]``
+    for model files with sampling_method "topk", ``ppl(token_ids) -> float32 [batch]`` for
+    files with sampling_method "ppl"."""
+
+    def __init__(self, weight_path, max_batch_size):
+        super().__init__("QuantGpt", weight_path, max_batch_size)
+
+    def infer(self, input_seq):
+        self._upload(input_seq)
+        self.infer_device()
+        return self._download(0).cpu().numpy()
+
+    sample = infer
+    ppl = infer
+
+    def set_step_record(self, logits, max_steps):
+        """Debug aid: device tensor [max_steps, batch, vocab] int8 that receives the
+        last-position logits of every sampling step."""
+        self._call("ls_model_set_step_record", self._h,
+                   _P(None if logits is None else logits.data_ptr()), _P(None), int(max_steps))
+
+    def steps_run(self):
+        return self._int("ls_model_get_steps_run")

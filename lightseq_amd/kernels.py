@@ -379,7 +379,87 @@ def refresh_cache_by_parent_i8(n_layer, rows, parent, k_old, v_old, k_new, v_new
          head_num, cur_step, max_step)
 
 
-__all__ = [n for n in dir() if n.startswith(("launch_", "ker_", "gemm_", "encself_", "quantize_",
+# --------------------------------------------------------------------------- #
+# GPT path
+# --------------------------------------------------------------------------- #
+def ker_gpt_embedding_i8I_launcher(batch_size, batch_seq_len, hidden_size, token_emb, pos_emb,
+                                   token_id, output, real_seq_len, padding_id, pos_offset,
+                                   dequant_scale):
+    _dev(token_emb, pos_emb, token_id, output, real_seq_len)
+    call("lsh_ker_gpt_embedding_i8I" + _suffix(output), batch_size, batch_seq_len, hidden_size,
+         current_stream(), ptr(token_emb), ptr(pos_emb), ptr(token_id), ptr(output),
+         ptr(real_seq_len), padding_id, pos_offset, dequant_scale)
+
+
+def gpt_scores_i8_i32o(k, q, scores, batch_head_num, batch_seq_len, dim_per_head):
+    _dev(k, q, scores)
+    call("lsh_gpt_scores_i8_i32o", ptr(k), ptr(q), ptr(scores), batch_head_num, batch_seq_len,
+         dim_per_head, current_stream())
+
+
+def ker_correlation_softmax_gpt_i32I_launcher(batch_size, batch_seq_len, head_num, correlation,
+                                              output, real_seq_len, attn_scale, dequant_scale):
+    _dev(correlation, output, real_seq_len)
+    call("lsh_ker_correlation_softmax_gpt_i32I" + _suffix(output), batch_size, batch_seq_len,
+         head_num, current_stream(), ptr(correlation), ptr(output), ptr(real_seq_len), attn_scale,
+         dequant_scale)
+
+
+def ker_arrange_qkv_with_cache_i8I_i8O_launcher(batch_token_num, hidden_size, ori_qkv, qkv_bias,
+                                                new_q, new_k, k_cache, new_v, v_cache,
+                                                batch_seq_len, dim_per_head, head_num,
+                                                dequant_scale, quant_scale, in_col32=False):
+    _dev(ori_qkv, qkv_bias, new_q, new_k, k_cache, new_v, v_cache)
+    call("lsh_ker_arrange_qkv_with_cache_i8I_i8O" + _suffix(qkv_bias), batch_token_num,
+         hidden_size, current_stream(), ptr(ori_qkv), ptr(qkv_bias), ptr(new_q), ptr(new_k),
+         ptr(k_cache), ptr(new_v), ptr(v_cache), batch_seq_len, dim_per_head, head_num,
+         dequant_scale, quant_scale, int(in_col32))
+
+
+def ker_topk_sample_i8I_launcher(batch_size, batch_seq_len, logits_seq_len, max_thread_per_block,
+                                 logits, old_input_ids, new_input_ids, real_seq_len, vocab_size, k,
+                                 unfinished, curandstate, eos_id, dequant_scale, in_col32=False):
+    _dev(logits, old_input_ids, new_input_ids, unfinished)
+    call("lsh_ker_topk_sample_i8I", batch_size, batch_seq_len, logits_seq_len,
+         max_thread_per_block, current_stream(), ptr(logits), ptr(old_input_ids),
+         ptr(new_input_ids), ptr(real_seq_len), vocab_size, k, ptr(unfinished), ptr(curandstate),
+         eos_id, dequant_scale, int(in_col32))
+
+
+def ker_ppl_i8I_launcher(batch_size, batch_seq_len, max_thread_per_block, logits, input_ids,
+                         real_seq_len, ppl, vocab_size, dequant_scale, in_col32=False):
+    _dev(logits, input_ids, real_seq_len, ppl)
+    call("lsh_ker_ppl_i8I", batch_size, batch_seq_len, max_thread_per_block, current_stream(),
+         ptr(logits), ptr(input_ids), ptr(real_seq_len), ptr(ppl), vocab_size, dequant_scale,
+         int(in_col32))
+
+
+def gpt_arrange_qkv_prefill(batch_token_num, hidden_size, ori_qkv, qkv_bias, q_codes, k_codes,
+                            v_deq, k_cache, v_cache, batch_seq_len, dim_per_head, head_num,
+                            max_step, dequant_scale, quant_scale):
+    _dev(ori_qkv, qkv_bias, q_codes, k_codes, v_deq, k_cache, v_cache)
+    call("lsh_gpt_arrange_qkv_prefill_f16", batch_token_num, hidden_size, current_stream(),
+         ptr(ori_qkv), ptr(qkv_bias), ptr(q_codes), ptr(k_codes), ptr(v_deq), ptr(k_cache),
+         ptr(v_cache), batch_seq_len, dim_per_head, head_num, max_step, dequant_scale, quant_scale)
+
+
+def gpt_prefill_attention(q_codes, k_codes, v, real_seq_len, ctx, ctx_q, quant_scale,
+                          dequant_scale, batch_size, batch_seq_len, head_num, dim_per_head):
+    """Causal prompt attention of the int8 GPT path in one kernel (fp16 storage)."""
+    _dev(q_codes, k_codes, v, real_seq_len, ctx, ctx_q)
+    call("lsh_gpt_prefill_attention_f16", ptr(q_codes), ptr(k_codes), ptr(v), ptr(real_seq_len),
+         ptr(ctx), ptr(ctx_q), quant_scale, dequant_scale, batch_size, batch_seq_len, head_num,
+         dim_per_head, current_stream())
+
+
+def gpt_greedy_step(logits, ids, last_ids, vocab_size, max_step, cur_len, batch_size, unfinished,
+                    eos_id):
+    _dev(logits, ids, last_ids, unfinished)
+    call("lsh_gpt_greedy_step", ptr(logits), ptr(ids), ptr(last_ids), vocab_size, max_step,
+         cur_len, batch_size, ptr(unfinished), eos_id, current_stream())
+
+
+__all__ = [n for n in dir() if n.startswith(("launch_", "ker_", "gemm_", "encself_", "quantize_", "gpt_",
                                              "decself_", "encdec_", "select_beam_", "beam_",
                                              "refresh_", "length_norm"))]
 _ = lib  # re-exported for callers that want lib.LSHError

@@ -72,6 +72,16 @@ _SIGNATURES = {
     "lsh_ker_write_topk_result": (False, "ppp" + "iiiiii" + "s"),
     "lsh_beam_search_step_i8I": (True, "pppppppppp" + "f" + "ii" + "f" + "iiii" + "s"),
     "lsh_refresh_cache_by_parent_i8": (False, "iis" + "ppppp" + "l" + "iiiii"),
+    # GPT path
+    "lsh_ker_gpt_embedding_i8I": (True, "iiis" + "ppppp" + "iif"),
+    "lsh_gpt_scores_i8_i32o": (False, "ppp" + "iii" + "s"),
+    "lsh_ker_correlation_softmax_gpt_i32I": (True, "iiis" + "ppp" + "ff"),
+    "lsh_ker_arrange_qkv_with_cache_i8I_i8O": (True, "iis" + "ppppppp" + "iii" + "ffi"),
+    "lsh_ker_topk_sample_i8I": (False, "iiiis" + "pppp" + "ii" + "pp" + "ifi"),
+    "lsh_ker_ppl_i8I": (False, "iiis" + "pppp" + "ifi"),
+    "lsh_gpt_arrange_qkv_prefill_f16": (False, "iis" + "ppppppp" + "iiii" + "ff"),
+    "lsh_gpt_prefill_attention_f16": (False, "pppppp" + "ff" + "iiii" + "s"),
+    "lsh_gpt_greedy_step": (False, "ppp" + "iiii" + "p" + "i" + "s"),
 }
 
 _lib = None

@@ -89,6 +89,23 @@ SCHEMAS = {
         "topk": (10, "int32"), "trg_end_id": (11, "int32"), "is_post_ln": (12, "bool"),
         "no_scale_embedding": (13, "bool"), "use_gelu": (14, "bool"), "multilg_type": (15, "int32"),
     },
+    # quant_gpt.proto
+    "QuantGptEncoderLayer": dict(_ENC_LAYER_COMMON, self_qkv_bias_out_clip_max=(24, "float")),
+    "QuantGptEmbeddingLayer": {
+        "token_embedding": (1, "bytes"), "position_embedding": (2, "rfloat"),
+        "norm_scale": (3, "rfloat"), "norm_bias": (4, "rfloat"), "emb_clip_max": (5, "float"),
+        "output_ln_clip_max": (6, "float"), "logits_clip_max": (7, "float"),
+    },
+    "QuantGptModelConf": {
+        "head_num": (1, "int32"), "src_padding_id": (2, "int32"), "sampling_method": (3, "string"),
+        "topp": (4, "float"), "topk": (5, "int32"), "eos_id": (6, "int32"),
+        "extra_decode_length": (7, "int32"),
+    },
+    "QuantGpt": {
+        "src_embedding": (1, "msg:QuantGptEmbeddingLayer"),
+        "encoder_stack": (2, "rmsg:QuantGptEncoderLayer"),
+        "model_conf": (3, "msg:QuantGptModelConf"),
+    },
     "QuantTransformer": {
         "src_embedding": (1, "msg:QuantEmbeddingLayer"),
         "encoder_stack": (2, "rmsg:QuantEncoderLayer"),

@@ -250,3 +250,81 @@ def write_quant_transformer(path, cfg, seed=0, ln_noise=0.02, eos_bias=None, w_s
     with open(path, "wb") as f:
         f.write(proto.encode("QuantTransformer", msg))
     return msg
+
+
+# --------------------------------------------------------------------------- #
+# QuantGpt (decoder-only, greedy / perplexity)
+# --------------------------------------------------------------------------- #
+def gpt_config(name):
+    """Shapes of the named synthetic decoder-only configurations."""
+    cfgs = {
+        # GPT-2-medium-shaped: 24 layers, hidden 1024, 16 heads, GELU, pre-LN, vocab 50257
+        "gpt2_medium": dict(n_layer=24, hidden=1024, inner=4096, head_num=16, max_step=640,
+                            vocab=50257, padding_id=50256, eos_id=50256, topk=1,
+                            extra_decode_length=128, sampling_method="topk"),
+        "tiny": dict(n_layer=2, hidden=128, inner=256, head_num=4, max_step=48, vocab=300,
+                     padding_id=0, eos_id=299, topk=1, extra_decode_length=16,
+                     sampling_method="topk"),
+    }
+    return dict(cfgs[name])
+
+
+def make_quant_gpt(cfg, seed=0, ln_noise=0.02, w_std=None):
+    """Build the QuantGpt message (a dict for :func:`proto.encode`).  The token embedding is
+    stored [hidden, vocab] as the reference's exporter writes it."""
+    rng = np.random.default_rng(seed)
+    H, I, L = cfg["hidden"], cfg["inner"], cfg["n_layer"]
+    w_std = float(cfg.get("w_std", W_STD) if w_std is None else w_std)
+    clip_e, clip_w = 4 * W_STD, 4 * w_std
+
+    def normal(*shape, std=W_STD):
+        return rng.standard_normal(shape, dtype=np.float32) * np.float32(std)
+
+    def ln_params():
+        return ((1 + normal(H, std=ln_noise)).astype(np.float32), normal(H, std=ln_noise))
+
+    def qk(rows, cols):
+        return quantize_u8(normal(rows, cols, std=w_std), clip_w).reshape(-1)
+
+    proj = float(4 * w_std * np.sqrt(H))
+    g, b = ln_params()
+    logit_sigma = W_STD * np.sqrt(H)
+    emb = {
+        "token_embedding": quantize_u8(normal(H, cfg["vocab"]), clip_e).reshape(-1),
+        "position_embedding": normal(cfg["max_step"], H, std=0.1).reshape(-1),
+        "norm_scale": g, "norm_bias": b, "emb_clip_max": clip_e,
+        "output_ln_clip_max": 4.0, "logits_clip_max": float(4 * logit_sigma),
+    }
+    layers = []
+    for _ in range(L):
+        g1, b1 = ln_params()
+        g2, b2 = ln_params()
+        layers.append({
+            "multihead_norm_scale": g1, "multihead_norm_bias": b1,
+            "multihead_project_kernel_qkv": qk(H, 3 * H), "multihead_project_bias_qkv": normal(3 * H),
+            "multihead_project_kernel_output": qk(H, H), "multihead_project_bias_output": normal(H),
+            "ffn_norm_scale": g2, "ffn_norm_bias": b2,
+            "ffn_first_kernel": qk(H, I), "ffn_first_bias": normal(I),
+            "ffn_second_kernel": qk(I, H), "ffn_second_bias": normal(H),
+            "multihead_project_kernel_qkv_clip_max": clip_w,
+            "multihead_project_kernel_output_clip_max": clip_w,
+            "ffn_first_kernel_clip_max": clip_w, "ffn_second_kernel_clip_max": clip_w,
+            "multihead_ln_clip_max": 4.0, "multihead_project_output_clip_max": proj / 2,
+            "ffn_ln_clip_max": 4.0, "ffn_first_act_clip_max": proj,
+            "multihead_qkv_dense_clip_max": proj,
+            "multihead_output_dense_clip_max": proj * proj / 8,
+            "ffn_first_output_clip_max": proj, "self_qkv_bias_out_clip_max": proj,
+        })
+    conf = {"head_num": cfg["head_num"], "src_padding_id": cfg["padding_id"],
+            "sampling_method": cfg.get("sampling_method", "topk"), "topp": 0.75,
+            "topk": cfg.get("topk", 1), "eos_id": cfg["eos_id"],
+            "extra_decode_length": cfg["extra_decode_length"]}
+    return {"src_embedding": emb, "encoder_stack": layers, "model_conf": conf}
+
+
+def write_quant_gpt(path, cfg, seed=0, ln_noise=0.02, w_std=None):
+    """Write a synthetic QuantGpt model file; returns the message dict."""
+    msg = make_quant_gpt(cfg, seed=seed, ln_noise=ln_noise, w_std=w_std)
+    with open(path, "wb") as f:
+        f.write(proto.encode("QuantGpt", msg))
+    return msg

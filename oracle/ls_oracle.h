@@ -358,6 +358,92 @@ int lso_quant_decoder(const lso_dec_weights* w, const void* enc_out,
                       int output_topk, int* result, int* out_len, float* scores,
                       lso_dec_trace* trace);
 
+/* ========================================================================= */
+/* GPT half (ls_oracle_gpt.c)                                                  */
+/* ========================================================================= */
+
+/* kernels/gptKernels_int8.cc.cu:21-106.  token_emb [vocab, hidden]; token_id
+ * [batch, seq_len]; real_seq_len[b] += number of non-padding tokens of row b. */
+void lso_gpt_embedding_i8I(const int8_t* token_emb, const void* pos_emb,
+                           const int* token_id, void* output, int* real_seq_len,
+                           int padding_id, int pos_offset, float dequant_scale,
+                           int batch, int seq_len, int hidden, int f16);
+
+/* model/quant_gpt_encoder.cc.cu:498-505: scores[bh, i, j] = sum_d q[bh,i,d] k[bh,j,d] */
+void lso_gpt_scores_i8(const int8_t* q, const int8_t* k, int32_t* scores,
+                       int batch_heads, int seq_len, int dim_per_head);
+
+/* kernels/gptKernels_int8.cc.cu:192-250.  Rows of padded queries are written as
+ * zeros (the reference leaves them untouched). */
+void lso_correlation_softmax_gpt_i32I(const int32_t* correlation, void* output,
+                                      const int* real_seq_len, int batch,
+                                      int seq_len, int head_num, float attn_scale,
+                                      float dequant_scale, int f16);
+
+/* kernels/gptKernels_int8.cc.cu:658-812: one new token per sequence; the caches
+ * are re-laid out from [batch, head, seq_len-1, d] to [batch, head, seq_len, d]
+ * with the new key / value appended; new_q [batch, head, 1, d]. */
+void lso_arrange_qkv_with_cache_i8I_i8O(const int8_t* ori_qkv, const void* qkv_bias,
+                                        int8_t* new_q, int8_t* new_k,
+                                        const int8_t* k_cache, int8_t* new_v,
+                                        const int8_t* v_cache, int batch,
+                                        int seq_len, int dim_per_head,
+                                        int head_num, float dequant_scale,
+                                        float quant_scale, int f16);
+
+/* kernels/gptKernels_int8.cc.cu:252-463 with k == 1 (greedy).  old ids
+ * [batch, seq_len] -> new ids [batch, seq_len + 1]; the sampled ids are also
+ * stored behind the old array (old_input_ids[batch*seq_len + b]); a sequence whose
+ * last token is eos_id gets eos_id again.  Ties at the maximum go to the lowest
+ * token id (the reference lets racing stores decide).  *unfinished is set to 1
+ * when any freshly sampled token differs from eos_id. */
+void lso_topk_sample_i8I_greedy(const int8_t* logits, int* old_input_ids,
+                                int* new_input_ids, int vocab_size, int batch,
+                                int seq_len, int logits_seq_len, int* unfinished,
+                                int eos_id, float dequant_scale);
+
+/* kernels/gptKernels_int8.cc.cu:108-190.  logits [batch, seq_len, vocab]; ppl[b] +=
+ * mean negative log-likelihood of tokens 1 .. real_seq_len-1. */
+void lso_ppl_i8I(const int8_t* logits, const int* input_ids, const int* real_seq_len,
+                 float* ppl, int vocab_size, float dequant_scale, int batch,
+                 int seq_len);
+
+/* ---- whole model: model/quant_gpt_encoder.cc.cu:253-824 ------------------- */
+typedef struct {
+  int n_layer, hidden, inner, head_num, max_step, vocab, padding_id, eos_id;
+  int extra_decode_length, f16;
+  const int8_t* tok_emb_q; /* [vocab, hidden] codes */
+  const void* pos_emb;
+  const void* out_ln_scale;
+  const void* out_ln_bias;
+  float emb_clip_max, output_ln_clip_max, logits_clip_max;
+  const void* const* ln1_scale;
+  const void* const* ln1_bias;
+  const int8_t* const* w_qkv;
+  const void* const* b_qkv;
+  const int8_t* const* w_out;
+  const void* const* b_out;
+  const void* const* ln2_scale;
+  const void* const* ln2_bias;
+  const int8_t* const* w_ffn1;
+  const void* const* b_ffn1;
+  const int8_t* const* w_ffn2;
+  const void* const* b_ffn2;
+  const float* clip_max; /* [n_layer * 12], proto/quant_gpt_weight.cc:228-240 */
+} lso_gpt_weights;
+
+/* sampling_method "ppl": ppl [batch].  Returns 0 on success. */
+int lso_quant_gpt_ppl(const lso_gpt_weights* w, const int* token_ids, int batch,
+                      int seq_len, float* ppl);
+/* sampling_method "topk" with topk == 1.  out_ids [batch, *out_len].
+ * logits_record: NULL or [max_step, batch, vocab] (the logits of the last position at
+ * every sampling step); forced_logits likewise replaces the oracle's own logits in the
+ * arg-max for the first forced_steps steps.  *steps_run counts sampling steps. */
+int lso_quant_gpt_sample(const lso_gpt_weights* w, const int* token_ids, int batch,
+                         int seq_len, int is_benchmark, int* out_ids, int* out_len,
+                         const int8_t* forced_logits, int forced_steps,
+                         int8_t* logits_record, int* steps_run);
+
 #ifdef __cplusplus
 }
 #endif

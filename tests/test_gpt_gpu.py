@@ -1,0 +1,339 @@
+"""GPU parity of the int8 GPT path: its kernels through the C ABI and the QuantGpt model
+through the model C ABI, against the CPU oracle.
+
+Bars: integer work (cache writes / re-layout, int32 scores, sampled ids given equal logits)
+bit-exact; int8 activations within +-1 code on <= 0.1 % of the elements; fp16 values within
+the tolerance written in each test.  Whole-run token equality is checked stage-conditionally
+(the oracle consumes the GPU's logits in its arg-max) and, on small models, free-running.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import assert_codes_close
+from helpers import DEV, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float16, np.float32]
+TD = {np.float16: torch.float16, np.float32: torch.float32}
+
+
+def _k():
+    from lightseq_amd import kernels
+    return kernels
+
+
+def _og():
+    from oracle import gpt
+    return gpt
+
+
+def _codes(rng, shape):
+    return rng.integers(-127, 128, size=shape, dtype=np.int8)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("batch,seq,hidden,vocab,offset", [(3, 7, 128, 50, 0), (2, 1, 1024, 300, 9),
+                                                           (1, 16, 72, 20, 3)])
+def test_gpt_embedding(rng, dtype, batch, seq, hidden, vocab, offset):
+    table = _codes(rng, (vocab, hidden))
+    pos = (rng.standard_normal((seq + offset + 2, hidden)) * 0.1).astype(dtype)
+    pad = 0
+    ids = rng.integers(0, vocab, size=(batch, seq), dtype=np.int32)
+    ids[0, seq // 2:] = pad
+    rsl0 = rng.integers(0, 5, size=batch).astype(np.int32)
+    dq = 0.08 / 127
+    want, want_rsl = _og().gpt_embedding_i8I(table, pos, ids, rsl0, pad, offset, dq)
+    out = torch.zeros(batch, seq, hidden, dtype=TD[dtype], device=DEV)
+    rsl = to_dev(rsl0)
+    _k().ker_gpt_embedding_i8I_launcher(batch, seq, hidden, to_dev(table), to_dev(pos), to_dev(ids),
+                                        out, rsl, pad, offset, dq)
+    np.testing.assert_array_equal(to_np(out), want)
+    np.testing.assert_array_equal(to_np(rsl), want_rsl)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("batch,heads,seq,d", [(2, 3, 9, 16), (1, 4, 130, 32), (3, 2, 64, 64)])
+def test_gpt_scores_and_softmax(rng, dtype, batch, heads, seq, d):
+    bh = batch * heads
+    q, k = _codes(rng, (bh, seq, d)), _codes(rng, (bh, seq, d))
+    want_sc = _og().gpt_scores_i8(q, k)
+    sc = torch.zeros(bh, seq, seq, dtype=torch.int32, device=DEV)
+    _k().gpt_scores_i8_i32o(to_dev(k), to_dev(q), sc, bh, seq, d)
+    np.testing.assert_array_equal(to_np(sc), want_sc)
+
+    rsl = rng.integers(max(1, seq // 2), seq + 1, size=batch).astype(np.int32)
+    rsl[0] = seq
+    dq, attn_scale = 4.0 / 127, float(np.float16(np.sqrt(1.0 / d)))
+    want = _og().correlation_softmax_gpt_i32I(want_sc, rsl, heads, attn_scale, dq, dtype)
+    out = torch.full((bh, seq, seq), 7.0, dtype=TD[dtype], device=DEV)
+    _k().ker_correlation_softmax_gpt_i32I_launcher(batch, seq, heads, sc, out, to_dev(rsl),
+                                                   attn_scale, dq)
+    got = to_np(out).astype(np.float32)
+    tol = 1e-3 if dtype == np.float16 else 2e-6
+    np.testing.assert_allclose(got, want.astype(np.float32), atol=tol, rtol=0)
+    assert not np.triu(got, 1).any()  # nothing to the right of the diagonal
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("batch,heads,seq,d", [(2, 3, 5, 16), (3, 16, 1, 64), (1, 2, 40, 10)])
+def test_arrange_qkv_with_cache(rng, dtype, batch, heads, seq, d):
+    H = heads * d
+    ori = _codes(rng, (batch, 3 * H))
+    bias = (rng.standard_normal(3 * H) * 0.5).astype(dtype)
+    kc, vc = _codes(rng, (batch, heads, seq - 1, d)), _codes(rng, (batch, heads, seq - 1, d))
+    dq, qs = 3.0 / 127, 127 / 2.5
+    wq, wk, wv = _og().arrange_qkv_with_cache_i8I_i8O(ori, bias, kc, vc, dq, qs)
+    q = torch.zeros(batch, heads, 1, d, dtype=torch.int8, device=DEV)
+    nk = torch.zeros(batch, heads, seq, d, dtype=torch.int8, device=DEV)
+    nv = torch.zeros_like(nk)
+    kcd = to_dev(kc) if seq > 1 else torch.zeros(1, dtype=torch.int8, device=DEV)
+    vcd = to_dev(vc) if seq > 1 else torch.zeros(1, dtype=torch.int8, device=DEV)
+    _k().ker_arrange_qkv_with_cache_i8I_i8O_launcher(batch * seq, H, to_dev(ori), to_dev(bias), q,
+                                                     nk, kcd, nv, vcd, seq, d, heads, dq, qs)
+    np.testing.assert_array_equal(to_np(q), wq)
+    np.testing.assert_array_equal(to_np(nk), wk)
+    np.testing.assert_array_equal(to_np(nv), wv)
+
+
+@pytest.mark.parametrize("batch,seq,vocab,lsl", [(4, 6, 300, 6), (3, 9, 50257, 1), (2, 1, 77, 1)])
+def test_topk_sample_greedy(rng, batch, seq, vocab, lsl):
+    eos = 5
+    logits = np.clip(rng.standard_normal((batch * lsl, vocab)) * 30, -127, 127).astype(np.int8)
+    logits[(0 + 1) * lsl - 1, 17:20] = 127  # a three-way tie at the maximum: lowest id wins
+    old = rng.integers(6, vocab, size=(batch, seq), dtype=np.int32)
+    old[1, -1] = eos  # an ended sequence stays ended
+    if batch > 2:
+        logits[(2 + 1) * lsl - 1, eos] = 127
+        logits[(2 + 1) * lsl - 1, :eos] = -5
+    w_new, w_last, w_unf = _og().topk_sample_i8I_greedy(logits, old, lsl, eos, 0.02)
+    assert w_last[0] == 17 and w_last[1] == eos
+    buf = torch.zeros(batch * seq + batch, dtype=torch.int32, device=DEV)
+    buf[:batch * seq] = to_dev(old.reshape(-1))
+    new = torch.zeros(batch, seq + 1, dtype=torch.int32, device=DEV)
+    unf = torch.zeros(1, dtype=torch.int32, device=DEV)
+    _k().ker_topk_sample_i8I_launcher(batch, seq, lsl, 1024, to_dev(logits), buf, new, None, vocab,
+                                      1, unf, None, eos, 0.02)
+    np.testing.assert_array_equal(to_np(new), w_new)
+    np.testing.assert_array_equal(to_np(buf)[batch * seq:], w_last)
+    assert int(to_np(unf)[0]) == w_unf
+
+    # the in-place step of the model gives the same tokens
+    max_step = seq + 3
+    ids = torch.zeros(batch, max_step, dtype=torch.int32, device=DEV)
+    ids[:, :seq] = to_dev(old)
+    last = torch.zeros(batch, dtype=torch.int32, device=DEV)
+    unf2 = torch.zeros(1, dtype=torch.int32, device=DEV)
+    last_rows = to_dev(np.ascontiguousarray(logits.reshape(batch, lsl, vocab)[:, -1]))
+    _k().gpt_greedy_step(last_rows, ids, last, vocab, max_step, seq, batch, unf2, eos)
+    np.testing.assert_array_equal(to_np(ids)[:, :seq + 1], w_new)
+    np.testing.assert_array_equal(to_np(last), w_last)
+    assert int(to_np(unf2)[0]) == w_unf
+
+
+def test_topk_sample_errors():
+    from lightseq_amd.lib import LSHError
+    z8 = torch.zeros(64, dtype=torch.int8, device=DEV)
+    zi = torch.zeros(64, dtype=torch.int32, device=DEV)
+    with pytest.raises(LSHError, match="only topk = 1"):
+        _k().ker_topk_sample_i8I_launcher(1, 4, 1, 1024, z8, zi, zi, None, 16, 4, zi, None, 1, 0.1)
+    with pytest.raises(LSHError, match=r"\[1,2,4,8,16,32\]"):
+        _k().ker_topk_sample_i8I_launcher(1, 4, 1, 1024, z8, zi, zi, None, 16, 3, zi, None, 1, 0.1)
+
+
+@pytest.mark.parametrize("batch,seq,vocab", [(3, 8, 300), (2, 5, 5000)])
+def test_ppl(rng, batch, seq, vocab):
+    logits = np.clip(rng.standard_normal((batch * seq, vocab)) * 30, -127, 127).astype(np.int8)
+    ids = rng.integers(0, vocab, size=(batch, seq), dtype=np.int32)
+    rsl = np.array([seq, max(2, seq - 3), 1][:batch], np.int32)
+    want = _og().ppl_i8I(logits, ids, rsl, 0.02)
+    ppl = torch.zeros(batch, dtype=torch.float32, device=DEV)
+    _k().ker_ppl_i8I_launcher(batch, seq, 1024, to_dev(logits), to_dev(ids), to_dev(rsl), ppl,
+                              vocab, 0.02)
+    np.testing.assert_allclose(to_np(ppl), want, rtol=2e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("batch,heads,seq,d,max_step", [(2, 2, 9, 32, 16), (2, 16, 130, 64, 160),
+                                                        (1, 4, 64, 64, 64), (3, 2, 200, 32, 256)])
+def test_prefill_attention_fused(oracle, rng, batch, heads, seq, d, max_step):
+    """gpt_arrange_qkv_prefill + gpt_prefill_attention == the reference's unfused chain."""
+    H, M, bh = heads * d, batch * seq, batch * heads
+    ori = _codes(rng, (M, 3 * H))
+    bias = (rng.standard_normal(3 * H) * 0.5).astype(np.float16)
+    dq_in, qs_cache = 3.0 / 127, 127 / 3.2
+    rsl = rng.integers(max(1, seq // 2), seq + 1, size=batch).astype(np.int32)
+    rsl[0] = seq
+    q8, k8, v8, dv = oracle.arrange_encself_qkv_i8I_i8O(ori, bias, batch, seq, heads, dq_in, qs_cache)
+    sc = _og().gpt_scores_i8(q8.reshape(bh, seq, d), k8.reshape(bh, seq, d))
+    attn_scale = float(np.float16(np.sqrt(1.0 / d)))
+    pr = _og().correlation_softmax_gpt_i32I(sc, rsl, heads, attn_scale, 1.0 / qs_cache, np.float16)
+    ctx = oracle.attn_context(pr, dv)
+    qs_out = 127 / 1.6
+    want_q = oracle.arrange_atten_output_i8O(ctx.reshape(batch, heads, seq, d), qs_out)
+
+    qc = torch.zeros(batch, heads, seq, d, dtype=torch.float16, device=DEV)
+    kc, vd = torch.zeros_like(qc), torch.zeros_like(qc)
+    kcache = torch.zeros(batch, heads, max_step, d, dtype=torch.int8, device=DEV)
+    vcache = torch.zeros_like(kcache)
+    _k().gpt_arrange_qkv_prefill(M, H, to_dev(ori), to_dev(bias), qc, kc, vd, kcache, vcache, seq,
+                                 d, heads, max_step, dq_in, qs_cache)
+    np.testing.assert_array_equal(to_np(qc), q8.astype(np.float16))
+    np.testing.assert_array_equal(to_np(kc), k8.astype(np.float16))
+    np.testing.assert_array_equal(to_np(vd), dv)
+    np.testing.assert_array_equal(to_np(kcache)[:, :, :seq], k8)
+    np.testing.assert_array_equal(to_np(vcache)[:, :, :seq], v8)
+    assert not to_np(kcache)[:, :, seq:].any()
+
+    ctx_d = torch.zeros(batch, heads, seq, d, dtype=torch.float16, device=DEV)
+    ctx_q = torch.zeros(M, H, dtype=torch.int8, device=DEV)
+    _k().gpt_prefill_attention(qc, kc, vd, to_dev(rsl), ctx_d, ctx_q, qs_out, 1.0 / qs_cache, batch,
+                               seq, heads, d)
+    got = to_np(ctx_d).astype(np.float32).reshape(ctx.shape)
+    np.testing.assert_allclose(got, ctx.astype(np.float32), atol=4e-3, rtol=0)
+    assert_codes_close(to_np(ctx_q), want_q.reshape(M, H), max_frac=5e-3, what="gpt ctx_q")
+    # padded queries give zeros
+    for b in range(batch):
+        assert not to_np(ctx_q).reshape(batch, seq, H)[b, rsl[b]:].any()
+
+
+# --------------------------------------------------------------------------- #
+# model
+# --------------------------------------------------------------------------- #
+def _make(tmp_path, cfg, seed, **kw):
+    from lightseq_amd import synthetic
+    path = os.path.join(str(tmp_path), "gpt_%d.pb" % seed)
+    msg = synthetic.write_quant_gpt(path, cfg, seed=seed, **kw)
+    return path, msg
+
+
+def _prompt(cfg, batch, seq, seed, pad_tail=0):
+    rng = np.random.default_rng(seed + 100)
+    hi = cfg["vocab"] - 1
+    ids = rng.integers(1, hi, size=(batch, seq), dtype=np.int32)
+    ids[ids == cfg["padding_id"]] = 1
+    ids[ids == cfg["eos_id"]] = 1
+    if pad_tail:
+        ids[-1, seq - pad_tail:] = cfg["padding_id"]
+    return ids
+
+
+def _run_sample(path, cfg, ids, max_batch, benchmark=False):
+    from lightseq_amd.inference import QuantGpt
+    model = QuantGpt(path, max_batch)
+    rec = torch.zeros(cfg["max_step"], ids.shape[0], cfg["vocab"], dtype=torch.int8, device=DEV)
+    model.set_step_record(rec, cfg["max_step"])
+    model.benchmark_mode(benchmark)
+    out = model.sample(ids)
+    steps = model.steps_run()
+    logits = rec.cpu().numpy()[:steps]
+    model.close()
+    return out, steps, logits
+
+
+def _check_sample(msg, cfg, ids, out, steps, logits, benchmark=False):
+    w = _og().gpt_weights_from_message(msg, cfg, np.float16)
+    r = _og().quant_gpt_sample(w, ids, is_benchmark=benchmark, forced_logits=logits, record=True)
+    assert r["steps_run"] == steps
+    np.testing.assert_array_equal(r["ids"], out)
+    diff = np.abs(r["logits"].astype(np.int32) - logits.astype(np.int32))
+    frac, frac2 = float((diff != 0).mean()), float((diff > 1).mean())
+    print("steps %d: %.3f%% of logit codes differ, %.4f%% by more than one code, max %d" %
+          (steps, 100 * frac, 100 * frac2, diff.max()))
+    # every int8-output GEMM turns one flipped input code into +-1 flips on a few percent
+    # of its outputs, so rows that saw a flip upstream are decorrelated at the rounding level
+    assert diff.max() <= 6
+    assert frac2 <= 2e-2 and frac <= 0.4
+    return w, r
+
+
+@pytest.mark.parametrize("seed,batch,seq,pad_tail", [(1, 3, 9, 0), (2, 2, 17, 4), (3, 1, 5, 0),
+                                                      (4, 4, 12, 3)])
+def test_tiny_gpt_sample(tmp_path, seed, batch, seq, pad_tail):
+    from lightseq_amd import synthetic
+    cfg = synthetic.gpt_config("tiny")
+    path, msg = _make(tmp_path, cfg, seed, w_std=0.2)
+    ids = _prompt(cfg, batch, seq, seed, pad_tail)
+    out, steps, logits = _run_sample(path, cfg, ids, max_batch=4)
+    assert out.shape[0] == batch and out.shape[1] == seq + steps
+    np.testing.assert_array_equal(out[:, :seq], ids)
+    w, _ = _check_sample(msg, cfg, ids, out, steps, logits)
+    if pad_tail == 0:
+        free = _og().quant_gpt_sample(w, ids)
+        assert free["ids"].shape == out.shape
+        same = float((free["ids"] == out).all(axis=1).mean())
+        assert same == 1.0, "only %.0f%% of the sequences agree with the free-running oracle" % (
+            100 * same)
+
+
+def test_gpt_benchmark_mode_and_eos(tmp_path):
+    from lightseq_amd import synthetic
+    cfg = synthetic.gpt_config("tiny")
+    path, msg = _make(tmp_path, cfg, 1, w_std=0.2)
+    ids = _prompt(cfg, 3, 9, 1)
+    out, steps, logits = _run_sample(path, cfg, ids, max_batch=3, benchmark=True)
+    limit = min(cfg["max_step"], ids.shape[1] + cfg["extra_decode_length"])
+    assert out.shape[1] == limit
+    _check_sample(msg, cfg, ids, out, steps, logits, benchmark=True)
+    # once a sequence produced <eos> it keeps producing it
+    for row in out:
+        hit = np.nonzero(row[ids.shape[1]:] == cfg["eos_id"])[0]
+        if hit.size:
+            assert (row[ids.shape[1] + hit[0]:] == cfg["eos_id"]).all()
+
+
+def test_tiny_gpt_ppl(tmp_path):
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import QuantGpt
+    cfg = synthetic.gpt_config("tiny")
+    cfg["sampling_method"] = "ppl"
+    path, msg = _make(tmp_path, cfg, 6, w_std=0.2)
+    ids = _prompt(cfg, 3, 11, 6, pad_tail=4)
+    model = QuantGpt(path, 3)
+    assert model.get_output_dtype(0) == 1 and model.get_output_max_shape(0) == [3]
+    got = model.ppl(ids)
+    model.close()
+    w = _og().gpt_weights_from_message(msg, cfg, np.float16)
+    want = _og().quant_gpt_ppl(w, ids)
+    assert got.shape == (3,)
+    # mean log-likelihood over ~10 positions, each moved by a few flipped logit codes at most
+    np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-3)
+
+
+def test_gpt_interface_and_errors(tmp_path):
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import LSModel, QuantGpt
+    from lightseq_amd.lib import LSHError
+    cfg = synthetic.gpt_config("tiny")
+    path, _ = _make(tmp_path, cfg, 8, w_std=0.2)
+    model = QuantGpt(path, 2)
+    assert model.get_input_name(0) == "token_ids" and model.get_output_name(0) == "result"
+    assert model.get_input_max_shape(0) == [2, cfg["max_step"]]
+    assert model.get_output_max_shape(0) == [2, cfg["max_step"]]
+    assert model.get_input_dtype(0) == 2 and model.get_output_dtype(0) == 2
+    a = model.sample(_prompt(cfg, 2, 7, 1))
+    b = model.sample(_prompt(cfg, 2, 7, 1))
+    np.testing.assert_array_equal(a, b)
+    with pytest.raises(LSHError, match="max_batch_size"):
+        model.sample(_prompt(cfg, 3, 5, 0))
+    model.close()
+    bad = dict(cfg, topk=4)
+    path2 = os.path.join(str(tmp_path), "topk4.pb")
+    synthetic.write_quant_gpt(path2, bad, seed=1)
+    with pytest.raises(LSHError, match="random sampling"):
+        LSModel("QuantGpt", path2, 2)
+
+
+def test_gpt2_medium_shape(tmp_path):
+    """GPT-2-medium-shaped model (hidden 1024, 16 heads, inner 4096, vocabulary 50257) with
+    fewer layers and a shorter prompt so that the oracle finishes in seconds."""
+    from lightseq_amd import synthetic
+    cfg = synthetic.gpt_config("gpt2_medium")
+    cfg.update(n_layer=2, max_step=96, extra_decode_length=8)
+    path, msg = _make(tmp_path, cfg, 12, w_std=0.05)
+    ids = _prompt(cfg, 2, 48, 12, pad_tail=5)
+    out, steps, logits = _run_sample(path, cfg, ids, max_batch=2)
+    assert steps >= 1 and out.shape[1] == 48 + steps
+    _check_sample(msg, cfg, ids, out, steps, logits)
