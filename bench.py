@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 transformer-layer forward path on one MI355X.
 
-Workload: the BERT-base-shaped int8 encoder stack --
+Default workload (``--workload bert_base``): the BERT-base-shaped int8 encoder stack --
 12 layers, hidden 768, 12 heads, FFN 3072 GELU, batch 32 x max seq 128, per-sequence
 valid lengths uniform in [32, 128] with right padding, token ids uniform over a
 30522 vocabulary, random-init weights ~N(0, 0.02) quantised per tensor -- run
@@ -11,12 +11,21 @@ HBM.  ``value`` = batch * seq_len * steps / wall time of the timed steps (padded
 tokens counted, as the reference's b32 x s128 figures do).
 
 The JSON line also carries
-  roofline      the dominant kernel (by total time) among the int8 GEMM
-                instantiations, timed with HIP events on the model's stream during a
-                second, instrumented pass over the same steps: achieved = 2*M*N*K per
-                launch / mean launch time, against the 5.0 POP/s dense int8 MFMA peak;
-  cpu_baseline  the CPU oracle (a C port of the reference's algorithm, OpenMP) timed
-                on this host on a bounded sample of the same workload.
+  roofline       the dominant kernel (by total time) among the int8 GEMM
+                 instantiations, timed with HIP events on the model's stream during a
+                 second, instrumented pass over the same steps: achieved = 2*M*N*K per
+                 launch / mean launch time, against the 5.0 POP/s dense int8 MFMA peak;
+  fused_kernels  the memory-bound fused kernels of one encoder layer at this workload's
+                 shapes, each timed alone with events on its stream: achieved GB/s =
+                 algorithmic bytes (every operand touched once) / mean launch time,
+                 against the 8 TB/s HBM peak;
+  cpu_baseline   the CPU oracle (a C port of the reference's algorithm, OpenMP) timed
+                 on this host on a bounded sample of the same workload.
+
+``--workload transformer_big`` and ``--workload gpt2_medium`` time the two generation
+workloads (beam-search translation, greedy GPT generation) through ``QuantTransformer`` /
+``QuantGpt`` in benchmark mode and report generated tokens/s; they print a line of the
+same form without the GEMM roofline.
 """
 import argparse
 import json
@@ -29,6 +38,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 INT8_MFMA_PEAK_TOPS = 5000.0  # dense int8, MI355X
+HBM_PEAK_GBS = 8000.0
 
 BATCH, SEQ = 32, 128
 
@@ -36,7 +46,6 @@ BATCH, SEQ = 32, 128
 def cpu_baseline(cfg, msg, ids, layers=12):
     """Oracle timed on the host: `layers` encoder layers of the real width at the full
     b32 x s128 batch, scaled to the 12-layer stack."""
-    import numpy as np
     from oracle import oracle
     from oracle.model_io import oracle_weights_from_message
     sub = dict(cfg, n_layer=layers)
@@ -54,22 +63,73 @@ def cpu_baseline(cfg, msg, ids, layers=12):
                          "" if layers == cfg["n_layer"] else ", scaled to the full stack")}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this path runs on one GPU only (every model object owns device 0 and "
-                 "one stream, as in the reference); --gpus %d is not supported" % args.gpus)
+def fused_kernel_rates(cfg, reps=50):
+    """Each memory-bound kernel of one encoder layer alone, at the workload's shapes."""
+    import torch
+    from lightseq_amd import kernels as K
+    dev = "cuda:0"
+    M, H, I, h = BATCH * SEQ, cfg["hidden"], cfg["inner"], cfg["head_num"]
+    d = H // h
+    g = torch.Generator(device=dev).manual_seed(0)
 
+    def i8(*shape):
+        return torch.randint(-127, 128, shape, dtype=torch.int8, device=dev, generator=g)
+
+    def f16(*shape):
+        return torch.randn(*shape, dtype=torch.float16, device=dev, generator=g)
+
+    x16, res16 = f16(M, H), f16(M, H)
+    q8_h, q8_3h, q8_i, out8_i = i8(M, H), i8(M, 3 * H), i8(M, I), i8(M, I)
+    acc32 = torch.randint(-2 ** 20, 2 ** 20, (M, H), dtype=torch.int32, device=dev, generator=g)
+    gam, bet, rb = f16(H), f16(H), f16(H)
+    b3h, bi = f16(3 * H), f16(I)
+    qkv = torch.zeros(3, BATCH, h, SEQ, d, dtype=torch.float16, device=dev)
+    qkv.copy_(f16(3, BATCH, h, SEQ, d))
+    mask = torch.zeros(BATCH, SEQ, dtype=torch.int32, device=dev)
+    ctx8 = i8(M, H)
+    mbd = M * H
+    cases = [
+        # name, algorithmic bytes, launcher
+        ("launch_quantize_tensor f16->i8", M * H * 3,
+         lambda: K.launch_quantize_tensor(x16, q8_h, M, H, 30.0)),
+        ("launch_dequantize_tensor i32->f16", M * H * 6,
+         lambda: K.launch_dequantize_tensor(acc32, x16, M, H, 1e-4)),
+        ("ker_residual_bias_ln_i8I_i8O", M * H * (1 + 2 + 1 + 2),
+         lambda: K.ker_residual_bias_ln_i8I_i8O_launcher(q8_h, gam, bet, rb, ctx8, res16, M, H,
+                                                         0.05, 30.0, 1024, True)),
+        ("ker_residual_bias_ln_i32I_i8O", M * H * (4 + 2 + 1 + 2),
+         lambda: K.ker_residual_bias_ln_i32I_i8O_launcher(acc32, gam, bet, rb, ctx8, res16, M, H,
+                                                          1e-4, 30.0, 1024, True)),
+        ("ker_bias_gelu_i8I_i8O", M * I * 2,
+         lambda: K.ker_bias_gelu_i8I_i8O_launcher(M, q8_i, out8_i, bi, I, 0.05, 30.0)),
+        ("ker_arrange_encself_qkv_i8I", M * 3 * H * (1 + 2),
+         lambda: K.ker_arrange_encself_qkv_i8I_launcher(M, H, q8_3h, b3h, qkv, mbd, SEQ, d, h, 1024,
+                                                        0.05)),
+        ("encself_attention (fused QK^T, softmax, PV, merge+quant)", M * H * (3 * 2 + 1),
+         lambda: K.encself_attention(qkv[0], qkv[1], qkv[2], mask, None, ctx8, 30.0, BATCH, SEQ, h,
+                                     d)),
+    ]
+    out = {}
+    for name, nbytes, fn in cases:
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        gbs = nbytes / (us * 1e-6) / 1e9
+        out[name] = {"avg_us": us, "algorithmic_bytes": nbytes, "GB/s": gbs,
+                     "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
+    return out
+
+
+def bench_bert(args):
     import torch
     from lightseq_amd import inference, synthetic
-
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: no GPU visible")
     cfg = synthetic.bert_config("bert_base")
     tmp = tempfile.mkdtemp(prefix="ls_bench_")
     path = os.path.join(tmp, "quant_bert_base.pb")
@@ -114,7 +174,6 @@ def main():
                                            "tops": 2.0 * s["m"] * s["n"] * s["k"] * s["launches"]
                                            / max(1e-12, s["total_ms"] * 1e-3) / 1e12}
                                for s in prof}}
-
     out = {
         "metric": "int8 tokens/sec BERT-base b32 s128; int8 GEMM % MFMA-i8 peak; fused GB/s",
         "value": tokens_per_s, "unit": "tokens/s",
@@ -128,9 +187,98 @@ def main():
                    "entry_point": "QuantBert / LSModel::Infer"},
         "roofline": roofline,
     }
+    model.close()
+    if not args.no_fused:
+        out["fused_kernels"] = fused_kernel_rates(cfg)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, msg, ids)
+    return out
+
+
+def bench_generation(args):
+    """Transformer-big beam search (batch 16 x beam 4, source 64, 64 steps) or
+    GPT-2-medium greedy generation (batch 16, prompt 512, 128 new tokens)."""
+    import numpy as np
+    import torch
+    from lightseq_amd import inference, synthetic
+    tmp = tempfile.mkdtemp(prefix="ls_bench_")
+    if args.workload == "transformer_big":
+        cfg = synthetic.transformer_config("transformer_big")
+        src_len, steps_wanted, batch = 64, 64, 16
+        # decoding runs min(max_step, src + extra) - 2 steps
+        cfg.update(max_step=128, extra_decode_length=steps_wanted + 2 - src_len)
+        path = os.path.join(tmp, "quant_transformer_big.pb")
+        synthetic.write_quant_transformer(path, cfg, seed=0)
+        ids, _ = synthetic.make_token_ids(dict(vocab=cfg["src_vocab"], padding_id=0), batch, src_len,
+                                          seed=0, min_len=src_len)
+        model = inference.QuantTransformer(path, batch)
+        entry = "QuantTransformer / LSModel::Infer"
+        desc = ("Transformer-big-shaped int8 encoder-decoder, beam search: hidden 1024, 16 heads, "
+                "FFN 4096 ReLU, 6+6 layers, batch 16 x beam 4, source length 64, 64 decode steps, "
+                "vocab 32000, random-init weights")
+    else:
+        cfg = synthetic.gpt_config("gpt2_medium")
+        src_len, steps_wanted, batch = 512, 128, 16
+        path = os.path.join(tmp, "quant_gpt2_medium.pb")
+        synthetic.write_quant_gpt(path, cfg, seed=0)
+        rng = np.random.default_rng(0)
+        ids = rng.integers(0, cfg["vocab"] - 1, size=(batch, src_len), dtype=np.int32)
+        model = inference.QuantGpt(path, batch)
+        entry = "QuantGpt / LSModel::Infer"
+        desc = ("GPT-2-medium-shaped int8 decoder-only generation: 24 layers, hidden 1024, 16 heads, "
+                "FFN 4096 GELU, pre-LN, vocab 50257, batch 16, prompt 512, 128 generated tokens, "
+                "greedy, random-init weights")
+    os.remove(path)
+    model.benchmark_mode(True)
+    model._upload(ids)
+    for _ in range(args.warmup):
+        model.infer_device()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.infer_device()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    steps_run = model.steps_run()
     model.close()
+    gen_tokens = batch * steps_run
+    return {
+        "metric": "generated tokens/sec (%s)" % args.workload,
+        "value": gen_tokens * args.steps / dt, "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": 1e3 * dt / args.steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": desc, "batch": batch, "source_len": src_len,
+                   "decode_steps": steps_run, "ms_per_decode_step": 1e3 * dt / args.steps / steps_run,
+                   "entry_point": entry},
+        "roofline": None,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default="bert_base",
+                    choices=["bert_base", "transformer_big", "gpt2_medium"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fused", action="store_true",
+                    help="skip the stand-alone timing of the fused kernels")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU only (every model object owns device 0 and "
+                 "one stream, as in the reference); --gpus %d is not supported" % args.gpus)
+    bert = args.workload == "bert_base"
+    if args.steps is None:
+        args.steps = 50 if bert else 3
+    if args.warmup is None:
+        args.warmup = 10 if bert else 1
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    out = bench_bert(args) if bert else bench_generation(args)
     print(json.dumps(out))
 
 
