@@ -102,14 +102,23 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ float round_h(float x) { return (float)(_Float16)x; }
 
-// GPT = true turns the kernel into the causal prompt attention of the int8 GPT path
+// MODE 1 turns the kernel into the causal prompt attention of the int8 GPT path
 // (inference/model/quant_gpt_encoder.cc.cu:498-523 with
 // inference/kernels/gptKernels_int8.cc.cu:192-222): q and k hold int8 codes as fp16
 // values, so the fp32 MFMA accumulators are the exact int32 scores; a score becomes
 // float(acc) * alpha * dq * dq without fp16 rounding, key j is visible to query i when
 // j <= i, `pad_mask` is the per-sequence real length and queries at or beyond it give
 // zeros.  Key blocks entirely to the right of the query block are skipped.
-template <int D, bool GPT>
+//
+// MODE 2 is the attention core of the csrc encoder layer
+// (csrc/layers/transformer_encoder_layer.cpp:121-135 with
+// csrc/kernels/cuda/softmax_kernels.cu:35-279): `pad_mask` points to the layer's additive
+// T=half mask [batch, S] (0 for tokens, a large negative value for padding), no query row
+// is zeroed, a non-zero `dq` masks future keys, and the context is written with the heads
+// merged, fp16 [batch, S, head_num * D].
+constexpr int kAttnEnc = 0, kAttnGpt = 1, kAttnLayer = 2;
+
+template <int D, int MODE>
 __global__ void __launch_bounds__(128)
 encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
                     const __half* __restrict__ v, const int* __restrict__ pad_mask,
@@ -121,6 +130,9 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   __shared__ _Float16 Ks[128 * KSTR];
   __shared__ _Float16 Vt[D * VSTR];
   __shared__ int msk[128];
+  __shared__ float addm[MODE == kAttnLayer ? 128 : 1];
+  constexpr bool GPT = MODE == kAttnGpt;
+  const bool causal = GPT || (MODE == kAttnLayer && dq != 0.f);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, g = lane >> 5;
@@ -139,7 +151,9 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
     else
       qreg[ks] = (v8h)(_Float16)0;
   }
-  const bool q_pad = qi >= S || (GPT ? qi >= pad_mask[b] : pad_mask[(long)b * S + qi] != 0);
+  const bool q_pad = qi >= S || (MODE == kAttnLayer ? false
+                                 : GPT              ? qi >= pad_mask[b]
+                                                    : pad_mask[(long)b * S + qi] != 0);
 
   float m = kFloatInfNeg, sum = 0.f;
   v16f sc[4];
@@ -150,7 +164,7 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
   int nkb = (S + 127) / 128;
-  if (GPT) nkb = min(nkb, min((int)blockIdx.x * 64 + 63, S - 1) / 128 + 1);
+  if (causal) nkb = min(nkb, min((int)blockIdx.x * 64 + 63, S - 1) / 128 + 1);
   for (int phase = 0; phase < 2; ++phase) {
     for (int kb = 0; kb < nkb; ++kb) {
       const int key0 = kb * 128;
@@ -172,10 +186,16 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
             for (int i = 0; i < 8; ++i) Vt[(ch * 8 + i) * VSTR + row] = vv[i];
           }
         }
-        if (GPT)
+        if (MODE == kAttnLayer) {
           msk[tid] = (key0 + tid < S) ? 0 : 1;
-        else
+          addm[tid] = (key0 + tid < S && pad_mask != nullptr)
+                          ? __half2float(reinterpret_cast<const __half*>(pad_mask)[(long)b * S + key0 + tid])
+                          : 0.f;
+        } else if (GPT) {
+          msk[tid] = (key0 + tid < S) ? 0 : 1;
+        } else {
           msk[tid] = (key0 + tid < S) ? pad_mask[(long)b * S + key0 + tid] : 1;
+        }
         __syncthreads();
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb) {
@@ -190,11 +210,17 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             const int key_local = sb * 32 + 8 * (i / 4) + 4 * g + (i % 4);
-            if (GPT)
+            if (MODE == kAttnLayer) {
+              float t = round_h(alpha * c[i]) + addm[key_local];
+              if (msk[key_local] || (causal && key0 + key_local > qi) || !(t > 0.5f * kFloatInfNeg))
+                t = kFloatInfNeg;
+              sc[sb][i] = t;
+            } else if (GPT) {
               sc[sb][i] = (msk[key_local] || key0 + key_local > qi) ? kFloatInfNeg
                                                                     : c[i] * alpha * dq * dq;
-            else
+            } else {
               sc[sb][i] = msk[key_local] ? kFloatInfNeg : round_h(alpha * c[i]);
+            }
           }
         }
       }
@@ -255,7 +281,10 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         half4_t t;
 #pragma unroll
         for (int j = 0; j < 4; ++j) t.v[j] = __float2half_rn(o[j]);
-        *reinterpret_cast<half4_t*>(ctx + ((long)bh * S + qi) * D + dd) = t;
+        if (MODE == kAttnLayer)
+          *reinterpret_cast<half4_t*>(ctx + tok * hidden + head * D + dd) = t;
+        else
+          *reinterpret_cast<half4_t*>(ctx + ((long)bh * S + qi) * D + dd) = t;
       }
       if (ctx_q != nullptr) {
         *reinterpret_cast<uint32_t*>(ctx_q + tok * hidden + head * D + dd) =
@@ -281,17 +310,17 @@ int encself_attention_f16(const __half* q, const __half* k, const __half* v, con
   dim3 grid((seq_len + 63) / 64, batch * head_num);
   switch (dim_per_head) {
     case 32:
-      encself_attn_kernel<32, false><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
+      encself_attn_kernel<32, kAttnEnc><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
                                                           quant_scale, seq_len, head_num, alpha,
                                                           0.f);
       break;
     case 64:
-      encself_attn_kernel<64, false><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
+      encself_attn_kernel<64, kAttnEnc><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
                                                           quant_scale, seq_len, head_num, alpha,
                                                           0.f);
       break;
     case 128:
-      encself_attn_kernel<128, false><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
+      encself_attn_kernel<128, kAttnEnc><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
                                                            quant_scale, seq_len, head_num, alpha,
                                                            0.f);
       break;
@@ -318,17 +347,17 @@ int gpt_prefill_attention_f16(const __half* q_codes, const __half* k_codes, cons
   dim3 grid((seq_len + 63) / 64, batch * head_num);
   switch (dim_per_head) {
     case 32:
-      encself_attn_kernel<32, true><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
+      encself_attn_kernel<32, kAttnGpt><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
                                                          ctx_q, quant_scale, seq_len, head_num,
                                                          alpha, dequant_scale);
       break;
     case 64:
-      encself_attn_kernel<64, true><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
+      encself_attn_kernel<64, kAttnGpt><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
                                                          ctx_q, quant_scale, seq_len, head_num,
                                                          alpha, dequant_scale);
       break;
     case 128:
-      encself_attn_kernel<128, true><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
+      encself_attn_kernel<128, kAttnGpt><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
                                                           ctx_q, quant_scale, seq_len, head_num,
                                                           alpha, dequant_scale);
       break;
@@ -337,6 +366,42 @@ int gpt_prefill_attention_f16(const __half* q_codes, const __half* k_codes, cons
                       "gpt_prefill_attention: dim_per_head must be 32, 64 or 128");
   }
   return lsh_check_launch("encself_attn_kernel<GPT>");
+}
+
+// Attention core of the csrc encoder layer: q, k, v fp16 [batch, heads, S, D], additive
+// fp16 mask [batch, S] (may be null), context fp16 [batch, S, heads * D].
+int layer_attention_f16(const __half* q, const __half* k, const __half* v, const __half* add_mask,
+                        __half* ctx, int batch, int seq_len, int head_num, int dim_per_head,
+                        bool mask_future, hipStream_t s) {
+  if (batch <= 0 || seq_len <= 0 || head_num <= 0 || !q || !k || !v || !ctx)
+    return lsh_fail(LSH_ERR_INVALID, "layer_attention: bad arguments");
+  if (seq_len > 1024) return lsh_fail(LSH_ERR_UNSUPPORTED, "layer_attention: seq_len > 1024");
+  if (((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
+        reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(ctx)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_INVALID, "layer_attention: pointers must be 16-byte aligned");
+  // strided_batch_gemm alpha: T(1.0) / T(sqrt(d)) (transformer_encoder_layer.cpp:48-50)
+  const float alpha = __half2float(
+      __float2half_rn(1.0f / __half2float(__float2half_rn(sqrtf((float)dim_per_head)))));
+  const int* m = reinterpret_cast<const int*>(add_mask);
+  const float causal = mask_future ? 1.f : 0.f;
+  dim3 grid((seq_len + 63) / 64, batch * head_num);
+  switch (dim_per_head) {
+    case 32:
+      encself_attn_kernel<32, kAttnLayer><<<grid, 128, 0, s>>>(q, k, v, m, ctx, nullptr, 0.f,
+                                                               seq_len, head_num, alpha, causal);
+      break;
+    case 64:
+      encself_attn_kernel<64, kAttnLayer><<<grid, 128, 0, s>>>(q, k, v, m, ctx, nullptr, 0.f,
+                                                               seq_len, head_num, alpha, causal);
+      break;
+    case 128:
+      encself_attn_kernel<128, kAttnLayer><<<grid, 128, 0, s>>>(q, k, v, m, ctx, nullptr, 0.f,
+                                                                seq_len, head_num, alpha, causal);
+      break;
+    default:
+      return lsh_fail(LSH_ERR_UNSUPPORTED, "layer_attention: dim_per_head must be 32, 64 or 128");
+  }
+  return lsh_check_launch("encself_attn_kernel<layer>");
 }
 
 }  // namespace lsh

@@ -98,6 +98,23 @@ struct EpiI8 {
   static const char* name() { return "EpiI8"; }
 };
 
+// The same with the scale read from device memory (the csrc layers keep their clip values
+// and the alpha derived from them on the device: csrc/kernels/cuda/cublas_wrappers.cpp:134
+// CUBLASLT_POINTER_MODE_DEVICE).
+struct EpiI8Dev {
+  int8_t* C;
+  const float* alpha;
+  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
+    const float a = alpha[0];
+    int q[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) q[i] = requant_acc(c[i], a);
+    store16_i8(C + m * N + n, n, N, q, full);
+  }
+  bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
+  static const char* name() { return "EpiI8Dev"; }
+};
+
 // requantise to the GEMM's int8 output code, then dequant + bias + activation +
 // requant exactly as the stand-alone bias/activation kernel would on that code.
 template <int ACT>
@@ -504,6 +521,12 @@ int gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K
                 hipStream_t s) {
   if (!C) return lsh_fail(LSH_ERR_INVALID, "int8 gemm: null output");
   return dispatch(A, W, EpiI8{C, alpha}, M, N, K, s);
+}
+
+int gemm_i8_i8o_dev_alpha(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K,
+                          const float* alpha, hipStream_t s) {
+  if (!C || !alpha) return lsh_fail(LSH_ERR_INVALID, "int8 gemm: null output or alpha");
+  return dispatch(A, W, EpiI8Dev{C, alpha}, M, N, K, s);
 }
 
 int gemm_i8_bias_act_i8o(const int8_t* A, const int8_t* W, int8_t* C, const __half* bias, int M,

@@ -233,6 +233,58 @@ int ppl_i8I(int batch_size, int batch_seq_len, hipStream_t s, const int8_t* logi
             const int* input_ids, const int* real_seq_len, float* ppl, int vocab_size,
             float dequant_scale);
 
+// ---- operator kernels of the csrc layer path (layer_ops.hip); clip values are device
+// ---- scalars of type T, dropout ratios must be 0 -------------------------------------
+template <typename T>
+int opb_quantize(int8_t* q, uint8_t* cmask, float* alpha, const T* f, const T* cmax, long numel,
+                 int alpha_count, int bit, hipStream_t s);
+template <typename T>
+int opb_fake_quantize(uint8_t* cmask, float* alpha, T* out, const T* in, const T* cmax,
+                      long numel, int bit, bool symmetry, hipStream_t s);
+template <typename T>
+int opb_dequantize(T* f, const int8_t* q, const T* cmax, long numel, hipStream_t s);
+// q_out != nullptr selects the quantising variant
+template <typename T>
+int opb_layer_norm(T* ln_res, int8_t* q_out, uint8_t* cmask, T* vars, T* means, const T* inp,
+                   const T* gamma, const T* beta, const T* cmax_out, int rows, int hidden,
+                   hipStream_t s);
+template <typename T>
+int opb_attn_softmax(T* vals, const T* mask, int batch, int heads, int from_len, int to_len,
+                     bool mask_future, hipStream_t s);
+template <typename T>
+int opb_quant_bias_add_transform_20314(T* out, uint8_t* cmask, const int8_t* in, const T* bias,
+                                       const T* cmax, int d0, int d1, int d2, int d3, int d4,
+                                       hipStream_t s, const T* out_cmax);
+// out_q != nullptr selects the quantising variant
+template <typename T>
+int opb_transform4d_0213(T* out, int8_t* out_q, uint8_t* cmask, const T* vals, const T* cmax,
+                         int batch, int seq, int hidden, int nhead, int tc, hipStream_t s);
+template <typename T>
+int opb_dropout(T* out, const T* vals, uint8_t* mask, long total, float ratio, hipStream_t s);
+template <typename T>
+int opb_dropout_res_bias(T* out, const T* vals, uint8_t* mask, const T* bias, const T* residual,
+                         long total, int dim, float ratio, hipStream_t s);
+// act: 0 gelu, 1 relu
+template <typename T>
+int opb_dropout_act_bias(int act, T* out, const T* vals, uint8_t* mask, const T* bias, long total,
+                         int dim, float ratio, hipStream_t s);
+// qout != nullptr: int8 result; else fout receives the fake-quantised T result
+template <typename T>
+int opb_quant_dropout_act_bias(int act, int8_t* qout, T* fout, uint8_t* cmask_out,
+                               uint8_t* cmask_in, uint8_t* dropout_mask, const int8_t* qin,
+                               const T* bias, const T* cmax_out, const T* cmax_in, long total,
+                               int dim, float ratio, bool symmetry, hipStream_t s);
+template <typename T>
+int opb_quant_dropout_res_bias(T* out, uint8_t* mask, const int8_t* qvals, const T* cmax,
+                               const T* bias, const T* residual, long total, int dim, float ratio,
+                               hipStream_t s);
+// int8 GEMM to int8 with the scale read from device memory (alpha[0])
+int gemm_i8_i8o_dev_alpha(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K,
+                          const float* alpha, hipStream_t s);
+int layer_attention_f16(const __half* q, const __half* k, const __half* v, const __half* add_mask,
+                        __half* ctx, int batch, int seq_len, int head_num, int dim_per_head,
+                        bool mask_future, hipStream_t s);
+
 // inference/kernels/transformerKernels.h:137-140
 inline float length_norm(int length, float alpha) {
   if (alpha < 0.f) return 1.f / length;

@@ -25,9 +25,10 @@ class LSHError(RuntimeError):
 
 
 _P, _I, _F, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
-_CODES = {"p": _P, "s": _P, "i": _I, "f": _F, "l": _L}
+_CODES = {"p": _P, "s": _P, "i": _I, "f": _F, "l": _L, "c": ctypes.c_char_p}
 
-# name -> (has _f16/_f32 variants, argument codes).  p pointer, s stream, i int, f float
+# name -> (has _f16/_f32 variants, argument codes).  p pointer, s stream, i int, f float,
+# l int64_t, c C string
 _SIGNATURES = {
     "lsh_launch_quantize_tensor": (True, "ppiifsi"),
     "lsh_launch_dequantize_tensor": (True, "ppiifsi"),
@@ -82,6 +83,36 @@ _SIGNATURES = {
     "lsh_gpt_arrange_qkv_prefill_f16": (False, "iis" + "ppppppp" + "iiii" + "ff"),
     "lsh_gpt_prefill_attention_f16": (False, "pppppp" + "ff" + "iiii" + "s"),
     "lsh_gpt_greedy_step": (False, "ppp" + "iiii" + "p" + "i" + "s"),
+    # operator launchers of the csrc layer path (include/lightseq_ops.h)
+    "lsh_launch_quantize": (True, "ppppp" + "ii" + "s"),
+    "lsh_launch_quantize_2d": (True, "ppppp" + "iii" + "s" + "i"),
+    "lsh_launch_fake_quantize": (True, "ppppp" + "ii" + "s" + "i"),
+    "lsh_launch_dequantize": (True, "ppp" + "ii" + "s"),
+    "lsh_launch_layer_norm": (True, "pppppp" + "ii" + "s"),
+    "lsh_launch_layer_norm_i8": (True, "pppppppp" + "ii" + "s"),
+    "lsh_launch_attn_softmax": (True, "pp" + "iiiii" + "s"),
+    "lsh_launch_quant_bias_add_transform_20314": (True, "ppppp" + "iiiii" + "s" + "p" + "i"),
+    "lsh_launch_transform4d_0213": (True, "pp" + "iiiii" + "s"),
+    "lsh_launch_quant_transform4d_0213": (True, "pppp" + "iiiii" + "s"),
+    "lsh_launch_ls_dropout": (True, "ppp" + "if" + "s" + "i"),
+    "lsh_launch_ls_dropout_res_bias": (True, "ppppp" + "iif" + "s"),
+    "lsh_launch_ls_dropout_act_bias_gelu": (True, "pppp" + "iif" + "s"),
+    "lsh_launch_ls_dropout_act_bias_relu": (True, "pppp" + "iif" + "s"),
+    "lsh_launch_ls_quant_dropout_act_bias_gelu": (True, "pppppppp" + "iif" + "s"),
+    "lsh_launch_ls_quant_dropout_act_bias_relu": (True, "pppppppp" + "iif" + "s"),
+    "lsh_launch_ls_fakequant_dropout_act_bias_gelu": (True, "pppppppp" + "iif" + "s" + "ii"),
+    "lsh_launch_ls_fakequant_dropout_act_bias_relu": (True, "pppppppp" + "iif" + "s" + "ii"),
+    "lsh_launch_ls_quant_dropout_res_bias": (True, "pppppp" + "iif" + "s" + "i"),
+    "lsh_feed_forward_i8": (False, "iii" + "ppppp" + "s"),
+    "lsh_layer_attention_f16": (False, "ppppp" + "iiiii" + "s"),
+    # layer interface
+    "ls_layer_set_stream": (False, "s"),
+    "ls_create_transformer_encoder_layer_fp16": (False, "iiiiii" + "fff" + "i" + "c" + "i"),
+    "ls_transformer_encoder_layer_fw_fp16": (False, "i" + "ppp" + "iiiii"),
+    "ls_assign_layer_weight_grad_fp16": (False, "pp" + "c" + "i"),
+    "ls_create_quant_linear_layer_fp16": (False, "iiii"),
+    "ls_quant_linear_layer_fw_fp16": (False, "i" + "pppp" + "iii"),
+    "ls_destroy_layer": (False, "c" + "i"),
 }
 
 _lib = None

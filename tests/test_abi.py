@@ -8,8 +8,8 @@ import re
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("lightseq_hip.h", "lightseq_model.h")]
-PROTO_RE = re.compile(r"^\s*(?:const\s+char\s*\*|int|float)\s+((?:lsh|ls_model)_\w+)\s*\(([^;]*?)\)\s*;",
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("lightseq_hip.h", "lightseq_ops.h", "lightseq_model.h")]
+PROTO_RE = re.compile(r"^\s*(?:const\s+char\s*\*|int|float)\s+((?:lsh|ls)_\w+)\s*\(([^;]*?)\)\s*;",
                       re.M | re.S)
 
 
@@ -26,6 +26,8 @@ def _code(arg):
     arg = arg.strip()
     if arg == "void":
         return ""
+    if re.match(r"const\s+char\s*\*", arg):
+        return "c"
     if "*" in arg:
         return "p"
     if arg.startswith("lsh_stream_t"):
@@ -63,9 +65,10 @@ def test_ctypes_table_matches_header():
             assert full in protos, full
             want = "".join(_code(a) for a in protos[full].split(","))
             assert want == codes, (full, want, codes)
-    # and nothing in lightseq_hip.h is left unbound
+    # and nothing in lightseq_hip.h / lightseq_ops.h is left unbound
     bound = {n + s for n, (t, _) in lib._SIGNATURES.items() for s in (("_f16", "_f32") if t else ("",))}
-    kernels_header = re.sub(r"/\*.*?\*/", "", open(HEADERS[0]).read(), flags=re.S)
+    kernels_header = re.sub(r"/\*.*?\*/", "", open(HEADERS[0]).read() + open(HEADERS[1]).read(),
+                            flags=re.S)
     declared = {n for n, _ in PROTO_RE.findall(kernels_header)} - {"lsh_last_error", "lsh_version",
                                                                          "lsh_length_norm"}
     assert declared == bound, declared ^ bound
