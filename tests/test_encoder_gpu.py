@@ -83,6 +83,56 @@ def test_transformer_base_layer_config(tmp_path, oracle):
     model.close()
 
 
+def test_transformer_base_layer_vs_quantisation_aware_layer(tmp_path, oracle):
+    """The same single layer against the float quantisation-aware layer the int8 engine is
+    exported from (training/ops/pytorch/torch_transformer_layers.py:537-679), restated in
+    oracle/qat.py.  In a post-LN model file the layer norms are rotated by one position
+    (examples/inference/python/export/huggingface/ls_torch_hf_quant_bert_export.py:159-177):
+    "multihead_norm" of layer 0 is the embedding layer norm, "ffn_norm" follows the attention
+    block and the norm stored with the embedding closes the layer.  The engine does not
+    quantise the fc2 output, so that quantiser of the module is off."""
+    from lightseq_amd import inference, synthetic
+    from oracle import qat
+    cfg, msg, path = _build(tmp_path, "transformer_base_layer", 0)
+    ids, _ = synthetic.make_token_ids(cfg, 8, 64, seed=0, min_len=64)
+    H, I = cfg["hidden"], cfg["inner"]
+    emb, l = msg["src_embedding"], msg["encoder_stack"][0]
+
+    def weight(name, rows, cols):
+        clip = np.float32(l[name + "_clip_max"])
+        codes = np.asarray(l[name], np.int32).reshape(rows, cols) - 127
+        return np.ascontiguousarray((codes.astype(np.float32) * (clip / np.float32(127))).T)
+
+    f = lambda v: np.asarray(v, np.float32)
+    p = {"qkv_w": weight("multihead_project_kernel_qkv", H, 3 * H),
+         "qkv_b": f(l["multihead_project_bias_qkv"]),
+         "out_w": weight("multihead_project_kernel_output", H, H),
+         "out_b": f(l["multihead_project_bias_output"]),
+         "ln1_w": f(l["ffn_norm_scale"]), "ln1_b": f(l["ffn_norm_bias"]),
+         "fc1_w": weight("ffn_first_kernel", H, I), "fc1_b": f(l["ffn_first_bias"]),
+         "fc2_w": weight("ffn_second_kernel", I, H), "fc2_b": f(l["ffn_second_bias"]),
+         "ln2_w": f(emb["norm_scale"]), "ln2_b": f(emb["norm_bias"])}
+    amax = {"qkv_in": l["multihead_ln_clip_max"], "qkv_w": l["multihead_project_kernel_qkv_clip_max"],
+            "qkv_out": l["multihead_qkv_dense_clip_max"],
+            "out_in": l["multihead_project_output_clip_max"],
+            "out_w": l["multihead_project_kernel_output_clip_max"],
+            "out_out": l["multihead_output_dense_clip_max"], "fc1_in": l["ffn_ln_clip_max"],
+            "fc1_w": l["ffn_first_kernel_clip_max"], "fc1_out": l["ffn_first_output_clip_max"],
+            "fc2_in": l["ffn_first_act_clip_max"], "fc2_w": l["ffn_second_kernel_clip_max"],
+            "fc2_out": 0.0}
+    tok = (np.asarray(emb["token_embedding"], np.float32).reshape(cfg["vocab"], H) - 127) * (
+        np.float32(emb["emb_clip_max"]) / 127)
+    x0 = tok[ids] + f(emb["position_embedding"]).reshape(cfg["max_step"], H)[None, :64]
+    x = qat.layer_norm(x0, f(l["multihead_norm_scale"]), f(l["multihead_norm_bias"]), eps=1e-12)
+    want = qat.encoder_layer(x, p, amax, cfg["head_num"], False, "relu", None,
+                             fc2_output_quant=False)
+    model = inference.QuantBert(path, 8)
+    got = model.infer(ids)
+    model.close()
+    d = np.abs(got.astype(np.float64) - want)
+    assert d.max() < 2e-2, (d.max(), d.mean())
+
+
 TAP_SPECS = [("ln1_q", "H", "i8"), ("qkv_q", "3H", "i8"), ("ctx_q", "H", "i8"), ("out_q", "H", "i8"),
              ("ln2_q", "H", "i8"), ("ffn1_q", "I", "i8"), ("act_q", "I", "i8"), ("ffn2_acc", "H", "i32"),
              ("res_attn", "H", "f16"), ("res_ffn", "H", "f16")]
