@@ -192,6 +192,97 @@ decself_attn_kernel(int32_t* __restrict__ scores, const int8_t* __restrict__ q,
   }
 }
 
+// The fused form at decode sizes: one workgroup (4 wavefronts) per (row, head).  A cached
+// key or value row of d bytes is read by d/16 adjacent lanes with one 16-byte load each, so a
+// wavefront covers 1024 contiguous bytes of cache per load instruction and every byte of
+// the cache is read once.  Scores are exact int32 dot products (v_dot4), probabilities live
+// in LDS, the value sum is accumulated per lane over its share of the steps and then reduced
+// across lanes (shuffles) and wavefronts (LDS): a tree instead of the ascending-step order
+// of the kernel above, so a context code can differ by one from it where the float sum
+// lands next to a rounding boundary.  Requires d in {32, 64, 128} and 16-byte aligned rows.
+template <int D>
+__global__ void __launch_bounds__(256)
+decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k_cache,
+                       const int8_t* __restrict__ v_cache, int8_t* __restrict__ new_v,
+                       int step_num, int max_step, int head_num, float attn_scale, float dq,
+                       float quant_scale) {
+#pragma clang fp contract(off)
+  constexpr int CH = D / 16;    // lanes per cache row
+  constexpr int KPW = 64 / CH;  // rows per wavefront per load
+  extern __shared__ float lds_f[];
+  const int padded = (step_num + 63) & ~63;
+  float* probs = lds_f;                 // [padded]
+  float* red = lds_f + padded;          // [16] block reductions
+  float* part = red + 16;               // [4][D] per-wavefront value sums
+  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+  const long bh = blockIdx.x;
+  const int c = lane % CH, grp = lane / CH;
+  const int8_t* kb = k_cache + bh * (long)max_step * D;
+  const int8_t* vb = v_cache + bh * (long)max_step * D;
+  const uint4 qv = *reinterpret_cast<const uint4*>(q + bh * D + c * 16);
+
+  // scores -> scaled logits in LDS
+  float mx = kFloatInfNeg;
+  for (int j0 = wid * KPW; j0 < step_num; j0 += 4 * KPW) {
+    const int j = j0 + grp;
+    int sc = 0;
+    if (j < step_num) {
+      const uint4 kv = *reinterpret_cast<const uint4*>(kb + (long)j * D + c * 16);
+      sc = __builtin_amdgcn_sdot4((int)qv.x, (int)kv.x, sc, false);
+      sc = __builtin_amdgcn_sdot4((int)qv.y, (int)kv.y, sc, false);
+      sc = __builtin_amdgcn_sdot4((int)qv.z, (int)kv.z, sc, false);
+      sc = __builtin_amdgcn_sdot4((int)qv.w, (int)kv.w, sc, false);
+    }
+#pragma unroll
+    for (int m = 1; m < CH; m <<= 1) sc += __shfl_xor(sc, m, 64);
+    if (j < step_num) {
+      const float val = (float)sc * dq * dq * attn_scale;
+      if (c == 0) probs[j] = val;
+      mx = fmaxf(mx, val);
+    }
+  }
+  mx = block_max(mx, red);
+  float sum = 0.f;
+  for (int j = tid; j < step_num; j += 256) {
+    const float e = __expf(probs[j] - mx);
+    probs[j] = e;
+    sum += e;
+  }
+  sum = block_sum(sum, red);
+  for (int j = tid; j < step_num; j += 256) probs[j] = probs[j] / sum;
+  __syncthreads();
+
+  // value sum: lane (grp, c) accumulates dims [16c, 16c+16) over steps grp, grp + KPW*4, ...
+  float acc[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) acc[k] = 0.f;
+  for (int j0 = wid * KPW; j0 < step_num; j0 += 4 * KPW) {
+    const int j = j0 + grp;
+    if (j < step_num) {
+      const uint4 vv = *reinterpret_cast<const uint4*>(vb + (long)j * D + c * 16);
+      const float p = probs[j];
+      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+      for (int k = 0; k < 16; ++k) acc[k] += (float)unpack_i8(w[k >> 2], k & 3) * p * dq;
+    }
+  }
+#pragma unroll
+  for (int m = CH; m < 64; m <<= 1)
+#pragma unroll
+    for (int k = 0; k < 16; ++k) acc[k] += __shfl_xor(acc[k], m, 64);
+  if (grp == 0) {
+#pragma unroll
+    for (int k = 0; k < 16; ++k) part[wid * D + c * 16 + k] = acc[k];
+  }
+  __syncthreads();
+  if (tid < D) {
+    const float v = (part[tid] + part[D + tid]) + (part[2 * D + tid] + part[3 * D + tid]);
+    const long row = bh / head_num;
+    const int head = (int)(bh % head_num);
+    new_v[row * ((long)head_num * D) + (long)head * D + tid] = (int8_t)float2int8(v, quant_scale);
+  }
+}
+
 static int decself_check(long bh_total, int step_num, int max_step, int head_num, int d) {
   if (bh_total <= 0 || head_num <= 0 || d <= 0 || max_step <= 0)
     return lsh_fail(LSH_ERR_INVALID, "decoder self attention: bad shape");
@@ -234,6 +325,21 @@ int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v
   if (!q || !k_cache || !v_cache || !new_v)
     return lsh_fail(LSH_ERR_INVALID, "decself_attention: null pointer");
   if (int rc = decself_check(batch_head_num, step_num, max_step, head_num, dim_per_head)) return rc;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
+                         reinterpret_cast<uintptr_t>(v_cache)) & 15u) == 0;
+  if (aligned && (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128)) {
+    const size_t lds = ((size_t)((step_num + 63) & ~63) + 16 + 4 * dim_per_head) * sizeof(float);
+#define LSH_DECSELF(D)                                                                          \
+  decself_attn_wg_kernel<D><<<batch_head_num, 256, lds, s>>>(q, k_cache, v_cache, new_v,         \
+                                                             step_num, max_step, head_num,      \
+                                                             attn_scale, dequant_scale,         \
+                                                             quant_scale)
+    if (dim_per_head == 32) LSH_DECSELF(32);
+    else if (dim_per_head == 64) LSH_DECSELF(64);
+    else LSH_DECSELF(128);
+#undef LSH_DECSELF
+    return lsh_check_launch("decself_attn_wg_kernel");
+  }
   decself_attn_kernel<2><<<(batch_head_num + 3) / 4, 256, decself_lds(step_num), s>>>(
       nullptr, q, k_cache, v_cache, new_v, batch_head_num, step_num, max_step, head_num,
       dim_per_head, attn_scale, dequant_scale, quant_scale);

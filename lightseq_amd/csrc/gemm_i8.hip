@@ -447,6 +447,80 @@ gemm_i8_generic_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------------
+// Decode-step path: M <= 64 rows (batch x beam of one generation step).  The product is
+// bound by streaming the weight matrix once from HBM, so the kernel is organised around
+// that stream: one workgroup owns 32 output columns (32 weight rows of K bytes, a contiguous
+// slab), its 4 wavefronts take the 128-byte K chunks round-robin, and every lane loads its
+// MFMA operands straight from global memory -- 64 contiguous bytes of one weight row per
+// chunk -- with all loads of a chunk pair in flight before the MFMAs.  There is no LDS
+// staging (each weight byte is used by exactly one wavefront) and no tile loop; the partial
+// accumulators of the 4 wavefronts meet in LDS and go through the same epilogues.
+// Preconditions: K % 128 == 0, operands 16-byte aligned.
+// ---------------------------------------------------------------------------------
+template <typename Epi, int MBLK>
+__global__ void __launch_bounds__(256)
+gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
+                      int N, int K, int, int, bool vec_store) {
+  __shared__ int red[4][MBLK][16][64];  // [wavefront][m block][register][lane]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  const int n0 = blockIdx.x * 32;
+  const int8_t* wp = W + (long)min(n0 + sigma(l32), N - 1) * K + g * 64;
+  const int8_t* ap[MBLK];
+#pragma unroll
+  for (int i = 0; i < MBLK; ++i) ap[i] = A + (long)min(i * 32 + l32, M - 1) * K + g * 64;
+  v16i acc[MBLK];
+#pragma unroll
+  for (int i = 0; i < MBLK; ++i) acc[i] = (v16i)0;
+  const int nch = K / kBK;
+  for (int ch = wave; ch < nch; ch += 8) {
+    const int k0 = ch * kBK;
+    const bool two = ch + 4 < nch;
+    const int k1 = two ? k0 + 4 * kBK : k0;
+    v4i wv[2][4], av[2][MBLK][4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      wv[0][ks] = *reinterpret_cast<const v4i*>(wp + k0 + ks * 16);
+      wv[1][ks] = *reinterpret_cast<const v4i*>(wp + k1 + ks * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < MBLK; ++i)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        av[0][i][ks] = *reinterpret_cast<const v4i*>(ap[i] + k0 + ks * 16);
+        av[1][i][ks] = *reinterpret_cast<const v4i*>(ap[i] + k1 + ks * 16);
+      }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int i = 0; i < MBLK; ++i)
+        acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv[0][ks], av[0][i][ks], acc[i], 0, 0, 0);
+    if (two) {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int i = 0; i < MBLK; ++i)
+          acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv[1][ks], av[1][i][ks], acc[i], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MBLK; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[wave][i][r][lane] = acc[i][r];
+  __syncthreads();
+  if (wave < MBLK) {
+    v16i c;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      c[r] = (red[0][wave][r][lane] + red[1][wave][r][lane]) +
+             (red[2][wave][r][lane] + red[3][wave][r][lane]);
+    const long m = wave * 32 + l32;
+    const int n = n0 + 16 * g;
+    if (m < M && n < N) epi.store16(m, n, N, c, vec_store && n + 16 <= N);
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------
 static thread_local hipEvent_t g_ev_start = nullptr, g_ev_stop = nullptr;
@@ -497,6 +571,15 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   const int tiles = tiles_m * tiles_n;
   const size_t smem = 2 * (size_t)(kBM + kBN) * kBK;
   static bool attr_stream = false, attr_generic = false;  // per Epi instantiation
+  static bool attr_skinny = true;                          // static LDS: nothing to set
+  if (M <= 64 && K % kBK == 0) {
+    const int grid = (N + 31) / 32;
+    if (M <= 32)
+      return launch(gemm_i8_skinny_kernel<Epi, 1>, grid, 0, A, W, epi, M, N, K, 0, 0, vec_store, s,
+                    &attr_skinny);
+    return launch(gemm_i8_skinny_kernel<Epi, 2>, grid, 0, A, W, epi, M, N, K, 0, 0, vec_store, s,
+                  &attr_skinny);
+  }
   if (stream_ok(M, N, K)) {
     const int grid = tiles < 512 ? tiles : 512;  // 2 resident workgroups per compute unit
     return launch(gemm_i8_stream_kernel<Epi>, grid, smem, A, W, epi, M, N, K, tiles_m, tiles_n,
@@ -507,6 +590,7 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
 }
 
 std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
+  if (M <= 64 && K % kBK == 0) return std::string("gemm_i8_skinny_kernel<") + epilogue + ">";
   return std::string(stream_ok(M, N, K) ? "gemm_i8_stream_kernel<" : "gemm_i8_generic_kernel<") +
          epilogue + ">";
 }

@@ -88,7 +88,9 @@ def test_arrange_decself_qkv(oracle, rng, dtype, rows, heads, d, max_step, step)
 
 
 @pytest.mark.parametrize("rows,heads,d,max_step,step_num", [(8, 4, 32, 16, 1), (4, 16, 64, 64, 64),
-                                                            (5, 3, 20, 200, 131), (2, 2, 8, 1024, 1000)])
+                                                            (5, 3, 20, 200, 131), (2, 2, 8, 1024, 1000),
+                                                            (16, 16, 64, 640, 577),
+                                                            (3, 4, 128, 256, 200)])
 def test_decself_attention(oracle, rng, rows, heads, d, max_step, step_num):
     q = _codes(rng, (rows, heads * d))
     kc = _codes(rng, (rows, heads, max_step, d))
@@ -113,14 +115,18 @@ def test_decself_attention(oracle, rng, rows, heads, d, max_step, step_num):
                                                       max_step, heads, d, attn_scale, dq, qs)
     assert_codes_close(to_np(out), want, what="fuse_softmax_new_value")
 
-    # the fused kernel reproduces the pair bit for bit
+    # the fused kernel reproduces the pair: bit for bit where it shares the ascending-step
+    # value sum (head sizes off the fast path), to the int8 bar where it sums as a tree
     want2 = torch.zeros_like(out)
     _k().ker_fuse_softmax_new_value_i32I_i8O_launcher(scores, vd, want2, bh, step_num, max_step,
                                                       heads, d, attn_scale, dq / 8, qs)
     fused = torch.zeros_like(out)
     _k().decself_attention_i8(qd, kd, vd, fused, bh, step_num, max_step, heads, d, attn_scale,
                               dq / 8, qs)
-    np.testing.assert_array_equal(to_np(fused), to_np(want2))
+    if d in (32, 64, 128):
+        assert_codes_close(to_np(fused), to_np(want2), what="decself_attention vs pair")
+    else:
+        np.testing.assert_array_equal(to_np(fused), to_np(want2))
     ref2 = oracle.fuse_softmax_new_value_i32I_i8O(want_scores, vc, step_num, attn_scale, dq / 8, qs)
     assert_codes_close(to_np(fused), ref2, what="decself_attention")
 

@@ -17,7 +17,10 @@ SMALL = [(1, 1, 16), (3, 5, 16), (32, 32, 32), (33, 31, 48), (64, 16, 128), (130
          (257, 129, 272), (300, 513, 400), (128, 256, 1024)]
 LARGE = [(4096, 2304, 768), (4096, 768, 768), (4096, 3072, 768), (4096, 768, 3072),
          (512, 1536, 512), (512, 2048, 512), (4096, 4096, 1024), (4096, 1024, 4096),
-         (1000, 30522 // 6, 128), (64, 1000, 1024)]
+         (1000, 30522 // 6, 128), (64, 1000, 1024),
+         # decode-step shapes (rows = batch x beam of one step)
+         (16, 3072, 1024), (16, 1024, 4096), (16, 50257, 1024), (64, 32000, 1024),
+         (64, 4096, 1024), (33, 1000, 256), (1, 64, 128), (48, 40, 384)]
 
 
 def _k():
@@ -100,7 +103,8 @@ def test_gemm_rejects_bad_k():
         _k().gemm_i8_i32o(a, a, c, 4, 4, 8)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 3072, 768), (4096, 3072, 768), (77, 160, 48)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 3072, 768), (4096, 3072, 768), (77, 160, 48),
+                                   (16, 4096, 1024), (64, 4096, 1024)])
 @pytest.mark.parametrize("act", ["gelu", "relu", "relu_narrow"])
 def test_fused_bias_act_epilogue_equals_unfused_pair(rng, M, N, K, act):
     """GEMM + bias/activation/requant in one kernel == int8-output GEMM followed by the
