@@ -211,6 +211,25 @@ int lsh_launch_scaled_colsum_f32(const void* inp, void* out, int rows, int cols,
  * model/cublas_helper.h:50-58 cublaslt_gemm<int32_t,int32_t>. */
 int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n, int k,
                      lsh_stream_t stream);
+/* The int32 product with K split into `ksplit` equal ranges computed by different workgroups
+ * (for shapes whose tile count would leave compute units idle, e.g. the second FFN product):
+ * range p writes the plane C + p * m * n, so C needs ksplit * m * n elements; the planes are
+ * summed by lsh_ker_residual_bias_ln_planes_i32I_i8O_f16 (integer sums: exact).  *used
+ * receives the split actually applied (1 when k does not divide into whole 128-byte steps);
+ * lsh_gemm_i8_preferred_ksplit returns the split the library would choose.  No counterpart
+ * in the reference. */
+int lsh_gemm_i8_i32o_splitk(const int8_t* A, const int8_t* W, int32_t* C, int m, int n, int k,
+                            int ksplit, int* used, lsh_stream_t stream);
+int lsh_gemm_i8_preferred_ksplit(int m, int n, int k);
+/* lsh_ker_residual_bias_ln_i32I_i8O_f16 reading `nparts` accumulator planes `part_stride`
+ * elements apart.  hidden_size % 8 == 0.  No counterpart in the reference. */
+int lsh_ker_residual_bias_ln_planes_i32I_i8O_f16(const int32_t* input, int nparts,
+                                                 int64_t part_stride, const void* scale,
+                                                 const void* bias, const void* residual_bias,
+                                                 int8_t* output, void* residual, int batch_tokens,
+                                                 int hidden_size, float dequant_scale,
+                                                 float quant_scale, lsh_stream_t stream,
+                                                 int is_post_ln, const void* colsum);
 /* int8 out: C = clamp(floor(float(acc) * alpha + 0.5), -127, 127).
  * model/cublas_helper.h:36-48 cublasLtMM_withAlgo_i8IO and
  * model/cublas_helper.h:50-58 cublaslt_gemm<int8_t,float>. */

@@ -322,6 +322,24 @@ int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n,
                      lsh_stream_t stream) {
   return gemm_i8_i32o(A, W, C, m, n, k, HS(stream));
 }
+int lsh_gemm_i8_i32o_splitk(const int8_t* A, const int8_t* W, int32_t* C, int m, int n, int k,
+                            int ksplit, int* used, lsh_stream_t stream) {
+  return gemm_i8_i32o_splitk(A, W, C, m, n, k, ksplit, used, HS(stream));
+}
+int lsh_gemm_i8_preferred_ksplit(int m, int n, int k) { return gemm_i8_preferred_ksplit(m, n, k); }
+int lsh_ker_residual_bias_ln_planes_i32I_i8O_f16(const int32_t* input, int nparts,
+                                                 int64_t part_stride, const void* scale,
+                                                 const void* bias, const void* residual_bias,
+                                                 int8_t* output, void* residual, int batch_tokens,
+                                                 int hidden_size, float dequant_scale,
+                                                 float quant_scale, lsh_stream_t stream,
+                                                 int is_post_ln, const void* colsum) {
+  return residual_bias_ln_i8O<__half, int32_t>(input, H(scale), H(bias), H(residual_bias), output,
+                                               HM(residual), batch_tokens, hidden_size,
+                                               dequant_scale, quant_scale, HS(stream),
+                                               is_post_ln != 0, H(colsum), nparts,
+                                               (long)part_stride);
+}
 int lsh_gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int m, int n, int k, float alpha,
                     lsh_stream_t stream) {
   return gemm_i8_i8o(A, W, C, m, n, k, alpha, HS(stream));

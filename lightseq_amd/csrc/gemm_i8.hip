@@ -187,7 +187,7 @@ struct EpiQkvF16 {
 template <typename Epi, int MB, int NB>
 __device__ __forceinline__ void store_tile_acc(const Epi& epi, const v16i (&acc)[MB][NB], int m0,
                                                int n0, int wm, int wn, int l32, int g, int M, int N,
-                                               bool vec_store) {
+                                               bool vec_store, long m_off = 0) {
 #pragma unroll
   for (int i = 0; i < MB; ++i) {
     const long m = m0 + wm * (MB * 32) + i * 32 + l32;
@@ -195,7 +195,7 @@ __device__ __forceinline__ void store_tile_acc(const Epi& epi, const v16i (&acc)
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
         const int n = n0 + wn * (NB * 32) + j * 32 + 16 * g;
-        if (n < N) epi.store16(m, n, N, acc[i][j], vec_store && n + 16 <= N);
+        if (n < N) epi.store16(m + m_off, n, N, acc[i][j], vec_store && n + 16 <= N);
       }
     }
   }
@@ -226,36 +226,42 @@ __device__ __forceinline__ void tile_of(int t, int nblk, int tiles_m, int tiles_
 template <typename Epi>
 __global__ void __launch_bounds__(256)
 gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
-                      int N, int K, int tiles_m, int tiles_n, bool vec_store) {
+                      int N, int K, int tiles_m, int tiles_n, bool vec_store, int ksplit) {
   constexpr int NST = 2;
   constexpr int STAGE = (kBM + kBN) * kBK;  // 32 KB: A tile then W tile
   constexpr int NA = kBM / 32, NW = kBN / 32;  // 1-KB DMA instructions per wavefront per stage
   extern __shared__ __align__(16) int8_t smem[];
-  const int nblk = tiles_m * tiles_n;
+  // work item = (K range, tile): with ksplit > 1 every tile is computed ksplit times over
+  // disjoint K ranges and range p stores to rows [p * M, (p + 1) * M) of the output
+  const int ntile = tiles_m * tiles_n;
+  const int nblk = ntile * ksplit;
   const int G = gridDim.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, g = lane >> 5;
   const int my_tiles = (nblk - (int)blockIdx.x + G - 1) / G;
-  const int nk = K / kBK;
+  const int kpart = K / ksplit;  // bytes of K per range (a multiple of kBK)
+  const int nk = kpart / kBK;
 
   // DMA sources: each instruction moves 8 rows x 128 B; lane i lands in LDS slot i of that
   // 1-KB block, so it fetches the chunk the swizzle puts there.  Row clamping keeps the
   // reads of partial tiles in bounds (the clamped rows are never stored).
   uint32_t a_src[NA], w_src[NW];
   auto set_src = [&](int j) {
+    const int item = blockIdx.x + j * G;
+    const uint32_t koff = (uint32_t)(item / ntile) * (uint32_t)kpart;
     int tm, tn;
-    tile_of(blockIdx.x + j * G, nblk, tiles_m, tiles_n, tm, tn);
+    tile_of(item % ntile, ntile, tiles_m, tiles_n, tm, tn);
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
       const int row = (wave + 4 * i) * 8 + (lane >> 3);
       const int c = (lane & 7) ^ key_act(row);
-      a_src[i] = (uint32_t)min(tm * kBM + row, M - 1) * (uint32_t)K + c * 16;
+      a_src[i] = (uint32_t)min(tm * kBM + row, M - 1) * (uint32_t)K + koff + c * 16;
     }
 #pragma unroll
     for (int i = 0; i < NW; ++i) {
       const int row = (wave + 4 * i) * 8 + (lane >> 3);
       const int c = (lane & 7) ^ key_wgt(row);
-      w_src[i] = (uint32_t)min(tn * kBN + row, N - 1) * (uint32_t)K + c * 16;
+      w_src[i] = (uint32_t)min(tn * kBN + row, N - 1) * (uint32_t)K + koff + c * 16;
     }
   };
   const uint32_t lds0 =
@@ -303,8 +309,9 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   issue_next();
   int st = 0;
   for (int j = 0; j < my_tiles; ++j) {
+    const int item = blockIdx.x + j * G;
     int tm, tn;
-    tile_of(blockIdx.x + j * G, nblk, tiles_m, tiles_n, tm, tn);
+    tile_of(item % ntile, ntile, tiles_m, tiles_n, tm, tn);
     v16i acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -338,7 +345,8 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
                 __builtin_amdgcn_mfma_i32_32x32x32_i8(av[ks][jj], bv[ks][i], acc[i][jj], 0, 0, 0);
       st ^= 1;
     }
-    store_tile_acc<Epi, 2, 2>(epi, acc, tm * kBM, tn * kBN, wm, wn, l32, g, M, N, vec_store);
+    store_tile_acc<Epi, 2, 2>(epi, acc, tm * kBM, tn * kBN, wm, wn, l32, g, M, N, vec_store,
+                              (long)(item / ntile) * M);
   }
   __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
 }
@@ -374,7 +382,7 @@ __device__ __forceinline__ void store_tile(int8_t* lds, int tid, const v4i (&reg
 template <typename Epi>
 __global__ void __launch_bounds__(256)
 gemm_i8_generic_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
-                       int N, int K, int tiles_m, int tiles_n, bool vec_store) {
+                       int N, int K, int tiles_m, int tiles_n, bool vec_store, int) {
   constexpr int kStage = (kBM + kBN) * kBK;
   extern __shared__ __align__(16) int8_t smem[];
   int tile_m, tile_n;
@@ -460,11 +468,15 @@ gemm_i8_generic_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ 
 template <typename Epi, int MBLK>
 __global__ void __launch_bounds__(256)
 gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
-                      int N, int K, int, int, bool vec_store) {
+                      int N, int K, int, int, bool vec_store, int ksplit) {
   __shared__ int red[4][MBLK][16][64];  // [wavefront][m block][register][lane]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, g = lane >> 5;
-  const int n0 = blockIdx.x * 32;
+  // blockIdx.x = column block + (K range) * column blocks; range p stores to rows
+  // [p * M, (p + 1) * M) of the output
+  const int ncol = (int)gridDim.x / ksplit;
+  const int part = (int)blockIdx.x / ncol;
+  const int n0 = ((int)blockIdx.x % ncol) * 32;
   const int8_t* wp = W + (long)min(n0 + sigma(l32), N - 1) * K + g * 64;
   const int8_t* ap[MBLK];
 #pragma unroll
@@ -472,8 +484,9 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   v16i acc[MBLK];
 #pragma unroll
   for (int i = 0; i < MBLK; ++i) acc[i] = (v16i)0;
-  const int nch = K / kBK;
-  for (int ch = wave; ch < nch; ch += 8) {
+  const int nch_part = K / kBK / ksplit;
+  const int nch = (part + 1) * nch_part;
+  for (int ch = part * nch_part + wave; ch < nch; ch += 8) {
     const int k0 = ch * kBK;
     const bool two = ch + 4 < nch;
     const int k1 = two ? k0 + 4 * kBK : k0;
@@ -516,7 +529,7 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
              (red[2][wave][r][lane] + red[3][wave][r][lane]);
     const long m = wave * 32 + l32;
     const int n = n0 + 16 * g;
-    if (m < M && n < N) epi.store16(m, n, N, c, vec_store && n + 16 <= N);
+    if (m < M && n < N) epi.store16(m + (long)part * M, n, N, c, vec_store && n + 16 <= N);
   }
 }
 
@@ -533,13 +546,13 @@ void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop) {
 static bool stream_ok(int M, int N, int K) {
   if (K % kBK != 0) return false;
   const unsigned long long lim = 0xffffffffull;
-  return (unsigned long long)(M - 1) * K + kBK < lim && (unsigned long long)(N - 1) * K + kBK < lim;
+  return (unsigned long long)M * K < lim && (unsigned long long)N * K < lim;
 }
 
 template <typename Kern, typename Epi>
 static int launch(Kern kern, int grid, size_t smem, const int8_t* A, const int8_t* W, Epi epi,
                   int M, int N, int K, int tiles_m, int tiles_n, bool vec_store, hipStream_t s,
-                  bool* attr_set) {
+                  bool* attr_set, int ksplit = 1) {
   if (!*attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -551,16 +564,16 @@ static int launch(Kern kern, int grid, size_t smem, const int8_t* A, const int8_
     hipEvent_t e0 = g_ev_start, e1 = g_ev_stop;
     g_ev_start = g_ev_stop = nullptr;
     hipExtLaunchKernelGGL(kern, dim3(grid), dim3(256), (unsigned)smem, s, e0, e1, 0, A, W, epi, M,
-                          N, K, tiles_m, tiles_n, vec_store);
+                          N, K, tiles_m, tiles_n, vec_store, ksplit);
   } else {
-    kern<<<grid, 256, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store);
+    kern<<<grid, 256, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store, ksplit);
   }
   return lsh_check_launch("gemm_i8_kernel");
 }
 
 template <typename Epi>
 static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int K,
-                    hipStream_t s) {
+                    hipStream_t s, int ksplit = 1) {
   if (M <= 0 || N <= 0 || K <= 0 || !A || !W)
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: bad arguments");
   if (K % 16 != 0) return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: K must be a multiple of 16");
@@ -572,19 +585,23 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   const size_t smem = 2 * (size_t)(kBM + kBN) * kBK;
   static bool attr_stream = false, attr_generic = false;  // per Epi instantiation
   static bool attr_skinny = true;                          // static LDS: nothing to set
+  if (ksplit < 1 || (ksplit > 1 && K % (ksplit * kBK) != 0))
+    return lsh_fail(LSH_ERR_INVALID, "int8 gemm: K does not split into whole 128-byte steps");
   if (M <= 64 && K % kBK == 0) {
-    const int grid = (N + 31) / 32;
+    const int grid = ((N + 31) / 32) * ksplit;
     if (M <= 32)
       return launch(gemm_i8_skinny_kernel<Epi, 1>, grid, 0, A, W, epi, M, N, K, 0, 0, vec_store, s,
-                    &attr_skinny);
+                    &attr_skinny, ksplit);
     return launch(gemm_i8_skinny_kernel<Epi, 2>, grid, 0, A, W, epi, M, N, K, 0, 0, vec_store, s,
-                  &attr_skinny);
+                  &attr_skinny, ksplit);
   }
   if (stream_ok(M, N, K)) {
-    const int grid = tiles < 512 ? tiles : 512;  // 2 resident workgroups per compute unit
+    const int items = tiles * ksplit;
+    const int grid = items < 512 ? items : 512;  // 2 resident workgroups per compute unit
     return launch(gemm_i8_stream_kernel<Epi>, grid, smem, A, W, epi, M, N, K, tiles_m, tiles_n,
-                  vec_store, s, &attr_stream);
+                  vec_store, s, &attr_stream, ksplit);
   }
+  if (ksplit != 1) return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: this shape cannot split K");
   return launch(gemm_i8_generic_kernel<Epi>, tiles, smem, A, W, epi, M, N, K, tiles_m, tiles_n,
                 vec_store, s, &attr_generic);
 }
@@ -599,6 +616,36 @@ int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int
                  hipStream_t s) {
   if (!C) return lsh_fail(LSH_ERR_INVALID, "int8 gemm: null output");
   return dispatch(A, W, EpiI32{C}, M, N, K, s);
+}
+
+// Heuristic split of K for int32-output products whose tile count leaves most of the 256
+// compute units idle (N = hidden, K = inner size of the second FFN product).
+int gemm_i8_preferred_ksplit(int M, int N, int K) {
+  if (K % kBK != 0) return 1;
+  const int nch = K / kBK;
+  int items, per_item_min;
+  if (M <= 64) {
+    items = (N + 31) / 32;
+    per_item_min = 4;  // one 128-byte step per wavefront
+  } else {
+    if (!stream_ok(M, N, K)) return 1;
+    items = ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN);
+    per_item_min = 6;
+  }
+  int ks = 1;
+  while (ks < 8 && items * ks * 2 <= (M <= 64 ? 256 : 512) && nch % (ks * 2) == 0 &&
+         nch / (ks * 2) >= per_item_min)
+    ks *= 2;
+  return ks;
+}
+
+int gemm_i8_i32o_splitk(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int K,
+                        int ksplit, int* used, hipStream_t s) {
+  if (!C) return lsh_fail(LSH_ERR_INVALID, "int8 gemm: null output");
+  if (ksplit < 1 || K % kBK != 0 || (K / kBK) % ksplit != 0 || (M > 64 && !stream_ok(M, N, K)))
+    ksplit = 1;
+  if (used) *used = ksplit;
+  return dispatch(A, W, EpiI32{C}, M, N, K, s, ksplit);
 }
 
 int gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K, float alpha,

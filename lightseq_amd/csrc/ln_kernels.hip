@@ -119,6 +119,162 @@ ln_rows_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
   }
 }
 
+// 8 consecutive elements per lane per step (one 16-byte load of fp16 data, 8 bytes of int8
+// codes, two 16-byte loads of int32 accumulators); LPR lanes share a row, so a wavefront
+// covers 64/LPR rows and a workgroup 4 * 64/LPR.  All loads of a lane are issued before the
+// first reduction.  `nparts` int32 accumulator planes `part_stride` elements apart are
+// summed first (the split-K form of the int32 GEMM); the sum of integers is exact.
+// Preconditions (checked by the launcher): hidden % 8 == 0, hidden <= LPR * 8 * ITER,
+// 16-byte aligned pointers.
+__device__ __forceinline__ void ld8_acc(const int8_t* p, long i, float (&o)[8]) {
+  uint2 w = *reinterpret_cast<const uint2*>(p + i);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    o[k] = (float)unpack_i8(w.x, k);
+    o[4 + k] = (float)unpack_i8(w.y, k);
+  }
+}
+__device__ __forceinline__ void ld8_acc(const int32_t* p, long i, int (&o)[8]) {
+  int4 a = *reinterpret_cast<const int4*>(p + i);
+  int4 b = *reinterpret_cast<const int4*>(p + i + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+  o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+__device__ __forceinline__ void ld8(const float* p, long i, float (&o)[8]) {
+  float a[4], b[4];
+  ld4(p, i, a);
+  ld4(p, i + 4, b);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) { o[k] = a[k]; o[4 + k] = b[k]; }
+}
+__device__ __forceinline__ void ld8(const __half* p, long i, float (&o)[8]) {
+  half8_t t = *reinterpret_cast<const half8_t*>(p + i);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) o[k] = __half2float(t.v[k]);
+}
+__device__ __forceinline__ void st8(float* p, long i, const float (&o)[8]) {
+  *reinterpret_cast<float4*>(p + i) = make_float4(o[0], o[1], o[2], o[3]);
+  *reinterpret_cast<float4*>(p + i + 4) = make_float4(o[4], o[5], o[6], o[7]);
+}
+__device__ __forceinline__ void st8(__half* p, long i, const float (&o)[8]) {
+  half8_t t;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) t.v[k] = __float2half_rn(o[k]);
+  *reinterpret_cast<half8_t*>(p + i) = t;
+}
+template <int LPR>
+__device__ __forceinline__ float row_sum(float v) {
+#pragma unroll
+  for (int m = LPR / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, kWave);
+  return v;
+}
+
+template <typename T, typename AccT, int MODE, int LPR, int ITER>
+__global__ void __launch_bounds__(256)
+ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
+                int8_t* __restrict__ out_q, const T* __restrict__ scale,
+                const T* __restrict__ bias, const T* __restrict__ residual_bias,
+                const T* __restrict__ colsum, int tokens, int hidden, float dequant_scale,
+                float quant_scale, int is_post_ln, int nparts, long part_stride) {
+  constexpr int RPW = kWave / LPR;
+  const int lane = threadIdx.x & 63;
+  const int sub = lane % LPR;
+  const int row = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPR;
+  const bool live = row < tokens;  // dead rows keep the shuffles convergent
+  const long base = (long)(live ? row : 0) * hidden;
+
+  float x[ITER][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    const int e = (it * LPR + sub) * 8;
+    if (e < hidden && live) {
+      float r[8];
+      ld8(residual, base + e, r);
+      if (MODE == kLnFirst) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[it][k] = TT<T>::safe(r[k]);
+      } else {
+        float a[8];
+        if constexpr (sizeof(AccT) == 4) {
+          int acc[8];
+          ld8_acc(gemm_out, base + e, acc);
+          for (int p = 1; p < nparts; ++p) {
+            int more[8];
+            ld8_acc(gemm_out + p * part_stride, base + e, more);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[k] += more[k];
+          }
+#pragma unroll
+          for (int k = 0; k < 8; ++k) a[k] = (float)acc[k];
+        } else {
+          ld8_acc(gemm_out, base + e, a);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[it][k] = a[k] * dequant_scale + TT<T>::safe(r[k]);
+        if (colsum != nullptr) {
+          float c[8];
+          ld8(colsum, e, c);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) x[it][k] += TT<T>::safe(c[k]);
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) sum += x[it][k];
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) x[it][k] = 0.f;
+    }
+  }
+  const float mean = row_sum<LPR>(sum) / (float)hidden;
+  float var = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    const int e = (it * LPR + sub) * 8;
+    if (e < hidden) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        float t = x[it][k] - mean;
+        var += t * t;
+      }
+    }
+  }
+  const float rstd = rsqrtf(row_sum<LPR>(var) / (float)hidden + kLnEpsilon);
+  if (!live) return;
+
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    const int e = (it * LPR + sub) * 8;
+    if (e < hidden) {
+      float g[8], b[8], o[8];
+      ld8(scale, e, g);
+      ld8(bias, e, b);
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        o[k] = (x[it][k] - mean) * rstd * TT<T>::safe(g[k]) + TT<T>::safe(b[k]);
+      if (MODE == kLnResOut) {
+        st8(out_t, base + e, o);
+      } else {
+        uint2 packed;
+        packed.x = pack4_i8(float2int8(o[0], quant_scale), float2int8(o[1], quant_scale),
+                            float2int8(o[2], quant_scale), float2int8(o[3], quant_scale));
+        packed.y = pack4_i8(float2int8(o[4], quant_scale), float2int8(o[5], quant_scale),
+                            float2int8(o[6], quant_scale), float2int8(o[7], quant_scale));
+        *reinterpret_cast<uint2*>(out_q + base + e) = packed;
+        float rb[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (residual_bias != nullptr) ld8(residual_bias, e, rb);
+        float w[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          float keep = is_post_ln ? o[k] : x[it][k];
+          w[k] = (MODE == kLnFirst) ? keep + rb[k] : TT<T>::rnd(keep) + rb[k];
+        }
+        st8(residual, base + e, w);
+      }
+    }
+  }
+}
+
 // Any hidden size / alignment: one workgroup per row, row staged in LDS.
 template <typename T, typename AccT, int MODE>
 __global__ void ln_rows_generic_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
@@ -167,12 +323,32 @@ template <typename T, typename AccT, int MODE>
 static int launch_ln(const AccT* gemm_out, T* residual, T* out_t, int8_t* out_q, const T* scale,
                      const T* bias, const T* residual_bias, const T* colsum, int tokens,
                      int hidden, float dequant_scale, float quant_scale, int is_post_ln,
-                     hipStream_t stream) {
+                     hipStream_t stream, int nparts = 1, long part_stride = 0) {
   if (tokens <= 0 || hidden <= 0) return lsh_fail(LSH_ERR_INVALID, "layer norm: empty shape");
+  if (nparts < 1 || (nparts > 1 && (sizeof(AccT) != 4 || part_stride % 4 != 0)))
+    return lsh_fail(LSH_ERR_INVALID, "layer norm: bad accumulator planes");
   const bool vec_ok = hidden % 4 == 0 && hidden <= 2048 && aligned16(gemm_out) &&
                       aligned16(residual) && aligned16(out_t) && aligned16(out_q) &&
                       aligned16(scale) && aligned16(bias) && aligned16(residual_bias) &&
                       aligned16(colsum);
+  if (vec_ok && hidden % 8 == 0) {
+    // LPR = 64 when the row fills whole 512-element steps, otherwise two rows per wavefront
+#define LSH_LN8_CASE(LPR, IT)                                                                    \
+  ln_rows8_kernel<T, AccT, MODE, LPR, IT>                                                        \
+      <<<(tokens + 4 * (64 / LPR) - 1) / (4 * (64 / LPR)), 256, 0, stream>>>(                    \
+          gemm_out, residual, out_t, out_q, scale, bias, residual_bias, colsum, tokens, hidden,  \
+          dequant_scale, quant_scale, is_post_ln, nparts, part_stride)
+    if (hidden <= 256) LSH_LN8_CASE(32, 1);
+    else if (hidden <= 512) LSH_LN8_CASE(32, 2);
+    else if (hidden <= 768) LSH_LN8_CASE(32, 3);
+    else if (hidden <= 1024) LSH_LN8_CASE(32, 4);
+    else if (hidden <= 1536) LSH_LN8_CASE(64, 3);
+    else LSH_LN8_CASE(64, 4);
+#undef LSH_LN8_CASE
+    return lsh_check_launch("ln_rows8_kernel");
+  }
+  if (nparts > 1)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "layer norm: accumulator planes need hidden % 8 == 0");
   if (!vec_ok) {
     if ((size_t)hidden * sizeof(float) > 160 * 1024 - 256)
       return lsh_fail(LSH_ERR_UNSUPPORTED, "layer norm: hidden size too large");
@@ -215,24 +391,25 @@ template <typename T, typename AccT>
 int residual_bias_ln_i8O(const AccT* input, const T* scale, const T* bias, const T* residual_bias,
                          int8_t* output, T* residual, int batch_tokens, int hidden_size,
                          float dequant_scale, float quant_scale, hipStream_t stream,
-                         bool is_post_ln, const T* colsum) {
+                         bool is_post_ln, const T* colsum, int nparts, long part_stride) {
   if (!input || !output || !scale || !bias || !residual)
     return lsh_fail(LSH_ERR_INVALID, "ker_residual_bias_ln_*_i8O: null pointer");
   return launch_ln<T, AccT, kLnResQuant>(input, residual, nullptr, output, scale, bias,
                                          residual_bias, colsum, batch_tokens, hidden_size,
-                                         dequant_scale, quant_scale, is_post_ln, stream);
+                                         dequant_scale, quant_scale, is_post_ln, stream, nparts,
+                                         part_stride);
 }
 
 template <typename T>
 int residual_bias_ln_i32I(const int32_t* input, const T* scale, const T* bias, const T* residual,
                           T* output, int batch_tokens, int hidden_size, float dequant_scale,
-                          hipStream_t stream, const T* colsum) {
+                          hipStream_t stream, const T* colsum, int nparts, long part_stride) {
   if (!input || !output || !scale || !bias || !residual)
     return lsh_fail(LSH_ERR_INVALID, "ker_residual_bias_ln_i32I: null pointer");
   // the kernel only reads `residual`; output may alias it (the reference calls it in place)
   return launch_ln<T, int32_t, kLnResOut>(input, const_cast<T*>(residual), output, nullptr, scale,
                                           bias, nullptr, colsum, batch_tokens, hidden_size,
-                                          dequant_scale, 0.f, 0, stream);
+                                          dequant_scale, 0.f, 0, stream, nparts, part_stride);
 }
 
 #define LSH_INST(T)                                                                              \
@@ -240,12 +417,12 @@ int residual_bias_ln_i32I(const int32_t* input, const T* scale, const T* bias, c
                                         const T*, float, bool);                                  \
   template int residual_bias_ln_i8O<T, int8_t>(const int8_t*, const T*, const T*, const T*,      \
                                                int8_t*, T*, int, int, float, float, hipStream_t, \
-                                               bool, const T*);                                  \
+                                               bool, const T*, int, long);                       \
   template int residual_bias_ln_i8O<T, int32_t>(const int32_t*, const T*, const T*, const T*,    \
                                                 int8_t*, T*, int, int, float, float,             \
-                                                hipStream_t, bool, const T*);                    \
+                                                hipStream_t, bool, const T*, int, long);         \
   template int residual_bias_ln_i32I<T>(const int32_t*, const T*, const T*, const T*, T*, int,   \
-                                        int, float, hipStream_t, const T*);
+                                        int, float, hipStream_t, const T*, int, long);
 LSH_INST(float)
 LSH_INST(__half)
 #undef LSH_INST

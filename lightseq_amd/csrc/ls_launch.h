@@ -56,11 +56,14 @@ template <typename T, typename AccT>
 int residual_bias_ln_i8O(const AccT* input, const T* scale, const T* bias, const T* residual_bias,
                          int8_t* output, T* residual, int batch_tokens, int hidden_size,
                          float dequant_scale, float quant_scale, hipStream_t stream,
-                         bool is_post_ln, const T* colsum);
+                         bool is_post_ln, const T* colsum, int nparts = 1, long part_stride = 0);
 template <typename T>
 int residual_bias_ln_i32I(const int32_t* input, const T* scale, const T* bias, const T* residual,
                           T* output, int batch_tokens, int hidden_size, float dequant_scale,
-                          hipStream_t stream, const T* colsum);
+                          hipStream_t stream, const T* colsum, int nparts = 1,
+                          long part_stride = 0);
+// `nparts` > 1: `input` holds that many int32 accumulator planes `part_stride` elements apart
+// (split-K GEMM output, gemm_i8_i32o_splitk) which are summed before the dequantisation.
 
 // ---- head split / merge, embedding (arrange_kernels.hip) -------------------------
 template <typename T>
@@ -98,6 +101,12 @@ int encself_attention_f16(const __half* q, const __half* k, const __half* v, con
 // C[M,N] = A[M,K] * W[N,K]^T, both operands K-contiguous.
 int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int K,
                  hipStream_t s);
+// K split into `ksplit` ranges; range p writes the plane C + p * M * N.  Returns the ksplit
+// actually used (1 when the shape does not split evenly) in *used.
+int gemm_i8_i32o_splitk(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int K,
+                        int ksplit, int* used, hipStream_t s);
+// The split the library prefers for an int32-output GEMM of this shape (1 = none).
+int gemm_i8_preferred_ksplit(int M, int N, int K);
 int gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K, float alpha,
                 hipStream_t s);
 // Fused epilogues (fp16 models).  Each produces exactly the bits of the int8-output GEMM

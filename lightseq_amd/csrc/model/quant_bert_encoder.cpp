@@ -45,7 +45,9 @@ void QuantBertEncoder::init_buffer() {
   const size_t wide = (size_t)tokens * std::max(I, 3 * H);
   _int8_ffn_in_buf.alloc(wide);
   _int8_ffn_out_buf.alloc(wide);
-  _int32_ffn_out_buf.alloc((size_t)tokens * H);
+  // room for the accumulator planes of a split-K second FFN product (up to 4 at encoder
+  // sizes, up to 8 for the few rows of a decode step)
+  _int32_ffn_out_buf.alloc(std::max((size_t)tokens * H * 4, (size_t)64 * H * 8));
 
   _int8_emb = upload_kernel(_tw.token_embedding, _tw._src_vocab_size, H, false, _stream);
   _pos_emb = upload_half(_tw.position_embedding, _stream);
@@ -251,8 +253,15 @@ void QuantBertEncoder::ffn_add_norm() {
   tap(taps.act_q, act_buf, (size_t)M * I);
 
   prof_begin(3, M, H, I, "EpiI32");
-  LSH_CALL(gemm_i8_i32o(act_buf, w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I, _stream));
-  if (taps.ffn2_acc && taps.tap_layer == _layer_id)
+  // K split over workgroups when the tile count would leave compute units idle; the planes
+  // are summed (exactly) by the layer-norm kernel that consumes them
+  const bool tap_acc = taps.ffn2_acc && taps.tap_layer == _layer_id;
+  int nparts = 1;
+  LSH_CALL(gemm_i8_i32o_splitk(act_buf, w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I,
+                               tap_acc ? 1 : std::min(4, gemm_i8_preferred_ksplit(M, H, I)),
+                               &nparts, _stream));
+  const long part_stride = (long)M * H;
+  if (tap_acc)
     CHECK_GPU_ERROR(hipMemcpyAsync(taps.ffn2_acc, _int32_ffn_out_buf.get(),
                                    (size_t)M * H * sizeof(int32_t), hipMemcpyDeviceToDevice,
                                    _stream));
@@ -266,14 +275,14 @@ void QuantBertEncoder::ffn_add_norm() {
   if (_layer_id == _tw._n_enc_layer - 1) {
     LSH_CALL(residual_bias_ln_i32I<__half>(_int32_ffn_out_buf.get(), _final_ln_scale.get(),
                                            _final_ln_bias.get(), _p_d_output, _p_d_output, M, H,
-                                           dequant_scale, _stream, colsum));
+                                           dequant_scale, _stream, colsum, nparts, part_stride));
   } else {
     const Layer& nx = _layers[_layer_id + 1];
     const float clip_next = _enc_clip_max[(_layer_id + 1) * _tw._clip_stride + 4];
     LSH_CALL((residual_bias_ln_i8O<__half, int32_t>(
         _int32_ffn_out_buf.get(), nx.ln1_scale.get(), nx.ln1_bias.get(), nx.b_out.get(),
         _int8_ffn_in_buf.get(), _p_d_output, M, H, dequant_scale, Q / clip_next, _stream,
-        _tw._is_post_ln, colsum)));
+        _tw._is_post_ln, colsum, nparts, part_stride)));
   }
 }
 

@@ -83,7 +83,8 @@ void QuantDecoder::init_buffer() {
   _buf_a.alloc(wide);
   _buf_b.alloc(wide);
   _logits.alloc(rows * (size_t)V);
-  _int32_ffn_out_buf.alloc(rows * H);
+  // up to 8 accumulator planes of the split-K second FFN product
+  _int32_ffn_out_buf.alloc(rows * H * 8);
   for (int i = 0; i < 2; ++i) {
     _self_k_cache[i].alloc((size_t)L * _layer_size_self_k);
     _self_v_cache[i].alloc((size_t)L * _layer_size_self_k);
@@ -332,7 +333,9 @@ void QuantDecoder::ffn_add_norm() {
   LSH_CALL(gemm_i8_bias_act_i8o(_buf_b.get(), w.w_ffn1.get(), _buf_a.get(), w.b_ffn1.get(), M, I,
                                 H, c[4] * c[10] / (c[16] * Q), c[16] / Q, Q / c[11], c[11], act,
                                 _stream));
-  LSH_CALL(gemm_i8_i32o(_buf_a.get(), w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I, _stream));
+  int nparts = 1;
+  LSH_CALL(gemm_i8_i32o_splitk(_buf_a.get(), w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I,
+                               gemm_i8_preferred_ksplit(M, H, I), &nparts, _stream));
 
   const float dequant_scale =
       _tw._use_gelu ? c[5] * c[11] / (Q * Q) : c[5] * c[11] / (2 * Q * Q);
@@ -353,7 +356,7 @@ void QuantDecoder::ffn_add_norm() {
   LSH_CALL((residual_bias_ln_i8O<__half, int32_t>(
       _int32_ffn_out_buf.get(), scale_ptr, bias_ptr, res_bias_ptr, _buf_a.get(),
       _cur_step_query.get(), M, H, dequant_scale, Q / clip_max, _stream, _tw._is_post_ln,
-      w.ffn2_colsum.get())));
+      w.ffn2_colsum.get(), nparts, (long)M * H)));
 }
 
 bool QuantDecoder::beam_search() {

@@ -68,7 +68,8 @@ void QuantGptEncoder::init_buffer() {
   _hid_last.alloc((size_t)_max_batch_size * H);
   // perplexity needs the logits of every position, sampling only of the last one
   _logits.alloc((_tw._sampling_method == "ppl" ? tokens : (size_t)_max_batch_size) * V);
-  _int32_ffn_out_buf.alloc(tokens * H);
+  // room for the accumulator planes of the split-K second FFN product
+  _int32_ffn_out_buf.alloc(std::max(tokens * H * 4, (size_t)64 * H * 8));
   _self_k_cache.alloc((size_t)L * _max_batch_dim);
   _self_v_cache.alloc((size_t)L * _max_batch_dim);
   CHECK_GPU_ERROR(hipMemsetAsync(_self_k_cache.get(), 0, _self_k_cache.size(), _stream));
@@ -110,7 +111,11 @@ void QuantGptEncoder::ffn_add_norm(int rows, int8_t* in, int8_t* tmp) {
   LSH_CALL(gemm_i8_bias_act_i8o(in, w.w_ffn1.get(), tmp, w.b_ffn1.get(), rows, I, H,
                                 c[2] * c[6] / (c[10] * Q), c[10] / Q, Q / c[7], c[7], kActGelu,
                                 _stream));
-  LSH_CALL(gemm_i8_i32o(tmp, w.w_ffn2.get(), _int32_ffn_out_buf.get(), rows, H, I, _stream));
+  int nparts = 1;
+  LSH_CALL(gemm_i8_i32o_splitk(tmp, w.w_ffn2.get(), _int32_ffn_out_buf.get(), rows, H, I,
+                               rows <= 64 ? gemm_i8_preferred_ksplit(rows, H, I)
+                                          : std::min(4, gemm_i8_preferred_ksplit(rows, H, I)),
+                               &nparts, _stream));
   const float dequant_scale = c[3] * c[7] / (Q * Q);
   const __half *scale_ptr, *bias_ptr, *res_bias_ptr;
   float clip_max;
@@ -128,7 +133,7 @@ void QuantGptEncoder::ffn_add_norm(int rows, int8_t* in, int8_t* tmp) {
   }
   LSH_CALL((residual_bias_ln_i8O<__half, int32_t>(
       _int32_ffn_out_buf.get(), scale_ptr, bias_ptr, res_bias_ptr, in, _query.get(), rows, H,
-      dequant_scale, Q / clip_max, _stream, false, nullptr)));
+      dequant_scale, Q / clip_max, _stream, false, nullptr, nparts, (long)rows * H)));
 }
 
 // all prompt positions at once (:253-291 / :299-341); leaves the int8 LayerNorm output of

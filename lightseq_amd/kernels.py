@@ -163,6 +163,30 @@ def gemm_i8_i32o(a, w, c, m, n, k):
     call("lsh_gemm_i8_i32o", ptr(a), ptr(w), ptr(c), m, n, k, current_stream())
 
 
+def gemm_i8_i32o_splitk(a, w, c, m, n, k, ksplit):
+    """K split into ``ksplit`` ranges; range p fills the plane c[p] of c [ksplit, m, n].
+    Returns the split applied."""
+    import ctypes
+    _dev(a, w, c)
+    used = ctypes.c_int(0)
+    call("lsh_gemm_i8_i32o_splitk", ptr(a), ptr(w), ptr(c), m, n, k, ksplit,
+         ctypes.cast(ctypes.byref(used), ctypes.c_void_p), current_stream())
+    return used.value
+
+
+def gemm_i8_preferred_ksplit(m, n, k):
+    return lib.load().lsh_gemm_i8_preferred_ksplit(m, n, k)
+
+
+def ker_residual_bias_ln_planes_i32I_i8O(inp, nparts, part_stride, scale, bias, residual_bias, out,
+                                         residual, batch_tokens, hidden_size, dequant_scale,
+                                         quant_scale, is_post_ln=False, colsum=None):
+    _dev(inp, scale, bias, residual_bias, out, residual, colsum)
+    call("lsh_ker_residual_bias_ln_planes_i32I_i8O_f16", ptr(inp), nparts, part_stride, ptr(scale),
+         ptr(bias), ptr(residual_bias), ptr(out), ptr(residual), batch_tokens, hidden_size,
+         dequant_scale, quant_scale, current_stream(), int(is_post_ln), ptr(colsum))
+
+
 def gemm_i8_i8o(a, w, c, m, n, k, alpha):
     """c[m,n] (int8) = clamp(floor(alpha * (a @ w^T) + 0.5), -127, 127)."""
     _dev(a, w, c)

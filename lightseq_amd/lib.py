@@ -47,6 +47,10 @@ _SIGNATURES = {
     "lsh_launch_scaled_colsum": (True, "ppiifs"),
     "lsh_gemm_i8_i32o": (False, "pppiiis"),
     "lsh_gemm_i8_i8o": (False, "pppiiifs"),
+    "lsh_gemm_i8_i32o_splitk": (False, "ppp" + "iiii" + "p" + "s"),
+    "lsh_gemm_i8_preferred_ksplit": (False, "iii"),
+    "lsh_ker_residual_bias_ln_planes_i32I_i8O_f16": (False, "p" + "il" + "ppppp" + "iiff" + "s" +
+                                                     "ip"),
     "lsh_gemm_i8_bias_gelu_i8o_f16": (False, "pppp" + "iiifffs"),
     "lsh_gemm_i8_bias_relu_i8o_f16": (False, "pppp" + "iiiffffis"),
     "lsh_gemm_i8_qkv_arrange_f16": (False, "pppp" + "iiiiiiffs"),

@@ -54,8 +54,13 @@ def test_tiny_stack_with_taps(tmp_path, oracle, cfg_name, batch, seq, over):
         valid = _valid(ids, cfg).reshape(-1)
         for name in ("ln1_q", "qkv_q", "ctx_q", "out_q", "ln2_q", "ffn1_q", "act_q"):
             g = bufs[name].cpu().numpy()
-            # padded query rows of the attention context are don't-care downstream
-            assert_codes_close(g[valid], taps[name][valid], max_frac=3e-3, what="%s layer %d" % (name, layer))
+            # padded query rows of the attention context are don't-care downstream.  Both runs
+            # are free-running here: the first layer sees identical inputs and meets the per-kernel
+            # bar; one flipped code there perturbs a whole accumulator row of the next GEMM, so
+            # deeper stages are held to "never more than one code" with a drift allowance (the
+            # stage-by-stage check on identical inputs is test_bert_base_two_layers_full_width)
+            assert_codes_close(g[valid], taps[name][valid], max_frac=3e-3 if layer == 0 else 0.1,
+                               what="%s layer %d" % (name, layer))
         # int32 accumulators: exact given the kernel's own int8 inputs
         act = bufs["act_q"].cpu().numpy()
         w2 = w["w_ffn2"][layer]

@@ -154,3 +154,42 @@ def test_fused_qkv_arrange_rejects_small_heads(rng):
     bias = torch.zeros(24, dtype=torch.float16, device=DEV)
     with pytest.raises(LSHError):
         k.gemm_i8_qkv_arrange(a, w, out, bias, 64, 8, 8, 16, 8, 1, 1.0, 1.0)
+
+
+@pytest.mark.parametrize("M,N,K,ksplit", [(4096, 768, 3072, 2), (16, 1024, 4096, 8), (64, 1024, 4096, 4),
+                                          (300, 256, 1024, 4), (33, 96, 256, 2)])
+def test_split_k_planes_sum_to_the_product(rng, M, N, K, ksplit):
+    a = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    c = torch.full((ksplit, M, N), 7, dtype=torch.int32, device=DEV)
+    used = _k().gemm_i8_i32o_splitk(to_dev(a), to_dev(w), c, M, N, K, ksplit)
+    assert used == ksplit
+    planes = to_np(c).astype(np.int64)
+    np.testing.assert_array_equal(planes.sum(0), _exact_i32(a, w))
+    kp = K // ksplit
+    np.testing.assert_array_equal(planes[1], _exact_i32(a[:, kp:2 * kp], w[:, kp:2 * kp]))
+    # a split that does not divide K into whole 128-byte steps is not applied
+    c1 = torch.zeros((3, M, N), dtype=torch.int32, device=DEV)
+    assert _k().gemm_i8_i32o_splitk(to_dev(a), to_dev(w), c1, M, N, K, 3) == (3 if (K // 128) % 3 == 0 else 1)
+    assert _k().gemm_i8_preferred_ksplit(4096, 768, 3072) == 2
+    assert _k().gemm_i8_preferred_ksplit(16, 1024, 4096) == 8
+    assert _k().gemm_i8_preferred_ksplit(4096, 3072, 768) == 1
+
+
+@pytest.mark.parametrize("rows,hidden,nparts", [(16, 1024, 8), (4096, 768, 2), (37, 512, 4)])
+def test_layer_norm_over_accumulator_planes(rng, rows, hidden, nparts):
+    planes = rng.integers(-20000, 20000, size=(nparts, rows, hidden), dtype=np.int32)
+    total = planes.sum(0).astype(np.int32)
+    g = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16)
+    b = (0.1 * rng.standard_normal(hidden)).astype(np.float16)
+    rb = (0.1 * rng.standard_normal(hidden)).astype(np.float16)
+    res = rng.standard_normal((rows, hidden)).astype(np.float16)
+    outs = []
+    for inp, n in ((planes, nparts), (total, 1)):
+        q = torch.zeros(rows, hidden, dtype=torch.int8, device=DEV)
+        r = to_dev(res.copy())
+        _k().ker_residual_bias_ln_planes_i32I_i8O(to_dev(inp), n, rows * hidden, to_dev(g), to_dev(b),
+                                                  to_dev(rb), q, r, rows, hidden, 3e-4, 127 / 4.0, True)
+        outs.append((to_np(q), to_np(r)))
+    np.testing.assert_array_equal(outs[0][0], outs[1][0])
+    np.testing.assert_array_equal(outs[0][1], outs[1][1])
