@@ -211,6 +211,17 @@ int lsh_launch_scaled_colsum_f32(const void* inp, void* out, int rows, int cols,
  * model/cublas_helper.h:50-58 cublaslt_gemm<int32_t,int32_t>. */
 int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n, int k,
                      lsh_stream_t stream);
+/* The bias + activation + requantisation epilogue as a table: after the requantisation an
+ * element is one of 255 codes, so what follows depends only on (column, code).
+ * lsh_build_act_lut fills lut [n, 256] (entry [col][code + 128]) with what
+ * lsh_gemm_i8_bias_{gelu,relu}_i8o_f16 computes for that code (act: 0 GELU, 1 ReLU, 2 ReLU
+ * with the narrow unsigned clip); lsh_gemm_i8_lut_i8o is the product with that table as its
+ * epilogue, bit-identical to the arithmetic form and much cheaper per element.  Build the
+ * table once per weight matrix.  No counterpart in the reference. */
+int lsh_build_act_lut(int8_t* lut, const void* bias_f16, int n, float dequant_scale,
+                      float quant_scale, float clip_max, int act, lsh_stream_t stream);
+int lsh_gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int m,
+                        int n, int k, float alpha, lsh_stream_t stream);
 /* The int32 product with K split into `ksplit` equal ranges computed by different workgroups
  * (for shapes whose tile count would leave compute units idle, e.g. the second FFN product):
  * range p writes the plane C + p * m * n, so C needs ksplit * m * n elements; the planes are

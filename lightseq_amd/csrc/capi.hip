@@ -322,6 +322,14 @@ int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n,
                      lsh_stream_t stream) {
   return gemm_i8_i32o(A, W, C, m, n, k, HS(stream));
 }
+int lsh_build_act_lut(int8_t* lut, const void* bias_f16, int n, float dequant_scale,
+                      float quant_scale, float clip_max, int act, lsh_stream_t stream) {
+  return build_act_lut(lut, H(bias_f16), n, dequant_scale, quant_scale, clip_max, act, HS(stream));
+}
+int lsh_gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int m,
+                        int n, int k, float alpha, lsh_stream_t stream) {
+  return gemm_i8_lut_i8o(A, W, C, lut, m, n, k, alpha, HS(stream));
+}
 int lsh_gemm_i8_i32o_splitk(const int8_t* A, const int8_t* W, int32_t* C, int m, int n, int k,
                             int ksplit, int* used, lsh_stream_t stream) {
   return gemm_i8_i32o_splitk(A, W, C, m, n, k, ksplit, used, HS(stream));

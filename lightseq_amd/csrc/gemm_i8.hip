@@ -150,6 +150,41 @@ struct EpiActI8 {
   static const char* name() { return ACT == kActGelu ? "EpiGeluI8" : "EpiReluI8"; }
 };
 
+// The same epilogue through a table.  After the requantisation an element is one of 255
+// codes, and what follows (dequantise, add the column's bias, activation, requantise)
+// depends only on that code and the column: table[n][code + 128], N x 256 bytes built once
+// per weight matrix by build_act_lut with the very device function EpiActI8 evaluates, so
+// the result is bit-identical.  The bias + GELU arithmetic costs ~35 vector instructions per
+// element -- more than the matrix cores spend on a K = 768 product -- while the lookup is
+// one byte load per element from a table that stays in L2 (768 KB for N = 3072); the lanes
+// of one load instruction read two table rows, i.e. a handful of cache lines.
+struct EpiLutI8 {
+  int8_t* C;
+  const int8_t* lut;
+  float alpha;
+  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
+    int q[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int col = n + i < N ? n + i : N - 1;
+      q[i] = lut[(long)col * 256 + requant_acc(c[i], alpha) + 128];
+    }
+    store16_i8(C + m * N + n, n, N, q, full);
+  }
+  bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
+  static const char* name() { return "EpiLutI8"; }
+};
+
+template <int ACT>
+__global__ void __launch_bounds__(256)
+build_act_lut_kernel(int8_t* __restrict__ lut, const __half* __restrict__ bias, int N,
+                     float dequant_scale, float quant_scale, float clip_max) {
+  const int n = blockIdx.x;
+  const int code = (int)threadIdx.x - 128;
+  lut[(long)n * 256 + threadIdx.x] = (int8_t)dequant_bias_act_requant<ACT>(
+      code, dequant_scale, __half2float(bias[n]), quant_scale, clip_max);
+}
+
 // requantise to the GEMM's int8 output code, then dequant + bias and scatter into the
 // three [B, h, S, d] fp16 tensors exactly as the QKV arrange kernel would.
 // Requires N == 3*h*d, d % 16 == 0.
@@ -628,9 +663,8 @@ int gemm_i8_preferred_ksplit(int M, int N, int K) {
     items = (N + 31) / 32;
     per_item_min = 4;  // one 128-byte step per wavefront
   } else {
-    if (!stream_ok(M, N, K)) return 1;
-    items = ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN);
-    per_item_min = 6;
+    // at encoder sizes the int32 planes cost more HBM writes than the idle units cost time
+    return 1;
   }
   int ks = 1;
   while (ks < 8 && items * ks * 2 <= (M <= 64 ? 256 : 512) && nch % (ks * 2) == 0 &&
@@ -678,6 +712,34 @@ int gemm_i8_bias_act_i8o(const int8_t* A, const int8_t* W, int8_t* C, const __ha
     default:
       return lsh_fail(LSH_ERR_INVALID, "int8 gemm (bias+act): unknown activation");
   }
+}
+
+int build_act_lut(int8_t* lut, const __half* bias, int N, float dequant_scale, float quant_scale,
+                  float clip_max, int act, hipStream_t s) {
+  if (!lut || !bias || N <= 0) return lsh_fail(LSH_ERR_INVALID, "build_act_lut: bad arguments");
+  switch (act) {
+    case kActGelu:
+      build_act_lut_kernel<kActGelu><<<N, 256, 0, s>>>(lut, bias, N, dequant_scale, quant_scale,
+                                                       clip_max);
+      break;
+    case kActRelu:
+      build_act_lut_kernel<kActRelu><<<N, 256, 0, s>>>(lut, bias, N, dequant_scale, quant_scale,
+                                                       clip_max);
+      break;
+    case kActReluNarrow:
+      build_act_lut_kernel<kActReluNarrow><<<N, 256, 0, s>>>(lut, bias, N, dequant_scale,
+                                                             quant_scale, clip_max);
+      break;
+    default:
+      return lsh_fail(LSH_ERR_INVALID, "build_act_lut: unknown activation");
+  }
+  return lsh_check_launch("build_act_lut_kernel");
+}
+
+int gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int M, int N,
+                    int K, float alpha, hipStream_t s) {
+  if (!C || !lut) return lsh_fail(LSH_ERR_INVALID, "int8 gemm (table epilogue): null pointer");
+  return dispatch(A, W, EpiLutI8{C, lut, alpha}, M, N, K, s);
 }
 
 int gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, __half* new_qkv, const __half* qkv_bias,

@@ -184,6 +184,23 @@ ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
   const long base = (long)(live ? row : 0) * hidden;
 
   float x[ITER][8];
+  // scale, bias and residual bias travel with the first round of loads, so the kernel has
+  // one global-memory round trip before its reductions and none after
+  float gs[ITER][8], bs[ITER][8], rbs[ITER][8];
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    const int e = (it * LPR + sub) * 8;
+    if (e < hidden) {
+      ld8(scale, e, gs[it]);
+      ld8(bias, e, bs[it]);
+      if (MODE != kLnResOut && residual_bias != nullptr) {
+        ld8(residual_bias, e, rbs[it]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) rbs[it][k] = 0.f;
+      }
+    }
+  }
   float sum = 0.f;
 #pragma unroll
   for (int it = 0; it < ITER; ++it) {
@@ -197,14 +214,18 @@ ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
       } else {
         float a[8];
         if constexpr (sizeof(AccT) == 4) {
-          int acc[8];
+          // all planes are requested before the first use (independent loads)
+          int acc[8], more[7][8];
           ld8_acc(gemm_out, base + e, acc);
-          for (int p = 1; p < nparts; ++p) {
-            int more[8];
-            ld8_acc(gemm_out + p * part_stride, base + e, more);
 #pragma unroll
-            for (int k = 0; k < 8; ++k) acc[k] += more[k];
-          }
+          for (int p = 1; p < 8; ++p)
+            if (p < nparts) ld8_acc(gemm_out + p * part_stride, base + e, more[p - 1]);
+#pragma unroll
+          for (int p = 1; p < 8; ++p)
+            if (p < nparts) {
+#pragma unroll
+              for (int k = 0; k < 8; ++k) acc[k] += more[p - 1][k];
+            }
 #pragma unroll
           for (int k = 0; k < 8; ++k) a[k] = (float)acc[k];
         } else {
@@ -246,12 +267,10 @@ ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
   for (int it = 0; it < ITER; ++it) {
     const int e = (it * LPR + sub) * 8;
     if (e < hidden) {
-      float g[8], b[8], o[8];
-      ld8(scale, e, g);
-      ld8(bias, e, b);
+      float o[8];
 #pragma unroll
       for (int k = 0; k < 8; ++k)
-        o[k] = (x[it][k] - mean) * rstd * TT<T>::safe(g[k]) + TT<T>::safe(b[k]);
+        o[k] = (x[it][k] - mean) * rstd * TT<T>::safe(gs[it][k]) + TT<T>::safe(bs[it][k]);
       if (MODE == kLnResOut) {
         st8(out_t, base + e, o);
       } else {
@@ -261,13 +280,11 @@ ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
         packed.y = pack4_i8(float2int8(o[4], quant_scale), float2int8(o[5], quant_scale),
                             float2int8(o[6], quant_scale), float2int8(o[7], quant_scale));
         *reinterpret_cast<uint2*>(out_q + base + e) = packed;
-        float rb[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        if (residual_bias != nullptr) ld8(residual_bias, e, rb);
         float w[8];
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           float keep = is_post_ln ? o[k] : x[it][k];
-          w[k] = (MODE == kLnFirst) ? keep + rb[k] : TT<T>::rnd(keep) + rb[k];
+          w[k] = (MODE == kLnFirst) ? keep + rbs[it][k] : TT<T>::rnd(keep) + rbs[it][k];
         }
         st8(residual, base + e, w);
       }

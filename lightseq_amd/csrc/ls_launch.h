@@ -115,6 +115,13 @@ int gemm_i8_i8o(const int8_t* A, const int8_t* W, int8_t* C, int M, int N, int K
 int gemm_i8_bias_act_i8o(const int8_t* A, const int8_t* W, int8_t* C, const __half* bias, int M,
                          int N, int K, float alpha, float dequant_scale, float quant_scale,
                          float clip_max, int act, hipStream_t s);
+// The same epilogue as a table lookup: `lut` [N, 256] int8, entry [n][code + 128] = what
+// gemm_i8_bias_act_i8o produces for requantised code `code` in column n; built once per
+// weight matrix by build_act_lut.  Bit-identical to gemm_i8_bias_act_i8o.
+int build_act_lut(int8_t* lut, const __half* bias, int N, float dequant_scale, float quant_scale,
+                  float clip_max, int act, hipStream_t s);
+int gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int M, int N,
+                    int K, float alpha, hipStream_t s);
 //   writes q, k, v as fp16 [B, h, S, d] at new_qkv + {0, 1, 2} * max_batch_dim
 int gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, __half* new_qkv,
                             const __half* qkv_bias, long max_batch_dim, int batch_tokens,

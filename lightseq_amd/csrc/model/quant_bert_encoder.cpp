@@ -71,6 +71,14 @@ void QuantBertEncoder::init_buffer() {
     d.w_out = upload_kernel(w.multihead_project_kernel_output, H, H, true, _stream);
     d.w_ffn1 = upload_kernel(w.ffn_first_kernel, H, I, true, _stream);
     d.w_ffn2 = upload_kernel(w.ffn_second_kernel, I, H, true, _stream);
+    {
+      // table of the FFN1 epilogue (dequantise, bias, activation, requantise) per output code
+      const float* c = &_enc_clip_max[l * _tw._clip_stride];
+      d.ffn1_act_lut.alloc((size_t)I * 256);
+      LSH_CALL(build_act_lut(d.ffn1_act_lut.get(), d.b_ffn1.get(), I, c[10] / _quant_range,
+                             _quant_range / c[7], c[7],
+                             _tw._use_gelu ? kActGelu : kActReluNarrow, _stream));
+    }
     if (!_tw._use_gelu) {
       // ReLU offset trick: colsum of the fp16-rounded dequantised FFN2 weight times
       // clip/2 (quant_bert_encoder.cc.cu:156-175)
@@ -230,10 +238,10 @@ void QuantBertEncoder::ffn_add_norm() {
   const int act = _tw._use_gelu ? kActGelu : kActReluNarrow;
   int8_t* act_buf = _int8_ffn_in_buf.get();
   if (_fuse && !tap_ffn1) {
-    prof_begin(2, M, I, H, gemm_i8_act_epilogue_name(act));
-    LSH_CALL(gemm_i8_bias_act_i8o(_int8_ffn_in_buf.get(), w.w_ffn1.get(), _int8_ffn_out_buf.get(),
-                                  w.b_ffn1.get(), M, I, H, c[2] * c[6] / (c[10] * Q), c[10] / Q,
-                                  Q / c[7], c[7], act, _stream));
+    (void)act;
+    prof_begin(2, M, I, H, "EpiLutI8");
+    LSH_CALL(gemm_i8_lut_i8o(_int8_ffn_in_buf.get(), w.w_ffn1.get(), _int8_ffn_out_buf.get(),
+                             w.ffn1_act_lut.get(), M, I, H, c[2] * c[6] / (c[10] * Q), _stream));
     act_buf = _int8_ffn_out_buf.get();
   } else {
     prof_begin(2, M, I, H, "EpiI8");

@@ -160,6 +160,13 @@ void QuantDecoder::init_buffer() {
     d.w_encdec_q = upload_kernel(w.encdec_project_kernel_q, H, H, true, _stream);
     d.w_encdec_out = upload_kernel(w.encdec_project_kernel_output, H, H, true, _stream);
     d.w_ffn1 = upload_kernel(w.ffn_first_kernel, H, I, true, _stream);
+    {
+      const float* c = &_dec_clip_max[l * 19];
+      d.ffn1_act_lut.alloc((size_t)I * 256);
+      LSH_CALL(build_act_lut(d.ffn1_act_lut.get(), d.b_ffn1.get(), I, c[16] / _quant_range,
+                             _quant_range / c[11], c[11],
+                             _tw._use_gelu ? kActGelu : kActReluNarrow, _stream));
+    }
     d.w_ffn2 = upload_kernel(w.ffn_second_kernel, I, H, true, _stream);
     if (!_tw._use_gelu) {
       // ReLU offset trick (:332-354): column sums of the fp16-rounded dequantised FFN2
@@ -329,10 +336,8 @@ void QuantDecoder::ffn_add_norm() {
   const float Q = _quant_range;
 
   // FFN1 GEMM with the bias + activation + requantisation in its epilogue
-  const int act = _tw._use_gelu ? kActGelu : kActReluNarrow;
-  LSH_CALL(gemm_i8_bias_act_i8o(_buf_b.get(), w.w_ffn1.get(), _buf_a.get(), w.b_ffn1.get(), M, I,
-                                H, c[4] * c[10] / (c[16] * Q), c[16] / Q, Q / c[11], c[11], act,
-                                _stream));
+  LSH_CALL(gemm_i8_lut_i8o(_buf_b.get(), w.w_ffn1.get(), _buf_a.get(), w.ffn1_act_lut.get(), M, I,
+                           H, c[4] * c[10] / (c[16] * Q), _stream));
   int nparts = 1;
   LSH_CALL(gemm_i8_i32o_splitk(_buf_a.get(), w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I,
                                gemm_i8_preferred_ksplit(M, H, I), &nparts, _stream));

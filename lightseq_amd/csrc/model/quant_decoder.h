@@ -94,6 +94,7 @@ class QuantDecoder {
       _kv_bias, _logit_bias;
   struct Layer {
     DeviceBuffer<int8_t> w_self_qkv, w_self_out, w_encdec_q, w_encdec_out, w_ffn1, w_ffn2;
+    DeviceBuffer<int8_t> ffn1_act_lut;  // [inner, 256]: bias + activation + requant per code
     DeviceBuffer<__half> self_ln_scale, self_ln_bias, b_self_qkv, b_self_out, encdec_ln_scale,
         encdec_ln_bias, b_encdec_q, b_encdec_out, ffn_ln_scale, ffn_ln_bias, b_ffn1, b_ffn2,
         ffn2_colsum;

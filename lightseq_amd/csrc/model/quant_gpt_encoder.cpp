@@ -96,6 +96,12 @@ void QuantGptEncoder::init_buffer() {
     d.w_qkv = upload_kernel(w.multihead_project_kernel_qkv, H, 3 * H, true, _stream);
     d.w_out = upload_kernel(w.multihead_project_kernel_output, H, H, true, _stream);
     d.w_ffn1 = upload_kernel(w.ffn_first_kernel, H, I, true, _stream);
+    {
+      const float* c = &_enc_clip_max[l * 12];
+      d.ffn1_act_lut.alloc((size_t)I * 256);
+      LSH_CALL(build_act_lut(d.ffn1_act_lut.get(), d.b_ffn1.get(), I, c[10] / _quant_range,
+                             _quant_range / c[7], c[7], kActGelu, _stream));
+    }
     d.w_ffn2 = upload_kernel(w.ffn_second_kernel, I, H, true, _stream);
   }
   CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
@@ -108,9 +114,8 @@ void QuantGptEncoder::ffn_add_norm(int rows, int8_t* in, int8_t* tmp) {
   const Layer& w = _layers[_layer_id];
   const float* c = &_enc_clip_max[_layer_id * 12];
   const float Q = _quant_range;
-  LSH_CALL(gemm_i8_bias_act_i8o(in, w.w_ffn1.get(), tmp, w.b_ffn1.get(), rows, I, H,
-                                c[2] * c[6] / (c[10] * Q), c[10] / Q, Q / c[7], c[7], kActGelu,
-                                _stream));
+  LSH_CALL(gemm_i8_lut_i8o(in, w.w_ffn1.get(), tmp, w.ffn1_act_lut.get(), rows, I, H,
+                           c[2] * c[6] / (c[10] * Q), _stream));
   int nparts = 1;
   LSH_CALL(gemm_i8_i32o_splitk(tmp, w.w_ffn2.get(), _int32_ffn_out_buf.get(), rows, H, I,
                                rows <= 64 ? gemm_i8_preferred_ksplit(rows, H, I)

@@ -77,6 +77,7 @@ class QuantGptEncoder {
   DeviceBuffer<__half> _pos_emb, _out_ln_scale, _out_ln_bias;
   struct Layer {
     DeviceBuffer<int8_t> w_qkv, w_out, w_ffn1, w_ffn2;
+    DeviceBuffer<int8_t> ffn1_act_lut;  // [inner, 256]: bias + GELU + requant per code
     DeviceBuffer<__half> ln1_scale, ln1_bias, b_qkv, b_out, ln2_scale, ln2_bias, b_ffn1, b_ffn2;
   };
   std::vector<Layer> _layers;

@@ -487,3 +487,17 @@ __all__ = [n for n in dir() if n.startswith(("launch_", "ker_", "gemm_", "encsel
                                              "decself_", "encdec_", "select_beam_", "beam_",
                                              "refresh_", "length_norm"))]
 _ = lib  # re-exported for callers that want lib.LSHError
+
+
+def build_act_lut(lut, bias, n, dequant_scale, quant_scale, clip_max, act):
+    """lut [n, 256] int8: bias + activation + requantisation per (column, code); act 0 GELU,
+    1 ReLU, 2 ReLU with the narrow unsigned clip."""
+    _dev(lut, bias)
+    call("lsh_build_act_lut", ptr(lut), ptr(bias), n, dequant_scale, quant_scale, clip_max, act,
+         current_stream())
+
+
+def gemm_i8_lut_i8o(a, w, c, lut, m, n, k, alpha):
+    """int8-output GEMM whose epilogue is the table built by :func:`build_act_lut`."""
+    _dev(a, w, c, lut)
+    call("lsh_gemm_i8_lut_i8o", ptr(a), ptr(w), ptr(c), ptr(lut), m, n, k, alpha, current_stream())

@@ -47,6 +47,8 @@ _SIGNATURES = {
     "lsh_launch_scaled_colsum": (True, "ppiifs"),
     "lsh_gemm_i8_i32o": (False, "pppiiis"),
     "lsh_gemm_i8_i8o": (False, "pppiiifs"),
+    "lsh_build_act_lut": (False, "pp" + "ifffi" + "s"),
+    "lsh_gemm_i8_lut_i8o": (False, "pppp" + "iiif" + "s"),
     "lsh_gemm_i8_i32o_splitk": (False, "ppp" + "iiii" + "p" + "s"),
     "lsh_gemm_i8_preferred_ksplit": (False, "iii"),
     "lsh_ker_residual_bias_ln_planes_i32I_i8O_f16": (False, "p" + "il" + "ppppp" + "iiff" + "s" +

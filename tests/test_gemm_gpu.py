@@ -126,6 +126,12 @@ def test_fused_bias_act_epilogue_equals_unfused_pair(rng, M, N, K, act):
         k.ker_bias_relu_i8I_i8O_launcher(M, tmp, want, bias, N, ds, qs, clip, False, False, narrow)
         k.gemm_i8_bias_relu_i8o(a, w, got, bias, M, N, K, alpha, ds, qs, clip, narrow)
     assert torch.equal(got, want)
+    # and the same epilogue as a per-column table of the 256 codes
+    lut = torch.zeros((N, 256), dtype=torch.int8, device=DEV)
+    k.build_act_lut(lut, bias, N, ds, qs, clip, {"gelu": 0, "relu": 1, "relu_narrow": 2}[act])
+    via_lut = torch.zeros_like(tmp)
+    k.gemm_i8_lut_i8o(a, w, via_lut, lut, M, N, K, alpha)
+    assert torch.equal(via_lut, want)
 
 
 @pytest.mark.parametrize("B,S,h,d,K", [(2, 16, 2, 64, 128), (32, 128, 12, 64, 768), (3, 10, 4, 16, 64)])
@@ -171,7 +177,7 @@ def test_split_k_planes_sum_to_the_product(rng, M, N, K, ksplit):
     # a split that does not divide K into whole 128-byte steps is not applied
     c1 = torch.zeros((3, M, N), dtype=torch.int32, device=DEV)
     assert _k().gemm_i8_i32o_splitk(to_dev(a), to_dev(w), c1, M, N, K, 3) == (3 if (K // 128) % 3 == 0 else 1)
-    assert _k().gemm_i8_preferred_ksplit(4096, 768, 3072) == 2
+    assert _k().gemm_i8_preferred_ksplit(4096, 768, 3072) == 1  # encoder sizes: not worth the planes
     assert _k().gemm_i8_preferred_ksplit(16, 1024, 4096) == 8
     assert _k().gemm_i8_preferred_ksplit(4096, 3072, 768) == 1
 
