@@ -191,6 +191,25 @@ def gemm_microbench(reps=40):
     return out
 
 
+TRAFFIC_SUMMARY = "bert_base_b32_s128_pmc_hbm_traffic.txt"
+
+
+def _profiled_traffic(kernel):
+    """HBM bytes per launch of ``kernel`` from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE and WRITE_SIZE runs of this same command, scaled by a plain copy kernel);
+    None when the summary holds no line for that kernel."""
+    import re
+    path = os.path.join(ROOT, "profiles", TRAFFIC_SUMMARY)
+    if not os.path.exists(path):
+        return None
+    short = kernel.replace("EpiGeluI8", "EpiActI8<0>")
+    for line in open(path):
+        m = re.match(r"traffic_bytes_per_launch\[(.+?)\] = (\d+)", line)
+        if m and m.group(1).replace("lsh::", "") == short:
+            return int(m.group(2))
+    return None
+
+
 def bench_bert(args):
     import torch
     from lightseq_amd import inference, synthetic
@@ -231,7 +250,8 @@ def bench_bert(args):
     avg_ms = dom["ms"] / dom["launches"]
     achieved = dom["ops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                "frac": achieved / INT8_MFMA_PEAK_TOPS, "traffic": None, "kernel": name,
+                "frac": achieved / INT8_MFMA_PEAK_TOPS, "traffic": _profiled_traffic(name),
+                "traffic_source": "profiles/" + TRAFFIC_SUMMARY, "kernel": name,
                 "sites": dom["sites"], "avg_launch_us": avg_ms * 1e3,
                 "gemm_sites": {s["site"]: {"kernel": s["kernel"], "mnk": [s["m"], s["n"], s["k"]],
                                            "avg_us": 1e3 * s["total_ms"] / max(1, s["launches"]),
@@ -330,6 +350,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true",
                     help="skip the stand-alone timing of the fused kernels")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 256 MiB device copies, a kernel of known HBM "
+                         "traffic against which profiler byte counters are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU only (every model object owns device 0 and "
@@ -343,6 +366,12 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     out = bench_bert(args) if bert else bench_generation(args)
     print(json.dumps(out))
 
