@@ -186,6 +186,16 @@ int lsh_encself_attention_f16(const void* q, const void* k, const void* v,
                               const int* src_padding_mask, void* ctx, int8_t* ctx_q,
                               float quant_scale, int batch_size, int batch_seq_len, int head_num,
                               int dim_per_head, lsh_stream_t stream);
+/* The same sequence preceded by ker_arrange_encself_qkv_i8I
+ * (kernels/transformerKernels_int8.cc.cu:1119-1172; call site
+ * model/quant_bert_encoder.cc.cu:313-319): qkv is the int8 output of the QKV product,
+ * [batch*seq_len, 3*hidden], qkv_bias fp16 [3*hidden]; each element is dequantised to
+ * half(half(code * dequant_scale) + bias) as it is read, so the fp16 q, k, v tensors
+ * are never written. */
+int lsh_encself_attention_i8qkv_f16(const int8_t* qkv, const void* qkv_bias, float dequant_scale,
+                                    const int* src_padding_mask, void* ctx, int8_t* ctx_q,
+                                    float quant_scale, int batch_size, int batch_seq_len,
+                                    int head_num, int dim_per_head, lsh_stream_t stream);
 
 /* ---- embedding ------------------------------------------------------------------------ */
 /* kernels/embKernels_int8.h:7-13 */

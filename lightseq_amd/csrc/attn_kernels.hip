@@ -88,7 +88,7 @@ template int correlation_softmax_encself<__half>(int, int, int, hipStream_t, __h
 // ---------------------------------------------------------------------------------
 // Fused encoder attention.
 //
-// Grid (ceil(S/64), B*h), 128 threads = 2 wavefronts, 32 queries per wavefront.
+// Grid (ceil(S / (32 NW)), B*h), NW wavefronts (2 or 4), 32 queries per wavefront.
 // Keys are processed in blocks of 128: K block row-major and V block transposed
 // are staged in LDS.  Scores are computed transposed (S^T = K Q^T) with
 // v_mfma_f32_32x32x16_f16 so that one lane owns one query: the row max / sum need
@@ -116,10 +116,51 @@ __device__ __forceinline__ float round_h(float x) { return (float)(_Float16)x; }
 // T=half mask [batch, S] (0 for tokens, a large negative value for padding), no query row
 // is zeroed, a non-zero `dq` masks future keys, and the context is written with the heads
 // merged, fp16 [batch, S, head_num * D].
-constexpr int kAttnEnc = 0, kAttnGpt = 1, kAttnLayer = 2;
+//
+// MODE 3 is MODE 0 reading the int8 output of the QKV product directly
+// (inference/model/quant_bert_encoder.cc.cu:305-319 leaves it as [tokens, 3 * hidden]
+// codes; ker_arrange_encself_qkv_i8I, transformerKernels_int8.cc.cu:1119-1172, turns
+// them into fp16 q, k, v): `q` points to the codes, `k` to the fp16 bias [3 * hidden],
+// `dq` is the dequantisation scale, and every element becomes
+// half(half(code * dq) + bias) while it is staged, which is what the arrange kernel
+// would have stored.  The fp16 q, k, v tensors are never written.
+constexpr int kAttnEnc = 0, kAttnGpt = 1, kAttnLayer = 2, kAttnEncI8 = 3;
 
-template <int D, int MODE>
-__global__ void __launch_bounds__(128)
+template <int N>
+__device__ __forceinline__ float ubyte_f32(uint32_t w) {  // one v_cvt_f32_ubyteN
+  return (float)((w >> (8 * N)) & 0xffu);
+}
+
+// 16 int8 codes -> 16 fp16 values half(half(code * dq) + bias)
+__device__ __forceinline__ void dequant16_bias(const uint4& w, const _Float16* __restrict__ bias,
+                                               float dq, v8h& lo, v8h& hi) {
+  // float(code) * dq == fma(float(code + 128), dq, -128 * dq): the product is exact before
+  // its single rounding either way, and -128 * dq is exact.  half(x) + half(b) in fp16
+  // arithmetic == half(float(x) + float(b)): the float sum of two halfs is exact unless
+  // one is below a quarter of the other's last place, where both round to the larger one.
+  const v8h b0 = *reinterpret_cast<const v8h*>(bias);
+  const v8h b1 = *reinterpret_cast<const v8h*>(bias + 8);
+  const float off = -128.f * dq;
+  const uint32_t u[4] = {w.x ^ 0x80808080u, w.y ^ 0x80808080u, w.z ^ 0x80808080u,
+                         w.w ^ 0x80808080u};
+  v8h xl, xh;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    xl[4 * j + 0] = (_Float16)fmaf(ubyte_f32<0>(u[j]), dq, off);
+    xl[4 * j + 1] = (_Float16)fmaf(ubyte_f32<1>(u[j]), dq, off);
+    xl[4 * j + 2] = (_Float16)fmaf(ubyte_f32<2>(u[j]), dq, off);
+    xl[4 * j + 3] = (_Float16)fmaf(ubyte_f32<3>(u[j]), dq, off);
+    xh[4 * j + 0] = (_Float16)fmaf(ubyte_f32<0>(u[2 + j]), dq, off);
+    xh[4 * j + 1] = (_Float16)fmaf(ubyte_f32<1>(u[2 + j]), dq, off);
+    xh[4 * j + 2] = (_Float16)fmaf(ubyte_f32<2>(u[2 + j]), dq, off);
+    xh[4 * j + 3] = (_Float16)fmaf(ubyte_f32<3>(u[2 + j]), dq, off);
+  }
+  lo = xl + b0;
+  hi = xh + b1;
+}
+
+template <int D, int MODE, int NW>
+__global__ void __launch_bounds__(64 * NW)
 encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
                     const __half* __restrict__ v, const int* __restrict__ pad_mask,
                     __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale, int S,
@@ -127,8 +168,8 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   constexpr int KSTR = D + 8;    // halfs per K row in LDS (pad kills bank conflicts)
   constexpr int VSTR = 128 + 4;  // halfs per V^T row in LDS
   constexpr int CH = D / 8;      // 16-byte chunks per row
-  __shared__ _Float16 Ks[128 * KSTR];
-  __shared__ _Float16 Vt[D * VSTR];
+  __shared__ __align__(16) _Float16 Ks[128 * KSTR];
+  __shared__ __align__(16) _Float16 Vt[D * VSTR];
   __shared__ int msk[128];
   __shared__ float addm[MODE == kAttnLayer ? 128 : 1];
   constexpr bool GPT = MODE == kAttnGpt;
@@ -138,18 +179,47 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   const int l32 = lane & 31, g = lane >> 5;
   const int bh = blockIdx.y;
   const int b = bh / head_num, head = bh % head_num;
-  const int qi = blockIdx.x * 64 + wave * 32 + l32;
+  constexpr int NT = 64 * NW;  // threads; 32 queries per wavefront
+  const int qi = blockIdx.x * (32 * NW) + wave * 32 + l32;
   const _Float16* qb = reinterpret_cast<const _Float16*>(q) + (long)bh * S * D;
   const _Float16* kbase = reinterpret_cast<const _Float16*>(k) + (long)bh * S * D;
   const _Float16* vbase = reinterpret_cast<const _Float16*>(v) + (long)bh * S * D;
 
+  // MODE 3: int8 codes [tokens, 3 * hidden] and the fp16 bias [3 * hidden]
+  const int hidden3 = 3 * head_num * D;
+  const int8_t* codes = reinterpret_cast<const int8_t*>(q) + (long)b * S * hidden3 + head * D;
+  const _Float16* bias = reinterpret_cast<const _Float16*>(k) + head * D;
+
   v8h qreg[D / 16];
+  if (MODE == kAttnEncI8) {
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) {
-    if (qi < S)
-      qreg[ks] = *reinterpret_cast<const v8h*>(qb + (long)qi * D + ks * 16 + g * 8);
-    else
-      qreg[ks] = (v8h)(_Float16)0;
+    for (int kp = 0; kp < D / 32; ++kp) {
+      // lane half g converts chunk kp * 32 + g * 16 .. + 16, then the halves swap their
+      // second part so that lane (l32, g) ends with d = ks * 16 + g * 8 .. + 8 for both ks
+      v8h lo = (v8h)(_Float16)0, hi = (v8h)(_Float16)0;
+      if (qi < S) {
+        const uint4 w =
+            *reinterpret_cast<const uint4*>(codes + (long)qi * hidden3 + kp * 32 + g * 16);
+        dequant16_bias(w, bias + kp * 32 + g * 16, dq, lo, hi);
+      }
+      // lane g=0 holds d 0..15 of this 32-block, lane g=1 holds d 16..31
+      v8h give = g == 0 ? hi : lo, take;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int t = __shfl_xor(reinterpret_cast<const int*>(&give)[j], 32, 64);
+        reinterpret_cast<int*>(&take)[j] = t;
+      }
+      qreg[2 * kp] = g == 0 ? lo : take;      // d = kp*32 + g*8 .. + 8
+      qreg[2 * kp + 1] = g == 0 ? take : hi;  // d = kp*32 + 16 + g*8 .. + 8
+    }
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) {
+      if (qi < S)
+        qreg[ks] = *reinterpret_cast<const v8h*>(qb + (long)qi * D + ks * 16 + g * 8);
+      else
+        qreg[ks] = (v8h)(_Float16)0;
+    }
   }
   const bool q_pad = qi >= S || (MODE == kAttnLayer ? false
                                  : GPT              ? qi >= pad_mask[b]
@@ -164,7 +234,7 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
   int nkb = (S + 127) / 128;
-  if (causal) nkb = min(nkb, min((int)blockIdx.x * 64 + 63, S - 1) / 128 + 1);
+  if (causal) nkb = min(nkb, min((int)(blockIdx.x + 1) * (32 * NW) - 1, S - 1) / 128 + 1);
   for (int phase = 0; phase < 2; ++phase) {
     for (int kb = 0; kb < nkb; ++kb) {
       const int key0 = kb * 128;
@@ -172,29 +242,83 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
       if (fresh) {
         __syncthreads();
         const bool want_v = phase == 1 || nkb == 1;
-        for (int c = tid; c < 128 * CH; c += 128) {
-          const int row = c / CH, ch = c % CH;
-          const int key = key0 + row;
-          v8h kv = (v8h)(_Float16)0, vv = (v8h)(_Float16)0;
-          if (key < S) {
-            kv = *reinterpret_cast<const v8h*>(kbase + (long)key * D + ch * 8);
-            if (want_v) vv = *reinterpret_cast<const v8h*>(vbase + (long)key * D + ch * 8);
+        if (MODE == kAttnEncI8) {
+          constexpr int C16 = D / 16;  // 16-code chunks per row
+          const int hid = head_num * D;
+          for (int c = tid; c < 128 * C16; c += NT) {
+            const int row = c / C16, ch = c % C16;
+            v8h lo = (v8h)(_Float16)0, hi = (v8h)(_Float16)0;
+            if (key0 + row < S) {
+              const uint4 w = *reinterpret_cast<const uint4*>(
+                  codes + (long)(key0 + row) * hidden3 + hid + ch * 16);
+              dequant16_bias(w, bias + hid + ch * 16, dq, lo, hi);
+            }
+            *reinterpret_cast<v8h*>(&Ks[row * KSTR + ch * 16]) = lo;
+            *reinterpret_cast<v8h*>(&Ks[row * KSTR + ch * 16 + 8]) = hi;
           }
-          *reinterpret_cast<v8h*>(&Ks[row * KSTR + ch * 8]) = kv;
           if (want_v) {
+            // a lane transposes a patch of 4 keys x 16 dims: 16 stores of 4 keys each
+            for (int p = tid; p < 32 * C16; p += NT) {
+              const int kg = p / C16, ch = p % C16;
+              v8h lo[4], hi[4];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) Vt[(ch * 8 + i) * VSTR + row] = vv[i];
+              for (int r = 0; r < 4; ++r) {
+                lo[r] = (v8h)(_Float16)0;
+                hi[r] = (v8h)(_Float16)0;
+                const int key = key0 + kg * 4 + r;
+                if (key < S) {
+                  const uint4 w = *reinterpret_cast<const uint4*>(
+                      codes + (long)key * hidden3 + 2 * hid + ch * 16);
+                  dequant16_bias(w, bias + 2 * hid + ch * 16, dq, lo[r], hi[r]);
+                }
+              }
+#pragma unroll
+              for (int i = 0; i < 8; ++i) {
+                *reinterpret_cast<v4h*>(&Vt[(ch * 16 + i) * VSTR + kg * 4]) =
+                    (v4h){lo[0][i], lo[1][i], lo[2][i], lo[3][i]};
+                *reinterpret_cast<v4h*>(&Vt[(ch * 16 + 8 + i) * VSTR + kg * 4]) =
+                    (v4h){hi[0][i], hi[1][i], hi[2][i], hi[3][i]};
+              }
+            }
+          }
+        } else {
+          for (int c = tid; c < 128 * CH; c += NT) {
+            const int row = c / CH, ch = c % CH;
+            v8h kv = (v8h)(_Float16)0;
+            if (key0 + row < S)
+              kv = *reinterpret_cast<const v8h*>(kbase + (long)(key0 + row) * D + ch * 8);
+            *reinterpret_cast<v8h*>(&Ks[row * KSTR + ch * 8]) = kv;
+          }
+          if (want_v) {
+            // a lane transposes a patch of 4 keys x 8 dims: 8 stores of 4 keys each
+            for (int p = tid; p < 32 * CH; p += NT) {
+              const int kg = p / CH, ch = p % CH;
+              v8h vv[4];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int key = key0 + kg * 4 + r;
+                vv[r] = key < S ? *reinterpret_cast<const v8h*>(vbase + (long)key * D + ch * 8)
+                                : (v8h)(_Float16)0;
+              }
+#pragma unroll
+              for (int i = 0; i < 8; ++i)
+                *reinterpret_cast<v4h*>(&Vt[(ch * 8 + i) * VSTR + kg * 4]) =
+                    (v4h){vv[0][i], vv[1][i], vv[2][i], vv[3][i]};
+            }
           }
         }
-        if (MODE == kAttnLayer) {
-          msk[tid] = (key0 + tid < S) ? 0 : 1;
-          addm[tid] = (key0 + tid < S && pad_mask != nullptr)
-                          ? __half2float(reinterpret_cast<const __half*>(pad_mask)[(long)b * S + key0 + tid])
-                          : 0.f;
-        } else if (GPT) {
-          msk[tid] = (key0 + tid < S) ? 0 : 1;
-        } else {
-          msk[tid] = (key0 + tid < S) ? pad_mask[(long)b * S + key0 + tid] : 1;
+        if (tid < 128) {
+          if (MODE == kAttnLayer) {
+            msk[tid] = (key0 + tid < S) ? 0 : 1;
+            addm[tid] = (key0 + tid < S && pad_mask != nullptr)
+                            ? __half2float(reinterpret_cast<const __half*>(
+                                  pad_mask)[(long)b * S + key0 + tid])
+                            : 0.f;
+          } else if (GPT) {
+            msk[tid] = (key0 + tid < S) ? 0 : 1;
+          } else {
+            msk[tid] = (key0 + tid < S) ? pad_mask[(long)b * S + key0 + tid] : 1;
+          }
         }
         __syncthreads();
 #pragma unroll
@@ -236,12 +360,24 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb)
 #pragma unroll
-          for (int i = 0; i < 16; ++i)
-            part += sc[sb][i] == kFloatInfNeg ? 0.f : __expf(sc[sb][i] - m_new);
+          for (int i = 0; i < 16; ++i) {
+            const float e = sc[sb][i] == kFloatInfNeg ? 0.f : __expf(sc[sb][i] - m_new);
+            part += e;
+            if (nkb == 1) sc[sb][i] = e;  // single key block: the second pass reuses it
+          }
         part += __shfl_xor(part, 32, 64);
         sum = sum * __expf(m - m_new) + part;
         m = m_new;
       } else {
+        // exp / sum is the correctly rounded quotient, as the reference's division gives:
+        // exp * (1 / sum) differs from it by one unit in the last place often enough to flip
+        // fp16 probabilities, and a deep stack amplifies such flips.  The quotient is formed
+        // by the sequence the compiler emits for a float division (refined reciprocal, two
+        // residual corrections) with the reciprocal taken once per query and without the
+        // range scaling, which only acts on quotients far below the smallest fp16 value.
+        const bool no_keys = !(sum > 0.f);
+        float rs = __builtin_amdgcn_rcpf(sum);
+        rs = fmaf(fmaf(-sum, rs, 1.f), rs, rs);
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb) {
 #pragma unroll
@@ -250,7 +386,11 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
               const float s = sc[sb][8 * t + j];
-              pb[j] = (_Float16)(s == kFloatInfNeg ? 0.f : __expf(s - m) / sum);
+              const float e = nkb == 1 ? s : (s == kFloatInfNeg ? 0.f : __expf(s - m));
+              float qt = e * rs;
+              qt = fmaf(fmaf(-sum, qt, e), rs, qt);
+              qt = fmaf(fmaf(-sum, qt, e), rs, qt);
+              pb[j] = (_Float16)(no_keys ? 0.f : qt);
             }
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) {
@@ -295,6 +435,34 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   }
 }
 
+// 4 wavefronts (128 queries) per workgroup once a sequence has more than 64 queries, so
+// that a (batch, head) pair with up to 128 keys is staged once; 2 wavefronts otherwise.
+template <int MODE>
+static bool launch_attn(int dim_per_head, int seq_len, int batch_heads, hipStream_t s,
+                        const __half* q, const __half* k, const __half* v, const int* pad_mask,
+                        __half* ctx, int8_t* ctx_q, float quant_scale, int head_num, float alpha,
+                        float dq) {
+#define LSH_ATTN(DD, NWV)                                                                      \
+  encself_attn_kernel<DD, MODE, NWV>                                                           \
+      <<<dim3((seq_len + 32 * NWV - 1) / (32 * NWV), batch_heads), 64 * NWV, 0, s>>>(          \
+          q, k, v, pad_mask, ctx, ctx_q, quant_scale, seq_len, head_num, alpha, dq)
+  const bool wide = seq_len > 64;
+  switch (dim_per_head) {
+    case 32:
+      if (wide) LSH_ATTN(32, 4); else LSH_ATTN(32, 2);
+      return true;
+    case 64:
+      if (wide) LSH_ATTN(64, 4); else LSH_ATTN(64, 2);
+      return true;
+    case 128:
+      if (wide) LSH_ATTN(128, 4); else LSH_ATTN(128, 2);
+      return true;
+    default:
+      return false;
+  }
+#undef LSH_ATTN
+}
+
 int encself_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,
                           __half* ctx, int8_t* ctx_q, float quant_scale, int batch, int seq_len,
                           int head_num, int dim_per_head, hipStream_t s) {
@@ -307,27 +475,32 @@ int encself_attention_f16(const __half* q, const __half* k, const __half* v, con
         reinterpret_cast<uintptr_t>(ctx_q)) & 15u) != 0)
     return lsh_fail(LSH_ERR_INVALID, "encself_attention: pointers must be 16-byte aligned");
   const float alpha = __half2float(__float2half_rn(sqrtf(1.f / (float)dim_per_head)));
-  dim3 grid((seq_len + 63) / 64, batch * head_num);
-  switch (dim_per_head) {
-    case 32:
-      encself_attn_kernel<32, kAttnEnc><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
-                                                          quant_scale, seq_len, head_num, alpha,
-                                                          0.f);
-      break;
-    case 64:
-      encself_attn_kernel<64, kAttnEnc><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
-                                                          quant_scale, seq_len, head_num, alpha,
-                                                          0.f);
-      break;
-    case 128:
-      encself_attn_kernel<128, kAttnEnc><<<grid, 128, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q,
-                                                           quant_scale, seq_len, head_num, alpha,
-                                                           0.f);
-      break;
-    default:
-      return lsh_fail(LSH_ERR_UNSUPPORTED, "encself_attention: dim_per_head must be 32, 64 or 128");
-  }
+  if (!launch_attn<kAttnEnc>(dim_per_head, seq_len, batch * head_num, s, q, k, v, pad_mask, ctx,
+                             ctx_q, quant_scale, head_num, alpha, 0.f))
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "encself_attention: dim_per_head must be 32, 64 or 128");
   return lsh_check_launch("encself_attn_kernel");
+}
+
+// The same attention reading the int8 output of the QKV product [batch * seq_len,
+// 3 * hidden] and the fp16 bias [3 * hidden] (MODE 3 above).
+int encself_attention_i8qkv(const int8_t* qkv, const __half* qkv_bias, float dequant_scale,
+                            const int* pad_mask, __half* ctx, int8_t* ctx_q, float quant_scale,
+                            int batch, int seq_len, int head_num, int dim_per_head, hipStream_t s) {
+  if (batch <= 0 || seq_len <= 0 || head_num <= 0 || !qkv || !qkv_bias || !pad_mask ||
+      (!ctx && !ctx_q))
+    return lsh_fail(LSH_ERR_INVALID, "encself_attention_i8qkv: bad arguments");
+  if (seq_len > 1024)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "encself_attention_i8qkv: seq_len > 1024");
+  if (((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(qkv_bias) |
+        reinterpret_cast<uintptr_t>(ctx) | reinterpret_cast<uintptr_t>(ctx_q)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_INVALID, "encself_attention_i8qkv: pointers must be 16-byte aligned");
+  const float alpha = __half2float(__float2half_rn(sqrtf(1.f / (float)dim_per_head)));
+  const __half* q = reinterpret_cast<const __half*>(qkv);
+  if (!launch_attn<kAttnEncI8>(dim_per_head, seq_len, batch * head_num, s, q, qkv_bias, nullptr,
+                               pad_mask, ctx, ctx_q, quant_scale, head_num, alpha, dequant_scale))
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                        "encself_attention_i8qkv: dim_per_head must be 32, 64 or 128");
+  return lsh_check_launch("encself_attn_kernel<i8 qkv>");
 }
 
 int gpt_prefill_attention_f16(const __half* q_codes, const __half* k_codes, const __half* v,
@@ -344,27 +517,11 @@ int gpt_prefill_attention_f16(const __half* q_codes, const __half* k_codes, cons
         reinterpret_cast<uintptr_t>(ctx_q)) & 15u) != 0)
     return lsh_fail(LSH_ERR_INVALID, "gpt_prefill_attention: pointers must be 16-byte aligned");
   const float alpha = __half2float(__float2half_rn(sqrtf(1.f / (float)dim_per_head)));
-  dim3 grid((seq_len + 63) / 64, batch * head_num);
-  switch (dim_per_head) {
-    case 32:
-      encself_attn_kernel<32, kAttnGpt><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
-                                                         ctx_q, quant_scale, seq_len, head_num,
-                                                         alpha, dequant_scale);
-      break;
-    case 64:
-      encself_attn_kernel<64, kAttnGpt><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
-                                                         ctx_q, quant_scale, seq_len, head_num,
-                                                         alpha, dequant_scale);
-      break;
-    case 128:
-      encself_attn_kernel<128, kAttnGpt><<<grid, 128, 0, s>>>(q_codes, k_codes, v, real_seq_len, ctx,
-                                                          ctx_q, quant_scale, seq_len, head_num,
-                                                          alpha, dequant_scale);
-      break;
-    default:
-      return lsh_fail(LSH_ERR_UNSUPPORTED,
-                      "gpt_prefill_attention: dim_per_head must be 32, 64 or 128");
-  }
+  if (!launch_attn<kAttnGpt>(dim_per_head, seq_len, batch * head_num, s, q_codes, k_codes, v,
+                             real_seq_len, ctx, ctx_q, quant_scale, head_num, alpha,
+                             dequant_scale))
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                        "gpt_prefill_attention: dim_per_head must be 32, 64 or 128");
   return lsh_check_launch("encself_attn_kernel<GPT>");
 }
 
@@ -384,23 +541,9 @@ int layer_attention_f16(const __half* q, const __half* k, const __half* v, const
       __float2half_rn(1.0f / __half2float(__float2half_rn(sqrtf((float)dim_per_head)))));
   const int* m = reinterpret_cast<const int*>(add_mask);
   const float causal = mask_future ? 1.f : 0.f;
-  dim3 grid((seq_len + 63) / 64, batch * head_num);
-  switch (dim_per_head) {
-    case 32:
-      encself_attn_kernel<32, kAttnLayer><<<grid, 128, 0, s>>>(q, k, v, m, ctx, nullptr, 0.f,
-                                                               seq_len, head_num, alpha, causal);
-      break;
-    case 64:
-      encself_attn_kernel<64, kAttnLayer><<<grid, 128, 0, s>>>(q, k, v, m, ctx, nullptr, 0.f,
-                                                               seq_len, head_num, alpha, causal);
-      break;
-    case 128:
-      encself_attn_kernel<128, kAttnLayer><<<grid, 128, 0, s>>>(q, k, v, m, ctx, nullptr, 0.f,
-                                                                seq_len, head_num, alpha, causal);
-      break;
-    default:
-      return lsh_fail(LSH_ERR_UNSUPPORTED, "layer_attention: dim_per_head must be 32, 64 or 128");
-  }
+  if (!launch_attn<kAttnLayer>(dim_per_head, seq_len, batch * head_num, s, q, k, v, m, ctx,
+                               nullptr, 0.f, head_num, alpha, causal))
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "layer_attention: dim_per_head must be 32, 64 or 128");
   return lsh_check_launch("encself_attn_kernel<layer>");
 }
 

@@ -286,6 +286,14 @@ int lsh_encself_attention_f16(const void* q, const void* k, const void* v,
   return encself_attention_f16(H(q), H(k), H(v), src_padding_mask, HM(ctx), ctx_q, quant_scale,
                                batch_size, batch_seq_len, head_num, dim_per_head, HS(stream));
 }
+int lsh_encself_attention_i8qkv_f16(const int8_t* qkv, const void* qkv_bias, float dequant_scale,
+                                    const int* src_padding_mask, void* ctx, int8_t* ctx_q,
+                                    float quant_scale, int batch_size, int batch_seq_len,
+                                    int head_num, int dim_per_head, lsh_stream_t stream) {
+  return encself_attention_i8qkv(qkv, H(qkv_bias), dequant_scale, src_padding_mask, HM(ctx), ctx_q,
+                                 quant_scale, batch_size, batch_seq_len, head_num, dim_per_head,
+                                 HS(stream));
+}
 
 // ---- embedding ----------------------------------------------------------------------------------
 int lsh_launch_enc_emb_i8I_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,

@@ -96,6 +96,12 @@ int correlation_softmax_encself(int batch_size, int batch_seq_len, int head_num,
 int encself_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,
                           __half* ctx, int8_t* ctx_q, float quant_scale, int batch, int seq_len,
                           int head_num, int dim_per_head, hipStream_t s);
+// The same attention fed by the int8 output of the QKV product ([batch * seq_len,
+// 3 * hidden] codes) and the fp16 bias [3 * hidden]: each element is dequantised as
+// ker_arrange_encself_qkv_i8I would have stored it, while it is staged.
+int encself_attention_i8qkv(const int8_t* qkv, const __half* qkv_bias, float dequant_scale,
+                            const int* pad_mask, __half* ctx, int8_t* ctx_q, float quant_scale,
+                            int batch, int seq_len, int head_num, int dim_per_head, hipStream_t s);
 
 // ---- int8 MFMA GEMM (gemm_i8.hip) -----------------------------------------------------
 // C[M,N] = A[M,K] * W[N,K]^T, both operands K-contiguous.

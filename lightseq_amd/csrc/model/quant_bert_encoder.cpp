@@ -181,32 +181,28 @@ void QuantBertEncoder::self_attention() {
   }
   tap(taps.ln1_q, _int8_ffn_in_buf.get(), (size_t)M * H);
 
-  // qkv = ori_q * qkv_wei, int8 out
-  // qkv = ori_q * qkv_wei -> int8 code -> dequant + bias, split heads -> fp16 q, k, v
-  // [B, h, S, d].  Fused into the GEMM epilogue unless the int8 GEMM output is tapped
-  // (or the head size does not allow it); both routes give the same bits.
+  // qkv = ori_q * qkv_wei -> int8 codes [M, 3H].  The fused route hands the codes and the
+  // bias to the attention kernel, which dequantises them as it stages q, k, v; the unfused
+  // route writes fp16 q, k, v [B, h, S, d] first.  Both give the same bits.
   const long mbd = (long)M * H;
-  const bool tap_qkv = taps.qkv_q && taps.tap_layer == _layer_id;
-  if (_fuse && !tap_qkv && _tw._dim_per_head % 16 == 0) {
-    prof_begin(0, M, 3 * H, H, "EpiQkvF16");
-    LSH_CALL(gemm_i8_qkv_arrange_f16(_int8_ffn_in_buf.get(), w.w_qkv.get(), _qkv_buf.get(),
-                                     w.b_qkv.get(), mbd, M, H, H, _batch_seq_len, _tw._head_num,
-                                     c[0] * c[4] / (c[8] * Q), c[8] / Q, _stream));
+  prof_begin(0, M, 3 * H, H, "EpiI8");
+  LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_qkv.get(), _int8_ffn_out_buf.get(), M, 3 * H,
+                       H, c[0] * c[4] / (c[8] * Q), _stream));
+  tap(taps.qkv_q, _int8_ffn_out_buf.get(), (size_t)M * 3 * H);
+  const int dph = _tw._dim_per_head;
+  if (_fuse && (dph == 32 || dph == 64 || dph == 128)) {
+    // scores -> masked softmax -> context -> merge heads + quantise, one kernel
+    LSH_CALL(encself_attention_i8qkv(_int8_ffn_out_buf.get(), w.b_qkv.get(), c[8] / Q,
+                                     _p_d_padding_mask, nullptr, _int8_ffn_in_buf.get(), Q / c[5],
+                                     _batch_size, _batch_seq_len, _tw._head_num, dph, _stream));
   } else {
-    prof_begin(0, M, 3 * H, H, "EpiI8");
-    LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_qkv.get(), _int8_ffn_out_buf.get(), M, 3 * H,
-                         H, c[0] * c[4] / (c[8] * Q), _stream));
-    tap(taps.qkv_q, _int8_ffn_out_buf.get(), (size_t)M * 3 * H);
     LSH_CALL(arrange_encself_qkv_i8I<__half>(M, H, _stream, _int8_ffn_out_buf.get(),
                                              w.b_qkv.get(), _qkv_buf.get(), mbd, _batch_seq_len,
-                                             _tw._dim_per_head, _tw._head_num, c[8] / Q));
+                                             dph, _tw._head_num, c[8] / Q));
+    LSH_CALL(encself_attention_f16(_qkv_buf.get(), _qkv_buf.get() + mbd, _qkv_buf.get() + 2 * mbd,
+                                   _p_d_padding_mask, nullptr, _int8_ffn_in_buf.get(), Q / c[5],
+                                   _batch_size, _batch_seq_len, _tw._head_num, dph, _stream));
   }
-
-  // scores -> masked softmax -> context -> merge heads + quantise, one kernel
-  LSH_CALL(encself_attention_f16(_qkv_buf.get(), _qkv_buf.get() + mbd, _qkv_buf.get() + 2 * mbd,
-                                 _p_d_padding_mask, nullptr, _int8_ffn_in_buf.get(), Q / c[5],
-                                 _batch_size, _batch_seq_len, _tw._head_num, _tw._dim_per_head,
-                                 _stream));
   tap(taps.ctx_q, _int8_ffn_in_buf.get(), (size_t)M * H);
 
   prof_begin(1, M, H, H, "EpiI8");

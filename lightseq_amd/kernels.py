@@ -143,6 +143,18 @@ def encself_attention(q, k, v, src_padding_mask, ctx, ctx_q, quant_scale, batch_
          current_stream())
 
 
+def encself_attention_i8qkv(qkv, qkv_bias, dequant_scale, src_padding_mask, ctx, ctx_q, quant_scale,
+                            batch_size, batch_seq_len, head_num, dim_per_head):
+    """Fused encoder attention fed by the int8 output of the QKV product [tokens, 3 * hidden]
+    and the fp16 bias [3 * hidden] (ker_arrange_encself_qkv_i8I applied while reading)."""
+    _dev(qkv, qkv_bias, src_padding_mask, ctx, ctx_q)
+    if qkv.dtype != torch.int8 or qkv_bias.dtype != torch.float16:
+        raise TypeError("encself_attention_i8qkv takes int8 codes and an fp16 bias")
+    call("lsh_encself_attention_i8qkv_f16", ptr(qkv), ptr(qkv_bias), dequant_scale,
+         ptr(src_padding_mask), ptr(ctx), ptr(ctx_q), quant_scale, batch_size, batch_seq_len,
+         head_num, dim_per_head, current_stream())
+
+
 def launch_enc_emb_i8I(token_emb, pos_emb, tokens, output, pad_mask, pad_id, batch_size, seq_len,
                        hidden_dim, lang_emb, lang_id, multilg_type, dequant_scale, scaled):
     _dev(token_emb, pos_emb, tokens, output, pad_mask)

@@ -43,6 +43,7 @@ _SIGNATURES = {
     "lsh_ker_arrange_atten_output_i8O": (True, "iispp" + "iiiifi"),
     "lsh_ker_correlation_softmax_encself": (True, "iiispp"),
     "lsh_encself_attention_f16": (False, "pppppp" + "fiiiis"),
+    "lsh_encself_attention_i8qkv_f16": (False, "ppfppp" + "fiiiis"),
     "lsh_launch_enc_emb_i8I": (True, "ppppp" + "iiiispp" + "ifi"),
     "lsh_launch_scaled_colsum": (True, "ppiifs"),
     "lsh_gemm_i8_i32o": (False, "pppiiis"),

@@ -266,6 +266,40 @@ def test_encself_attention_fused(oracle, rng, B, S, h, d):
         assert np.all(got[b][:, mask[b] == 1, :] == 0)
 
 
+@pytest.mark.parametrize("B,S,h,d", [(2, 128, 3, 64), (3, 50, 2, 64), (1, 200, 2, 64), (2, 64, 4, 32),
+                                     (1, 7, 1, 64), (2, 130, 2, 128)])
+def test_encself_attention_from_int8_qkv(oracle, rng, B, S, h, d):
+    """Attention fed by the int8 QKV product == ker_arrange_encself_qkv_i8I followed by the
+    fused attention on its fp16 q, k, v, bit for bit; and the oracle's sequence to the
+    usual bar."""
+    H = h * d
+    codes = rng.integers(-127, 128, size=(B * S, 3 * H), dtype=np.int8)
+    bias = _randT(rng, (3 * H,), np.float16, 0.3)
+    mask = _pad_mask(rng, B, S)
+    ds, qs = 1.4 / 127, 127 / 0.9
+    # two-kernel route
+    arr = torch.zeros((3, B, h, S, d), dtype=torch.float16, device=DEV)
+    _k().ker_arrange_encself_qkv_i8I_launcher(B * S, H, to_dev(codes), to_dev(bias), arr, B * S * H, S,
+                                              d, h, 1024, ds)
+    ctx0 = torch.zeros((B, h, S, d), dtype=torch.float16, device=DEV)
+    ctxq0 = torch.zeros((B * S, H), dtype=torch.int8, device=DEV)
+    _k().encself_attention(arr[0], arr[1], arr[2], to_dev(mask), ctx0, ctxq0, qs, B, S, h, d)
+    # one-kernel route
+    ctx1 = torch.full((B, h, S, d), 7.0, dtype=torch.float16, device=DEV)
+    ctxq1 = torch.full((B * S, H), 7, dtype=torch.int8, device=DEV)
+    _k().encself_attention_i8qkv(to_dev(codes), to_dev(bias), ds, to_dev(mask), ctx1, ctxq1, qs, B, S,
+                                 h, d)
+    np.testing.assert_array_equal(to_np(ctx1).view(np.uint16), to_np(ctx0).view(np.uint16))
+    np.testing.assert_array_equal(to_np(ctxq1), to_np(ctxq0))
+    # against the restatement of the reference's sequence
+    q, k, v = oracle.arrange_encself_qkv_i8I(codes, bias, B, S, h, ds)
+    probs = oracle.correlation_softmax_encself(oracle.attn_scores(q, k, np.sqrt(1.0 / d)), mask)
+    want_ctx = oracle.attn_context(probs, v)
+    np.testing.assert_allclose(to_np(ctx1).astype(np.float32), want_ctx.astype(np.float32), atol=3e-3,
+                               rtol=0)
+    assert_codes_close(to_np(ctxq1), oracle.arrange_atten_output_i8O(want_ctx, qs), max_frac=5e-3)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("scaled", [False, True])
 def test_enc_emb(oracle, rng, dtype, scaled):
