@@ -356,12 +356,13 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
           for (int i = 0; i < 16; ++i) bm = fmaxf(bm, sc[sb][i]);
         bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
         const float m_new = fmaxf(m, bm);
+        const float mref = m_new == kFloatInfNeg ? 0.f : m_new;
         float part = 0.f;
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            const float e = sc[sb][i] == kFloatInfNeg ? 0.f : __expf(sc[sb][i] - m_new);
+            const float e = __expf(sc[sb][i] - mref);
             part += e;
             if (nkb == 1) sc[sb][i] = e;  // single key block: the second pass reuses it
           }
@@ -375,9 +376,9 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         // by the sequence the compiler emits for a float division (refined reciprocal, two
         // residual corrections) with the reciprocal taken once per query and without the
         // range scaling, which only acts on quotients far below the smallest fp16 value.
-        const bool no_keys = !(sum > 0.f);
         float rs = __builtin_amdgcn_rcpf(sum);
-        rs = fmaf(fmaf(-sum, rs, 1.f), rs, rs);
+        rs = sum > 0.f ? fmaf(fmaf(-sum, rs, 1.f), rs, rs) : 0.f;  // no visible key: all zero
+        const float mref = m == kFloatInfNeg ? 0.f : m;
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb) {
 #pragma unroll
@@ -386,11 +387,14 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
               const float s = sc[sb][8 * t + j];
-              const float e = nkb == 1 ? s : (s == kFloatInfNeg ? 0.f : __expf(s - m));
+              const float e = nkb == 1 ? s : __expf(s - mref);
               float qt = e * rs;
               qt = fmaf(fmaf(-sum, qt, e), rs, qt);
               qt = fmaf(fmaf(-sum, qt, e), rs, qt);
-              pb[j] = (_Float16)(no_keys ? 0.f : qt);
+              // keep the float quotient a value of its own: folded into the last correction,
+              // the conversion to fp16 would round once instead of twice
+              asm volatile("" : "+v"(qt));
+              pb[j] = (_Float16)qt;
             }
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) {
