@@ -8,6 +8,8 @@
 // Replaces inference/model/quant_bert_encoder.cc.cu:321-347 (two cuBLAS strided
 // batched GEMMs + ker_correlation_softmax_encself + ker_arrange_atten_output_i8O)
 // and inference/kernels/transformerKernels.cc.cu:1119-1172.
+#include <type_traits>
+
 #include "ls_device.cuh"
 #include "ls_launch.h"
 
@@ -160,7 +162,9 @@ __device__ __forceinline__ void dequant16_bias(const uint4& w, const _Float16* _
 }
 
 template <int D, int MODE, int NW>
-__global__ void __launch_bounds__(64 * NW)
+// Two workgroups of four wavefronts share a compute unit for head sizes up to 64 (the
+// compiler is told to stay within that register budget); 128 needs the whole file.
+__global__ void __launch_bounds__(64 * NW, D <= 64 ? 2 : 1)
 encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
                     const __half* __restrict__ v, const int* __restrict__ pad_mask,
                     __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale, int S,
@@ -358,14 +362,20 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         const float m_new = fmaxf(m, bm);
         const float mref = m_new == kFloatInfNeg ? 0.f : m_new;
         float part = 0.f;
+        if (nkb == 1) {  // single key block: the second pass reuses the exponentials
 #pragma unroll
-        for (int sb = 0; sb < 4; ++sb)
+          for (int sb = 0; sb < 4; ++sb)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const float e = __expf(sc[sb][i] - mref);
-            part += e;
-            if (nkb == 1) sc[sb][i] = e;  // single key block: the second pass reuses it
-          }
+            for (int i = 0; i < 16; ++i) {
+              sc[sb][i] = __expf(sc[sb][i] - mref);
+              part += sc[sb][i];
+            }
+        } else {
+#pragma unroll
+          for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) part += __expf(sc[sb][i] - mref);
+        }
         part += __shfl_xor(part, 32, 64);
         sum = sum * __expf(m - m_new) + part;
         m = m_new;
@@ -379,6 +389,10 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         float rs = __builtin_amdgcn_rcpf(sum);
         rs = sum > 0.f ? fmaf(fmaf(-sum, rs, 1.f), rs, rs) : 0.f;  // no visible key: all zero
         const float mref = m == kFloatInfNeg ? 0.f : m;
+        // one instance per case, chosen by a uniform branch, so that neither evaluates the
+        // other's exponentials
+        auto pv_pass = [&](auto reuse_tag) {
+        constexpr bool REUSE = decltype(reuse_tag)::value;
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb) {
 #pragma unroll
@@ -387,7 +401,7 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
               const float s = sc[sb][8 * t + j];
-              const float e = nkb == 1 ? s : __expf(s - mref);
+              const float e = REUSE ? s : __expf(s - mref);
               float qt = e * rs;
               qt = fmaf(fmaf(-sum, qt, e), rs, qt);
               qt = fmaf(fmaf(-sum, qt, e), rs, qt);
@@ -406,6 +420,11 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
             }
           }
         }
+        };
+        if (nkb == 1)
+          pv_pass(std::true_type{});
+        else
+          pv_pass(std::false_type{});
       }
     }
   }
