@@ -221,25 +221,44 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
   const int8_t* vb = v_cache + bh * (long)max_step * D;
   const uint4 qv = *reinterpret_cast<const uint4*>(q + bh * D + c * 16);
 
+  // The cache is read in rounds of UN independent 16-byte loads per lane (UN * 4 * KPW
+  // steps per round), all issued before the first is used: a step costs one memory round
+  // trip per round instead of one per KPW * 4 cached steps.
+  constexpr int UN = 8;
+  const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
   // scores -> scaled logits in LDS
   float mx = kFloatInfNeg;
-  for (int j0 = wid * KPW; j0 < step_num; j0 += 4 * KPW) {
-    const int j = j0 + grp;
-    int sc = 0;
-    if (j < step_num) {
-      const uint4 kv = *reinterpret_cast<const uint4*>(kb + (long)j * D + c * 16);
-      sc = __builtin_amdgcn_sdot4((int)qv.x, (int)kv.x, sc, false);
-      sc = __builtin_amdgcn_sdot4((int)qv.y, (int)kv.y, sc, false);
-      sc = __builtin_amdgcn_sdot4((int)qv.z, (int)kv.z, sc, false);
-      sc = __builtin_amdgcn_sdot4((int)qv.w, (int)kv.w, sc, false);
+  for (int base = wid * KPW; base < step_num; base += UN * 4 * KPW) {
+    uint4 kv[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int j = base + u * 4 * KPW + grp;
+      kv[u] = j < step_num ? *reinterpret_cast<const uint4*>(kb + (long)j * D + c * 16) : zero4;
     }
 #pragma unroll
-    for (int m = 1; m < CH; m <<= 1) sc += __shfl_xor(sc, m, 64);
-    if (j < step_num) {
-      const float val = (float)sc * dq * dq * attn_scale;
-      if (c == 0) probs[j] = val;
-      mx = fmaxf(mx, val);
+    for (int u = 0; u < UN; ++u) {
+      const int j = base + u * 4 * KPW + grp;
+      int sc = 0;
+      sc = __builtin_amdgcn_sdot4((int)qv.x, (int)kv[u].x, sc, false);
+      sc = __builtin_amdgcn_sdot4((int)qv.y, (int)kv[u].y, sc, false);
+      sc = __builtin_amdgcn_sdot4((int)qv.z, (int)kv[u].z, sc, false);
+      sc = __builtin_amdgcn_sdot4((int)qv.w, (int)kv[u].w, sc, false);
+#pragma unroll
+      for (int m = 1; m < CH; m <<= 1) sc += __shfl_xor(sc, m, 64);
+      if (j < step_num) {
+        const float val = (float)sc * dq * dq * attn_scale;
+        if (c == 0) probs[j] = val;
+        mx = fmaxf(mx, val);
+      }
     }
+  }
+  // the first round of value loads travels while the softmax is computed
+  uint4 vv0[UN];
+#pragma unroll
+  for (int u = 0; u < UN; ++u) {
+    const int j = wid * KPW + u * 4 * KPW + grp;
+    vv0[u] = j < step_num ? *reinterpret_cast<const uint4*>(vb + (long)j * D + c * 16) : zero4;
   }
   mx = block_max(mx, red);
   float sum = 0.f;
@@ -256,14 +275,25 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
   float acc[16];
 #pragma unroll
   for (int k = 0; k < 16; ++k) acc[k] = 0.f;
-  for (int j0 = wid * KPW; j0 < step_num; j0 += 4 * KPW) {
-    const int j = j0 + grp;
-    if (j < step_num) {
-      const uint4 vv = *reinterpret_cast<const uint4*>(vb + (long)j * D + c * 16);
-      const float p = probs[j];
-      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+  for (int base = wid * KPW; base < step_num; base += UN * 4 * KPW) {
+    uint4 vv[UN];
 #pragma unroll
-      for (int k = 0; k < 16; ++k) acc[k] += (float)unpack_i8(w[k >> 2], k & 3) * p * dq;
+    for (int u = 0; u < UN; ++u) {
+      const int j = base + u * 4 * KPW + grp;
+      if (base == wid * KPW)
+        vv[u] = vv0[u];
+      else
+        vv[u] = j < step_num ? *reinterpret_cast<const uint4*>(vb + (long)j * D + c * 16) : zero4;
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int j = base + u * 4 * KPW + grp;
+      if (j < step_num) {  // same ascending order of steps per lane as a plain loop
+        const float p = probs[j];
+        const uint32_t w[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
+#pragma unroll
+        for (int k = 0; k < 16; ++k) acc[k] += (float)unpack_i8(w[k >> 2], k & 3) * p * dq;
+      }
     }
   }
 #pragma unroll
