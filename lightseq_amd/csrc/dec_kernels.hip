@@ -200,8 +200,8 @@ decself_attn_kernel(int32_t* __restrict__ scores, const int8_t* __restrict__ q,
 // across lanes (shuffles) and wavefronts (LDS): a tree instead of the ascending-step order
 // of the kernel above, so a context code can differ by one from it where the float sum
 // lands next to a rounding boundary.  Requires d in {32, 64, 128} and 16-byte aligned rows.
-template <int D>
-__global__ void __launch_bounds__(256)
+template <int D, int NWV>
+__global__ void __launch_bounds__(64 * NWV)
 decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k_cache,
                        const int8_t* __restrict__ v_cache, int8_t* __restrict__ new_v,
                        int step_num, int max_step, int head_num, float attn_scale, float dq,
@@ -213,7 +213,7 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
   const int padded = (step_num + 63) & ~63;
   float* probs = lds_f;                 // [padded]
   float* red = lds_f + padded;          // [16] block reductions
-  float* part = red + 16;               // [4][D] per-wavefront value sums
+  float* part = red + 16;               // [NWV][D] per-wavefront value sums
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const long bh = blockIdx.x;
   const int c = lane % CH, grp = lane / CH;
@@ -221,24 +221,24 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
   const int8_t* vb = v_cache + bh * (long)max_step * D;
   const uint4 qv = *reinterpret_cast<const uint4*>(q + bh * D + c * 16);
 
-  // The cache is read in rounds of UN independent 16-byte loads per lane (UN * 4 * KPW
+  // The cache is read in rounds of UN independent 16-byte loads per lane (UN * NWV * KPW
   // steps per round), all issued before the first is used: a step costs one memory round
   // trip per round instead of one per KPW * 4 cached steps.
   constexpr int UN = 8;
-  const uint4 zero4 = make_uint4(0, 0, 0, 0);
 
   // scores -> scaled logits in LDS
   float mx = kFloatInfNeg;
-  for (int base = wid * KPW; base < step_num; base += UN * 4 * KPW) {
+  for (int base = wid * KPW; base < step_num; base += UN * NWV * KPW) {
     uint4 kv[UN];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int j = base + u * 4 * KPW + grp;
-      kv[u] = j < step_num ? *reinterpret_cast<const uint4*>(kb + (long)j * D + c * 16) : zero4;
+      const int j = base + u * NWV * KPW + grp;
+      // clamped instead of predicated: unconditional loads stay back to back
+      kv[u] = *reinterpret_cast<const uint4*>(kb + (long)min(j, step_num - 1) * D + c * 16);
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int j = base + u * 4 * KPW + grp;
+      const int j = base + u * NWV * KPW + grp;
       int sc = 0;
       sc = __builtin_amdgcn_sdot4((int)qv.x, (int)kv[u].x, sc, false);
       sc = __builtin_amdgcn_sdot4((int)qv.y, (int)kv[u].y, sc, false);
@@ -257,37 +257,37 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
   uint4 vv0[UN];
 #pragma unroll
   for (int u = 0; u < UN; ++u) {
-    const int j = wid * KPW + u * 4 * KPW + grp;
-    vv0[u] = j < step_num ? *reinterpret_cast<const uint4*>(vb + (long)j * D + c * 16) : zero4;
+    const int j = wid * KPW + u * NWV * KPW + grp;
+    vv0[u] = *reinterpret_cast<const uint4*>(vb + (long)min(j, step_num - 1) * D + c * 16);
   }
   mx = block_max(mx, red);
   float sum = 0.f;
-  for (int j = tid; j < step_num; j += 256) {
+  for (int j = tid; j < step_num; j += 64 * NWV) {
     const float e = __expf(probs[j] - mx);
     probs[j] = e;
     sum += e;
   }
   sum = block_sum(sum, red);
-  for (int j = tid; j < step_num; j += 256) probs[j] = probs[j] / sum;
+  for (int j = tid; j < step_num; j += 64 * NWV) probs[j] = probs[j] / sum;
   __syncthreads();
 
-  // value sum: lane (grp, c) accumulates dims [16c, 16c+16) over steps grp, grp + KPW*4, ...
+  // value sum: lane (grp, c) accumulates dims [16c, 16c+16) over steps grp, grp + KPW * NWV, ...
   float acc[16];
 #pragma unroll
   for (int k = 0; k < 16; ++k) acc[k] = 0.f;
-  for (int base = wid * KPW; base < step_num; base += UN * 4 * KPW) {
+  for (int base = wid * KPW; base < step_num; base += UN * NWV * KPW) {
     uint4 vv[UN];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int j = base + u * 4 * KPW + grp;
+      const int j = base + u * NWV * KPW + grp;
       if (base == wid * KPW)
         vv[u] = vv0[u];
       else
-        vv[u] = j < step_num ? *reinterpret_cast<const uint4*>(vb + (long)j * D + c * 16) : zero4;
+        vv[u] = *reinterpret_cast<const uint4*>(vb + (long)min(j, step_num - 1) * D + c * 16);
     }
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int j = base + u * 4 * KPW + grp;
+      const int j = base + u * NWV * KPW + grp;
       if (j < step_num) {  // same ascending order of steps per lane as a plain loop
         const float p = probs[j];
         const uint32_t w[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
@@ -306,7 +306,14 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
   }
   __syncthreads();
   if (tid < D) {
-    const float v = (part[tid] + part[D + tid]) + (part[2 * D + tid] + part[3 * D + tid]);
+    float t[NWV];  // pairwise tree over the wavefronts' partial sums
+#pragma unroll
+    for (int i = 0; i < NWV; ++i) t[i] = part[i * D + tid];
+#pragma unroll
+    for (int st = 1; st < NWV; st *= 2)
+#pragma unroll
+      for (int i = 0; i < NWV; i += 2 * st) t[i] += t[i + st];
+    const float v = t[0];
     const long row = bh / head_num;
     const int head = (int)(bh % head_num);
     new_v[row * ((long)head_num * D) + (long)head * D + tid] = (int8_t)float2int8(v, quant_scale);
@@ -358,12 +365,13 @@ int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v
   const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
                          reinterpret_cast<uintptr_t>(v_cache)) & 15u) == 0;
   if (aligned && (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128)) {
-    const size_t lds = ((size_t)((step_num + 63) & ~63) + 16 + 4 * dim_per_head) * sizeof(float);
+    constexpr int kWaves = 8;  // one workgroup per compute unit: width buys loads in flight
+    const size_t lds =
+        ((size_t)((step_num + 63) & ~63) + 16 + kWaves * dim_per_head) * sizeof(float);
 #define LSH_DECSELF(D)                                                                          \
-  decself_attn_wg_kernel<D><<<batch_head_num, 256, lds, s>>>(q, k_cache, v_cache, new_v,         \
-                                                             step_num, max_step, head_num,      \
-                                                             attn_scale, dequant_scale,         \
-                                                             quant_scale)
+  decself_attn_wg_kernel<D, kWaves><<<batch_head_num, 64 * kWaves, lds, s>>>(                   \
+      q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,      \
+      quant_scale)
     if (dim_per_head == 32) LSH_DECSELF(32);
     else if (dim_per_head == 64) LSH_DECSELF(64);
     else LSH_DECSELF(128);
