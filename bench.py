@@ -11,10 +11,11 @@ HBM.  ``value`` = batch * seq_len * steps / wall time of the timed steps (padded
 tokens counted, as the reference's b32 x s128 figures do).
 
 The JSON line also carries
-  roofline       the dominant kernel (by total time) among the int8 GEMM
-                 instantiations, timed with HIP events on the model's stream during a
-                 second, instrumented pass over the same steps: achieved = 2*M*N*K per
-                 launch / mean launch time, against the 5.0 POP/s dense int8 MFMA peak;
+  roofline       the dominant kernel launch (by total time) among the int8 GEMM sites
+                 of a layer (one kernel instantiation at one shape), timed with HIP events
+                 on the model's stream during a second, instrumented pass over the same
+                 steps: achieved = 2*M*N*K per launch / mean launch time, against the
+                 5.0 POP/s dense int8 MFMA peak;
   fused_kernels  the memory-bound fused kernels of one encoder layer at this workload's
                  shapes, each timed alone over back-to-back launches queued behind a long
                  kernel (so the host's launch cost is not what is measured): achieved
@@ -194,18 +195,18 @@ def gemm_microbench(reps=40):
 TRAFFIC_SUMMARY = "bert_base_b32_s128_pmc_hbm_traffic.txt"
 
 
-def _profiled_traffic(kernel):
-    """HBM bytes per launch of ``kernel`` from the committed rocprofv3 --pmc summary
-    (FETCH_SIZE and WRITE_SIZE runs of this same command, scaled by a plain copy kernel);
-    None when the summary holds no line for that kernel."""
+def _profiled_traffic(kernel, site):
+    """HBM bytes per launch of ``kernel`` at GEMM site ``site`` from the committed
+    rocprofv3 --pmc summary (FETCH_SIZE and WRITE_SIZE runs of this same command, scaled by
+    a plain copy kernel); None when the summary holds no line for that kernel and site."""
     import re
     path = os.path.join(ROOT, "profiles", TRAFFIC_SUMMARY)
     if not os.path.exists(path):
         return None
-    short = kernel.replace("EpiGeluI8", "EpiActI8<0>")
+    want = kernel.replace("EpiGeluI8", "EpiActI8<0>") + " @ " + site
     for line in open(path):
         m = re.match(r"traffic_bytes_per_launch\[(.+?)\] = (\d+)", line)
-        if m and m.group(1).replace("lsh::", "") == short:
+        if m and m.group(1).replace("lsh::", "") == want:
             return int(m.group(2))
     return None
 
@@ -240,17 +241,18 @@ def bench_bert(args):
     prof = model.get_profile()
     model.set_profiling(False)
     by_kernel = {}
-    for site in prof:
-        k = by_kernel.setdefault(site["kernel"], {"ms": 0.0, "launches": 0, "ops": 0.0, "sites": []})
+    for site in prof:  # one entry per (instantiation, shape): a site has one shape
+        k = by_kernel.setdefault((site["kernel"], site["site"]),
+                                 {"ms": 0.0, "launches": 0, "ops": 0.0, "sites": []})
         k["ms"] += site["total_ms"]
         k["launches"] += site["launches"]
         k["ops"] += 2.0 * site["m"] * site["n"] * site["k"] * site["launches"]
         k["sites"].append(site["site"])
-    name, dom = max(by_kernel.items(), key=lambda kv: kv[1]["ms"])
+    (name, dom_site), dom = max(by_kernel.items(), key=lambda kv: kv[1]["ms"])
     avg_ms = dom["ms"] / dom["launches"]
     achieved = dom["ops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                "frac": achieved / INT8_MFMA_PEAK_TOPS, "traffic": _profiled_traffic(name),
+                "frac": achieved / INT8_MFMA_PEAK_TOPS, "traffic": _profiled_traffic(name, dom_site),
                 "traffic_source": "profiles/" + TRAFFIC_SUMMARY, "kernel": name,
                 "sites": dom["sites"], "avg_launch_us": avg_ms * 1e3,
                 "gemm_sites": {s["site"]: {"kernel": s["kernel"], "mnk": [s["m"], s["n"], s["k"]],
