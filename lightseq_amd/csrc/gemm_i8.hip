@@ -6,8 +6,14 @@
 // Replaces the cuBLASLt int8 GEMMs and their tuned-algorithm table
 // (inference/model/cublas_helper.cc:31-225,361-489, cublas_algo_map.cc).
 //
-// Two kernels share the tile geometry and the epilogues:
+// Three kernels share the epilogues (the first two also the tile geometry):
 //
+//  * gemm_i8_skinny_kernel -- M <= 64 (decode steps), K % 128 == 0.  A workgroup owns 32
+//    output columns for all rows; its 4 wavefronts split the 128-byte K chunks of the
+//    workgroup's K range, load operands from global memory straight into MFMA registers
+//    (no LDS staging, no barrier in the loop) and sum their partial tiles through LDS.
+//    The weight matrix is read once, by ceil(N/32) * ksplit workgroups; with ksplit > 1
+//    range p stores its int32 partial sums to plane p of the output ([ksplit][M][N]).
 //  * gemm_i8_stream_kernel -- the fast path (K % 128 == 0).  Persistent: 2 workgroups
 //    per compute unit walk a list of 128x128 tiles; operand stages (128 rows x 128 B
 //    each for A and W) are brought from L2 straight into LDS with

@@ -1,10 +1,14 @@
 // LayerNorm family of the int8 layer path: dequant + residual (+colsum) +
 // LayerNorm + quant, one HBM pass.
 //
-// Layout: one 64-lane wavefront owns one token row and keeps it in registers
-// (4 consecutive elements per lane per step, so a row of `hidden` elements takes
-// ceil(hidden/256) steps); mean and variance are the reference's two-pass form,
-// reduced with cross-lane shuffles.  Four rows per 256-thread workgroup.
+// Two layouts, both keeping a token row in registers with the reference's two-pass mean
+// and variance reduced by cross-lane shuffles:
+//  * ln_rows8_kernel (hidden % 8 == 0): a row belongs to LPR lanes (32: two rows per
+//    wavefront), 8 consecutive elements per lane per step (16-byte fp16, 32-byte int32
+//    accesses); scale, bias and residual bias are fetched with the first round of loads;
+//    with nparts > 1 the int32 input is the exact integer sum of nparts split-K
+//    accumulator planes, loaded independently.
+//  * ln_rows_kernel (any hidden): one wavefront per row, 4 elements per lane per step.
 //
 // Replaces inference/kernels/transformerKernels_int8.cc.cu:149-863.
 #include "ls_device.cuh"
