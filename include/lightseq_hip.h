@@ -221,6 +221,18 @@ int lsh_launch_scaled_colsum_f32(const void* inp, void* out, int rows, int cols,
  * model/cublas_helper.h:50-58 cublaslt_gemm<int32_t,int32_t>. */
 int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n, int k,
                      lsh_stream_t stream);
+/* Decode-step QKV product with ker_arrange_decself_qkv_i8I_i8O
+ * (kernels/transformerKernels_int8.cc.cu:1432-1513; call sites model/quant_decoder.cc.cu:660-674,
+ * model/quant_gpt_encoder.cc.cu:640-653) as its epilogue: A [step_token_num, k] x W [3*hidden, k]
+ * -> int8 code (alpha) -> code * dequant_scale + bias -> int8 (quant_scale); q codes to new_q
+ * [step_token_num, hidden], k and v codes to slot step_id of the caches [step_token_num,
+ * head_num, max_step, hidden/head_num].  Same bits as lsh_gemm_i8_i8o followed by
+ * lsh_ker_arrange_decself_qkv_i8I_i8O_f16.  No counterpart in the reference. */
+int lsh_gemm_i8_decself_qkv_i8o_f16(const int8_t* A, const int8_t* W, const void* qkv_bias,
+                                    int8_t* new_q, int8_t* new_k, int8_t* new_v,
+                                    int step_token_num, int hidden, int k, int head_num,
+                                    int max_step, int step_id, float alpha, float dequant_scale,
+                                    float quant_scale, lsh_stream_t stream);
 /* The bias + activation + requantisation epilogue as a table: after the requantisation an
  * element is one of 255 codes, so what follows depends only on (column, code).
  * lsh_build_act_lut fills lut [n, 256] (entry [col][code + 128]) with what

@@ -334,6 +334,15 @@ int lsh_build_act_lut(int8_t* lut, const void* bias_f16, int n, float dequant_sc
                       float quant_scale, float clip_max, int act, lsh_stream_t stream) {
   return build_act_lut(lut, H(bias_f16), n, dequant_scale, quant_scale, clip_max, act, HS(stream));
 }
+int lsh_gemm_i8_decself_qkv_i8o_f16(const int8_t* A, const int8_t* W, const void* qkv_bias,
+                                    int8_t* new_q, int8_t* new_k, int8_t* new_v,
+                                    int step_token_num, int hidden, int k, int head_num,
+                                    int max_step, int step_id, float alpha, float dequant_scale,
+                                    float quant_scale, lsh_stream_t stream) {
+  return gemm_i8_decself_qkv_i8o(A, W, H(qkv_bias), new_q, new_k, new_v, step_token_num, hidden, k,
+                                 head_num, max_step, step_id, alpha, dequant_scale, quant_scale,
+                                 HS(stream));
+}
 int lsh_gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int m,
                         int n, int k, float alpha, lsh_stream_t stream) {
   return gemm_i8_lut_i8o(A, W, C, lut, m, n, k, alpha, HS(stream));

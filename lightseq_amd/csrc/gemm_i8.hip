@@ -104,6 +104,50 @@ struct EpiI8 {
   static const char* name() { return "EpiI8"; }
 };
 
+// Decode-step QKV product followed by ker_arrange_decself_qkv_i8I_i8O
+// (inference/kernels/transformerKernels_int8.cc.cu:1432-1513; call sites
+// model/quant_decoder.cc.cu:660-674, model/quant_gpt_encoder.cc.cu:640-653): the int8 code
+// of the product is dequantised, biased and requantised with the cache scale; columns
+// [0, H) go to new_q [M, H], [H, 2H) and [2H, 3H) to slot step_id of the K and V caches
+// [M, heads, max_step, d].  Same float arithmetic as the stand-alone kernel (no fused
+// multiply-add).
+struct EpiDecQkvI8 {
+  int8_t *new_q, *new_k, *new_v;
+  const __half* bias;
+  float alpha, dequant_scale, quant_scale;
+  int hidden, head_num, dim_per_head, max_step, step_id;
+  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool) const {
+#pragma clang fp contract(off)
+    const int part = n / hidden, i = n - part * hidden;
+    const half8_t b0 = *reinterpret_cast<const half8_t*>(bias + n);
+    const half8_t b1 = *reinterpret_cast<const half8_t*>(bias + n + 8);
+    int q[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const float b = __half2float(k < 8 ? b0.v[k] : b1.v[k - 8]);
+      const float val = (float)requant_acc(c[k], alpha) * dequant_scale + b;
+      q[k] = float2int8(val, quant_scale);
+    }
+    int8_t* dst;
+    if (part == 0) {
+      dst = new_q + m * hidden + i;
+    } else {
+      const int head = i / dim_per_head, dim = i - head * dim_per_head;
+      dst = (part == 1 ? new_k : new_v) +
+            ((m * head_num + head) * max_step + step_id) * dim_per_head + dim;
+    }
+    uint4 o;
+    o.x = pack4_i8(q[0], q[1], q[2], q[3]);
+    o.y = pack4_i8(q[4], q[5], q[6], q[7]);
+    o.z = pack4_i8(q[8], q[9], q[10], q[11]);
+    o.w = pack4_i8(q[12], q[13], q[14], q[15]);
+    *reinterpret_cast<uint4*>(dst) = o;
+    (void)N;
+  }
+  bool vec_ok(int) const { return true; }
+  static const char* name() { return "EpiDecQkvI8"; }
+};
+
 // The same with the scale read from device memory (the csrc layers keep their clip values
 // and the alpha derived from them on the device: csrc/kernels/cuda/cublas_wrappers.cpp:134
 // CUBLASLT_POINTER_MODE_DEVICE).
@@ -746,6 +790,27 @@ int gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* l
                     int K, float alpha, hipStream_t s) {
   if (!C || !lut) return lsh_fail(LSH_ERR_INVALID, "int8 gemm (table epilogue): null pointer");
   return dispatch(A, W, EpiLutI8{C, lut, alpha}, M, N, K, s);
+}
+
+int gemm_i8_decself_qkv_i8o(const int8_t* A, const int8_t* W, const __half* qkv_bias, int8_t* new_q,
+                            int8_t* new_k, int8_t* new_v, int step_token_num, int hidden, int K,
+                            int head_num, int max_step, int step_id, float alpha,
+                            float dequant_scale, float quant_scale, hipStream_t s) {
+  if (!qkv_bias || !new_q || !new_k || !new_v || head_num <= 0 || hidden <= 0 ||
+      hidden % head_num != 0 || max_step <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "int8 gemm (decoder qkv): bad arguments");
+  if (step_id < 0 || step_id >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "int8 gemm (decoder qkv): step_id outside the cache");
+  const int d = hidden / head_num;
+  if (d % 16 != 0 ||
+      ((reinterpret_cast<uintptr_t>(qkv_bias) | reinterpret_cast<uintptr_t>(new_q) |
+        reinterpret_cast<uintptr_t>(new_k) | reinterpret_cast<uintptr_t>(new_v)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "int8 gemm (decoder qkv): needs dim_per_head % 16 == 0 and aligned outputs");
+  return dispatch(A, W,
+                  EpiDecQkvI8{new_q, new_k, new_v, qkv_bias, alpha, dequant_scale, quant_scale,
+                              hidden, head_num, d, max_step, step_id},
+                  step_token_num, 3 * hidden, K, s);
 }
 
 int gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, __half* new_qkv, const __half* qkv_bias,

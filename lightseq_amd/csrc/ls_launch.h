@@ -126,6 +126,12 @@ int gemm_i8_bias_act_i8o(const int8_t* A, const int8_t* W, int8_t* C, const __ha
 // weight matrix by build_act_lut.  Bit-identical to gemm_i8_bias_act_i8o.
 int build_act_lut(int8_t* lut, const __half* bias, int N, float dequant_scale, float quant_scale,
                   float clip_max, int act, hipStream_t s);
+// Decode-step QKV product with ker_arrange_decself_qkv_i8I_i8O as its epilogue: q codes to
+// new_q [M, hidden], k and v codes to slot step_id of the caches [M, heads, max_step, d].
+int gemm_i8_decself_qkv_i8o(const int8_t* A, const int8_t* W, const __half* qkv_bias, int8_t* new_q,
+                            int8_t* new_k, int8_t* new_v, int step_token_num, int hidden, int K,
+                            int head_num, int max_step, int step_id, float alpha,
+                            float dequant_scale, float quant_scale, hipStream_t s);
 int gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int M, int N,
                     int K, float alpha, hipStream_t s);
 //   writes q, k, v as fp16 [B, h, S, d] at new_qkv + {0, 1, 2} * max_batch_dim

@@ -82,6 +82,7 @@ void QuantDecoder::init_buffer() {
   const size_t wide = rows * (size_t)std::max(I, 3 * H);
   _buf_a.alloc(wide);
   _buf_b.alloc(wide);
+  _buf_q.alloc(wide);
   _logits.alloc(rows * (size_t)V);
   // up to 8 accumulator planes of the split-K second FFN product
   _int32_ffn_out_buf.alloc(rows * H * 8);
@@ -284,17 +285,25 @@ void QuantDecoder::self_attention() {
                                            w.self_ln_scale.get(), w.self_ln_bias.get(),
                                            w.b_self_out.get(), Q / c[6], _tw._is_post_ln));
   }
-  LSH_CALL(gemm_i8_i8o(_buf_a.get(), w.w_self_qkv.get(), _buf_b.get(), M, 3 * H, H,
-                       c[0] * c[6] / (c[12] * Q), _stream));
-  // q -> _buf_a, k / v -> slot _cur_step of the caches (all three with the cache clip)
-  LSH_CALL(arrange_decself_qkv_i8I_i8O<__half>(M, H, _stream, _buf_b.get(), w.b_self_qkv.get(),
-                                               _buf_a.get(), k_cache, v_cache, _tw._head_num,
-                                               _tw._dim_per_head, _tw._max_step, _cur_step,
-                                               c[12] / Q, Q / c[18]));
+  // QKV product; its epilogue is ker_arrange_decself_qkv_i8I_i8O: q -> _buf_q, k / v -> slot
+  // _cur_step of the caches (all three with the cache clip)
+  if (_tw._dim_per_head % 16 == 0) {
+    LSH_CALL(gemm_i8_decself_qkv_i8o(_buf_a.get(), w.w_self_qkv.get(), w.b_self_qkv.get(),
+                                     _buf_q.get(), k_cache, v_cache, M, H, H, _tw._head_num,
+                                     _tw._max_step, _cur_step, c[0] * c[6] / (c[12] * Q),
+                                     c[12] / Q, Q / c[18], _stream));
+  } else {
+    LSH_CALL(gemm_i8_i8o(_buf_a.get(), w.w_self_qkv.get(), _buf_b.get(), M, 3 * H, H,
+                         c[0] * c[6] / (c[12] * Q), _stream));
+    LSH_CALL(arrange_decself_qkv_i8I_i8O<__half>(M, H, _stream, _buf_b.get(), w.b_self_qkv.get(),
+                                                 _buf_q.get(), k_cache, v_cache, _tw._head_num,
+                                                 _tw._dim_per_head, _tw._max_step, _cur_step,
+                                                 c[12] / Q, Q / c[18]));
+  }
   // int8 q.K -> softmax -> new value, one kernel
   const float attn_scale =
       __half2float(__float2half_rn(sqrtf(1.f / (float)_tw._dim_per_head)));
-  LSH_CALL(decself_attention_i8(_buf_a.get(), k_cache, v_cache, _buf_b.get(), M * _tw._head_num,
+  LSH_CALL(decself_attention_i8(_buf_q.get(), k_cache, v_cache, _buf_b.get(), M * _tw._head_num,
                                 _cur_step + 1, _tw._max_step, _tw._head_num, _tw._dim_per_head,
                                 attn_scale, c[18] / Q, Q / c[7], _stream));
   LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_self_out.get(), _buf_a.get(), M, H, H,

@@ -80,7 +80,7 @@ class QuantDecoder {
   DeviceBuffer<__half> _encdec_k, _encdec_v;      // [n_layer][max_batch*max_step*H]
   DeviceBuffer<__half> _encoder_out_buf;          // [tokens, n_layer*2*H]
   DeviceBuffer<__half> _cur_step_query, _query_buf1;
-  DeviceBuffer<int8_t> _buf_a, _buf_b, _logits;
+  DeviceBuffer<int8_t> _buf_a, _buf_b, _buf_q, _logits;
   DeviceBuffer<int32_t> _int32_ffn_out_buf;
   DeviceBuffer<int8_t> _self_k_cache[2], _self_v_cache[2];  // [n_layer][rows*max_step*H]
   int _cache_cur = 0;

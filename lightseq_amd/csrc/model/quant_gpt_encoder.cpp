@@ -65,6 +65,7 @@ void QuantGptEncoder::init_buffer() {
   const size_t wide = tokens * (size_t)std::max(I, 3 * H);
   _buf_a.alloc(wide);
   _buf_b.alloc(wide);
+  _buf_q.alloc(wide);
   _hid_last.alloc((size_t)_max_batch_size * H);
   // perplexity needs the logits of every position, sampling only of the last one
   _logits.alloc((_tw._sampling_method == "ppl" ? tokens : (size_t)_max_batch_size) * V);
@@ -195,13 +196,22 @@ void QuantGptEncoder::step_pass() {
     if (_layer_id == 0)
       LSH_CALL(norm_layer_resual_i8O<__half>(B, H, _stream, _query.get(), a, w.ln1_scale.get(),
                                              w.ln1_bias.get(), w.b_out.get(), Q / c[4], false));
-    LSH_CALL(gemm_i8_i8o(a, w.w_qkv.get(), b, B, 3 * H, H, c[0] * c[4] / (c[8] * Q), _stream));
-    // q -> a, k / v appended to the caches at the token's position
-    LSH_CALL(arrange_decself_qkv_i8I_i8O<__half>(B, H, _stream, b, w.b_qkv.get(), a, k_cache,
-                                                 v_cache, _tw._head_num, _tw._dim_per_head,
-                                                 _tw._max_step, _batch_seq_len - 1, c[8] / Q,
-                                                 Q / c[11]));
-    LSH_CALL(decself_attention_i8(a, k_cache, v_cache, b, B * _tw._head_num, _batch_seq_len,
+    // QKV product; its epilogue is ker_arrange_decself_qkv_i8I_i8O: q -> _buf_q, k / v appended
+    // to the caches at the token's position
+    if (_tw._dim_per_head % 16 == 0) {
+      LSH_CALL(gemm_i8_decself_qkv_i8o(a, w.w_qkv.get(), w.b_qkv.get(), _buf_q.get(), k_cache,
+                                       v_cache, B, H, H, _tw._head_num, _tw._max_step,
+                                       _batch_seq_len - 1, c[0] * c[4] / (c[8] * Q), c[8] / Q,
+                                       Q / c[11], _stream));
+    } else {
+      LSH_CALL(gemm_i8_i8o(a, w.w_qkv.get(), b, B, 3 * H, H, c[0] * c[4] / (c[8] * Q), _stream));
+      LSH_CALL(arrange_decself_qkv_i8I_i8O<__half>(B, H, _stream, b, w.b_qkv.get(), _buf_q.get(),
+                                                   k_cache, v_cache, _tw._head_num,
+                                                   _tw._dim_per_head, _tw._max_step,
+                                                   _batch_seq_len - 1, c[8] / Q, Q / c[11]));
+    }
+    LSH_CALL(decself_attention_i8(_buf_q.get(), k_cache, v_cache, b, B * _tw._head_num,
+                                  _batch_seq_len,
                                   _tw._max_step, _tw._head_num, _tw._dim_per_head, _atten_scaler,
                                   c[11] / Q, Q / c[5], _stream));
     LSH_CALL(gemm_i8_i8o(b, w.w_out.get(), a, B, H, H, c[1] * c[5] / (c[9] * Q), _stream));

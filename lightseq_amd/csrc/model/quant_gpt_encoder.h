@@ -70,7 +70,7 @@ class QuantGptEncoder {
 
   DeviceBuffer<int> _real_seq_len, _ids, _last_ids, _unfinished;
   DeviceBuffer<__half> _query, _qkv_buf;  // q codes | k codes | v, each max_batch_dim
-  DeviceBuffer<int8_t> _buf_a, _buf_b, _hid_last, _logits;
+  DeviceBuffer<int8_t> _buf_a, _buf_b, _buf_q, _hid_last, _logits;
   DeviceBuffer<int32_t> _int32_ffn_out_buf;
   DeviceBuffer<int8_t> _self_k_cache, _self_v_cache;  // [n_layer][max_batch_dim]
   DeviceBuffer<int8_t> _int8_emb;                     // [vocab, H]

@@ -509,6 +509,15 @@ def build_act_lut(lut, bias, n, dequant_scale, quant_scale, clip_max, act):
          current_stream())
 
 
+def gemm_i8_decself_qkv_i8o(a, w, qkv_bias, new_q, new_k, new_v, step_token_num, hidden, k, head_num,
+                            max_step, step_id, alpha, dequant_scale, quant_scale):
+    """Decode-step QKV product with ker_arrange_decself_qkv_i8I_i8O as its epilogue."""
+    _dev(a, w, qkv_bias, new_q, new_k, new_v)
+    call("lsh_gemm_i8_decself_qkv_i8o_f16", ptr(a), ptr(w), ptr(qkv_bias), ptr(new_q), ptr(new_k),
+         ptr(new_v), step_token_num, hidden, k, head_num, max_step, step_id, alpha, dequant_scale,
+         quant_scale, current_stream())
+
+
 def gemm_i8_lut_i8o(a, w, c, lut, m, n, k, alpha):
     """int8-output GEMM whose epilogue is the table built by :func:`build_act_lut`."""
     _dev(a, w, c, lut)

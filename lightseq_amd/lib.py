@@ -50,6 +50,7 @@ _SIGNATURES = {
     "lsh_gemm_i8_i8o": (False, "pppiiifs"),
     "lsh_build_act_lut": (False, "pp" + "ifffi" + "s"),
     "lsh_gemm_i8_lut_i8o": (False, "pppp" + "iiif" + "s"),
+    "lsh_gemm_i8_decself_qkv_i8o_f16": (False, "pppppp" + "iiiiii" + "fff" + "s"),
     "lsh_gemm_i8_i32o_splitk": (False, "ppp" + "iiii" + "p" + "s"),
     "lsh_gemm_i8_preferred_ksplit": (False, "iii"),
     "lsh_ker_residual_bias_ln_planes_i32I_i8O_f16": (False, "p" + "il" + "ppppp" + "iiff" + "s" +

@@ -1,0 +1,73 @@
+"""GPU parity of the fused decode-step launches against the launcher sequences they replace,
+through the C ABI: integer outputs bit for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import DEV, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _k():
+    from lightseq_amd import kernels
+    return kernels
+
+
+@pytest.mark.parametrize("M,heads,d,K,max_step,step", [(16, 16, 64, 1024, 40, 7), (64, 16, 64, 1024, 24, 23),
+                                                       (3, 4, 32, 256, 9, 0), (7, 2, 128, 384, 5, 4),
+                                                       (200, 4, 64, 256, 6, 2)])
+def test_qkv_product_with_cache_append_equals_the_pair(rng, M, heads, d, K, max_step, step):
+    """lsh_gemm_i8_decself_qkv_i8o == lsh_gemm_i8_i8o followed by
+    ker_arrange_decself_qkv_i8I_i8O: q codes, and the cache slots (all other slots untouched)."""
+    H = heads * d
+    a = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(3 * H, K), dtype=np.int8)
+    bias = (rng.standard_normal(3 * H) * 0.4).astype(np.float16)
+    alpha = 2.5 / (np.sqrt(K) * 127)
+    ds, qs = 3.0 / 127, 127 / 3.5
+    fill = rng.integers(-127, 128, size=(2, M, heads, max_step, d), dtype=np.int8)
+
+    # reference sequence
+    c = torch.zeros((M, 3 * H), dtype=torch.int8, device=DEV)
+    _k().gemm_i8_i8o(to_dev(a), to_dev(w), c, M, 3 * H, K, alpha)
+    q0 = torch.zeros((M, H), dtype=torch.int8, device=DEV)
+    kv0 = to_dev(fill.copy())
+    _k().ker_arrange_decself_qkv_i8I_i8O_launcher(M, H, c, to_dev(bias), q0, kv0[0], kv0[1], heads, d,
+                                                  max_step, step, 1024, ds, qs)
+    # fused
+    q1 = torch.full((M, H), 5, dtype=torch.int8, device=DEV)
+    kv1 = to_dev(fill.copy())
+    _k().gemm_i8_decself_qkv_i8o(to_dev(a), to_dev(w), to_dev(bias), q1, kv1[0], kv1[1], M, H, K, heads,
+                                 max_step, step, alpha, ds, qs)
+    np.testing.assert_array_equal(to_np(q1), to_np(q0))
+    np.testing.assert_array_equal(to_np(kv1), to_np(kv0))
+    # only slot `step` of the caches changed
+    got = to_np(kv1)
+    keep = np.ones(max_step, dtype=bool)
+    keep[step] = False
+    np.testing.assert_array_equal(got[:, :, :, keep, :], fill[:, :, :, keep, :])
+
+
+def test_qkv_product_with_cache_append_rejects_bad_arguments(rng):
+    from lightseq_amd.lib import LSHError
+    M, heads, d, K, max_step = 4, 2, 24, 128, 4  # d not a multiple of 16
+    H = heads * d
+    a = torch.zeros((M, K), dtype=torch.int8, device=DEV)
+    w = torch.zeros((3 * H, K), dtype=torch.int8, device=DEV)
+    bias = torch.zeros(3 * H, dtype=torch.float16, device=DEV)
+    q = torch.zeros((M, H), dtype=torch.int8, device=DEV)
+    kv = torch.zeros((2, M, heads, max_step, d), dtype=torch.int8, device=DEV)
+    with pytest.raises(LSHError):
+        _k().gemm_i8_decself_qkv_i8o(a, w, bias, q, kv[0], kv[1], M, H, K, heads, max_step, 0, 1e-3, 1e-2,
+                                     30.0)
+    d = 32
+    H = heads * d
+    w = torch.zeros((3 * H, K), dtype=torch.int8, device=DEV)
+    bias = torch.zeros(3 * H, dtype=torch.float16, device=DEV)
+    q = torch.zeros((M, H), dtype=torch.int8, device=DEV)
+    kv = torch.zeros((2, M, heads, max_step, d), dtype=torch.int8, device=DEV)
+    with pytest.raises(LSHError):  # step outside the cache
+        _k().gemm_i8_decself_qkv_i8o(a, w, bias, q, kv[0], kv[1], M, H, K, heads, max_step, max_step, 1e-3,
+                                     1e-2, 30.0)
