@@ -221,6 +221,13 @@ int lsh_launch_scaled_colsum_f32(const void* inp, void* out, int rows, int cols,
  * model/cublas_helper.h:50-58 cublaslt_gemm<int32_t,int32_t>. */
 int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n, int k,
                      lsh_stream_t stream);
+/* Selects, for the calling thread's later layer-norm launches (the lsh_ker_norm_layer_* and
+ * lsh_ker_residual_bias_ln_* entry points, hidden <= 1024, 16-byte aligned operands), the
+ * kernel that gives a workgroup to each row: its small code starts faster on launches of a
+ * few rows (decode steps).  It adds a row's elements in another order than the default
+ * kernel, so keep one setting for all launches whose results are compared with each other.
+ * Returns the previous setting (0 / 1).  No counterpart in the reference. */
+int lsh_layer_norm_row_kernel(int on);
 /* Decode-step QKV product with ker_arrange_decself_qkv_i8I_i8O
  * (kernels/transformerKernels_int8.cc.cu:1432-1513; call sites model/quant_decoder.cc.cu:660-674,
  * model/quant_gpt_encoder.cc.cu:640-653) as its epilogue: A [step_token_num, k] x W [3*hidden, k]

@@ -105,6 +105,7 @@ int lsh_launch_dequantize_tensor_f32(const int32_t* input, void* output, int bat
 }
 
 // ---- LayerNorm family --------------------------------------------------------------
+int lsh_layer_norm_row_kernel(int on) { return ln_set_few_rows(on != 0) ? 1 : 0; }
 int lsh_ker_norm_layer_resual_i8O_f16(int token_num, int hidden_size, lsh_stream_t stream,
                                       void* input, int8_t* output, const void* scale,
                                       const void* bias, const void* residual_bias,

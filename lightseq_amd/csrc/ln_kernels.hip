@@ -338,6 +338,114 @@ __global__ void ln_rows_generic_kernel(const AccT* __restrict__ gemm_out, T* res
   }
 }
 
+// One row per workgroup, 4 consecutive elements per lane (hidden <= 4 * blockDim.x, hidden
+// % 4 == 0), reductions across the wavefronts through LDS, the accumulator planes summed in
+// a rolled loop.  The code is a fifth of the 8-wide kernel's: a kernel's instructions are
+// fetched cold on every launch (about 0.35 us per KB measured), which is what a launch
+// over a few rows costs most.
+template <typename T, typename AccT, int MODE>
+__global__ void __launch_bounds__(1024)
+ln_row_wg_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
+                 int8_t* __restrict__ out_q, const T* __restrict__ scale,
+                 const T* __restrict__ bias, const T* __restrict__ residual_bias,
+                 const T* __restrict__ colsum, int hidden, float dequant_scale,
+                 float quant_scale, int is_post_ln, int nparts, long part_stride, int tokens,
+                 int tpr) {
+  // `tpr` threads (a multiple of 64) per row, blockDim.x / tpr rows per workgroup
+  __shared__ float red[2][16];
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wpr = tpr >> 6;                  // wavefronts per row
+  const int rib = threadIdx.x / tpr;         // row within the workgroup
+  const int row = blockIdx.x * (blockDim.x / tpr) + rib;
+  const int e = (threadIdx.x - rib * tpr) * 4;
+  const bool on = e < hidden && row < tokens;
+  const long base = (long)(row < tokens ? row : 0) * hidden;
+  auto row_total = [&](float v, float* r) {  // sum over the row's wavefronts
+    v = wave_sum(v);
+    if (lane == 0) r[wid] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < wpr; ++i) t += r[rib * wpr + i];
+    return t;
+  };
+  float x[4] = {0.f, 0.f, 0.f, 0.f}, g[4], b[4], rb[4] = {0.f, 0.f, 0.f, 0.f};
+  if (on) {
+    ld4(scale, e, g);
+    ld4(bias, e, b);
+    if (MODE != kLnResOut && residual_bias != nullptr) ld4(residual_bias, e, rb);
+    float r[4];
+    ld4(residual, base + e, r);
+    if (MODE == kLnFirst) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) x[k] = TT<T>::safe(r[k]);
+    } else {
+      float a[4];
+      if constexpr (sizeof(AccT) == 4) {
+        int4 acc = *reinterpret_cast<const int4*>(gemm_out + base + e);
+        for (int p = 1; p < nparts; ++p) {
+          const int4 m = *reinterpret_cast<const int4*>(gemm_out + p * part_stride + base + e);
+          acc.x += m.x; acc.y += m.y; acc.z += m.z; acc.w += m.w;
+        }
+        a[0] = (float)acc.x; a[1] = (float)acc.y; a[2] = (float)acc.z; a[3] = (float)acc.w;
+      } else {
+        ld4_acc(gemm_out, base + e, a);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) x[k] = a[k] * dequant_scale + TT<T>::safe(r[k]);
+      if (colsum != nullptr) {
+        float c[4];
+        ld4(colsum, e, c);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) x[k] += TT<T>::safe(c[k]);
+      }
+    }
+  }
+  const float mean = row_total((x[0] + x[1]) + (x[2] + x[3]), red[0]) / (float)hidden;
+  float var = 0.f;
+  if (on) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float t = x[k] - mean;
+      var += t * t;
+    }
+  }
+  const float rstd = rsqrtf(row_total(var, red[1]) / (float)hidden + kLnEpsilon);
+  if (!on) return;
+  float o[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) o[k] = (x[k] - mean) * rstd * TT<T>::safe(g[k]) + TT<T>::safe(b[k]);
+  if (MODE == kLnResOut) {
+    st4(out_t, base + e, o);
+  } else {
+    *reinterpret_cast<uint32_t*>(out_q + base + e) =
+        pack4_i8(float2int8(o[0], quant_scale), float2int8(o[1], quant_scale),
+                 float2int8(o[2], quant_scale), float2int8(o[3], quant_scale));
+    float w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float keep = is_post_ln ? o[k] : x[k];
+      w[k] = (MODE == kLnFirst) ? keep + rb[k] : TT<T>::rnd(keep) + rb[k];
+    }
+    st4(residual, base + e, w);
+  }
+}
+
+// The workgroup-per-row kernel is chosen by the caller, never by the row count: the two
+// kernels add a row's elements in different orders, and a sequence's result must not depend
+// on how many other rows share its launch.  The decode-step paths (a few rows per launch)
+// select it for the duration of a step; everything else runs the 8-wide kernel.  Measured at
+// hidden 768 / 1024: 3.3-4.7 us against 4.2-5.9 us up to 1024 rows, 8.6-10.9 us against
+// 7.3-8.3 us at 4096 rows; more than one row per workgroup was slower at every size.
+static thread_local bool g_ln_few_rows = false;
+LnFewRowsScope::LnFewRowsScope() : _prev(g_ln_few_rows) { g_ln_few_rows = true; }
+LnFewRowsScope::~LnFewRowsScope() { g_ln_few_rows = _prev; }
+bool ln_set_few_rows(bool on) {
+  const bool prev = g_ln_few_rows;
+  g_ln_few_rows = on;
+  return prev;
+}
+constexpr int kLnRowsPerWg = 1;
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <typename T, typename AccT, int MODE>
@@ -352,6 +460,14 @@ static int launch_ln(const AccT* gemm_out, T* residual, T* out_t, int8_t* out_q,
                       aligned16(residual) && aligned16(out_t) && aligned16(out_q) &&
                       aligned16(scale) && aligned16(bias) && aligned16(residual_bias) &&
                       aligned16(colsum);
+  if (vec_ok && hidden <= 1024 && g_ln_few_rows) {
+    const int tpr = ((hidden / 4 + 63) / 64) * 64;
+    const int rpb = kLnRowsPerWg * tpr <= 1024 ? kLnRowsPerWg : 1;
+    ln_row_wg_kernel<T, AccT, MODE><<<(tokens + rpb - 1) / rpb, rpb * tpr, 0, stream>>>(
+        gemm_out, residual, out_t, out_q, scale, bias, residual_bias, colsum, hidden,
+        dequant_scale, quant_scale, is_post_ln, nparts, part_stride, tokens, tpr);
+    return lsh_check_launch("ln_row_wg_kernel");
+  }
   if (vec_ok && hidden % 8 == 0) {
     // LPR = 64 when the row fills whole 512-element steps, otherwise two rows per wavefront
 #define LSH_LN8_CASE(LPR, IT)                                                                    \
@@ -362,7 +478,7 @@ static int launch_ln(const AccT* gemm_out, T* residual, T* out_t, int8_t* out_q,
     if (hidden <= 256) LSH_LN8_CASE(32, 1);
     else if (hidden <= 512) LSH_LN8_CASE(32, 2);
     else if (hidden <= 768) LSH_LN8_CASE(32, 3);
-    else if (hidden <= 1024) LSH_LN8_CASE(32, 4);
+    else if (hidden <= 1024) LSH_LN8_CASE(64, 2);
     else if (hidden <= 1536) LSH_LN8_CASE(64, 3);
     else LSH_LN8_CASE(64, 4);
 #undef LSH_LN8_CASE

@@ -64,6 +64,23 @@ int residual_bias_ln_i32I(const int32_t* input, const T* scale, const T* bias, c
                           long part_stride = 0);
 // `nparts` > 1: `input` holds that many int32 accumulator planes `part_stride` elements apart
 // (split-K GEMM output, gemm_i8_i32o_splitk) which are summed before the dequantisation.
+//
+// While an object of this type lives, the calling thread's layer-norm launches (hidden <=
+// 1024, aligned operands) use the workgroup-per-row kernel, whose small code starts faster
+// on launches of a few rows.  It sums a row in another order than the default kernel, so a
+// caller keeps one choice for all launches whose results it compares (the decode-step
+// loops hold it for every step).
+struct LnFewRowsScope {
+  LnFewRowsScope();
+  ~LnFewRowsScope();
+  LnFewRowsScope(const LnFewRowsScope&) = delete;
+  LnFewRowsScope& operator=(const LnFewRowsScope&) = delete;
+
+ private:
+  bool _prev;
+};
+// The same switch without a scope (returns the previous setting).
+bool ln_set_few_rows(bool on);
 
 // ---- head split / merge, embedding (arrange_kernels.hip) -------------------------
 template <typename T>

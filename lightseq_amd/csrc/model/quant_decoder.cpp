@@ -246,6 +246,7 @@ void QuantDecoder::project_encoder_output() {
 }
 
 bool QuantDecoder::run_step() {
+  LnFewRowsScope few_rows;  // every step of every batch size: layer norms by the row kernel
   embedding();
   for (_layer_id = 0; _layer_id < _tw._n_dec_layer; _layer_id++) {
     self_attention();

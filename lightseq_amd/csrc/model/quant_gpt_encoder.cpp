@@ -181,6 +181,7 @@ void QuantGptEncoder::prompt_pass(const int* ids) {
 
 // one cached step for the tokens in _last_ids at position _batch_seq_len - 1 (:363-377)
 void QuantGptEncoder::step_pass() {
+  LnFewRowsScope few_rows;  // every step of every batch size: layer norms by the row kernel
   const int H = _tw._hidden_size, B = _batch_size;
   const float Q = _quant_range;
   LSH_CALL(gpt_embedding_i8I<__half>(B, 1, H, _stream, _int8_emb.get(), _pos_emb.get(),

@@ -186,6 +186,12 @@ def gemm_i8_i32o_splitk(a, w, c, m, n, k, ksplit):
     return used.value
 
 
+def layer_norm_row_kernel(on):
+    """Select (True) or deselect the workgroup-per-row layer-norm kernel for this thread's
+    later launches; returns the previous setting."""
+    return bool(lib.load().lsh_layer_norm_row_kernel(int(bool(on))))
+
+
 def gemm_i8_preferred_ksplit(m, n, k):
     return lib.load().lsh_gemm_i8_preferred_ksplit(m, n, k)
 

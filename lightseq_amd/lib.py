@@ -53,6 +53,7 @@ _SIGNATURES = {
     "lsh_gemm_i8_decself_qkv_i8o_f16": (False, "pppppp" + "iiiiii" + "fff" + "s"),
     "lsh_gemm_i8_i32o_splitk": (False, "ppp" + "iiii" + "p" + "s"),
     "lsh_gemm_i8_preferred_ksplit": (False, "iii"),
+    "lsh_layer_norm_row_kernel": (False, "i"),
     "lsh_ker_residual_bias_ln_planes_i32I_i8O_f16": (False, "p" + "il" + "ppppp" + "iiff" + "s" +
                                                      "ip"),
     "lsh_gemm_i8_bias_gelu_i8o_f16": (False, "pppp" + "iiifffs"),
