@@ -269,7 +269,11 @@ struct EpiQkvF16 {
   static const char* name() { return "EpiQkvF16"; }
 };
 
-template <typename Epi, int MB, int NB>
+// FULL: every 16-column group of the output exists and may be stored as a vector (N % 16
+// == 0 and the epilogue's alignment holds), so the scalar tail path is not even compiled:
+// a kernel's instructions are fetched cold on every launch, and code that is never run
+// still sits between the lines that are.
+template <typename Epi, int MB, int NB, bool FULL = false>
 __device__ __forceinline__ void store_tile_acc(const Epi& epi, const v16i (&acc)[MB][NB], int m0,
                                                int n0, int wm, int wn, int l32, int g, int M, int N,
                                                bool vec_store, long m_off = 0) {
@@ -280,7 +284,8 @@ __device__ __forceinline__ void store_tile_acc(const Epi& epi, const v16i (&acc)
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
         const int n = n0 + wn * (NB * 32) + j * 32 + 16 * g;
-        if (n < N) epi.store16(m + m_off, n, N, acc[i][j], vec_store && n + 16 <= N);
+        if (n < N)
+          epi.store16(m + m_off, n, N, acc[i][j], FULL ? true : (vec_store && n + 16 <= N));
       }
     }
   }
@@ -308,7 +313,7 @@ __device__ __forceinline__ void tile_of(int t, int nblk, int tiles_m, int tiles_
 // Preconditions (checked by the dispatcher): K % 128 == 0, (rows-1)*K + 128 < 2^32 for
 // both operands, operands 16-byte aligned.
 // ---------------------------------------------------------------------------------
-template <typename Epi>
+template <typename Epi, bool FULL>
 __global__ void __launch_bounds__(256)
 gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
                       int N, int K, int tiles_m, int tiles_n, bool vec_store, int ksplit) {
@@ -430,8 +435,8 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
                 __builtin_amdgcn_mfma_i32_32x32x32_i8(av[ks][jj], bv[ks][i], acc[i][jj], 0, 0, 0);
       st ^= 1;
     }
-    store_tile_acc<Epi, 2, 2>(epi, acc, tm * kBM, tn * kBN, wm, wn, l32, g, M, N, vec_store,
-                              (long)(item / ntile) * M);
+    store_tile_acc<Epi, 2, 2, FULL>(epi, acc, tm * kBM, tn * kBN, wm, wn, l32, g, M, N, vec_store,
+                                    (long)(item / ntile) * M);
   }
   __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
 }
@@ -550,7 +555,7 @@ gemm_i8_generic_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ 
 // accumulators of the 4 wavefronts meet in LDS and go through the same epilogues.
 // Preconditions: K % 128 == 0, operands 16-byte aligned.
 // ---------------------------------------------------------------------------------
-template <typename Epi, int MBLK>
+template <typename Epi, int MBLK, bool FULL>
 __global__ void __launch_bounds__(256)
 gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
                       int N, int K, int, int, bool vec_store, int ksplit) {
@@ -614,7 +619,8 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
              (red[2][wave][r][lane] + red[3][wave][r][lane]);
     const long m = wave * 32 + l32;
     const int n = n0 + 16 * g;
-    if (m < M && n < N) epi.store16(m + (long)part * M, n, N, c, vec_store && n + 16 <= N);
+    if (m < M && n < N)
+      epi.store16(m + (long)part * M, n, N, c, FULL ? true : (vec_store && n + 16 <= N));
   }
 }
 
@@ -668,23 +674,34 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   const int tiles_m = (M + kBM - 1) / kBM, tiles_n = (N + kBN - 1) / kBN;
   const int tiles = tiles_m * tiles_n;
   const size_t smem = 2 * (size_t)(kBM + kBN) * kBK;
-  static bool attr_stream = false, attr_generic = false;  // per Epi instantiation
-  static bool attr_skinny = true;                          // static LDS: nothing to set
+  static bool attr_stream = false, attr_stream_full = false, attr_generic = false;  // per Epi
+  static bool attr_skinny = true;  // static LDS: nothing to set
   if (ksplit < 1 || (ksplit > 1 && K % (ksplit * kBK) != 0))
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: K does not split into whole 128-byte steps");
+  const bool full = vec_store && N % 16 == 0;  // no column tail: the lean instantiation
   if (M <= 64 && K % kBK == 0) {
     const int grid = ((N + 31) / 32) * ksplit;
-    if (M <= 32)
-      return launch(gemm_i8_skinny_kernel<Epi, 1>, grid, 0, A, W, epi, M, N, K, 0, 0, vec_store, s,
-                    &attr_skinny, ksplit);
-    return launch(gemm_i8_skinny_kernel<Epi, 2>, grid, 0, A, W, epi, M, N, K, 0, 0, vec_store, s,
-                  &attr_skinny, ksplit);
+    if (M <= 32) {
+      if (full)
+        return launch(gemm_i8_skinny_kernel<Epi, 1, true>, grid, 0, A, W, epi, M, N, K, 0, 0,
+                      vec_store, s, &attr_skinny, ksplit);
+      return launch(gemm_i8_skinny_kernel<Epi, 1, false>, grid, 0, A, W, epi, M, N, K, 0, 0,
+                    vec_store, s, &attr_skinny, ksplit);
+    }
+    if (full)
+      return launch(gemm_i8_skinny_kernel<Epi, 2, true>, grid, 0, A, W, epi, M, N, K, 0, 0,
+                    vec_store, s, &attr_skinny, ksplit);
+    return launch(gemm_i8_skinny_kernel<Epi, 2, false>, grid, 0, A, W, epi, M, N, K, 0, 0,
+                  vec_store, s, &attr_skinny, ksplit);
   }
   if (stream_ok(M, N, K)) {
     const int items = tiles * ksplit;
     const int grid = items < 512 ? items : 512;  // 2 resident workgroups per compute unit
-    return launch(gemm_i8_stream_kernel<Epi>, grid, smem, A, W, epi, M, N, K, tiles_m, tiles_n,
-                  vec_store, s, &attr_stream, ksplit);
+    if (full)
+      return launch(gemm_i8_stream_kernel<Epi, true>, grid, smem, A, W, epi, M, N, K, tiles_m,
+                    tiles_n, vec_store, s, &attr_stream_full, ksplit);
+    return launch(gemm_i8_stream_kernel<Epi, false>, grid, smem, A, W, epi, M, N, K, tiles_m,
+                  tiles_n, vec_store, s, &attr_stream, ksplit);
   }
   if (ksplit != 1) return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: this shape cannot split K");
   return launch(gemm_i8_generic_kernel<Epi>, tiles, smem, A, W, epi, M, N, K, tiles_m, tiles_n,

@@ -218,18 +218,16 @@ ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
       } else {
         float a[8];
         if constexpr (sizeof(AccT) == 4) {
-          // all planes are requested before the first use (independent loads)
-          int acc[8], more[7][8];
+          // further planes in a rolled loop: launches of a few rows, where the planes come
+          // from, use the row kernel, and this one stays small
+          int acc[8];
           ld8_acc(gemm_out, base + e, acc);
+          for (int p = 1; p < nparts; ++p) {
+            int more[8];
+            ld8_acc(gemm_out + p * part_stride, base + e, more);
 #pragma unroll
-          for (int p = 1; p < 8; ++p)
-            if (p < nparts) ld8_acc(gemm_out + p * part_stride, base + e, more[p - 1]);
-#pragma unroll
-          for (int p = 1; p < 8; ++p)
-            if (p < nparts) {
-#pragma unroll
-              for (int k = 0; k < 8; ++k) acc[k] += more[p - 1][k];
-            }
+            for (int k = 0; k < 8; ++k) acc[k] += more[k];
+          }
 #pragma unroll
           for (int k = 0; k < 8; ++k) a[k] = (float)acc[k];
         } else {
