@@ -161,7 +161,8 @@ __device__ __forceinline__ void dequant16_bias(const uint4& w, const _Float16* _
   hi = xh + b1;
 }
 
-template <int D, int MODE, int NW>
+// ONE: the sequence fits one block of 128 keys; the multi-block paths are not compiled.
+template <int D, int MODE, int NW, bool ONE>
 // Two workgroups of four wavefronts share a compute unit for head sizes up to 64 (the
 // compiler is told to stay within that register budget); 128 needs the whole file.
 __global__ void __launch_bounds__(64 * NW, D <= 64 ? 2 : 1)
@@ -237,8 +238,9 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
-  int nkb = (S + 127) / 128;
-  if (causal) nkb = min(nkb, min((int)(blockIdx.x + 1) * (32 * NW) - 1, S - 1) / 128 + 1);
+  int nkb = ONE ? 1 : (S + 127) / 128;
+  if (!ONE && causal) nkb = min(nkb, min((int)(blockIdx.x + 1) * (32 * NW) - 1, S - 1) / 128 + 1);
+  if (ONE) nkb = 1;  // (a constant for the compiler)
   for (int phase = 0; phase < 2; ++phase) {
     for (int kb = 0; kb < nkb; ++kb) {
       const int key0 = kb * 128;
@@ -466,19 +468,24 @@ static bool launch_attn(int dim_per_head, int seq_len, int batch_heads, hipStrea
                         __half* ctx, int8_t* ctx_q, float quant_scale, int head_num, float alpha,
                         float dq) {
 #define LSH_ATTN(DD, NWV)                                                                      \
-  encself_attn_kernel<DD, MODE, NWV>                                                           \
+  if (seq_len <= 128)                                                                          \
+    encself_attn_kernel<DD, MODE, NWV, true>                                                   \
+        <<<dim3((seq_len + 32 * NWV - 1) / (32 * NWV), batch_heads), 64 * NWV, 0, s>>>(        \
+            q, k, v, pad_mask, ctx, ctx_q, quant_scale, seq_len, head_num, alpha, dq);         \
+  else                                                                                         \
+    encself_attn_kernel<DD, MODE, NWV, false>                                                  \
       <<<dim3((seq_len + 32 * NWV - 1) / (32 * NWV), batch_heads), 64 * NWV, 0, s>>>(          \
           q, k, v, pad_mask, ctx, ctx_q, quant_scale, seq_len, head_num, alpha, dq)
   const bool wide = seq_len > 64;
   switch (dim_per_head) {
     case 32:
-      if (wide) LSH_ATTN(32, 4); else LSH_ATTN(32, 2);
+      if (wide) { LSH_ATTN(32, 4); } else { LSH_ATTN(32, 2); }
       return true;
     case 64:
-      if (wide) LSH_ATTN(64, 4); else LSH_ATTN(64, 2);
+      if (wide) { LSH_ATTN(64, 4); } else { LSH_ATTN(64, 2); }
       return true;
     case 128:
-      if (wide) LSH_ATTN(128, 4); else LSH_ATTN(128, 2);
+      if (wide) { LSH_ATTN(128, 4); } else { LSH_ATTN(128, 2); }
       return true;
     default:
       return false;
