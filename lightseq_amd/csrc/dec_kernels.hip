@@ -575,6 +575,87 @@ encdec_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   }
 }
 
+// The same for head sizes 32 / 64 / 128 with 16-byte aligned operands: a key row and the
+// query are read as 16-byte vectors and the value rows eight steps at a time, every load
+// issued before the first is used; the sums run in the same order as above (dimension by
+// dimension for a score, step by step for a context element), so the results are the same
+// bits.
+template <int D>
+__global__ void __launch_bounds__(256)
+encdec_attn_vec_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
+                       const __half* __restrict__ v, const int* __restrict__ pad_mask,
+                       __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale,
+                       long waves_total, int beam_size, int head_num, int seq_len,
+                       float alpha_h) {
+#pragma clang fp contract(off)
+  extern __shared__ float probs_all[];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const long w = (long)blockIdx.x * 4 + wid;
+  if (w >= waves_total) return;
+  const int padded = (seq_len + 63) & ~63;
+  float* probs = probs_all + (long)wid * padded;
+  const long bh = w / beam_size;
+  const int beam = (int)(w % beam_size);
+  const long b = bh / head_num;
+  const int head = (int)(bh % head_num);
+  const int* mask = pad_mask + b * seq_len;
+  const __half* qp = q + w * D;  // [B, h, beam, d]
+  const __half* kb = k + bh * (long)seq_len * D;
+  const __half* vb = v + bh * (long)seq_len * D;
+
+  half8_t qv[D / 8];
+#pragma unroll
+  for (int c = 0; c < D / 8; ++c) qv[c] = *reinterpret_cast<const half8_t*>(qp + c * 8);
+
+  float mx = kFloatInfNeg;
+  for (int j = lane; j < padded; j += 64) {
+    float sc = kFloatInfNeg;
+    if (j < seq_len) {
+      half8_t kv[D / 8];
+#pragma unroll
+      for (int c = 0; c < D / 8; ++c)
+        kv[c] = *reinterpret_cast<const half8_t*>(kb + (long)j * D + c * 8);
+      float acc = 0.f;
+#pragma unroll
+      for (int c = 0; c < D / 8; ++c)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc += __half2float(qv[c].v[e]) * __half2float(kv[c].v[e]);
+      sc = TT<__half>::rnd(alpha_h * acc);
+      if (!mask[j]) mx = fmaxf(mx, sc);
+    }
+    probs[j] = sc;
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int j = lane; j < padded; j += 64) {
+    const float e = (j < seq_len && !mask[j]) ? __expf(probs[j] - mx) : 0.f;
+    probs[j] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  for (int j = lane; j < padded; j += 64) probs[j] = TT<__half>::rnd(probs[j] / sum);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const long row = b * beam_size + beam;
+  for (int dd = lane; dd < D; dd += 64) {
+    float acc = 0.f;
+    for (int j0 = 0; j0 < seq_len; j0 += 8) {
+      __half vv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)  // clamped, not predicated: the loads stay back to back
+        vv[u] = vb[(long)min(j0 + u, seq_len - 1) * D + dd];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (j0 + u < seq_len) acc += probs[j0 + u] * __half2float(vv[u]);
+    }
+    const float c = TT<__half>::rnd(acc);
+    if (ctx) ctx[w * D + dd] = __float2half_rn(c);
+    if (ctx_q)
+      ctx_q[row * ((long)head_num * D) + (long)head * D + dd] = (int8_t)float2int8(c, quant_scale);
+  }
+}
+
 int encdec_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,
                          __half* ctx, int8_t* ctx_q, float quant_scale, int batch_size,
                          int beam_size, int head_num, int batch_seq_len, int dim_per_head,
@@ -587,6 +668,19 @@ int encdec_attention_f16(const __half* q, const __half* k, const __half* v, cons
   const long waves = (long)batch_size * head_num * beam_size;
   const float alpha_h = __half2float(__float2half_rn(sqrtf(1.f / (float)dim_per_head)));
   const size_t lds = (size_t)4 * ((batch_seq_len + 63) & ~63) * sizeof(float);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
+                         reinterpret_cast<uintptr_t>(v)) & 15u) == 0;
+  if (aligned && (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128)) {
+#define LSH_ENCDEC(D)                                                                           \
+  encdec_attn_vec_kernel<D><<<(int)((waves + 3) / 4), 256, lds, s>>>(                           \
+      q, k, v, pad_mask, ctx, ctx_q, quant_scale, waves, beam_size, head_num, batch_seq_len,    \
+      alpha_h)
+    if (dim_per_head == 32) LSH_ENCDEC(32);
+    else if (dim_per_head == 64) LSH_ENCDEC(64);
+    else LSH_ENCDEC(128);
+#undef LSH_ENCDEC
+    return lsh_check_launch("encdec_attn_vec_kernel");
+  }
   encdec_attn_kernel<<<(int)((waves + 3) / 4), 256, lds, s>>>(
       q, k, v, pad_mask, ctx, ctx_q, quant_scale, waves, beam_size, head_num, batch_seq_len,
       dim_per_head, alpha_h);

@@ -71,3 +71,29 @@ def test_qkv_product_with_cache_append_rejects_bad_arguments(rng):
     with pytest.raises(LSHError):  # step outside the cache
         _k().gemm_i8_decself_qkv_i8o(a, w, bias, q, kv[0], kv[1], M, H, K, heads, max_step, max_step, 1e-3,
                                      1e-2, 30.0)
+
+
+@pytest.mark.parametrize("B,beam,heads,S,d", [(3, 4, 2, 37, 64), (2, 2, 3, 64, 32), (1, 4, 2, 130, 128),
+                                              (16, 4, 16, 64, 64)])
+def test_cross_attention_vector_kernel_equals_the_scalar_one(rng, B, beam, heads, S, d):
+    """lsh_encdec_attention_f16 picks a vector-load kernel for 16-byte aligned operands and
+    head sizes 32 / 64 / 128; it sums in the same order as the general kernel, so a query
+    buffer shifted by 8 bytes (general kernel) gives the same context bits and codes."""
+    q = (rng.standard_normal((B, heads, beam, d)) * 0.7).astype(np.float16)
+    k = (rng.standard_normal((B, heads, S, d)) * 0.7).astype(np.float16)
+    v = (rng.standard_normal((B, heads, S, d)) * 0.7).astype(np.float16)
+    mask = np.zeros((B, S), dtype=np.int32)
+    for b in range(B):
+        mask[b, rng.integers(S // 2, S + 1):] = 1
+    qs = 127 / 1.5
+    outs = []
+    for shift in (0, 4):  # halfs: 0 keeps the 16-byte alignment, 4 breaks it
+        qbuf = torch.zeros(q.size + 8, dtype=torch.float16, device=DEV)
+        qd = qbuf[shift:shift + q.size].view(B, heads, beam, d)
+        qd.copy_(to_dev(q))
+        ctx = torch.zeros((B, heads, beam, d), dtype=torch.float16, device=DEV)
+        ctx_q = torch.zeros((B * beam, heads * d), dtype=torch.int8, device=DEV)
+        _k().encdec_attention(qd, to_dev(k), to_dev(v), to_dev(mask), ctx, ctx_q, qs, B, beam, heads, S, d)
+        outs.append((to_np(ctx), to_np(ctx_q)))
+    np.testing.assert_array_equal(outs[0][0].view(np.uint16), outs[1][0].view(np.uint16))
+    np.testing.assert_array_equal(outs[0][1], outs[1][1])
