@@ -200,7 +200,7 @@ decself_attn_kernel(int32_t* __restrict__ scores, const int8_t* __restrict__ q,
 // across lanes (shuffles) and wavefronts (LDS): a tree instead of the ascending-step order
 // of the kernel above, so a context code can differ by one from it where the float sum
 // lands next to a rounding boundary.  Requires d in {32, 64, 128} and 16-byte aligned rows.
-template <int D, int NWV>
+template <int D, int NWV, int UN>
 __global__ void __launch_bounds__(64 * NWV)
 decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k_cache,
                        const int8_t* __restrict__ v_cache, int8_t* __restrict__ new_v,
@@ -224,7 +224,6 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
   // The cache is read in rounds of UN independent 16-byte loads per lane (UN * NWV * KPW
   // steps per round), all issued before the first is used: a step costs one memory round
   // trip per round instead of one per KPW * 4 cached steps.
-  constexpr int UN = 8;
 
   // scores -> scaled logits in LDS
   float mx = kFloatInfNeg;
@@ -365,16 +364,30 @@ int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v
   const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
                          reinterpret_cast<uintptr_t>(v_cache)) & 15u) == 0;
   if (aligned && (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128)) {
-    constexpr int kWaves = 8;  // one workgroup per compute unit: width buys loads in flight
+    // 8 wavefronts once the cache is long (width buys loads in flight), 4 below.  The
+    // choice depends on the step count only, never on the number of rows: the two widths
+    // sum the values in different trees, and a row's result must not depend on its batch.
+    // The loads in flight per lane (UN) follow the cache length too: unrolled rounds that
+    // a short cache never fills are code to fetch and clamped loads to wait for.
+    const bool wide = step_num > 256;
     const size_t lds =
-        ((size_t)((step_num + 63) & ~63) + 16 + kWaves * dim_per_head) * sizeof(float);
+        ((size_t)((step_num + 63) & ~63) + 16 + (wide ? 8 : 4) * dim_per_head) * sizeof(float);
 #define LSH_DECSELF(D)                                                                          \
-  decself_attn_wg_kernel<D, kWaves><<<batch_head_num, 64 * kWaves, lds, s>>>(                   \
-      q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,      \
-      quant_scale)
-    if (dim_per_head == 32) LSH_DECSELF(32);
-    else if (dim_per_head == 64) LSH_DECSELF(64);
-    else LSH_DECSELF(128);
+  if (wide)                                                                                     \
+    decself_attn_wg_kernel<D, 8, 8><<<batch_head_num, 512, lds, s>>>(                           \
+        q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
+        quant_scale);                                                                           \
+  else if (step_num > 128 * 64 / D)                                                             \
+    decself_attn_wg_kernel<D, 4, 4><<<batch_head_num, 256, lds, s>>>(                           \
+        q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
+        quant_scale);                                                                           \
+  else                                                                                          \
+    decself_attn_wg_kernel<D, 4, 2><<<batch_head_num, 256, lds, s>>>(                           \
+        q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
+        quant_scale)
+    if (dim_per_head == 32) { LSH_DECSELF(32); }
+    else if (dim_per_head == 64) { LSH_DECSELF(64); }
+    else { LSH_DECSELF(128); }
 #undef LSH_DECSELF
     return lsh_check_launch("decself_attn_wg_kernel");
   }
@@ -640,13 +653,14 @@ encdec_attn_vec_kernel(const __half* __restrict__ q, const __half* __restrict__ 
   const long row = b * beam_size + beam;
   for (int dd = lane; dd < D; dd += 64) {
     float acc = 0.f;
-    for (int j0 = 0; j0 < seq_len; j0 += 8) {
-      __half vv[8];
+    constexpr int UV = 32;  // value rows in flight per lane
+    for (int j0 = 0; j0 < seq_len; j0 += UV) {
+      __half vv[UV];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)  // clamped, not predicated: the loads stay back to back
+      for (int u = 0; u < UV; ++u)  // clamped, not predicated: the loads stay back to back
         vv[u] = vb[(long)min(j0 + u, seq_len - 1) * D + dd];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < UV; ++u)
         if (j0 + u < seq_len) acc += probs[j0 + u] * __half2float(vv[u]);
     }
     const float c = TT<__half>::rnd(acc);
