@@ -563,6 +563,117 @@ beam_topk_kernel(const int8_t* __restrict__ logits, const T* __restrict__ logit_
   }
 }
 
+// The same selection for vocabularies of up to 32 * 1024 entries with the row's logits kept
+// in registers: thread t loads its ids t, t + 1024, ... once (all loads in flight together)
+// and every later pass -- maximum, sum of exponentials in the same ascending order, the
+// `beam_size` arg-max rounds -- works on registers.  Same arithmetic and the same order as
+// beam_topk_kernel, hence the same bits.  VEC (vocab % 16 == 0, 16-byte aligned rows):
+// thread t owns ids 16 t .. 16 t + 15 of each 16384-id half instead and reads them with
+// 16-byte loads; the sum of exponentials then runs in another order (a last-place
+// difference of the log-sum-exp, shared by all candidates of the row).
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(1024)
+beam_topk_reg_kernel(const int8_t* __restrict__ logits, const T* __restrict__ logit_bias,
+                     const float* __restrict__ seq_probs, const float* __restrict__ seq_score,
+                     const int* __restrict__ alive_seq, float dq, float* __restrict__ top_score,
+                     int* __restrict__ top_idx, int vocab, int max_step, float length_norm,
+                     int cur_step, int beam_size, int end_id) {
+#pragma clang fp contract(off)
+  constexpr int NI = 32;
+  __shared__ float red[32];
+  __shared__ ScoreIdx wbest[16];
+  const int row = blockIdx.x, t = threadIdx.x;
+  const int lane = t & 63, wid = t >> 6;
+  const int batch_id = row / beam_size, beam_id = row % beam_size;
+  float* os = top_score + (long)row * beam_size;
+  int* oi = top_idx + (long)row * beam_size;
+  if (cur_step != 0 && alive_seq[(long)row * max_step + cur_step] == end_id) {
+    if (t < beam_size) {
+      os[t] = t == 0 ? seq_score[row] : -INFINITY;
+      oi[t] = t == 0 ? end_id + beam_id * vocab : kNoCand;
+    }
+    return;
+  }
+  const int8_t* lr = logits + (long)row * vocab;
+  float lg[NI];
+  auto id_of = [&](int i) { return VEC ? (i >> 4) * 16384 + 16 * t + (i & 15) : t + 1024 * i; };
+  if (VEC) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int v0 = h * 16384 + 16 * t;
+      if (v0 < vocab) {
+        const uint4 w = *reinterpret_cast<const uint4*>(lr + v0);
+        float b[16];
+        ld4(logit_bias, v0, *reinterpret_cast<float(*)[4]>(b));
+        ld4(logit_bias, v0 + 4, *reinterpret_cast<float(*)[4]>(b + 4));
+        ld4(logit_bias, v0 + 8, *reinterpret_cast<float(*)[4]>(b + 8));
+        ld4(logit_bias, v0 + 12, *reinterpret_cast<float(*)[4]>(b + 12));
+        const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          lg[h * 16 + e] = (float)unpack_i8(ws[e >> 2], e & 3) * dq + b[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) lg[h * 16 + e] = 0.f;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int v = t + 1024 * i;
+      lg[i] = v < vocab ? logit_of(lr, logit_bias, v, dq) : 0.f;
+    }
+  }
+  float tmax = kFloatInfNeg;
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+    if (id_of(i) < vocab) tmax = fmaxf(tmax, lg[i]);
+  const float max_logit = block_max(tmax, red);
+  float se = 0.f;
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+    if (id_of(i) < vocab) se += __expf(fmaxf(lg[i] - max_logit, kLogitThreshMin));
+  const float sum_exp = block_sum(se, red);
+  const float base = seq_probs[row] - logf(sum_exp) - max_logit;
+#pragma unroll
+  for (int i = 0; i < NI; ++i) lg[i] = cand_score(lg[i], base, length_norm, batch_id);
+  // A thread keeps the first of its own candidates that comes after the last pick; a round
+  // is a block-wide arg-max over these, and only the thread that owned the pick looks
+  // through its registers again (every other thread's candidate still comes after it).
+  auto my_first_after = [&](const ScoreIdx& prev) {
+    ScoreIdx best;
+    best.s = -INFINITY;
+    best.i = kNoCand;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      ScoreIdx c;
+      c.s = lg[i];
+      c.i = id_of(i);
+      if (c.i < vocab && before(prev, c) && before(c, best)) best = c;
+    }
+    return best;
+  };
+  ScoreIdx prev;
+  prev.s = INFINITY;
+  prev.i = -1;
+  ScoreIdx mine = my_first_after(prev);
+  for (int k = 0; k < beam_size; ++k) {
+    ScoreIdx best = wave_first(mine);
+    __syncthreads();
+    if (lane == 0) wbest[wid] = best;
+    __syncthreads();
+    best = wbest[0];
+    for (int w2 = 1; w2 < 16; ++w2)
+      if (before(wbest[w2], best)) best = wbest[w2];
+    if (t == 0) {
+      os[k] = best.i == kNoCand ? -INFINITY : best.s;
+      oi[k] = best.i == kNoCand ? kNoCand : beam_id * vocab + best.i;
+    }
+    prev = best;
+    if (best.i == mine.i && best.i != kNoCand) mine = my_first_after(prev);
+  }
+}
+
 // beam_merge_kernel: one block, one wavefront per sentence (sentences are dealt to the
 // wavefronts round-robin).  Picks the sentence's best `beam_size` of its
 // beam_size * beam_size proposals in (score descending, candidate id ascending) order
@@ -646,9 +757,21 @@ int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_p
     return lsh_fail(LSH_ERR_INVALID, "beam_search_step: the sequence buffers must differ");
   if ((long)beam_size * vocab_size > 0x7ffffffe)
     return lsh_fail(LSH_ERR_UNSUPPORTED, "beam_search_step: beam_size * vocab_size overflows");
-  beam_topk_kernel<T><<<batch_size * beam_size, 1024, 0, s>>>(
-      logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score, top_idx,
-      vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+  const bool vec = vocab_size % 16 == 0 &&
+                   ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(logit_bias)) &
+                    15u) == 0;
+  if (vocab_size <= 32 * 1024 && vec)
+    beam_topk_reg_kernel<T, true><<<batch_size * beam_size, 1024, 0, s>>>(
+        logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score,
+        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+  else if (vocab_size <= 32 * 1024)
+    beam_topk_reg_kernel<T, false><<<batch_size * beam_size, 1024, 0, s>>>(
+        logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score,
+        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+  else
+    beam_topk_kernel<T><<<batch_size * beam_size, 1024, 0, s>>>(
+        logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score,
+        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
   if (int rc = lsh_check_launch("beam_topk_kernel")) return rc;
   beam_merge_kernel<<<1, 1024, 0, s>>>(top_score, top_idx, old_alive_seq, new_alive_seq,
                                        seq_probs, seq_score, parent, num_finished, batch_size,

@@ -257,6 +257,8 @@ BEAM_CASES = [  # batch, beam, vocab, max_step, cur_step, threads
     (2, 1, 500, 16, 2, 1024),
     (1, 32, 5000, 16, 4, 1024),
     (2, 16, 2100, 16, 1, 32),
+    (2, 4, 32768, 16, 2, 1024),   # largest vocabulary of the register-resident top-k kernel
+    (1, 4, 40000, 16, 2, 1024),   # beyond it: the looping kernel
 ]
 
 
