@@ -295,6 +295,13 @@ __device__ __forceinline__ void store_tile_acc(const Epi& epi, const v16i (&acc)
 // dealt round-robin to the 8 XCDs; renumber so that each XCD (own L2) works on a
 // contiguous run of tiles, walked in column-major order of 8-tile-tall groups so that a
 // run shares W columns and A rows.
+// Work-item counts stay below 2^24 (checked by the dispatcher): with both operands masked to
+// 24 bits the compiler divides through a float reciprocal, a dozen instructions instead of
+// the forty of a full 32-bit division -- this arithmetic runs before the first load of a
+// launch and sits in the kernel four times.
+__device__ __forceinline__ int div24(int a, int b) {
+  return (int)(((unsigned)a & 0xffffffu) / ((unsigned)b & 0xffffffu));
+}
 __device__ __forceinline__ void tile_of(int t, int nblk, int tiles_m, int tiles_n, int& tile_m,
                                         int& tile_n) {
   const int per = nblk / 8, rem = nblk % 8;
@@ -302,10 +309,12 @@ __device__ __forceinline__ void tile_of(int t, int nblk, int tiles_m, int tiles_
   const int pid = xcd * per + (xcd < rem ? xcd : rem) + loc;
   constexpr int GROUP = 8;
   const int group_sz = GROUP * tiles_n;
-  const int first_m = (pid / group_sz) * GROUP;
+  const int grp = div24(pid, group_sz);
+  const int in_grp = pid - grp * group_sz;
+  const int first_m = grp * GROUP;
   const int gm = min(tiles_m - first_m, GROUP);
-  tile_m = first_m + (pid % group_sz) % gm;
-  tile_n = (pid % group_sz) / gm;
+  tile_n = div24(in_grp, gm);
+  tile_m = first_m + (in_grp - tile_n * gm);
 }
 
 // ---------------------------------------------------------------------------------
@@ -338,9 +347,10 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   uint32_t a_src[NA], w_src[NW];
   auto set_src = [&](int j) {
     const int item = blockIdx.x + j * G;
-    const uint32_t koff = (uint32_t)(item / ntile) * (uint32_t)kpart;
+    const int part = ksplit == 1 ? 0 : div24(item, ntile);
+    const uint32_t koff = (uint32_t)part * (uint32_t)kpart;
     int tm, tn;
-    tile_of(item % ntile, ntile, tiles_m, tiles_n, tm, tn);
+    tile_of(item - part * ntile, ntile, tiles_m, tiles_n, tm, tn);
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
       const int row = (wave + 4 * i) * 8 + (lane >> 3);
@@ -400,8 +410,9 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   int st = 0;
   for (int j = 0; j < my_tiles; ++j) {
     const int item = blockIdx.x + j * G;
+    const int part = ksplit == 1 ? 0 : div24(item, ntile);
     int tm, tn;
-    tile_of(item % ntile, ntile, tiles_m, tiles_n, tm, tn);
+    tile_of(item - part * ntile, ntile, tiles_m, tiles_n, tm, tn);
     v16i acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -436,7 +447,7 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
       st ^= 1;
     }
     store_tile_acc<Epi, 2, 2, FULL>(epi, acc, tm * kBM, tn * kBN, wm, wn, l32, g, M, N, vec_store,
-                                    (long)(item / ntile) * M);
+                                    (long)part * M);
   }
   __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
 }
@@ -678,6 +689,8 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   static bool attr_skinny = true;  // static LDS: nothing to set
   if (ksplit < 1 || (ksplit > 1 && K % (ksplit * kBK) != 0))
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: K does not split into whole 128-byte steps");
+  if ((long)tiles_m * tiles_n * ksplit >= (1L << 24))
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: more than 2^24 output tiles");
   const bool full = vec_store && N % 16 == 0;  // no column tail: the lean instantiation
   if (M <= 64 && K % kBK == 0) {
     const int grid = ((N + 31) / 32) * ksplit;
