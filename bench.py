@@ -114,6 +114,9 @@ def fused_kernel_rates(cfg, reps=50):
         ("encself_attention (fused QK^T, softmax, PV, merge+quant)", M * H * (3 * 2 + 1),
          lambda: K.encself_attention(qkv[0], qkv[1], qkv[2], mask, None, ctx8, 30.0, BATCH, SEQ, h,
                                      d)),
+        ("encself_attention on the int8 QKV product (what the model runs)", M * H * (3 + 1),
+         lambda: K.encself_attention_i8qkv(q8_3h, b3h, 0.05, mask, None, ctx8, 30.0, BATCH, SEQ, h,
+                                           d)),
     ]
     out = {}
     for name, nbytes, fn in cases:

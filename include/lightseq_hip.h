@@ -240,6 +240,15 @@ int lsh_gemm_i8_decself_qkv_i8o_f16(const int8_t* A, const int8_t* W, const void
                                     int step_token_num, int hidden, int k, int head_num,
                                     int max_step, int step_id, float alpha, float dequant_scale,
                                     float quant_scale, lsh_stream_t stream);
+/* Decode-step cross-attention query product with ker_arrange_encdec_q_i8I
+ * (kernels/transformerKernels_int8.cc.cu:1596-1645; call site model/quant_decoder.cc.cu:745-760)
+ * as its epilogue: A [step_token_num, k] x W [hidden, k] -> int8 code (alpha) ->
+ * half(code * dequant_scale) + bias -> fp16 new_q [step_token_num / beam_size, head_num,
+ * beam_size, hidden / head_num].  Same bits as lsh_gemm_i8_i8o followed by
+ * lsh_ker_arrange_encdec_q_i8I_f16.  No counterpart in the reference. */
+int lsh_gemm_i8_encdec_q_f16(const int8_t* A, const int8_t* W, const void* q_bias, void* new_q,
+                             int step_token_num, int hidden, int k, int beam_size, int head_num,
+                             float alpha, float dequant_scale, lsh_stream_t stream);
 /* The bias + activation + requantisation epilogue as a table: after the requantisation an
  * element is one of 255 codes, so what follows depends only on (column, code).
  * lsh_build_act_lut fills lut [n, 256] (entry [col][code + 128]) with what

@@ -344,6 +344,12 @@ int lsh_gemm_i8_decself_qkv_i8o_f16(const int8_t* A, const int8_t* W, const void
                                  head_num, max_step, step_id, alpha, dequant_scale, quant_scale,
                                  HS(stream));
 }
+int lsh_gemm_i8_encdec_q_f16(const int8_t* A, const int8_t* W, const void* q_bias, void* new_q,
+                             int step_token_num, int hidden, int k, int beam_size, int head_num,
+                             float alpha, float dequant_scale, lsh_stream_t stream) {
+  return gemm_i8_encdec_q_f16(A, W, H(q_bias), HM(new_q), step_token_num, hidden, k, beam_size,
+                              head_num, alpha, dequant_scale, HS(stream));
+}
 int lsh_gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int m,
                         int n, int k, float alpha, lsh_stream_t stream) {
   return gemm_i8_lut_i8o(A, W, C, lut, m, n, k, alpha, HS(stream));

@@ -148,6 +148,37 @@ struct EpiDecQkvI8 {
   static const char* name() { return "EpiDecQkvI8"; }
 };
 
+// Decode-step cross-attention query product followed by ker_arrange_encdec_q_i8I
+// (inference/kernels/transformerKernels_int8.cc.cu:1596-1645; call site
+// model/quant_decoder.cc.cu:745-760): code -> half(code * dq) + bias (a half add) -> fp16 q
+// [batch, heads, beam, d].
+struct EpiEncdecQF16 {
+  __half* new_q;
+  const __half* bias;
+  float alpha, dequant_scale;
+  int beam_size, head_num, dim_per_head;
+  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool) const {
+    const int head = n / dim_per_head, dim = n - head * dim_per_head;
+    const long batch_id = m / beam_size, beam_id = m - batch_id * beam_size;
+    __half* dst = new_q + ((batch_id * head_num + head) * beam_size + beam_id) * dim_per_head + dim;
+    const half8_t b0 = *reinterpret_cast<const half8_t*>(bias + n);
+    const half8_t b1 = *reinterpret_cast<const half8_t*>(bias + n + 8);
+    half8_t lo, hi;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      lo.v[k] = __float2half_rn(dequant_add_bias_h(requant_acc(c[k], alpha), dequant_scale,
+                                                   __half2float(b0.v[k])));
+      hi.v[k] = __float2half_rn(dequant_add_bias_h(requant_acc(c[8 + k], alpha), dequant_scale,
+                                                   __half2float(b1.v[k])));
+    }
+    *reinterpret_cast<half8_t*>(dst) = lo;
+    *reinterpret_cast<half8_t*>(dst + 8) = hi;
+    (void)N;
+  }
+  bool vec_ok(int) const { return true; }
+  static const char* name() { return "EpiEncdecQF16"; }
+};
+
 // The same with the scale read from device memory (the csrc layers keep their clip values
 // and the alpha derived from them on the device: csrc/kernels/cuda/cublas_wrappers.cpp:134
 // CUBLASLT_POINTER_MODE_DEVICE).
@@ -841,6 +872,21 @@ int gemm_i8_decself_qkv_i8o(const int8_t* A, const int8_t* W, const __half* qkv_
                   EpiDecQkvI8{new_q, new_k, new_v, qkv_bias, alpha, dequant_scale, quant_scale,
                               hidden, head_num, d, max_step, step_id},
                   step_token_num, 3 * hidden, K, s);
+}
+
+int gemm_i8_encdec_q_f16(const int8_t* A, const int8_t* W, const __half* q_bias, __half* new_q,
+                         int step_token_num, int hidden, int K, int beam_size, int head_num,
+                         float alpha, float dequant_scale, hipStream_t s) {
+  if (!q_bias || !new_q || head_num <= 0 || hidden <= 0 || hidden % head_num != 0 ||
+      beam_size <= 0 || step_token_num <= 0 || step_token_num % beam_size != 0)
+    return lsh_fail(LSH_ERR_INVALID, "int8 gemm (cross-attention q): bad arguments");
+  const int d = hidden / head_num;
+  if (d % 16 != 0 ||
+      ((reinterpret_cast<uintptr_t>(q_bias) | reinterpret_cast<uintptr_t>(new_q)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "int8 gemm (cross-attention q): needs dim_per_head % 16 == 0 and aligned output");
+  return dispatch(A, W, EpiEncdecQF16{new_q, q_bias, alpha, dequant_scale, beam_size, head_num, d},
+                  step_token_num, hidden, K, s);
 }
 
 int gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, __half* new_qkv, const __half* qkv_bias,

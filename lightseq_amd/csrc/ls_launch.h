@@ -149,6 +149,11 @@ int gemm_i8_decself_qkv_i8o(const int8_t* A, const int8_t* W, const __half* qkv_
                             int8_t* new_k, int8_t* new_v, int step_token_num, int hidden, int K,
                             int head_num, int max_step, int step_id, float alpha,
                             float dequant_scale, float quant_scale, hipStream_t s);
+// Decode-step cross-attention query product with ker_arrange_encdec_q_i8I as its epilogue:
+// fp16 q [batch, heads, beam, d].
+int gemm_i8_encdec_q_f16(const int8_t* A, const int8_t* W, const __half* q_bias, __half* new_q,
+                         int step_token_num, int hidden, int K, int beam_size, int head_num,
+                         float alpha, float dequant_scale, hipStream_t s);
 int gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int M, int N,
                     int K, float alpha, hipStream_t s);
 //   writes q, k, v as fp16 [B, h, S, d] at new_qkv + {0, 1, 2} * max_batch_dim

@@ -321,11 +321,18 @@ void QuantDecoder::encdec_attention() {
   const float* c = &_dec_clip_max[_layer_id * 19];
   const float Q = _quant_range;
 
-  LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_encdec_q.get(), _buf_a.get(), M, H, H,
-                       c[2] * c[8] / (c[14] * Q), _stream));
-  LSH_CALL(arrange_encdec_q_i8I<__half>(M, H, _stream, _buf_a.get(), w.b_encdec_q.get(),
-                                        _query_buf1.get(), _tw._beam_size, _tw._dim_per_head,
-                                        _tw._head_num, c[14] / Q));
+  // q product; its epilogue is ker_arrange_encdec_q_i8I (fp16 q [batch, heads, beam, d])
+  if (_tw._dim_per_head % 16 == 0) {
+    LSH_CALL(gemm_i8_encdec_q_f16(_buf_b.get(), w.w_encdec_q.get(), w.b_encdec_q.get(),
+                                  _query_buf1.get(), M, H, H, _tw._beam_size, _tw._head_num,
+                                  c[2] * c[8] / (c[14] * Q), c[14] / Q, _stream));
+  } else {
+    LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_encdec_q.get(), _buf_a.get(), M, H, H,
+                         c[2] * c[8] / (c[14] * Q), _stream));
+    LSH_CALL(arrange_encdec_q_i8I<__half>(M, H, _stream, _buf_a.get(), w.b_encdec_q.get(),
+                                          _query_buf1.get(), _tw._beam_size, _tw._dim_per_head,
+                                          _tw._head_num, c[14] / Q));
+  }
   // scores -> masked softmax -> context -> merge heads + quantise, one kernel
   LSH_CALL(encdec_attention_f16(
       _query_buf1.get(), _encdec_k.get() + (size_t)_layer_id * _layer_size_encdec_k,

@@ -524,6 +524,14 @@ def gemm_i8_decself_qkv_i8o(a, w, qkv_bias, new_q, new_k, new_v, step_token_num,
          quant_scale, current_stream())
 
 
+def gemm_i8_encdec_q(a, w, q_bias, new_q, step_token_num, hidden, k, beam_size, head_num, alpha,
+                     dequant_scale):
+    """Decode-step cross-attention query product with ker_arrange_encdec_q_i8I as its epilogue."""
+    _dev(a, w, q_bias, new_q)
+    call("lsh_gemm_i8_encdec_q_f16", ptr(a), ptr(w), ptr(q_bias), ptr(new_q), step_token_num, hidden,
+         k, beam_size, head_num, alpha, dequant_scale, current_stream())
+
+
 def gemm_i8_lut_i8o(a, w, c, lut, m, n, k, alpha):
     """int8-output GEMM whose epilogue is the table built by :func:`build_act_lut`."""
     _dev(a, w, c, lut)

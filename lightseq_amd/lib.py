@@ -51,6 +51,7 @@ _SIGNATURES = {
     "lsh_build_act_lut": (False, "pp" + "ifffi" + "s"),
     "lsh_gemm_i8_lut_i8o": (False, "pppp" + "iiif" + "s"),
     "lsh_gemm_i8_decself_qkv_i8o_f16": (False, "pppppp" + "iiiiii" + "fff" + "s"),
+    "lsh_gemm_i8_encdec_q_f16": (False, "pppp" + "iiiii" + "ff" + "s"),
     "lsh_gemm_i8_i32o_splitk": (False, "ppp" + "iiii" + "p" + "s"),
     "lsh_gemm_i8_preferred_ksplit": (False, "iii"),
     "lsh_layer_norm_row_kernel": (False, "i"),

@@ -97,3 +97,21 @@ def test_cross_attention_vector_kernel_equals_the_scalar_one(rng, B, beam, heads
         outs.append((to_np(ctx), to_np(ctx_q)))
     np.testing.assert_array_equal(outs[0][0].view(np.uint16), outs[1][0].view(np.uint16))
     np.testing.assert_array_equal(outs[0][1], outs[1][1])
+
+
+@pytest.mark.parametrize("batch,beam,heads,d,K", [(16, 4, 16, 64, 1024), (3, 2, 4, 32, 256), (2, 1, 2, 128, 384),
+                                                  (40, 4, 4, 64, 256)])
+def test_cross_attention_q_product_equals_the_pair(rng, batch, beam, heads, d, K):
+    """lsh_gemm_i8_encdec_q_f16 == lsh_gemm_i8_i8o followed by ker_arrange_encdec_q_i8I, bit for bit."""
+    M, H = batch * beam, heads * d
+    a = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(H, K), dtype=np.int8)
+    bias = (rng.standard_normal(H) * 0.4).astype(np.float16)
+    alpha, ds = 2.5 / (np.sqrt(K) * 127), 3.0 / 127
+    c = torch.zeros((M, H), dtype=torch.int8, device=DEV)
+    _k().gemm_i8_i8o(to_dev(a), to_dev(w), c, M, H, K, alpha)
+    q0 = torch.zeros((batch, heads, beam, d), dtype=torch.float16, device=DEV)
+    _k().ker_arrange_encdec_q_i8I_launcher(M, H, c, to_dev(bias), q0, beam, d, heads, 1024, ds)
+    q1 = torch.full((batch, heads, beam, d), 3.0, dtype=torch.float16, device=DEV)
+    _k().gemm_i8_encdec_q(to_dev(a), to_dev(w), to_dev(bias), q1, M, H, K, beam, heads, alpha, ds)
+    np.testing.assert_array_equal(to_np(q1).view(np.uint16), to_np(q0).view(np.uint16))
