@@ -96,6 +96,21 @@ int lsh_launch_quant_bias_add_transform_20314_f32(void* output, uint8_t* clip_ma
                                                   int dim_2, int dim_3, int dim_4,
                                                   lsh_stream_t stream, const void* out_clip_max,
                                                   int in_col32);
+/* kernels.h:72-75 launch_bias_add_transform_20314 (transform_kernels.cu:140-235): input
+ * [dim_0, dim_1, dim_2, dim_3, dim_4] + bias [dim_2, dim_3, dim_4] -> [dim_2, dim_0, dim_3,
+ * dim_1, dim_4] */
+int lsh_launch_bias_add_transform_20314_f16(void* output, const void* input, const void* bias,
+                                            int dim_0, int dim_1, int dim_2, int dim_3, int dim_4,
+                                            lsh_stream_t stream);
+int lsh_launch_bias_add_transform_20314_f32(void* output, const void* input, const void* bias,
+                                            int dim_0, int dim_1, int dim_2, int dim_3, int dim_4,
+                                            lsh_stream_t stream);
+/* kernels.h:183-185 launch_concat3_dim1 (general_kernels.cu:187-234): inp1 [sz0, sz1_1, sz2]
+ * and inp2 [sz0, sz1_2, sz2] joined along dimension 1; inp1 may be null when sz1_1 is 0 */
+int lsh_launch_concat3_dim1_f16(const void* inp1, const void* inp2, void* output, int sz0, int sz2,
+                                int sz1_1, int sz1_2, lsh_stream_t stream);
+int lsh_launch_concat3_dim1_f32(const void* inp1, const void* inp2, void* output, int sz0, int sz2,
+                                int sz1_1, int sz1_2, lsh_stream_t stream);
 /* kernels.h:95-98 launch_transform4d_0213 (transform_kernels.cu:444-560) */
 int lsh_launch_transform4d_0213_f16(void* output, const void* vals, int batch_size, int seq_len,
                                     int hidden_dim, int nhead, int trans_count,
@@ -220,6 +235,15 @@ int lsh_feed_forward_i8(int bsz, int output_size, int input_size, const int8_t* 
 int lsh_layer_attention_f16(const void* q, const void* k, const void* v, const void* attn_mask,
                             void* ctx, int batch_size, int seq_len, int heads, int dim_per_head,
                             int mask_future, lsh_stream_t stream);
+/* The same with its own number of keys, as the decoder layer needs it
+ * (layers/transformer_decoder_layer.cpp:173-189 a cached decoding step: from_len 1, to_len
+ * step + 1; :333-357 cross attention: to_len = source length).  q: [batch, heads, from_len,
+ * dim_per_head]; k, v: [batch, heads, to_len, dim_per_head]; attn_mask [batch, to_len] additive
+ * or null; ctx: [batch, from_len, heads * dim_per_head].  mask_future needs from_len == to_len. */
+int lsh_layer_cross_attention_f16(const void* q, const void* k, const void* v,
+                                  const void* attn_mask, void* ctx, int batch_size, int from_len,
+                                  int to_len, int heads, int dim_per_head, int mask_future,
+                                  lsh_stream_t stream);
 
 /* ---- layers (pybind/pybind_layer.cpp) ----------------------------------------------------------- */
 /* Context::Instance().set_stream (ops/includes/context.h:14-43): the stream every layer
@@ -241,10 +265,41 @@ int ls_create_transformer_encoder_layer_fp16(int layer_id, int max_batch_tokens,
 int ls_transformer_encoder_layer_fw_fp16(int layer_id, const void* input, const void* input_mask,
                                          void* output, int batch_size, int seq_len,
                                          int training_mode, int prelayernorm, int quant_mode);
-/* pybind_layer.cpp assign_layer_weight_grad<__half>: binds the flat fp16 parameter blob
- * (transformer_encoder_layer.h:66-105: qkvw, qkvb, ow, ob, nw, nb, inter_w, inter_b, out_w,
- * out_b, ffn_nw, ffn_nb, 12 clip_max) of layer "TransformerEncoderLayer"; the gradient blob is
- * accepted and ignored. */
+/* pybind_layer.cpp:110-132 create_transformer_decoder_layer<__half>: registers a
+ * TransformerDecoderLayer (layers/includes/transformer_decoder_layer.h:19-32) under layer_id.
+ * Create every decoder layer of a stack before binding the parameters of layer 0: its blob
+ * holds the cross-attention k/v projection of all of them. */
+int ls_create_transformer_decoder_layer_fp16(int layer_id, int max_batch_tokens, int max_seq_len,
+                                             int hidden_dim, int num_heads, int intermediate_size,
+                                             float attn_prob_dropout_ratio,
+                                             float activation_dropout_ratio,
+                                             float hidden_dropout_ratio, int is_pre_ln,
+                                             const char* activation_fn);
+/* pybind_layer.cpp:134-185 transformer_decoder_layer_fw<__half>.  step < 0: the whole target
+ * sequence, dec_input fp16 [batch, trg_seq_len, hidden], cache null.  step >= 0: one decoding
+ * step, trg_seq_len is the beam size, dec_input [batch * beam, 1, hidden] and cache points to
+ * 5 device pointers: new k, new v [batch * beam * heads, step + 1, head_dim] (written),
+ * previous k, v [.., step, head_dim] (read; may be null at step 0), and, for layer 0, the
+ * cross-attention k/v of all layers [layers * 2, batch, heads, src_seq_len, head_dim] (written
+ * at step 0).  enc_output fp16 [batch, src_seq_len, hidden] is read by layer 0 only;
+ * enc_mask fp16 [batch, src_seq_len] additive or null.  The reference derives step and the
+ * lengths from its tensor arguments; here they are explicit.  training_mode must be 0 and
+ * quant_mode 1. */
+int ls_transformer_decoder_layer_fw_fp16(int layer_id, const void* dec_input,
+                                         const void* enc_output, const void* enc_mask,
+                                         void* dec_output, int batch_size, int trg_seq_len,
+                                         int src_seq_len, int step, void* const* cache,
+                                         int training_mode, int prelayernorm, int quant_mode);
+/* Number of fp16 elements the parameter blob of a registered layer holds ("TransformerEncoderLayer"
+ * or "TransformerDecoderLayer"), written to *count; no counterpart in the reference, whose
+ * Python side computes it. */
+int ls_layer_param_count(const char* layer_name, int layer_id, long long* count);
+/* pybind_layer.cpp assign_layer_weight_grad<__half>: binds the flat fp16 parameter blob of
+ * layer "TransformerEncoderLayer" (transformer_encoder_layer.h:66-105: qkvw, qkvb, ow, ob, nw,
+ * nb, inter_w, inter_b, out_w, out_b, ffn_nw, ffn_nb, 12 clip_max) or "TransformerDecoderLayer"
+ * (transformer_decoder_layer.h:100-168: self attention qkvw, qkvb, ow, ob, nw, nb; cross
+ * attention qw, qb, ow, ob, nw, nb; inter_w, inter_b, out_w, out_b, ffn_nw, ffn_nb; 24
+ * clip_max; layer 0: kvw, kvb of all layers); the gradient blob is accepted and ignored. */
 int ls_assign_layer_weight_grad_fp16(const void* weights, void* grads, const char* layer_name,
                                      int layer_id);
 /* pybind_layer.cpp create_quant_linear_layer<__half> / quant_linear_layer_fw<__half>

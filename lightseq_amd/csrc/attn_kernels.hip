@@ -169,7 +169,10 @@ __global__ void __launch_bounds__(64 * NW, D <= 64 ? 2 : 1)
 encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
                     const __half* __restrict__ v, const int* __restrict__ pad_mask,
                     __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale, int S,
-                    int head_num, float alpha, float dq) {
+                    int head_num, float alpha, float dq, int key_len) {
+  // number of keys: the layer mode (MODE 2) may attend over another sequence (cross
+  // attention, cached decoding); everywhere else keys and queries are the same S positions
+  const int Sk = MODE == kAttnLayer ? key_len : S;
   constexpr int KSTR = D + 8;    // halfs per K row in LDS (pad kills bank conflicts)
   constexpr int VSTR = 128 + 4;  // halfs per V^T row in LDS
   constexpr int CH = D / 8;      // 16-byte chunks per row
@@ -187,8 +190,8 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   constexpr int NT = 64 * NW;  // threads; 32 queries per wavefront
   const int qi = blockIdx.x * (32 * NW) + wave * 32 + l32;
   const _Float16* qb = reinterpret_cast<const _Float16*>(q) + (long)bh * S * D;
-  const _Float16* kbase = reinterpret_cast<const _Float16*>(k) + (long)bh * S * D;
-  const _Float16* vbase = reinterpret_cast<const _Float16*>(v) + (long)bh * S * D;
+  const _Float16* kbase = reinterpret_cast<const _Float16*>(k) + (long)bh * Sk * D;
+  const _Float16* vbase = reinterpret_cast<const _Float16*>(v) + (long)bh * Sk * D;
 
   // MODE 3: int8 codes [tokens, 3 * hidden] and the fp16 bias [3 * hidden]
   const int hidden3 = 3 * head_num * D;
@@ -238,8 +241,8 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
-  int nkb = ONE ? 1 : (S + 127) / 128;
-  if (!ONE && causal) nkb = min(nkb, min((int)(blockIdx.x + 1) * (32 * NW) - 1, S - 1) / 128 + 1);
+  int nkb = ONE ? 1 : (Sk + 127) / 128;
+  if (!ONE && causal) nkb = min(nkb, min((int)(blockIdx.x + 1) * (32 * NW) - 1, Sk - 1) / 128 + 1);
   if (ONE) nkb = 1;  // (a constant for the compiler)
   for (int phase = 0; phase < 2; ++phase) {
     for (int kb = 0; kb < nkb; ++kb) {
@@ -291,7 +294,7 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
           for (int c = tid; c < 128 * CH; c += NT) {
             const int row = c / CH, ch = c % CH;
             v8h kv = (v8h)(_Float16)0;
-            if (key0 + row < S)
+            if (key0 + row < Sk)
               kv = *reinterpret_cast<const v8h*>(kbase + (long)(key0 + row) * D + ch * 8);
             *reinterpret_cast<v8h*>(&Ks[row * KSTR + ch * 8]) = kv;
           }
@@ -303,7 +306,7 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
                 const int key = key0 + kg * 4 + r;
-                vv[r] = key < S ? *reinterpret_cast<const v8h*>(vbase + (long)key * D + ch * 8)
+                vv[r] = key < Sk ? *reinterpret_cast<const v8h*>(vbase + (long)key * D + ch * 8)
                                 : (v8h)(_Float16)0;
               }
 #pragma unroll
@@ -315,10 +318,10 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         }
         if (tid < 128) {
           if (MODE == kAttnLayer) {
-            msk[tid] = (key0 + tid < S) ? 0 : 1;
-            addm[tid] = (key0 + tid < S && pad_mask != nullptr)
+            msk[tid] = (key0 + tid < Sk) ? 0 : 1;
+            addm[tid] = (key0 + tid < Sk && pad_mask != nullptr)
                             ? __half2float(reinterpret_cast<const __half*>(
-                                  pad_mask)[(long)b * S + key0 + tid])
+                                  pad_mask)[(long)b * Sk + key0 + tid])
                             : 0.f;
           } else if (GPT) {
             msk[tid] = (key0 + tid < S) ? 0 : 1;
@@ -466,16 +469,17 @@ template <int MODE>
 static bool launch_attn(int dim_per_head, int seq_len, int batch_heads, hipStream_t s,
                         const __half* q, const __half* k, const __half* v, const int* pad_mask,
                         __half* ctx, int8_t* ctx_q, float quant_scale, int head_num, float alpha,
-                        float dq) {
+                        float dq, int key_len = -1) {
+  if (key_len < 0) key_len = seq_len;  // self attention: as many keys as queries
 #define LSH_ATTN(DD, NWV)                                                                      \
-  if (seq_len <= 128)                                                                          \
+  if (key_len <= 128)                                                                          \
     encself_attn_kernel<DD, MODE, NWV, true>                                                   \
         <<<dim3((seq_len + 32 * NWV - 1) / (32 * NWV), batch_heads), 64 * NWV, 0, s>>>(        \
-            q, k, v, pad_mask, ctx, ctx_q, quant_scale, seq_len, head_num, alpha, dq);         \
+            q, k, v, pad_mask, ctx, ctx_q, quant_scale, seq_len, head_num, alpha, dq, key_len); \
   else                                                                                         \
     encself_attn_kernel<DD, MODE, NWV, false>                                                  \
       <<<dim3((seq_len + 32 * NWV - 1) / (32 * NWV), batch_heads), 64 * NWV, 0, s>>>(          \
-          q, k, v, pad_mask, ctx, ctx_q, quant_scale, seq_len, head_num, alpha, dq)
+          q, k, v, pad_mask, ctx, ctx_q, quant_scale, seq_len, head_num, alpha, dq, key_len)
   const bool wide = seq_len > 64;
   switch (dim_per_head) {
     case 32:
@@ -560,9 +564,24 @@ int gpt_prefill_attention_f16(const __half* q_codes, const __half* k_codes, cons
 int layer_attention_f16(const __half* q, const __half* k, const __half* v, const __half* add_mask,
                         __half* ctx, int batch, int seq_len, int head_num, int dim_per_head,
                         bool mask_future, hipStream_t s) {
-  if (batch <= 0 || seq_len <= 0 || head_num <= 0 || !q || !k || !v || !ctx)
+  return layer_cross_attention_f16(q, k, v, add_mask, ctx, batch, seq_len, seq_len, head_num,
+                                   dim_per_head, mask_future, s);
+}
+
+// The same with its own number of keys: q [batch, heads, q_len, D], k and v [batch, heads,
+// k_len, D], additive mask [batch, k_len] (may be null), context [batch, q_len, heads * D].
+// The decoder layer of the csrc tree uses it for the cross attention (k_len = source length;
+// csrc/layers/transformer_decoder_layer.cpp:333-357) and for a cached step (q_len = 1,
+// k_len = step + 1, :173-189).  mask_future needs q_len == k_len.
+int layer_cross_attention_f16(const __half* q, const __half* k, const __half* v,
+                              const __half* add_mask, __half* ctx, int batch, int seq_len,
+                              int key_len, int head_num, int dim_per_head, bool mask_future,
+                              hipStream_t s) {
+  if (batch <= 0 || seq_len <= 0 || key_len <= 0 || head_num <= 0 || !q || !k || !v || !ctx ||
+      (mask_future && seq_len != key_len))
     return lsh_fail(LSH_ERR_INVALID, "layer_attention: bad arguments");
-  if (seq_len > 1024) return lsh_fail(LSH_ERR_UNSUPPORTED, "layer_attention: seq_len > 1024");
+  if (seq_len > 1024 || key_len > 1024)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "layer_attention: seq_len > 1024");
   if (((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
         reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(ctx)) & 15u) != 0)
     return lsh_fail(LSH_ERR_INVALID, "layer_attention: pointers must be 16-byte aligned");
@@ -572,7 +591,7 @@ int layer_attention_f16(const __half* q, const __half* k, const __half* v, const
   const int* m = reinterpret_cast<const int*>(add_mask);
   const float causal = mask_future ? 1.f : 0.f;
   if (!launch_attn<kAttnLayer>(dim_per_head, seq_len, batch * head_num, s, q, k, v, m, ctx,
-                               nullptr, 0.f, head_num, alpha, causal))
+                               nullptr, 0.f, head_num, alpha, causal, key_len))
     return lsh_fail(LSH_ERR_UNSUPPORTED, "layer_attention: dim_per_head must be 32, 64 or 128");
   return lsh_check_launch("encself_attn_kernel<layer>");
 }

@@ -94,6 +94,18 @@ LSH_BOTH(lsh_launch_quant_bias_add_transform_20314,
                                                       C<T>(clip_max), dim_0, dim_1, dim_2, dim_3,
                                                       dim_4, HS(stream), C<T>(out_clip_max));)
 
+LSH_BOTH(lsh_launch_bias_add_transform_20314,
+         (void* output, const void* input, const void* bias, int dim_0, int dim_1, int dim_2,
+          int dim_3, int dim_4, lsh_stream_t stream),
+         return opb_bias_add_transform_20314<T>(M<T>(output), C<T>(input), C<T>(bias), dim_0,
+                                                dim_1, dim_2, dim_3, dim_4, HS(stream));)
+
+LSH_BOTH(lsh_launch_concat3_dim1,
+         (const void* inp1, const void* inp2, void* output, int sz0, int sz2, int sz1_1,
+          int sz1_2, lsh_stream_t stream),
+         return opb_concat3_dim1<T>(C<T>(inp1), C<T>(inp2), M<T>(output), sz0, sz2, sz1_1, sz1_2,
+                                    HS(stream));)
+
 LSH_BOTH(lsh_launch_transform4d_0213,
          (void* output, const void* vals, int batch_size, int seq_len, int hidden_dim, int nhead,
           int trans_count, lsh_stream_t stream),
@@ -180,6 +192,15 @@ int lsh_layer_attention_f16(const void* q, const void* k, const void* v, const v
   return layer_attention_f16(C<__half>(q), C<__half>(k), C<__half>(v), C<__half>(attn_mask),
                              M<__half>(ctx), batch_size, seq_len, heads, dim_per_head,
                              mask_future != 0, HS(stream));
+}
+
+int lsh_layer_cross_attention_f16(const void* q, const void* k, const void* v,
+                                  const void* attn_mask, void* ctx, int batch_size, int from_len,
+                                  int to_len, int heads, int dim_per_head, int mask_future,
+                                  lsh_stream_t stream) {
+  return layer_cross_attention_f16(C<__half>(q), C<__half>(k), C<__half>(v), C<__half>(attn_mask),
+                                   M<__half>(ctx), batch_size, from_len, to_len, heads,
+                                   dim_per_head, mask_future != 0, HS(stream));
 }
 
 }  // extern "C"

@@ -332,6 +332,56 @@ quant_bias_add_transform_20314_kernel(T* __restrict__ out, const int8_t* __restr
   stv(out, o, x);
 }
 
+// T [d0, d1, d2, d3, d4] -> T [d2, d0, d3, d1, d4] with bias [d2, d3, d4] added
+// (launch_bias_add_transform_20314, transform_kernels.cu:140-235); T=half adds in half.
+template <typename T>
+__global__ void __launch_bounds__(256)
+bias_add_transform_20314_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                const T* __restrict__ bias, int d0, int d1, int d2, int d3,
+                                int d4, long nvec) {
+  constexpr int N = Vec<T>::N;
+  const long v = (long)blockIdx.x * 256 + threadIdx.x;
+  if (v >= nvec) return;
+  const long i = v * N;
+  const int d34 = d3 * d4;
+  const int e34 = (int)(i % d34);
+  long r = i / d34;
+  const int i2 = (int)(r % d2);
+  r /= d2;
+  const int i1 = (int)(r % d1);
+  const int i0 = (int)(r / d1);
+  const int i3 = e34 / d4, i4 = e34 % d4;
+  float x[N], b[N];
+  ldv(in, i, x);
+  ldv(bias, (long)i2 * d34 + e34, b);
+#pragma unroll
+  for (int k = 0; k < N; ++k) x[k] = TT<T>::rnd(x[k] + b[k]);
+  const long o = ((((long)i2 * d0 + i0) * d3 + i3) * d1 + i1) * d4 + i4;
+  stv(out, o, x);
+}
+
+// [sz0, sz1_1, sz2] ++ [sz0, sz1_2, sz2] -> [sz0, sz1_1 + sz1_2, sz2] along dim 1
+// (launch_concat3_dim1, general_kernels.cu:187-234)
+template <typename T>
+__global__ void __launch_bounds__(256)
+concat3_dim1_kernel(const T* __restrict__ inp1, const T* __restrict__ inp2, T* __restrict__ out,
+                    int sz2, int sz1_1, int sz1_2, long nvec) {
+  constexpr int N = Vec<T>::N;
+  const long v = (long)blockIdx.x * 256 + threadIdx.x;
+  if (v >= nvec) return;
+  const long i = v * N;
+  const int i2 = (int)(i % sz2);
+  long r = i / sz2;
+  const int i1 = (int)(r % (sz1_1 + sz1_2));
+  const long i0 = r / (sz1_1 + sz1_2);
+  float x[N];
+  if (i1 < sz1_1)
+    ldv(inp1, (i0 * sz1_1 + i1) * sz2 + i2, x);
+  else
+    ldv(inp2, (i0 * sz1_2 + (i1 - sz1_1)) * sz2 + i2, x);
+  stv(out, i, x);
+}
+
 // T [tc, b, nh, s, ad] -> [b, s, tc, nh, ad], optionally quantised
 template <typename T, bool QUANT>
 __global__ void __launch_bounds__(256)
@@ -570,6 +620,36 @@ int opb_quant_bias_add_transform_20314(T* out, uint8_t* cmask, const int8_t* in,
 }
 
 template <typename T>
+int opb_bias_add_transform_20314(T* out, const T* in, const T* bias, int d0, int d1, int d2,
+                                 int d3, int d4, hipStream_t s) {
+  if (!out || !in || !bias)
+    return lsh_fail(LSH_ERR_INVALID, "launch_bias_add_transform_20314: null pointer");
+  if (d0 <= 0 || d1 <= 0 || d2 <= 0 || d3 <= 0 || d4 <= 0 || d4 % Vec<T>::N != 0)
+    return lsh_fail(LSH_ERR_INVALID,
+                    "launch_bias_add_transform_20314: dim_4 must be a multiple of the vector "
+                    "width");
+  const long nvec = (long)d0 * d1 * d2 * d3 * d4 / Vec<T>::N;
+  bias_add_transform_20314_kernel<T><<<grid_for(nvec), 256, 0, s>>>(out, in, bias, d0, d1, d2,
+                                                                    d3, d4, nvec);
+  return lsh_check_launch("bias_add_transform_20314_kernel");
+}
+
+template <typename T>
+int opb_concat3_dim1(const T* inp1, const T* inp2, T* out, int sz0, int sz2, int sz1_1,
+                     int sz1_2, hipStream_t s) {
+  if (!out || (!inp1 && sz1_1 > 0) || (!inp2 && sz1_2 > 0))
+    return lsh_fail(LSH_ERR_INVALID, "launch_concat3_dim1: null pointer");
+  if (sz0 <= 0 || sz2 <= 0 || sz1_1 < 0 || sz1_2 < 0 || sz1_1 + sz1_2 == 0 ||
+      sz2 % Vec<T>::N != 0)
+    return lsh_fail(LSH_ERR_INVALID,
+                    "launch_concat3_dim1: the last dimension must be a multiple of the vector "
+                    "width");
+  const long nvec = (long)sz0 * (sz1_1 + sz1_2) * sz2 / Vec<T>::N;
+  concat3_dim1_kernel<T><<<grid_for(nvec), 256, 0, s>>>(inp1, inp2, out, sz2, sz1_1, sz1_2, nvec);
+  return lsh_check_launch("concat3_dim1_kernel");
+}
+
+template <typename T>
 int opb_transform4d_0213(T* out, int8_t* out_q, uint8_t* cmask, const T* vals, const T* cmax,
                          int batch, int seq, int hidden, int nhead, int tc, hipStream_t s) {
   const bool quant = out_q != nullptr;
@@ -687,6 +767,9 @@ int opb_quant_dropout_res_bias(T* out, uint8_t* mask, const int8_t* qvals, const
                                                      hipStream_t, const T*);                     \
   template int opb_transform4d_0213<T>(T*, int8_t*, uint8_t*, const T*, const T*, int, int, int, \
                                        int, int, hipStream_t);                                   \
+  template int opb_bias_add_transform_20314<T>(T*, const T*, const T*, int, int, int, int, int,  \
+                                               hipStream_t);                                     \
+  template int opb_concat3_dim1<T>(const T*, const T*, T*, int, int, int, int, hipStream_t);     \
   template int opb_dropout<T>(T*, const T*, uint8_t*, long, float, hipStream_t);                 \
   template int opb_dropout_res_bias<T>(T*, const T*, uint8_t*, const T*, const T*, long, int,    \
                                        float, hipStream_t);                                      \

@@ -4,10 +4,12 @@
 #include <map>
 #include <memory>
 #include <string>
+#include <vector>
 
 #include "../../../include/lightseq_ops.h"
 #include "context.h"
 #include "quant_linear_layer.h"
+#include "transformer_decoder_layer.h"
 #include "transformer_encoder_layer.h"
 
 using namespace lightseq::hip;
@@ -15,6 +17,7 @@ using namespace lightseq::hip;
 namespace {
 
 std::map<int, std::shared_ptr<TransformerEncoderLayer<__half>>> s_transformer_encoder_layers;
+std::map<int, std::shared_ptr<TransformerDecoderLayer<__half>>> s_transformer_decoder_layers;
 std::map<int, std::shared_ptr<QuantLinearLayer<__half>>> s_quant_linear_layers;
 
 template <typename F>
@@ -75,14 +78,73 @@ int ls_transformer_encoder_layer_fw_fp16(int layer_id, const void* input, const 
   });
 }
 
+int ls_create_transformer_decoder_layer_fp16(int layer_id, int max_batch_tokens, int max_seq_len,
+                                             int hidden_dim, int num_heads, int intermediate_size,
+                                             float attn_prob_dropout_ratio,
+                                             float activation_dropout_ratio,
+                                             float hidden_dropout_ratio, int is_pre_ln,
+                                             const char* activation_fn) {
+  return guarded([&] {
+    if (!activation_fn) throw std::runtime_error("activation_fn is null");
+    s_transformer_decoder_layers.erase(layer_id);  // a replaced layer leaves the shared count first
+    s_transformer_decoder_layers[layer_id] = std::make_shared<TransformerDecoderLayer<__half>>(
+        layer_id, max_batch_tokens, max_seq_len, hidden_dim, num_heads, intermediate_size,
+        attn_prob_dropout_ratio, activation_dropout_ratio, hidden_dropout_ratio, is_pre_ln != 0,
+        std::string(activation_fn));
+  });
+}
+
+int ls_transformer_decoder_layer_fw_fp16(int layer_id, const void* dec_input,
+                                         const void* enc_output, const void* enc_mask,
+                                         void* dec_output, int batch_size, int trg_seq_len,
+                                         int src_seq_len, int step, void* const* cache,
+                                         int training_mode, int prelayernorm, int quant_mode) {
+  (void)prelayernorm;  // fixed at construction, as in the reference (the argument is unused there)
+  return guarded([&] {
+    auto layer = find_layer(s_transformer_decoder_layers, layer_id, "Decoder layer");
+    std::vector<__half*> cache_vec;
+    if (step >= 0) {
+      if (!cache) throw std::runtime_error("a decoding step needs the cache pointers");
+      for (int i = 0; i < 5; ++i) cache_vec.push_back(reinterpret_cast<__half*>(cache[i]));
+    }
+    layer->set_cur_batch_shape(batch_size, trg_seq_len, src_seq_len, step);
+    layer->SetTrainingMode(training_mode != 0);
+    layer->SetQuantMode(quant_mode != 0);
+    layer->Forward(reinterpret_cast<const __half*>(dec_input),
+                   reinterpret_cast<const __half*>(enc_output),
+                   reinterpret_cast<const __half*>(enc_mask),
+                   reinterpret_cast<__half*>(dec_output), cache_vec);
+  });
+}
+
+int ls_layer_param_count(const char* layer_name, int layer_id, long long* count) {
+  return guarded([&] {
+    const std::string name = layer_name ? layer_name : "";
+    if (!count) throw std::runtime_error("layer_param_count: null result pointer");
+    if (name == "TransformerEncoderLayer")
+      *count = (long long)find_layer(s_transformer_encoder_layers, layer_id, "Encoder layer")
+                   ->param_count();
+    else if (name == "TransformerDecoderLayer")
+      *count = (long long)find_layer(s_transformer_decoder_layers, layer_id, "Decoder layer")
+                   ->param_count();
+    else
+      throw std::runtime_error("layer_param_count: unknown layer name");
+  });
+}
+
 int ls_assign_layer_weight_grad_fp16(const void* weights, void* grads, const char* layer_name,
                                      int layer_id) {
   (void)grads;
   return guarded([&] {
-    if (!layer_name || std::string(layer_name) != "TransformerEncoderLayer")
+    const std::string name = layer_name ? layer_name : "";
+    if (name == "TransformerEncoderLayer")
+      find_layer(s_transformer_encoder_layers, layer_id, "Encoder layer")
+          ->assign_weight_ptr(reinterpret_cast<const __half*>(weights));
+    else if (name == "TransformerDecoderLayer")
+      find_layer(s_transformer_decoder_layers, layer_id, "Decoder layer")
+          ->assign_weight_ptr(reinterpret_cast<const __half*>(weights));
+    else
       throw std::runtime_error("assign_layer_weight_grad: unknown layer name");
-    find_layer(s_transformer_encoder_layers, layer_id, "Encoder layer")
-        ->assign_weight_ptr(reinterpret_cast<const __half*>(weights));
   });
 }
 
@@ -111,6 +173,8 @@ int ls_destroy_layer(const char* layer_name, int layer_id) {
     const std::string name = layer_name ? layer_name : "";
     if (name == "TransformerEncoderLayer")
       s_transformer_encoder_layers.erase(layer_id);
+    else if (name == "TransformerDecoderLayer")
+      s_transformer_decoder_layers.erase(layer_id);
     else if (name == "QuantLinearLayer")
       s_quant_linear_layers.erase(layer_id);
     else

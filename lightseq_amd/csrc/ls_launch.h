@@ -305,6 +305,15 @@ template <typename T>
 int opb_quant_bias_add_transform_20314(T* out, uint8_t* cmask, const int8_t* in, const T* bias,
                                        const T* cmax, int d0, int d1, int d2, int d3, int d4,
                                        hipStream_t s, const T* out_cmax);
+// launch_bias_add_transform_20314 (transform_kernels.cu:140-235): T [d0,d1,d2,d3,d4] + bias
+// [d2,d3,d4] -> [d2,d0,d3,d1,d4]
+template <typename T>
+int opb_bias_add_transform_20314(T* out, const T* in, const T* bias, int d0, int d1, int d2,
+                                 int d3, int d4, hipStream_t s);
+// launch_concat3_dim1 (general_kernels.cu:187-234): [sz0,sz1_1,sz2] ++ [sz0,sz1_2,sz2] on dim 1
+template <typename T>
+int opb_concat3_dim1(const T* inp1, const T* inp2, T* out, int sz0, int sz2, int sz1_1,
+                     int sz1_2, hipStream_t s);
 // out_q != nullptr selects the quantising variant
 template <typename T>
 int opb_transform4d_0213(T* out, int8_t* out_q, uint8_t* cmask, const T* vals, const T* cmax,
@@ -334,6 +343,11 @@ int gemm_i8_i8o_dev_alpha(const int8_t* A, const int8_t* W, int8_t* C, int M, in
 int layer_attention_f16(const __half* q, const __half* k, const __half* v, const __half* add_mask,
                         __half* ctx, int batch, int seq_len, int head_num, int dim_per_head,
                         bool mask_future, hipStream_t s);
+// The same with its own number of keys (cross attention, cached decoding step).
+int layer_cross_attention_f16(const __half* q, const __half* k, const __half* v,
+                              const __half* add_mask, __half* ctx, int batch, int seq_len,
+                              int key_len, int head_num, int dim_per_head, bool mask_future,
+                              hipStream_t s);
 
 // inference/kernels/transformerKernels.h:137-140
 inline float length_norm(int length, float alpha) {

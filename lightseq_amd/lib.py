@@ -102,6 +102,8 @@ _SIGNATURES = {
     "lsh_launch_layer_norm_i8": (True, "pppppppp" + "ii" + "s"),
     "lsh_launch_attn_softmax": (True, "pp" + "iiiii" + "s"),
     "lsh_launch_quant_bias_add_transform_20314": (True, "ppppp" + "iiiii" + "s" + "p" + "i"),
+    "lsh_launch_bias_add_transform_20314": (True, "ppp" + "iiiii" + "s"),
+    "lsh_launch_concat3_dim1": (True, "ppp" + "iiii" + "s"),
     "lsh_launch_transform4d_0213": (True, "pp" + "iiiii" + "s"),
     "lsh_launch_quant_transform4d_0213": (True, "pppp" + "iiiii" + "s"),
     "lsh_launch_ls_dropout": (True, "ppp" + "if" + "s" + "i"),
@@ -115,10 +117,14 @@ _SIGNATURES = {
     "lsh_launch_ls_quant_dropout_res_bias": (True, "pppppp" + "iif" + "s" + "i"),
     "lsh_feed_forward_i8": (False, "iii" + "ppppp" + "s"),
     "lsh_layer_attention_f16": (False, "ppppp" + "iiiii" + "s"),
+    "lsh_layer_cross_attention_f16": (False, "ppppp" + "iiiiii" + "s"),
     # layer interface
     "ls_layer_set_stream": (False, "s"),
     "ls_create_transformer_encoder_layer_fp16": (False, "iiiiii" + "fff" + "i" + "c" + "i"),
     "ls_transformer_encoder_layer_fw_fp16": (False, "i" + "ppp" + "iiiii"),
+    "ls_create_transformer_decoder_layer_fp16": (False, "iiiiii" + "fff" + "i" + "c"),
+    "ls_transformer_decoder_layer_fw_fp16": (False, "i" + "pppp" + "iiii" + "p" + "iii"),
+    "ls_layer_param_count": (False, "c" + "i" + "p"),
     "ls_assign_layer_weight_grad_fp16": (False, "pp" + "c" + "i"),
     "ls_create_quant_linear_layer_fp16": (False, "iiii"),
     "ls_quant_linear_layer_fw_fp16": (False, "i" + "pppp" + "iii"),

@@ -65,6 +65,20 @@ def launch_quant_bias_add_transform_20314(output, clip_mask, inp, bias, clip_max
          current_stream(), ptr(out_clip_max), int(in_col32))
 
 
+def launch_bias_add_transform_20314(output, inp, bias, dim_0, dim_1, dim_2, dim_3, dim_4):
+    """kernels.h:72-75: [d0, d1, d2, d3, d4] + bias [d2, d3, d4] -> [d2, d0, d3, d1, d4]."""
+    _dev(output, inp, bias)
+    call("lsh_launch_bias_add_transform_20314" + _suffix(output), ptr(output), ptr(inp),
+         ptr(bias), dim_0, dim_1, dim_2, dim_3, dim_4, current_stream())
+
+
+def launch_concat3_dim1(inp1, inp2, output, sz0, sz2, sz1_1, sz1_2):
+    """kernels.h:183-185: [sz0, sz1_1, sz2] ++ [sz0, sz1_2, sz2] along dimension 1."""
+    _dev(inp1, inp2, output)
+    call("lsh_launch_concat3_dim1" + _suffix(output), ptr(inp1), ptr(inp2), ptr(output), sz0,
+         sz2, sz1_1, sz1_2, current_stream())
+
+
 def launch_transform4d_0213(output, vals, batch_size, seq_len, hidden_dim, nhead, trans_count):
     _dev(output, vals)
     call("lsh_launch_transform4d_0213" + _suffix(vals), ptr(output), ptr(vals), batch_size,
@@ -135,3 +149,11 @@ def layer_attention(q, k, v, attn_mask, ctx, batch_size, seq_len, heads, dim_per
     _dev(q, k, v, attn_mask, ctx)
     call("lsh_layer_attention_f16", ptr(q), ptr(k), ptr(v), ptr(attn_mask), ptr(ctx), batch_size,
          seq_len, heads, dim_per_head, int(mask_future), current_stream())
+
+
+def layer_cross_attention(q, k, v, attn_mask, ctx, batch_size, from_len, to_len, heads,
+                          dim_per_head, mask_future=False):
+    """Attention core with its own number of keys (cross attention, cached decoding step)."""
+    _dev(q, k, v, attn_mask, ctx)
+    call("lsh_layer_cross_attention_f16", ptr(q), ptr(k), ptr(v), ptr(attn_mask), ptr(ctx),
+         batch_size, from_len, to_len, heads, dim_per_head, int(mask_future), current_stream())

@@ -1,6 +1,7 @@
 """CPU restatement (numpy) of the reference's csrc operator/layer forward path in quantised
 mode: the ``launch_*`` kernels of ``lightseq/csrc/kernels/cuda`` and the forward of
-``TransformerEncoderLayer<T>`` / ``QuantLinearLayer<T>`` built from them.
+``TransformerEncoderLayer<T>`` / ``TransformerDecoderLayer<T>`` / ``QuantLinearLayer<T>``
+built from them.
 
 TEST INFRASTRUCTURE ONLY: imported by ``tests/`` -- never by the shipped package.
 
@@ -173,6 +174,24 @@ def launch_quant_bias_add_transform_20314(inp, bias, clip_max, dim0, dim1, dim2,
     return np.ascontiguousarray(v.astype(dt).transpose(2, 0, 3, 1, 4))
 
 
+def launch_bias_add_transform_20314(inp, bias, dim0, dim1, dim2, dim3, dim4):
+    """transform_kernels.cu:140-235: T [d0,d1,d2,d3,d4] + bias [d2,d3,d4] -> [d2,d0,d3,d1,d4];
+    the sum is formed in T (half2 add for T=half)."""
+    dt = np.asarray(inp).dtype
+    x = np.asarray(inp).reshape(dim0, dim1, dim2, dim3, dim4)
+    b = np.broadcast_to(np.asarray(bias, dt).reshape(1, 1, dim2, dim3, dim4), x.shape)
+    v = _hadd(x, b) if dt == np.float16 else _f(x) + _f(b)
+    return np.ascontiguousarray(v.astype(dt).transpose(2, 0, 3, 1, 4))
+
+
+def launch_concat3_dim1(inp1, inp2, sz0, sz2, sz1_1, sz1_2):
+    """general_kernels.cu:187-234: [sz0, sz1_1, sz2] ++ [sz0, sz1_2, sz2] along dimension 1."""
+    b = np.asarray(inp2).reshape(sz0, sz1_2, sz2)
+    if sz1_1 == 0:
+        return b.copy()
+    return np.concatenate([np.asarray(inp1).reshape(sz0, sz1_1, sz2), b], axis=1)
+
+
 def launch_transform4d_0213(vals, batch, seq_len, hidden, nhead, trans_count):
     """transform_kernels.cu:444-560: [tc, b, nh, s, ad] -> [b, s, tc, nh, ad]."""
     v = np.asarray(vals).reshape(trans_count, batch, nhead, seq_len, hidden // nhead)
@@ -342,6 +361,146 @@ def encoder_layer_forward(para, x, mask, nhead, inter, pre_ln, act, mask_future=
     if not pre_ln:
         out = launch_layer_norm(out, p["ffn_nw"], p["ffn_nb"])[0]
     return out.reshape(bsz, seq, hs)
+
+
+def split_decoder_params(para, hidden, inter, layer_id, nlayer):
+    """transformer_decoder_layer.h:100-168 assign_weight_ptr: views into the flat blob."""
+    hs, ims = hidden, inter
+    sizes = [("attn_qkvw", hs * hs * 3), ("attn_qkvb", hs * 3), ("attn_ow", hs * hs),
+             ("attn_ob", hs), ("attn_nw", hs), ("attn_nb", hs),
+             ("encdec_attn_qw", hs * hs), ("encdec_attn_qb", hs), ("encdec_attn_ow", hs * hs),
+             ("encdec_attn_ob", hs), ("encdec_attn_nw", hs), ("encdec_attn_nb", hs),
+             ("inter_w", hs * ims), ("inter_b", ims), ("output_w", hs * ims), ("output_b", hs),
+             ("ffn_nw", hs), ("ffn_nb", hs), ("clip_max", 24)]
+    if layer_id == 0:
+        sizes += [("encdec_attn_kvw", nlayer * 2 * hs * hs), ("encdec_attn_kvb", nlayer * 2 * hs)]
+    out, off = {}, 0
+    for name, n in sizes:
+        out[name] = para[off:off + n]
+        off += n
+    assert off == para.size, (off, para.size)
+    for name, rows in (("attn_qkvw", 3 * hs), ("attn_ow", hs), ("encdec_attn_qw", hs),
+                       ("encdec_attn_ow", hs), ("inter_w", ims), ("output_w", hs)):
+        out[name] = out[name].reshape(rows, -1)
+    if layer_id == 0:
+        out["encdec_attn_kvw"] = out["encdec_attn_kvw"].reshape(nlayer * 2 * hs, hs)
+    return out
+
+
+def _attention(q, k, v, bsz, nhead, mask, mask_future):
+    """StridedBatchGemm (scores, scaled in T) + launch_attn_softmax + StridedBatchGemm
+    (context) + launch_transform4d_0213, as the layers chain them
+    (transformer_decoder_layer.cpp:182-205).  q T [bsz * nhead, from, hd]; k, v [.., to, hd]."""
+    dt = q.dtype
+    bh, fl, hd = q.shape
+    tl = k.shape[1]
+    alpha_s = F32(dt.type(1.0) / dt.type(np.sqrt(F32(hd))))
+    sc = (alpha_s * np.einsum("bid,bjd->bij", q.astype(np.float64), k.astype(np.float64))
+          .astype(F32)).astype(dt)
+    pr = launch_attn_softmax(sc.reshape(bsz, nhead, fl, tl), mask, mask_future)
+    ctx = np.einsum("bij,bjd->bid", pr.reshape(bh, fl, tl).astype(np.float64),
+                    v.astype(np.float64)).astype(F32).astype(dt)
+    return launch_transform4d_0213(ctx, bsz, fl, nhead * hd, nhead, 1).reshape(bsz * fl, nhead * hd)
+
+
+def _quant_linear_i8(x, w, cmax3):
+    """launch_quantize of the input (start bit 2) and the weight (start bit 4), int8 GEMM to
+    int8 with alpha = cmax_in * cmax_w / (cmax_out * 127)."""
+    qin, _, alpha = launch_quantize(x, cmax3, 2, True)
+    qw, _ = launch_quantize(w, cmax3[1:], 4)
+    return igemm_i8(qin, qw, alpha)
+
+
+def decoder_encdec_kv(para0, enc_out, nhead, inter, nlayer):
+    """transformer_decoder_layer.cpp:236-262 encdec_kv_fw of layer 0 in quantised mode: the
+    cross-attention k and v of every decoder layer, T [nlayer * 2, B, nhead, S_src, hd].  Only
+    the weight is fake-quantised (clip value encdec_kv_cmax[1]); the product is in T."""
+    bsz, src, hs = enc_out.shape
+    p = split_decoder_params(np.asarray(para0), hs, inter, 0, nlayer)
+    kv_c = _f(p["clip_max"])[18:23]
+    fake_w, _ = launch_fake_quantize(p["encdec_attn_kvw"], kv_c[1:], 4)
+    kv = gemm_T(np.asarray(enc_out).reshape(bsz * src, hs), fake_w)
+    return launch_bias_add_transform_20314(kv, p["encdec_attn_kvb"], bsz, src, nlayer * 2, nhead,
+                                           hs // nhead)
+
+
+def decoder_layer_forward(para, layer_id, nlayer, x, encdec_kv, enc_mask, nhead, inter, pre_ln,
+                          act, cache=None, beam=1, taps=None):
+    """layers/transformer_decoder_layer.cpp:91-547 in quantised mode, dropout off.
+
+    cache None: x T [B, trg_len, H], self attention over the whole target sequence with future
+    positions masked.  cache a dict: one decoding step, x T [B * beam, 1, H];
+    ``cache["k"]`` / ``cache["v"]`` hold T [B * beam * nhead, step, hd] (absent at step 0) and
+    are replaced by the arrays one position longer (:173-180).  encdec_kv: the array of
+    :func:`decoder_encdec_kv`; enc_mask T [B, S_src] additive.  Returns T like x."""
+    x = np.asarray(x)
+    dt = x.dtype
+    hs = x.shape[-1]
+    hd = hs // nhead
+    p = split_decoder_params(np.asarray(para), hs, inter, layer_id, nlayer)
+    cm = _f(p["clip_max"])
+    qkv_c, out_c, eq_c, eo_c, inter_c, ffn2_c, cache_c = (cm[0:3], cm[3:6], cm[6:9], cm[9:12],
+                                                         cm[12:15], cm[15:18], cm[23])
+    taps = {} if taps is None else taps
+    predict = cache is not None
+    if predict:
+        assert x.shape[1] == 1 and x.shape[0] % beam == 0
+        batch, trg_len = x.shape[0] // beam, beam  # :67-70: trg_seq_len is the beam size
+        sa_batch, from_len = x.shape[0], 1
+    else:
+        batch, trg_len = x.shape[0], x.shape[1]
+        sa_batch, from_len = batch, trg_len
+    tok = batch * trg_len
+    inp = x.reshape(tok, hs)
+    ln = lambda v, w, b: launch_layer_norm(v, p[w], p[b])[0]
+
+    # ---- self attention (:91-233)
+    ln_in = ln(inp, "attn_nw", "attn_nb") if pre_ln else inp
+    qout = _quant_linear_i8(ln_in, p["attn_qkvw"], qkv_c)
+    qkv = launch_quant_bias_add_transform_20314(qout, p["attn_qkvb"], qkv_c[2], sa_batch,
+                                                from_len, 3, nhead, hd, cache_c)
+    q, k, v = (qkv[i].reshape(sa_batch * nhead, from_len, hd) for i in range(3))
+    if predict:
+        step = 0 if cache.get("k") is None else cache["k"].shape[1]
+        k = launch_concat3_dim1(cache.get("k"), k, sa_batch * nhead, hd, step, 1)
+        v = launch_concat3_dim1(cache.get("v"), v, sa_batch * nhead, hd, step, 1)
+        cache["k"], cache["v"] = k, v
+    ctx = _attention(q, k, v, sa_batch, nhead, None, not predict)
+    taps["attn_ctx"] = ctx
+    qout = _quant_linear_i8(ctx, p["attn_ow"], out_c)
+    h1 = launch_ls_quant_dropout_res_bias(qout, out_c[2], p["attn_ob"], inp)
+    if not pre_ln:
+        h1 = ln(h1, "attn_nw", "attn_nb")
+    taps["attn_out"] = h1
+
+    # ---- cross attention (:278-412): batch sequences of trg_len queries each
+    ln_in = ln(h1, "encdec_attn_nw", "encdec_attn_nb") if pre_ln else h1
+    qout = _quant_linear_i8(ln_in, p["encdec_attn_qw"], eq_c)
+    eq = launch_quant_bias_add_transform_20314(qout, p["encdec_attn_qb"], eq_c[2], batch, trg_len,
+                                               1, nhead, hd, None)
+    src = encdec_kv.shape[3]
+    ek = np.asarray(encdec_kv)[2 * layer_id].reshape(batch * nhead, src, hd)
+    ev = np.asarray(encdec_kv)[2 * layer_id + 1].reshape(batch * nhead, src, hd)
+    ctx = _attention(eq[0].reshape(batch * nhead, trg_len, hd), ek, ev, batch, nhead, enc_mask,
+                     False)
+    taps["encdec_ctx"] = ctx
+    qout = _quant_linear_i8(ctx, p["encdec_attn_ow"], eo_c)
+    h2 = launch_ls_quant_dropout_res_bias(qout, eo_c[2], p["encdec_attn_ob"], h1)
+    if not pre_ln:
+        h2 = ln(h2, "encdec_attn_nw", "encdec_attn_nb")
+    taps["encdec_out"] = h2
+
+    # ---- feed-forward (:415-483)
+    ff1_inp = ln(h2, "ffn_nw", "ffn_nb") if pre_ln else h2
+    relu_inp = _quant_linear_i8(ff1_inp, p["inter_w"], inter_c)
+    ff2_inp, _ = launch_ls_fakequant_dropout_act_bias(
+        relu_inp, p["inter_b"], inter_c[2], ffn2_c[0], act, symmetry=(act != "relu"))
+    fake_w, _ = launch_fake_quantize(p["output_w"], ffn2_c[1:], 4)
+    out = gemm_T(ff2_inp, fake_w)
+    out = launch_ls_dropout_res_bias(out, p["output_b"], h2)
+    if not pre_ln:
+        out = ln(out, "ffn_nw", "ffn_nb")
+    return out.reshape(x.shape)
 
 
 def quant_linear_forward(x, weight, clip_max3):
