@@ -15,16 +15,16 @@
 //    The weight matrix is read once, by ceil(N/32) * ksplit workgroups; with ksplit > 1
 //    range p stores its int32 partial sums to plane p of the output ([ksplit][M][N]).
 //  * gemm_i8_stream_kernel -- the fast path (K % 128 == 0).  Persistent: 2 workgroups
-//    per compute unit walk a list of 128x128 tiles; operand stages (128 rows x 128 B
-//    each for A and W) are brought from L2 straight into LDS with
-//    global_load_lds_dwordx4 (no VGPR staging) into a 2-stage ring, and the prefetch
-//    cursor runs ahead of the compute cursor across tile boundaries, so a tile's first
-//    loads are in flight while the previous tile is still in its K loop / epilogue.
+//    per compute unit walk a list of 128x64 tiles; operand stages (128 rows of A and 64 of
+//    W, 128 B each) are brought from L2 straight into LDS with global_load_lds_dwordx4
+//    (no VGPR staging) into a 3-stage ring, and the prefetch cursor runs two K steps ahead
+//    of the compute cursor across tile boundaries, so a tile's first loads are in flight
+//    while the previous tile is still in its K loop / epilogue.
 //  * gemm_i8_generic_kernel -- any K % 16 == 0, any alignment of M and N: register
 //    staged, zero-filled tails, one tile per workgroup.
 //
-// Common geometry.  256 threads = 4 wavefronts (2x2), 64x64 accumulators per wavefront
-// as 2x2 MFMA blocks.  LDS rows are 128 B = eight 16-byte chunks, XOR swizzled for the
+// Common geometry.  256 threads = 4 wavefronts (2x2); per wavefront 64x64 accumulators as
+// 2x2 MFMA blocks (64x32 as 2x1 in the fast path).  LDS rows are 128 B = eight 16-byte chunks, XOR swizzled for the
 // 64-bank LDS (a ds_read_b128 is served 16 lanes per clock; the 16 lanes must hit 16
 // distinct 16-byte slots of a 256-byte window).  The W tile is the MFMA "A" operand so
 // that consecutive accumulator registers of a lane run along N, and the W rows fed to
@@ -36,6 +36,7 @@
 #include <hip/hip_ext.h>
 
 #include <string>
+#include <type_traits>
 
 namespace lsh {
 
@@ -349,13 +350,182 @@ __device__ __forceinline__ void tile_of(int t, int nblk, int tiles_m, int tiles_
 }
 
 // ---------------------------------------------------------------------------------
-// Fast path: persistent, direct-to-LDS, 2-stage ring, cross-tile prefetch.
+// Fast path: persistent, direct-to-LDS, 3-stage ring, cross-tile prefetch, 128x64 tiles.
 // Preconditions (checked by the dispatcher): K % 128 == 0, (rows-1)*K + 128 < 2^32 for
 // both operands, operands 16-byte aligned.
+//
+// One K step = 128 bytes of K = four 32-byte slices of 2 (rows) x 1 (columns) MFMA blocks per
+// wavefront.  The operand fragments of slice s + 1 are read from LDS into a second set of
+// registers while the MFMAs of slice s run, and the loop turns right after the step's
+// barrier: the last slice of a step is multiplied after the first fragments of the next
+// step have been requested, so neither the LDS latency nor the meeting of the wavefronts
+// leaves the matrix unit idle.  The barrier of step i proves that the loads of step i + 1
+// have landed and that every wavefront has read all of step i; the loads of step i + 3 then
+// go into the stage of step i.  72 KB of LDS: two workgroups per compute unit.
 // ---------------------------------------------------------------------------------
+constexpr int kSBN = 64;  // tile width of the fast path
+constexpr int kStreamStages = 3;
+constexpr size_t kStreamLds = (size_t)kStreamStages * (kBM + kSBN) * kBK;
+
 template <typename Epi, bool FULL>
 __global__ void __launch_bounds__(256)
 gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
+                      int N, int K, int tiles_m, int tiles_n, bool vec_store, int ksplit) {
+  constexpr int NST = kStreamStages;
+  constexpr int STAGE = (kBM + kSBN) * kBK;      // 24 KB: A tile then W tile
+  constexpr int NA = kBM / 32, NW = kSBN / 32;   // 1-KB DMA instructions per wavefront per stage
+  constexpr int PER = NA + NW;
+  extern __shared__ __align__(16) int8_t smem[];
+  // work item = (K range, tile): with ksplit > 1 every tile is computed ksplit times over
+  // disjoint K ranges and range p stores to rows [p * M, (p + 1) * M) of the output
+  const int ntile = tiles_m * tiles_n;
+  const int nblk = ntile * ksplit;
+  const int G = gridDim.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, g = lane >> 5;
+  const int my_tiles = (nblk - (int)blockIdx.x + G - 1) / G;
+  const int kpart = K / ksplit;  // bytes of K per range (a multiple of kBK)
+  const int nk = kpart / kBK;
+  const int total_it = my_tiles * nk;
+
+  // DMA sources: each instruction moves 8 rows x 128 B; lane i lands in LDS slot i of that
+  // 1-KB block, so it fetches the chunk the swizzle puts there.  Row clamping keeps the
+  // reads of partial tiles in bounds (the clamped rows are never stored).
+  uint32_t a_src[NA], w_src[NW];
+  auto set_src = [&](int j) {
+    const int item = blockIdx.x + j * G;
+    const int part = ksplit == 1 ? 0 : div24(item, ntile);
+    const uint32_t koff = (uint32_t)part * (uint32_t)kpart;
+    int tm, tn;
+    tile_of(item - part * ntile, ntile, tiles_m, tiles_n, tm, tn);
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int row = (wave + 4 * i) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ key_act(row);
+      a_src[i] = (uint32_t)min(tm * kBM + row, M - 1) * (uint32_t)K + koff + c * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int row = (wave + 4 * i) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ key_wgt(row);
+      w_src[i] = (uint32_t)min(tn * kSBN + row, N - 1) * (uint32_t)K + koff + c * 16;
+    }
+  };
+  const uint32_t lds0 =
+      (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+  // Issued through inline asm so that the compiler's wait-count insertion does not see an
+  // outstanding LDS write and drain vmcnt before every ds_read; the waits are explicit.
+  auto dma1 = [&](const int8_t* base, uint32_t voff, uint32_t lds) {
+    lds = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff),
+                 "s"(base)
+                 : "memory");
+  };
+  int p_j = 0, p_kt = 0, p_st = 0;  // prefetch cursor: work item, K step, ring slot
+  auto issue_next = [&]() {
+    if (p_j < my_tiles) {
+      const uint32_t base = lds0 + p_st * STAGE;
+#pragma unroll
+      for (int i = 0; i < NA; ++i) dma1(A + p_kt * kBK, a_src[i], base + (wave + 4 * i) * 1024);
+#pragma unroll
+      for (int i = 0; i < NW; ++i)
+        dma1(W + p_kt * kBK, w_src[i], base + kBM * kBK + (wave + 4 * i) * 1024);
+      if (++p_kt == nk) {
+        p_kt = 0;
+        if (++p_j < my_tiles) set_src(p_j);
+      }
+      if (++p_st == NST) p_st = 0;
+    }
+  };
+  // at most `groups` (0 or 1) of the youngest load groups may still be in flight.  Stores of
+  // an epilogue count as well and only make the wait stricter; loads complete in order.
+  auto wait_groups = [&](int groups) {
+    if (groups >= 1)
+      __builtin_amdgcn_s_waitcnt(PER | (7 << 4) | (15 << 8));  // vmcnt(PER)
+    else
+      __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0)
+  };
+
+  int a_off[2], a_key[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = wm * 64 + i * 32 + l32;
+    a_off[i] = row * kBK;
+    a_key[i] = key_act(row);
+  }
+  const int w_row = wn * 32 + sigma(l32);
+  const int w_off = kBM * kBK + w_row * kBK, w_key = key_wgt(w_row);
+  struct Frag {
+    v4i a[2], w;
+  };
+  auto load_frag = [&](Frag& f, const int8_t* stage, int ks) {
+    const int chunk = 2 * ks + g;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      f.a[i] = *reinterpret_cast<const v4i*>(stage + a_off[i] + ((chunk ^ a_key[i]) << 4));
+    f.w = *reinterpret_cast<const v4i*>(stage + w_off + ((chunk ^ w_key) << 4));
+  };
+  v16i acc[2][1];
+  auto mma = [&](const Frag& f) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w, f.a[i], acc[i][0], 0, 0, 0);
+  };
+
+  if (my_tiles > 0) set_src(0);
+  issue_next();
+  issue_next();
+  wait_groups(min(1, total_it - 1));
+  __builtin_amdgcn_s_barrier();
+  Frag f0, f1;
+  int st = 0, kt = 0, j = 0, tm = 0, tn = 0, part = 0;
+  for (int it = 0;; ++it) {
+    const int8_t* stage = smem + st * STAGE;
+    if (it < total_it) {
+      issue_next();  // step it + 2 into the stage step it - 1 has finished with
+      load_frag(f0, stage, 0);
+    }
+    if (it > 0) mma(f1);  // last slice of step it - 1
+    if (kt == 0) {
+      if (it > 0)
+        store_tile_acc<Epi, 2, 1, FULL>(epi, acc, tm * kBM, tn * kSBN, wm, wn, l32, g, M, N,
+                                        vec_store, (long)part * M);
+      if (it == total_it) break;
+      const int item = blockIdx.x + j * G;
+      part = ksplit == 1 ? 0 : div24(item, ntile);
+      tile_of(item - part * ntile, ntile, tiles_m, tiles_n, tm, tn);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) acc[i][0] = (v16i)0;
+    }
+    load_frag(f1, stage, 1);
+    mma(f0);
+    load_frag(f0, stage, 2);
+    mma(f1);
+    load_frag(f1, stage, 3);
+    mma(f0);
+    // step it + 1 has landed for this wavefront, and its own reads of step it are done ...
+    wait_groups(min(1, total_it - 2 - it));
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    // ... and for everyone
+    __builtin_amdgcn_s_barrier();
+    if (++st == NST) st = 0;
+    if (++kt == nk) {
+      kt = 0;
+      ++j;
+    }
+  }
+  __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
+}
+
+// The earlier form of the fast path: 128x128 tiles (2x2 MFMA blocks per wavefront), 2-stage
+// ring, all fragments of a step read before its MFMAs.  Kept for the epilogues that load
+// (activation tables, bias): their loads are younger than the operand groups in flight, so
+// waiting for them drains the ring at every tile boundary, and this form has half as many
+// boundaries (same box, FFN1 of BERT-base with the tabulated GELU: 22.6 us here, 24.5 us with
+// the 128x64 kernel; the other three products of the layer are 1-2 us faster there).
+template <typename Epi, bool FULL>
+__global__ void __launch_bounds__(256)
+gemm_i8_stream128_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
                       int N, int K, int tiles_m, int tiles_n, bool vec_store, int ksplit) {
   constexpr int NST = 2;
   constexpr int STAGE = (kBM + kBN) * kBK;  // 32 KB: A tile then W tile
@@ -704,6 +874,14 @@ static int launch(Kern kern, int grid, size_t smem, const int8_t* A, const int8_
   return lsh_check_launch("gemm_i8_kernel");
 }
 
+// Epilogues that run the 128x128 form of the fast path
+template <typename Epi>
+struct wide_tiles : std::false_type {};
+template <>
+struct wide_tiles<EpiLutI8> : std::true_type {};
+template <int ACT>
+struct wide_tiles<EpiActI8<ACT>> : std::true_type {};
+
 template <typename Epi>
 static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int K,
                     hipStream_t s, int ksplit = 1) {
@@ -713,9 +891,13 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   if (((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(W)) & 15u) != 0)
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: operands must be 16-byte aligned");
   const bool vec_store = epi.vec_ok(N);
-  const int tiles_m = (M + kBM - 1) / kBM, tiles_n = (N + kBN - 1) / kBN;
+  // 128 x 64 tiles in the fast path, 128 x 128 in its wide form and in the generic kernel
+  const bool stream = stream_ok(M, N, K);
+  const bool narrow = stream && !wide_tiles<Epi>::value;
+  const int tiles_m = (M + kBM - 1) / kBM;
+  const int tiles_n = narrow ? (N + kSBN - 1) / kSBN : (N + kBN - 1) / kBN;
   const int tiles = tiles_m * tiles_n;
-  const size_t smem = 2 * (size_t)(kBM + kBN) * kBK;
+  const size_t smem = narrow ? kStreamLds : 2 * (size_t)(kBM + kBN) * kBK;
   static bool attr_stream = false, attr_stream_full = false, attr_generic = false;  // per Epi
   static bool attr_skinny = true;  // static LDS: nothing to set
   if (ksplit < 1 || (ksplit > 1 && K % (ksplit * kBK) != 0))
@@ -738,9 +920,16 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
     return launch(gemm_i8_skinny_kernel<Epi, 2, false>, grid, 0, A, W, epi, M, N, K, 0, 0,
                   vec_store, s, &attr_skinny, ksplit);
   }
-  if (stream_ok(M, N, K)) {
+  if (stream) {
     const int items = tiles * ksplit;
     const int grid = items < 512 ? items : 512;  // 2 resident workgroups per compute unit
+    if (!narrow) {
+      if (full)
+        return launch(gemm_i8_stream128_kernel<Epi, true>, grid, smem, A, W, epi, M, N, K,
+                      tiles_m, tiles_n, vec_store, s, &attr_stream_full, ksplit);
+      return launch(gemm_i8_stream128_kernel<Epi, false>, grid, smem, A, W, epi, M, N, K, tiles_m,
+                    tiles_n, vec_store, s, &attr_stream, ksplit);
+    }
     if (full)
       return launch(gemm_i8_stream_kernel<Epi, true>, grid, smem, A, W, epi, M, N, K, tiles_m,
                     tiles_n, vec_store, s, &attr_stream_full, ksplit);
@@ -754,8 +943,10 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
 
 std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
   if (M <= 64 && K % kBK == 0) return std::string("gemm_i8_skinny_kernel<") + epilogue + ">";
-  return std::string(stream_ok(M, N, K) ? "gemm_i8_stream_kernel<" : "gemm_i8_generic_kernel<") +
-         epilogue + ">";
+  if (!stream_ok(M, N, K)) return std::string("gemm_i8_generic_kernel<") + epilogue + ">";
+  const std::string e = epilogue ? epilogue : "";
+  const bool wide = e.rfind("EpiLutI8", 0) == 0 || e.rfind("EpiActI8", 0) == 0;
+  return std::string(wide ? "gemm_i8_stream128_kernel<" : "gemm_i8_stream_kernel<") + e + ">";
 }
 
 int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int K,
