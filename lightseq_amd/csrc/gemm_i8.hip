@@ -874,6 +874,18 @@ static int launch(Kern kern, int grid, size_t smem, const int8_t* A, const int8_
   return lsh_check_launch("gemm_i8_kernel");
 }
 
+// The 128x64 kernel wins where a tile's K loop is long against its boundary (epilogue, restart
+// of the fragment pipeline), where 128x128 tiles would leave compute units without one, and
+// where the half-size tiles fill the last round of the 512 resident workgroups better; with
+// short K loops and whole rounds of tiles the wide form has half as many boundaries to pay
+// (4096 x 4096 x 1024, int8 out: 26.3 us wide, 31.0 us narrow; 4096 x 768 x 3072: 21.8 and 20.0;
+// 4096 x 2304 x 768: 15.8 and 15.3).
+static bool narrow_pays(int M, int N, int K, int ksplit) {
+  const long wide_items = (long)((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) * ksplit;
+  const long rounds_wide = (wide_items + 511) / 512, half_rounds_narrow = (2 * wide_items + 511) / 512;
+  return K / ksplit / kBK >= 12 || wide_items < 256 || half_rounds_narrow < 2 * rounds_wide;
+}
+
 // Epilogues that run the 128x128 form of the fast path
 template <typename Epi>
 struct wide_tiles : std::false_type {};
@@ -893,7 +905,7 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   const bool vec_store = epi.vec_ok(N);
   // 128 x 64 tiles in the fast path, 128 x 128 in its wide form and in the generic kernel
   const bool stream = stream_ok(M, N, K);
-  const bool narrow = stream && !wide_tiles<Epi>::value;
+  const bool narrow = stream && !wide_tiles<Epi>::value && narrow_pays(M, N, K, ksplit);
   const int tiles_m = (M + kBM - 1) / kBM;
   const int tiles_n = narrow ? (N + kSBN - 1) / kSBN : (N + kBN - 1) / kBN;
   const int tiles = tiles_m * tiles_n;
@@ -945,7 +957,8 @@ std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
   if (M <= 64 && K % kBK == 0) return std::string("gemm_i8_skinny_kernel<") + epilogue + ">";
   if (!stream_ok(M, N, K)) return std::string("gemm_i8_generic_kernel<") + epilogue + ">";
   const std::string e = epilogue ? epilogue : "";
-  const bool wide = e.rfind("EpiLutI8", 0) == 0 || e.rfind("EpiActI8", 0) == 0;
+  const bool wide = e.rfind("EpiLutI8", 0) == 0 || e.rfind("EpiActI8", 0) == 0 ||
+                    !narrow_pays(M, N, K, 1);
   return std::string(wide ? "gemm_i8_stream128_kernel<" : "gemm_i8_stream_kernel<") + e + ">";
 }
 
