@@ -18,6 +18,8 @@ SMALL = [(1, 1, 16), (3, 5, 16), (32, 32, 32), (33, 31, 48), (64, 16, 128), (130
 LARGE = [(4096, 2304, 768), (4096, 768, 768), (4096, 3072, 768), (4096, 768, 3072),
          (512, 1536, 512), (512, 2048, 512), (4096, 4096, 1024), (4096, 1024, 4096),
          (1000, 30522 // 6, 128), (64, 1000, 1024),
+         # ragged rows and columns in the 128x64 kernel (column tails of 40 and of 8), a single K step
+         (200, 1000, 1536), (130, 72, 256), (256, 192, 128),
          # decode-step shapes (rows = batch x beam of one step)
          (16, 3072, 1024), (16, 1024, 4096), (16, 50257, 1024), (64, 32000, 1024),
          (64, 4096, 1024), (33, 1000, 256), (1, 64, 128), (48, 40, 384)]
