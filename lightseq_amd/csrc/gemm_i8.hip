@@ -886,13 +886,14 @@ static bool narrow_pays(int M, int N, int K, int ksplit) {
   return K / ksplit / kBK >= 12 || wide_items < 256 || half_rounds_narrow < 2 * rounds_wide;
 }
 
-// Epilogues that run the 128x128 form of the fast path
+// Epilogues that run the 128x128 form of the fast path: every one that reads memory (tables,
+// bias vectors, a scale kept in device memory)
 template <typename Epi>
-struct wide_tiles : std::false_type {};
+struct wide_tiles : std::true_type {};
 template <>
-struct wide_tiles<EpiLutI8> : std::true_type {};
-template <int ACT>
-struct wide_tiles<EpiActI8<ACT>> : std::true_type {};
+struct wide_tiles<EpiI32> : std::false_type {};
+template <>
+struct wide_tiles<EpiI8> : std::false_type {};
 
 template <typename Epi>
 static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int K,
@@ -957,8 +958,7 @@ std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
   if (M <= 64 && K % kBK == 0) return std::string("gemm_i8_skinny_kernel<") + epilogue + ">";
   if (!stream_ok(M, N, K)) return std::string("gemm_i8_generic_kernel<") + epilogue + ">";
   const std::string e = epilogue ? epilogue : "";
-  const bool wide = e.rfind("EpiLutI8", 0) == 0 || e.rfind("EpiActI8", 0) == 0 ||
-                    !narrow_pays(M, N, K, 1);
+  const bool wide = (e != "EpiI32" && e != "EpiI8") || !narrow_pays(M, N, K, 1);
   return std::string(wide ? "gemm_i8_stream128_kernel<" : "gemm_i8_stream_kernel<") + e + ">";
 }
 
