@@ -227,6 +227,19 @@ int lsh_launch_ls_quant_dropout_res_bias_f32(void* out, uint8_t* mask, const int
 int lsh_feed_forward_i8(int bsz, int output_size, int input_size, const int8_t* qinput_ptr,
                         const int8_t* qweight_ptr, const float* alpha_ptr, const float* beta_ptr,
                         int8_t* qout_ptr, lsh_stream_t stream);
+/* StridedBatchGemm<T>::Forward (ops/includes/strided_batch_gemm.h:45-57 over
+ * cublas_strided_batched_gemm, kernels/cuda/cublas_wrappers.cpp): per batch element, in
+ * column-major terms, output (m x n) = alpha * op(A) (m x k) * op(B) (k x n) + beta * output,
+ * with strides m*k, n*k, m*n; op_a / op_b: 0 = N, 1 = T (the values of cublasOperation_t).
+ * The layers configure it as (T, N; m = to_len, n = from_len, k = head_dim; alpha =
+ * 1/sqrt(head_dim)) for the scores and (N, N; m = head_dim, n = from_len, k = to_len) for the
+ * context (layers/transformer_encoder_layer.cpp:34-42, :121-141). */
+int lsh_strided_batch_gemm_f16(int bsz, int m, int n, int k, float alpha, float beta, int op_a,
+                               int op_b, const void* buffer_a, const void* buffer_b,
+                               void* output, lsh_stream_t stream);
+int lsh_strided_batch_gemm_f32(int bsz, int m, int n, int k, float alpha, float beta, int op_a,
+                               int op_b, const void* buffer_a, const void* buffer_b,
+                               void* output, lsh_stream_t stream);
 /* Attention core of the layer in one kernel, fp16: replaces StridedBatchGemm (scores) +
  * launch_attn_softmax + Dropout::dropout + StridedBatchGemm (context) +
  * launch_transform4d_0213 of layers/transformer_encoder_layer.cpp:121-148.  No single

@@ -194,6 +194,12 @@ int lsh_layer_attention_f16(const void* q, const void* k, const void* v, const v
                              mask_future != 0, HS(stream));
 }
 
+LSH_BOTH(lsh_strided_batch_gemm,
+         (int bsz, int m, int n, int k, float alpha, float beta, int op_a, int op_b,
+          const void* buffer_a, const void* buffer_b, void* output, lsh_stream_t stream),
+         return strided_batch_gemm<T>(bsz, m, n, k, alpha, beta, op_a, op_b, C<T>(buffer_a),
+                                      C<T>(buffer_b), M<T>(output), HS(stream));)
+
 int lsh_layer_cross_attention_f16(const void* q, const void* k, const void* v,
                                   const void* attn_mask, void* ctx, int batch_size, int from_len,
                                   int to_len, int heads, int dim_per_head, int mask_future,

@@ -59,4 +59,52 @@ int gemm_f16_nt(const __half* A, const __half* W, __half* C, int M, int N, int K
   return lsh_check_launch("gemm_f16_nt_kernel");
 }
 
+// StridedBatchGemm<T>::Forward (ops/includes/strided_batch_gemm.h:45-57,
+// cublas_strided_batched_gemm of kernels/cuda/cublas_wrappers.cpp): per batch, in cuBLAS's
+// column-major terms, C (m x n) = alpha * op(A) (m x k) * op(B) (k x n) + beta * C with
+// strides m*k, n*k, m*n.  Read as row-major arrays: out[n][m]; A is [m][k] when op_A = T and
+// [k][m] when N; B is [n][k] when op_B = N and [k][n] when T.  fp32 accumulation, one thread
+// per output element (m fastest): the layers of this library run the fused attention kernel,
+// this stand-alone form exists for callers of the operator and is written for clarity.
+template <typename T>
+__global__ void __launch_bounds__(256)
+strided_batch_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* C, int m, int n,
+                          int k, float alpha, float beta, int ta, int tb, long total) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int i = (int)(idx % m);
+  const long r = idx / m;
+  const int j = (int)(r % n);
+  const long b = r / n;
+  const T* a = A + b * (long)m * k;
+  const T* bb = B + b * (long)n * k;
+  const long a_step = ta ? 1 : m, a0 = ta ? (long)i * k : i;
+  const long b_step = tb ? n : 1, b0 = tb ? j : (long)j * k;
+  float acc = 0.f;
+  for (int kk = 0; kk < k; ++kk)
+    acc = fmaf((float)a[a0 + kk * a_step], (float)bb[b0 + kk * b_step], acc);
+  float v = alpha * acc;
+  if (beta != 0.f) v += beta * (float)C[idx];
+  C[idx] = (T)v;
+}
+
+template <typename T>
+int strided_batch_gemm(int bsz, int m, int n, int k, float alpha, float beta, int op_a, int op_b,
+                       const T* A, const T* B, T* C, hipStream_t s) {
+  if (!A || !B || !C || bsz <= 0 || m <= 0 || n <= 0 || k <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "StridedBatchGemm: bad arguments");
+  if ((op_a != 0 && op_a != 1) || (op_b != 0 && op_b != 1))
+    return lsh_fail(LSH_ERR_INVALID, "StridedBatchGemm: op must be 0 (N) or 1 (T)");
+  const long total = (long)bsz * m * n;
+  if ((total + 255) / 256 > 0x7fffffffL)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "StridedBatchGemm: too many output elements");
+  strided_batch_gemm_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, s>>>(
+      A, B, C, m, n, k, alpha, beta, op_a, op_b, total);
+  return lsh_check_launch("strided_batch_gemm_kernel");
+}
+template int strided_batch_gemm<__half>(int, int, int, int, float, float, int, int, const __half*,
+                                        const __half*, __half*, hipStream_t);
+template int strided_batch_gemm<float>(int, int, int, int, float, float, int, int, const float*,
+                                       const float*, float*, hipStream_t);
+
 }  // namespace lsh

@@ -171,6 +171,10 @@ void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop);
 
 // ---- fp16 MFMA GEMM (gemm_f16.hip) ------------------------------------------------------
 int gemm_f16_nt(const __half* A, const __half* W, __half* C, int M, int N, int K, hipStream_t s);
+// StridedBatchGemm<T>::Forward (ops/includes/strided_batch_gemm.h:45-57); op: 0 = N, 1 = T
+template <typename T>
+int strided_batch_gemm(int bsz, int m, int n, int k, float alpha, float beta, int op_a, int op_b,
+                       const T* A, const T* B, T* C, hipStream_t s);
 
 // ---- decoder step (dec_kernels.hip) -----------------------------------------------------
 template <typename T>

@@ -116,6 +116,7 @@ _SIGNATURES = {
     "lsh_launch_ls_fakequant_dropout_act_bias_relu": (True, "pppppppp" + "iif" + "s" + "ii"),
     "lsh_launch_ls_quant_dropout_res_bias": (True, "pppppp" + "iif" + "s" + "i"),
     "lsh_feed_forward_i8": (False, "iii" + "ppppp" + "s"),
+    "lsh_strided_batch_gemm": (True, "iiii" + "ff" + "ii" + "ppp" + "s"),
     "lsh_layer_attention_f16": (False, "ppppp" + "iiiii" + "s"),
     "lsh_layer_cross_attention_f16": (False, "ppppp" + "iiiiii" + "s"),
     # layer interface

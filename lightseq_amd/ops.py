@@ -144,6 +144,14 @@ def feed_forward_i8(bsz, output_size, input_size, qinput, qweight, alpha, beta, 
          ptr(alpha), ptr(beta), ptr(qout), current_stream())
 
 
+def strided_batch_gemm(bsz, m, n, k, alpha, beta, op_a, op_b, buffer_a, buffer_b, output):
+    """``StridedBatchGemm<T>::Forward`` (ops/includes/strided_batch_gemm.h:45-57); op 0 = N,
+    1 = T; column-major cuBLAS semantics with strides m*k, n*k, m*n."""
+    _dev(buffer_a, buffer_b, output)
+    call("lsh_strided_batch_gemm" + _suffix(output), bsz, m, n, k, float(alpha), float(beta),
+         int(op_a), int(op_b), ptr(buffer_a), ptr(buffer_b), ptr(output), current_stream())
+
+
 def layer_attention(q, k, v, attn_mask, ctx, batch_size, seq_len, heads, dim_per_head,
                     mask_future=False):
     _dev(q, k, v, attn_mask, ctx)

@@ -286,6 +286,22 @@ def gemm_T(x, w):
     return (np.asarray(x).astype(np.float64) @ np.asarray(w).astype(np.float64).T).astype(F32).astype(dt)
 
 
+def strided_batch_gemm(a, b, m, n, k, alpha, beta=0.0, op_a=0, op_b=0, c=None):
+    """ops/includes/strided_batch_gemm.h:45-57 (cublasGemmStridedBatchedEx, float32
+    accumulation): per batch element, column-major, C (m x n) = alpha op(A) op(B) + beta C.
+    As row-major arrays: A [bsz, m, k] if op_a = T else [bsz, k, m]; B [bsz, n, k] if op_b = N
+    else [bsz, k, n]; result [bsz, n, m] of the operands' type."""
+    dt = np.asarray(a).dtype
+    a64 = np.asarray(a).astype(np.float64)
+    b64 = np.asarray(b).astype(np.float64)
+    am = a64.reshape(-1, m, k) if op_a else a64.reshape(-1, k, m).transpose(0, 2, 1)  # [bsz, m, k]
+    bm = b64.reshape(-1, k, n).transpose(0, 2, 1) if op_b else b64.reshape(-1, n, k)  # [bsz, n, k]
+    out = F32(alpha) * np.einsum("bjk,bik->bji", bm, am).astype(F32)
+    if beta != 0.0:
+        out = out + F32(beta) * _f(c).reshape(out.shape)
+    return out.astype(dt)
+
+
 def split_params(para, hidden, inter):
     """transformer_encoder_layer.h:66-105 assign_weight_ptr: views into the flat blob."""
     hs, ims = hidden, inter
