@@ -380,9 +380,19 @@ ln_row_wg_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
       float a[4];
       if constexpr (sizeof(AccT) == 4) {
         int4 acc = *reinterpret_cast<const int4*>(gemm_out + base + e);
-        for (int p = 1; p < nparts; ++p) {
-          const int4 m = *reinterpret_cast<const int4*>(gemm_out + p * part_stride + base + e);
-          acc.x += m.x; acc.y += m.y; acc.z += m.z; acc.w += m.w;
+        // four planes per round trip (integer sums: any order gives the same bits); a plane
+        // index beyond the last is clamped for the load and its value dropped
+        for (int p = 1; p < nparts; p += 4) {
+          int4 m[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            m[u] = *reinterpret_cast<const int4*>(
+                gemm_out + (long)min(p + u, nparts - 1) * part_stride + base + e);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (p + u < nparts) {
+              acc.x += m[u].x; acc.y += m[u].y; acc.z += m[u].z; acc.w += m[u].w;
+            }
         }
         a[0] = (float)acc.x; a[1] = (float)acc.y; a[2] = (float)acc.z; a[3] = (float)acc.w;
       } else {
