@@ -361,17 +361,19 @@ __device__ __forceinline__ void tile_of(int t, int nblk, int tiles_m, int tiles_
 // step have been requested, so neither the LDS latency nor the meeting of the wavefronts
 // leaves the matrix unit idle.  The barrier of step i proves that the loads of step i + 1
 // have landed and that every wavefront has read all of step i; the loads of step i + 3 then
-// go into the stage of step i.  72 KB of LDS: two workgroups per compute unit.
+// go into the stage of step i.  72 KB of LDS: two workgroups per compute unit.  With short K
+// loops (TNST = 2: 48 KB, three workgroups per compute unit, loads one step ahead) a third
+// resident workgroup hides more than the deeper ring (4096 x 2304 x 768: 14.0 against 15.0 us;
+// 4096 x 768 x 3072 with int32 output: 21.5 against 20.5 us).
 // ---------------------------------------------------------------------------------
 constexpr int kSBN = 64;  // tile width of the fast path
-constexpr int kStreamStages = 3;
-constexpr size_t kStreamLds = (size_t)kStreamStages * (kBM + kSBN) * kBK;
+constexpr size_t kStreamStageBytes = (size_t)(kBM + kSBN) * kBK;
 
-template <typename Epi, bool FULL>
+template <typename Epi, bool FULL, int TNST>
 __global__ void __launch_bounds__(256)
 gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
                       int N, int K, int tiles_m, int tiles_n, bool vec_store, int ksplit) {
-  constexpr int NST = kStreamStages;
+  constexpr int NST = TNST;  // 3: loads two K steps ahead; 2: one step ahead, 48 KB
   constexpr int STAGE = (kBM + kSBN) * kBK;      // 24 KB: A tile then W tile
   constexpr int NA = kBM / 32, NW = kSBN / 32;   // 1-KB DMA instructions per wavefront per stage
   constexpr int PER = NA + NW;
@@ -473,9 +475,9 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   };
 
   if (my_tiles > 0) set_src(0);
-  issue_next();
-  issue_next();
-  wait_groups(min(1, total_it - 1));
+#pragma unroll
+  for (int i = 0; i < NST - 1; ++i) issue_next();
+  wait_groups(min(NST - 2, total_it - 1));
   __builtin_amdgcn_s_barrier();
   Frag f0, f1;
   int st = 0, kt = 0, j = 0, tm = 0, tn = 0, part = 0;
@@ -504,7 +506,7 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
     load_frag(f1, stage, 3);
     mma(f0);
     // step it + 1 has landed for this wavefront, and its own reads of step it are done ...
-    wait_groups(min(1, total_it - 2 - it));
+    wait_groups(min(NST - 2, total_it - 2 - it));
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
     // ... and for everyone
     __builtin_amdgcn_s_barrier();
@@ -910,8 +912,11 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   const int tiles_m = (M + kBM - 1) / kBM;
   const int tiles_n = narrow ? (N + kSBN - 1) / kSBN : (N + kBN - 1) / kBN;
   const int tiles = tiles_m * tiles_n;
-  const size_t smem = narrow ? kStreamLds : 2 * (size_t)(kBM + kBN) * kBK;
-  static bool attr_stream = false, attr_stream_full = false, attr_generic = false;  // per Epi
+  const bool deep = K / ksplit / kBK >= 12;  // long K loop: 3 stages, else 2 and a third workgroup
+  const size_t smem = narrow ? (deep ? 3 : 2) * kStreamStageBytes : 2 * (size_t)(kBM + kBN) * kBK;
+  // per Epi and kernel function: [0] column tail compiled in, [1] lean
+  static bool attr_wide[2] = {false, false}, attr_deep[2] = {false, false},
+              attr_shallow[2] = {false, false}, attr_generic = false;
   static bool attr_skinny = true;  // static LDS: nothing to set
   if (ksplit < 1 || (ksplit > 1 && K % (ksplit * kBK) != 0))
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: K does not split into whole 128-byte steps");
@@ -935,19 +940,28 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   }
   if (stream) {
     const int items = tiles * ksplit;
-    const int grid = items < 512 ? items : 512;  // 2 resident workgroups per compute unit
+    // resident workgroups per compute unit: 2 (64 or 72 KB of LDS each) or 3 (48 KB)
+    const int cap = narrow && !deep ? 768 : 512;
+    const int grid = items < cap ? items : cap;
     if (!narrow) {
       if (full)
         return launch(gemm_i8_stream128_kernel<Epi, true>, grid, smem, A, W, epi, M, N, K,
-                      tiles_m, tiles_n, vec_store, s, &attr_stream_full, ksplit);
+                      tiles_m, tiles_n, vec_store, s, &attr_wide[1], ksplit);
       return launch(gemm_i8_stream128_kernel<Epi, false>, grid, smem, A, W, epi, M, N, K, tiles_m,
-                    tiles_n, vec_store, s, &attr_stream, ksplit);
+                    tiles_n, vec_store, s, &attr_wide[0], ksplit);
+    }
+    if (deep) {
+      if (full)
+        return launch(gemm_i8_stream_kernel<Epi, true, 3>, grid, smem, A, W, epi, M, N, K, tiles_m,
+                      tiles_n, vec_store, s, &attr_deep[1], ksplit);
+      return launch(gemm_i8_stream_kernel<Epi, false, 3>, grid, smem, A, W, epi, M, N, K, tiles_m,
+                    tiles_n, vec_store, s, &attr_deep[0], ksplit);
     }
     if (full)
-      return launch(gemm_i8_stream_kernel<Epi, true>, grid, smem, A, W, epi, M, N, K, tiles_m,
-                    tiles_n, vec_store, s, &attr_stream_full, ksplit);
-    return launch(gemm_i8_stream_kernel<Epi, false>, grid, smem, A, W, epi, M, N, K, tiles_m,
-                  tiles_n, vec_store, s, &attr_stream, ksplit);
+      return launch(gemm_i8_stream_kernel<Epi, true, 2>, grid, smem, A, W, epi, M, N, K, tiles_m,
+                    tiles_n, vec_store, s, &attr_shallow[1], ksplit);
+    return launch(gemm_i8_stream_kernel<Epi, false, 2>, grid, smem, A, W, epi, M, N, K, tiles_m,
+                  tiles_n, vec_store, s, &attr_shallow[0], ksplit);
   }
   if (ksplit != 1) return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: this shape cannot split K");
   return launch(gemm_i8_generic_kernel<Epi>, tiles, smem, A, W, epi, M, N, K, tiles_m, tiles_n,
