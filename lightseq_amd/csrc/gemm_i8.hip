@@ -253,6 +253,15 @@ struct EpiLutI8 {
     }
     store16_i8(C + m * N + n, n, N, q, full);
   }
+  // the same with the table rows of the tile's columns staged in LDS (`tab`: 256 bytes per
+  // column, first row = the tile's first column; n_local = n - first column)
+  __device__ __forceinline__ void store16_lds(long m, int n, int N, const v16i& c, bool full,
+                                              const int8_t* tab, int n_local) const {
+    int q[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) q[i] = tab[(n_local + i) * 256 + requant_acc(c[i], alpha) + 128];
+    store16_i8(C + m * N + n, n, N, q, full);
+  }
   bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
   static const char* name() { return "EpiLutI8"; }
 };
@@ -369,7 +378,7 @@ __device__ __forceinline__ void tile_of(int t, int nblk, int tiles_m, int tiles_
 constexpr int kSBN = 64;  // tile width of the fast path
 constexpr size_t kStreamStageBytes = (size_t)(kBM + kSBN) * kBK;
 
-template <typename Epi, bool FULL, int TNST>
+template <typename Epi, bool FULL, int TNST, bool LDSTAB = false>
 __global__ void __launch_bounds__(256)
 gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
                       int N, int K, int tiles_m, int tiles_n, bool vec_store, int ksplit) {
@@ -439,6 +448,28 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
       if (++p_st == NST) p_st = 0;
     }
   };
+  // LDSTAB (the tabulated epilogue, TNST = 2): the 64 table rows of a tile's columns (16 KB)
+  // are brought into LDS behind the ring while the tile's K loop runs -- four 1-KB loads per
+  // wavefront, issued once every wavefront has finished the previous tile's epilogue -- and
+  // the epilogue looks its bytes up there instead of in global memory.
+  constexpr int NTAB = kSBN * 256 / 1024 / 4;  // table loads per wavefront and tile
+  int8_t* const tab_lds = smem + NST * STAGE;
+  auto issue_table = [&](int j) {
+    if constexpr (LDSTAB) {
+      const int item = blockIdx.x + j * G;
+      const int part = ksplit == 1 ? 0 : div24(item, ntile);
+      int tm, tn;
+      tile_of(item - part * ntile, ntile, tiles_m, tiles_n, tm, tn);
+      const long first = (long)tn * kSBN * 256, last = (long)N * 256 - 16;  // bytes of the table
+#pragma unroll
+      for (int i = 0; i < NTAB; ++i) {
+        const int q = wave + 4 * i;
+        const long off = min(first + q * 1024 + lane * 16, last);  // rows beyond N: never stored
+        dma1(reinterpret_cast<const int8_t*>(epi.lut), (uint32_t)off,
+             lds0 + NST * STAGE + q * 1024);
+      }
+    }
+  };
   // at most `groups` (0 or 1) of the youngest load groups may still be in flight.  Stores of
   // an epilogue count as well and only make the wait stricter; loads complete in order.
   auto wait_groups = [&](int groups) {
@@ -475,6 +506,7 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   };
 
   if (my_tiles > 0) set_src(0);
+  if (my_tiles > 0) issue_table(0);
 #pragma unroll
   for (int i = 0; i < NST - 1; ++i) issue_next();
   wait_groups(min(NST - 2, total_it - 1));
@@ -489,9 +521,25 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
     }
     if (it > 0) mma(f1);  // last slice of step it - 1
     if (kt == 0) {
-      if (it > 0)
-        store_tile_acc<Epi, 2, 1, FULL>(epi, acc, tm * kBM, tn * kSBN, wm, wn, l32, g, M, N,
-                                        vec_store, (long)part * M);
+      if (it > 0) {
+        if constexpr (LDSTAB) {
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const long m = tm * kBM + wm * 64 + i * 32 + l32;
+            const int n = tn * kSBN + wn * 32 + 16 * g;
+            if (m < M && n < N)
+              epi.store16_lds(m + (long)part * M, n, N, acc[i][0],
+                              FULL ? true : (vec_store && n + 16 <= N), tab_lds, wn * 32 + 16 * g);
+          }
+          // every wavefront is done with this table before the next one is loaded over it
+          __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+          __builtin_amdgcn_s_barrier();
+          if (it < total_it) issue_table(j);
+        } else {
+          store_tile_acc<Epi, 2, 1, FULL>(epi, acc, tm * kBM, tn * kSBN, wm, wn, l32, g, M, N,
+                                          vec_store, (long)part * M);
+        }
+      }
       if (it == total_it) break;
       const int item = blockIdx.x + j * G;
       part = ksplit == 1 ? 0 : div24(item, ntile);
@@ -506,7 +554,12 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
     load_frag(f1, stage, 3);
     mma(f0);
     // step it + 1 has landed for this wavefront, and its own reads of step it are done ...
-    wait_groups(min(NST - 2, total_it - 2 - it));
+    if (LDSTAB && kt == 0 && it > 0 && nk >= 2)
+      // the table loads of this tile were issued after the next step's group: they may stay in
+      // flight (loads complete in order), the second step's wait then covers them
+      __builtin_amdgcn_s_waitcnt(NTAB | (7 << 4) | (15 << 8));  // vmcnt(NTAB)
+    else
+      wait_groups(min(NST - 2, total_it - 2 - it));
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
     // ... and for everyone
     __builtin_amdgcn_s_barrier();
@@ -938,6 +991,22 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
     return launch(gemm_i8_skinny_kernel<Epi, 2, false>, grid, 0, A, W, epi, M, N, K, 0, 0,
                   vec_store, s, &attr_skinny, ksplit);
   }
+  if constexpr (std::is_same<Epi, EpiLutI8>::value) {
+    // the tabulated epilogue: 128 x 64 tiles, 2 stages + 16 KB of table rows in LDS
+    if (stream && ksplit == 1 && K / kBK >= 2) {
+      const int tn64 = (N + kSBN - 1) / kSBN;
+      if ((long)tiles_m * tn64 >= (1L << 24))
+        return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: more than 2^24 output tiles");
+      const int items = tiles_m * tn64;
+      const size_t lds = 2 * kStreamStageBytes + (size_t)kSBN * 256;
+      static bool attr_tab[2] = {false, false};
+      if (full)
+        return launch(gemm_i8_stream_kernel<Epi, true, 2, true>, items < 512 ? items : 512, lds, A,
+                      W, epi, M, N, K, tiles_m, tn64, vec_store, s, &attr_tab[1], 1);
+      return launch(gemm_i8_stream_kernel<Epi, false, 2, true>, items < 512 ? items : 512, lds, A,
+                    W, epi, M, N, K, tiles_m, tn64, vec_store, s, &attr_tab[0], 1);
+    }
+  }
   if (stream) {
     const int items = tiles * ksplit;
     // resident workgroups per compute unit: 2 (64 or 72 KB of LDS each) or 3 (48 KB)
@@ -972,6 +1041,7 @@ std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
   if (M <= 64 && K % kBK == 0) return std::string("gemm_i8_skinny_kernel<") + epilogue + ">";
   if (!stream_ok(M, N, K)) return std::string("gemm_i8_generic_kernel<") + epilogue + ">";
   const std::string e = epilogue ? epilogue : "";
+  if (e == "EpiLutI8" && K / kBK >= 2) return "gemm_i8_stream_kernel<EpiLutI8>";
   const bool wide = (e != "EpiI32" && e != "EpiI8") || !narrow_pays(M, N, K, 1);
   return std::string(wide ? "gemm_i8_stream128_kernel<" : "gemm_i8_stream_kernel<") + e + ">";
 }
