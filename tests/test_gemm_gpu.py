@@ -106,7 +106,9 @@ def test_gemm_rejects_bad_k():
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 3072, 768), (4096, 3072, 768), (77, 160, 48),
-                                   (16, 4096, 1024), (64, 4096, 1024)])
+                                   (16, 4096, 1024), (64, 4096, 1024),
+                                   # ragged columns with the table rows in LDS (last tile: 40 and 16 columns)
+                                   (200, 1000, 256), (130, 208, 384)])
 @pytest.mark.parametrize("act", ["gelu", "relu", "relu_narrow"])
 def test_fused_bias_act_epilogue_equals_unfused_pair(rng, M, N, K, act):
     """GEMM + bias/activation/requant in one kernel == int8-output GEMM followed by the
