@@ -6,7 +6,7 @@
 // Replaces the cuBLASLt int8 GEMMs and their tuned-algorithm table
 // (inference/model/cublas_helper.cc:31-225,361-489, cublas_algo_map.cc).
 //
-// Three kernels share the epilogues (the first two also the tile geometry):
+// Four kernels share the epilogues:
 //
 //  * gemm_i8_skinny_kernel -- M <= 64 (decode steps), K % 128 == 0.  A workgroup owns 32
 //    output columns for all rows; its 4 wavefronts split the 128-byte K chunks of the
@@ -19,7 +19,11 @@
 //    W, 128 B each) are brought from L2 straight into LDS with global_load_lds_dwordx4
 //    (no VGPR staging) into a 3-stage ring, and the prefetch cursor runs two K steps ahead
 //    of the compute cursor across tile boundaries, so a tile's first loads are in flight
-//    while the previous tile is still in its K loop / epilogue.
+//    while the previous tile is still in its K loop / epilogue.  K loops of fewer than 12
+//    steps use a 2-stage ring and 3 workgroups per compute unit; the tabulated epilogue
+//    keeps the table rows of its tile in LDS behind a 2-stage ring.
+//  * gemm_i8_stream128_kernel -- the same path with 128x128 tiles and a 2-stage ring, for
+//    the epilogues that read global memory and for short K loops over many tiles.
 //  * gemm_i8_generic_kernel -- any K % 16 == 0, any alignment of M and N: register
 //    staged, zero-filled tails, one tile per workgroup.
 //
