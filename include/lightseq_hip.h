@@ -529,6 +529,21 @@ int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, c
                                    int8_t* v_new, int64_t layer_offset, int beam_size,
                                    int dim_per_head, int head_num, int cur_step, int max_step);
 
+/* lsh_beam_search_step_i8I_f16 for callers that cannot allocate device memory (code
+ * under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  The proposal workspace (top_score / top_idx) is a
+ * static device array inside the library, 512 KiB per GPU, so the step is limited to
+ * batch_size * beam_size * beam_size <= 65536 (LSH_ERR_UNSUPPORTED beyond); the call
+ * allocates and frees nothing.  All calls on one GPU share that GPU's array: calls
+ * that overlap in time on one GPU race.  Results are identical to
+ * lsh_beam_search_step_i8I_f16. */
+int lsh_beam_search_step_noalloc_i8I_f16(const int8_t* logits, const void* logit_bias,
+                                         float* seq_probs, float* seq_score,
+                                         const int* old_alive_seq, int* new_alive_seq, int* parent,
+                                         int* num_finished, float dequant_scale, int vocab_size,
+                                         int max_step, float length_norm, int cur_step,
+                                         int batch_size, int beam_size, int end_id,
+                                         lsh_stream_t stream);
 /* ======================================================================== */
 /* GPT path                                                                   */
 /* ======================================================================== */

@@ -15,6 +15,8 @@
 #include "ls_device.cuh"
 #include "ls_launch.h"
 
+#include <mutex>
+
 namespace lsh {
 
 constexpr float kMinLogProb = -2000.f;      // inference/kernels/transformerKernels.h:12
@@ -785,5 +787,61 @@ template int beam_search_step_i8I<float>(const int8_t*, const float*, float*, fl
 template int beam_search_step_i8I<__half>(const int8_t*, const __half*, float*, float*, const int*,
                                           int*, float*, int*, int*, int*, float, int, int, float,
                                           int, int, int, int, hipStream_t);
+
+// ---------------------------------------------------------------------------------
+// The search step for callers that cannot allocate device memory (code under HIP graph
+// capture, serving loops, harnesses that forbid hipMalloc).  The proposals of the per-row
+// top-k -- the workspace that beam_search_step_i8I takes as top_score / top_idx -- live in
+// a file-scope device array instead.  Every GPU holds its own copy of the array at its own
+// address: the address is asked for once per device, with that device current, and host
+// code only ever uses the pointer it got back, never the array's name.  All calls on one
+// GPU share that GPU's array, so calls that overlap in time on one GPU race; nothing in
+// it has to start at zero (the top-k kernels write every slot the merge reads).
+// ---------------------------------------------------------------------------------
+constexpr int kStaticBeamEntries = 65536;  // batch_size * beam_size * beam_size, at most
+constexpr int kStaticBeamDevices = 64;
+static __device__ __align__(256) unsigned char scratch[(size_t)kStaticBeamEntries * 8];
+static std::mutex g_scratch_mutex;
+static unsigned char* g_scratch_ptr[kStaticBeamDevices] = {};
+
+static int scratch_of_current_device(unsigned char** out) {
+  int dev = -1;
+  if (int rc = lsh_check_hip(hipGetDevice(&dev), "hipGetDevice(beam_search_step_noalloc)")) return rc;
+  if (dev < 0 || dev >= kStaticBeamDevices)
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "beam_search_step_noalloc: device index out of range");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (int rc = lsh_check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)),
+                               "hipGetSymbolAddress(beam_search_step_noalloc)"))
+      return rc;
+    if (!p) return lsh_fail(LSH_ERR_HIP, "beam_search_step_noalloc: null scratch address");
+    g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return LSH_OK;
+}
+
+int beam_search_step_noalloc_i8I_f16(const int8_t* logits, const __half* logit_bias,
+                                     float* seq_probs, float* seq_score, const int* old_alive_seq,
+                                     int* new_alive_seq, int* parent, int* num_finished,
+                                     float dequant_scale, int vocab_size, int max_step,
+                                     float length_norm, int cur_step, int batch_size, int beam_size,
+                                     int end_id, hipStream_t s) {
+  if (batch_size <= 0 || beam_size < 1 || beam_size > 32)
+    return lsh_fail(LSH_ERR_INVALID, "beam_search_step_noalloc: bad batch_size or beam_size");
+  if ((long)batch_size * beam_size * beam_size > kStaticBeamEntries)
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "beam_search_step_noalloc: batch_size * beam_size^2 exceeds the 65536 proposals "
+                    "of the static workspace; use lsh_beam_search_step_i8I with a caller workspace");
+  unsigned char* ws = nullptr;
+  if (int rc = scratch_of_current_device(&ws)) return rc;
+  float* top_score = reinterpret_cast<float*>(ws);
+  int* top_idx = reinterpret_cast<int*>(ws + (size_t)kStaticBeamEntries * 4);
+  return beam_search_step_i8I<__half>(logits, logit_bias, seq_probs, seq_score, old_alive_seq,
+                                      new_alive_seq, top_score, top_idx, parent, num_finished,
+                                      dequant_scale, vocab_size, max_step, length_norm, cur_step,
+                                      batch_size, beam_size, end_id, s);
+}
 
 }  // namespace lsh

@@ -604,6 +604,19 @@ LSH_BEAM_STEP(lsh_beam_search_step_i8I_f32, float, F)
 #undef LSH_BEAM_STEP
 
 int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, const int* parent,
+int lsh_beam_search_step_noalloc_i8I_f16(const int8_t* logits, const void* logit_bias,
+                                         float* seq_probs, float* seq_score,
+                                         const int* old_alive_seq, int* new_alive_seq, int* parent,
+                                         int* num_finished, float dequant_scale, int vocab_size,
+                                         int max_step, float length_norm_v, int cur_step,
+                                         int batch_size, int beam_size, int end_id,
+                                         lsh_stream_t stream) {
+  return beam_search_step_noalloc_i8I_f16(logits, H(logit_bias), seq_probs, seq_score,
+                                          old_alive_seq, new_alive_seq, parent, num_finished,
+                                          dequant_scale, vocab_size, max_step, length_norm_v,
+                                          cur_step, batch_size, beam_size, end_id, HS(stream));
+}
+
                                    const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
                                    int8_t* v_new, int64_t layer_offset, int beam_size,
                                    int dim_per_head, int head_num, int cur_step, int max_step) {

@@ -253,6 +253,13 @@ int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_p
 // ---- GPT path (gpt_kernels.hip, attn_kernels.hip) ------------------------------------------
 // vocab_size <= 0 disables the token-id clamp, max_step <= 0 the position check
 template <typename T>
+// the same step with its proposal workspace in a static device array (allocates nothing)
+int beam_search_step_noalloc_i8I_f16(const int8_t* logits, const __half* logit_bias,
+                                     float* seq_probs, float* seq_score, const int* old_alive_seq,
+                                     int* new_alive_seq, int* parent, int* num_finished,
+                                     float dequant_scale, int vocab_size, int max_step,
+                                     float length_norm, int cur_step, int batch_size, int beam_size,
+                                     int end_id, hipStream_t s);
 int gpt_embedding_i8I(int batch_size, int batch_seq_len, int hidden_size, hipStream_t s,
                       const int8_t* token_emb, const T* pos_emb, const int* token_id, T* output,
                       int* real_seq_len, int padding_id, int pos_offset, float dequant_scale,

@@ -413,6 +413,20 @@ def beam_search_step_i8I(logits, logit_bias, seq_probs, seq_score, old_alive_seq
          length_norm_value, cur_step, batch_size, beam_size, end_id, current_stream())
 
 
+def beam_search_step_noalloc_i8I(logits, logit_bias, seq_probs, seq_score, old_alive_seq,
+                                 new_alive_seq, parent, num_finished, dequant_scale, vocab_size,
+                                 max_step, length_norm_value, cur_step, batch_size, beam_size,
+                                 end_id):
+    """``beam_search_step_i8I`` (fp16 bias) with the proposal workspace inside the library:
+    allocates nothing; batch_size * beam_size**2 <= 65536."""
+    _dev(logits, logit_bias, seq_probs, seq_score, old_alive_seq, new_alive_seq, parent,
+         num_finished)
+    call("lsh_beam_search_step_noalloc_i8I_f16", ptr(logits), ptr(logit_bias), ptr(seq_probs),
+         ptr(seq_score), ptr(old_alive_seq), ptr(new_alive_seq), ptr(parent), ptr(num_finished),
+         dequant_scale, vocab_size, max_step, length_norm_value, cur_step, batch_size, beam_size,
+         end_id, current_stream())
+
+
 def refresh_cache_by_parent_i8(n_layer, rows, parent, k_old, v_old, k_new, v_new, layer_offset,
                                beam_size, dim_per_head, head_num, cur_step, max_step):
     _dev(parent, k_old, v_old, k_new, v_new)

@@ -83,6 +83,7 @@ _SIGNATURES = {
     "lsh_ker_write_topk_result": (False, "ppp" + "iiiiii" + "s"),
     "lsh_beam_search_step_i8I": (True, "pppppppppp" + "f" + "ii" + "f" + "iiii" + "s"),
     "lsh_refresh_cache_by_parent_i8": (False, "iis" + "ppppp" + "l" + "iiiii"),
+    "lsh_beam_search_step_noalloc_i8I_f16": (False, "pppppppp" + "f" + "ii" + "f" + "iiii" + "s"),
     # GPT path
     "lsh_ker_gpt_embedding_i8I": (True, "iiis" + "ppppp" + "iif"),
     "lsh_gpt_scores_i8_i32o": (False, "ppp" + "iii" + "s"),
