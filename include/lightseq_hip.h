@@ -228,6 +228,13 @@ int lsh_gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int m, int n,
  * kernel, so keep one setting for all launches whose results are compared with each other.
  * Returns the previous setting (0 / 1).  No counterpart in the reference. */
 int lsh_layer_norm_row_kernel(int on);
+/* Process-wide switch (default on; returns the previous setting, 0 / 1): products with
+ * thousands of rows and columns run one 256 x 192 / 256 x 256 / 256 x 128 output tile per
+ * workgroup on 8 wavefronts; off sends them to the persistent 128 x 64 / 128 x 128 kernels
+ * instead.  Results are identical either way (integer sums); the switch exists to measure
+ * one against the other.  No counterpart in the reference (its cuBLASLt algorithm table
+ * plays this part: model/cublas_algo_map.cc). */
+int lsh_gemm_i8_tile_kernel(int on);
 /* Decode-step QKV product with ker_arrange_decself_qkv_i8I_i8O
  * (kernels/transformerKernels_int8.cc.cu:1432-1513; call sites model/quant_decoder.cc.cu:660-674,
  * model/quant_gpt_encoder.cc.cu:640-653) as its epilogue: A [step_token_num, k] x W [3*hidden, k]
@@ -522,13 +529,6 @@ int lsh_beam_search_step_i8I_f32(const int8_t* logits, const void* logit_bias, f
                                  float dequant_scale, int vocab_size, int max_step,
                                  float length_norm, int cur_step, int batch_size, int beam_size,
                                  int end_id, lsh_stream_t stream);
-/* Cache reorder driven by the parent table of lsh_beam_search_step_i8I (same copy as
- * lsh_ker_refresh_cache_i8).  rows = batch * beam. */
-int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, const int* parent,
-                                   const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
-                                   int8_t* v_new, int64_t layer_offset, int beam_size,
-                                   int dim_per_head, int head_num, int cur_step, int max_step);
-
 /* lsh_beam_search_step_i8I_f16 for callers that cannot allocate device memory (code
  * under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  No
  * counterpart in the reference.  The proposal workspace (top_score / top_idx) is a
@@ -544,6 +544,13 @@ int lsh_beam_search_step_noalloc_i8I_f16(const int8_t* logits, const void* logit
                                          int max_step, float length_norm, int cur_step,
                                          int batch_size, int beam_size, int end_id,
                                          lsh_stream_t stream);
+/* Cache reorder driven by the parent table of lsh_beam_search_step_i8I (same copy as
+ * lsh_ker_refresh_cache_i8).  rows = batch * beam. */
+int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, const int* parent,
+                                   const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
+                                   int8_t* v_new, int64_t layer_offset, int beam_size,
+                                   int dim_per_head, int head_num, int cur_step, int max_step);
+
 /* ======================================================================== */
 /* GPT path                                                                   */
 /* ======================================================================== */

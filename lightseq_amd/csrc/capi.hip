@@ -106,6 +106,7 @@ int lsh_launch_dequantize_tensor_f32(const int32_t* input, void* output, int bat
 
 // ---- LayerNorm family --------------------------------------------------------------
 int lsh_layer_norm_row_kernel(int on) { return ln_set_few_rows(on != 0) ? 1 : 0; }
+int lsh_gemm_i8_tile_kernel(int on) { return gemm_i8_enable_tile_kernel(on != 0) ? 1 : 0; }
 int lsh_ker_norm_layer_resual_i8O_f16(int token_num, int hidden_size, lsh_stream_t stream,
                                       void* input, int8_t* output, const void* scale,
                                       const void* bias, const void* residual_bias,
@@ -603,7 +604,6 @@ LSH_BEAM_STEP(lsh_beam_search_step_i8I_f16, __half, H)
 LSH_BEAM_STEP(lsh_beam_search_step_i8I_f32, float, F)
 #undef LSH_BEAM_STEP
 
-int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, const int* parent,
 int lsh_beam_search_step_noalloc_i8I_f16(const int8_t* logits, const void* logit_bias,
                                          float* seq_probs, float* seq_score,
                                          const int* old_alive_seq, int* new_alive_seq, int* parent,
@@ -617,6 +617,7 @@ int lsh_beam_search_step_noalloc_i8I_f16(const int8_t* logits, const void* logit
                                           cur_step, batch_size, beam_size, end_id, HS(stream));
 }
 
+int lsh_refresh_cache_by_parent_i8(int n_layer, int rows, lsh_stream_t stream, const int* parent,
                                    const int8_t* k_old, const int8_t* v_old, int8_t* k_new,
                                    int8_t* v_new, int64_t layer_offset, int beam_size,
                                    int dim_per_head, int head_num, int cur_step, int max_step) {

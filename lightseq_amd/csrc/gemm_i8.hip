@@ -39,6 +39,7 @@
 
 #include <hip/hip_ext.h>
 
+#include <mutex>
 #include <string>
 #include <type_traits>
 
@@ -96,10 +97,23 @@ __device__ __forceinline__ void store16_i8(int8_t* p, int n, int N, const int (&
   }
 }
 
+__device__ __forceinline__ uint4 requant16_packed(const v16i& c, float alpha) {
+  uint4 o;
+  o.x = requant_acc_pack4(c[0], c[1], c[2], c[3], alpha);
+  o.y = requant_acc_pack4(c[4], c[5], c[6], c[7], alpha);
+  o.z = requant_acc_pack4(c[8], c[9], c[10], c[11], alpha);
+  o.w = requant_acc_pack4(c[12], c[13], c[14], c[15], alpha);
+  return o;
+}
+
 struct EpiI8 {
   int8_t* C;
   float alpha;
   __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
+    if (full) {
+      *reinterpret_cast<uint4*>(C + m * N + n) = requant16_packed(c, alpha);
+      return;
+    }
     int q[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) q[i] = requant_acc(c[i], alpha);
@@ -192,6 +206,10 @@ struct EpiI8Dev {
   const float* alpha;
   __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
     const float a = alpha[0];
+    if (full) {
+      *reinterpret_cast<uint4*>(C + m * N + n) = requant16_packed(c, a);
+      return;
+    }
     int q[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) q[i] = requant_acc(c[i], a);
@@ -263,12 +281,17 @@ struct EpiLutI8 {
                                               const int8_t* tab, int n_local) const {
     int q[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) q[i] = tab[(n_local + i) * 256 + requant_acc(c[i], alpha) + 128];
+    for (int i = 0; i < 16; ++i)
+      q[i] = tab[(n_local + i) * 256 + requant_acc_fast(c[i], alpha) + 128];
     store16_i8(C + m * N + n, n, N, q, full);
   }
   bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
   static const char* name() { return "EpiLutI8"; }
 };
+
+template <typename Epi>
+__device__ __forceinline__ const int8_t* epi_lut(const Epi&) { return nullptr; }
+__device__ __forceinline__ const int8_t* epi_lut(const EpiLutI8& e) { return e.lut; }
 
 template <int ACT>
 __global__ void __launch_bounds__(256)
@@ -713,6 +736,207 @@ gemm_i8_stream128_kernel(const int8_t* __restrict__ A, const int8_t* __restrict_
 }
 
 // ---------------------------------------------------------------------------------
+// Wide-tile path: one large output tile per workgroup, for products with enough of them to
+// give every compute unit one (M and N in the thousands).
+//
+// What the measurements on this part say: under int8 MFMA load the shader clock sits near
+// 1.6 GHz (of 2.4), a kernel's stores cost their bytes / ~4.7 TB/s after its last wavefront
+// has finished (the write-back of the XCD's L2 at the kernel boundary), a launch needs
+// ~1.3 us before its first operands have landed (the L2 starts cold), and one wavefront per
+// SIMD keeps the matrix unit ~2/3 busy where two keep it ~95 % busy.  So: 8 wavefronts (two
+// per SIMD) share one 256 x 192 / 256 x 256 / 256 x 128 tile -- operand bytes per MFMA fall
+// with the tile area per compute unit, which is what both the 64 B/clk global->LDS path and
+// the LDS port are short of -- with 64 x 96 / 128 x 64 / 64 x 64 wavefront tiles; K steps of
+// 128 bytes go through a ring of NST stages filled by global_load_lds_dwordx4; fragments are
+// double-buffered per 32-byte slice and the issue order inside a slice is pinned (one LDS
+// read after each of the first MFMAs).  The step's barrier sits before the last slice's
+// MFMAs; after it the freed stage is refilled with step kt + NST.
+// The tabulated epilogue brings its TN x 256-byte table into the stage that the
+// second-to-last step frees, while the last step is multiplied.
+// Preconditions (checked by the dispatcher): K % 128 == 0, K / 128 >= NST, N % 16 == 0 and the
+// epilogue's vector path legal, 32-bit operand offsets, operands 16-byte aligned.
+// ---------------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <typename Epi, int WGM, int WGN, int MB, int NB, int NST>
+__global__ void __launch_bounds__(64 * WGM * WGN)
+gemm_i8_tile_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
+                    int N, int K, int tiles_m, int tiles_n, bool, int) {
+  constexpr bool LUT = std::is_same<Epi, EpiLutI8>::value;
+  constexpr int NWV = WGM * WGN;
+  constexpr int TM = WGM * MB * 32, TN = WGN * NB * 32;
+  constexpr int STAGE = (TM + TN) * kBK;
+  constexpr int NA = TM / 8 / NWV, NW = TN / 8 / NWV, PER = NA + NW;  // 1-KB loads per wavefront
+  constexpr int NTAB = TN / 4 / NWV;  // table loads per wavefront
+  static_assert(TM % (8 * NWV) == 0 && TN % (8 * NWV) == 0, "stage rows split over the wavefronts");
+  static_assert((NST - 1) * PER < 64, "vmcnt range");
+  static_assert(!LUT || (TM >= TN && TN % (4 * NWV) == 0), "table fits a freed stage");
+  extern __shared__ __align__(16) int8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN, l32 = lane & 31, g = lane >> 5;
+  int tm, tn;
+  tile_of(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tm, tn);
+  const int nk = K / kBK;
+
+  uint32_t a_src[NA], w_src[NW];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int row = (wave + NWV * i) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ key_act(row);
+    a_src[i] = (uint32_t)min(tm * TM + row, M - 1) * (uint32_t)K + c * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    const int row = (wave + NWV * i) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ key_wgt(row);
+    w_src[i] = (uint32_t)min(tn * TN + row, N - 1) * (uint32_t)K + c * 16;
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+  auto dma1 = [&](const int8_t* base, uint32_t voff, uint32_t lds) {
+    lds = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff),
+                 "s"(base)
+                 : "memory");
+  };
+  auto issue = [&](int kt, int slot) {  // K step kt into ring slot `slot`
+    const uint32_t base = lds0 + slot * STAGE;
+#pragma unroll
+    for (int i = 0; i < NA; ++i) dma1(A + kt * kBK, a_src[i], base + (wave + NWV * i) * 1024);
+#pragma unroll
+    for (int i = 0; i < NW; ++i)
+      dma1(W + kt * kBK, w_src[i], base + TM * kBK + (wave + NWV * i) * 1024);
+  };
+  // LDS byte offset of this lane's fragment chunk for K slice 0; slice ks is at (offset ^ (ks << 5)):
+  // chunk index 2 * ks + g, swizzled by the row key, and 2 * ks only touches bits 1-2 of it
+  int a_base[MB], w_base[NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int row = wm * (MB * 32) + i * 32 + l32;
+    a_base[i] = row * kBK + ((g ^ key_act(row)) << 4);
+  }
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const int row = wn * (NB * 32) + j * 32 + sigma(l32);
+    w_base[j] = TM * kBK + row * kBK + ((g ^ key_wgt(row)) << 4);
+  }
+  struct Frag {
+    v4i a[MB], w[NB];
+  };
+  auto load_frag = [&](Frag& f, const int8_t* stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+      f.a[i] = *reinterpret_cast<const v4i*>(stage + (a_base[i] ^ (ks << 5)));
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      f.w[j] = *reinterpret_cast<const v4i*>(stage + (w_base[j] ^ (ks << 5)));
+  };
+  v16i acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) acc[i][j] = (v16i)0;
+  auto mma = [&](const Frag& f) {
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[j], f.a[i], acc[i][j], 0, 0, 0);
+  };
+  // issue order of one slice: an LDS read of the next slice after each of the first MFMAs
+  auto pattern = [&]() {
+#pragma unroll
+    for (int q = 0; q < MB + NB; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    if (MB * NB > MB + NB) __builtin_amdgcn_sched_group_barrier(0x008, MB * NB - (MB + NB), 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  Frag f[2];
+  auto slices = [&](const int8_t* stage) {  // slices 1..3 read, slices 0..2 multiplied
+#pragma unroll
+    for (int ks = 1; ks < 4; ++ks) {
+      load_frag(f[ks & 1], stage, ks);
+      mma(f[(ks - 1) & 1]);
+      pattern();
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < NST; ++s) issue(s, s);
+  wait_vmcnt<(NST - 1) * PER>();
+  __builtin_amdgcn_s_barrier();
+  load_frag(f[0], smem, 0);
+  int slot = 0;
+  // steady state: a step ends by refilling its own slot with step kt + NST
+  for (int kt = 0; kt < nk - NST; ++kt) {
+    slices(smem + slot * STAGE);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront has read all of the stage
+    wait_vmcnt<(NST - 2) * PER>();       // its own loads of step kt + 1 have landed ...
+    __builtin_amdgcn_s_barrier();        // ... and everyone's; everyone is done with step kt
+    issue(kt + NST, slot);
+    __builtin_amdgcn_sched_barrier(0);
+    if (++slot == NST) slot = 0;
+    load_frag(f[0], smem + slot * STAGE, 0);
+    mma(f[1]);
+    pattern();
+  }
+  // drain: NST - 1 steps without a refill, then the last step
+  int tab_slot = 0;
+#pragma unroll
+  for (int t = 0; t < NST - 1; ++t) {
+    slices(smem + slot * STAGE);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    if (NST - 2 - t == 0) wait_vmcnt<0>();
+    else if (NST - 2 - t == 1) wait_vmcnt<PER>();
+    else wait_vmcnt<2 * PER>();
+    __builtin_amdgcn_s_barrier();
+    if (LUT && t == NST - 2) {
+      // the slot of the second-to-last step is free: the tile's table rows go there
+      tab_slot = slot;
+      const long first = (long)tn * TN * 256, last = (long)N * 256 - 16;
+#pragma unroll
+      for (int i = 0; i < NTAB; ++i) {
+        const int q = wave + NWV * i;
+        const long off = min(first + q * 1024 + lane * 16, last);  // rows beyond N: never stored
+        dma1(reinterpret_cast<const int8_t*>(epi_lut(epi)), (uint32_t)off,
+             lds0 + slot * STAGE + q * 1024);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (++slot == NST) slot = 0;
+    load_frag(f[0], smem + slot * STAGE, 0);
+    mma(f[1]);
+    pattern();
+  }
+  slices(smem + slot * STAGE);
+  mma(f[1]);
+  if (LUT) {
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+  }
+  const int8_t* tab = smem + tab_slot * STAGE;
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const long m = (long)tm * TM + wm * (MB * 32) + i * 32 + l32;
+    if (m < M) {
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int nl = wn * (NB * 32) + j * 32 + 16 * g;
+        const int n = tn * TN + nl;
+        if (n < N) {
+          if constexpr (LUT) epi.store16_lds(m, n, N, acc[i][j], true, tab, nl);
+          else epi.store16(m, n, N, acc[i][j], true);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
 // Generic path: register-staged double buffering, zero-filled tails.
 // ---------------------------------------------------------------------------------
 template <int ROWS>
@@ -899,6 +1123,8 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
 // host side
 // ---------------------------------------------------------------------------------
 static thread_local hipEvent_t g_ev_start = nullptr, g_ev_stop = nullptr;
+// switch for A/B measurements of the one-tile-per-workgroup kernel against the persistent ones
+static bool g_tile_kernel_enabled = true;
 
 void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop) {
   g_ev_start = start;
@@ -911,24 +1137,41 @@ static bool stream_ok(int M, int N, int K) {
   return (unsigned long long)M * K < lim && (unsigned long long)N * K < lim;
 }
 
-template <typename Kern, typename Epi>
-static int launch(Kern kern, int grid, size_t smem, const int8_t* A, const int8_t* W, Epi epi,
-                  int M, int N, int K, int tiles_m, int tiles_n, bool vec_store, hipStream_t s,
-                  bool* attr_set, int ksplit = 1) {
-  if (!*attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return lsh_check_hip(e, "hipFuncSetAttribute(gemm_i8)");
-    *attr_set = true;
+// The dynamic-LDS limit of a kernel function is raised once per device, under a lock, the
+// first time that function is launched there (a function's LDS size is fixed by its template
+// parameters).
+template <auto Kern>
+static int raise_lds_limit(size_t smem) {
+  static std::mutex mu;
+  static unsigned long long done = 0;  // bit per device index
+  int dev = 0;
+  if (int rc = lsh_check_hip(hipGetDevice(&dev), "hipGetDevice(gemm_i8)")) return rc;
+  if (dev < 0 || dev >= 64) return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: device index out of range");
+  std::lock_guard<std::mutex> lock(mu);
+  if (!(done >> dev & 1ull)) {
+    if (smem > 0) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(Kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      if (e != hipSuccess) return lsh_check_hip(e, "hipFuncSetAttribute(gemm_i8)");
+    }
+    done |= 1ull << dev;
   }
+  return LSH_OK;
+}
+
+template <auto Kern, typename Epi>
+static int launch(int grid, int threads, size_t smem, const int8_t* A, const int8_t* W, Epi epi,
+                  int M, int N, int K, int tiles_m, int tiles_n, bool vec_store, hipStream_t s,
+                  int ksplit = 1) {
+  if (int rc = raise_lds_limit<Kern>(smem)) return rc;
   if (g_ev_start != nullptr) {
     // kernel-exact begin/end timestamps on the launch stream
     hipEvent_t e0 = g_ev_start, e1 = g_ev_stop;
     g_ev_start = g_ev_stop = nullptr;
-    hipExtLaunchKernelGGL(kern, dim3(grid), dim3(256), (unsigned)smem, s, e0, e1, 0, A, W, epi, M,
-                          N, K, tiles_m, tiles_n, vec_store, ksplit);
+    hipExtLaunchKernelGGL(Kern, dim3(grid), dim3(threads), (unsigned)smem, s, e0, e1, 0, A, W, epi,
+                          M, N, K, tiles_m, tiles_n, vec_store, ksplit);
   } else {
-    kern<<<grid, 256, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store, ksplit);
+    Kern<<<grid, threads, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store, ksplit);
   }
   return lsh_check_launch("gemm_i8_kernel");
 }
@@ -954,6 +1197,51 @@ struct wide_tiles<EpiI32> : std::false_type {};
 template <>
 struct wide_tiles<EpiI8> : std::false_type {};
 
+// Epilogues compiled for the one-tile-per-workgroup kernel (the products of a whole batch);
+// the two decode-step epilogues only ever see M <= 64.
+template <typename Epi>
+struct has_tile_kernel : std::true_type {};
+template <>
+struct has_tile_kernel<EpiDecQkvI8> : std::false_type {};
+template <>
+struct has_tile_kernel<EpiEncdecQF16> : std::false_type {};
+
+// Tile shapes of gemm_i8_tile_kernel, all with 8 wavefronts and a 2-stage ring (3 for 256 x 128).
+enum TileShape { kTileNone = 0, kTile256x256, kTile256x192, kTile256x128 };
+struct TileChoice {
+  TileShape shape;
+  int tm, tn;
+};
+// One workgroup per compute unit and round: the cost of a shape is its number of rounds times
+// the tile area, plus the operand bytes a tile streams per K byte (rows + columns), which is
+// what separates shapes of equal area.  Shapes that would leave more than a quarter of the
+// 256 compute units without a tile in the last round, or give fewer than 128 tiles, are left to
+// the persistent kernels.
+static TileChoice choose_tile(int M, int N, int K) {
+  TileChoice best{kTileNone, 0, 0};
+  if (K % kBK != 0 || K / kBK < 3 || M < 1024 || N < 1024) return best;
+  const struct {
+    TileShape shape;
+    int tm, tn;
+  } cand[] = {{kTile256x256, 256, 256}, {kTile256x192, 256, 192}, {kTile256x128, 256, 128}};
+  double best_cost = 0;
+  for (const auto& c : cand) {
+    const long tiles = (long)((M + c.tm - 1) / c.tm) * ((N + c.tn - 1) / c.tn);
+    if (tiles < 128) continue;
+    const long rounds = (tiles + 255) / 256;
+    const long last = tiles - (rounds - 1) * 256;
+    if (last < 144) continue;
+    // wasted columns / rows of partial tiles count through the padded area
+    const double area = (double)c.tm * c.tn;
+    const double cost = rounds * area * (1.0 + 48.0 * (c.tm + c.tn) / area);
+    if (best.shape == kTileNone || cost < best_cost) {
+      best = TileChoice{c.shape, c.tm, c.tn};
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
 template <typename Epi>
 static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int K,
                     hipStream_t s, int ksplit = 1) {
@@ -971,10 +1259,6 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   const int tiles = tiles_m * tiles_n;
   const bool deep = K / ksplit / kBK >= 12;  // long K loop: 3 stages, else 2 and a third workgroup
   const size_t smem = narrow ? (deep ? 3 : 2) * kStreamStageBytes : 2 * (size_t)(kBM + kBN) * kBK;
-  // per Epi and kernel function: [0] column tail compiled in, [1] lean
-  static bool attr_wide[2] = {false, false}, attr_deep[2] = {false, false},
-              attr_shallow[2] = {false, false}, attr_generic = false;
-  static bool attr_skinny = true;  // static LDS: nothing to set
   if (ksplit < 1 || (ksplit > 1 && K % (ksplit * kBK) != 0))
     return lsh_fail(LSH_ERR_INVALID, "int8 gemm: K does not split into whole 128-byte steps");
   if ((long)tiles_m * tiles_n * ksplit >= (1L << 24))
@@ -984,16 +1268,35 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
     const int grid = ((N + 31) / 32) * ksplit;
     if (M <= 32) {
       if (full)
-        return launch(gemm_i8_skinny_kernel<Epi, 1, true>, grid, 0, A, W, epi, M, N, K, 0, 0,
-                      vec_store, s, &attr_skinny, ksplit);
-      return launch(gemm_i8_skinny_kernel<Epi, 1, false>, grid, 0, A, W, epi, M, N, K, 0, 0,
-                    vec_store, s, &attr_skinny, ksplit);
+        return launch<gemm_i8_skinny_kernel<Epi, 1, true>>(grid, 256, 0, A, W, epi, M, N, K, 0, 0,
+                                                           vec_store, s, ksplit);
+      return launch<gemm_i8_skinny_kernel<Epi, 1, false>>(grid, 256, 0, A, W, epi, M, N, K, 0, 0,
+                                                          vec_store, s, ksplit);
     }
     if (full)
-      return launch(gemm_i8_skinny_kernel<Epi, 2, true>, grid, 0, A, W, epi, M, N, K, 0, 0,
-                    vec_store, s, &attr_skinny, ksplit);
-    return launch(gemm_i8_skinny_kernel<Epi, 2, false>, grid, 0, A, W, epi, M, N, K, 0, 0,
-                  vec_store, s, &attr_skinny, ksplit);
+      return launch<gemm_i8_skinny_kernel<Epi, 2, true>>(grid, 256, 0, A, W, epi, M, N, K, 0, 0,
+                                                         vec_store, s, ksplit);
+    return launch<gemm_i8_skinny_kernel<Epi, 2, false>>(grid, 256, 0, A, W, epi, M, N, K, 0, 0,
+                                                        vec_store, s, ksplit);
+  }
+  if constexpr (has_tile_kernel<Epi>::value) {
+    if (stream && full && ksplit == 1 && g_tile_kernel_enabled) {
+      const TileChoice c = choose_tile(M, N, K);
+      const int tm = c.tm ? (M + c.tm - 1) / c.tm : 0, tn = c.tn ? (N + c.tn - 1) / c.tn : 0;
+      switch (c.shape) {
+        case kTile256x256:
+          return launch<gemm_i8_tile_kernel<Epi, 2, 4, 4, 2, 2>>(tm * tn, 512, 2 * 512 * kBK, A, W,
+                                                                 epi, M, N, K, tm, tn, true, s);
+        case kTile256x192:
+          return launch<gemm_i8_tile_kernel<Epi, 4, 2, 2, 3, 2>>(tm * tn, 512, 2 * 448 * kBK, A, W,
+                                                                 epi, M, N, K, tm, tn, true, s);
+        case kTile256x128:
+          return launch<gemm_i8_tile_kernel<Epi, 4, 2, 2, 2, 3>>(tm * tn, 512, 3 * 384 * kBK, A, W,
+                                                                 epi, M, N, K, tm, tn, true, s);
+        default:
+          break;
+      }
+    }
   }
   if constexpr (std::is_same<Epi, EpiLutI8>::value) {
     // the tabulated epilogue: 128 x 64 tiles, 2 stages + 16 KB of table rows in LDS
@@ -1003,12 +1306,13 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
         return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: more than 2^24 output tiles");
       const int items = tiles_m * tn64;
       const size_t lds = 2 * kStreamStageBytes + (size_t)kSBN * 256;
-      static bool attr_tab[2] = {false, false};
       if (full)
-        return launch(gemm_i8_stream_kernel<Epi, true, 2, true>, items < 512 ? items : 512, lds, A,
-                      W, epi, M, N, K, tiles_m, tn64, vec_store, s, &attr_tab[1], 1);
-      return launch(gemm_i8_stream_kernel<Epi, false, 2, true>, items < 512 ? items : 512, lds, A,
-                    W, epi, M, N, K, tiles_m, tn64, vec_store, s, &attr_tab[0], 1);
+        return launch<gemm_i8_stream_kernel<Epi, true, 2, true>>(items < 512 ? items : 512, 256, lds,
+                                                                 A, W, epi, M, N, K, tiles_m, tn64,
+                                                                 vec_store, s, 1);
+      return launch<gemm_i8_stream_kernel<Epi, false, 2, true>>(items < 512 ? items : 512, 256, lds,
+                                                                A, W, epi, M, N, K, tiles_m, tn64,
+                                                                vec_store, s, 1);
     }
   }
   if (stream) {
@@ -1018,33 +1322,41 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
     const int grid = items < cap ? items : cap;
     if (!narrow) {
       if (full)
-        return launch(gemm_i8_stream128_kernel<Epi, true>, grid, smem, A, W, epi, M, N, K,
-                      tiles_m, tiles_n, vec_store, s, &attr_wide[1], ksplit);
-      return launch(gemm_i8_stream128_kernel<Epi, false>, grid, smem, A, W, epi, M, N, K, tiles_m,
-                    tiles_n, vec_store, s, &attr_wide[0], ksplit);
+        return launch<gemm_i8_stream128_kernel<Epi, true>>(grid, 256, smem, A, W, epi, M, N, K,
+                                                           tiles_m, tiles_n, vec_store, s, ksplit);
+      return launch<gemm_i8_stream128_kernel<Epi, false>>(grid, 256, smem, A, W, epi, M, N, K,
+                                                          tiles_m, tiles_n, vec_store, s, ksplit);
     }
     if (deep) {
       if (full)
-        return launch(gemm_i8_stream_kernel<Epi, true, 3>, grid, smem, A, W, epi, M, N, K, tiles_m,
-                      tiles_n, vec_store, s, &attr_deep[1], ksplit);
-      return launch(gemm_i8_stream_kernel<Epi, false, 3>, grid, smem, A, W, epi, M, N, K, tiles_m,
-                    tiles_n, vec_store, s, &attr_deep[0], ksplit);
+        return launch<gemm_i8_stream_kernel<Epi, true, 3>>(grid, 256, smem, A, W, epi, M, N, K,
+                                                           tiles_m, tiles_n, vec_store, s, ksplit);
+      return launch<gemm_i8_stream_kernel<Epi, false, 3>>(grid, 256, smem, A, W, epi, M, N, K,
+                                                          tiles_m, tiles_n, vec_store, s, ksplit);
     }
     if (full)
-      return launch(gemm_i8_stream_kernel<Epi, true, 2>, grid, smem, A, W, epi, M, N, K, tiles_m,
-                    tiles_n, vec_store, s, &attr_shallow[1], ksplit);
-    return launch(gemm_i8_stream_kernel<Epi, false, 2>, grid, smem, A, W, epi, M, N, K, tiles_m,
-                  tiles_n, vec_store, s, &attr_shallow[0], ksplit);
+      return launch<gemm_i8_stream_kernel<Epi, true, 2>>(grid, 256, smem, A, W, epi, M, N, K,
+                                                         tiles_m, tiles_n, vec_store, s, ksplit);
+    return launch<gemm_i8_stream_kernel<Epi, false, 2>>(grid, 256, smem, A, W, epi, M, N, K,
+                                                        tiles_m, tiles_n, vec_store, s, ksplit);
   }
   if (ksplit != 1) return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: this shape cannot split K");
-  return launch(gemm_i8_generic_kernel<Epi>, tiles, smem, A, W, epi, M, N, K, tiles_m, tiles_n,
-                vec_store, s, &attr_generic);
+  return launch<gemm_i8_generic_kernel<Epi>>(tiles, 256, smem, A, W, epi, M, N, K, tiles_m,
+                                             tiles_n, vec_store, s);
+}
+
+bool gemm_i8_enable_tile_kernel(bool on) {
+  const bool prev = g_tile_kernel_enabled;
+  g_tile_kernel_enabled = on;
+  return prev;
 }
 
 std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
   if (M <= 64 && K % kBK == 0) return std::string("gemm_i8_skinny_kernel<") + epilogue + ">";
   if (!stream_ok(M, N, K)) return std::string("gemm_i8_generic_kernel<") + epilogue + ">";
   const std::string e = epilogue ? epilogue : "";
+  if (g_tile_kernel_enabled && N % 16 == 0 && choose_tile(M, N, K).shape != kTileNone)
+    return "gemm_i8_tile_kernel<" + e + ">";
   if (e == "EpiLutI8" && K / kBK >= 2) return "gemm_i8_stream_kernel<EpiLutI8>";
   const bool wide = (e != "EpiI32" && e != "EpiI8") || !narrow_pays(M, N, K, 1);
   return std::string(wide ? "gemm_i8_stream128_kernel<" : "gemm_i8_stream_kernel<") + e + ">";

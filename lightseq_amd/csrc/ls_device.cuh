@@ -56,6 +56,39 @@ __device__ __forceinline__ int requant_acc(int acc, float alpha) {
   int q = (int)floorf(f + 0.5f);
   return max(-127, min(127, q));
 }
+// requant_acc in fewer instructions, bit for bit the same code: for every float y,
+// floor(med3(y, -127, 127.5)) == clamp(floor(y), -127, 127), so the clamp can precede the one
+// instruction that floors and converts.
+__device__ __forceinline__ float requant_acc_clamped(int acc, float alpha) {
+#pragma clang fp contract(off)
+  float f = (float)acc * alpha;
+  f = f + 0.5f;
+  return __builtin_amdgcn_fmed3f(f, -127.f, 127.5f);
+}
+__device__ __forceinline__ int requant_acc_fast(int acc, float alpha) {
+  int q;
+  asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(q) : "v"(requant_acc_clamped(acc, alpha)));
+  return q;
+}
+// four accumulators -> four codes in one word; the conversion writes its low byte in place
+__device__ __forceinline__ uint32_t requant_acc_pack4(int a0, int a1, int a2, int a3, float alpha) {
+  const float y0 = requant_acc_clamped(a0, alpha), y1 = requant_acc_clamped(a1, alpha);
+  const float y2 = requant_acc_clamped(a2, alpha), y3 = requant_acc_clamped(a3, alpha);
+  uint32_t p;
+  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD"
+      : "=v"(p)
+      : "v"(y0));
+  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
+      : "+v"(p)
+      : "v"(y1));
+  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
+      : "+v"(p)
+      : "v"(y2));
+  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
+      : "+v"(p)
+      : "v"(y3));
+  return p;
+}
 // inference/kernels/common.h:17-23
 __device__ __forceinline__ float gelu_tanh(float x) {
   float cdf = 0.5f * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));

@@ -168,6 +168,9 @@ const char* gemm_i8_act_epilogue_name(int act);
 // The next int8 GEMM launched from this thread records kernel-exact begin / end
 // timestamps into the two events (hipExtLaunchKernelGGL), then the hook clears itself.
 void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop);
+// A/B switch: route large products to the persistent kernels instead of the one-tile-per-
+// workgroup kernel (on by default)
+bool gemm_i8_enable_tile_kernel(bool on);  // returns the previous setting
 
 // ---- fp16 MFMA GEMM (gemm_f16.hip) ------------------------------------------------------
 int gemm_f16_nt(const __half* A, const __half* W, __half* C, int M, int N, int K, hipStream_t s);
@@ -250,9 +253,6 @@ int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_p
                          float* top_score, int* top_idx, int* parent, int* num_finished,
                          float dequant_scale, int vocab_size, int max_step, float length_norm,
                          int cur_step, int batch_size, int beam_size, int end_id, hipStream_t s);
-// ---- GPT path (gpt_kernels.hip, attn_kernels.hip) ------------------------------------------
-// vocab_size <= 0 disables the token-id clamp, max_step <= 0 the position check
-template <typename T>
 // the same step with its proposal workspace in a static device array (allocates nothing)
 int beam_search_step_noalloc_i8I_f16(const int8_t* logits, const __half* logit_bias,
                                      float* seq_probs, float* seq_score, const int* old_alive_seq,
@@ -260,6 +260,9 @@ int beam_search_step_noalloc_i8I_f16(const int8_t* logits, const __half* logit_b
                                      float dequant_scale, int vocab_size, int max_step,
                                      float length_norm, int cur_step, int batch_size, int beam_size,
                                      int end_id, hipStream_t s);
+// ---- GPT path (gpt_kernels.hip, attn_kernels.hip) ------------------------------------------
+// vocab_size <= 0 disables the token-id clamp, max_step <= 0 the position check
+template <typename T>
 int gpt_embedding_i8I(int batch_size, int batch_seq_len, int hidden_size, hipStream_t s,
                       const int8_t* token_emb, const T* pos_emb, const int* token_id, T* output,
                       int* real_seq_len, int padding_id, int pos_offset, float dequant_scale,

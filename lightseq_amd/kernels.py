@@ -546,6 +546,12 @@ def gemm_i8_encdec_q(a, w, q_bias, new_q, step_token_num, hidden, k, beam_size, 
          k, beam_size, head_num, alpha, dequant_scale, current_stream())
 
 
+def gemm_i8_tile_kernel(on):
+    """Route large products to the one-tile-per-workgroup kernel (default) or to the persistent
+    kernels; returns the previous setting."""
+    return bool(lib.load().lsh_gemm_i8_tile_kernel(int(bool(on))))
+
+
 def gemm_i8_lut_i8o(a, w, c, lut, m, n, k, alpha):
     """int8-output GEMM whose epilogue is the table built by :func:`build_act_lut`."""
     _dev(a, w, c, lut)

@@ -55,6 +55,7 @@ _SIGNATURES = {
     "lsh_gemm_i8_i32o_splitk": (False, "ppp" + "iiii" + "p" + "s"),
     "lsh_gemm_i8_preferred_ksplit": (False, "iii"),
     "lsh_layer_norm_row_kernel": (False, "i"),
+    "lsh_gemm_i8_tile_kernel": (False, "i"),
     "lsh_ker_residual_bias_ln_planes_i32I_i8O_f16": (False, "p" + "il" + "ppppp" + "iiff" + "s" +
                                                      "ip"),
     "lsh_gemm_i8_bias_gelu_i8o_f16": (False, "pppp" + "iiifffs"),
@@ -82,8 +83,8 @@ _SIGNATURES = {
     "lsh_ker_write_trg_tokenid_neg_penalty": (False, "ppp" + "iiiiii" + "s"),
     "lsh_ker_write_topk_result": (False, "ppp" + "iiiiii" + "s"),
     "lsh_beam_search_step_i8I": (True, "pppppppppp" + "f" + "ii" + "f" + "iiii" + "s"),
-    "lsh_refresh_cache_by_parent_i8": (False, "iis" + "ppppp" + "l" + "iiiii"),
     "lsh_beam_search_step_noalloc_i8I_f16": (False, "pppppppp" + "f" + "ii" + "f" + "iiii" + "s"),
+    "lsh_refresh_cache_by_parent_i8": (False, "iis" + "ppppp" + "l" + "iiiii"),
     # GPT path
     "lsh_ker_gpt_embedding_i8I": (True, "iiis" + "ppppp" + "iif"),
     "lsh_gpt_scores_i8_i32o": (False, "ppp" + "iii" + "s"),

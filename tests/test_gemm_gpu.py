@@ -20,6 +20,9 @@ LARGE = [(4096, 2304, 768), (4096, 768, 768), (4096, 3072, 768), (4096, 768, 307
          (1000, 30522 // 6, 128), (64, 1000, 1024),
          # ragged rows and columns in the 128x64 kernel (column tails of 40 and of 8), a single K step
          (200, 1000, 1536), (130, 72, 256), (256, 192, 128),
+         # one output tile per workgroup: 256 x 256 with ragged rows and a 16-column last tile,
+         # 256 x 192 with ragged rows and the shortest K loop it takes, 256 x 128 (K loop = ring depth)
+         (4000, 3088, 768), (3900, 3072, 384), (8192, 1024, 384), (8192, 1024, 1024),
          # decode-step shapes (rows = batch x beam of one step)
          (16, 3072, 1024), (16, 1024, 4096), (16, 50257, 1024), (64, 32000, 1024),
          (64, 4096, 1024), (33, 1000, 256), (1, 64, 128), (48, 40, 384)]
@@ -105,7 +108,57 @@ def test_gemm_rejects_bad_k():
         _k().gemm_i8_i32o(a, a, c, 4, 4, 8)
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 2304, 768), (4096, 4096, 1024), (4000, 3088, 768), (8192, 1024, 384)])
+def test_tile_kernel_equals_persistent_kernels(rng, M, N, K):
+    """The one-tile-per-workgroup kernel and the persistent kernels give the same bytes."""
+    k = _k()
+    a = to_dev(rng.integers(-127, 128, size=(M, K), dtype=np.int8))
+    w = to_dev(rng.integers(-127, 128, size=(N, K), dtype=np.int8))
+    alpha = 3.0 / (np.sqrt(K) * 127)
+    outs = []
+    prev = k.gemm_i8_tile_kernel(True)
+    try:
+        for on in (True, False):
+            k.gemm_i8_tile_kernel(on)
+            c32 = torch.zeros((M, N), dtype=torch.int32, device=DEV)
+            c8 = torch.zeros((M, N), dtype=torch.int8, device=DEV)
+            k.gemm_i8_i32o(a, w, c32, M, N, K)
+            k.gemm_i8_i8o(a, w, c8, M, N, K, alpha)
+            outs.append((c32, c8))
+    finally:
+        k.gemm_i8_tile_kernel(prev)
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+def test_fused_gelu_epilogue_at_the_microbenchmark_shape(oracle, rng):
+    """4096 x 4096 x 1024 with clip values 4.0 / 0.08 / 6.0: the fused bias + GELU + requant
+    epilogue (arithmetic and tabulated) against the oracle's stand-alone kernel on the exact
+    int8 product."""
+    M, N, K = 4096, 4096, 1024
+    a = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    bias = (0.02 * rng.standard_normal(N)).astype(np.float16)
+    c_in, c_w, c_out, c_act = 4.0, 0.08, 6.0, 6.0
+    alpha = np.float32(c_in * c_w / (c_out * 127))
+    f = _exact_i32(a, w).astype(np.float32) * alpha
+    prod8 = np.clip(np.floor(f + np.float32(0.5)), -127, 127).astype(np.int8)
+    ds, qs = c_out / 127, 127 / c_act
+    want = oracle.bias_gelu_i8I_i8O(prod8, bias, ds, qs)
+    k = _k()
+    ad, wd, bd = to_dev(a), to_dev(w), to_dev(bias)
+    got = torch.zeros((M, N), dtype=torch.int8, device=DEV)
+    k.gemm_i8_bias_gelu_i8o(ad, wd, got, bd, M, N, K, float(alpha), ds, qs)
+    from conftest import assert_codes_close
+    assert_codes_close(to_np(got), want, what="fused GELU epilogue vs oracle")
+    lut = torch.zeros((N, 256), dtype=torch.int8, device=DEV)
+    k.build_act_lut(lut, bd, N, ds, qs, c_act, 0)
+    via_lut = torch.zeros_like(got)
+    k.gemm_i8_lut_i8o(ad, wd, via_lut, lut, M, N, K, float(alpha))
+    assert torch.equal(via_lut, got)
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 3072, 768), (4096, 3072, 768), (77, 160, 48),
+                                   (4000, 3088, 768), (8192, 1024, 384),
                                    (16, 4096, 1024), (64, 4096, 1024),
                                    # ragged columns with the table rows in LDS (last tile: 40 and 16 columns)
                                    (200, 1000, 256), (130, 208, 384)])
