@@ -23,6 +23,8 @@ LARGE = [(4096, 2304, 768), (4096, 768, 768), (4096, 3072, 768), (4096, 768, 307
          # one output tile per workgroup: 256 x 256 with ragged rows and a 16-column last tile,
          # 256 x 192 with ragged rows and the shortest K loop it takes, 256 x 128 (K loop = ring depth)
          (4000, 3088, 768), (3900, 3072, 384), (8192, 1024, 384), (8192, 1024, 1024),
+         # 128 x 96 tiles on 4 wavefronts (narrow outputs), ragged rows, both ring depths
+         (4000, 768, 384), (3000, 960, 1536),
          # decode-step shapes (rows = batch x beam of one step)
          (16, 3072, 1024), (16, 1024, 4096), (16, 50257, 1024), (64, 32000, 1024),
          (64, 4096, 1024), (33, 1000, 256), (1, 64, 128), (48, 40, 384)]
@@ -108,7 +110,8 @@ def test_gemm_rejects_bad_k():
         _k().gemm_i8_i32o(a, a, c, 4, 4, 8)
 
 
-@pytest.mark.parametrize("M,N,K", [(4096, 2304, 768), (4096, 4096, 1024), (4000, 3088, 768), (8192, 1024, 384)])
+@pytest.mark.parametrize("M,N,K", [(4096, 2304, 768), (4096, 4096, 1024), (4000, 3088, 768), (8192, 1024, 384),
+                                   (4096, 768, 3072), (4096, 768, 768)])
 def test_tile_kernel_equals_persistent_kernels(rng, M, N, K):
     """The one-tile-per-workgroup kernel and the persistent kernels give the same bytes."""
     k = _k()
@@ -158,7 +161,7 @@ def test_fused_gelu_epilogue_at_the_microbenchmark_shape(oracle, rng):
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 128), (300, 3072, 768), (4096, 3072, 768), (77, 160, 48),
-                                   (4000, 3088, 768), (8192, 1024, 384),
+                                   (4000, 3088, 768), (8192, 1024, 384), (4096, 768, 768),
                                    (16, 4096, 1024), (64, 4096, 1024),
                                    # ragged columns with the table rows in LDS (last tile: 40 and 16 columns)
                                    (200, 1000, 256), (130, 208, 384)])
