@@ -26,7 +26,15 @@ The JSON line also carries
                  bias+GELU+requantisation epilogue, and the stand-alone
                  dequant-bias-GELU-requant kernel, timed the same way;
   cpu_baseline   the CPU oracle (a C port of the reference's algorithm, OpenMP) timed
-                 on this host on a bounded sample of the same workload.
+                 on this host on a bounded sample of the same workload, and beside it
+                 (``torch_cpu``) a PyTorch-CPU restatement of the layer with the formulas of
+                 the reference's kernel tests (F.linear on dequantised codes, F.layer_norm,
+                 tanh-GELU, fake quantisation between the stages) -- baselines only.
+
+``step_ms`` holds the median, 10th and 90th percentile of the per-step times between HIP
+events recorded on the model's stream; ``roofline.measured_peak`` is what a loop of nothing
+but register-resident int8 MFMAs sustains on this box, ``frac_of_measured_peak`` the dominant
+launch against that.
 
 ``--workload transformer_big`` and ``--workload gpt2_medium`` time the two generation
 workloads (beam-search translation, greedy GPT generation) through ``QuantTransformer`` /
@@ -64,9 +72,80 @@ def cpu_baseline(cfg, msg, ids, layers=12):
     full = dt * cfg["n_layer"] / layers
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     return {"value": ids.size / full, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "what": "oracle/ls_oracle*.c: plain-C restatement of the reference's int8 kernels, OpenMP",
             "sample": "one step: %d of %d encoder layers at batch %d x seq %d, %.1f s of CPU work%s"
                       % (layers, cfg["n_layer"], ids.shape[0], ids.shape[1], dt,
                          "" if layers == cfg["n_layer"] else ", scaled to the full stack")}
+
+
+def torch_cpu_baseline(cfg, ids, layers=2):
+    """PyTorch-CPU restatement of the int8 encoder layer with the formulas the reference's
+    kernel tests use as their baselines (tests/test_ls_kernels.py: F.layer_norm, F.linear on
+    dequantised int8 codes, relu / gelu of the dequantised sum, quantise by
+    clamp(floor(x / scale + 0.5))), fp32, all host threads.  A baseline, not a checker:
+    `layers` layers at the full batch, scaled to the stack."""
+    import torch
+    import torch.nn.functional as F
+    B, S = ids.shape
+    H, I, h = cfg["hidden"], cfg["inner"], cfg["head_num"]
+    d = H // h
+    g = torch.Generator().manual_seed(0)
+
+    def fq(x, clip):  # fake quantisation: quantise + dequantise
+        s = clip / 127.0
+        return torch.clamp(torch.floor(x / s + 0.5), -127, 127) * s
+
+    ws = [dict(qkv=fq(torch.randn(3 * H, H, generator=g) * 0.02, 0.08), o=fq(torch.randn(H, H, generator=g) * 0.02, 0.08),
+               f1=fq(torch.randn(I, H, generator=g) * 0.02, 0.08), f2=fq(torch.randn(H, I, generator=g) * 0.02, 0.08),
+               b_qkv=torch.zeros(3 * H), b_o=torch.zeros(H), b1=torch.zeros(I), b2=torch.zeros(H),
+               g1=torch.ones(H), be1=torch.zeros(H), g2=torch.ones(H), be2=torch.zeros(H)) for _ in range(layers)]
+    x = torch.randn(B, S, H, generator=g)
+    mask = torch.from_numpy((ids == cfg["padding_id"])).view(B, 1, 1, S)
+
+    def layer(x, w):
+        B = x.shape[0]
+        mask_b = mask[:B]
+        q0 = fq(F.layer_norm(x, (H,), w["g1"], w["be1"], 1e-12), 4.0)
+        qkv = fq(F.linear(q0, w["qkv"]), 8.0) + w["b_qkv"]
+        q, k, v = (t.reshape(B, S, h, d).transpose(1, 2) for t in qkv.split(H, dim=-1))
+        p = torch.softmax((q @ k.transpose(-1, -2) / d ** 0.5).masked_fill(mask_b, -1e8), -1)
+        ctx = fq((p @ v).transpose(1, 2).reshape(B, S, H), 2.0)
+        r = fq(F.linear(ctx, w["o"]), 4.0) + w["b_o"] + x
+        q1 = fq(F.layer_norm(r, (H,), w["g2"], w["be2"], 1e-12), 4.0)
+        a = fq(F.gelu(fq(F.linear(q1, w["f1"]), 8.0) + w["b1"], approximate="tanh"), 6.0)
+        return F.linear(a, w["f2"]) + w["b2"] + r
+
+    with torch.no_grad():
+        layer(x[:2], ws[0])
+        t0 = time.perf_counter()
+        for w in ws:
+            x = layer(x, w)
+        dt = time.perf_counter() - t0
+    full = dt * cfg["n_layer"] / layers
+    return {"value": ids.size / full, "unit": "tokens/s", "cores": torch.get_num_threads(),
+            "kind": "PyTorch-CPU fp32 restatement of the reference's kernel-test baselines",
+            "sample": "%d of %d layers at batch %d x seq %d, %.1f s of CPU work, scaled to the full stack"
+                      % (layers, cfg["n_layer"], B, S, dt)}
+
+
+def measured_mfma_peak(reps=5):
+    """TOP/s of a loop of independent register-resident int8 MFMAs (lsh_mfma_i8_peak_probe),
+    2 workgroups per compute unit, timed with HIP events on the launch stream."""
+    import torch
+    from lightseq_amd import kernels as K
+    wgs = 2 * torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.zeros(wgs * 256, dtype=torch.int32, device="cuda:0")
+    K.mfma_i8_peak_probe(out, wgs, 200)
+    torch.cuda.synchronize()
+    best = 0.0
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        ops = K.mfma_i8_peak_probe(out, wgs, 4000)
+        e1.record()
+        torch.cuda.synchronize()
+        best = max(best, ops / (e0.elapsed_time(e1) * 1e-3) / 1e12)
+    return best
 
 
 def fused_kernel_rates(cfg, reps=50):
@@ -192,7 +271,27 @@ def gemm_microbench(reps=40):
             "avg_us": us, "algorithmic_bytes": nbytes, "GB/s": nbytes / (us * 1e-6) / 1e9,
             "frac_of_hbm_peak": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
         out["%dx%dx%d" % (M, N, Kd)] = res
+    out["vendor_yardstick torch._int_mm (int32 out, same box; not used by the library)"] = _int_mm_yardstick(reps)
     return out
+
+
+def _int_mm_yardstick(reps):
+    """torch._int_mm (the vendor library's int8 GEMM as PyTorch-ROCm reaches it) on the layer's
+    four products and the two micro-benchmark shapes, int32 output, timed like the rest."""
+    import torch
+    dev = "cuda:0"
+    res = {}
+    for M, N, Kd in ((4096, 2304, 768), (4096, 768, 768), (4096, 3072, 768), (4096, 768, 3072),
+                     (4096, 4096, 1024), (4096, 1024, 4096)):
+        key = "%dx%dx%d" % (M, N, Kd)
+        try:
+            a = torch.randint(-127, 128, (M, Kd), dtype=torch.int8, device=dev)
+            b = torch.randint(-127, 128, (N, Kd), dtype=torch.int8, device=dev).t()
+            us = _queued_time_us(lambda: torch._int_mm(a, b), reps)
+            res[key] = {"avg_us": us, "TOP/s": 2.0 * M * N * Kd / (us * 1e-6) / 1e12}
+        except Exception as e:  # record why the yardstick is missing
+            res[key] = {"error": repr(e)[:200]}
+    return res
 
 
 TRAFFIC_SUMMARY = "bert_base_b32_s128_pmc_hbm_traffic.txt"
@@ -212,6 +311,26 @@ def _profiled_traffic(kernel, site):
         if m and m.group(1).replace("lsh::", "") == want:
             return int(m.group(2))
     return None
+
+
+def _per_step_event_times(model, steps):
+    """Per-step GPU time between HIP events recorded on the model's own stream (a second pass
+    over the same steps): median, 10th and 90th percentile, milliseconds."""
+    import numpy as np
+    import torch
+    stream = torch.cuda.ExternalStream(model.get_stream())
+    times = []
+    for _ in range(steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        model.infer_device()
+        e1.record(stream)
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    t = np.asarray(times)
+    return {"median": float(np.median(t)), "p10": float(np.percentile(t, 10)),
+            "p90": float(np.percentile(t, 90)), "steps": int(steps),
+            "how": "HIP events on the model's stream around each Infer()"}
 
 
 def bench_bert(args):
@@ -236,6 +355,7 @@ def bench_bert(args):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     tokens_per_s = BATCH * SEQ * args.steps / dt
+    step_ms = _per_step_event_times(model, args.steps)
 
     # instrumented pass: HIP events around every int8 GEMM launch on the model's stream
     model.set_profiling(True)
@@ -254,8 +374,13 @@ def bench_bert(args):
     (name, dom_site), dom = max(by_kernel.items(), key=lambda kv: kv[1]["ms"])
     avg_ms = dom["ms"] / dom["launches"]
     achieved = dom["ops"] / dom["launches"] / (avg_ms * 1e-3) / 1e12
+    measured_peak = measured_mfma_peak()
     roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                "frac": achieved / INT8_MFMA_PEAK_TOPS, "traffic": _profiled_traffic(name, dom_site),
+                "frac": achieved / INT8_MFMA_PEAK_TOPS, "measured_peak": measured_peak,
+                "frac_of_measured_peak": achieved / measured_peak,
+                "measured_peak_how": "register-resident v_mfma_i32_32x32x32_i8 loop, 2 workgroups per "
+                                     "compute unit (lsh_mfma_i8_peak_probe)",
+                "traffic": _profiled_traffic(name, dom_site),
                 "traffic_source": "profiles/" + TRAFFIC_SUMMARY, "kernel": name,
                 "sites": dom["sites"], "avg_launch_us": avg_ms * 1e3,
                 "gemm_sites": {s["site"]: {"kernel": s["kernel"], "mnk": [s["m"], s["n"], s["k"]],
@@ -267,8 +392,8 @@ def bench_bert(args):
         "metric": "int8 tokens/sec BERT-base b32 s128; int8 GEMM % MFMA-i8 peak; fused GB/s",
         "value": tokens_per_s, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": 1e3 * dt / args.steps, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "ms_per_step": 1e3 * dt / args.steps, "step_ms": step_ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "BERT-base-shaped int8 encoder stack: 12 layers, hidden 768, 12 heads, "
                                "FFN 3072 GELU, batch 32 x seq 128, valid lengths U[32,128] right-padded, "
                                "vocab 30522, random-init N(0,0.02) weights quantised per tensor",
@@ -282,6 +407,7 @@ def bench_bert(args):
         out["gemm_microbench"] = gemm_microbench()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, msg, ids)
+        out["cpu_baseline"]["torch_cpu"] = torch_cpu_baseline(cfg, ids)
     return out
 
 
@@ -364,9 +490,9 @@ def main():
                  "one stream, as in the reference); --gpus %d is not supported" % args.gpus)
     bert = args.workload == "bert_base"
     if args.steps is None:
-        args.steps = 50 if bert else 3
+        args.steps = 100 if bert else 3
     if args.warmup is None:
-        args.warmup = 10 if bert else 1
+        args.warmup = 20 if bert else 1
 
     import torch
     if not torch.cuda.is_available():

@@ -235,6 +235,12 @@ int lsh_layer_norm_row_kernel(int on);
  * one against the other.  No counterpart in the reference (its cuBLASLt algorithm table
  * plays this part: model/cublas_algo_map.cc). */
 int lsh_gemm_i8_tile_kernel(int on);
+/* Measurement aid, no counterpart in the reference: one launch of `workgroups` x 4 wavefronts
+ * that issue nothing but independent int8 MFMAs (v_mfma_i32_32x32x32_i8) on register-resident
+ * operands, `iters` x 8 each.  out: workgroups * 256 ints (checksums, so that nothing is
+ * optimised away); *ops receives the integer operations of the launch.  Timed by the caller:
+ * ops / time is what the matrix units sustain at the clock the part holds under that load. */
+int lsh_mfma_i8_peak_probe(int* out, int workgroups, int iters, double* ops, lsh_stream_t stream);
 /* Decode-step QKV product with ker_arrange_decself_qkv_i8I_i8O
  * (kernels/transformerKernels_int8.cc.cu:1432-1513; call sites model/quant_decoder.cc.cu:660-674,
  * model/quant_gpt_encoder.cc.cu:640-653) as its epilogue: A [step_token_num, k] x W [3*hidden, k]

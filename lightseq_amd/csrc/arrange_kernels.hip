@@ -207,18 +207,20 @@ int arrange_atten_output_i8O(int batch_token_num, int hidden_size, hipStream_t s
 
 // ---------------------------------------------------------------------------------
 // token embedding from an int8 table + position embedding; writes the pad mask.
+// vocab > 0: token ids are clamped into the table (an id outside it must not become a read
+// outside the allocation); vocab <= 0: ids are used as they are, as the reference does.
 template <typename T>
 __global__ void __launch_bounds__(256)
 enc_emb_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__ pos_emb,
                const int* __restrict__ tokens, T* __restrict__ output, int* __restrict__ pad_mask,
-               int pad_id, long total8, int seq_len, int hidden8, float scale) {
+               int pad_id, long total8, int seq_len, int hidden8, float scale, int vocab) {
   long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const long stride = (long)gridDim.x * blockDim.x;
   for (; idx < total8; idx += stride) {
     const int dim8 = (int)(idx % hidden8);
     const long tok_idx = idx / hidden8;
     const int seq = (int)(tok_idx % seq_len);
-    const int token = tokens[tok_idx];
+    int token = tokens[tok_idx];
     float v[8];
     if (token == pad_id) {
       if (dim8 == 0) pad_mask[tok_idx] = 1;
@@ -226,6 +228,7 @@ enc_emb_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__ pos_e
       for (int k = 0; k < 8; ++k) v[k] = 0.f;
     } else {
       if (dim8 == 0) pad_mask[tok_idx] = 0;
+      if (vocab > 0) token = min(max(token, 0), vocab - 1);
       float p[8];
       unpack8(*reinterpret_cast<const uint2*>(token_emb + ((long)token * hidden8 + dim8) * 8), v);
       ld8(pos_emb, ((long)seq * hidden8 + dim8) * 8, p);
@@ -239,7 +242,7 @@ enc_emb_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__ pos_e
 template <typename T>
 int enc_emb_i8I(const int8_t* token_emb, const T* pos_emb, const int* tokens, T* output,
                 int* pad_mask, int pad_id, int batch_size, int seq_len, int hidden_dim,
-                hipStream_t s, float dequant_scale, bool scaled) {
+                hipStream_t s, float dequant_scale, bool scaled, int vocab_size) {
   if (batch_size <= 0 || seq_len <= 0 || hidden_dim <= 0 || !token_emb || !pos_emb || !tokens ||
       !output || !pad_mask)
     return lsh_fail(LSH_ERR_INVALID, "launch_enc_emb_i8I: bad arguments");
@@ -252,7 +255,7 @@ int enc_emb_i8I(const int8_t* token_emb, const T* pos_emb, const int* tokens, T*
   const long total8 = (long)batch_size * seq_len * (hidden_dim / 8);
   enc_emb_kernel<T><<<grid_for(total8), 256, 0, s>>>(token_emb, pos_emb, tokens, output, pad_mask,
                                                      pad_id, total8, seq_len, hidden_dim / 8,
-                                                     scale);
+                                                     scale, vocab_size);
   return lsh_check_launch("enc_emb_kernel");
 }
 
@@ -265,7 +268,7 @@ int enc_emb_i8I(const int8_t* token_emb, const T* pos_emb, const int* tokens, T*
   template int arrange_atten_output_i8O<T>(int, int, hipStream_t, const T*, int8_t*, int, int,    \
                                            int, float);                                           \
   template int enc_emb_i8I<T>(const int8_t*, const T*, const int*, T*, int*, int, int, int, int,  \
-                              hipStream_t, float, bool);
+                              hipStream_t, float, bool, int);
 LSH_INST(float)
 LSH_INST(__half)
 #undef LSH_INST

@@ -107,6 +107,9 @@ int lsh_launch_dequantize_tensor_f32(const int32_t* input, void* output, int bat
 // ---- LayerNorm family --------------------------------------------------------------
 int lsh_layer_norm_row_kernel(int on) { return ln_set_few_rows(on != 0) ? 1 : 0; }
 int lsh_gemm_i8_tile_kernel(int on) { return gemm_i8_enable_tile_kernel(on != 0) ? 1 : 0; }
+int lsh_mfma_i8_peak_probe(int* out, int workgroups, int iters, double* ops, lsh_stream_t stream) {
+  return mfma_i8_peak_probe(out, workgroups, iters, ops, HS(stream));
+}
 int lsh_ker_norm_layer_resual_i8O_f16(int token_num, int hidden_size, lsh_stream_t stream,
                                       void* input, int8_t* output, const void* scale,
                                       const void* bias, const void* residual_bias,
@@ -306,7 +309,7 @@ int lsh_launch_enc_emb_i8I_f16(const int8_t* token_emb, const void* pos_emb, con
   if (multilg_type != 0) return lsh_fail(LSH_ERR_INVALID, "multilingle not supported");
   return enc_emb_i8I<__half>(token_emb, H(pos_emb), tokens, HM(output), pad_mask, pad_id,
                              batch_size, seq_len, hidden_dim, HS(stream), dequant_scale,
-                             scaled != 0);
+                             scaled != 0, 0);
 }
 int lsh_launch_enc_emb_i8I_f32(const int8_t* token_emb, const void* pos_emb, const int* tokens,
                                void* output, int* pad_mask, int pad_id, int batch_size,
@@ -316,7 +319,7 @@ int lsh_launch_enc_emb_i8I_f32(const int8_t* token_emb, const void* pos_emb, con
   if (multilg_type != 0) return lsh_fail(LSH_ERR_INVALID, "multilingle not supported");
   return enc_emb_i8I<float>(token_emb, F(pos_emb), tokens, FM(output), pad_mask, pad_id,
                             batch_size, seq_len, hidden_dim, HS(stream), dequant_scale,
-                            scaled != 0);
+                            scaled != 0, 0);
 }
 int lsh_launch_scaled_colsum_f16(const void* inp, void* out, int rows, int cols, float scale,
                                  lsh_stream_t stream) {

@@ -1526,6 +1526,36 @@ int gemm_i8_qkv_arrange_f16(const int8_t* A, const int8_t* W, __half* new_qkv, c
                   batch_tokens, 3 * hidden, K, s);
 }
 
+// Measurement aid: nothing but independent int8 MFMAs on register-resident operands, 8
+// accumulator blocks per wavefront, 4 wavefronts per workgroup.  What the matrix units
+// sustain at the clock the part holds under this load, as opposed to the nominal peak.
+__global__ void __launch_bounds__(256)
+mfma_i8_peak_kernel(int* __restrict__ out, int iters) {
+  v4i a = {(int)threadIdx.x * 0x01010101, 0x7f81037d, 0x22e1c3a5, (int)blockIdx.x};
+  v4i b = {0x5a3c1e7f, (int)threadIdx.x * 0x00010203, (int)0x81ff7f01u, 0x13579bdf};
+  v16i c[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) c[i] = (v16i)0;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c[i], 0, 0, 0);
+  }
+  int sum = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) sum += c[i][j];
+  out[blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
+int mfma_i8_peak_probe(int* out, int workgroups, int iters, double* ops, hipStream_t s) {
+  if (!out || workgroups <= 0 || iters <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "mfma_i8_peak_probe: bad arguments");
+  mfma_i8_peak_kernel<<<workgroups, 256, 0, s>>>(out, iters);
+  if (ops) *ops = (double)workgroups * 4 * iters * 8 * (2.0 * 32 * 32 * 32);
+  return lsh_check_launch("mfma_i8_peak_kernel");
+}
+
 const char* gemm_i8_act_epilogue_name(int act) {
   return act == kActGelu ? EpiActI8<kActGelu>::name() : EpiActI8<kActRelu>::name();
 }

@@ -98,10 +98,11 @@ template <typename T>
 int arrange_atten_output_i8O(int batch_token_num, int hidden_size, hipStream_t s, const T* ori_q,
                              int8_t* new_q, int beam_size, int dim_per_head, int head_num,
                              float quant_scale);
+// vocab_size > 0 clamps the token ids into the table; <= 0 uses them unchecked
 template <typename T>
 int enc_emb_i8I(const int8_t* token_emb, const T* pos_emb, const int* tokens, T* output,
                 int* pad_mask, int pad_id, int batch_size, int seq_len, int hidden_dim,
-                hipStream_t s, float dequant_scale, bool scaled);
+                hipStream_t s, float dequant_scale, bool scaled, int vocab_size);
 
 // ---- encoder attention (attn_kernels.hip) ------------------------------------------
 template <typename T>
@@ -171,6 +172,9 @@ void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop);
 // A/B switch: route large products to the persistent kernels instead of the one-tile-per-
 // workgroup kernel (on by default)
 bool gemm_i8_enable_tile_kernel(bool on);  // returns the previous setting
+// register-resident int8 MFMA loop (measurement aid): out needs workgroups * 256 ints; *ops
+// receives the integer operations of one launch
+int mfma_i8_peak_probe(int* out, int workgroups, int iters, double* ops, hipStream_t s);
 
 // ---- fp16 MFMA GEMM (gemm_f16.hip) ------------------------------------------------------
 int gemm_f16_nt(const __half* A, const __half* W, __half* C, int M, int N, int K, hipStream_t s);

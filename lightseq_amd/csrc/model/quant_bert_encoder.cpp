@@ -32,8 +32,8 @@ std::string QuantBertEncoder::check() {
     return "wrong clip_max table size";
   if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)
     return "violate hidden_size % 16 = 0 and inner_size % 16 = 0 (int8 MFMA GEMM)";
-  if (_tw._dim_per_head != 32 && _tw._dim_per_head != 64)
-    return "violate dim_per_head in {32, 64} (fused attention kernel)";
+  if (_tw._dim_per_head != 32 && _tw._dim_per_head != 64 && _tw._dim_per_head != 128)
+    return "violate dim_per_head in {32, 64, 128} (fused attention kernel)";
   if (_tw._max_step > 1024) return "violate max_step <= 1024";
   return "";
 }
@@ -161,7 +161,7 @@ void QuantBertEncoder::run_one_infer(int batch_size, int batch_seq_len) {
   LSH_CALL(enc_emb_i8I<__half>(_int8_emb.get(), _pos_emb.get(), _p_d_token_id, _p_d_output,
                                _p_d_padding_mask, _tw._padding_id, batch_size, batch_seq_len,
                                _tw._hidden_size, _stream, _src_emb_clip_max / _quant_range,
-                               _tw._scale_embedding));
+                               _tw._scale_embedding, _tw._src_vocab_size));
   for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
     self_attention();
     ffn_add_norm();

@@ -57,7 +57,8 @@ std::string QuantDecoder::check() {
   if (m != "beam_search" && m != "topk" && m != "topp" && m != "topk_greedy")
     return std::string("unsupported sampling_method: ") + m;
   if (m != "beam_search")
-    return "sampling_method " + m + " is not available in this build (beam_search only)";
+    return "sampling_method " + m + " (topk = " + std::to_string(_tw._topk) + ", topp = " +
+           std::to_string(_tw._topp) + ") is not available in this build (beam_search only)";
   if (_tw._diverse_lambda != 0.f) return "diverse beam search is not available in this build";
   if (_tw._max_step > 1024) return "max_step should not greater than 1024";
   if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)

@@ -39,7 +39,10 @@ std::string QuantGptEncoder::check() {
     return std::string("unsupported sampling_method: ") + m;
   if (_tw._topk <= 0) return "topk must be positive";
   if (m == "topp" || (m == "topk" && _tw._topk != 1))
-    return "random sampling (topp, topk > 1) is not available in this build: use topk = 1 or ppl";
+    return "random sampling is not available in this build: the model file asks for sampling_method " +
+           m + " with topk = " + std::to_string(_tw._topk) + ", topp = " + std::to_string(_tw._topp) +
+           " (a file that sets no topk gets the format's default, 4); export it with topk = 1 "
+           "(greedy) or sampling_method ppl";
   if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)
     return "violate hidden_size % 16 = 0 and inner_size % 16 = 0 (int8 MFMA GEMM)";
   if (_tw._dim_per_head != 32 && _tw._dim_per_head != 64 && _tw._dim_per_head != 128)

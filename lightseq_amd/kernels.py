@@ -552,6 +552,15 @@ def gemm_i8_tile_kernel(on):
     return bool(lib.load().lsh_gemm_i8_tile_kernel(int(bool(on))))
 
 
+def mfma_i8_peak_probe(out, workgroups, iters):
+    """Launch the register-resident int8 MFMA loop; returns the integer operations of the launch."""
+    import ctypes
+    _dev(out)
+    ops = ctypes.c_double(0.0)
+    call("lsh_mfma_i8_peak_probe", ptr(out), workgroups, iters, ctypes.addressof(ops), current_stream())
+    return ops.value
+
+
 def gemm_i8_lut_i8o(a, w, c, lut, m, n, k, alpha):
     """int8-output GEMM whose epilogue is the table built by :func:`build_act_lut`."""
     _dev(a, w, c, lut)

@@ -93,3 +93,18 @@ def test_status_codes_without_gpu():
     rc = L.lsh_launch_enc_emb_i8I_f16(None, None, None, None, None, 0, 1, 1, 8, None, None, None, 1,
                                       ctypes.c_float(1.0), 0)
     assert rc == lib.LSH_ERR_INVALID and "multilingle" in lib.last_error()
+
+
+def test_reference_module_name_exposes_the_int8_models():
+    """`import lightseq.inference as lsi` is what the reference's users write
+    (lightseq/inference/pywrapper/wrapper.cc:944-976 registers the classes there)."""
+    import lightseq.inference as lsi
+    from lightseq_amd import inference
+    assert lsi.QuantBert is inference.QuantBert
+    assert lsi.QuantTransformer is inference.QuantTransformer
+    assert lsi.QuantGpt is inference.QuantGpt
+    for method in ("infer",):
+        assert callable(getattr(lsi.QuantBert, method)) and callable(getattr(lsi.QuantTransformer, method))
+    assert callable(lsi.QuantGpt.sample) and callable(lsi.QuantGpt.ppl)
+    with pytest.raises(AttributeError, match="only the int8 models"):
+        lsi.Bert

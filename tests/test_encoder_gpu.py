@@ -33,6 +33,7 @@ def _valid(ids, cfg):
     ("tiny", 2, 33, {"use_gelu": False}),
     ("tiny", 2, 16, {"is_post_ln": False}),
     ("tiny", 1, 64, {"is_post_ln": False, "use_gelu": False}),
+    ("tiny", 2, 24, {"hidden": 256, "inner": 512, "head_num": 2}),   # 128-wide heads
 ])
 def test_tiny_stack_with_taps(tmp_path, oracle, cfg_name, batch, seq, over):
     from lightseq_amd import inference, synthetic
@@ -245,6 +246,42 @@ def test_bert_base_full_stack_properties(tmp_path):
     v = ids != cfg["padding_id"]
     np.testing.assert_allclose(z[v].mean(-1), 0.0, atol=2e-2)
     np.testing.assert_allclose(z[v].std(-1), 1.0, atol=2e-2)
+    model.close()
+
+
+def test_reference_module_name_runs_unchanged(tmp_path):
+    """A script written against the reference's module runs as it is."""
+    import lightseq.inference as lsi
+    from lightseq_amd import synthetic
+    cfg, _msg, path = _build(tmp_path, "tiny", 2)
+    ids, _ = synthetic.make_token_ids(cfg, 3, 12, seed=1)
+    model = lsi.QuantBert(path, 4)
+    out = model.infer(ids)
+    assert out.shape == (3, 12, cfg["hidden"]) and out.dtype == np.float32
+    assert np.isfinite(out).all() and np.abs(out).max() > 0
+
+
+def test_token_ids_outside_the_table_are_clamped(tmp_path):
+    """An id below 0 or beyond the vocabulary must not become a read outside the embedding
+    table: the model clamps it (the decoder and GPT embeddings do the same)."""
+    from lightseq_amd import inference, synthetic
+    cfg, _msg, path = _build(tmp_path, "tiny", 4)
+    ids, _ = synthetic.make_token_ids(cfg, 2, 16, seed=6)
+    bad = ids.copy()
+    pos = [(0, 1), (0, 3), (1, 0), (1, 2)]
+    for (b, t), v in zip(pos, (cfg["vocab"], cfg["vocab"] + 12345, 2 ** 31 - 1, cfg["vocab"] + 1)):
+        assert ids[b, t] != cfg["padding_id"]
+        bad[b, t] = v
+    clamped = np.minimum(bad, cfg["vocab"] - 1)
+    model = inference.QuantBert(path, 2)
+    got = model.infer_fp16(bad)
+    want = model.infer_fp16(clamped)
+    np.testing.assert_array_equal(got.view(np.uint16), want.view(np.uint16))
+    # negative ids read row 0 of the table (they are not the padding id, so they stay unmasked)
+    neg = ids.copy()
+    neg[0, 1], neg[1, 2] = -7, -(2 ** 31)
+    out = model.infer_fp16(neg)
+    assert np.isfinite(out.astype(np.float32)).all()
     model.close()
 
 

@@ -157,7 +157,9 @@ def test_ppl(rng, batch, seq, vocab):
 
 
 @pytest.mark.parametrize("batch,heads,seq,d,max_step", [(2, 2, 9, 32, 16), (2, 16, 130, 64, 160),
-                                                        (1, 4, 64, 64, 64), (3, 2, 200, 32, 256)])
+                                                        (1, 4, 64, 64, 64), (3, 2, 200, 32, 256),
+                                                        # the prompt length of the generation benchmark
+                                                        (2, 4, 512, 64, 640)])
 def test_prefill_attention_fused(oracle, rng, batch, heads, seq, d, max_step):
     """gpt_arrange_qkv_prefill + gpt_prefill_attention == the reference's unfused chain."""
     H, M, bh = heads * d, batch * seq, batch * heads
@@ -337,3 +339,49 @@ def test_gpt2_medium_shape(tmp_path):
     out, steps, logits = _run_sample(path, cfg, ids, max_batch=2)
     assert steps >= 1 and out.shape[1] == 48 + steps
     _check_sample(msg, cfg, ids, out, steps, logits)
+
+
+def test_gpt2_medium_full_size_properties(tmp_path):
+    """The generation benchmark at its stated size -- 24 layers, hidden 1024, 16 heads, inner
+    4096, vocabulary 50257, batch 16, prompt 512, 128 generated tokens, greedy -- through
+    QuantGpt.  The oracle would take minutes here, so the run is held to what must be true at
+    any size: every generated token is the first arg-max of that step's recorded logits, the
+    prompt is kept, the run is deterministic, and a sequence's tokens do not depend on the rest
+    of its batch."""
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import QuantGpt
+    cfg = synthetic.gpt_config("gpt2_medium")
+    batch, prompt, new = 16, 512, 128
+    assert cfg["n_layer"] == 24 and cfg["max_step"] >= prompt + new
+    cfg.update(extra_decode_length=new)
+    path, _ = _make(tmp_path, cfg, 21)
+    ids = _prompt(cfg, batch, prompt, 21)
+    model = QuantGpt(path, batch)
+    rec = torch.zeros(new, batch, cfg["vocab"], dtype=torch.int8, device=DEV)
+    model.set_step_record(rec, new)
+    model.benchmark_mode(True)   # no early stop: all 128 steps run
+    out = model.sample(ids)
+    steps = model.steps_run()
+    assert steps == new and out.shape == (batch, prompt + new)
+    np.testing.assert_array_equal(out[:, :prompt], ids)
+    logits = rec.cpu().numpy()
+    gen = out[:, prompt:]
+    eos = cfg["eos_id"]
+    done = np.zeros(batch, bool)
+    for t in range(steps):
+        want = logits[t].astype(np.int32).argmax(axis=1)   # numpy: first maximum = lowest id
+        live = ~done
+        np.testing.assert_array_equal(gen[live, t], want[live], err_msg="step %d" % t)
+        assert (gen[done, t] == eos).all()                  # finished rows stay on <eos>
+        done |= gen[:, t] == eos
+    # deterministic; the record of a second run is the same bytes
+    rec2 = torch.zeros_like(rec)
+    model.set_step_record(rec2, new)
+    out2 = model.sample(ids)
+    np.testing.assert_array_equal(out2, out)
+    assert torch.equal(rec, rec2)
+    # a sequence does not depend on the rest of its batch
+    model.set_step_record(None, 0)
+    sub = model.sample(ids[5:8])
+    np.testing.assert_array_equal(sub, out[5:8])
+    model.close()

@@ -241,3 +241,83 @@ def test_transformer_big_shape(oracle, tmp_path):
     gpu = _run_gpu(path, cfg, ids, max_batch=4)
     _, frac = _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
     print("transformer-big shape: %d steps, %.3f%% logit codes differ" % (gpu["steps"], 100 * frac))
+
+
+def test_transformer_big_full_size_properties(oracle, tmp_path):
+    """The translation benchmark at its stated size -- 6 + 6 layers, hidden 1024, 16 heads,
+    inner 4096, vocabulary 32000, batch 16 x beam 4, source length 64, 64 decoding steps --
+    through QuantTransformer.  The oracle's decoder would take minutes here; the run is held
+    to what must be true at any size: replaying the search kernels of the oracle over the
+    recorded logits reproduces every step's sequences, the final ids and the scores of finished
+    beams, the run is deterministic, and a sentence does not depend on the rest of its batch."""
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import QuantTransformer
+    cfg = synthetic.transformer_config("transformer_big")
+    batch, src_len, steps_wanted = 16, 64, 64
+    assert cfg["n_enc_layer"] == 6 and cfg["n_dec_layer"] == 6 and cfg["beam_size"] == 4
+    cfg.update(max_step=128, extra_decode_length=steps_wanted + 2 - src_len)
+    path, msg = _make(tmp_path, cfg, 31)
+    ids = _src_ids(cfg, batch, src_len, 31)
+    ids[ids == cfg["padding_id"]] = 7   # full-length sources, as the benchmark uses
+    beam, V, max_step = cfg["beam_size"], cfg["trg_vocab"], cfg["max_step"]
+    rows = batch * beam
+    model = QuantTransformer(path, batch)
+    rec_l = torch.zeros(steps_wanted, rows, V, dtype=torch.int8, device=DEV)
+    rec_a = torch.zeros(steps_wanted, rows, max_step, dtype=torch.int32, device=DEV)
+    model.set_step_record(rec_l, rec_a, steps_wanted)
+    model.benchmark_mode(True)   # no early stop: all 64 steps run
+    tokens, scores = model.infer(ids)
+    steps = model.steps_run()
+    assert steps == steps_wanted and tokens.shape[:2] == (batch, beam)
+    logits, alive_rec = rec_l.cpu().numpy(), rec_a.cpu().numpy()
+
+    # replay of the search over the recorded logits with the oracle's kernels
+    # (select_beam_rough_topk -> scan + sort -> refresh_result: model/quant_decoder.cc.cu:988-1057)
+    _, dec_w = _oracle_weights(msg, cfg)
+    bias = np.ascontiguousarray(dec_w["logit_bias"])
+    dq = dec_w["logits_clip_max"] / 127
+    end_id = dec_w["end_id"]
+    alive = np.full((rows, max_step), dec_w["start_id"], np.int32)
+    probs = np.where(np.arange(rows) % beam == 0, 0.0, -1000.0).astype(np.float32)
+    score = np.zeros(rows, np.float32)
+    live = np.zeros((steps, rows), bool)   # beams that have not ended before step t
+    for t in range(steps):
+        live[t] = alive[:, t] != end_id
+        ln = oracle.length_norm(t + 1, cfg["length_penalty"]) if cfg["length_penalty"] >= 0 else 1.0
+        idx, sc, num = oracle.select_beam_rough_topk_i8I(logits[t], bias, probs, score, alive, dq, ln,
+                                                         t, 1024, beam, end_id)
+        s_idx, s_sc, s_num = oracle.scan_sort_candidates(idx, sc, num)
+        alive, probs, score, _fin = oracle.refresh_result(s_idx, s_sc, s_num, alive, probs, score, V, t,
+                                                          ln, end_id, beam)
+        np.testing.assert_array_equal(alive_rec[t][:, :t + 2], alive[:, :t + 2], err_msg="step %d" % t)
+    # the output writer over the replayed state (ker_write_topk_result) gives the model's output
+    want_tok, want_sc = oracle.write_topk_result(alive, score, beam, end_id, tokens.shape[2])
+    np.testing.assert_array_equal(tokens.reshape(rows, -1), want_tok)
+    finished = (alive[:, 1:steps + 1] == end_id).any(axis=1)
+    np.testing.assert_allclose(scores.reshape(-1)[finished], want_sc[finished], rtol=2e-6, atol=2e-4)
+    # nothing was written past the decoded length
+    assert (alive_rec[steps - 1][:, steps + 1:] == alive_rec[0][:, steps + 1:]).all()
+
+    # deterministic, same bytes in the record of a second run
+    rec_l2 = torch.zeros_like(rec_l)
+    model.set_step_record(rec_l2, rec_a, steps_wanted)
+    tokens2, scores2 = model.infer(ids)
+    np.testing.assert_array_equal(tokens2, tokens)
+    # (scores of unfinished beams are whatever the score buffer held, as in the reference)
+    np.testing.assert_array_equal(scores2.reshape(-1)[finished], scores.reshape(-1)[finished])
+    # logits of live beams are the same bytes; an ended beam keeps being stepped, but the cache
+    # reorder skips it (as ker_refresh_cache does), so its row reads stale cache lines and its
+    # logits, which nothing consumes, are not reproducible
+    assert live.sum() > 0.5 * live.size
+    l2 = rec_l2.cpu().numpy()
+    for t in range(steps):
+        np.testing.assert_array_equal(l2[t][live[t]], logits[t][live[t]], err_msg="step %d" % t)
+    # a sentence does not depend on the rest of its batch
+    model.set_step_record(None, None, 0)
+    sub, sub_sc = model.infer(ids[3:6])
+    np.testing.assert_array_equal(sub, tokens[3:6])
+    fin_sub = finished.reshape(batch, beam)[3:6]
+    # a finished beam's score carries its sentence's offset of -2000 per batch index
+    off = 2000.0 * (np.arange(batch)[3:6, None] - np.arange(3)[:, None])
+    np.testing.assert_allclose((sub_sc - off)[fin_sub], scores[3:6][fin_sub], rtol=1e-6, atol=1e-3)
+    model.close()
