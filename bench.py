@@ -446,7 +446,11 @@ def bench_generation(args):
                 "greedy, random-init weights")
     os.remove(path)
     model.benchmark_mode(True)
+    model.graph_mode(args.graphs)
     model._upload(ids)
+    if args.graphs:
+        for _ in range(2):  # first call: keys seen; second: graphs captured
+            model.infer_device()
     for _ in range(args.warmup):
         model.infer_device()
     torch.cuda.synchronize()
@@ -466,7 +470,7 @@ def bench_generation(args):
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": desc, "batch": batch, "source_len": src_len,
                    "decode_steps": steps_run, "ms_per_decode_step": 1e3 * dt / args.steps / steps_run,
-                   "entry_point": entry},
+                   "hip_graph_steps": bool(args.graphs), "entry_point": entry},
         "roofline": None,
     }
 
@@ -481,9 +485,12 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true",
                     help="skip the stand-alone timing of the fused kernels")
+    ap.add_argument("--graphs", action="store_true",
+                    help="generation workloads: replay the steps as HIP graphs (ls_model_set_graph_mode)")
     ap.add_argument("--copy-calibration", action="store_true",
-                    help="also run three plain 256 MiB device copies, a kernel of known HBM "
-                         "traffic against which profiler byte counters are scaled")
+                    help="also run three plain 256 MiB device copies (dst = src + 1, one elementwise "
+                         "kernel each), a kernel of known HBM traffic against which profiler byte "
+                         "counters are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU only (every model object owns device 0 and "
@@ -498,10 +505,11 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     if args.copy_calibration:
+        # an elementwise kernel (not a copy engine): reads 256 MiB, writes 256 MiB
         src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda:0")
         dst = torch.empty_like(src)
         for _ in range(3):
-            dst.copy_(src)
+            torch.add(src, 1, out=dst)
         torch.cuda.synchronize()
     out = bench_bert(args) if bert else bench_generation(args)
     print(json.dumps(out))

@@ -85,6 +85,17 @@ int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst);
  * NULL).  ls_model_get_steps_run gives the number of steps the last Infer() ran. */
 int ls_model_set_step_record(ls_model* model, int8_t* logits, int* alive_seq, int max_steps);
 int ls_model_get_steps_run(ls_model* model, int* steps);
+/* No counterpart in the reference (its step loops launch kernel by kernel:
+ * model/quant_decoder.cc.cu:446-454, quant_gpt_encoder.cc.cu:361-389).  QuantTransformer and
+ * QuantGpt: when on, every generation step -- embedding, the layer stack, the logits GEMM, the
+ * search / sampling kernels and the cache reorder -- is replayed as one HIP graph.  A step's
+ * launches depend only on the shapes of the call and the step's position, so graphs are kept
+ * per (batch size, source or prompt length, step): the first call with a key runs eagerly, the
+ * second captures, later ones replay.  The early-stop word is read back between replays as
+ * before.  Ignored while a step record is set.  Results are identical either way.
+ * ls_model_get_graph_stats: graphs captured so far, steps replayed so far. */
+int ls_model_set_graph_mode(ls_model* model, int on);
+int ls_model_get_graph_stats(ls_model* model, int* captured, long long* replayed);
 
 #ifdef __cplusplus
 }

@@ -31,6 +31,8 @@ template <typename T>
 int quantize_transpose(const T* input, int8_t* output, int rows, int cols, float quant_scale,
                        bool transpose, hipStream_t s);
 // stored uint8 (= code + 127) kernels -> int8 codes (optionally transposed) / T values
+// p[0..n) = value by a kernel (graph-capture safe, unlike hipMemsetAsync here)
+int fill_i32(int* p, int value, int n, hipStream_t s);
 int stored_u8_to_i8(const uint8_t* input, int8_t* output, int rows, int cols, bool transpose,
                     hipStream_t s);
 template <typename T>

@@ -254,6 +254,37 @@ int ls_model_set_step_record(ls_model* model, int8_t* logits, int* alive_seq, in
   return LSH_OK;
 }
 
+int ls_model_set_graph_mode(ls_model* model, int on) {
+  NEED_MODEL(model);
+  if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get())) {
+    qg->encoder()->graph_mode(on != 0);
+    return LSH_OK;
+  }
+  if (QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get())) {
+    qt->decoder()->graph_mode(on != 0);
+    return LSH_OK;
+  }
+  return lsh::lsh_fail(LSH_ERR_UNSUPPORTED,
+                       "graph mode applies to the generation steps of QuantTransformer and QuantGpt");
+}
+
+int ls_model_get_graph_stats(ls_model* model, int* captured, long long* replayed) {
+  NEED_MODEL(model);
+  if (!captured || !replayed) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");
+  if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get())) {
+    *captured = qg->encoder()->graphs_captured();
+    *replayed = qg->encoder()->graphs_replayed();
+    return LSH_OK;
+  }
+  if (QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get())) {
+    *captured = qt->decoder()->graphs_captured();
+    *replayed = qt->decoder()->graphs_replayed();
+    return LSH_OK;
+  }
+  return lsh::lsh_fail(LSH_ERR_UNSUPPORTED,
+                       "graph mode applies to the generation steps of QuantTransformer and QuantGpt");
+}
+
 int ls_model_get_steps_run(ls_model* model, int* steps) {
   NEED_MODEL(model);
   if (!steps) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");

@@ -6,8 +6,11 @@
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
 #include <stdexcept>
 #include <string>
+#include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
 #include "../ls_launch.h"
@@ -63,6 +66,77 @@ class DeviceBuffer {
   }
   T* p_ = nullptr;
   size_t n_ = 0;
+};
+
+// HIP graphs of a generation step.  A step is a fixed sequence of launches whose arguments
+// depend only on the shapes of the call and on the position of the step, so the sequence
+// enqueued for one key is the sequence for every later call with that key.
+//   first time a key is seen   the step runs eagerly (kernel attributes get set, nothing is kept)
+//   second time                the step is captured from the stream, instantiated and launched
+//   later                      one hipGraphLaunch
+// The body may only enqueue kernels and device-to-device copies on the stream: no memset nodes
+// (they replay wrongly on this platform), no synchronisation, no host reads.
+class StepGraphs {
+ public:
+  StepGraphs() {}
+  StepGraphs(const StepGraphs&) = delete;
+  StepGraphs& operator=(const StepGraphs&) = delete;
+  ~StepGraphs() { clear(); }
+  void clear() {
+    for (auto& kv : execs_) (void)hipGraphExecDestroy(kv.second);
+    execs_.clear();
+    seen_.clear();
+  }
+  int captured() const { return captured_; }
+  long replayed() const { return replayed_; }
+
+  template <typename Body>
+  void run(uint64_t key, hipStream_t stream, bool enabled, Body&& body) {
+    if (!enabled) {
+      body();
+      return;
+    }
+    auto it = execs_.find(key);
+    if (it != execs_.end()) {
+      CHECK_GPU_ERROR(hipGraphLaunch(it->second, stream));
+      ++replayed_;
+      return;
+    }
+    if (seen_.insert(key).second) {  // first encounter
+      body();
+      return;
+    }
+    if (execs_.size() >= kMaxGraphs) clear_execs();
+    hipGraph_t graph = nullptr;
+    CHECK_GPU_ERROR(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    try {
+      body();
+    } catch (...) {
+      (void)hipStreamEndCapture(stream, &graph);
+      if (graph) (void)hipGraphDestroy(graph);
+      throw;
+    }
+    CHECK_GPU_ERROR(hipStreamEndCapture(stream, &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    CHECK_GPU_ERROR(e);
+    execs_[key] = exec;
+    ++captured_;
+    CHECK_GPU_ERROR(hipGraphLaunch(exec, stream));
+    ++replayed_;
+  }
+
+ private:
+  void clear_execs() {
+    for (auto& kv : execs_) (void)hipGraphExecDestroy(kv.second);
+    execs_.clear();
+  }
+  static constexpr size_t kMaxGraphs = 4096;
+  std::unordered_map<uint64_t, hipGraphExec_t> execs_;
+  std::unordered_set<uint64_t> seen_;
+  int captured_ = 0;
+  long replayed_ = 0;
 };
 
 inline std::vector<__half> to_half(const std::vector<float>& v) {

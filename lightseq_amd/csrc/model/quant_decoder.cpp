@@ -202,6 +202,11 @@ void QuantDecoder::run_one_infer(int batch_size, int batch_seq_len) {
   _batch_max_decode_length =
       std::min(_tw._max_step, batch_seq_len + _tw._extra_decode_length) - 1;
   _steps_run = 0;
+  // every call starts from the same halves of the double-buffered sequences and caches (column
+  // 0 of both sequence buffers holds the start token; everything else is rewritten as the
+  // steps go), so that a step's launches are the same from call to call
+  _alive_cur = 0;
+  _cache_cur = 0;
 
   project_encoder_output();
   CHECK_GPU_ERROR(hipMemcpyAsync(_alive_seq_probs.get(), _h_alive_seq_probs.data(),
@@ -247,6 +252,27 @@ void QuantDecoder::project_encoder_output() {
 }
 
 bool QuantDecoder::run_step() {
+  // The launches of a step depend on the shapes of the call, the step index and which of the
+  // two sequence / cache buffers is current: one graph per such key.
+  const uint64_t key = ((uint64_t)_batch_size << 40) | ((uint64_t)_batch_seq_len << 24) |
+                       ((uint64_t)_cur_step << 8) | (uint64_t)(_alive_cur << 1 | _cache_cur);
+  _graphs.run(key, _stream, _use_graphs && !_rec_logits && !_rec_alive, [&] { enqueue_step(); });
+  ++_steps_run;
+  _alive_cur ^= 1;
+  if (_cur_step > 0) _cache_cur ^= 1;
+  if (!_is_benchmark) {
+    // the one device-to-host word of a step: all beams finished -> stop early
+    CHECK_GPU_ERROR(hipMemcpyAsync(_h_num_finished, _num_finished.get(), sizeof(int),
+                                   hipMemcpyDeviceToHost, _stream));
+    CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+    if (*_h_num_finished == _step_token_num) return true;
+  }
+  return false;
+}
+
+// everything a step puts on the stream: embedding, the layer stack, the logits, the search
+// and the cache reorder (kernels and device-to-device copies only, so that it can be captured)
+void QuantDecoder::enqueue_step() {
   LnFewRowsScope few_rows;  // every step of every batch size: layer norms by the row kernel
   embedding();
   for (_layer_id = 0; _layer_id < _tw._n_dec_layer; _layer_id++) {
@@ -263,8 +289,7 @@ bool QuantDecoder::run_step() {
     CHECK_GPU_ERROR(hipMemcpyAsync(
         _rec_logits + (size_t)_cur_step * _step_token_num * _tw._trg_vocab_size, _logits.get(),
         (size_t)_step_token_num * _tw._trg_vocab_size, hipMemcpyDeviceToDevice, _stream));
-  ++_steps_run;
-  return beam_search();
+  beam_search();
 }
 
 void QuantDecoder::embedding() {
@@ -382,7 +407,7 @@ void QuantDecoder::ffn_add_norm() {
       w.ffn2_colsum.get(), nparts, (long)M * H)));
 }
 
-bool QuantDecoder::beam_search() {
+void QuantDecoder::beam_search() {
   int* alive = _alive_seq[_alive_cur].get();
   int* alive_new = _alive_seq[_alive_cur ^ 1].get();
   LSH_CALL(beam_search_step_i8I<__half>(
@@ -390,21 +415,13 @@ bool QuantDecoder::beam_search() {
       alive_new, _top_score.get(), _top_idx.get(), _parent.get(), _num_finished.get(),
       _logits_clip_max / _quant_range, _tw._trg_vocab_size, _tw._max_step,
       _h_length_norm[_cur_step], _cur_step, _batch_size, _tw._beam_size, _tw._end_id, _stream));
-  _alive_cur ^= 1;
   if (_rec_alive && _cur_step < _rec_max_steps)
     CHECK_GPU_ERROR(hipMemcpyAsync(
         _rec_alive + (size_t)_cur_step * _step_token_num * _tw._max_step, alive_new,
         (size_t)_step_token_num * _tw._max_step * sizeof(int), hipMemcpyDeviceToDevice, _stream));
 
-  if (!_is_benchmark) {
-    // the one device-to-host word of a step: all beams finished -> stop early
-    CHECK_GPU_ERROR(hipMemcpyAsync(_h_num_finished, _num_finished.get(), sizeof(int),
-                                   hipMemcpyDeviceToHost, _stream));
-    CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
-    if (*_h_num_finished == _step_token_num) return true;
-  }
-
-  /* ---refresh cache: k, v for decoder self attention--- */
+  /* ---refresh cache: k, v for decoder self attention--- (also on a step that turns out to be
+   * the last one: the early-stop test reads the finished count after the step) */
   if (_cur_step > 0) {
     LSH_CALL(refresh_cache_by_parent_i8(
         _tw._n_dec_layer, _step_token_num, _stream, _parent.get(),
@@ -412,9 +429,7 @@ bool QuantDecoder::beam_search() {
         _self_k_cache[_cache_cur ^ 1].get(), _self_v_cache[_cache_cur ^ 1].get(),
         _layer_size_self_k, _tw._beam_size, _tw._dim_per_head, _tw._head_num, _cur_step,
         _tw._max_step));
-    _cache_cur ^= 1;
   }
-  return false;
 }
 
 }  // namespace hip

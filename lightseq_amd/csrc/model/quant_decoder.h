@@ -41,6 +41,11 @@ class QuantDecoder {
     _rec_max_steps = max_steps;
   }
   int steps_run() const { return _steps_run; }
+  // Replay decoding steps through HIP graphs, one per (batch, source length, step, buffer
+  // parity): see StepGraphs.  Off while a step record is set.
+  void graph_mode(bool on) { _use_graphs = on; }
+  int graphs_captured() const { return _graphs.captured(); }
+  long graphs_replayed() const { return _graphs.replayed(); }
 
   const int* _p_d_padding_mask;
   const __half* _p_d_encoder_output;
@@ -56,7 +61,8 @@ class QuantDecoder {
   void self_attention();
   void encdec_attention();
   void ffn_add_norm();
-  bool beam_search();
+  void enqueue_step();
+  void beam_search();
 
   const int _max_batch_size;
   QuantTransformerWeight& _tw;
@@ -65,6 +71,8 @@ class QuantDecoder {
   const float _trg_emb_clip_max, _output_ln_clip_max, _logits_clip_max;
   const std::vector<float> _dec_clip_max;
   bool _is_benchmark = false;
+  bool _use_graphs = false;
+  StepGraphs _graphs;
 
   int _batch_size = 0, _batch_seq_len = 0, _batch_token_num = 0, _step_token_num = 0;
   int _batch_max_decode_length = 0, _layer_id = 0, _steps_run = 0;

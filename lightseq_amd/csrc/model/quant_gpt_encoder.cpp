@@ -182,8 +182,9 @@ void QuantGptEncoder::prompt_pass(const int* ids) {
   }
 }
 
-// one cached step for the tokens in _last_ids at position _batch_seq_len - 1 (:363-377)
-void QuantGptEncoder::step_pass() {
+// one cached step for the tokens in _last_ids at position _batch_seq_len - 1 (:363-377);
+// returns the buffer that holds the int8 LayerNorm output of the last layer [batch, hidden]
+const int8_t* QuantGptEncoder::step_pass() {
   LnFewRowsScope few_rows;  // every step of every batch size: layer norms by the row kernel
   const int H = _tw._hidden_size, B = _batch_size;
   const float Q = _quant_range;
@@ -225,22 +226,26 @@ void QuantGptEncoder::step_pass() {
     ffn_add_norm(B, b, a);
     std::swap(a, b);  // `a` names the buffer holding the layer's int8 LayerNorm output
   }
-  CHECK_GPU_ERROR(hipMemcpyAsync(_hid_last.get(), a, (size_t)B * H, hipMemcpyDeviceToDevice,
-                                 _stream));
+  return a;
 }
 
-// logits of the last position + greedy choice; returns the unfinished flag (:399-487)
-int QuantGptEncoder::sample_one_token() {
+// logits of the last position + greedy choice, enqueued only (:399-487)
+void QuantGptEncoder::enqueue_sampling(const int8_t* hidden) {
   const int H = _tw._hidden_size, V = _tw._src_vocab_size, B = _batch_size;
-  LSH_CALL(gemm_i8_i8o(_hid_last.get(), _int8_emb.get(), _logits.get(), B, V, H,
+  LSH_CALL(gemm_i8_i8o(hidden, _int8_emb.get(), _logits.get(), B, V, H,
                        _output_ln_clip_max * _src_emb_clip_max / (_logits_clip_max * _quant_range),
                        _stream));
   if (_rec_logits && _steps_run < _rec_max_steps)
     CHECK_GPU_ERROR(hipMemcpyAsync(_rec_logits + (size_t)_steps_run * B * V, _logits.get(),
                                    (size_t)B * V, hipMemcpyDeviceToDevice, _stream));
-  CHECK_GPU_ERROR(hipMemsetAsync(_unfinished.get(), 0, sizeof(int), _stream));
+  LSH_CALL(fill_i32(_unfinished.get(), 0, 1, _stream));
   LSH_CALL(gpt_greedy_step(_logits.get(), _ids.get(), _last_ids.get(), V, _tw._max_step,
                            _batch_seq_len, B, _unfinished.get(), _tw._eos_id, _stream));
+}
+
+// host side of a sampled token: counters and the unfinished flag (one word back from the device)
+int QuantGptEncoder::finish_token() {
+  const int B = _batch_size;
   const bool first = _steps_run == 0;
   ++_steps_run;
   _batch_seq_len++;
@@ -279,10 +284,14 @@ int QuantGptEncoder::run_one_sample(int batch_size, int batch_seq_len) {
                                    hipMemcpyDeviceToDevice, _stream));
   if (_batch_seq_len < _tw._max_step) {
     // (:347-353) after the prompt pass the run ends when nothing is unfinished
-    if (!(sample_one_token() == 0 || _batch_seq_len >= _batch_max_seq_len)) {
+    enqueue_sampling(_hid_last.get());
+    if (!(finish_token() == 0 || _batch_seq_len >= _batch_max_seq_len)) {
       while (_batch_seq_len < _batch_max_seq_len) {
-        step_pass();
-        int unfinished = sample_one_token();
+        // the launches of a step depend on the batch size and the position only
+        const uint64_t key = ((uint64_t)_batch_size << 32) | (uint32_t)_batch_seq_len;
+        _graphs.run(key, _stream, _use_graphs && !_rec_logits,
+                    [&] { enqueue_sampling(step_pass()); });
+        int unfinished = finish_token();
         if (!unfinished && !_is_benchmark) break;
       }
     }

@@ -41,6 +41,11 @@ class QuantGptEncoder {
     _rec_max_steps = max_steps;
   }
   int steps_run() const { return _steps_run; }
+  // Replay the cached steps through HIP graphs, one per (batch size, position): see StepGraphs.
+  // Off while a step record is set.
+  void graph_mode(bool on) { _use_graphs = on; }
+  int graphs_captured() const { return _graphs.captured(); }
+  long graphs_replayed() const { return _graphs.replayed(); }
 
   const int* _p_d_token_id;
   float* _p_d_ppl;
@@ -48,9 +53,10 @@ class QuantGptEncoder {
 
  private:
   void prompt_pass(const int* ids);
-  void step_pass();
+  const int8_t* step_pass();
   void ffn_add_norm(int rows, int8_t* in, int8_t* tmp);
-  int sample_one_token();
+  void enqueue_sampling(const int8_t* hidden);
+  int finish_token();
 
   const int _max_batch_size;
   const QuantGptWeight& _tw;
@@ -60,6 +66,8 @@ class QuantGptEncoder {
   const std::vector<float> _enc_clip_max;
   const float _atten_scaler;
   bool _is_benchmark = false;
+  bool _use_graphs = false;
+  StepGraphs _graphs;
 
   int _batch_size = 0, _batch_seq_len = 0, _batch_token_num = 0, _batch_max_seq_len = 0;
   int _layer_id = 0, _steps_run = 0;

@@ -220,6 +220,18 @@ int stored_u8_dequant(const uint8_t* input, T* output, long n, float clip_max, h
 template int stored_u8_dequant<float>(const uint8_t*, float*, long, float, hipStream_t);
 template int stored_u8_dequant<__half>(const uint8_t*, __half*, long, float, hipStream_t);
 
+// A fill kernel for the words a generation step must clear: a memset node in a captured
+// graph replays wrongly on this platform, a kernel node does not.
+__global__ void fill_i32_kernel(int* __restrict__ p, int value, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = value;
+}
+int fill_i32(int* p, int value, int n, hipStream_t s) {
+  if (!p || n <= 0) return lsh_fail(LSH_ERR_INVALID, "fill_i32: bad arguments");
+  fill_i32_kernel<<<(n + 255) / 256, 256, 0, s>>>(p, value, n);
+  return lsh_check_launch("fill_i32_kernel");
+}
+
 #define LSH_INST(T)                                                                          \
   template int quantize_tensor<T>(const T*, int8_t*, long, float, hipStream_t);              \
   template int dequantize_tensor<T>(const int32_t*, T*, long, float, hipStream_t);           \

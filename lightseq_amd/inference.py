@@ -56,6 +56,8 @@ def _bind():
         "ls_model_get_profile": [_P, ctypes.c_char_p, _I],
         "ls_model_set_step_record": [_P, _P, _P, _I],
         "ls_model_get_steps_run": [_P, ip],
+        "ls_model_set_graph_mode": [_P, _I],
+        "ls_model_get_graph_stats": [_P, ip, ctypes.POINTER(ctypes.c_longlong)],
     }
     for name, argtypes in sigs.items():
         fn = getattr(L, name)
@@ -169,6 +171,16 @@ class LSModel:
         buf = ctypes.create_string_buffer(8192)
         self._call("ls_model_get_profile", self._h, buf, 8192)
         return json.loads(buf.value.decode())
+
+    def graph_mode(self, flag):
+        """QuantTransformer / QuantGpt: replay generation steps as HIP graphs."""
+        self._call("ls_model_set_graph_mode", self._h, int(bool(flag)))
+
+    def graph_stats(self):
+        """(graphs captured, steps replayed) so far."""
+        cap, rep = ctypes.c_int(0), ctypes.c_longlong(0)
+        self._call("ls_model_get_graph_stats", self._h, ctypes.byref(cap), ctypes.byref(rep))
+        return cap.value, rep.value
 
     def set_tap(self, layer, name, tensor):
         self._call("ls_model_set_tap", self._h, int(layer), name.encode(),

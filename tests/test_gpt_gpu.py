@@ -384,4 +384,47 @@ def test_gpt2_medium_full_size_properties(tmp_path):
     model.set_step_record(None, 0)
     sub = model.sample(ids[5:8])
     np.testing.assert_array_equal(sub, out[5:8])
+    # the steps replayed as HIP graphs (seen, captured, replayed twice) give the same tokens
+    model.graph_mode(True)
+    for rep in range(4):
+        np.testing.assert_array_equal(model.sample(ids), out, err_msg="graph run %d" % rep)
+    captured, replayed = model.graph_stats()
+    assert captured == new - 1 and replayed == 3 * captured, (captured, replayed)
+    model.close()
+
+
+@pytest.mark.parametrize("benchmark", [False, True])
+def test_graph_replay_of_the_steps_equals_eager(tmp_path, benchmark):
+    """Steps replayed as HIP graphs give the eager run's tokens: several replays, with eager work
+    of this program (another batch shape, a torch kernel, synchronisations) between them."""
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import QuantGpt
+    cfg = synthetic.gpt_config("tiny")
+    path, _ = _make(tmp_path, cfg, 5, w_std=0.2)
+    ids = _prompt(cfg, 3, 9, 5)
+    other = _prompt(cfg, 2, 6, 6)
+    model = QuantGpt(path, 4)
+    model.benchmark_mode(benchmark)
+    want, want_other = model.sample(ids), model.sample(other)
+    steps = model.steps_run()
+    model.graph_mode(True)
+    scratch = torch.zeros(1 << 16, device=DEV)
+    for rep in range(5):       # 1st: eager (keys seen), 2nd: capture + launch, then replays
+        got = model.sample(ids)
+        np.testing.assert_array_equal(got, want, err_msg="replay %d" % rep)
+        scratch.add_(1.0)
+        torch.cuda.synchronize()
+        if rep % 2 == 0:
+            np.testing.assert_array_equal(model.sample(other), want_other)
+    captured, replayed = model.graph_stats()
+    assert captured >= 1 and replayed >= 3 * captured, (captured, replayed)
+    # recording switches the graphs off and still gives the same tokens
+    rec = torch.zeros(cfg["max_step"], 3, cfg["vocab"], dtype=torch.int8, device=DEV)
+    model.set_step_record(rec, cfg["max_step"])
+    np.testing.assert_array_equal(model.sample(ids), want)
+    assert model.graph_stats()[1] == replayed
+    model.graph_mode(False)
+    model.set_step_record(None, 0)
+    np.testing.assert_array_equal(model.sample(ids), want)
+    assert steps >= 1
     model.close()

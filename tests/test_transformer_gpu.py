@@ -320,4 +320,42 @@ def test_transformer_big_full_size_properties(oracle, tmp_path):
     # a finished beam's score carries its sentence's offset of -2000 per batch index
     off = 2000.0 * (np.arange(batch)[3:6, None] - np.arange(3)[:, None])
     np.testing.assert_allclose((sub_sc - off)[fin_sub], scores[3:6][fin_sub], rtol=1e-6, atol=1e-3)
+    # the steps replayed as HIP graphs (seen, captured, replayed twice) give the same beams
+    model.graph_mode(True)
+    for rep in range(4):
+        tg, sg = model.infer(ids)
+        np.testing.assert_array_equal(tg, tokens, err_msg="graph run %d" % rep)
+        np.testing.assert_array_equal(sg.reshape(-1)[finished], scores.reshape(-1)[finished])
+    captured, replayed = model.graph_stats()
+    assert captured >= steps and replayed >= 2 * steps, (captured, replayed)
+    model.close()
+
+
+@pytest.mark.parametrize("benchmark", [False, True])
+def test_graph_replay_of_the_steps_equals_eager(tmp_path, benchmark):
+    """Decoding steps replayed as HIP graphs give the eager run's beams: several replays, with
+    eager work of this program (another batch shape, a torch kernel, synchronisations) between."""
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import QuantTransformer
+    cfg = synthetic.transformer_config("tiny")
+    sigma = 0.02 * np.sqrt(cfg["hidden"])
+    path, _ = _make(tmp_path, cfg, 9, eos_bias=2.0 * sigma, w_std=0.2)
+    ids, other = _src_ids(cfg, 3, 10, 4), _src_ids(cfg, 2, 7, 5)
+    model = QuantTransformer(path, 4)
+    model.benchmark_mode(benchmark)
+    want, _ = model.infer(ids)
+    want_other, _ = model.infer(other)
+    model.graph_mode(True)
+    scratch = torch.zeros(1 << 16, device=DEV)
+    for rep in range(6):
+        got, _ = model.infer(ids)
+        np.testing.assert_array_equal(got, want, err_msg="replay %d" % rep)
+        scratch.add_(1.0)
+        torch.cuda.synchronize()
+        if rep % 2 == 0:
+            np.testing.assert_array_equal(model.infer(other)[0], want_other)
+    captured, replayed = model.graph_stats()
+    assert captured >= 1 and replayed >= 3 * captured, (captured, replayed)
+    model.graph_mode(False)
+    np.testing.assert_array_equal(model.infer(ids)[0], want)
     model.close()
