@@ -235,6 +235,20 @@ int lsh_layer_norm_row_kernel(int on);
  * one against the other.  No counterpart in the reference (its cuBLASLt algorithm table
  * plays this part: model/cublas_algo_map.cc). */
 int lsh_gemm_i8_tile_kernel(int on);
+/* The attention out-projection and the LayerNorm after it as one kernel: what
+ * lsh_gemm_i8_i8o(A, W, alpha) followed by lsh_ker_residual_bias_ln_i8I_i8O_f16 leaves in
+ * `output` (int8 [batch_tokens, hidden_size]) and `residual`, byte for byte (the product is
+ * requantised to its int8 code before the dequant + residual, as
+ * inference/model/quant_bert_encoder.cc.cu:361-396 does), without the int8 product ever
+ * reaching memory.  hidden_size == k in {512, 768, 1024}; w_tiled is W [hidden_size, k]
+ * re-ordered once by lsh_tile_weight_16x64 (blocks of 16 rows x 64 bytes in MFMA lane order).
+ * No counterpart in the reference. */
+int lsh_tile_weight_16x64(const int8_t* w, int8_t* tiled, int n, int k, lsh_stream_t stream);
+int lsh_gemm_i8_residual_ln_i8O_f16(const int8_t* A, const int8_t* w_tiled, float alpha,
+                                    const void* scale, const void* bias, const void* residual_bias,
+                                    int8_t* output, void* residual, int batch_tokens,
+                                    int hidden_size, int k, float dequant_scale, float quant_scale,
+                                    lsh_stream_t stream, int is_post_ln);
 /* Measurement aid, no counterpart in the reference: one launch of `workgroups` x 4 wavefronts
  * that issue nothing but independent int8 MFMAs (v_mfma_i32_32x32x32_i8) on register-resident
  * operands, `iters` x 8 each.  out: workgroups * 256 ints (checksums, so that nothing is

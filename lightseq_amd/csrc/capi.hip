@@ -107,6 +107,18 @@ int lsh_launch_dequantize_tensor_f32(const int32_t* input, void* output, int bat
 // ---- LayerNorm family --------------------------------------------------------------
 int lsh_layer_norm_row_kernel(int on) { return ln_set_few_rows(on != 0) ? 1 : 0; }
 int lsh_gemm_i8_tile_kernel(int on) { return gemm_i8_enable_tile_kernel(on != 0) ? 1 : 0; }
+int lsh_tile_weight_16x64(const int8_t* w, int8_t* tiled, int n, int k, lsh_stream_t stream) {
+  return tile_weight_16x64(w, tiled, n, k, HS(stream));
+}
+int lsh_gemm_i8_residual_ln_i8O_f16(const int8_t* A, const int8_t* w_tiled, float alpha,
+                                    const void* scale, const void* bias, const void* residual_bias,
+                                    int8_t* output, void* residual, int batch_tokens,
+                                    int hidden_size, int k, float dequant_scale, float quant_scale,
+                                    lsh_stream_t stream, int is_post_ln) {
+  return gemm_i8_residual_ln_i8O<__half>(A, w_tiled, alpha, H(scale), H(bias), H(residual_bias),
+                                         output, HM(residual), batch_tokens, hidden_size, k,
+                                         dequant_scale, quant_scale, HS(stream), is_post_ln != 0);
+}
 int lsh_mfma_i8_peak_probe(int* out, int workgroups, int iters, double* ops, lsh_stream_t stream) {
   return mfma_i8_peak_probe(out, workgroups, iters, ops, HS(stream));
 }

@@ -14,6 +14,8 @@
 #include "ls_device.cuh"
 #include "ls_launch.h"
 
+#include <hip/hip_ext.h>
+
 namespace lsh {
 
 enum LnMode {
@@ -173,18 +175,16 @@ __device__ __forceinline__ float row_sum(float v) {
   return v;
 }
 
+// One row of the 8-wide kernel: `sub` is the lane's index among the LPR lanes of the row,
+// `live` false for a row beyond the tensor (its lanes still take part in the shuffles).
+// gemm_out is read at gemm_out[row * hidden + column] and may point anywhere a flat load
+// reaches (the fused GEMM + LayerNorm kernel passes a tile staged in LDS).
 template <typename T, typename AccT, int MODE, int LPR, int ITER>
-__global__ void __launch_bounds__(256)
-ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
-                int8_t* __restrict__ out_q, const T* __restrict__ scale,
-                const T* __restrict__ bias, const T* __restrict__ residual_bias,
-                const T* __restrict__ colsum, int tokens, int hidden, float dequant_scale,
-                float quant_scale, int is_post_ln, int nparts, long part_stride) {
-  constexpr int RPW = kWave / LPR;
-  const int lane = threadIdx.x & 63;
-  const int sub = lane % LPR;
-  const int row = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPR;
-  const bool live = row < tokens;  // dead rows keep the shuffles convergent
+__device__ __forceinline__ void
+ln_rows8_row(int row, bool live, int sub, const AccT* __restrict__ gemm_out, T* residual, T* out_t,
+             int8_t* __restrict__ out_q, const T* __restrict__ scale, const T* __restrict__ bias,
+             const T* __restrict__ residual_bias, const T* __restrict__ colsum, int hidden,
+             float dequant_scale, float quant_scale, int is_post_ln, int nparts, long part_stride) {
   const long base = (long)(live ? row : 0) * hidden;
 
   float x[ITER][8];
@@ -291,6 +291,123 @@ ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
         st8(residual, base + e, w);
       }
     }
+  }
+}
+
+template <typename T, typename AccT, int MODE, int LPR, int ITER>
+__global__ void __launch_bounds__(256)
+ln_rows8_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
+                int8_t* __restrict__ out_q, const T* __restrict__ scale,
+                const T* __restrict__ bias, const T* __restrict__ residual_bias,
+                const T* __restrict__ colsum, int tokens, int hidden, float dequant_scale,
+                float quant_scale, int is_post_ln, int nparts, long part_stride) {
+  constexpr int RPW = kWave / LPR;
+  const int lane = threadIdx.x & 63;
+  const int row = (blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPR;
+  // dead rows keep the shuffles convergent
+  ln_rows8_row<T, AccT, MODE, LPR, ITER>(row, row < tokens, lane % LPR, gemm_out, residual, out_t,
+                                         out_q, scale, bias, residual_bias, colsum, hidden,
+                                         dequant_scale, quant_scale, is_post_ln, nparts,
+                                         part_stride);
+}
+
+// ---------------------------------------------------------------------------------
+// Out-projection GEMM + dequant + residual + LayerNorm + quant in one kernel, for products
+// whose output is one hidden-size-wide row per token (N = K = hidden in {512, 768, 1024}).
+// Replaces the pair cublasLtMM_withAlgo_i8IO + ker_residual_bias_ln_i8I_i8O
+// (inference/model/quant_bert_encoder.cc.cu:361-396) with the same rounding points -- the
+// product is requantised to its int8 code first, then dequantised, added to the residual and
+// normalised -- and the very row routine of the stand-alone kernel, so the two routes give
+// the same bytes.
+//
+// A workgroup owns 16 token rows and all N columns: 8 wavefronts x NT 16-column blocks,
+// v_mfma_i32_16x16x64_i8 with the weight block as the row operand.  The 16 x K activation
+// panel and the weights are read straight into MFMA registers, three K slices in flight, the
+// weights from a copy tiled at load time so that a wavefront's fragment is 1 KB contiguous.  Nothing goes through LDS but the
+// 16 x N tile of int8 codes handed to the row routine (two rows per wavefront, as it expects).
+// Every workgroup streams the whole weight matrix (it stays in the XCD's L2), which is what
+// bounds the kernel: N * K bytes per compute unit at ~64 B/clk.
+// ---------------------------------------------------------------------------------
+typedef int ln_v4i __attribute__((ext_vector_type(4)));
+
+// [N, K] int8 row-major -> blocks of 16 rows x 64 bytes in MFMA lane order:
+// tiled[((n / 16) * (K / 64) + k / 64) * 1024 + lane * 16 + b] with lane = (k % 64) / 16 * 16 + n % 16
+__global__ void __launch_bounds__(256)
+tile_weight_16x64_kernel(const int8_t* __restrict__ w, int8_t* __restrict__ tiled, int N, int K) {
+  const long chunk = (long)blockIdx.x * 256 + threadIdx.x;  // one 16-byte chunk each
+  const long total = (long)N * K / 16;
+  if (chunk >= total) return;
+  const int lane = (int)(chunk & 63);
+  const long blk = chunk >> 6;
+  const int ks = (int)(blk % (K / 64)), nt = (int)(blk / (K / 64));
+  const int n = nt * 16 + (lane & 15), k = ks * 64 + (lane >> 4) * 16;
+  *reinterpret_cast<ln_v4i*>(tiled + chunk * 16) =
+      *reinterpret_cast<const ln_v4i*>(w + (long)n * K + k);
+}
+
+template <typename T, int NT, int KS, int LPR, int ITER>
+__global__ void __launch_bounds__(512)
+gemm_ln_rows16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ Wt, float alpha,
+                      T* residual, int8_t* __restrict__ out_q, const T* __restrict__ scale,
+                      const T* __restrict__ bias, const T* __restrict__ residual_bias, int tokens,
+                      float dequant_scale, float quant_scale, int is_post_ln) {
+  constexpr int N = 8 * NT * 16, K = KS * 64;
+  __shared__ __align__(16) int8_t codes[16 * N];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r0 = blockIdx.x * 16;
+  // The K slices are walked from a starting slice that differs between the workgroups of an
+  // XCD (workgroup b runs on XCD b % 8), wrapping around: integer sums commute, and workgroups
+  // that all stream the same weight matrix in the same order at the same time would queue up
+  // on the same L2 channel.
+  const int rot = ((int)blockIdx.x >> 3) % KS;
+  // activation fragments: row r0 + lane % 16 (clamped: rows beyond the tensor are never stored)
+  const int8_t* ap = A + (long)min(r0 + (lane & 15), tokens - 1) * K + (lane >> 4) * 16;
+  // weight fragments of this wavefront's NT column blocks
+  const int8_t* wp = Wt + ((long)wave * NT * KS * 64 + lane) * 16;
+  ln_v4i wf[3][NT], af[3];
+  auto load_slice = [&](int i) {  // i-th slice of this workgroup's walk, into ring slot i % 3
+    int ks = i + rot;
+    if (ks >= KS) ks -= KS;
+    af[i % 3] = *reinterpret_cast<const ln_v4i*>(ap + ks * 64);
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      wf[i % 3][t] = *reinterpret_cast<const ln_v4i*>(wp + ((long)t * KS + ks) * 1024);
+  };
+  ln_v4i acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = (ln_v4i)0;
+  load_slice(0);
+  if (KS > 1) load_slice(1);
+  // the scheduling barriers keep the loads of slice i + 2 ahead of the MFMAs of slice i:
+  // left alone, the compiler sinks every load to just before its use and the loop waits for
+  // memory at each step
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < KS; ++i) {
+    if (i + 2 < KS) load_slice(i + 2);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+      acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[i % 3][t], af[i % 3], acc[t], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // lane holds C[token lane % 16][column block * 16 + 4 * (lane / 16) + 0..3]
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int n = (wave * NT + t) * 16 + 4 * (lane >> 4);
+    *reinterpret_cast<uint32_t*>(codes + (lane & 15) * N + n) =
+        requant_acc_pack4(acc[t][0], acc[t][1], acc[t][2], acc[t][3], alpha);
+  }
+  __syncthreads();
+  // the stand-alone kernel's row routine with the lane layout it uses for this hidden size
+  // (LPR lanes per row), fed from the staged codes
+  constexpr int RPW = kWave / LPR;
+#pragma unroll
+  for (int pass = 0; pass < 16 / (8 * RPW); ++pass) {
+    const int row = r0 + (pass * 8 + wave) * RPW + lane / LPR;
+    ln_rows8_row<T, int8_t, kLnResQuant, LPR, ITER>(
+        row, row < tokens, lane % LPR, codes - (long)r0 * N, residual, nullptr, out_q, scale, bias,
+        residual_bias, nullptr, N, dequant_scale, quant_scale, is_post_ln, 1, 0);
   }
 }
 
@@ -520,6 +637,60 @@ static int launch_ln(const AccT* gemm_out, T* residual, T* out_t, int8_t* out_q,
 #undef LSH_LN_CASE
   return lsh_check_launch("ln_rows_kernel");
 }
+
+int tile_weight_16x64(const int8_t* w, int8_t* tiled, int N, int K, hipStream_t s) {
+  if (!w || !tiled || N <= 0 || K <= 0 || N % 16 != 0 || K % 64 != 0 || !aligned16(w) ||
+      !aligned16(tiled))
+    return lsh_fail(LSH_ERR_INVALID, "tile_weight_16x64: needs N % 16 == 0, K % 64 == 0, aligned pointers");
+  const long chunks = (long)N * K / 16;
+  tile_weight_16x64_kernel<<<(int)((chunks + 255) / 256), 256, 0, s>>>(w, tiled, N, K);
+  return lsh_check_launch("tile_weight_16x64_kernel");
+}
+
+static thread_local hipEvent_t g_gln_ev_start = nullptr, g_gln_ev_stop = nullptr;
+void gemm_ln_time_next_launch(hipEvent_t start, hipEvent_t stop) {
+  g_gln_ev_start = start;
+  g_gln_ev_stop = stop;
+}
+
+bool gemm_ln_fused_supported(int hidden, int K) {
+  return hidden == K && (hidden == 512 || hidden == 768 || hidden == 1024);
+}
+
+template <typename T>
+int gemm_i8_residual_ln_i8O(const int8_t* A, const int8_t* w_tiled, float alpha, const T* scale,
+                            const T* bias, const T* residual_bias, int8_t* output, T* residual,
+                            int batch_tokens, int hidden_size, int K, float dequant_scale,
+                            float quant_scale, hipStream_t stream, bool is_post_ln) {
+  if (!A || !w_tiled || !scale || !bias || !output || !residual || batch_tokens <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "gemm_i8_residual_ln_i8O: bad arguments");
+  if (!gemm_ln_fused_supported(hidden_size, K))
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "gemm_i8_residual_ln_i8O: needs hidden == K in {512, 768, 1024}");
+  if (!aligned16(A) || !aligned16(w_tiled) || !aligned16(scale) || !aligned16(bias) ||
+      !aligned16(residual_bias) || !aligned16(output) || !aligned16(residual))
+    return lsh_fail(LSH_ERR_INVALID, "gemm_i8_residual_ln_i8O: pointers must be 16-byte aligned");
+  const int grid = (batch_tokens + 15) / 16;
+  // kernel-exact begin / end timestamps when the caller asked for them
+  hipEvent_t e0 = g_gln_ev_start, e1 = g_gln_ev_stop;
+  g_gln_ev_start = g_gln_ev_stop = nullptr;
+  const int post = is_post_ln ? 1 : 0;
+#define LSH_GLN(NT, KS, LPR, IT)                                                               \
+  hipExtLaunchKernelGGL((gemm_ln_rows16_kernel<T, NT, KS, LPR, IT>), dim3(grid), dim3(512), 0,  \
+                        stream, e0, e1, 0, A, w_tiled, alpha, residual, output, scale, bias,    \
+                        residual_bias, batch_tokens, dequant_scale, quant_scale, post)
+  if (hidden_size == 512) LSH_GLN(4, 8, 32, 2);
+  else if (hidden_size == 768) LSH_GLN(6, 12, 32, 3);
+  else LSH_GLN(8, 16, 64, 2);
+#undef LSH_GLN
+  return lsh_check_launch("gemm_ln_rows16_kernel");
+}
+template int gemm_i8_residual_ln_i8O<__half>(const int8_t*, const int8_t*, float, const __half*,
+                                             const __half*, const __half*, int8_t*, __half*, int,
+                                             int, int, float, float, hipStream_t, bool);
+template int gemm_i8_residual_ln_i8O<float>(const int8_t*, const int8_t*, float, const float*,
+                                            const float*, const float*, int8_t*, float*, int, int,
+                                            int, float, float, hipStream_t, bool);
 
 template <typename T>
 int norm_layer_resual_i8O(int token_num, int hidden_size, hipStream_t stream, T* input,

@@ -106,6 +106,19 @@ int enc_emb_i8I(const int8_t* token_emb, const T* pos_emb, const int* tokens, T*
                 int* pad_mask, int pad_id, int batch_size, int seq_len, int hidden_dim,
                 hipStream_t s, float dequant_scale, bool scaled, int vocab_size);
 
+// ---- out-projection GEMM + residual LayerNorm in one kernel (ln_kernels.hip) -------------
+// [N, K] int8 -> the 16-row x 64-byte MFMA-ordered tiling the fused kernel streams
+int tile_weight_16x64(const int8_t* w, int8_t* tiled, int N, int K, hipStream_t s);
+bool gemm_ln_fused_supported(int hidden, int K);
+// the next fused launch of this thread records its own begin / end timestamps into the events
+void gemm_ln_time_next_launch(hipEvent_t start, hipEvent_t stop);
+// output / residual as residual_bias_ln_i8O would leave them after gemm_i8_i8o(A, W, alpha)
+template <typename T>
+int gemm_i8_residual_ln_i8O(const int8_t* A, const int8_t* w_tiled, float alpha, const T* scale,
+                            const T* bias, const T* residual_bias, int8_t* output, T* residual,
+                            int batch_tokens, int hidden_size, int K, float dequant_scale,
+                            float quant_scale, hipStream_t stream, bool is_post_ln);
+
 // ---- encoder attention (attn_kernels.hip) ------------------------------------------
 template <typename T>
 int correlation_softmax_encself(int batch_size, int batch_seq_len, int head_num, hipStream_t s,

@@ -69,6 +69,10 @@ void QuantBertEncoder::init_buffer() {
     d.b_ffn2 = upload_half(w.ffn_second_bias, _stream);
     d.w_qkv = upload_kernel(w.multihead_project_kernel_qkv, H, 3 * H, true, _stream);
     d.w_out = upload_kernel(w.multihead_project_kernel_output, H, H, true, _stream);
+    if (gemm_ln_fused_supported(H, H)) {
+      d.w_out_tiled.alloc((size_t)H * H);
+      LSH_CALL(tile_weight_16x64(d.w_out.get(), d.w_out_tiled.get(), H, H, _stream));
+    }
     d.w_ffn1 = upload_kernel(w.ffn_first_kernel, H, I, true, _stream);
     d.w_ffn2 = upload_kernel(w.ffn_second_kernel, I, H, true, _stream);
     {
@@ -111,10 +115,11 @@ void QuantBertEncoder::reset_profile() {
 
 void QuantBertEncoder::prof_begin(int site, int m, int n, int k, const char* epilogue) {
   if (!_profiling) return;
+  const bool fused_ln = std::string(epilogue) == "fused_ln";
   SiteProfile& p = _profile[site];
-  if (p.m != m || p.n != n || p.k != k) {
+  if (p.m != m || p.n != n || p.k != k || p.kernel.empty()) {
     p.m = m; p.n = n; p.k = k;
-    p.kernel = gemm_i8_kernel_name(m, n, k, epilogue);
+    p.kernel = fused_ln ? "gemm_ln_rows16_kernel" : gemm_i8_kernel_name(m, n, k, epilogue);
   }
   Pending pe;
   pe.site = site;
@@ -126,8 +131,9 @@ void QuantBertEncoder::prof_begin(int site, int m, int n, int k, const char* epi
       _event_pool.pop_back();
     }
   }
-  // the GEMM launcher records the kernel's own begin / end timestamps into the events
-  gemm_i8_time_next_launch(pe.e0, pe.e1);
+  // the launcher records the kernel's own begin / end timestamps into the events
+  if (fused_ln) gemm_ln_time_next_launch(pe.e0, pe.e1);
+  else gemm_i8_time_next_launch(pe.e0, pe.e1);
   _pending.push_back(pe);
 }
 
@@ -205,18 +211,32 @@ void QuantBertEncoder::self_attention() {
   }
   tap(taps.ctx_q, _int8_ffn_in_buf.get(), (size_t)M * H);
 
-  prof_begin(1, M, H, H, "EpiI8");
-  LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_out.get(), _int8_ffn_out_buf.get(), M, H, H,
-                       c[1] * c[5] / (c[9] * Q), _stream));
-  tap(taps.out_q, _int8_ffn_out_buf.get(), (size_t)M * H);
+  const bool tap_out = (taps.out_q || taps.res_attn) && taps.tap_layer == _layer_id;
+  if (_fuse && !tap_out && w.w_out_tiled.get() != nullptr) {
+    // out-projection + dequant + residual + LayerNorm + quant in one kernel: the int8 product
+    // never reaches memory.  Same bytes as the pair below; reads _int8_ffn_in_buf (context codes)
+    // and must not overwrite it, so the LayerNorm output goes to _int8_ffn_out_buf and the two
+    // buffers swap roles.
+    prof_begin(1, M, H, H, "fused_ln");
+    LSH_CALL(gemm_i8_residual_ln_i8O<__half>(
+        _int8_ffn_in_buf.get(), w.w_out_tiled.get(), c[1] * c[5] / (c[9] * Q), w.ln2_scale.get(),
+        w.ln2_bias.get(), w.b_ffn2.get(), _int8_ffn_out_buf.get(), _p_d_output, M, H, H, c[9] / Q,
+        Q / c[6], _stream, _tw._is_post_ln));
+    std::swap(_int8_ffn_in_buf, _int8_ffn_out_buf);
+  } else {
+    prof_begin(1, M, H, H, "EpiI8");
+    LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_out.get(), _int8_ffn_out_buf.get(), M, H, H,
+                         c[1] * c[5] / (c[9] * Q), _stream));
+    tap(taps.out_q, _int8_ffn_out_buf.get(), (size_t)M * H);
 
-  if (taps.res_attn && taps.tap_layer == _layer_id)
-    CHECK_GPU_ERROR(hipMemcpyAsync(taps.res_attn, _p_d_output, (size_t)M * H * sizeof(__half),
-                                   hipMemcpyDeviceToDevice, _stream));
-  LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(
-      _int8_ffn_out_buf.get(), w.ln2_scale.get(), w.ln2_bias.get(), w.b_ffn2.get(),
-      _int8_ffn_in_buf.get(), _p_d_output, M, H, c[9] / Q, Q / c[6], _stream, _tw._is_post_ln,
-      nullptr)));
+    if (taps.res_attn && taps.tap_layer == _layer_id)
+      CHECK_GPU_ERROR(hipMemcpyAsync(taps.res_attn, _p_d_output, (size_t)M * H * sizeof(__half),
+                                     hipMemcpyDeviceToDevice, _stream));
+    LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(
+        _int8_ffn_out_buf.get(), w.ln2_scale.get(), w.ln2_bias.get(), w.b_ffn2.get(),
+        _int8_ffn_in_buf.get(), _p_d_output, M, H, c[9] / Q, Q / c[6], _stream, _tw._is_post_ln,
+        nullptr)));
+  }
   tap(taps.ln2_q, _int8_ffn_in_buf.get(), (size_t)M * H);
 }
 

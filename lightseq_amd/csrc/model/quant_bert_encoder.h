@@ -87,6 +87,7 @@ class QuantBertEncoder {
   DeviceBuffer<__half> _pos_emb, _final_ln_scale, _final_ln_bias;
   struct Layer {
     DeviceBuffer<int8_t> w_qkv, w_out, w_ffn1, w_ffn2;  // [N, K] int8
+    DeviceBuffer<int8_t> w_out_tiled;  // w_out in 16 x 64 MFMA tiles (fused out-projection + LN)
     DeviceBuffer<int8_t> ffn1_act_lut;  // [inner, 256]: bias + activation + requant per code
     DeviceBuffer<__half> ln1_scale, ln1_bias, b_qkv, b_out, ln2_scale, ln2_bias, b_ffn1, b_ffn2,
         ffn2_colsum;

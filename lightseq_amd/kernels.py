@@ -552,6 +552,21 @@ def gemm_i8_tile_kernel(on):
     return bool(lib.load().lsh_gemm_i8_tile_kernel(int(bool(on))))
 
 
+def tile_weight_16x64(w, tiled, n, k):
+    """[n, k] int8 -> the MFMA-ordered tiling :func:`gemm_i8_residual_ln_i8O` streams."""
+    _dev(w, tiled)
+    call("lsh_tile_weight_16x64", ptr(w), ptr(tiled), n, k, current_stream())
+
+
+def gemm_i8_residual_ln_i8O(a, w_tiled, alpha, scale, bias, residual_bias, output, residual,
+                            batch_tokens, hidden_size, k, dequant_scale, quant_scale, is_post_ln):
+    """Out-projection GEMM + ``ker_residual_bias_ln_i8I_i8O`` in one kernel (fp16)."""
+    _dev(a, w_tiled, scale, bias, residual_bias, output, residual)
+    call("lsh_gemm_i8_residual_ln_i8O_f16", ptr(a), ptr(w_tiled), alpha, ptr(scale), ptr(bias),
+         ptr(residual_bias), ptr(output), ptr(residual), batch_tokens, hidden_size, k,
+         dequant_scale, quant_scale, current_stream(), int(bool(is_post_ln)))
+
+
 def mfma_i8_peak_probe(out, workgroups, iters):
     """Launch the register-resident int8 MFMA loop; returns the integer operations of the launch."""
     import ctypes

@@ -57,6 +57,8 @@ _SIGNATURES = {
     "lsh_layer_norm_row_kernel": (False, "i"),
     "lsh_gemm_i8_tile_kernel": (False, "i"),
     "lsh_mfma_i8_peak_probe": (False, "piips"),
+    "lsh_tile_weight_16x64": (False, "ppiis"),
+    "lsh_gemm_i8_residual_ln_i8O_f16": (False, "pp" + "f" + "ppppp" + "iii" + "ff" + "s" + "i"),
     "lsh_ker_residual_bias_ln_planes_i32I_i8O_f16": (False, "p" + "il" + "ppppp" + "iiff" + "s" +
                                                      "ip"),
     "lsh_gemm_i8_bias_gelu_i8o_f16": (False, "pppp" + "iiifffs"),

@@ -259,3 +259,36 @@ def test_layer_norm_over_accumulator_planes(rng, rows, hidden, nparts):
         outs.append((to_np(q), to_np(r)))
     np.testing.assert_array_equal(outs[0][0], outs[1][0])
     np.testing.assert_array_equal(outs[0][1], outs[1][1])
+
+
+@pytest.mark.parametrize("M,H", [(4096, 768), (1000, 1024), (300, 512), (17, 768), (8192, 1024)])
+@pytest.mark.parametrize("post_ln", [True, False])
+def test_fused_outproj_layernorm_equals_unfused_pair(rng, M, H, post_ln):
+    """Out-projection GEMM + residual LayerNorm + quantisation in one kernel == the int8-output
+    GEMM followed by ker_residual_bias_ln_i8I_i8O, byte for byte (int8 output and fp16 residual)."""
+    k = _k()
+    a = to_dev(rng.integers(-127, 128, size=(M, H), dtype=np.int8))
+    w = to_dev(rng.integers(-127, 128, size=(H, H), dtype=np.int8))
+    g = to_dev((1 + 0.1 * rng.standard_normal(H)).astype(np.float16))
+    b = to_dev((0.1 * rng.standard_normal(H)).astype(np.float16))
+    rb = to_dev((0.1 * rng.standard_normal(H)).astype(np.float16))
+    res = rng.standard_normal((M, H)).astype(np.float16)
+    alpha, dq, qs = 3.0 / (np.sqrt(H) * 127), 2.5 / 127, 127 / 4.0
+    tmp = torch.zeros((M, H), dtype=torch.int8, device=DEV)
+    want_q, want_r = torch.zeros_like(tmp), to_dev(res.copy())
+    k.gemm_i8_i8o(a, w, tmp, M, H, H, alpha)
+    k.ker_residual_bias_ln_i8I_i8O_launcher(tmp, g, b, rb, want_q, want_r, M, H, dq, qs, 1024, post_ln)
+    wt = torch.zeros_like(w)
+    k.tile_weight_16x64(w, wt, H, H)
+    got_q, got_r = torch.full_like(tmp, 7), to_dev(res.copy())
+    k.gemm_i8_residual_ln_i8O(a, wt, alpha, g, b, rb, got_q, got_r, M, H, H, dq, qs, post_ln)
+    assert torch.equal(got_q, want_q)
+    assert torch.equal(got_r.view(torch.int16), want_r.view(torch.int16))
+
+
+def test_fused_outproj_layernorm_rejects_other_sizes():
+    from lightseq_amd.lib import LSHError
+    z8 = torch.zeros(640 * 640, dtype=torch.int8, device=DEV)
+    zh = torch.zeros(640 * 16, dtype=torch.float16, device=DEV)
+    with pytest.raises(LSHError, match="512, 768, 1024"):
+        _k().gemm_i8_residual_ln_i8O(z8, z8, 1.0, zh, zh, zh, z8, zh, 16, 640, 640, 1.0, 1.0, True)
