@@ -11,6 +11,8 @@
 #include <type_traits>
 
 #include "ls_device.cuh"
+
+#include <utility>
 #include "ls_launch.h"
 
 namespace lsh {
@@ -161,6 +163,50 @@ __device__ __forceinline__ void dequant16_bias(const uint4& w, const _Float16* _
   hi = xh + b1;
 }
 
+// 8 int8 codes -> 8 fp16 values, the same arithmetic as dequant16_bias
+__device__ __forceinline__ v8h dequant8_bias(const uint2& w, const _Float16* __restrict__ bias,
+                                             float dq) {
+  const v8h b0 = *reinterpret_cast<const v8h*>(bias);
+  const float off = -128.f * dq;
+  const uint32_t u0 = w.x ^ 0x80808080u, u1 = w.y ^ 0x80808080u;
+  v8h x;
+  x[0] = (_Float16)fmaf(ubyte_f32<0>(u0), dq, off);
+  x[1] = (_Float16)fmaf(ubyte_f32<1>(u0), dq, off);
+  x[2] = (_Float16)fmaf(ubyte_f32<2>(u0), dq, off);
+  x[3] = (_Float16)fmaf(ubyte_f32<3>(u0), dq, off);
+  x[4] = (_Float16)fmaf(ubyte_f32<0>(u1), dq, off);
+  x[5] = (_Float16)fmaf(ubyte_f32<1>(u1), dq, off);
+  x[6] = (_Float16)fmaf(ubyte_f32<2>(u1), dq, off);
+  x[7] = (_Float16)fmaf(ubyte_f32<3>(u1), dq, off);
+  return x + b0;
+}
+
+// float2int8 of four values packed into one word, bit for bit: floor(med3(y, -127, 127.5)) ==
+// clamp(floor(y), -127, 127) for every float y, so one converting instruction per value
+// floors, converts and writes its byte in place.
+__device__ __forceinline__ uint32_t float2int8_pack4(float x0, float x1, float x2, float x3,
+                                                     float quant_scale) {
+#pragma clang fp contract(off)
+  const float y0 = __builtin_amdgcn_fmed3f(x0 * quant_scale + 0.5f, -127.f, 127.5f);
+  const float y1 = __builtin_amdgcn_fmed3f(x1 * quant_scale + 0.5f, -127.f, 127.5f);
+  const float y2 = __builtin_amdgcn_fmed3f(x2 * quant_scale + 0.5f, -127.f, 127.5f);
+  const float y3 = __builtin_amdgcn_fmed3f(x3 * quant_scale + 0.5f, -127.f, 127.5f);
+  uint32_t p;
+  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD"
+      : "=v"(p)
+      : "v"(y0));
+  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
+      : "+v"(p)
+      : "v"(y1));
+  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
+      : "+v"(p)
+      : "v"(y2));
+  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
+      : "+v"(p)
+      : "v"(y3));
+  return p;
+}
+
 // ONE: the sequence fits one block of 128 keys; the multi-block paths are not compiled.
 template <int D, int MODE, int NW, bool ONE>
 // Two workgroups of four wavefronts share a compute unit for head sizes up to 64 (the
@@ -199,7 +245,90 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   const _Float16* bias = reinterpret_cast<const _Float16*>(k) + head * D;
 
   v8h qreg[D / 16];
-  if (MODE == kAttnEncI8) {
+  // FAST (int8 QKV, at most 128 keys): every byte the workgroup reads -- query, key and value
+  // codes, padding mask -- is requested before any of it is converted, so the kernel waits
+  // for memory once; the padding mask is kept as two 64-bit words in scalar registers.
+  constexpr bool FAST = ONE && MODE == kAttnEncI8;
+  uint64_t pad_lo = 0, pad_hi = 0;  // bit j: key j (pad_lo) / key 64 + j (pad_hi) is masked
+  bool padk0 = false, padk1 = false;  // this lane's two bits of them (j = lane)
+  if constexpr (FAST) {
+    constexpr int C16 = D / 16, KCH = 128 * C16 / NT;  // 16-code key chunks per thread
+    constexpr int CH8 = D / 8, NP = 32 * CH8;          // value patches of 4 keys x 8 dims
+    constexpr int VP = (NP + NT - 1) / NT;
+    static_assert(128 * C16 % NT == 0, "key chunks must divide evenly over the threads");
+    const int hid = head_num * D;
+    uint4 wq[D / 32], wk[KCH];
+    uint2 wv[VP][4];
+    // rows past the end read the last row instead (an unconditional load; a conditional one
+    // would become a branch with its own wait) and are zeroed when they are converted
+#pragma unroll
+    for (int kp = 0; kp < D / 32; ++kp)
+      wq[kp] = *reinterpret_cast<const uint4*>(codes + (long)min(qi, S - 1) * hidden3 + kp * 32 +
+                                               g * 16);
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + i * NT, row = c / C16, ch = c % C16;
+      wk[i] = *reinterpret_cast<const uint4*>(codes + (long)min(row, S - 1) * hidden3 + hid +
+                                              ch * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+      const int pidx = min(tid + i * NT, NP - 1), kg = pidx / CH8, ch = pidx % CH8;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        wv[i][r] = *reinterpret_cast<const uint2*>(codes + (long)min(kg * 4 + r, S - 1) * hidden3 +
+                                                   2 * hid + ch * 8);
+    }
+    const int pm0 = pad_mask[(long)b * S + min(lane, S - 1)];
+    const int pm1 = pad_mask[(long)b * S + min(lane + 64, S - 1)];
+    __builtin_amdgcn_sched_barrier(0);
+    // queries: lane half g converts chunk kp * 32 + g * 16 .. + 16, then the halves swap their
+    // second part (see the general path below)
+#pragma unroll
+    for (int kp = 0; kp < D / 32; ++kp) {
+      v8h lo, hi;
+      dequant16_bias(wq[kp], bias + kp * 32 + g * 16, dq, lo, hi);
+      if (qi >= S) lo = hi = (v8h)(_Float16)0;
+      v8h give = g == 0 ? hi : lo, take;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int t = __shfl_xor(reinterpret_cast<const int*>(&give)[j], 32, 64);
+        reinterpret_cast<int*>(&take)[j] = t;
+      }
+      qreg[2 * kp] = g == 0 ? lo : take;
+      qreg[2 * kp + 1] = g == 0 ? take : hi;
+    }
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + i * NT, row = c / C16, ch = c % C16;
+      v8h lo, hi;
+      dequant16_bias(wk[i], bias + hid + ch * 16, dq, lo, hi);
+      if (row >= S) lo = hi = (v8h)(_Float16)0;
+      *reinterpret_cast<v8h*>(&Ks[row * KSTR + ch * 16]) = lo;
+      *reinterpret_cast<v8h*>(&Ks[row * KSTR + ch * 16 + 8]) = hi;
+    }
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+      const int pidx = tid + i * NT, kg = pidx / CH8, ch = pidx % CH8;
+      if (pidx < NP) {
+        v8h x[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          x[r] = dequant8_bias(wv[i][r], bias + 2 * hid + ch * 8, dq);
+          if (kg * 4 + r >= S) x[r] = (v8h)(_Float16)0;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          *reinterpret_cast<v4h*>(&Vt[(ch * 8 + e) * VSTR + kg * 4]) =
+              (v4h){x[0][e], x[1][e], x[2][e], x[3][e]};
+      }
+    }
+    padk0 = pm0 != 0 || lane >= S;
+    padk1 = pm1 != 0 || lane + 64 >= S;
+    pad_lo = __ballot(padk0);
+    pad_hi = __ballot(padk1);
+    __syncthreads();
+  } else if (MODE == kAttnEncI8) {
 #pragma unroll
     for (int kp = 0; kp < D / 32; ++kp) {
       // lane half g converts chunk kp * 32 + g * 16 .. + 16, then the halves swap their
@@ -229,9 +358,13 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         qreg[ks] = (v8h)(_Float16)0;
     }
   }
-  const bool q_pad = qi >= S || (MODE == kAttnLayer ? false
-                                 : GPT              ? qi >= pad_mask[b]
-                                                    : pad_mask[(long)b * S + qi] != 0);
+  bool q_pad;
+  if constexpr (FAST)
+    q_pad = qi >= S || (((qi < 64 ? pad_lo : pad_hi) >> (qi & 63)) & 1) != 0;
+  else
+    q_pad = qi >= S || (MODE == kAttnLayer ? false
+                        : GPT              ? qi >= pad_mask[b]
+                                           : pad_mask[(long)b * S + qi] != 0);
 
   float m = kFloatInfNeg, sum = 0.f;
   v16f sc[4];
@@ -241,13 +374,54 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
+  if constexpr (FAST) {
+    // All key fragments are requested from LDS before the first product, and the products of
+    // the four blocks of 32 keys are interleaved, so neither the LDS latency nor the
+    // dependence between the products of one block is waited for.  Padding costs no vector
+    // instruction per score: one more product per block adds -65504 * 65504 to the scores of
+    // the padded keys (contraction slot 0 of the lane half that holds the key's flag: lane
+    // g * 32 + l32 owns keys g * 32 + l32 and 64 + g * 32 + l32), which the conversion to
+    // fp16 turns into -inf exactly as the mask would; all other scores receive +0.
+    v8h kf[4][D / 16];
+#pragma unroll
+    for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks)
+        kf[sb][ks] = *reinterpret_cast<const v8h*>(&Ks[(sb * 32 + l32) * KSTR + ks * 16 + g * 8]);
+    v8h bx = (v8h)(_Float16)0, ax[4];
+    bx[0] = (_Float16)65504.f;
+#pragma unroll
+    for (int sb = 0; sb < 4; ++sb) {
+      ax[sb] = (v8h)(_Float16)0;
+      ax[sb][0] = (g == (sb & 1) && (sb < 2 ? padk0 : padk1)) ? (_Float16)-65504.f : (_Float16)0;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    v16f c[4];
+#pragma unroll
+    for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) c[sb][i] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks)
+#pragma unroll
+      for (int sb = 0; sb < 4; ++sb)
+        c[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[sb][ks], qreg[ks], c[sb], 0, 0, 0);
+#pragma unroll
+    for (int sb = 0; sb < 4; ++sb)
+      c[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax[sb], bx, c[sb], 0, 0, 0);
+#pragma unroll
+    for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sc[sb][i] = round_h(alpha * c[sb][i]);
+  }
+
   int nkb = ONE ? 1 : (Sk + 127) / 128;
   if (!ONE && causal) nkb = min(nkb, min((int)(blockIdx.x + 1) * (32 * NW) - 1, Sk - 1) / 128 + 1);
   if (ONE) nkb = 1;  // (a constant for the compiler)
   for (int phase = 0; phase < 2; ++phase) {
     for (int kb = 0; kb < nkb; ++kb) {
       const int key0 = kb * 128;
-      const bool fresh = !(nkb == 1 && phase == 1);
+      const bool fresh = !FAST && !(nkb == 1 && phase == 1);
       if (fresh) {
         __syncthreads();
         const bool want_v = phase == 1 || nkb == 1;
@@ -368,11 +542,15 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         const float mref = m_new == kFloatInfNeg ? 0.f : m_new;
         float part = 0.f;
         if (nkb == 1) {  // single key block: the second pass reuses the exponentials
+          const float nm = -mref * 1.44269504088896340736f;
 #pragma unroll
           for (int sb = 0; sb < 4; ++sb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-              sc[sb][i] = __expf(sc[sb][i] - mref);
+              // one key block: exp(s - m) as 2^(s * log2(e) - m * log2(e)), one multiply-add
+              sc[sb][i] = ONE ? __builtin_amdgcn_exp2f(
+                                     fmaf(sc[sb][i], 1.44269504088896340736f, nm))
+                               : __expf(sc[sb][i] - mref);
               part += sc[sb][i];
             }
         } else {
@@ -398,6 +576,21 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         // other's exponentials
         auto pv_pass = [&](auto reuse_tag) {
         constexpr bool REUSE = decltype(reuse_tag)::value;
+        // FAST: all value fragments are requested from LDS before the quotients are formed
+        v4h vf[FAST ? 4 : 1][2][D / 32][2];
+        if constexpr (FAST) {
+#pragma unroll
+          for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+              for (int db = 0; db < D / 32; ++db) {
+                const _Float16* vrow = &Vt[(db * 32 + l32) * VSTR + sb * 32 + 16 * t + 4 * g];
+                vf[sb][t][db][0] = *reinterpret_cast<const v4h*>(vrow);
+                vf[sb][t][db][1] = *reinterpret_cast<const v4h*>(vrow + 8);
+              }
+          __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb) {
 #pragma unroll
@@ -409,7 +602,10 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
               const float e = REUSE ? s : __expf(s - mref);
               float qt = e * rs;
               qt = fmaf(fmaf(-sum, qt, e), rs, qt);
-              qt = fmaf(fmaf(-sum, qt, e), rs, qt);
+              // one key block keeps one correction: with the refined reciprocal the first one
+              // already lands on the correctly rounded quotient except within 2^-22 of a
+              // rounding boundary of the float quotient
+              if constexpr (!ONE) qt = fmaf(fmaf(-sum, qt, e), rs, qt);
               // keep the float quotient a value of its own: folded into the last correction,
               // the conversion to fp16 would round once instead of twice
               asm volatile("" : "+v"(qt));
@@ -418,8 +614,14 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) {
               const _Float16* vrow = &Vt[(db * 32 + l32) * VSTR + sb * 32 + 16 * t + 4 * g];
-              v4h lo = *reinterpret_cast<const v4h*>(vrow);
-              v4h hi = *reinterpret_cast<const v4h*>(vrow + 8);
+              v4h lo, hi;
+              if constexpr (FAST) {
+                lo = vf[sb][t][db][0];
+                hi = vf[sb][t][db][1];
+              } else {
+                lo = *reinterpret_cast<const v4h*>(vrow);
+                hi = *reinterpret_cast<const v4h*>(vrow + 8);
+              }
               v8h a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
               acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, acc[db], 0, 0, 0);
             }
@@ -444,20 +646,20 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
       const int dd = db * 32 + 8 * vg + 4 * g;
       float o[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) o[j] = q_pad ? 0.f : round_h(acc[db][4 * vg + j]);
+      for (int j = 0; j < 4; ++j) o[j] = round_h(acc[db][4 * vg + j]);
       if (ctx != nullptr) {
         half4_t t;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) t.v[j] = __float2half_rn(o[j]);
+        for (int j = 0; j < 4; ++j) t.v[j] = __float2half_rn(q_pad ? 0.f : o[j]);
         if (MODE == kAttnLayer)
           *reinterpret_cast<half4_t*>(ctx + tok * hidden + head * D + dd) = t;
         else
           *reinterpret_cast<half4_t*>(ctx + ((long)bh * S + qi) * D + dd) = t;
       }
       if (ctx_q != nullptr) {
-        *reinterpret_cast<uint32_t*>(ctx_q + tok * hidden + head * D + dd) =
-            pack4_i8(float2int8(o[0], quant_scale), float2int8(o[1], quant_scale),
-                     float2int8(o[2], quant_scale), float2int8(o[3], quant_scale));
+        // a padded query gives zeros, whose code is 0
+        const uint32_t w4 = float2int8_pack4(o[0], o[1], o[2], o[3], quant_scale);
+        *reinterpret_cast<uint32_t*>(ctx_q + tok * hidden + head * D + dd) = q_pad ? 0u : w4;
       }
     }
   }
