@@ -197,6 +197,19 @@ int lsh_encself_attention_i8qkv_f16(const int8_t* qkv, const void* qkv_bias, flo
                                     float quant_scale, int batch_size, int batch_seq_len,
                                     int head_num, int dim_per_head, lsh_stream_t stream);
 
+/* The QKV projection and the attention above in one kernel, for heads of 64 dimensions,
+ * sequences of at most 128 tokens and hidden % 128 == 0 (LSH_ERR_UNSUPPORTED otherwise):
+ * x int8 [batch*seq_len, hidden], qkv_weight int8 [3*hidden, hidden]; requant_alpha is the
+ * alpha of the int8-output GEMM (quant_bert_encoder.cc.cu:305-319), dequant_scale the one
+ * of ker_arrange_encself_qkv_i8I.  Replaces quant_bert_encoder.cc.cu:305-347 in one launch;
+ * the result is byte-identical to lsh_gemm_i8_i8o followed by
+ * lsh_encself_attention_i8qkv_f16. */
+int lsh_qkv_attention_i8_f16(const int8_t* x, const int8_t* qkv_weight, const void* qkv_bias,
+                             const int* src_padding_mask, int8_t* ctx_q, float requant_alpha,
+                             float dequant_scale, float quant_scale, int batch_size,
+                             int batch_seq_len, int head_num, int dim_per_head,
+                             lsh_stream_t stream);
+
 /* ---- embedding ------------------------------------------------------------------------ */
 /* kernels/embKernels_int8.h:7-13 */
 int lsh_launch_enc_emb_i8I_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,

@@ -11,9 +11,8 @@
 #include <type_traits>
 
 #include "ls_device.cuh"
-
-#include <utility>
 #include "ls_launch.h"
+#include "tile_common.cuh"
 
 namespace lsh {
 
@@ -100,12 +99,6 @@ template int correlation_softmax_encself<__half>(int, int, int, hipStream_t, __h
 // directly as its B operand (the MFMA contraction slots are mapped onto the keys a
 // lane already holds).  Two passes over the key blocks (max+sum, then P V); with a
 // single key block (S <= 128) the scores stay in registers between the passes.
-typedef _Float16 v8h __attribute__((ext_vector_type(8)));
-typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-
-__device__ __forceinline__ float round_h(float x) { return (float)(_Float16)x; }
-
 // MODE 1 turns the kernel into the causal prompt attention of the int8 GPT path
 // (inference/model/quant_gpt_encoder.cc.cu:498-523 with
 // inference/kernels/gptKernels_int8.cc.cu:192-222): q and k hold int8 codes as fp16
@@ -130,83 +123,6 @@ __device__ __forceinline__ float round_h(float x) { return (float)(_Float16)x; }
 // would have stored.  The fp16 q, k, v tensors are never written.
 constexpr int kAttnEnc = 0, kAttnGpt = 1, kAttnLayer = 2, kAttnEncI8 = 3;
 
-template <int N>
-__device__ __forceinline__ float ubyte_f32(uint32_t w) {  // one v_cvt_f32_ubyteN
-  return (float)((w >> (8 * N)) & 0xffu);
-}
-
-// 16 int8 codes -> 16 fp16 values half(half(code * dq) + bias)
-__device__ __forceinline__ void dequant16_bias(const uint4& w, const _Float16* __restrict__ bias,
-                                               float dq, v8h& lo, v8h& hi) {
-  // float(code) * dq == fma(float(code + 128), dq, -128 * dq): the product is exact before
-  // its single rounding either way, and -128 * dq is exact.  half(x) + half(b) in fp16
-  // arithmetic == half(float(x) + float(b)): the float sum of two halfs is exact unless
-  // one is below a quarter of the other's last place, where both round to the larger one.
-  const v8h b0 = *reinterpret_cast<const v8h*>(bias);
-  const v8h b1 = *reinterpret_cast<const v8h*>(bias + 8);
-  const float off = -128.f * dq;
-  const uint32_t u[4] = {w.x ^ 0x80808080u, w.y ^ 0x80808080u, w.z ^ 0x80808080u,
-                         w.w ^ 0x80808080u};
-  v8h xl, xh;
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    xl[4 * j + 0] = (_Float16)fmaf(ubyte_f32<0>(u[j]), dq, off);
-    xl[4 * j + 1] = (_Float16)fmaf(ubyte_f32<1>(u[j]), dq, off);
-    xl[4 * j + 2] = (_Float16)fmaf(ubyte_f32<2>(u[j]), dq, off);
-    xl[4 * j + 3] = (_Float16)fmaf(ubyte_f32<3>(u[j]), dq, off);
-    xh[4 * j + 0] = (_Float16)fmaf(ubyte_f32<0>(u[2 + j]), dq, off);
-    xh[4 * j + 1] = (_Float16)fmaf(ubyte_f32<1>(u[2 + j]), dq, off);
-    xh[4 * j + 2] = (_Float16)fmaf(ubyte_f32<2>(u[2 + j]), dq, off);
-    xh[4 * j + 3] = (_Float16)fmaf(ubyte_f32<3>(u[2 + j]), dq, off);
-  }
-  lo = xl + b0;
-  hi = xh + b1;
-}
-
-// 8 int8 codes -> 8 fp16 values, the same arithmetic as dequant16_bias
-__device__ __forceinline__ v8h dequant8_bias(const uint2& w, const _Float16* __restrict__ bias,
-                                             float dq) {
-  const v8h b0 = *reinterpret_cast<const v8h*>(bias);
-  const float off = -128.f * dq;
-  const uint32_t u0 = w.x ^ 0x80808080u, u1 = w.y ^ 0x80808080u;
-  v8h x;
-  x[0] = (_Float16)fmaf(ubyte_f32<0>(u0), dq, off);
-  x[1] = (_Float16)fmaf(ubyte_f32<1>(u0), dq, off);
-  x[2] = (_Float16)fmaf(ubyte_f32<2>(u0), dq, off);
-  x[3] = (_Float16)fmaf(ubyte_f32<3>(u0), dq, off);
-  x[4] = (_Float16)fmaf(ubyte_f32<0>(u1), dq, off);
-  x[5] = (_Float16)fmaf(ubyte_f32<1>(u1), dq, off);
-  x[6] = (_Float16)fmaf(ubyte_f32<2>(u1), dq, off);
-  x[7] = (_Float16)fmaf(ubyte_f32<3>(u1), dq, off);
-  return x + b0;
-}
-
-// float2int8 of four values packed into one word, bit for bit: floor(med3(y, -127, 127.5)) ==
-// clamp(floor(y), -127, 127) for every float y, so one converting instruction per value
-// floors, converts and writes its byte in place.
-__device__ __forceinline__ uint32_t float2int8_pack4(float x0, float x1, float x2, float x3,
-                                                     float quant_scale) {
-#pragma clang fp contract(off)
-  const float y0 = __builtin_amdgcn_fmed3f(x0 * quant_scale + 0.5f, -127.f, 127.5f);
-  const float y1 = __builtin_amdgcn_fmed3f(x1 * quant_scale + 0.5f, -127.f, 127.5f);
-  const float y2 = __builtin_amdgcn_fmed3f(x2 * quant_scale + 0.5f, -127.f, 127.5f);
-  const float y3 = __builtin_amdgcn_fmed3f(x3 * quant_scale + 0.5f, -127.f, 127.5f);
-  uint32_t p;
-  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD"
-      : "=v"(p)
-      : "v"(y0));
-  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
-      : "+v"(p)
-      : "v"(y1));
-  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
-      : "+v"(p)
-      : "v"(y2));
-  asm("v_cvt_flr_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD"
-      : "+v"(p)
-      : "v"(y3));
-  return p;
-}
-
 // ONE: the sequence fits one block of 128 keys; the multi-block paths are not compiled.
 template <int D, int MODE, int NW, bool ONE>
 // Two workgroups of four wavefronts share a compute unit for head sizes up to 64 (the
@@ -219,8 +135,8 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   // number of keys: the layer mode (MODE 2) may attend over another sequence (cross
   // attention, cached decoding); everywhere else keys and queries are the same S positions
   const int Sk = MODE == kAttnLayer ? key_len : S;
-  constexpr int KSTR = D + 8;    // halfs per K row in LDS (pad kills bank conflicts)
-  constexpr int VSTR = 128 + 4;  // halfs per V^T row in LDS
+  constexpr int KSTR = attn_kstr(D);  // halfs per K row in LDS (pad kills bank conflicts)
+  constexpr int VSTR = kAttnVstr;     // halfs per V^T row in LDS
   constexpr int CH = D / 8;      // 16-byte chunks per row
   __shared__ __align__(16) _Float16 Ks[128 * KSTR];
   __shared__ __align__(16) _Float16 Vt[D * VSTR];
@@ -249,8 +165,6 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
   // codes, padding mask -- is requested before any of it is converted, so the kernel waits
   // for memory once; the padding mask is kept as two 64-bit words in scalar registers.
   constexpr bool FAST = ONE && MODE == kAttnEncI8;
-  uint64_t pad_lo = 0, pad_hi = 0;  // bit j: key j (pad_lo) / key 64 + j (pad_hi) is masked
-  bool padk0 = false, padk1 = false;  // this lane's two bits of them (j = lane)
   if constexpr (FAST) {
     constexpr int C16 = D / 16, KCH = 128 * C16 / NT;  // 16-code key chunks per thread
     constexpr int CH8 = D / 8, NP = 32 * CH8;          // value patches of 4 keys x 8 dims
@@ -323,11 +237,16 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
               (v4h){x[0][e], x[1][e], x[2][e], x[3][e]};
       }
     }
-    padk0 = pm0 != 0 || lane >= S;
-    padk1 = pm1 != 0 || lane + 64 >= S;
-    pad_lo = __ballot(padk0);
-    pad_hi = __ballot(padk1);
+    const bool padk0 = pm0 != 0 || lane >= S, padk1 = pm1 != 0 || lane + 64 >= S;
+    // the padding flag of this lane's query (queries and keys are the same positions)
+    const uint64_t pad_q = __ballot(wave < 2 ? padk0 : padk1);
+    const bool q_pad = qi >= S || ((pad_q >> ((wave & 1) * 32 + l32)) & 1) != 0;
     __syncthreads();
+    const long tok = (long)b * S + qi;
+    attend_block128<D>(Ks, Vt, qreg, padk0, padk1, q_pad, qi < S, alpha, quant_scale,
+                       ctx ? ctx + ((long)bh * S + qi) * D : nullptr,
+                       ctx_q ? ctx_q + tok * (head_num * D) + head * D : nullptr, l32, g);
+    return;
   } else if (MODE == kAttnEncI8) {
 #pragma unroll
     for (int kp = 0; kp < D / 32; ++kp) {
@@ -358,13 +277,9 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         qreg[ks] = (v8h)(_Float16)0;
     }
   }
-  bool q_pad;
-  if constexpr (FAST)
-    q_pad = qi >= S || (((qi < 64 ? pad_lo : pad_hi) >> (qi & 63)) & 1) != 0;
-  else
-    q_pad = qi >= S || (MODE == kAttnLayer ? false
-                        : GPT              ? qi >= pad_mask[b]
-                                           : pad_mask[(long)b * S + qi] != 0);
+  const bool q_pad = qi >= S || (MODE == kAttnLayer ? false
+                                 : GPT              ? qi >= pad_mask[b]
+                                                    : pad_mask[(long)b * S + qi] != 0);
 
   float m = kFloatInfNeg, sum = 0.f;
   v16f sc[4];
@@ -374,54 +289,13 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
-  if constexpr (FAST) {
-    // All key fragments are requested from LDS before the first product, and the products of
-    // the four blocks of 32 keys are interleaved, so neither the LDS latency nor the
-    // dependence between the products of one block is waited for.  Padding costs no vector
-    // instruction per score: one more product per block adds -65504 * 65504 to the scores of
-    // the padded keys (contraction slot 0 of the lane half that holds the key's flag: lane
-    // g * 32 + l32 owns keys g * 32 + l32 and 64 + g * 32 + l32), which the conversion to
-    // fp16 turns into -inf exactly as the mask would; all other scores receive +0.
-    v8h kf[4][D / 16];
-#pragma unroll
-    for (int sb = 0; sb < 4; ++sb)
-#pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks)
-        kf[sb][ks] = *reinterpret_cast<const v8h*>(&Ks[(sb * 32 + l32) * KSTR + ks * 16 + g * 8]);
-    v8h bx = (v8h)(_Float16)0, ax[4];
-    bx[0] = (_Float16)65504.f;
-#pragma unroll
-    for (int sb = 0; sb < 4; ++sb) {
-      ax[sb] = (v8h)(_Float16)0;
-      ax[sb][0] = (g == (sb & 1) && (sb < 2 ? padk0 : padk1)) ? (_Float16)-65504.f : (_Float16)0;
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    v16f c[4];
-#pragma unroll
-    for (int sb = 0; sb < 4; ++sb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) c[sb][i] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks)
-#pragma unroll
-      for (int sb = 0; sb < 4; ++sb)
-        c[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[sb][ks], qreg[ks], c[sb], 0, 0, 0);
-#pragma unroll
-    for (int sb = 0; sb < 4; ++sb)
-      c[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax[sb], bx, c[sb], 0, 0, 0);
-#pragma unroll
-    for (int sb = 0; sb < 4; ++sb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) sc[sb][i] = round_h(alpha * c[sb][i]);
-  }
-
   int nkb = ONE ? 1 : (Sk + 127) / 128;
   if (!ONE && causal) nkb = min(nkb, min((int)(blockIdx.x + 1) * (32 * NW) - 1, Sk - 1) / 128 + 1);
   if (ONE) nkb = 1;  // (a constant for the compiler)
   for (int phase = 0; phase < 2; ++phase) {
     for (int kb = 0; kb < nkb; ++kb) {
       const int key0 = kb * 128;
-      const bool fresh = !FAST && !(nkb == 1 && phase == 1);
+      const bool fresh = !(nkb == 1 && phase == 1);
       if (fresh) {
         __syncthreads();
         const bool want_v = phase == 1 || nkb == 1;
@@ -576,21 +450,6 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
         // other's exponentials
         auto pv_pass = [&](auto reuse_tag) {
         constexpr bool REUSE = decltype(reuse_tag)::value;
-        // FAST: all value fragments are requested from LDS before the quotients are formed
-        v4h vf[FAST ? 4 : 1][2][D / 32][2];
-        if constexpr (FAST) {
-#pragma unroll
-          for (int sb = 0; sb < 4; ++sb)
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-              for (int db = 0; db < D / 32; ++db) {
-                const _Float16* vrow = &Vt[(db * 32 + l32) * VSTR + sb * 32 + 16 * t + 4 * g];
-                vf[sb][t][db][0] = *reinterpret_cast<const v4h*>(vrow);
-                vf[sb][t][db][1] = *reinterpret_cast<const v4h*>(vrow + 8);
-              }
-          __builtin_amdgcn_sched_barrier(0);
-        }
 #pragma unroll
         for (int sb = 0; sb < 4; ++sb) {
 #pragma unroll
@@ -614,14 +473,8 @@ encself_attn_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) {
               const _Float16* vrow = &Vt[(db * 32 + l32) * VSTR + sb * 32 + 16 * t + 4 * g];
-              v4h lo, hi;
-              if constexpr (FAST) {
-                lo = vf[sb][t][db][0];
-                hi = vf[sb][t][db][1];
-              } else {
-                lo = *reinterpret_cast<const v4h*>(vrow);
-                hi = *reinterpret_cast<const v4h*>(vrow + 8);
-              }
+              v4h lo = *reinterpret_cast<const v4h*>(vrow);
+              v4h hi = *reinterpret_cast<const v4h*>(vrow + 8);
               v8h a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
               acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb, acc[db], 0, 0, 0);
             }

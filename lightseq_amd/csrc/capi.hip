@@ -312,6 +312,16 @@ int lsh_encself_attention_i8qkv_f16(const int8_t* qkv, const void* qkv_bias, flo
                                  HS(stream));
 }
 
+int lsh_qkv_attention_i8_f16(const int8_t* x, const int8_t* qkv_weight, const void* qkv_bias,
+                             const int* src_padding_mask, int8_t* ctx_q, float requant_alpha,
+                             float dequant_scale, float quant_scale, int batch_size,
+                             int batch_seq_len, int head_num, int dim_per_head,
+                             lsh_stream_t stream) {
+  return qkv_attention_i8(x, qkv_weight, H(qkv_bias), src_padding_mask, ctx_q, requant_alpha,
+                          dequant_scale, quant_scale, batch_size, batch_seq_len, head_num,
+                          dim_per_head, HS(stream));
+}
+
 // ---- embedding ----------------------------------------------------------------------------------
 int lsh_launch_enc_emb_i8I_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,
                                void* output, int* pad_mask, int pad_id, int batch_size,

@@ -36,6 +36,7 @@
 // columns of C: one 16-byte store for int8 output, two for fp16.
 #include "ls_device.cuh"
 #include "ls_launch.h"
+#include "tile_common.cuh"
 
 #include <hip/hip_ext.h>
 
@@ -45,19 +46,7 @@
 
 namespace lsh {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-constexpr int kBK = 128;  // bytes of K per LDS stage
 constexpr int kBM = 128, kBN = 128;
-
-// swizzle keys (3 bits) of a tile row, for the activation tile (rows read in natural
-// order) and the weight tile (rows read in sigma order)
-__device__ __forceinline__ int key_act(int row) { return (row >> 1) & 7; }
-__device__ __forceinline__ int key_wgt(int row) { return ((row >> 1) & 3) | (((row >> 4) & 1) << 2); }
-// MFMA row r (0..31) of the weight operand -> local column of C, chosen so that the
-// accumulators c[0..15] of lane (l%32, g=l/32) are columns 16g .. 16g+15.
-__device__ __forceinline__ int sigma(int r) { return 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3); }
 
 // ---------------------------------------------------------------------------------
 // Epilogues.  store16(m, n, N, c, full): c[0..15] are C[m, n .. n+15]; `full` means all
@@ -95,15 +84,6 @@ __device__ __forceinline__ void store16_i8(int8_t* p, int n, int N, const int (&
     for (int i = 0; i < 16; ++i)
       if (n + i < N) p[i] = (int8_t)q[i];
   }
-}
-
-__device__ __forceinline__ uint4 requant16_packed(const v16i& c, float alpha) {
-  uint4 o;
-  o.x = requant_acc_pack4(c[0], c[1], c[2], c[3], alpha);
-  o.y = requant_acc_pack4(c[4], c[5], c[6], c[7], alpha);
-  o.z = requant_acc_pack4(c[8], c[9], c[10], c[11], alpha);
-  o.w = requant_acc_pack4(c[12], c[13], c[14], c[15], alpha);
-  return o;
 }
 
 struct EpiI8 {
@@ -756,11 +736,6 @@ gemm_i8_stream128_kernel(const int8_t* __restrict__ A, const int8_t* __restrict_
 // Preconditions (checked by the dispatcher): K % 128 == 0, K / 128 >= NST, N % 16 == 0 and the
 // epilogue's vector path legal, 32-bit operand offsets, operands 16-byte aligned.
 // ---------------------------------------------------------------------------------
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
 template <typename Epi, int WGM, int WGN, int MB, int NB, int NST>
 __global__ void __launch_bounds__(64 * WGM * WGN)
 gemm_i8_tile_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,

@@ -136,6 +136,17 @@ int encself_attention_i8qkv(const int8_t* qkv, const __half* qkv_bias, float deq
                             const int* pad_mask, __half* ctx, int8_t* ctx_q, float quant_scale,
                             int batch, int seq_len, int head_num, int dim_per_head, hipStream_t s);
 
+// QKV projection + encoder attention of a (sequence, head) pair in one kernel
+// (qkv_attn_kernels.hip): x int8 [batch * seq_len, hidden], qkv_weight int8 [3 * hidden, hidden],
+// ctx_q int8 [batch * seq_len, hidden]; byte-identical to gemm_i8_i8o (alpha = requant_alpha)
+// followed by encself_attention_i8qkv.  Needs dim_per_head 64, seq_len <= 128, hidden % 128 == 0.
+bool qkv_attention_fused_supported(int batch, int seq_len, int head_num, int dim_per_head);
+void qkv_attention_time_next_launch(hipEvent_t start, hipEvent_t stop);
+int qkv_attention_i8(const int8_t* x, const int8_t* qkv_weight, const __half* qkv_bias,
+                     const int* pad_mask, int8_t* ctx_q, float requant_alpha, float dequant_scale,
+                     float quant_scale, int batch, int seq_len, int head_num, int dim_per_head,
+                     hipStream_t s);
+
 // ---- int8 MFMA GEMM (gemm_i8.hip) -----------------------------------------------------
 // C[M,N] = A[M,K] * W[N,K]^T, both operands K-contiguous.
 int gemm_i8_i32o(const int8_t* A, const int8_t* W, int32_t* C, int M, int N, int K,

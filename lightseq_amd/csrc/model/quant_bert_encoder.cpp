@@ -116,10 +116,13 @@ void QuantBertEncoder::reset_profile() {
 void QuantBertEncoder::prof_begin(int site, int m, int n, int k, const char* epilogue) {
   if (!_profiling) return;
   const bool fused_ln = std::string(epilogue) == "fused_ln";
+  const bool fused_qa = std::string(epilogue) == "fused_qkv_attn";
   SiteProfile& p = _profile[site];
   if (p.m != m || p.n != n || p.k != k || p.kernel.empty()) {
     p.m = m; p.n = n; p.k = k;
-    p.kernel = fused_ln ? "gemm_ln_rows16_kernel" : gemm_i8_kernel_name(m, n, k, epilogue);
+    p.kernel = fused_ln   ? "gemm_ln_rows16_kernel"
+               : fused_qa ? "qkv_attn_kernel"
+                          : gemm_i8_kernel_name(m, n, k, epilogue);
   }
   Pending pe;
   pe.site = site;
@@ -133,6 +136,7 @@ void QuantBertEncoder::prof_begin(int site, int m, int n, int k, const char* epi
   }
   // the launcher records the kernel's own begin / end timestamps into the events
   if (fused_ln) gemm_ln_time_next_launch(pe.e0, pe.e1);
+  else if (fused_qa) qkv_attention_time_next_launch(pe.e0, pe.e1);
   else gemm_i8_time_next_launch(pe.e0, pe.e1);
   _pending.push_back(pe);
 }
@@ -187,27 +191,44 @@ void QuantBertEncoder::self_attention() {
   }
   tap(taps.ln1_q, _int8_ffn_in_buf.get(), (size_t)M * H);
 
-  // qkv = ori_q * qkv_wei -> int8 codes [M, 3H].  The fused route hands the codes and the
-  // bias to the attention kernel, which dequantises them as it stages q, k, v; the unfused
-  // route writes fp16 q, k, v [B, h, S, d] first.  Both give the same bits.
+  // qkv = ori_q * qkv_wei -> int8 codes [M, 3H] -> fp16 q, k, v -> attention -> int8 context.
+  // Three routes with the same bits: (a) one kernel per (sequence, head) that keeps codes and
+  // q, k, v on the compute unit (heads of 64, at most 128 tokens, codes not tapped); (b) the
+  // GEMM, then an attention kernel that dequantises the codes as it stages q, k, v; (c) the
+  // GEMM, the arrange kernel writing fp16 q, k, v [B, h, S, d], the attention on those.
   const long mbd = (long)M * H;
-  prof_begin(0, M, 3 * H, H, "EpiI8");
-  LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_qkv.get(), _int8_ffn_out_buf.get(), M, 3 * H,
-                       H, c[0] * c[4] / (c[8] * Q), _stream));
-  tap(taps.qkv_q, _int8_ffn_out_buf.get(), (size_t)M * 3 * H);
   const int dph = _tw._dim_per_head;
-  if (_fuse && (dph == 32 || dph == 64 || dph == 128)) {
-    // scores -> masked softmax -> context -> merge heads + quantise, one kernel
-    LSH_CALL(encself_attention_i8qkv(_int8_ffn_out_buf.get(), w.b_qkv.get(), c[8] / Q,
-                                     _p_d_padding_mask, nullptr, _int8_ffn_in_buf.get(), Q / c[5],
-                                     _batch_size, _batch_seq_len, _tw._head_num, dph, _stream));
+  const bool tap_qkv = taps.qkv_q && taps.tap_layer == _layer_id;
+  if (_fuse && !tap_qkv &&
+      qkv_attention_fused_supported(_batch_size, _batch_seq_len, _tw._head_num, dph)) {
+    prof_begin(0, M, 3 * H, H, "fused_qkv_attn");
+    // reads _int8_ffn_in_buf and must not overwrite it: the context goes to _int8_ffn_out_buf
+    // and the two buffers swap roles
+    LSH_CALL(qkv_attention_i8(_int8_ffn_in_buf.get(), w.w_qkv.get(), w.b_qkv.get(),
+                              _p_d_padding_mask, _int8_ffn_out_buf.get(), c[0] * c[4] / (c[8] * Q),
+                              c[8] / Q, Q / c[5], _batch_size, _batch_seq_len, _tw._head_num, dph,
+                              _stream));
+    std::swap(_int8_ffn_in_buf, _int8_ffn_out_buf);
   } else {
-    LSH_CALL(arrange_encself_qkv_i8I<__half>(M, H, _stream, _int8_ffn_out_buf.get(),
-                                             w.b_qkv.get(), _qkv_buf.get(), mbd, _batch_seq_len,
-                                             dph, _tw._head_num, c[8] / Q));
-    LSH_CALL(encself_attention_f16(_qkv_buf.get(), _qkv_buf.get() + mbd, _qkv_buf.get() + 2 * mbd,
-                                   _p_d_padding_mask, nullptr, _int8_ffn_in_buf.get(), Q / c[5],
-                                   _batch_size, _batch_seq_len, _tw._head_num, dph, _stream));
+    prof_begin(0, M, 3 * H, H, "EpiI8");
+    LSH_CALL(gemm_i8_i8o(_int8_ffn_in_buf.get(), w.w_qkv.get(), _int8_ffn_out_buf.get(), M, 3 * H,
+                         H, c[0] * c[4] / (c[8] * Q), _stream));
+    tap(taps.qkv_q, _int8_ffn_out_buf.get(), (size_t)M * 3 * H);
+    if (_fuse && (dph == 32 || dph == 64 || dph == 128)) {
+      // scores -> masked softmax -> context -> merge heads + quantise, one kernel
+      LSH_CALL(encself_attention_i8qkv(_int8_ffn_out_buf.get(), w.b_qkv.get(), c[8] / Q,
+                                       _p_d_padding_mask, nullptr, _int8_ffn_in_buf.get(),
+                                       Q / c[5], _batch_size, _batch_seq_len, _tw._head_num, dph,
+                                       _stream));
+    } else {
+      LSH_CALL(arrange_encself_qkv_i8I<__half>(M, H, _stream, _int8_ffn_out_buf.get(),
+                                               w.b_qkv.get(), _qkv_buf.get(), mbd, _batch_seq_len,
+                                               dph, _tw._head_num, c[8] / Q));
+      LSH_CALL(encself_attention_f16(_qkv_buf.get(), _qkv_buf.get() + mbd,
+                                     _qkv_buf.get() + 2 * mbd, _p_d_padding_mask, nullptr,
+                                     _int8_ffn_in_buf.get(), Q / c[5], _batch_size, _batch_seq_len,
+                                     _tw._head_num, dph, _stream));
+    }
   }
   tap(taps.ctx_q, _int8_ffn_in_buf.get(), (size_t)M * H);
 

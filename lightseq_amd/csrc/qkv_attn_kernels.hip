@@ -1,0 +1,288 @@
+// QKV projection and encoder self-attention of one (sequence, head) pair in one kernel.
+//
+// Replaces, for sequences of at most 128 tokens and heads of 64 dimensions, the chain
+// inference/model/quant_bert_encoder.cc.cu:305-347 (int8 QKV GEMM -> ker_arrange_encself_qkv_i8I
+// -> two strided batched GEMMs + ker_correlation_softmax_encself -> ker_arrange_atten_output_i8O):
+// neither the int8 QKV codes [tokens, 3 * hidden] nor the fp16 q, k, v leave the compute unit.
+//
+// A workgroup (4 wavefronts) owns sequence b and head h:
+//  1. the 128 x 192 int8 product X_b W_h^T (X_b: the tokens of the sequence, W_h: the 64 query,
+//     64 key and 64 value rows of the head), K walked in 128-byte steps through a two-stage LDS
+//     ring filled by global_load_lds_dwordx4, 64 x 96 accumulators per wavefront -- the loop of
+//     the int8 GEMM tile kernel;
+//  2. every accumulator becomes the int8 code the stand-alone GEMM would have stored
+//     (requant_acc), then the fp16 value half(half(code * dq) + bias) that the arrange kernel
+//     would have stored, and goes to LDS over the drained ring: queries and keys row-major,
+//     values transposed;
+//  3. the attention of one block of keys (attend_block128), context written as int8 codes.
+// Results are byte-identical to the chain of stand-alone kernels.
+#include "ls_device.cuh"
+#include "ls_launch.h"
+#include "tile_common.cuh"
+
+#include <hip/hip_ext.h>
+
+#include <mutex>
+
+namespace lsh {
+
+namespace {
+constexpr int kQaD = 64;                         // head size
+constexpr int kQaTM = 128, kQaTN = 3 * kQaD;     // tokens x (q | k | v) columns of a workgroup
+constexpr int kQaStage = (kQaTM + kQaTN) * kBK;  // bytes of one ring stage
+constexpr int kQaNst = 2;
+}  // namespace
+
+__global__ void __launch_bounds__(256, 2)
+qkv_attn_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
+                const _Float16* __restrict__ bias, const int* __restrict__ pad_mask,
+                int8_t* __restrict__ ctx_q, float requant_alpha, float dq, float quant_scale,
+                float alpha, int S, int batch, int head_num, int K) {
+  constexpr int D = kQaD, WGN = 2, MB = 2, NB = 3, NWV = 4, TM = kQaTM, TN = kQaTN;
+  constexpr int STAGE = kQaStage, NST = kQaNst;
+  constexpr int NA = TM / 8 / NWV, NW = TN / 8 / NWV, PER = NA + NW;  // 1-KB loads per wavefront
+  extern __shared__ __align__(16) int8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN, l32 = lane & 31, g = lane >> 5;
+  // Workgroups are dealt to the 8 XCDs round-robin; with a batch that is a multiple of 8 all
+  // heads of a sequence run on one XCD, so its L2 fetches the sequence's activations once.
+  int b, head;
+  if ((batch & 7) == 0) {
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    b = xcd + 8 * (j / head_num);
+    head = j % head_num;
+  } else {
+    b = blockIdx.x / head_num;
+    head = blockIdx.x % head_num;
+  }
+  const int hidden = head_num * D;
+  const int nk = K / kBK;
+
+  // padding flags of keys `lane` and `64 + lane` (requested first, used after the product)
+  const int pm0 = pad_mask[(long)b * S + min(lane, S - 1)];
+  const int pm1 = pad_mask[(long)b * S + min(lane + 64, S - 1)];
+
+  uint32_t a_src[NA], w_src[NW];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int row = (wave + NWV * i) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ key_act(row);
+    // tokens past the end of the sequence read its last token and are zeroed in step 2
+    a_src[i] = (uint32_t)(b * S + min(row, S - 1)) * (uint32_t)K + c * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    const int row = (wave + NWV * i) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ key_wgt(row);
+    // tile column `row`: part row / 64 (q, k, v), dimension row % 64 of this head
+    w_src[i] = (uint32_t)((row >> 6) * hidden + head * D + (row & 63)) * (uint32_t)K + c * 16;
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+  auto dma1 = [&](const int8_t* base, uint32_t voff, uint32_t lds) {
+    lds = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff),
+                 "s"(base)
+                 : "memory");
+  };
+  auto issue = [&](int kt, int slot) {  // K step kt into ring slot `slot`
+    const uint32_t base = lds0 + slot * STAGE;
+#pragma unroll
+    for (int i = 0; i < NA; ++i) dma1(A + kt * kBK, a_src[i], base + (wave + NWV * i) * 1024);
+#pragma unroll
+    for (int i = 0; i < NW; ++i)
+      dma1(W + kt * kBK, w_src[i], base + TM * kBK + (wave + NWV * i) * 1024);
+  };
+  // LDS byte offset of this lane's fragment chunk for K slice 0; slice ks is at (offset ^ (ks << 5))
+  int a_base[MB], w_base[NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int row = wm * (MB * 32) + i * 32 + l32;
+    a_base[i] = row * kBK + ((g ^ key_act(row)) << 4);
+  }
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const int row = wn * (NB * 32) + j * 32 + sigma(l32);
+    w_base[j] = TM * kBK + row * kBK + ((g ^ key_wgt(row)) << 4);
+  }
+  struct Frag {
+    v4i a[MB], w[NB];
+  };
+  auto load_frag = [&](Frag& f, const int8_t* stage, int ks) {
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+      f.a[i] = *reinterpret_cast<const v4i*>(stage + (a_base[i] ^ (ks << 5)));
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      f.w[j] = *reinterpret_cast<const v4i*>(stage + (w_base[j] ^ (ks << 5)));
+  };
+  v16i acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) acc[i][j] = (v16i)0;
+  auto mma = [&](const Frag& f) {
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[j], f.a[i], acc[i][j], 0, 0, 0);
+  };
+  // issue order of one slice: an LDS read of the next slice after each of the first MFMAs
+  auto pattern = [&]() {
+#pragma unroll
+    for (int q = 0; q < MB + NB; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, MB * NB - (MB + NB), 0);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  Frag f[2];
+  auto slices = [&](const int8_t* stage) {  // slices 1..3 read, slices 0..2 multiplied
+#pragma unroll
+    for (int ks = 1; ks < 4; ++ks) {
+      load_frag(f[ks & 1], stage, ks);
+      mma(f[(ks - 1) & 1]);
+      pattern();
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < NST; ++s) issue(s, s);
+  wait_vmcnt<(NST - 1) * PER>();
+  __builtin_amdgcn_s_barrier();
+  load_frag(f[0], smem, 0);
+  int slot = 0;
+  // steady state: a step ends by refilling its own slot with step kt + NST
+  for (int kt = 0; kt < nk - NST; ++kt) {
+    slices(smem + slot * STAGE);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront has read all of the stage
+    wait_vmcnt<(NST - 2) * PER>();       // its own loads of step kt + 1 have landed ...
+    __builtin_amdgcn_s_barrier();        // ... and everyone's; everyone is done with step kt
+    issue(kt + NST, slot);
+    __builtin_amdgcn_sched_barrier(0);
+    if (++slot == NST) slot = 0;
+    load_frag(f[0], smem + slot * STAGE, 0);
+    mma(f[1]);
+    pattern();
+  }
+  // drain: NST - 1 steps without a refill, then the last step
+#pragma unroll
+  for (int t = 0; t < NST - 1; ++t) {
+    slices(smem + slot * STAGE);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    if (++slot == NST) slot = 0;
+    load_frag(f[0], smem + slot * STAGE, 0);
+    mma(f[1]);
+    pattern();
+  }
+  slices(smem + slot * STAGE);
+  mma(f[1]);
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();  // the ring is drained: its memory now holds q, k, v
+
+  // ---- step 2: accumulators -> int8 codes -> fp16 q, k (row-major) and v (transposed) ----
+  constexpr int KSTR = attn_kstr(D), VSTR = kAttnVstr;
+  _Float16* Qs = reinterpret_cast<_Float16*>(smem);
+  _Float16* Ks = Qs + 128 * KSTR;
+  _Float16* Vt = Ks + 128 * KSTR;
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int t = wm * (MB * 32) + i * 32 + l32;  // token of the sequence
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      // this lane's 16 accumulators are columns wn * 96 + j * 32 + 16 g .. + 16 of the tile
+      const int blk = wn * NB + j, part = blk >> 1, d0 = (blk & 1) * 32 + 16 * g;
+      const uint4 codes = requant16_packed(acc[i][j], requant_alpha);
+      v8h lo, hi;
+      dequant16_bias(codes, bias + part * hidden + head * D + d0, dq, lo, hi);
+      if (t >= S) lo = hi = (v8h)(_Float16)0;
+      if (part == 2) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          Vt[(d0 + e) * VSTR + t] = lo[e];
+          Vt[(d0 + 8 + e) * VSTR + t] = hi[e];
+        }
+      } else {
+        _Float16* dst = (part == 0 ? Qs : Ks) + t * KSTR + d0;
+        *reinterpret_cast<v8h*>(dst) = lo;
+        *reinterpret_cast<v8h*>(dst + 8) = hi;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- step 3: attention; wavefront w owns queries 32 w .. 32 w + 31 ----
+  const int qi = wave * 32 + l32;
+  v8h qreg[D / 16];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks)
+    qreg[ks] = *reinterpret_cast<const v8h*>(&Qs[qi * KSTR + ks * 16 + g * 8]);
+  const bool padk0 = pm0 != 0 || lane >= S, padk1 = pm1 != 0 || lane + 64 >= S;
+  const uint64_t pad_q = __ballot(wave < 2 ? padk0 : padk1);
+  const bool q_pad = qi >= S || ((pad_q >> ((wave & 1) * 32 + l32)) & 1) != 0;
+  attend_block128<D>(Ks, Vt, qreg, padk0, padk1, q_pad, qi < S, alpha, quant_scale, nullptr,
+                     ctx_q + ((long)b * S + qi) * hidden + head * D, l32, g);
+}
+
+// The next launch on this thread records its begin / end timestamps into these events.
+static thread_local hipEvent_t g_qa_ev_start = nullptr, g_qa_ev_stop = nullptr;
+void qkv_attention_time_next_launch(hipEvent_t start, hipEvent_t stop) {
+  g_qa_ev_start = start;
+  g_qa_ev_stop = stop;
+}
+
+bool qkv_attention_fused_supported(int batch, int seq_len, int head_num, int dim_per_head) {
+  const long hidden = (long)head_num * dim_per_head;
+  return dim_per_head == kQaD && seq_len >= 1 && seq_len <= kQaTM && hidden % kBK == 0 &&
+         hidden / kBK >= kQaNst && (long)batch * seq_len * hidden < (1l << 32) &&
+         3 * hidden * hidden < (1l << 32);
+}
+
+// qkv_weight int8 [3 * hidden, hidden] (K-contiguous), qkv_bias fp16 [3 * hidden], x int8
+// [batch * seq_len, hidden], pad_mask int32 [batch, seq_len] (non-zero = padding), ctx_q int8
+// [batch * seq_len, hidden].  requant_alpha: int32 accumulator -> int8 QKV code (the alpha of the
+// stand-alone requantising GEMM); dequant_scale: QKV code -> float; quant_scale: context -> int8.
+int qkv_attention_i8(const int8_t* x, const int8_t* qkv_weight, const __half* qkv_bias,
+                     const int* pad_mask, int8_t* ctx_q, float requant_alpha, float dequant_scale,
+                     float quant_scale, int batch, int seq_len, int head_num, int dim_per_head,
+                     hipStream_t s) {
+  if (!x || !qkv_weight || !qkv_bias || !pad_mask || !ctx_q || batch <= 0 || seq_len <= 0 ||
+      head_num <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "qkv_attention_i8: bad arguments");
+  if (!qkv_attention_fused_supported(batch, seq_len, head_num, dim_per_head))
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "qkv_attention_i8: needs dim_per_head 64, seq_len <= 128, hidden % 128 == 0");
+  if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(qkv_weight) |
+        reinterpret_cast<uintptr_t>(qkv_bias) | reinterpret_cast<uintptr_t>(ctx_q)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_INVALID, "qkv_attention_i8: pointers must be 16-byte aligned");
+  constexpr size_t smem = (size_t)kQaNst * kQaStage;
+  {
+    // the ring is larger than the default dynamic LDS limit: raise it once per device
+    static std::mutex mu;
+    static unsigned long long raised = 0;
+    int dev = 0;
+    if (lsh_check_hip(hipGetDevice(&dev), "hipGetDevice")) return LSH_ERR_HIP;
+    std::lock_guard<std::mutex> lock(mu);
+    if (dev >= 64 || !((raised >> dev) & 1)) {
+      if (lsh_check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(qkv_attn_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem),
+                        "hipFuncSetAttribute(qkv_attn_kernel)"))
+        return LSH_ERR_HIP;
+      if (dev < 64) raised |= 1ull << dev;
+    }
+  }
+  const int hidden = head_num * dim_per_head;
+  const float alpha = __half2float(__float2half_rn(sqrtf(1.f / (float)dim_per_head)));
+  hipEvent_t e0 = g_qa_ev_start, e1 = g_qa_ev_stop;
+  g_qa_ev_start = g_qa_ev_stop = nullptr;
+  hipExtLaunchKernelGGL(qkv_attn_kernel, dim3(batch * head_num), dim3(256), smem, s, e0, e1, 0, x,
+                        qkv_weight, reinterpret_cast<const _Float16*>(qkv_bias), pad_mask, ctx_q,
+                        requant_alpha, dequant_scale, quant_scale, alpha, seq_len, batch, head_num,
+                        hidden);
+  return lsh_check_launch("qkv_attn_kernel");
+}
+
+}  // namespace lsh

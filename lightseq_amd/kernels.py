@@ -155,6 +155,18 @@ def encself_attention_i8qkv(qkv, qkv_bias, dequant_scale, src_padding_mask, ctx,
          head_num, dim_per_head, current_stream())
 
 
+def qkv_attention_i8(x, qkv_weight, qkv_bias, src_padding_mask, ctx_q, requant_alpha, dequant_scale,
+                     quant_scale, batch_size, batch_seq_len, head_num, dim_per_head):
+    """QKV projection + encoder attention in one kernel (heads of 64, at most 128 tokens):
+    the same bytes as gemm_i8_i8o(alpha=requant_alpha) followed by encself_attention_i8qkv."""
+    _dev(x, qkv_weight, qkv_bias, src_padding_mask, ctx_q)
+    if x.dtype != torch.int8 or qkv_weight.dtype != torch.int8 or qkv_bias.dtype != torch.float16:
+        raise TypeError("qkv_attention_i8 takes int8 activations and weights and an fp16 bias")
+    call("lsh_qkv_attention_i8_f16", ptr(x), ptr(qkv_weight), ptr(qkv_bias), ptr(src_padding_mask),
+         ptr(ctx_q), requant_alpha, dequant_scale, quant_scale, batch_size, batch_seq_len, head_num,
+         dim_per_head, current_stream())
+
+
 def launch_enc_emb_i8I(token_emb, pos_emb, tokens, output, pad_mask, pad_id, batch_size, seq_len,
                        hidden_dim, lang_emb, lang_id, multilg_type, dequant_scale, scaled):
     _dev(token_emb, pos_emb, tokens, output, pad_mask)

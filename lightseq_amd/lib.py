@@ -44,6 +44,7 @@ _SIGNATURES = {
     "lsh_ker_correlation_softmax_encself": (True, "iiispp"),
     "lsh_encself_attention_f16": (False, "pppppp" + "fiiiis"),
     "lsh_encself_attention_i8qkv_f16": (False, "ppfppp" + "fiiiis"),
+    "lsh_qkv_attention_i8_f16": (False, "ppppp" + "fff" + "iiiis"),
     "lsh_launch_enc_emb_i8I": (True, "ppppp" + "iiiispp" + "ifi"),
     "lsh_launch_scaled_colsum": (True, "ppiifs"),
     "lsh_gemm_i8_i32o": (False, "pppiiis"),

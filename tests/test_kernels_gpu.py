@@ -266,6 +266,46 @@ def test_encself_attention_fused(oracle, rng, B, S, h, d):
         assert np.all(got[b][:, mask[b] == 1, :] == 0)
 
 
+@pytest.mark.parametrize("B,S,h", [(2, 128, 4), (3, 50, 6), (8, 128, 12), (1, 7, 4), (16, 96, 4),
+                                   (5, 128, 16)])
+def test_qkv_projection_and_attention_in_one_kernel(rng, B, S, h):
+    """lsh_qkv_attention_i8 == the int8-output QKV GEMM followed by the attention on its codes,
+    byte for byte (the chain of quant_bert_encoder.cc.cu:305-347)."""
+    d = 64
+    H = h * d
+    x = rng.integers(-127, 128, size=(B * S, H), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(3 * H, H), dtype=np.int8)
+    bias = _randT(rng, (3 * H,), np.float16, 0.3)
+    mask = _pad_mask(rng, B, S)
+    # accumulators of K = H random products spread ~ 127^2 sqrt(H) / 3: alpha brings them to codes
+    alpha = 127.0 / (3.0 * 127 * 127 * np.sqrt(H) / 3.0)
+    ds, qs = 1.4 / 127, 127 / 0.9
+    xd, wd, bd, md = to_dev(x), to_dev(w), to_dev(bias), to_dev(mask)
+    codes = torch.zeros((B * S, 3 * H), dtype=torch.int8, device=DEV)
+    _k().gemm_i8_i8o(xd, wd, codes, B * S, 3 * H, H, alpha)
+    assert 20 < float(codes.float().abs().mean()) < 100          # the codes use their range
+    want = torch.full((B * S, H), 7, dtype=torch.int8, device=DEV)
+    _k().encself_attention_i8qkv(codes, bd, ds, md, None, want, qs, B, S, h, d)
+    got = torch.full((B * S, H), 9, dtype=torch.int8, device=DEV)
+    _k().qkv_attention_i8(xd, wd, bd, md, got, alpha, ds, qs, B, S, h, d)
+    np.testing.assert_array_equal(to_np(got), to_np(want))
+    assert to_np(got).any()
+
+
+def test_qkv_projection_and_attention_in_one_kernel_rejects_other_shapes(rng):
+    import lightseq_amd.lib as L
+    for B, S, h, d in [(2, 128, 4, 32), (2, 129, 4, 64), (2, 64, 2, 64), (2, 64, 3, 64)]:
+        H = h * d
+        x = torch.zeros((B * S, H), dtype=torch.int8, device=DEV)
+        w = torch.zeros((3 * H, H), dtype=torch.int8, device=DEV)
+        bias = torch.zeros((3 * H,), dtype=torch.float16, device=DEV)
+        mask = torch.zeros((B, S), dtype=torch.int32, device=DEV)
+        out = torch.zeros((B * S, H), dtype=torch.int8, device=DEV)
+        with pytest.raises(L.LSHError) as e:
+            _k().qkv_attention_i8(x, w, bias, mask, out, 1e-3, 0.01, 100.0, B, S, h, d)
+        assert e.value.code == L.LSH_ERR_UNSUPPORTED
+
+
 @pytest.mark.parametrize("B,S,h,d", [(2, 128, 3, 64), (3, 50, 2, 64), (1, 200, 2, 64), (2, 64, 4, 32),
                                      (1, 7, 1, 64), (2, 130, 2, 128)])
 def test_encself_attention_from_int8_qkv(oracle, rng, B, S, h, d):
