@@ -333,6 +333,51 @@ def _per_step_event_times(model, steps):
             "how": "HIP events on the model's stream around each Infer()"}
 
 
+def _write_model(cfg):
+    from lightseq_amd import synthetic
+    tmp = tempfile.mkdtemp(prefix="ls_bench_")
+    path = os.path.join(tmp, "quant_bert_base.pb")
+    synthetic.write_quant_bert(path, cfg, seed=0)
+    return path
+
+
+def two_batches_in_flight(path_factory, steps):
+    """Not the headline number: the same workload with two model instances (each with its own
+    stream and buffers) driven by two host threads, so that two batches of 32 x 128 are in
+    flight at once and the launch ramp and write-back of one instance's kernels overlap the
+    other's compute.  Every step is still one Infer() over one batch."""
+    import threading
+    import torch
+    from lightseq_amd import inference, synthetic
+    cfg = synthetic.bert_config("bert_base")
+    path = path_factory()
+    ids, _ = synthetic.make_token_ids(cfg, BATCH, SEQ, seed=0, min_len=32)
+    models = [inference.QuantBert(path, BATCH) for _ in range(2)]
+    os.remove(path)
+    for m in models:
+        m._upload(ids)
+        for _ in range(5):
+            m.infer_device()
+    torch.cuda.synchronize()
+
+    def loop(m):
+        for _ in range(steps):
+            m.infer_device()
+    threads = [threading.Thread(target=loop, args=(m,)) for m in models]
+    t0 = time.perf_counter()
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for m in models:
+        m.close()
+    return {"value": 2 * BATCH * SEQ * steps / dt, "unit": "tokens/s", "instances": 2,
+            "steps_per_instance": steps, "ms_per_step_per_instance": 1e3 * dt / steps,
+            "what": "two QuantBert instances on two host threads, one Infer() per batch each"}
+
+
 def bench_bert(args):
     import torch
     from lightseq_amd import inference, synthetic
@@ -403,6 +448,8 @@ def bench_bert(args):
     }
     model.close()
     if not args.no_fused:
+        out["two_batches_in_flight"] = two_batches_in_flight(path_factory=lambda: _write_model(cfg),
+                                                             steps=args.steps)
         out["fused_kernels"] = fused_kernel_rates(cfg)
         out["gemm_microbench"] = gemm_microbench()
     if not args.no_cpu_baseline:

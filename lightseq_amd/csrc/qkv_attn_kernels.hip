@@ -23,6 +23,7 @@
 #include <hip/hip_ext.h>
 
 #include <mutex>
+#include <type_traits>
 
 namespace lsh {
 
@@ -116,16 +117,15 @@ qkv_attn_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
       f.w[j] = *reinterpret_cast<const v4i*>(stage + (w_base[j] ^ (ks << 5)));
   };
   v16i acc[MB][NB];
-#pragma unroll
-  for (int i = 0; i < MB; ++i)
-#pragma unroll
-    for (int j = 0; j < NB; ++j) acc[i][j] = (v16i)0;
-  auto mma = [&](const Frag& f) {
+  // the first products of the tile start from a zero that is an operand of the instruction,
+  // not 96 cleared registers
+  auto mma = [&](const Frag& f, auto first) {
 #pragma unroll
     for (int i = 0; i < MB; ++i)
 #pragma unroll
       for (int j = 0; j < NB; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[j], f.a[i], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+            f.w[j], f.a[i], decltype(first)::value ? (v16i)0 : acc[i][j], 0, 0, 0);
   };
   // issue order of one slice: an LDS read of the next slice after each of the first MFMAs
   auto pattern = [&]() {
@@ -138,13 +138,29 @@ qkv_attn_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
     __builtin_amdgcn_sched_barrier(0);
   };
   Frag f[2];
-  auto slices = [&](const int8_t* stage) {  // slices 1..3 read, slices 0..2 multiplied
+  auto slices = [&](const int8_t* stage, auto first) {  // slices 1..3 read, slices 0..2 multiplied
 #pragma unroll
     for (int ks = 1; ks < 4; ++ks) {
       load_frag(f[ks & 1], stage, ks);
-      mma(f[(ks - 1) & 1]);
+      if (ks == 1) mma(f[0], first);
+      else mma(f[(ks - 1) & 1], std::false_type{});
       pattern();
     }
+  };
+  static_assert(NST == 2, "the step below refills the slot it has just read");
+  int slot = 0;
+  // one K step but the last: multiply the stage in `slot`, then refill it with step kt + 2
+  auto step = [&](int kt, auto first) {
+    slices(smem + slot * STAGE, first);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront has read all of the stage
+    wait_vmcnt<0>();                     // its own loads of step kt + 1 have landed ...
+    __builtin_amdgcn_s_barrier();        // ... and everyone's; everyone is done with step kt
+    if (kt + NST < nk) issue(kt + NST, slot);
+    __builtin_amdgcn_sched_barrier(0);
+    slot ^= 1;
+    load_frag(f[0], smem + slot * STAGE, 0);
+    mma(f[1], std::false_type{});
+    pattern();
   };
 
 #pragma unroll
@@ -152,34 +168,10 @@ qkv_attn_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
   wait_vmcnt<(NST - 1) * PER>();
   __builtin_amdgcn_s_barrier();
   load_frag(f[0], smem, 0);
-  int slot = 0;
-  // steady state: a step ends by refilling its own slot with step kt + NST
-  for (int kt = 0; kt < nk - NST; ++kt) {
-    slices(smem + slot * STAGE);
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront has read all of the stage
-    wait_vmcnt<(NST - 2) * PER>();       // its own loads of step kt + 1 have landed ...
-    __builtin_amdgcn_s_barrier();        // ... and everyone's; everyone is done with step kt
-    issue(kt + NST, slot);
-    __builtin_amdgcn_sched_barrier(0);
-    if (++slot == NST) slot = 0;
-    load_frag(f[0], smem + slot * STAGE, 0);
-    mma(f[1]);
-    pattern();
-  }
-  // drain: NST - 1 steps without a refill, then the last step
-#pragma unroll
-  for (int t = 0; t < NST - 1; ++t) {
-    slices(smem + slot * STAGE);
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-    if (++slot == NST) slot = 0;
-    load_frag(f[0], smem + slot * STAGE, 0);
-    mma(f[1]);
-    pattern();
-  }
-  slices(smem + slot * STAGE);
-  mma(f[1]);
+  step(0, std::true_type{});
+  for (int kt = 1; kt < nk - 1; ++kt) step(kt, std::false_type{});
+  slices(smem + slot * STAGE, std::false_type{});
+  mma(f[1], std::false_type{});
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_s_barrier();  // the ring is drained: its memory now holds q, k, v
 
@@ -195,9 +187,9 @@ qkv_attn_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W,
     for (int j = 0; j < NB; ++j) {
       // this lane's 16 accumulators are columns wn * 96 + j * 32 + 16 g .. + 16 of the tile
       const int blk = wn * NB + j, part = blk >> 1, d0 = (blk & 1) * 32 + 16 * g;
-      const uint4 codes = requant16_packed(acc[i][j], requant_alpha);
       v8h lo, hi;
-      dequant16_bias(codes, bias + part * hidden + head * D + d0, dq, lo, hi);
+      requant_dequant16_bias(acc[i][j], requant_alpha, bias + part * hidden + head * D + d0, dq, lo,
+                             hi);
       if (t >= S) lo = hi = (v8h)(_Float16)0;
       if (part == 2) {
 #pragma unroll

@@ -76,6 +76,24 @@ __device__ __forceinline__ void dequant16_bias(const uint4& w, const _Float16* _
   hi = xh + b1;
 }
 
+// 16 int32 accumulators -> the 16 fp16 values half(half(code * dq) + bias) of their int8 codes
+// code = requant_acc(acc, alpha), without forming the codes as bytes: floor(med3(y, -127, 127.5))
+// is the code as a float, and half(float(code) * dq) is what dequant16_bias computes from it.
+__device__ __forceinline__ void requant_dequant16_bias(const v16i& c, float alpha,
+                                                       const _Float16* __restrict__ bias, float dq,
+                                                       v8h& lo, v8h& hi) {
+  const v8h b0 = *reinterpret_cast<const v8h*>(bias);
+  const v8h b1 = *reinterpret_cast<const v8h*>(bias + 8);
+  v8h xl, xh;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    xl[j] = (_Float16)(floorf(requant_acc_clamped(c[j], alpha)) * dq);
+    xh[j] = (_Float16)(floorf(requant_acc_clamped(c[8 + j], alpha)) * dq);
+  }
+  lo = xl + b0;
+  hi = xh + b1;
+}
+
 // 8 int8 codes -> 8 fp16 values, the same arithmetic as dequant16_bias
 __device__ __forceinline__ v8h dequant8_bias(const uint2& w, const _Float16* __restrict__ bias,
                                              float dq) {
