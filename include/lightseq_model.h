@@ -76,6 +76,23 @@ int ls_model_get_profile(ls_model* model, char* buf, int capacity);
  * res_attn res_ffn (fp16 [tokens, hidden]: the residual stream as the LayerNorm kernel
  * after the attention out-projection / after FFN2 reads it).  dst NULL clears. */
 int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst);
+/* No counterpart in the reference.  Names that start with "dec." tap one generation step
+ * of QuantTransformer's decoder or of QuantGpt instead: the intermediate of decoder layer
+ * `layer` at the step given to ls_model_set_tap_step() (QuantTransformer: the decoding step,
+ * from 0; QuantGpt: the number of tokens sampled before the cached step, from 1).
+ * QuantTransformer (rows = batch * beam): dec.self_ln_q dec.self_q dec.self_ctx_q
+ * dec.self_out_q dec.encdec_ln_q dec.encdec_ctx_q dec.encdec_out_q dec.ffn_ln_q
+ * dec.next_ln_q (int8 [rows, hidden]), dec.ffn1_act_q (int8 [rows, inner]), dec.ffn2_acc
+ * (int32 [rows, hidden]), dec.self_k_cache dec.self_v_cache (int8 [rows, heads, max_step,
+ * d], after the step's append), dec.encdec_q (fp16 [batch, heads, beam, d]), dec.encdec_k
+ * dec.encdec_v (fp16 [batch, heads, src_len, d]), dec.res_in dec.res_self dec.res_encdec
+ * dec.res_out (fp16 [rows, hidden]: the residual stream at the start of the layer and
+ * after each of its three layer norms).
+ * QuantGpt (rows = batch): dec.ln1_q dec.self_q dec.ctx_q dec.out_q dec.ln2_q
+ * dec.next_ln_q (int8 [rows, hidden]), dec.act_q (int8 [rows, inner]), dec.ffn2_acc,
+ * dec.k_cache dec.v_cache, dec.res_in dec.res_attn dec.res_out.
+ * While any step tap is set the steps are not replayed as graphs. */
+int ls_model_set_tap_step(ls_model* model, int step);
 /* QuantTransformer only: the tap "enc_out" (layer ignored) receives the encoder output
  * [batch, seq_len, hidden] fp16 of every Infer().
  *

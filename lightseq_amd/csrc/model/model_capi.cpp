@@ -220,6 +220,19 @@ int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst) {
     qt->set_encoder_output_tap(static_cast<__half*>(dst));
     return LSH_OK;
   }
+  // "dec.<name>": an intermediate of a generation step of QuantTransformer's decoder or of
+  // QuantGpt (layer `layer`, at the step given to ls_model_set_tap_step)
+  if (!strncmp(name, "dec.", 4)) {
+    if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get())) {
+      qg->encoder()->step_taps.set(layer, name + 4, dst);
+      return LSH_OK;
+    }
+    if (QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get())) {
+      qt->decoder()->step_taps.set(layer, name + 4, dst);
+      return LSH_OK;
+    }
+    return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "step taps belong to QuantTransformer and QuantGpt");
+  }
   QuantBertEncoder* enc = encoder_of(model);
   if (!enc) return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "this model has no tapped encoder stack");
   auto& t = enc->taps;
@@ -237,6 +250,19 @@ int ls_model_set_tap(ls_model* model, int layer, const char* name, void* dst) {
   else if (!strcmp(name, "res_ffn")) t.res_ffn = static_cast<__half*>(dst);
   else return lsh::lsh_fail(LSH_ERR_INVALID, "unknown tap name");
   return LSH_OK;
+}
+
+int ls_model_set_tap_step(ls_model* model, int step) {
+  NEED_MODEL(model);
+  if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get())) {
+    qg->encoder()->step_taps.set_step(step);
+    return LSH_OK;
+  }
+  if (QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get())) {
+    qt->decoder()->step_taps.set_step(step);
+    return LSH_OK;
+  }
+  return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "step taps belong to QuantTransformer and QuantGpt");
 }
 
 int ls_model_set_step_record(ls_model* model, int8_t* logits, int* alive_seq, int max_steps) {

@@ -8,6 +8,7 @@
 
 #include <cstdint>
 #include <stdexcept>
+#include <map>
 #include <string>
 #include <unordered_map>
 #include <unordered_set>
@@ -66,6 +67,33 @@ class DeviceBuffer {
   }
   T* p_ = nullptr;
   size_t n_ = 0;
+};
+
+// Debug taps of a generation step (parity bisection): device-to-device copies of named
+// intermediates of decoder layer `layer` at step `step` into buffers the caller owns.  A name
+// registered with a null pointer is forgotten.  A layer < 0 at the copy site means "any".
+class StepTaps {
+ public:
+  void set(int layer, const std::string& name, void* dst) {
+    _layer = layer;
+    if (dst) _dst[name] = dst;
+    else _dst.erase(name);
+  }
+  void set_step(int step) { _step = step; }
+  bool any() const { return !_dst.empty(); }
+  bool wants(int layer, int step, const char* name) const {
+    return !_dst.empty() && step == _step && (layer < 0 || layer == _layer) && _dst.count(name);
+  }
+  void copy(int layer, int step, const char* name, const void* src, size_t bytes,
+            hipStream_t stream) const {
+    if (!wants(layer, step, name)) return;
+    if (hipMemcpyAsync(_dst.at(name), src, bytes, hipMemcpyDeviceToDevice, stream) != hipSuccess)
+      throw std::runtime_error(std::string("tap copy failed: ") + name);
+  }
+
+ private:
+  int _layer = -1, _step = -1;
+  std::map<std::string, void*> _dst;
 };
 
 // HIP graphs of a generation step.  A step is a fixed sequence of launches whose arguments

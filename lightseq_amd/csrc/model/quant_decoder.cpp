@@ -256,7 +256,8 @@ bool QuantDecoder::run_step() {
   // two sequence / cache buffers is current: one graph per such key.
   const uint64_t key = ((uint64_t)_batch_size << 40) | ((uint64_t)_batch_seq_len << 24) |
                        ((uint64_t)_cur_step << 8) | (uint64_t)(_alive_cur << 1 | _cache_cur);
-  _graphs.run(key, _stream, _use_graphs && !_rec_logits && !_rec_alive, [&] { enqueue_step(); });
+  _graphs.run(key, _stream, _use_graphs && !_rec_logits && !_rec_alive && !step_taps.any(),
+              [&] { enqueue_step(); });
   ++_steps_run;
   _alive_cur ^= 1;
   if (_cur_step > 0) _cache_cur ^= 1;
@@ -292,6 +293,15 @@ void QuantDecoder::enqueue_step() {
   beam_search();
 }
 
+// Step taps (debug): name -> what is copied, of layer step_taps' layer at its step.
+//   self_ln_q, self_q, self_ctx_q, self_out_q, encdec_ln_q, encdec_ctx_q, encdec_out_q, ffn_ln_q,
+//   next_ln_q: int8 [rows, hidden];  ffn1_act_q: int8 [rows, inner];  ffn2_acc: int32 [rows, hidden]
+//   self_k_cache, self_v_cache: the layer's int8 caches [rows, heads, max_step, d] after the append
+//   encdec_q: fp16 [batch, heads, beam, d];  encdec_k, encdec_v: fp16 [batch, heads, src_len, d]
+//   res_in, res_self, res_encdec, res_out: the fp16 residual stream [rows, hidden] at the start of
+//   the layer, after the first, the second and the last layer norm
+#define TAP(name, ptr, bytes) step_taps.copy(_layer_id, _cur_step, name, ptr, bytes, _stream)
+
 void QuantDecoder::embedding() {
   LSH_CALL(dec_emb_i8I<__half>(_int8_trg_emb.get(), _pos_emb.get(), _alive_seq[_alive_cur].get(),
                                _cur_step_query.get(), _batch_size, _tw._beam_size,
@@ -312,6 +322,9 @@ void QuantDecoder::self_attention() {
                                            w.self_ln_scale.get(), w.self_ln_bias.get(),
                                            w.b_self_out.get(), Q / c[6], _tw._is_post_ln));
   }
+  const size_t mh = (size_t)M * H;
+  TAP("self_ln_q", _buf_a.get(), mh);
+  TAP("res_in", _cur_step_query.get(), mh * sizeof(__half));
   // QKV product; its epilogue is ker_arrange_decself_qkv_i8I_i8O: q -> _buf_q, k / v -> slot
   // _cur_step of the caches (all three with the cache clip)
   if (_tw._dim_per_head % 16 == 0) {
@@ -327,18 +340,25 @@ void QuantDecoder::self_attention() {
                                                  _tw._dim_per_head, _tw._max_step, _cur_step,
                                                  c[12] / Q, Q / c[18]));
   }
+  TAP("self_q", _buf_q.get(), mh);
+  TAP("self_k_cache", k_cache, mh * _tw._max_step);
+  TAP("self_v_cache", v_cache, mh * _tw._max_step);
   // int8 q.K -> softmax -> new value, one kernel
   const float attn_scale =
       __half2float(__float2half_rn(sqrtf(1.f / (float)_tw._dim_per_head)));
   LSH_CALL(decself_attention_i8(_buf_q.get(), k_cache, v_cache, _buf_b.get(), M * _tw._head_num,
                                 _cur_step + 1, _tw._max_step, _tw._head_num, _tw._dim_per_head,
                                 attn_scale, c[18] / Q, Q / c[7], _stream));
+  TAP("self_ctx_q", _buf_b.get(), mh);
   LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_self_out.get(), _buf_a.get(), M, H, H,
                        c[1] * c[7] / (c[13] * Q), _stream));
+  TAP("self_out_q", _buf_a.get(), mh);
   LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(
       _buf_a.get(), w.encdec_ln_scale.get(), w.encdec_ln_bias.get(), w.b_encdec_out.get(),
       _buf_b.get(), _cur_step_query.get(), M, H, c[13] / Q, Q / c[8], _stream, _tw._is_post_ln,
       nullptr)));
+  TAP("encdec_ln_q", _buf_b.get(), mh);
+  TAP("res_self", _cur_step_query.get(), mh * sizeof(__half));
 }
 
 void QuantDecoder::encdec_attention() {
@@ -359,17 +379,27 @@ void QuantDecoder::encdec_attention() {
                                           _query_buf1.get(), _tw._beam_size, _tw._dim_per_head,
                                           _tw._head_num, c[14] / Q));
   }
+  const size_t mh = (size_t)M * H;
+  TAP("encdec_q", _query_buf1.get(), mh * sizeof(__half));
+  TAP("encdec_k", _encdec_k.get() + (size_t)_layer_id * _layer_size_encdec_k,
+      (size_t)_batch_token_num * H * sizeof(__half));
+  TAP("encdec_v", _encdec_v.get() + (size_t)_layer_id * _layer_size_encdec_k,
+      (size_t)_batch_token_num * H * sizeof(__half));
   // scores -> masked softmax -> context -> merge heads + quantise, one kernel
   LSH_CALL(encdec_attention_f16(
       _query_buf1.get(), _encdec_k.get() + (size_t)_layer_id * _layer_size_encdec_k,
       _encdec_v.get() + (size_t)_layer_id * _layer_size_encdec_k, _p_d_padding_mask, nullptr,
       _buf_b.get(), Q / c[9], _batch_size, _tw._beam_size, _tw._head_num, _batch_seq_len,
       _tw._dim_per_head, _stream));
+  TAP("encdec_ctx_q", _buf_b.get(), mh);
   LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_encdec_out.get(), _buf_a.get(), M, H, H,
                        c[3] * c[9] / (c[15] * Q), _stream));
+  TAP("encdec_out_q", _buf_a.get(), mh);
   LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(
       _buf_a.get(), w.ffn_ln_scale.get(), w.ffn_ln_bias.get(), w.b_ffn2.get(), _buf_b.get(),
       _cur_step_query.get(), M, H, c[15] / Q, Q / c[10], _stream, _tw._is_post_ln, nullptr)));
+  TAP("ffn_ln_q", _buf_b.get(), mh);
+  TAP("res_encdec", _cur_step_query.get(), mh * sizeof(__half));
 }
 
 void QuantDecoder::ffn_add_norm() {
@@ -381,9 +411,14 @@ void QuantDecoder::ffn_add_norm() {
   // FFN1 GEMM with the bias + activation + requantisation in its epilogue
   LSH_CALL(gemm_i8_lut_i8o(_buf_b.get(), w.w_ffn1.get(), _buf_a.get(), w.ffn1_act_lut.get(), M, I,
                            H, c[4] * c[10] / (c[16] * Q), _stream));
+  TAP("ffn1_act_q", _buf_a.get(), (size_t)M * I);
   int nparts = 1;
+  // a tapped accumulator is one plane (the planes of a split product sum to it exactly)
+  const bool tap_acc = step_taps.wants(_layer_id, _cur_step, "ffn2_acc");
   LSH_CALL(gemm_i8_i32o_splitk(_buf_a.get(), w.w_ffn2.get(), _int32_ffn_out_buf.get(), M, H, I,
-                               gemm_i8_preferred_ksplit(M, H, I), &nparts, _stream));
+                               tap_acc ? 1 : gemm_i8_preferred_ksplit(M, H, I), &nparts,
+                               _stream));
+  TAP("ffn2_acc", _int32_ffn_out_buf.get(), (size_t)M * H * sizeof(int32_t));
 
   const float dequant_scale =
       _tw._use_gelu ? c[5] * c[11] / (Q * Q) : c[5] * c[11] / (2 * Q * Q);
@@ -405,7 +440,11 @@ void QuantDecoder::ffn_add_norm() {
       _int32_ffn_out_buf.get(), scale_ptr, bias_ptr, res_bias_ptr, _buf_a.get(),
       _cur_step_query.get(), M, H, dequant_scale, Q / clip_max, _stream, _tw._is_post_ln,
       w.ffn2_colsum.get(), nparts, (long)M * H)));
+  TAP("next_ln_q", _buf_a.get(), (size_t)M * H);
+  TAP("res_out", _cur_step_query.get(), (size_t)M * H * sizeof(__half));
 }
+
+#undef TAP
 
 void QuantDecoder::beam_search() {
   int* alive = _alive_seq[_alive_cur].get();

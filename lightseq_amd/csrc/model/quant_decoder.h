@@ -44,6 +44,8 @@ class QuantDecoder {
   // Replay decoding steps through HIP graphs, one per (batch, source length, step, buffer
   // parity): see StepGraphs.  Off while a step record is set.
   void graph_mode(bool on) { _use_graphs = on; }
+  // copies of the intermediates of one layer at one step (names: see quant_decoder.cpp)
+  StepTaps step_taps;
   int graphs_captured() const { return _graphs.captured(); }
   long graphs_replayed() const { return _graphs.replayed(); }
 

@@ -113,6 +113,13 @@ void QuantGptEncoder::init_buffer() {
 
 // FFN block and the LayerNorm that follows it (:646-776).  `in` holds the int8
 // LayerNorm output and receives the next one; `tmp` is scratch of the same size.
+// Step taps (debug): name -> what is copied, of the tapped layer at the tapped cached step.
+//   ln1_q, self_q, ctx_q, out_q, ln2_q, next_ln_q: int8 [batch, hidden];  act_q: int8 [batch, inner]
+//   ffn2_acc: int32 [batch, hidden];  k_cache, v_cache: the layer's int8 caches [batch, heads,
+//   max_step, d] after the append;  res_in, res_attn, res_out: the fp16 residual stream [batch,
+//   hidden] at the start of the layer, after the first and after the last layer norm
+#define TAP(name, ptr, bytes) step_taps.copy(_layer_id, _tap_step, name, ptr, bytes, _stream)
+
 void QuantGptEncoder::ffn_add_norm(int rows, int8_t* in, int8_t* tmp) {
   const int H = _tw._hidden_size, I = _tw._inner_size;
   const Layer& w = _layers[_layer_id];
@@ -120,11 +127,16 @@ void QuantGptEncoder::ffn_add_norm(int rows, int8_t* in, int8_t* tmp) {
   const float Q = _quant_range;
   LSH_CALL(gemm_i8_lut_i8o(in, w.w_ffn1.get(), tmp, w.ffn1_act_lut.get(), rows, I, H,
                            c[2] * c[6] / (c[10] * Q), _stream));
+  TAP("act_q", tmp, (size_t)rows * I);
   int nparts = 1;
+  // a tapped accumulator is one plane (the planes of a split product sum to it exactly)
+  const bool tap_acc = step_taps.wants(_layer_id, _tap_step, "ffn2_acc");
   LSH_CALL(gemm_i8_i32o_splitk(tmp, w.w_ffn2.get(), _int32_ffn_out_buf.get(), rows, H, I,
-                               rows <= 64 ? gemm_i8_preferred_ksplit(rows, H, I)
-                                          : std::min(4, gemm_i8_preferred_ksplit(rows, H, I)),
+                               tap_acc      ? 1
+                               : rows <= 64 ? gemm_i8_preferred_ksplit(rows, H, I)
+                                            : std::min(4, gemm_i8_preferred_ksplit(rows, H, I)),
                                &nparts, _stream));
+  TAP("ffn2_acc", _int32_ffn_out_buf.get(), (size_t)rows * H * sizeof(int32_t));
   const float dequant_scale = c[3] * c[7] / (Q * Q);
   const __half *scale_ptr, *bias_ptr, *res_bias_ptr;
   float clip_max;
@@ -143,6 +155,8 @@ void QuantGptEncoder::ffn_add_norm(int rows, int8_t* in, int8_t* tmp) {
   LSH_CALL((residual_bias_ln_i8O<__half, int32_t>(
       _int32_ffn_out_buf.get(), scale_ptr, bias_ptr, res_bias_ptr, in, _query.get(), rows, H,
       dequant_scale, Q / clip_max, _stream, false, nullptr, nparts, (long)rows * H)));
+  TAP("next_ln_q", in, (size_t)rows * H);
+  TAP("res_out", _query.get(), (size_t)rows * H * sizeof(__half));
 }
 
 // all prompt positions at once (:253-291 / :299-341); leaves the int8 LayerNorm output of
@@ -193,6 +207,8 @@ const int8_t* QuantGptEncoder::step_pass() {
                                      _tw._padding_id, _batch_seq_len - 1, _src_emb_clip_max / Q,
                                      _tw._src_vocab_size, _tw._max_step));
   int8_t *a = _buf_a.get(), *b = _buf_b.get();
+  _tap_step = _steps_run;
+  const size_t bh = (size_t)B * H;
   for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
     const Layer& w = _layers[_layer_id];
     const float* c = &_enc_clip_max[_layer_id * 12];
@@ -201,6 +217,8 @@ const int8_t* QuantGptEncoder::step_pass() {
     if (_layer_id == 0)
       LSH_CALL(norm_layer_resual_i8O<__half>(B, H, _stream, _query.get(), a, w.ln1_scale.get(),
                                              w.ln1_bias.get(), w.b_out.get(), Q / c[4], false));
+    TAP("ln1_q", a, bh);
+    TAP("res_in", _query.get(), bh * sizeof(__half));
     // QKV product; its epilogue is ker_arrange_decself_qkv_i8I_i8O: q -> _buf_q, k / v appended
     // to the caches at the token's position
     if (_tw._dim_per_head % 16 == 0) {
@@ -215,19 +233,29 @@ const int8_t* QuantGptEncoder::step_pass() {
                                                    _tw._dim_per_head, _tw._max_step,
                                                    _batch_seq_len - 1, c[8] / Q, Q / c[11]));
     }
+    TAP("self_q", _buf_q.get(), bh);
+    TAP("k_cache", k_cache, bh * _tw._max_step);
+    TAP("v_cache", v_cache, bh * _tw._max_step);
     LSH_CALL(decself_attention_i8(_buf_q.get(), k_cache, v_cache, b, B * _tw._head_num,
                                   _batch_seq_len,
                                   _tw._max_step, _tw._head_num, _tw._dim_per_head, _atten_scaler,
                                   c[11] / Q, Q / c[5], _stream));
+    TAP("ctx_q", b, bh);
     LSH_CALL(gemm_i8_i8o(b, w.w_out.get(), a, B, H, H, c[1] * c[5] / (c[9] * Q), _stream));
+    TAP("out_q", a, bh);
     LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(a, w.ln2_scale.get(), w.ln2_bias.get(),
                                                    w.b_ffn2.get(), b, _query.get(), B, H,
                                                    c[9] / Q, Q / c[6], _stream, false, nullptr)));
+    TAP("ln2_q", b, bh);
+    TAP("res_attn", _query.get(), bh * sizeof(__half));
     ffn_add_norm(B, b, a);
     std::swap(a, b);  // `a` names the buffer holding the layer's int8 LayerNorm output
   }
+  _tap_step = -2;
   return a;
 }
+
+#undef TAP
 
 // logits of the last position + greedy choice, enqueued only (:399-487)
 void QuantGptEncoder::enqueue_sampling(const int8_t* hidden) {
@@ -289,7 +317,7 @@ int QuantGptEncoder::run_one_sample(int batch_size, int batch_seq_len) {
       while (_batch_seq_len < _batch_max_seq_len) {
         // the launches of a step depend on the batch size and the position only
         const uint64_t key = ((uint64_t)_batch_size << 32) | (uint32_t)_batch_seq_len;
-        _graphs.run(key, _stream, _use_graphs && !_rec_logits,
+        _graphs.run(key, _stream, _use_graphs && !_rec_logits && !step_taps.any(),
                     [&] { enqueue_sampling(step_pass()); });
         int unfinished = finish_token();
         if (!unfinished && !_is_benchmark) break;

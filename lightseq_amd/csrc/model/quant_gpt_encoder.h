@@ -44,6 +44,8 @@ class QuantGptEncoder {
   // Replay the cached steps through HIP graphs, one per (batch size, position): see StepGraphs.
   // Off while a step record is set.
   void graph_mode(bool on) { _use_graphs = on; }
+  // copies of the intermediates of one layer at one cached step (names: see step_pass)
+  StepTaps step_taps;
   int graphs_captured() const { return _graphs.captured(); }
   long graphs_replayed() const { return _graphs.replayed(); }
 
@@ -74,6 +76,7 @@ class QuantGptEncoder {
   long _max_batch_dim;
   int* _h_unfinished = nullptr;  // pinned
   int8_t* _rec_logits = nullptr;
+  int _tap_step = -2;  // the cached step being enqueued (tokens sampled so far), -2 outside one
   int _rec_max_steps = 0;
 
   DeviceBuffer<int> _real_seq_len, _ids, _last_ids, _unfinished;

@@ -52,6 +52,7 @@ def _bind():
         "ls_model_benchmark_mode": [_P, _I],
         "ls_model_get_stream": [_P, pp],
         "ls_model_set_tap": [_P, _I, ctypes.c_char_p, _P],
+        "ls_model_set_tap_step": [_P, _I],
         "ls_model_set_profiling": [_P, _I],
         "ls_model_get_profile": [_P, ctypes.c_char_p, _I],
         "ls_model_set_step_record": [_P, _P, _P, _I],
@@ -181,6 +182,10 @@ class LSModel:
         cap, rep = ctypes.c_int(0), ctypes.c_longlong(0)
         self._call("ls_model_get_graph_stats", self._h, ctypes.byref(cap), ctypes.byref(rep))
         return cap.value, rep.value
+
+    def set_tap_step(self, step):
+        """The generation step whose "dec.*" taps are copied (QuantTransformer, QuantGpt)."""
+        self._call("ls_model_set_tap_step", self._h, int(step))
 
     def set_tap(self, layer, name, tensor):
         self._call("ls_model_set_tap", self._h, int(layer), name.encode(),

@@ -246,8 +246,11 @@ def _check_sample(msg, cfg, ids, out, steps, logits, benchmark=False):
           (steps, 100 * frac, 100 * frac2, diff.max()))
     # every int8-output GEMM turns one flipped input code into +-1 flips on a few percent
     # of its outputs, so rows that saw a flip upstream are decorrelated at the rounding level
-    assert diff.max() <= 6
-    assert frac2 <= 2e-2 and frac <= 0.4
+    # (every stage of a cached step is held to its own bar, on the GPU's own stage inputs, by
+    # test_cached_step_stage_by_stage_at_gpt2_medium_width; this bounds the drift of two runs
+    # that each read their own caches)
+    assert diff.max() <= 4
+    assert frac2 <= 1e-2 and frac <= 0.25
     return w, r
 
 
@@ -339,6 +342,102 @@ def test_gpt2_medium_shape(tmp_path):
     out, steps, logits = _run_sample(path, cfg, ids, max_batch=2)
     assert steps >= 1 and out.shape[1] == 48 + steps
     _check_sample(msg, cfg, ids, out, steps, logits)
+
+
+GPT_TAPS_I8 = ["ln1_q", "self_q", "ctx_q", "out_q", "ln2_q", "next_ln_q"]
+GPT_TAPS_F16 = ["res_in", "res_attn", "res_out"]
+
+
+def _gpt_step_taps(path, cfg, ids, layer, step):
+    """One sample() with every intermediate of layer `layer` at cached step `step` tapped."""
+    from lightseq_amd.inference import QuantGpt
+    batch = ids.shape[0]
+    H, I, h = cfg["hidden"], cfg["inner"], cfg["head_num"]
+    model = QuantGpt(path, batch)
+    t = {n: torch.zeros(batch, H, dtype=torch.int8, device=DEV) for n in GPT_TAPS_I8}
+    t.update({n: torch.zeros(batch, H, dtype=torch.float16, device=DEV) for n in GPT_TAPS_F16})
+    t["act_q"] = torch.zeros(batch, I, dtype=torch.int8, device=DEV)
+    t["ffn2_acc"] = torch.zeros(batch, H, dtype=torch.int32, device=DEV)
+    for n in ("k_cache", "v_cache"):
+        t[n] = torch.zeros(batch, h, cfg["max_step"], H // h, dtype=torch.int8, device=DEV)
+    for n, buf in t.items():
+        model.set_tap(layer, "dec." + n, buf)
+    model.set_tap_step(step)
+    model.benchmark_mode(True)   # no early stop: the tapped step is reached
+    model.sample(ids)
+    steps = model.steps_run()
+    out = {n: buf.cpu().numpy() for n, buf in t.items()}
+    model.close()
+    return out, steps
+
+
+def _check_gpt_step_stages(w, cfg, tp, layer, pos):
+    """Every stage of one layer of a cached step (the new token sits at position `pos`) against
+    the oracle's kernel for that stage, each fed the GPU's own stage input
+    (model/quant_gpt_encoder.cc.cu:560-760): int8 GEMM outputs, the appended cache rows and the
+    int32 FFN2 accumulator bit for bit, layer-norm and attention codes within one code on at most
+    0.1 % of the elements."""
+    from oracle import oracle
+    Q = np.float32(127)
+    c = w["clip_max"][layer * 12:(layer + 1) * 12]
+    h, H = cfg["head_num"], cfg["hidden"]
+    d = H // h
+    W = lambda name: w[name][layer]
+    eq = np.testing.assert_array_equal
+
+    codes = oracle.gemm_i8_i8(tp["ln1_q"], W("w_qkv"), c[0] * c[4] / (c[8] * Q))
+    k_c, v_c = tp["k_cache"].copy(), tp["v_cache"].copy()
+    k_c[:, :, pos, :] = 99
+    v_c[:, :, pos, :] = 99
+    new_q = oracle.arrange_decself_qkv_i8I_i8O(codes, W("b_qkv"), k_c, v_c, pos, c[8] / Q, Q / c[11])
+    eq(tp["self_q"], new_q)
+    eq(tp["k_cache"][:, :, :pos + 1], k_c[:, :, :pos + 1])
+    eq(tp["v_cache"][:, :, :pos + 1], v_c[:, :, :pos + 1])
+    scores = oracle.decself_scores(tp["self_q"], tp["k_cache"], pos + 1)
+    attn_scale = float(np.float16(np.sqrt(np.float32(1.0) / np.float32(d))))
+    ctx = oracle.fuse_softmax_new_value_i32I_i8O(scores, tp["v_cache"], pos + 1, attn_scale, c[11] / Q,
+                                                 Q / c[5])
+    assert_codes_close(tp["ctx_q"], ctx, max_frac=1e-3, what="cached self-attention context")
+    eq(tp["out_q"], oracle.gemm_i8_i8(tp["ctx_q"], W("w_out"), c[1] * c[5] / (c[9] * Q)))
+    ln_q, res = oracle.residual_bias_ln_i8O(tp["out_q"], W("ln2_scale"), W("ln2_bias"), W("b_ffn2"),
+                                            tp["res_in"], c[9] / Q, Q / c[6], False)
+    assert_codes_close(tp["ln2_q"], ln_q, max_frac=1e-3, what="layer norm before the FFN")
+    np.testing.assert_allclose(tp["res_attn"].astype(np.float32), res.astype(np.float32), atol=2e-2)
+
+    codes = oracle.gemm_i8_i8(tp["ln2_q"], W("w_ffn1"), c[2] * c[6] / (c[10] * Q))
+    eq(tp["act_q"], oracle.bias_gelu_i8I_i8O(codes, W("b_ffn1"), c[10] / Q, Q / c[7]))
+    eq(tp["ffn2_acc"], oracle.gemm_i8_i32(tp["act_q"], W("w_ffn2")))
+    if layer == w["n_layer"] - 1:
+        sc_, bi_, rb_, clip = w["out_ln_scale"], w["out_ln_bias"], None, w["output_ln_clip_max"]
+    else:
+        sc_, bi_, rb_ = w["ln1_scale"][layer + 1], w["ln1_bias"][layer + 1], w["b_out"][layer + 1]
+        clip = w["clip_max"][(layer + 1) * 12 + 4]
+    ln_q, res = oracle.residual_bias_ln_i8O(tp["ffn2_acc"], sc_, bi_, rb_, tp["res_attn"],
+                                            c[3] * c[7] / (Q * Q), Q / clip, False)
+    assert_codes_close(tp["next_ln_q"], ln_q, max_frac=1e-3, what="layer norm after the FFN")
+    np.testing.assert_allclose(tp["res_out"].astype(np.float32), res.astype(np.float32), atol=2e-2)
+
+
+@pytest.mark.parametrize("layer", [0, 1])
+def test_cached_step_stage_by_stage_at_gpt2_medium_width(tmp_path, layer):
+    """One cached step of a GPT-2-medium-shaped model (hidden 1024, 16 heads, inner 4096), stage
+    by stage through the step taps, at the first cached step, a middle one and the last."""
+    from lightseq_amd import synthetic
+    cfg = synthetic.gpt_config("gpt2_medium")
+    cfg.update(n_layer=2, max_step=96, extra_decode_length=24)
+    path, msg = _make(tmp_path, cfg, 12, w_std=0.05)
+    prompt_len = 48
+    ids = _prompt(cfg, 2, prompt_len, 12)
+    w = _og().gpt_weights_from_message(msg, cfg, np.float16)
+    last = None
+    for step in (1, 11, -1):
+        if step < 0:
+            step = last
+        tp, steps = _gpt_step_taps(path, cfg, ids, layer, step)
+        last = steps - 1
+        assert 1 <= step < steps
+        assert np.abs(tp["ln1_q"]).max() > 0 and np.abs(tp["ffn2_acc"]).max() > 0
+        _check_gpt_step_stages(w, cfg, tp, layer, prompt_len + step - 1)
 
 
 def test_gpt2_medium_full_size_properties(tmp_path):

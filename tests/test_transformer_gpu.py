@@ -106,8 +106,11 @@ def _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch):
     d0 = diff[0]
     assert d0.max() <= 3 and (d0 > 1).mean() <= 2e-3 and (d0 != 0).mean() <= 0.1, \
         "step 0 logits differ: max %d, %.3f%% != 0" % (d0.max(), 100 * (d0 != 0).mean())
-    assert diff.max() <= 6, "logit codes differ by %d" % diff.max()
-    assert frac2 <= 2e-2, "%.3f%% of logit codes differ by more than one code" % (100 * frac2)
+    # (every stage of a step is held to its own bar, on the GPU's own stage inputs, by
+    # test_decoder_step_stage_by_stage_at_transformer_big_width; what is bounded here is how far
+    # two runs that each read their own caches drift apart at the rounding level)
+    assert diff.max() <= 4, "logit codes differ by %d" % diff.max()
+    assert frac2 <= 1.2e-2, "%.3f%% of logit codes differ by more than one code" % (100 * frac2)
     assert frac <= max_logit_mismatch, "%.3f%% of logit codes differ" % (100 * frac)
     return r, frac
 
@@ -130,7 +133,7 @@ def test_tiny_transformer(oracle, tmp_path, seed, eos, batch, seq):
     gpu = _run_gpu(path, cfg, ids, max_batch=4)
     assert gpu["tokens"].shape[:2] == (batch, cfg["beam_size"])
     assert gpu["scores"].shape == (batch, cfg["beam_size"])
-    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.02)
 
     # free-running oracle (its own encoder output and logits): identical ids
     enc_w, dec_w = _oracle_weights(msg, cfg)
@@ -153,7 +156,7 @@ def test_early_stop_and_benchmark_mode(oracle, tmp_path):
     limit = min(cfg["max_step"], ids.shape[1] + cfg["extra_decode_length"]) - 1
     assert gpu["steps"] < limit - 1, "expected an early stop"
     assert gpu["tokens"].shape[2] == gpu["steps"]
-    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.02)
 
     bench = _run_gpu(path, cfg, ids, max_batch=3, benchmark=True)
     assert bench["steps"] == limit - 1
@@ -175,7 +178,7 @@ def test_gelu_post_ln_variant(oracle, tmp_path):
     path, msg = _make(tmp_path, cfg, 5, eos_bias=2.0 * sigma, w_std=0.2)
     ids = _src_ids(cfg, 2, 9, 5)
     gpu = _run_gpu(path, cfg, ids, max_batch=2)
-    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.02)
 
 
 def test_repeated_infer_is_deterministic(tmp_path):
@@ -239,8 +242,143 @@ def test_transformer_big_shape(oracle, tmp_path):
     path, msg = _make(tmp_path, cfg, 11, eos_bias=2.5 * sigma, w_std=0.05)
     ids = _src_ids(cfg, 4, 16, 3)
     gpu = _run_gpu(path, cfg, ids, max_batch=4)
-    _, frac = _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.4)
+    _, frac = _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.33)
     print("transformer-big shape: %d steps, %.3f%% logit codes differ" % (gpu["steps"], 100 * frac))
+
+
+DEC_TAPS_I8 = ["self_ln_q", "self_q", "self_ctx_q", "self_out_q", "encdec_ln_q", "encdec_ctx_q",
+               "encdec_out_q", "ffn_ln_q", "next_ln_q"]
+DEC_TAPS_F16 = ["res_in", "res_self", "res_encdec", "res_out"]
+
+
+def _decoder_step_taps(path, cfg, ids, layer, step):
+    """One Infer() with every intermediate of decoder layer `layer` at step `step` tapped."""
+    from lightseq_amd.inference import QuantTransformer
+    batch, seq = ids.shape
+    H, I, h = cfg["hidden"], cfg["inner"], cfg["head_num"]
+    rows, d = batch * cfg["beam_size"], H // h
+    model = QuantTransformer(path, batch)
+    t = {n: torch.zeros(rows, H, dtype=torch.int8, device=DEV) for n in DEC_TAPS_I8}
+    t.update({n: torch.zeros(rows, H, dtype=torch.float16, device=DEV) for n in DEC_TAPS_F16})
+    t["ffn1_act_q"] = torch.zeros(rows, I, dtype=torch.int8, device=DEV)
+    t["ffn2_acc"] = torch.zeros(rows, H, dtype=torch.int32, device=DEV)
+    for n in ("self_k_cache", "self_v_cache"):
+        t[n] = torch.zeros(rows, h, cfg["max_step"], d, dtype=torch.int8, device=DEV)
+    t["encdec_q"] = torch.zeros(batch, h, cfg["beam_size"], d, dtype=torch.float16, device=DEV)
+    for n in ("encdec_k", "encdec_v"):
+        t[n] = torch.zeros(batch, h, seq, d, dtype=torch.float16, device=DEV)
+    for n, buf in t.items():
+        model.set_tap(layer, "dec." + n, buf)
+    model.set_tap_step(step)
+    model.benchmark_mode(True)   # no early stop: the tapped step is reached
+    model.infer(ids)
+    steps = model.steps_run()
+    out = {n: buf.cpu().numpy() for n, buf in t.items()}
+    model.close()
+    return out, steps
+
+
+def _check_decoder_step_stages(oracle, dec_w, cfg, mask, tp, layer, step):
+    """Every stage of one decoder layer at one step against the oracle's kernel for that
+    stage, each fed the GPU's own stage input (model/quant_decoder.cc.cu:620-949): int8 GEMM
+    outputs, appended cache rows and the int32 FFN2 accumulator bit for bit, layer-norm and
+    attention codes within one code on at most 0.1 % / 0.5 % of the elements."""
+    from conftest import assert_codes_close
+    Q = np.float32(127)
+    c = dec_w["clip_max"][layer * 19:(layer + 1) * 19]
+    beam, h = cfg["beam_size"], cfg["head_num"]
+    H = cfg["hidden"]
+    d = H // h
+    post = dec_w["is_post_ln"]
+    W = lambda name: dec_w[name][layer]
+    eq = np.testing.assert_array_equal
+
+    # self attention: QKV product + split / cache append
+    codes = oracle.gemm_i8_i8(tp["self_ln_q"], W("w_self_qkv"), c[0] * c[6] / (c[12] * Q))
+    k_c, v_c = tp["self_k_cache"].copy(), tp["self_v_cache"].copy()
+    k_c[:, :, step, :] = 99
+    v_c[:, :, step, :] = 99
+    new_q = oracle.arrange_decself_qkv_i8I_i8O(codes, W("b_self_qkv"), k_c, v_c, step, c[12] / Q,
+                                               Q / c[18])
+    eq(tp["self_q"], new_q)
+    eq(tp["self_k_cache"][:, :, :step + 1], k_c[:, :, :step + 1])
+    eq(tp["self_v_cache"][:, :, :step + 1], v_c[:, :, :step + 1])
+    # int8 scores -> softmax -> new value
+    scores = oracle.decself_scores(tp["self_q"], tp["self_k_cache"], step + 1)
+    attn_scale = float(np.float16(np.sqrt(np.float32(1.0) / np.float32(d))))
+    ctx = oracle.fuse_softmax_new_value_i32I_i8O(scores, tp["self_v_cache"], step + 1, attn_scale,
+                                                 c[18] / Q, Q / c[7])
+    assert_codes_close(tp["self_ctx_q"], ctx, max_frac=1e-3, what="decoder self-attention context")
+    # out projection, residual + layer norm
+    eq(tp["self_out_q"], oracle.gemm_i8_i8(tp["self_ctx_q"], W("w_self_out"), c[1] * c[7] / (c[13] * Q)))
+    ln_q, res = oracle.residual_bias_ln_i8O(tp["self_out_q"], W("encdec_ln_scale"), W("encdec_ln_bias"),
+                                            W("b_encdec_out"), tp["res_in"], c[13] / Q, Q / c[8], post)
+    assert_codes_close(tp["encdec_ln_q"], ln_q, max_frac=1e-3, what="layer norm before cross attention")
+    np.testing.assert_allclose(tp["res_self"].astype(np.float32), res.astype(np.float32), atol=2e-2)
+
+    # cross attention: q product + head split, attention over the projected encoder output
+    codes = oracle.gemm_i8_i8(tp["encdec_ln_q"], W("w_encdec_q"), c[2] * c[8] / (c[14] * Q))
+    q = oracle.arrange_encdec_q_i8I(codes, W("b_encdec_q"), beam, h, c[14] / Q)
+    eq(tp["encdec_q"].view(np.uint16), q.view(np.uint16))
+    batch, seq = mask.shape
+    bh = batch * h
+    sc = oracle.attn_scores_rect(tp["encdec_q"].reshape(bh, beam, d), tp["encdec_k"].reshape(bh, seq, d),
+                                 float(np.sqrt(np.float32(1.0) / np.float32(d))))
+    pr = oracle.correlation_softmax_encdec(sc.reshape(batch, h * beam, seq), mask)
+    cx = oracle.attn_context_rect(pr.reshape(bh, beam, seq), tp["encdec_v"].reshape(bh, seq, d))
+    want = oracle.arrange_atten_output_i8O(cx.reshape(batch, h, beam, d), Q / c[9])
+    assert_codes_close(tp["encdec_ctx_q"], want.reshape(batch * beam, H), max_frac=5e-3,
+                       what="cross-attention context")
+    eq(tp["encdec_out_q"], oracle.gemm_i8_i8(tp["encdec_ctx_q"], W("w_encdec_out"), c[3] * c[9] / (c[15] * Q)))
+    ln_q, res = oracle.residual_bias_ln_i8O(tp["encdec_out_q"], W("ffn_ln_scale"), W("ffn_ln_bias"),
+                                            W("b_ffn2"), tp["res_self"], c[15] / Q, Q / c[10], post)
+    assert_codes_close(tp["ffn_ln_q"], ln_q, max_frac=1e-3, what="layer norm before the FFN")
+    np.testing.assert_allclose(tp["res_encdec"].astype(np.float32), res.astype(np.float32), atol=2e-2)
+
+    # FFN: first product + bias + activation + requantisation, second product, layer norm
+    codes = oracle.gemm_i8_i8(tp["ffn_ln_q"], W("w_ffn1"), c[4] * c[10] / (c[16] * Q))
+    if dec_w["use_gelu"]:
+        act = oracle.bias_gelu_i8I_i8O(codes, W("b_ffn1"), c[16] / Q, Q / c[11])
+    else:
+        act = oracle.bias_relu_i8I_i8O(codes, W("b_ffn1"), c[16] / Q, Q / c[11], c[11], True)
+    eq(tp["ffn1_act_q"], act)
+    eq(tp["ffn2_acc"], oracle.gemm_i8_i32(tp["ffn1_act_q"], W("w_ffn2")))
+    last = layer == dec_w["n_layer"] - 1
+    dq = c[5] * c[11] / (Q * Q) if dec_w["use_gelu"] else c[5] * c[11] / (2 * Q * Q)
+    if last:
+        sc_, bi_, rb_, clip = dec_w["out_ln_scale"], dec_w["out_ln_bias"], None, dec_w["output_ln_clip_max"]
+    else:
+        sc_, bi_, rb_ = (dec_w[n][layer + 1] for n in ("self_ln_scale", "self_ln_bias", "b_self_out"))
+        clip = dec_w["clip_max"][(layer + 1) * 19 + 6]
+    colsum = None if dec_w["ffn2_colsum"] is None else dec_w["ffn2_colsum"][layer]
+    ln_q, res = oracle.residual_bias_ln_i8O(tp["ffn2_acc"], sc_, bi_, rb_, tp["res_encdec"], dq, Q / clip,
+                                            post, colsum)
+    assert_codes_close(tp["next_ln_q"], ln_q, max_frac=1e-3, what="layer norm after the FFN")
+    np.testing.assert_allclose(tp["res_out"].astype(np.float32), res.astype(np.float32), atol=2e-2)
+
+
+@pytest.mark.parametrize("layer", [0, 1])
+def test_decoder_step_stage_by_stage_at_transformer_big_width(oracle, tmp_path, layer):
+    """One decoding step of a Transformer-big-shaped model (hidden 1024, 16 heads, inner 4096,
+    beam 4), stage by stage through the decoder's step taps, at the first step, a middle step
+    and the last step."""
+    from lightseq_amd import synthetic
+    cfg = synthetic.transformer_config("transformer_big")
+    cfg.update(n_enc_layer=2, n_dec_layer=2, max_step=32, extra_decode_length=12)
+    sigma = 0.02 * np.sqrt(cfg["hidden"])
+    path, msg = _make(tmp_path, cfg, 11, eos_bias=2.5 * sigma, w_std=0.05)
+    ids = _src_ids(cfg, 4, 16, 3)
+    _, dec_w = _oracle_weights(msg, cfg)
+    mask = (ids == cfg["padding_id"]).astype(np.int32)
+    last_step = None
+    for step in (0, 9, -1):
+        if step < 0:
+            step = last_step
+        tp, steps = _decoder_step_taps(path, cfg, ids, layer, step)
+        last_step = steps - 1
+        assert step < steps
+        assert np.abs(tp["self_ln_q"]).max() > 0 and np.abs(tp["ffn2_acc"]).max() > 0
+        _check_decoder_step_stages(oracle, dec_w, cfg, mask, tp, layer, step)
 
 
 def test_transformer_big_full_size_properties(oracle, tmp_path):
