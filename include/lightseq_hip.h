@@ -655,6 +655,15 @@ int lsh_ker_ppl_i8I(int batch_size, int batch_seq_len, int max_thread_per_block,
                     const int* real_seq_len, float* ppl, int vocab_size, float dequant_scale,
                     int in_col32);
 
+/* No counterpart in the reference: lsh_ker_ppl_i8I with a workspace of batch_size *
+ * batch_seq_len floats, so that every (sequence, position) pair gets its own workgroup and
+ * a second kernel adds a sequence's terms in ascending order; the same bits as
+ * lsh_ker_ppl_i8I, which walks a sequence's positions in one workgroup (what QuantGpt runs
+ * for files with sampling_method "ppl"). */
+int lsh_ker_ppl_i8I_workspace(int batch_size, int batch_seq_len, lsh_stream_t stream,
+                              const int8_t* logits, const int* input_ids, const int* real_seq_len,
+                              float* ppl, int vocab_size, float dequant_scale, float* workspace);
+
 /* Prompt pass of the model, no single counterpart in the reference:
  *  - lsh_gpt_arrange_qkv_prefill_f16 = ker_arrange_encself_qkv_i8I_i8O_launcher
  *    (model/quant_gpt_encoder.cc.cu:489-496) writing q / k as fp16 code values and v

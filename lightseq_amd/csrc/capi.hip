@@ -728,6 +728,13 @@ int lsh_ker_ppl_i8I(int batch_size, int batch_seq_len, int max_thread_per_block,
   return ppl_i8I(batch_size, batch_seq_len, HS(stream), logits, input_ids, real_seq_len, ppl,
                  vocab_size, dequant_scale);
 }
+int lsh_ker_ppl_i8I_workspace(int batch_size, int batch_seq_len, lsh_stream_t stream,
+                              const int8_t* logits, const int* input_ids, const int* real_seq_len,
+                              float* ppl, int vocab_size, float dequant_scale, float* workspace) {
+  if (!workspace) return lsh_fail(LSH_ERR_INVALID, "ker_ppl_i8I: null workspace");
+  return ppl_i8I(batch_size, batch_seq_len, HS(stream), logits, input_ids, real_seq_len, ppl,
+                 vocab_size, dequant_scale, workspace);
+}
 int lsh_gpt_arrange_qkv_prefill_f16(int batch_token_num, int hidden_size, lsh_stream_t stream,
                                     const int8_t* ori_qkv, const void* qkv_bias, void* q_codes,
                                     void* k_codes, void* v_deq, int8_t* k_cache, int8_t* v_cache,

@@ -390,42 +390,83 @@ int gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_siz
 }
 
 // ---------------------------------------------------------------------------------
-// perplexity (inference/kernels/gptKernels_int8.cc.cu:108-190).  One block per sequence
-// walks its positions in order, so the sum has a fixed order (the reference adds the
-// per-position terms with float atomics).
+// perplexity (inference/kernels/gptKernels_int8.cc.cu:108-190).  The per-position terms of a
+// sequence are added in ascending position order, so the sum has a fixed order (the reference
+// adds them with float atomics).  With a workspace of batch * seq_len floats every (sequence,
+// position) pair gets its own workgroup and a second kernel adds a sequence's terms in order;
+// without one a workgroup per sequence walks its positions.  Both give the same bits.
 // ---------------------------------------------------------------------------------
+// -log p(next token) / (len - 1) of position s of sequence b, the same in every thread
+__device__ __forceinline__ float ppl_term(const int8_t* __restrict__ logits,
+                                          const int* __restrict__ input_ids, int b, int s, int len,
+                                          int vocab, int seq_len, float dq, float* red) {
+#pragma clang fp contract(off)
+  const long tok = (long)b * seq_len + s;
+  const int8_t* lr = logits + tok * vocab;
+  float mx = kFloatInfNeg;
+  for (int v = threadIdx.x; v < vocab; v += blockDim.x) mx = fmaxf(mx, (float)lr[v] * dq);
+  mx = block_max(mx, red);
+  float se = 0.f;
+  for (int v = threadIdx.x; v < vocab; v += blockDim.x)
+    se += __expf(fmaxf((float)lr[v] * dq - mx, kLogitThreshMin));
+  se = block_sum(se, red);
+  int target = input_ids[tok + 1];
+  target = min(max(target, 0), vocab - 1);
+  const float log_prob = ((float)lr[target] * dq - mx - logf(se)) / (float)(len - 1);
+  return -log_prob;
+}
+
 __global__ void __launch_bounds__(1024)
 ppl_kernel(const int8_t* __restrict__ logits, const int* __restrict__ input_ids,
            const int* __restrict__ real_seq_len, float* ppl, int vocab, int seq_len, float dq) {
-#pragma clang fp contract(off)
   __shared__ float red[16];
   const int b = blockIdx.x;
   const int len = real_seq_len[b];
   float total = 0.f;
-  for (int s = 0; s < seq_len && s < len - 1; ++s) {
-    const long tok = (long)b * seq_len + s;
-    const int8_t* lr = logits + tok * vocab;
-    float mx = kFloatInfNeg;
-    for (int v = threadIdx.x; v < vocab; v += blockDim.x) mx = fmaxf(mx, (float)lr[v] * dq);
-    mx = block_max(mx, red);
-    float se = 0.f;
-    for (int v = threadIdx.x; v < vocab; v += blockDim.x)
-      se += __expf(fmaxf((float)lr[v] * dq - mx, kLogitThreshMin));
-    se = block_sum(se, red);
-    int target = input_ids[tok + 1];
-    target = min(max(target, 0), vocab - 1);
-    const float log_prob = ((float)lr[target] * dq - mx - logf(se)) / (float)(len - 1);
-    total += -log_prob;
-  }
+  for (int s = 0; s < seq_len && s < len - 1; ++s)
+    total += ppl_term(logits, input_ids, b, s, len, vocab, seq_len, dq, red);
   if (threadIdx.x == 0) ppl[b] += total;
+}
+
+// grid (seq_len, batch): terms[b * seq_len + s]
+__global__ void __launch_bounds__(1024)
+ppl_terms_kernel(const int8_t* __restrict__ logits, const int* __restrict__ input_ids,
+                 const int* __restrict__ real_seq_len, float* __restrict__ terms, int vocab,
+                 int seq_len, float dq) {
+  __shared__ float red[16];
+  const int b = blockIdx.y, s = blockIdx.x;
+  const int len = real_seq_len[b];
+  if (s >= len - 1) return;  // (uniform: no term, nothing read by the sum)
+  const float t = ppl_term(logits, input_ids, b, s, len, vocab, seq_len, dq, red);
+  if (threadIdx.x == 0) terms[(long)b * seq_len + s] = t;
+}
+
+__global__ void ppl_sum_kernel(const float* __restrict__ terms,
+                               const int* __restrict__ real_seq_len, float* ppl, int batch,
+                               int seq_len) {
+#pragma clang fp contract(off)
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= batch) return;
+  const int len = real_seq_len[b];
+  float total = 0.f;
+  for (int s = 0; s < seq_len && s < len - 1; ++s) total += terms[(long)b * seq_len + s];
+  ppl[b] += total;
 }
 
 int ppl_i8I(int batch_size, int batch_seq_len, hipStream_t s, const int8_t* logits,
             const int* input_ids, const int* real_seq_len, float* ppl, int vocab_size,
-            float dequant_scale) {
+            float dequant_scale, float* workspace) {
   if (!logits || !input_ids || !real_seq_len || !ppl || batch_size <= 0 || batch_seq_len <= 0 ||
       vocab_size <= 0)
     return lsh_fail(LSH_ERR_INVALID, "ker_ppl_i8I: bad arguments");
+  if (workspace != nullptr && batch_size <= 65535) {
+    ppl_terms_kernel<<<dim3(batch_seq_len, batch_size), 1024, 0, s>>>(
+        logits, input_ids, real_seq_len, workspace, vocab_size, batch_seq_len, dequant_scale);
+    if (int rc = lsh_check_launch("ppl_terms_kernel")) return rc;
+    ppl_sum_kernel<<<(batch_size + 63) / 64, 64, 0, s>>>(workspace, real_seq_len, ppl, batch_size,
+                                                         batch_seq_len);
+    return lsh_check_launch("ppl_sum_kernel");
+  }
   ppl_kernel<<<batch_size, 1024, 0, s>>>(logits, input_ids, real_seq_len, ppl, vocab_size,
                                          batch_seq_len, dequant_scale);
   return lsh_check_launch("ppl_kernel");

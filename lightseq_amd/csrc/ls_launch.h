@@ -325,7 +325,8 @@ int gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_siz
                     int cur_len, int batch_size, int* unfinished, int eos_id, hipStream_t s);
 int ppl_i8I(int batch_size, int batch_seq_len, hipStream_t s, const int8_t* logits,
             const int* input_ids, const int* real_seq_len, float* ppl, int vocab_size,
-            float dequant_scale);
+            float dequant_scale, float* workspace = nullptr);  // workspace: batch * seq_len floats
+                                                               // -> one workgroup per position
 
 // ---- operator kernels of the csrc layer path (layer_ops.hip); clip values are device
 // ---- scalars of type T, dropout ratios must be 0 -------------------------------------

@@ -69,6 +69,25 @@ class DeviceBuffer {
   size_t n_ = 0;
 };
 
+// A HIP stream of the default priority that is destroyed with its owner.
+class StreamOwner {
+ public:
+  StreamOwner() = default;
+  StreamOwner(const StreamOwner&) = delete;
+  StreamOwner& operator=(const StreamOwner&) = delete;
+  ~StreamOwner() {
+    if (s_) (void)hipStreamDestroy(s_);
+  }
+  void create() {
+    if (!s_) CHECK_GPU_ERROR(hipStreamCreate(&s_));
+  }
+  hipStream_t get() const { return s_; }
+  operator hipStream_t() const { return s_; }
+
+ private:
+  hipStream_t s_ = nullptr;
+};
+
 // Debug taps of a generation step (parity bisection): device-to-device copies of named
 // intermediates of decoder layer `layer` at step `step` into buffers the caller owns.  A name
 // registered with a null pointer is forgotten.  A layer < 0 at the copy site means "any".

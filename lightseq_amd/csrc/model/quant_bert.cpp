@@ -7,19 +7,19 @@ QuantBert::QuantBert(const std::string weight_path, const int max_batch_size)
     : LSModel({"token_ids"}, {"encoder_output"}), _max_batch_size(max_batch_size) {
   if (max_batch_size <= 0) throw std::runtime_error("max_batch_size must be positive");
   CHECK_GPU_ERROR(hipSetDevice(0));
-  CHECK_GPU_ERROR(hipStreamCreate(&stream_));
+  stream_.create();
 
   std::string res = tw_.initializing(weight_path);
   if (!res.empty()) throw std::runtime_error(res);
 
   const size_t tokens = (size_t)_max_batch_size * tw_._max_step;
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_input_), tokens * sizeof(int)));
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_padding_mask_), tokens * sizeof(int)));
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_encoder_output_),
-                            tokens * tw_._hidden_size * sizeof(__half)));
+  d_input_.alloc(tokens);
+  d_padding_mask_.alloc(tokens);
+  d_encoder_output_.alloc(tokens * tw_._hidden_size);
 
-  encoder_ = std::make_shared<QuantBertEncoder>(max_batch_size, d_input_, d_padding_mask_,
-                                                d_encoder_output_, tw_, stream_);
+  encoder_ = std::make_shared<QuantBertEncoder>(max_batch_size, d_input_.get(),
+                                                d_padding_mask_.get(), d_encoder_output_.get(),
+                                                tw_, stream_);
   res = encoder_->check();
   if (!res.empty()) throw std::runtime_error(res);
   encoder_->init_buffer();
@@ -27,11 +27,7 @@ QuantBert::QuantBert(const std::string weight_path, const int max_batch_size)
 }
 
 QuantBert::~QuantBert() {
-  encoder_.reset();
-  if (d_input_) (void)hipFree(d_input_);
-  if (d_padding_mask_) (void)hipFree(d_padding_mask_);
-  if (d_encoder_output_) (void)hipFree(d_encoder_output_);
-  if (stream_) (void)hipStreamDestroy(stream_);
+  encoder_.reset();  // before the buffers and the stream it uses (members, released after this)
 }
 
 void QuantBert::Infer() {

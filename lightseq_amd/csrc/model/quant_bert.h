@@ -25,18 +25,18 @@ class QuantBert : public LSModel {
   DataType get_input_dtype(int index) override;
   DataType get_output_dtype(int index) override;
   void benchmark_mode(bool) override {}
-  void* get_stream() override { return stream_; }
+  void* get_stream() override { return stream_.get(); }
 
   QuantBertEncoder* encoder() { return encoder_.get(); }
   const QuantBertWeight& weight() const { return tw_; }
 
  private:
+  // owners first: released after the encoder, also when the constructor throws half way
+  StreamOwner stream_;
+  DeviceBuffer<int> d_input_, d_padding_mask_;
+  DeviceBuffer<__half> d_encoder_output_;
   std::shared_ptr<QuantBertEncoder> encoder_;
-  int* d_input_ = nullptr;
-  int* d_padding_mask_ = nullptr;
-  __half* d_encoder_output_ = nullptr;
   int _max_batch_size;
-  hipStream_t stream_ = nullptr;
   QuantBertWeight tw_;
 };
 

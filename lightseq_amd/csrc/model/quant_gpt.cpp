@@ -7,18 +7,18 @@ QuantGpt::QuantGpt(const std::string weight_path, const int max_batch_size)
     : LSModel({"token_ids"}, {"result"}), _max_batch_size(max_batch_size) {
   if (max_batch_size <= 0) throw std::runtime_error("max_batch_size must be positive");
   CHECK_GPU_ERROR(hipSetDevice(0));
-  CHECK_GPU_ERROR(hipStreamCreate(&stream_));
+  stream_.create();
 
   std::string res = tw_.initializing(weight_path);
   if (!res.empty()) throw std::runtime_error(res);
 
   const size_t tokens = (size_t)_max_batch_size * tw_._max_step;
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_input_), tokens * sizeof(int)));
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_sample_id), tokens * sizeof(int)));
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_ppl), _max_batch_size * sizeof(float)));
+  d_input_.alloc(tokens);
+  d_sample_id.alloc(tokens);
+  d_ppl.alloc(_max_batch_size);
 
-  encoder_ = std::make_shared<QuantGptEncoder>(max_batch_size, d_input_, d_ppl, d_sample_id, tw_,
-                                               stream_);
+  encoder_ = std::make_shared<QuantGptEncoder>(max_batch_size, d_input_.get(), d_ppl.get(),
+                                               d_sample_id.get(), tw_, stream_);
   res = encoder_->check();
   if (!res.empty()) throw std::runtime_error(res);
   encoder_->init_buffer();
@@ -26,11 +26,7 @@ QuantGpt::QuantGpt(const std::string weight_path, const int max_batch_size)
 }
 
 QuantGpt::~QuantGpt() {
-  encoder_.reset();
-  if (d_input_) (void)hipFree(d_input_);
-  if (d_sample_id) (void)hipFree(d_sample_id);
-  if (d_ppl) (void)hipFree(d_ppl);
-  if (stream_) (void)hipStreamDestroy(stream_);
+  encoder_.reset();  // before the buffers and the stream it uses (members, released after this)
 }
 
 void QuantGpt::Infer() {

@@ -26,19 +26,19 @@ class QuantGpt : public LSModel {
   DataType get_input_dtype(int index) override;
   DataType get_output_dtype(int index) override;
   void benchmark_mode(bool is_benchmark) override { encoder_->benchmark_mode(is_benchmark); }
-  void* get_stream() override { return stream_; }
+  void* get_stream() override { return stream_.get(); }
 
   QuantGptEncoder* encoder() { return encoder_.get(); }
   const QuantGptWeight& weight() const { return tw_; }
 
  private:
   bool is_ppl() const { return tw_._sampling_method == "ppl"; }
+  // owners first: released after the encoder, also when the constructor throws half way
+  StreamOwner stream_;
+  DeviceBuffer<int> d_input_, d_sample_id;
+  DeviceBuffer<float> d_ppl;
   std::shared_ptr<QuantGptEncoder> encoder_;
-  int* d_input_ = nullptr;
-  int* d_sample_id = nullptr;
-  float* d_ppl = nullptr;
   int _max_batch_size;
-  hipStream_t stream_ = nullptr;
   QuantGptWeight tw_;
 };
 

@@ -349,8 +349,10 @@ void QuantGptEncoder::run_one_infer(int batch_size, int batch_seq_len) {
   LSH_CALL(gemm_i8_i8o(_buf_a.get(), _int8_emb.get(), _logits.get(), _batch_token_num, V, H,
                        _output_ln_clip_max * _src_emb_clip_max / (_logits_clip_max * _quant_range),
                        _stream));
+  // the FFN2 accumulator buffer (tokens * hidden int32, idle by now) holds the per-position terms
   LSH_CALL(ppl_i8I(batch_size, batch_seq_len, _stream, _logits.get(), _p_d_token_id,
-                   _real_seq_len.get(), _p_d_ppl, V, _logits_clip_max / _quant_range));
+                   _real_seq_len.get(), _p_d_ppl, V, _logits_clip_max / _quant_range,
+                   reinterpret_cast<float*>(_int32_ffn_out_buf.get())));
 }
 
 }  // namespace hip

@@ -7,26 +7,26 @@ QuantTransformer::QuantTransformer(const std::string weight_path, const int max_
     : LSModel({"source_ids"}, {"target_ids", "target_scores"}), _max_batch_size(max_batch_size) {
   if (max_batch_size <= 0) throw std::runtime_error("max_batch_size must be positive");
   CHECK_GPU_ERROR(hipSetDevice(0));
-  CHECK_GPU_ERROR(hipStreamCreate(&stream_));
+  stream_.create();
 
   std::string res = tw_.initializing(weight_path);
   if (!res.empty()) throw std::runtime_error(res);
   if (tw_._sampling_method == "topk" || tw_._sampling_method == "topp") tw_._beam_size = 1;
 
   const size_t tokens = (size_t)_max_batch_size * tw_._max_step;
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_input_), tokens * sizeof(int)));
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_padding_mask_), tokens * sizeof(int)));
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_encoder_output_),
-                            tokens * tw_._hidden_size * sizeof(__half)));
-  CHECK_GPU_ERROR(hipMalloc(reinterpret_cast<void**>(&d_output_),
-                            tokens * std::max(tw_._beam_size, 1) * sizeof(int)));
+  d_input_.alloc(tokens);
+  d_padding_mask_.alloc(tokens);
+  d_encoder_output_.alloc(tokens * tw_._hidden_size);
+  d_output_.alloc(tokens * std::max(tw_._beam_size, 1));
 
-  encoder_ = std::make_shared<QuantBertEncoder>(max_batch_size, d_input_, d_padding_mask_,
-                                                d_encoder_output_, tw_.enc, stream_);
+  encoder_ = std::make_shared<QuantBertEncoder>(max_batch_size, d_input_.get(),
+                                                d_padding_mask_.get(), d_encoder_output_.get(),
+                                                tw_.enc, stream_);
   res = encoder_->check();
   if (!res.empty()) throw std::runtime_error(res);
-  decoder_ = std::make_shared<QuantDecoder>(max_batch_size, d_padding_mask_, d_encoder_output_,
-                                            d_output_, tw_, stream_, true);
+  decoder_ = std::make_shared<QuantDecoder>(max_batch_size, d_padding_mask_.get(),
+                                            d_encoder_output_.get(), d_output_.get(), tw_,
+                                            stream_, true);
   res = decoder_->check();
   if (!res.empty()) throw std::runtime_error(res);
   encoder_->init_buffer();
@@ -36,12 +36,7 @@ QuantTransformer::QuantTransformer(const std::string weight_path, const int max_
 
 QuantTransformer::~QuantTransformer() {
   decoder_.reset();
-  encoder_.reset();
-  if (d_input_) (void)hipFree(d_input_);
-  if (d_padding_mask_) (void)hipFree(d_padding_mask_);
-  if (d_encoder_output_) (void)hipFree(d_encoder_output_);
-  if (d_output_) (void)hipFree(d_output_);
-  if (stream_) (void)hipStreamDestroy(stream_);
+  encoder_.reset();  // before the buffers and the stream they use (members, released after this)
 }
 
 void QuantTransformer::Infer() {
@@ -50,7 +45,7 @@ void QuantTransformer::Infer() {
   if (tw_._multilg_type != 0) throw std::runtime_error("multilingle not supported");
   encoder_->run_one_infer(batch_size, seq_len);
   if (enc_out_tap_)
-    CHECK_GPU_ERROR(hipMemcpyAsync(enc_out_tap_, d_encoder_output_,
+    CHECK_GPU_ERROR(hipMemcpyAsync(enc_out_tap_, d_encoder_output_.get(),
                                    (size_t)batch_size * seq_len * tw_._hidden_size * sizeof(__half),
                                    hipMemcpyDeviceToDevice, stream_));
   decoder_->run_one_infer(batch_size, seq_len);

@@ -28,7 +28,7 @@ class QuantTransformer : public LSModel {
   DataType get_input_dtype(int index) override;
   DataType get_output_dtype(int index) override;
   void benchmark_mode(bool is_benchmark) override;
-  void* get_stream() override { return stream_; }
+  void* get_stream() override { return stream_.get(); }
 
   QuantBertEncoder* encoder() { return encoder_.get(); }
   QuantDecoder* decoder() { return decoder_.get(); }
@@ -38,15 +38,15 @@ class QuantTransformer : public LSModel {
   void set_encoder_output_tap(__half* dst) { enc_out_tap_ = dst; }
 
  private:
+  // owners first: the stream and the buffers outlive the encoder and decoder that use them,
+  // and are released when the constructor throws half way (unsupported files are common)
+  StreamOwner stream_;
+  DeviceBuffer<int> d_input_, d_padding_mask_, d_output_;
+  DeviceBuffer<__half> d_encoder_output_;
   std::shared_ptr<QuantBertEncoder> encoder_;
   std::shared_ptr<QuantDecoder> decoder_;
-  int* d_input_ = nullptr;
-  int* d_padding_mask_ = nullptr;
-  __half* d_encoder_output_ = nullptr;
-  int* d_output_ = nullptr;
   __half* enc_out_tap_ = nullptr;
   int _max_batch_size;
-  hipStream_t stream_ = nullptr;
   QuantTransformerWeight tw_;
 };
 

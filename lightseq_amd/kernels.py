@@ -502,6 +502,16 @@ def ker_ppl_i8I_launcher(batch_size, batch_seq_len, max_thread_per_block, logits
          int(in_col32))
 
 
+def ker_ppl_i8I_workspace(batch_size, batch_seq_len, logits, input_ids, real_seq_len, ppl,
+                          vocab_size, dequant_scale, workspace):
+    """ker_ppl_i8I with one workgroup per position; workspace: batch * seq_len float32."""
+    _dev(logits, input_ids, real_seq_len, ppl, workspace)
+    if workspace.dtype != torch.float32 or workspace.numel() < batch_size * batch_seq_len:
+        raise ValueError("workspace must hold batch_size * batch_seq_len float32")
+    call("lsh_ker_ppl_i8I_workspace", batch_size, batch_seq_len, current_stream(), ptr(logits),
+         ptr(input_ids), ptr(real_seq_len), ptr(ppl), vocab_size, dequant_scale, ptr(workspace))
+
+
 def gpt_arrange_qkv_prefill(batch_token_num, hidden_size, ori_qkv, qkv_bias, q_codes, k_codes,
                             v_deq, k_cache, v_cache, batch_seq_len, dim_per_head, head_num,
                             max_step, dequant_scale, quant_scale):

@@ -96,6 +96,7 @@ _SIGNATURES = {
     "lsh_ker_arrange_qkv_with_cache_i8I_i8O": (True, "iis" + "ppppppp" + "iii" + "ffi"),
     "lsh_ker_topk_sample_i8I": (False, "iiiis" + "pppp" + "ii" + "pp" + "ifi"),
     "lsh_ker_ppl_i8I": (False, "iiis" + "pppp" + "ifi"),
+    "lsh_ker_ppl_i8I_workspace": (False, "iis" + "pppp" + "if" + "p"),
     "lsh_gpt_arrange_qkv_prefill_f16": (False, "iis" + "ppppppp" + "iiii" + "ff"),
     "lsh_gpt_prefill_attention_f16": (False, "pppppp" + "ff" + "iiii" + "s"),
     "lsh_gpt_greedy_step": (False, "ppp" + "iiii" + "p" + "i" + "s"),

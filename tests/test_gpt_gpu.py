@@ -144,7 +144,7 @@ def test_topk_sample_errors():
         _k().ker_topk_sample_i8I_launcher(1, 4, 1, 1024, z8, zi, zi, None, 16, 3, zi, None, 1, 0.1)
 
 
-@pytest.mark.parametrize("batch,seq,vocab", [(3, 8, 300), (2, 5, 5000)])
+@pytest.mark.parametrize("batch,seq,vocab", [(3, 8, 300), (2, 5, 5000), (3, 40, 50257)])
 def test_ppl(rng, batch, seq, vocab):
     logits = np.clip(rng.standard_normal((batch * seq, vocab)) * 30, -127, 127).astype(np.int8)
     ids = rng.integers(0, vocab, size=(batch, seq), dtype=np.int32)
@@ -154,6 +154,11 @@ def test_ppl(rng, batch, seq, vocab):
     _k().ker_ppl_i8I_launcher(batch, seq, 1024, to_dev(logits), to_dev(ids), to_dev(rsl), ppl,
                               vocab, 0.02)
     np.testing.assert_allclose(to_np(ppl), want, rtol=2e-5, atol=1e-5)
+    # one workgroup per position + an ordered sum: the same bits (what the model runs)
+    ppl2 = torch.zeros(batch, dtype=torch.float32, device=DEV)
+    ws = torch.full((batch * seq,), 7.0, dtype=torch.float32, device=DEV)
+    _k().ker_ppl_i8I_workspace(batch, seq, to_dev(logits), to_dev(ids), to_dev(rsl), ppl2, vocab, 0.02, ws)
+    np.testing.assert_array_equal(to_np(ppl2).view(np.uint32), to_np(ppl).view(np.uint32))
 
 
 @pytest.mark.parametrize("batch,heads,seq,d,max_step", [(2, 2, 9, 32, 16), (2, 16, 130, 64, 160),

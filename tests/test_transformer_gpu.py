@@ -133,7 +133,7 @@ def test_tiny_transformer(oracle, tmp_path, seed, eos, batch, seq):
     gpu = _run_gpu(path, cfg, ids, max_batch=4)
     assert gpu["tokens"].shape[:2] == (batch, cfg["beam_size"])
     assert gpu["scores"].shape == (batch, cfg["beam_size"])
-    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.02)
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.05)
 
     # free-running oracle (its own encoder output and logits): identical ids
     enc_w, dec_w = _oracle_weights(msg, cfg)
@@ -156,7 +156,7 @@ def test_early_stop_and_benchmark_mode(oracle, tmp_path):
     limit = min(cfg["max_step"], ids.shape[1] + cfg["extra_decode_length"]) - 1
     assert gpu["steps"] < limit - 1, "expected an early stop"
     assert gpu["tokens"].shape[2] == gpu["steps"]
-    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.02)
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.05)
 
     bench = _run_gpu(path, cfg, ids, max_batch=3, benchmark=True)
     assert bench["steps"] == limit - 1
@@ -178,7 +178,7 @@ def test_gelu_post_ln_variant(oracle, tmp_path):
     path, msg = _make(tmp_path, cfg, 5, eos_bias=2.0 * sigma, w_std=0.2)
     ids = _src_ids(cfg, 2, 9, 5)
     gpu = _run_gpu(path, cfg, ids, max_batch=2)
-    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.02)
+    _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch=0.05)
 
 
 def test_repeated_infer_is_deterministic(tmp_path):
