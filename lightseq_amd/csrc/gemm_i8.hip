@@ -40,6 +40,7 @@
 
 #include <hip/hip_ext.h>
 
+#include <cstdlib>
 #include <mutex>
 #include <string>
 #include <type_traits>
@@ -1346,8 +1347,9 @@ std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
   if (M <= 64 && K % kBK == 0) return std::string("gemm_i8_skinny_kernel<") + epilogue + ">";
   if (!stream_ok(M, N, K)) return std::string("gemm_i8_generic_kernel<") + epilogue + ">";
   const std::string e = epilogue ? epilogue : "";
-  if (g_tile_kernel_enabled && N % 16 == 0 && choose_tile(M, N, K).shape != kTileNone)
+  if (g_tile_kernel_enabled && N % 16 == 0 && choose_tile(M, N, K).shape != kTileNone) {
     return "gemm_i8_tile_kernel<" + e + ">";
+  }
   if (e == "EpiLutI8" && K / kBK >= 2) return "gemm_i8_stream_kernel<EpiLutI8>";
   const bool wide = (e != "EpiI32" && e != "EpiI8") || !narrow_pays(M, N, K, 1);
   return std::string(wide ? "gemm_i8_stream128_kernel<" : "gemm_i8_stream_kernel<") + e + ">";
