@@ -144,18 +144,95 @@ TAP_SPECS = [("ln1_q", "H", "i8"), ("qkv_q", "3H", "i8"), ("ctx_q", "H", "i8"), 
              ("res_attn", "H", "f16"), ("res_ffn", "H", "f16")]
 
 
-def _run_with_taps(model, ids, layer, M, H, I):
+# taps that leave the layer on its fused kernels (the others make it take the unfused route)
+PASSIVE_TAPS = ("ln1_q", "ctx_q", "ln2_q", "act_q")
+
+
+def _run_with_taps(model, ids, layer, M, H, I, only=None):
     width = {"H": H, "3H": 3 * H, "I": I}
     dts = {"i8": torch.int8, "i32": torch.int32, "f16": torch.float16}
     bufs = {}
     for name, wd, dt in TAP_SPECS:
+        if only is not None and name not in only:
+            continue
         bufs[name] = torch.zeros((M, width[wd]), dtype=dts[dt], device=DEV)
         model.set_tap(layer, name, bufs[name])
     out = model.infer_fp16(ids)
     taps = {k: v.cpu().numpy() for k, v in bufs.items()}
-    for name, _, _ in TAP_SPECS:
+    for name in bufs:
         model.set_tap(layer, name, None)
     return out, taps
+
+
+def _check_encoder_layer_stages(oracle, w, cfg, t, layer, B, S, mask, valid):
+    """Every stage of encoder layer `layer` against the oracle's kernel for that stage, each fed
+    the GPU's own stage input (the taps `t`): GEMM codes and the FFN2 accumulator bit for bit,
+    attention / layer-norm / activation codes to the +-1 code / 0.1 % bar.  Returns the oracle's
+    int8 input of the next layer (or None for the last layer)."""
+    H, I, h = cfg["hidden"], cfg["inner"], cfg["head_num"]
+    Q = np.float32(127)
+    c = w["clip_max"][layer * 11:(layer + 1) * 11]
+    np.testing.assert_array_equal(
+        t["qkv_q"], oracle.gemm_i8_i8(t["ln1_q"], w["w_qkv"][layer], c[0] * c[4] / (c[8] * Q)))
+    np.testing.assert_array_equal(
+        t["out_q"], oracle.gemm_i8_i8(t["ctx_q"], w["w_out"][layer], c[1] * c[5] / (c[9] * Q)))
+    np.testing.assert_array_equal(
+        t["ffn1_q"], oracle.gemm_i8_i8(t["ln2_q"], w["w_ffn1"][layer], c[2] * c[6] / (c[10] * Q)))
+    np.testing.assert_array_equal(t["ffn2_acc"], oracle.gemm_i8_i32(t["act_q"], w["w_ffn2"][layer]))
+    qkv = oracle.arrange_encself_qkv_i8I(t["qkv_q"], w["b_qkv"][layer], B, S, h, c[8] / Q)
+    probs = oracle.correlation_softmax_encself(
+        oracle.attn_scores(qkv[0], qkv[1], np.sqrt(1.0 / (H // h))), mask)
+    ctx_q = oracle.arrange_atten_output_i8O(oracle.attn_context(probs, qkv[2]), Q / c[5])
+    assert_codes_close(t["ctx_q"][valid], ctx_q[valid], what="ctx_q layer %d" % layer)
+    ln2_q, _ = oracle.residual_bias_ln_i8O(t["out_q"], w["ln2_scale"][layer], w["ln2_bias"][layer],
+                                           w["b_ffn2"][layer], t["res_attn"], c[9] / Q, Q / c[6],
+                                           cfg["is_post_ln"])
+    assert_codes_close(t["ln2_q"], ln2_q, what="ln2_q layer %d" % layer)
+    if cfg["use_gelu"]:
+        act_q = oracle.bias_gelu_i8I_i8O(t["ffn1_q"], w["b_ffn1"][layer], c[10] / Q, Q / c[7])
+    else:
+        act_q = oracle.bias_relu_i8I_i8O(t["ffn1_q"], w["b_ffn1"][layer], c[10] / Q, Q / c[7], c[7], True)
+    assert_codes_close(t["act_q"], act_q, what="act_q layer %d" % layer)
+    if layer == w["n_layer"] - 1:
+        return None
+    cn = w["clip_max"][(layer + 1) * 11:(layer + 2) * 11]
+    dq = c[3] * c[7] / (Q * Q)
+    ln1_next, _ = oracle.residual_bias_ln_i8O(t["ffn2_acc"], w["ln1_scale"][layer + 1],
+                                              w["ln1_bias"][layer + 1], w["b_out"][layer + 1],
+                                              t["res_ffn"], dq, Q / cn[4], cfg["is_post_ln"])
+    return ln1_next
+
+
+def test_bert_base_every_layer_stage_by_stage(tmp_path, oracle):
+    """The benchmark stack itself (12 layers, hidden 768, 12 heads, FFN 3072 GELU, batch 32 x
+    seq 128, ragged lengths): every stage of every layer against the oracle's kernel for it,
+    fed the GPU's own stage input; and the fused kernels a layer normally runs (QKV + attention,
+    out-projection + layer norm, FFN1 + table) leave the same bytes in place as the unfused
+    kernels that the taps switch the layer to."""
+    from lightseq_amd import inference, synthetic
+    cfg, msg, path = _build(tmp_path, "bert_base", 4, vocab=2000, max_step=128)
+    B, S, H, I = 32, 128, cfg["hidden"], cfg["inner"]
+    M = B * S
+    ids, lens = synthetic.make_token_ids(cfg, B, S, seed=4, min_len=32)
+    w = oracle_weights_from_message(msg, cfg)
+    assert w["n_layer"] == 12
+    mask = (ids == cfg["padding_id"]).astype(np.int32)
+    valid = _valid(ids, cfg).reshape(-1)
+    model = inference.QuantBert(path, B)
+    ln1_next = None
+    for layer in range(12):
+        _, t = _run_with_taps(model, ids, layer, M, H, I)
+        if ln1_next is not None:
+            assert_codes_close(t["ln1_q"], ln1_next, what="ln1_q layer %d" % layer)
+        ln1_next = _check_encoder_layer_stages(oracle, w, cfg, t, layer, B, S, mask, valid)
+        # the same layer on its fused kernels
+        _, f = _run_with_taps(model, ids, layer, M, H, I, only=PASSIVE_TAPS)
+        for name in PASSIVE_TAPS:
+            if name == "ctx_q":   # padded queries: zeros on both routes, but compare what matters
+                np.testing.assert_array_equal(f[name][valid], t[name][valid])
+            else:
+                np.testing.assert_array_equal(f[name], t[name])
+    model.close()
 
 
 def test_bert_base_two_layers_full_width(tmp_path, oracle):
