@@ -18,32 +18,50 @@ enum DataType {
   kByte = 7, kUInt8 = 8, kUInt16 = 9, kUInt32 = 10, kUInt64 = 11, kFloat64 = 12
 };
 
+// One input or output of a model: what the accessor functions of LSModel answer from.  `slot`
+// is where the model keeps the device pointer of this tensor (inside its encoder / decoder).
+struct IoSlot {
+  DataType dtype = kNotSupported;
+  std::vector<int> max_shape;
+  void** slot = nullptr;
+};
+
 class LSModel {
  public:
   LSModel(std::vector<std::string> input_names, std::vector<std::string> output_names)
       : kInputNames(std::move(input_names)), kOutputNames(std::move(output_names)) {
     input_shapes_.resize(kInputNames.size());
     output_shapes_.resize(kOutputNames.size());
+    inputs_.resize(kInputNames.size());
+    outputs_.resize(kOutputNames.size());
   }
   virtual ~LSModel() {}
   virtual void Infer() = 0;
 
-  virtual void set_input_ptr(int index, void* input_ptr) = 0;
+  // The accessors below are answered from the descriptor table that the model's constructor
+  // fills (describe_input / describe_output); a model overrides none of them.
+  virtual void set_input_ptr(int index, void* input_ptr) { *slot_of(inputs_, index, "input").slot = input_ptr; }
   void set_input_shape(int index, std::vector<int> shape) {
     input_shapes_.at(index) = std::move(shape);
   }
-  virtual std::vector<int> get_input_max_shape(int index) = 0;
+  virtual std::vector<int> get_input_max_shape(int index) {
+    return slot_of(inputs_, index, "input").max_shape;
+  }
   std::string get_input_name(int index) { return kInputNames.at(index); }
   int get_input_size() { return (int)kInputNames.size(); }
-  virtual DataType get_input_dtype(int index) = 0;
+  virtual DataType get_input_dtype(int index) { return slot_of(inputs_, index, "input").dtype; }
 
-  virtual void set_output_ptr(int index, void* output_ptr) = 0;
-  virtual const void* get_output_ptr(int index) = 0;
+  virtual void set_output_ptr(int index, void* output_ptr) {
+    *slot_of(outputs_, index, "output").slot = output_ptr;
+  }
+  virtual const void* get_output_ptr(int index) { return *slot_of(outputs_, index, "output").slot; }
   std::string get_output_name(int index) { return kOutputNames.at(index); }
   int get_output_size() { return (int)kOutputNames.size(); }
   std::vector<int> get_output_shape(int index) { return output_shapes_.at(index); }
-  virtual std::vector<int> get_output_max_shape(int index) = 0;
-  virtual DataType get_output_dtype(int index) = 0;
+  virtual std::vector<int> get_output_max_shape(int index) {
+    return slot_of(outputs_, index, "output").max_shape;
+  }
+  virtual DataType get_output_dtype(int index) { return slot_of(outputs_, index, "output").dtype; }
 
   virtual void benchmark_mode(bool is_benchmark) = 0;
 
@@ -54,10 +72,26 @@ class LSModel {
   void set_output_shape(int index, std::vector<int> shape) {
     output_shapes_.at(index) = std::move(shape);
   }
+  template <typename T>
+  void describe_input(int index, DataType dtype, std::vector<int> max_shape, T** slot) {
+    inputs_.at(index) = IoSlot{dtype, std::move(max_shape), (void**)slot};
+  }
+  template <typename T>
+  void describe_output(int index, DataType dtype, std::vector<int> max_shape, T** slot) {
+    outputs_.at(index) = IoSlot{dtype, std::move(max_shape), (void**)slot};
+  }
   const std::vector<std::string> kInputNames;
   const std::vector<std::string> kOutputNames;
   std::vector<std::vector<int>> input_shapes_;
   std::vector<std::vector<int>> output_shapes_;
+
+ private:
+  static IoSlot& slot_of(std::vector<IoSlot>& table, int index, const char* what) {
+    if (index < 0 || index >= (int)table.size() || table[index].slot == nullptr)
+      throw std::runtime_error(std::string("invalid ") + what + " index");
+    return table[index];
+  }
+  std::vector<IoSlot> inputs_, outputs_;
 };
 
 typedef LSModel* (*LSModelConstructor)(const std::string, const int);

@@ -24,6 +24,9 @@ QuantBert::QuantBert(const std::string weight_path, const int max_batch_size)
   if (!res.empty()) throw std::runtime_error(res);
   encoder_->init_buffer();
   CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+  describe_input(0, kInt32, {_max_batch_size, tw_._max_step}, &encoder_->_p_d_token_id);
+  describe_output(0, kFloat16, {_max_batch_size, tw_._max_step, tw_._hidden_size},
+                  &encoder_->_p_d_output);
 }
 
 QuantBert::~QuantBert() {
@@ -37,41 +40,6 @@ void QuantBert::Infer() {
   CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
   encoder_->collect_profile();
   set_output_shape(0, {batch_size, seq_len, tw_._hidden_size});
-}
-
-void QuantBert::set_input_ptr(int index, void* input_ptr) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  encoder_->_p_d_token_id = static_cast<int*>(input_ptr);
-}
-
-void QuantBert::set_output_ptr(int index, void* output_ptr) {
-  if (index != 0) throw std::runtime_error("invalid output index");
-  encoder_->_p_d_output = static_cast<__half*>(output_ptr);
-}
-
-const void* QuantBert::get_output_ptr(int index) {
-  if (index != 0) throw std::runtime_error("invalid output index");
-  return static_cast<void*>(encoder_->_p_d_output);
-}
-
-std::vector<int> QuantBert::get_input_max_shape(int index) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  return {_max_batch_size, tw_._max_step};
-}
-
-std::vector<int> QuantBert::get_output_max_shape(int index) {
-  if (index != 0) throw std::runtime_error("invalid output index");
-  return {_max_batch_size, tw_._max_step, tw_._hidden_size};
-}
-
-DataType QuantBert::get_input_dtype(int index) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  return DataType::kInt32;
-}
-
-DataType QuantBert::get_output_dtype(int index) {
-  if (index != 0) throw std::runtime_error("invalid output index");
-  return DataType::kFloat16;
 }
 
 LSMODEL_REGISTER(QuantBert)

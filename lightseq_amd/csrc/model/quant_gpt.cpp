@@ -23,6 +23,10 @@ QuantGpt::QuantGpt(const std::string weight_path, const int max_batch_size)
   if (!res.empty()) throw std::runtime_error(res);
   encoder_->init_buffer();
   CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+  describe_input(0, kInt32, {_max_batch_size, tw_._max_step}, &encoder_->_p_d_token_id);
+  // a file configured for perplexity returns one float per sequence, otherwise the sampled ids
+  if (is_ppl()) describe_output(0, kFloat32, {_max_batch_size}, &encoder_->_p_d_ppl);
+  else describe_output(0, kInt32, {_max_batch_size, tw_._max_step}, &encoder_->_p_d_sample_id);
 }
 
 QuantGpt::~QuantGpt() {
@@ -43,46 +47,6 @@ void QuantGpt::Infer() {
   } else {
     throw std::runtime_error("Unsupported sampling_method");
   }
-}
-
-void QuantGpt::set_input_ptr(int index, void* input_ptr) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  encoder_->_p_d_token_id = static_cast<int*>(input_ptr);
-}
-
-void QuantGpt::set_output_ptr(int index, void* output_ptr) {
-  if (index != 0) throw std::runtime_error("invalid output index");
-  if (is_ppl())
-    encoder_->_p_d_ppl = static_cast<float*>(output_ptr);
-  else
-    encoder_->_p_d_sample_id = static_cast<int*>(output_ptr);
-}
-
-const void* QuantGpt::get_output_ptr(int index) {
-  if (index != 0) throw std::runtime_error("invalid output index");
-  if (is_ppl()) return static_cast<void*>(encoder_->_p_d_ppl);
-  return static_cast<void*>(encoder_->_p_d_sample_id);
-}
-
-std::vector<int> QuantGpt::get_input_max_shape(int index) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  return {_max_batch_size, tw_._max_step};
-}
-
-std::vector<int> QuantGpt::get_output_max_shape(int index) {
-  if (index != 0) throw std::runtime_error("invalid output index");
-  if (is_ppl()) return {_max_batch_size};
-  return {_max_batch_size, tw_._max_step};
-}
-
-DataType QuantGpt::get_input_dtype(int index) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  return DataType::kInt32;
-}
-
-DataType QuantGpt::get_output_dtype(int index) {
-  if (index != 0) throw std::runtime_error("invalid output index");
-  return is_ppl() ? DataType::kFloat32 : DataType::kInt32;
 }
 
 LSMODEL_REGISTER(QuantGpt)

@@ -32,6 +32,11 @@ QuantTransformer::QuantTransformer(const std::string weight_path, const int max_
   encoder_->init_buffer();
   decoder_->init_buffer();
   CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+  describe_input(0, kInt32, {_max_batch_size, tw_._max_step}, &encoder_->_p_d_token_id);
+  describe_output(0, kInt32, {_max_batch_size, tw_._beam_size, tw_._max_step},
+                  &decoder_->_p_d_result);
+  describe_output(1, kFloat32, {_max_batch_size, tw_._beam_size},
+                  &decoder_->_p_d_alive_seq_score);
 }
 
 QuantTransformer::~QuantTransformer() {
@@ -55,53 +60,6 @@ void QuantTransformer::Infer() {
   int output_k = decoder_->_output_topk ? tw_._beam_size : 1;
   set_output_shape(0, {batch_size, output_k, output_seq_len});
   set_output_shape(1, {batch_size, output_k});
-}
-
-void QuantTransformer::set_input_ptr(int index, void* input_ptr) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  encoder_->_p_d_token_id = static_cast<int*>(input_ptr);
-}
-
-void QuantTransformer::set_output_ptr(int index, void* output_ptr) {
-  switch (index) {
-    case 0: decoder_->_p_d_result = static_cast<int*>(output_ptr); break;
-    case 1: decoder_->_p_d_alive_seq_score = static_cast<float*>(output_ptr); break;
-    default: throw std::runtime_error("invalid input index");
-  }
-}
-
-const void* QuantTransformer::get_output_ptr(int index) {
-  switch (index) {
-    case 0: return static_cast<void*>(decoder_->_p_d_result);
-    case 1: return static_cast<void*>(decoder_->_p_d_alive_seq_score);
-    default: throw std::runtime_error("invalid output index");
-  }
-}
-
-std::vector<int> QuantTransformer::get_input_max_shape(int index) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  return {_max_batch_size, tw_._max_step};
-}
-
-std::vector<int> QuantTransformer::get_output_max_shape(int index) {
-  switch (index) {
-    case 0: return {_max_batch_size, tw_._beam_size, tw_._max_step};
-    case 1: return {_max_batch_size, tw_._beam_size};
-    default: throw std::runtime_error("invalid output index");
-  }
-}
-
-DataType QuantTransformer::get_input_dtype(int index) {
-  if (index != 0) throw std::runtime_error("invalid input index");
-  return DataType::kInt32;
-}
-
-DataType QuantTransformer::get_output_dtype(int index) {
-  switch (index) {
-    case 0: return DataType::kInt32;
-    case 1: return DataType::kFloat32;
-    default: throw std::runtime_error("invalid output index");
-  }
 }
 
 void QuantTransformer::benchmark_mode(bool is_benchmark) {

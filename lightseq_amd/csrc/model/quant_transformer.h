@@ -20,13 +20,6 @@ class QuantTransformer : public LSModel {
   ~QuantTransformer();
 
   void Infer() override;
-  void set_input_ptr(int index, void* input_ptr) override;
-  void set_output_ptr(int index, void* output_ptr) override;
-  const void* get_output_ptr(int index) override;
-  std::vector<int> get_input_max_shape(int index) override;
-  std::vector<int> get_output_max_shape(int index) override;
-  DataType get_input_dtype(int index) override;
-  DataType get_output_dtype(int index) override;
   void benchmark_mode(bool is_benchmark) override;
   void* get_stream() override { return stream_.get(); }
 
