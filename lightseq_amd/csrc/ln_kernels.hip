@@ -184,7 +184,9 @@ __device__ __forceinline__ void
 ln_rows8_row(int row, bool live, int sub, const AccT* __restrict__ gemm_out, T* residual, T* out_t,
              int8_t* __restrict__ out_q, const T* __restrict__ scale, const T* __restrict__ bias,
              const T* __restrict__ residual_bias, const T* __restrict__ colsum, int hidden,
-             float dequant_scale, float quant_scale, int is_post_ln, int nparts, long part_stride) {
+             float dequant_scale, float quant_scale, int is_post_ln, int nparts, long part_stride,
+             const half8_t* pre_res = nullptr) {
+  // pre_res (fp16 only): the lane's ITER residual chunks, already loaded by the caller
   const long base = (long)(live ? row : 0) * hidden;
 
   float x[ITER][8];
@@ -211,7 +213,12 @@ ln_rows8_row(int row, bool live, int sub, const AccT* __restrict__ gemm_out, T* 
     const int e = (it * LPR + sub) * 8;
     if (e < hidden && live) {
       float r[8];
-      ld8(residual, base + e, r);
+      if (sizeof(T) == 2 && pre_res != nullptr) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) r[k] = __half2float(pre_res[it].v[k]);
+      } else {
+        ld8(residual, base + e, r);
+      }
       if (MODE == kLnFirst) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) x[it][k] = TT<T>::safe(r[k]);
@@ -376,6 +383,22 @@ gemm_ln_rows16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   ln_v4i acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = (ln_v4i)0;
+  // the residual rows the layer norm will add are requested now, so that they have arrived
+  // when the product is done (same lane layout as the row routine below)
+  constexpr int RPW = kWave / LPR, PASSES = 16 / (8 * RPW);
+  half8_t pre[PASSES][ITER];
+  if constexpr (sizeof(T) == 2) {
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      const int row = min(r0 + (pass * 8 + wave) * RPW + lane / LPR, tokens - 1);
+#pragma unroll
+      for (int it = 0; it < ITER; ++it) {
+        const int e = min((it * LPR + lane % LPR) * 8, N - 8);
+        pre[pass][it] = *reinterpret_cast<const half8_t*>(
+            reinterpret_cast<const __half*>(residual) + (long)row * N + e);
+      }
+    }
+  }
   load_slice(0);
   if (KS > 1) load_slice(1);
   // the scheduling barriers keep the loads of slice i + 2 ahead of the MFMAs of slice i:
@@ -401,13 +424,13 @@ gemm_ln_rows16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   __syncthreads();
   // the stand-alone kernel's row routine with the lane layout it uses for this hidden size
   // (LPR lanes per row), fed from the staged codes
-  constexpr int RPW = kWave / LPR;
 #pragma unroll
-  for (int pass = 0; pass < 16 / (8 * RPW); ++pass) {
+  for (int pass = 0; pass < PASSES; ++pass) {
     const int row = r0 + (pass * 8 + wave) * RPW + lane / LPR;
     ln_rows8_row<T, int8_t, kLnResQuant, LPR, ITER>(
         row, row < tokens, lane % LPR, codes - (long)r0 * N, residual, nullptr, out_q, scale, bias,
-        residual_bias, nullptr, N, dequant_scale, quant_scale, is_post_ln, 1, 0);
+        residual_bias, nullptr, N, dequant_scale, quant_scale, is_post_ln, 1, 0,
+        sizeof(T) == 2 ? pre[pass] : nullptr);
   }
 }
 
