@@ -34,6 +34,10 @@ def _valid(ids, cfg):
     ("tiny", 2, 16, {"is_post_ln": False}),
     ("tiny", 1, 64, {"is_post_ln": False, "use_gelu": False}),
     ("tiny", 2, 24, {"hidden": 256, "inner": 512, "head_num": 2}),   # 128-wide heads
+    # heads of 64 at hidden 256: the layers run the QKV + attention kernel (<= 128 tokens) ...
+    ("tiny", 3, 33, {"hidden": 256, "inner": 512, "head_num": 4}),
+    # ... and the GEMM followed by the multi-block attention kernel beyond 128 tokens
+    ("tiny", 2, 160, {"hidden": 256, "inner": 512, "head_num": 4, "max_step": 192}),
 ])
 def test_tiny_stack_with_taps(tmp_path, oracle, cfg_name, batch, seq, over):
     from lightseq_amd import inference, synthetic
