@@ -21,7 +21,7 @@ The JSON line also carries
                  kernel (so the host's launch cost is not what is measured): achieved
                  GB/s = algorithmic bytes (every operand touched once) / mean time per
                  launch, against the 8 TB/s HBM peak;
-  gemm_microbench  the 4096x4096x1024 and 4096x1024x4096 int8 products (uniform codes in
+  gemm_microbench  the 4096x4096x1024 and 4096x1024x4096 int8 products (and 8192^3; uniform codes in
                  [-127, 127]) with int32 output, requantised int8 output and the fused
                  bias+GELU+requantisation epilogue, and the stand-alone
                  dequant-bias-GELU-requant kernel, timed the same way;
@@ -272,7 +272,40 @@ def gemm_microbench(reps=40):
             "frac_of_hbm_peak": nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
         out["%dx%dx%d" % (M, N, Kd)] = res
     out["vendor_yardstick torch._int_mm (int32 out, same box; not used by the library)"] = _int_mm_yardstick(reps)
+    out["large product 8192x8192x8192 (where launch, first-operand and write-back costs vanish)"] = \
+        _large_product(max(reps // 4, 5))
     return out
+
+
+def _large_product(reps):
+    """The library's int8 GEMM and the vendor's on a product large enough that only the tile loop
+    is timed: what the loop reaches on this box, and what the vendor's hand-tuned kernel does."""
+    import torch
+    from lightseq_amd import kernels as K
+    dev = "cuda:0"
+    M = N = Kd = 8192
+    g = torch.Generator(device=dev).manual_seed(1)
+    a = torch.randint(-127, 128, (M, Kd), dtype=torch.int8, device=dev, generator=g)
+    w = torch.randint(-127, 128, (N, Kd), dtype=torch.int8, device=dev, generator=g)
+    c8 = torch.zeros(M, N, dtype=torch.int8, device=dev)
+    c32 = torch.zeros(M, N, dtype=torch.int32, device=dev)
+    ops = 2.0 * M * N * Kd
+    res = {}
+    cases = {
+        "int8 out (requantising epilogue)": lambda: K.gemm_i8_i8o(a, w, c8, M, N, Kd, 1e-4),
+        "int32 out": lambda: K.gemm_i8_i32o(a, w, c32, M, N, Kd),
+    }
+    for name, fn in cases.items():
+        us = _queued_time_us(fn, reps)
+        res[name] = {"avg_us": us, "TOP/s": ops / (us * 1e-6) / 1e12,
+                     "frac_of_int8_mfma_peak": ops / (us * 1e-6) / 1e12 / INT8_MFMA_PEAK_TOPS}
+    try:
+        wt = w.t()
+        us = _queued_time_us(lambda: torch._int_mm(a, wt), reps)
+        res["vendor torch._int_mm (int32 out)"] = {"avg_us": us, "TOP/s": ops / (us * 1e-6) / 1e12}
+    except Exception as e:
+        res["vendor torch._int_mm (int32 out)"] = {"error": repr(e)[:200]}
+    return res
 
 
 def _int_mm_yardstick(reps):
