@@ -248,6 +248,13 @@ int lsh_layer_norm_row_kernel(int on);
  * one against the other.  No counterpart in the reference (its cuBLASLt algorithm table
  * plays this part: model/cublas_algo_map.cc). */
 int lsh_gemm_i8_tile_kernel(int on);
+/* Process-wide switch (default on; returns the previous setting, 0 / 1): with at least 1024
+ * rows and a feature dimension that is a multiple of 64, lsh_ker_bias_gelu_i8I_i8O_* tabulates
+ * the 256 codes of each column per workgroup in LDS and looks the elements up instead of
+ * evaluating the GELU per element.  The table comes from the same routine, so the results are
+ * the same bytes; the switch exists to measure and to test one against the other.  No
+ * counterpart in the reference. */
+int lsh_bias_act_lut_kernel(int on);
 /* The attention out-projection and the LayerNorm after it as one kernel: what
  * lsh_gemm_i8_i8o(A, W, alpha) followed by lsh_ker_residual_bias_ln_i8I_i8O_f16 leaves in
  * `output` (int8 [batch_tokens, hidden_size]) and `residual`, byte for byte (the product is

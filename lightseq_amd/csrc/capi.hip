@@ -107,6 +107,7 @@ int lsh_launch_dequantize_tensor_f32(const int32_t* input, void* output, int bat
 // ---- LayerNorm family --------------------------------------------------------------
 int lsh_layer_norm_row_kernel(int on) { return ln_set_few_rows(on != 0) ? 1 : 0; }
 int lsh_gemm_i8_tile_kernel(int on) { return gemm_i8_enable_tile_kernel(on != 0) ? 1 : 0; }
+int lsh_bias_act_lut_kernel(int on) { return bias_act_enable_lut_kernel(on != 0) ? 1 : 0; }
 int lsh_tile_weight_16x64(const int8_t* w, int8_t* tiled, int n, int k, lsh_stream_t stream) {
   return tile_weight_16x64(w, tiled, n, k, HS(stream));
 }

@@ -198,6 +198,7 @@ void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop);
 // A/B switch: route large products to the persistent kernels instead of the one-tile-per-
 // workgroup kernel (on by default)
 bool gemm_i8_enable_tile_kernel(bool on);  // returns the previous setting
+bool bias_act_enable_lut_kernel(bool on);  // returns the previous setting
 // register-resident int8 MFMA loop (measurement aid): out needs workgroups * 256 ints; *ops
 // receives the integer operations of one launch
 int mfma_i8_peak_probe(int* out, int workgroups, int iters, double* ops, hipStream_t s);

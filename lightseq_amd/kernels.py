@@ -574,6 +574,12 @@ def gemm_i8_tile_kernel(on):
     return bool(lib.load().lsh_gemm_i8_tile_kernel(int(bool(on))))
 
 
+def bias_act_lut_kernel(on):
+    """Let ker_bias_gelu_i8I_i8O tabulate each column's 256 codes in LDS for tensors of 1024
+    rows and more (default) or always evaluate per element; returns the previous setting."""
+    return bool(lib.load().lsh_bias_act_lut_kernel(int(bool(on))))
+
+
 def tile_weight_16x64(w, tiled, n, k):
     """[n, k] int8 -> the MFMA-ordered tiling :func:`gemm_i8_residual_ln_i8O` streams."""
     _dev(w, tiled)

@@ -57,6 +57,7 @@ _SIGNATURES = {
     "lsh_gemm_i8_preferred_ksplit": (False, "iii"),
     "lsh_layer_norm_row_kernel": (False, "i"),
     "lsh_gemm_i8_tile_kernel": (False, "i"),
+    "lsh_bias_act_lut_kernel": (False, "i"),
     "lsh_mfma_i8_peak_probe": (False, "piips"),
     "lsh_tile_weight_16x64": (False, "ppiis"),
     "lsh_gemm_i8_residual_ln_i8O_f16": (False, "pp" + "f" + "ppppp" + "iii" + "ff" + "s" + "i"),

@@ -151,6 +151,35 @@ def test_bias_gelu(oracle, rng, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4096, 3072), (1024, 64), (1500, 192), (5000, 1088), (2049, 320), (3000, 1280), (16500, 256), (20000, 64)])
+def test_bias_gelu_tabulated_equals_evaluated(oracle, rng, dtype, shape):
+    """With 1024 rows or more the kernel looks the codes up in per-column tables built in LDS:
+    the same bytes as evaluating every element (all 256 input codes occur, -128 included), in
+    place as well, and within the oracle's tolerance."""
+    tokens, feat = shape
+    x = rng.integers(-128, 128, size=shape, dtype=np.int8)
+    bias = _randT(rng, (feat,), dtype, 0.3)
+    ds, qs = 2.2 / 127, 127 / 2.2
+    xd, bd = to_dev(x), to_dev(bias)
+    tab = torch.zeros(shape, dtype=torch.int8, device=DEV)
+    ev = torch.zeros(shape, dtype=torch.int8, device=DEV)
+    k = _k()
+    k.ker_bias_gelu_i8I_i8O_launcher(tokens, xd, tab, bd, feat, ds, qs)
+    prev = k.bias_act_lut_kernel(False)
+    try:
+        k.ker_bias_gelu_i8I_i8O_launcher(tokens, xd, ev, bd, feat, ds, qs)
+    finally:
+        k.bias_act_lut_kernel(prev)
+    assert prev is True
+    assert torch.equal(tab, ev)
+    inplace = xd.clone()
+    k.ker_bias_gelu_i8I_i8O_launcher(tokens, inplace, inplace, bd, feat, ds, qs)
+    assert torch.equal(inplace, ev)
+    valid = x != -128  # the oracle's domain is the symmetric code range
+    assert_codes_close(to_np(tab)[valid], oracle.bias_gelu_i8I_i8O(np.where(valid, x, 0).astype(np.int8), bias, ds, qs)[valid])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("narrow", [False, True])
 @pytest.mark.parametrize("shape", [(33, 2048), (5, 100)])
 def test_bias_relu(oracle, rng, dtype, narrow, shape):
