@@ -148,8 +148,9 @@ def measured_mfma_peak(reps=5):
     return best
 
 
-def fused_kernel_rates(cfg, reps=50):
-    """Each memory-bound kernel of one encoder layer alone, at the workload's shapes."""
+def fused_kernel_rates(cfg, reps=50, BATCH=BATCH):
+    """Each memory-bound kernel of one encoder layer alone, at the workload's shapes (or, with
+    another ``BATCH``, on tensors large enough that launch and first-byte costs vanish)."""
     import torch
     from lightseq_amd import kernels as K
     dev = "cuda:0"
@@ -492,6 +493,8 @@ def bench_bert(args):
         out["two_batches_in_flight"] = two_batches_in_flight(path_factory=lambda: _write_model(cfg),
                                                              steps=args.steps)
         out["fused_kernels"] = fused_kernel_rates(cfg)
+        out["fused_kernels_at_batch_512 (same kernels on 16 x the rows)"] = \
+            fused_kernel_rates(cfg, reps=20, BATCH=512)
         out["gemm_microbench"] = gemm_microbench()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, msg, ids)
