@@ -248,6 +248,12 @@ int lsh_layer_norm_row_kernel(int on);
  * one against the other.  No counterpart in the reference (its cuBLASLt algorithm table
  * plays this part: model/cublas_algo_map.cc). */
 int lsh_gemm_i8_tile_kernel(int on);
+/* Process-wide switch (default on; returns the previous setting, 0 / 1): products of at most
+ * 64 rows (decode steps) whose K range per workgroup is a multiple of 256 run on 16 x 16 x 64
+ * matrix instructions, where a load instruction of a wavefront reads whole 64-byte segments of
+ * 16 weight rows; off sends them to the 32 x 32 x 32 kernel that serves the other K.  Results
+ * are identical either way (integer sums).  No counterpart in the reference. */
+int lsh_gemm_i8_decode_kernel_16x16(int on);
 /* Process-wide switch (default on; returns the previous setting, 0 / 1): with at least 1024
  * rows and a feature dimension that is a multiple of 64, lsh_ker_bias_gelu_i8I_i8O_* tabulates
  * the 256 codes of each column per workgroup in LDS and looks the elements up instead of
@@ -287,6 +293,31 @@ int lsh_gemm_i8_decself_qkv_i8o_f16(const int8_t* A, const int8_t* W, const void
                                     int step_token_num, int hidden, int k, int head_num,
                                     int max_step, int step_id, float alpha, float dequant_scale,
                                     float quant_scale, lsh_stream_t stream);
+/* lsh_gemm_i8_decself_qkv_i8o_f16 followed by lsh_decself_attention_i8 (step_num = step_id + 1)
+ * as one launch, for heads of 64 dimensions, hidden % 128 == 0, hidden <= 1024 and max_step <=
+ * 4096 (LSH_ERR_UNSUPPORTED otherwise): x int8 [rows, hidden] x qkv_weight [3*hidden, hidden]
+ * -> q codes to new_q [rows, hidden], k and v codes to slot step_id of the caches [rows,
+ * head_num, max_step, 64] (the same bytes as the stand-alone product), then the attention of
+ * every (row, head) over slots 0..step_id -> int8 context codes ctx [rows, hidden] (the same
+ * bytes as the stand-alone attention for caches of more than 64 and at most 256 steps; with
+ * other lengths the value sums run in another tree and a code can differ by one next to a
+ * rounding boundary).  alpha, dequant_scale, cache_quant_scale: the scales of the product;
+ * attn_scale, cache_dequant_scale, ctx_quant_scale: those of the attention.  ctx must not alias
+ * x.  Replaces the launches of model/quant_decoder.cc.cu:660-700 and
+ * model/quant_gpt_encoder.cc.cu:640-680.  No counterpart in the reference. */
+int lsh_decself_qkv_attention_i8_f16(const int8_t* x, const int8_t* qkv_weight,
+                                     const void* qkv_bias, int8_t* new_q, int8_t* k_cache,
+                                     int8_t* v_cache, int8_t* ctx, int rows, int hidden,
+                                     int head_num, int max_step, int step_id, float alpha,
+                                     float dequant_scale, float cache_quant_scale,
+                                     float attn_scale, float cache_dequant_scale,
+                                     float ctx_quant_scale, lsh_stream_t stream);
+/* Process-wide switch (default off; returns the previous setting, 0 / 1): QuantTransformer and
+ * QuantGpt run the decode-step self attention through lsh_decself_qkv_attention_i8_f16 where it
+ * is supported, or through the two launches it replaces.  Off by default: measured on whole
+ * generation runs the single launch is no faster than the pair (the projection of a head is
+ * too little work to hide its weight stream).  No counterpart in the reference. */
+int lsh_decself_qkv_attention_in_models(int on);
 /* Decode-step cross-attention query product with ker_arrange_encdec_q_i8I
  * (kernels/transformerKernels_int8.cc.cu:1596-1645; call site model/quant_decoder.cc.cu:745-760)
  * as its epilogue: A [step_token_num, k] x W [hidden, k] -> int8 code (alpha) ->

@@ -107,6 +107,9 @@ int lsh_launch_dequantize_tensor_f32(const int32_t* input, void* output, int bat
 // ---- LayerNorm family --------------------------------------------------------------
 int lsh_layer_norm_row_kernel(int on) { return ln_set_few_rows(on != 0) ? 1 : 0; }
 int lsh_gemm_i8_tile_kernel(int on) { return gemm_i8_enable_tile_kernel(on != 0) ? 1 : 0; }
+int lsh_gemm_i8_decode_kernel_16x16(int on) {
+  return gemm_i8_enable_skinny16_kernel(on != 0) ? 1 : 0;
+}
 int lsh_bias_act_lut_kernel(int on) { return bias_act_enable_lut_kernel(on != 0) ? 1 : 0; }
 int lsh_tile_weight_16x64(const int8_t* w, int8_t* tiled, int n, int k, lsh_stream_t stream) {
   return tile_weight_16x64(w, tiled, n, k, HS(stream));
@@ -370,6 +373,21 @@ int lsh_gemm_i8_decself_qkv_i8o_f16(const int8_t* A, const int8_t* W, const void
   return gemm_i8_decself_qkv_i8o(A, W, H(qkv_bias), new_q, new_k, new_v, step_token_num, hidden, k,
                                  head_num, max_step, step_id, alpha, dequant_scale, quant_scale,
                                  HS(stream));
+}
+int lsh_decself_qkv_attention_in_models(int on) {
+  return decself_qkv_attention_enable(on != 0) ? 1 : 0;
+}
+int lsh_decself_qkv_attention_i8_f16(const int8_t* x, const int8_t* qkv_weight,
+                                     const void* qkv_bias, int8_t* new_q, int8_t* k_cache,
+                                     int8_t* v_cache, int8_t* ctx, int rows, int hidden,
+                                     int head_num, int max_step, int step_id, float alpha,
+                                     float dequant_scale, float cache_quant_scale,
+                                     float attn_scale, float cache_dequant_scale,
+                                     float ctx_quant_scale, lsh_stream_t stream) {
+  return decself_qkv_attention_i8(x, qkv_weight, H(qkv_bias), new_q, k_cache, v_cache, ctx, rows,
+                                  hidden, head_num, max_step, step_id, alpha, dequant_scale,
+                                  cache_quant_scale, attn_scale, cache_dequant_scale,
+                                  ctx_quant_scale, HS(stream));
 }
 int lsh_gemm_i8_encdec_q_f16(const int8_t* A, const int8_t* W, const void* q_bias, void* new_q,
                              int step_token_num, int hidden, int k, int beam_size, int head_num,

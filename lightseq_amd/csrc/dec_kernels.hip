@@ -6,6 +6,7 @@
 // rows, not tiling.  A wavefront owns one (row, head) pair in the attention kernels;
 // all cross-lane traffic is wave reductions, and sums run in a fixed order so that a
 // step is reproducible bit for bit.
+#include "dec_attend.cuh"
 #include "ls_device.cuh"
 #include "ls_launch.h"
 
@@ -206,117 +207,15 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
                        const int8_t* __restrict__ v_cache, int8_t* __restrict__ new_v,
                        int step_num, int max_step, int head_num, float attn_scale, float dq,
                        float quant_scale) {
-#pragma clang fp contract(off)
-  constexpr int CH = D / 16;    // lanes per cache row
-  constexpr int KPW = 64 / CH;  // rows per wavefront per load
   extern __shared__ float lds_f[];
-  const int padded = (step_num + 63) & ~63;
-  float* probs = lds_f;                 // [padded]
-  float* red = lds_f + padded;          // [16] block reductions
-  float* part = red + 16;               // [NWV][D] per-wavefront value sums
-  const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
   const long bh = blockIdx.x;
-  const int c = lane % CH, grp = lane / CH;
-  const int8_t* kb = k_cache + bh * (long)max_step * D;
-  const int8_t* vb = v_cache + bh * (long)max_step * D;
-  const uint4 qv = *reinterpret_cast<const uint4*>(q + bh * D + c * 16);
-
-  // The cache is read in rounds of UN independent 16-byte loads per lane (UN * NWV * KPW
-  // steps per round), all issued before the first is used: a step costs one memory round
-  // trip per round instead of one per KPW * 4 cached steps.
-
-  // scores -> scaled logits in LDS
-  float mx = kFloatInfNeg;
-  for (int base = wid * KPW; base < step_num; base += UN * NWV * KPW) {
-    uint4 kv[UN];
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int j = base + u * NWV * KPW + grp;
-      // clamped instead of predicated: unconditional loads stay back to back
-      kv[u] = *reinterpret_cast<const uint4*>(kb + (long)min(j, step_num - 1) * D + c * 16);
-    }
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int j = base + u * NWV * KPW + grp;
-      int sc = 0;
-      sc = __builtin_amdgcn_sdot4((int)qv.x, (int)kv[u].x, sc, false);
-      sc = __builtin_amdgcn_sdot4((int)qv.y, (int)kv[u].y, sc, false);
-      sc = __builtin_amdgcn_sdot4((int)qv.z, (int)kv[u].z, sc, false);
-      sc = __builtin_amdgcn_sdot4((int)qv.w, (int)kv[u].w, sc, false);
-#pragma unroll
-      for (int m = 1; m < CH; m <<= 1) sc += __shfl_xor(sc, m, 64);
-      if (j < step_num) {
-        const float val = (float)sc * dq * dq * attn_scale;
-        if (c == 0) probs[j] = val;
-        mx = fmaxf(mx, val);
-      }
-    }
-  }
-  // the first round of value loads travels while the softmax is computed
-  uint4 vv0[UN];
-#pragma unroll
-  for (int u = 0; u < UN; ++u) {
-    const int j = wid * KPW + u * NWV * KPW + grp;
-    vv0[u] = *reinterpret_cast<const uint4*>(vb + (long)min(j, step_num - 1) * D + c * 16);
-  }
-  mx = block_max(mx, red);
-  float sum = 0.f;
-  for (int j = tid; j < step_num; j += 64 * NWV) {
-    const float e = __expf(probs[j] - mx);
-    probs[j] = e;
-    sum += e;
-  }
-  sum = block_sum(sum, red);
-  for (int j = tid; j < step_num; j += 64 * NWV) probs[j] = probs[j] / sum;
-  __syncthreads();
-
-  // value sum: lane (grp, c) accumulates dims [16c, 16c+16) over steps grp, grp + KPW * NWV, ...
-  float acc[16];
-#pragma unroll
-  for (int k = 0; k < 16; ++k) acc[k] = 0.f;
-  for (int base = wid * KPW; base < step_num; base += UN * NWV * KPW) {
-    uint4 vv[UN];
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int j = base + u * NWV * KPW + grp;
-      if (base == wid * KPW)
-        vv[u] = vv0[u];
-      else
-        vv[u] = *reinterpret_cast<const uint4*>(vb + (long)min(j, step_num - 1) * D + c * 16);
-    }
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int j = base + u * NWV * KPW + grp;
-      if (j < step_num) {  // same ascending order of steps per lane as a plain loop
-        const float p = probs[j];
-        const uint32_t w[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
-#pragma unroll
-        for (int k = 0; k < 16; ++k) acc[k] += (float)unpack_i8(w[k >> 2], k & 3) * p * dq;
-      }
-    }
-  }
-#pragma unroll
-  for (int m = CH; m < 64; m <<= 1)
-#pragma unroll
-    for (int k = 0; k < 16; ++k) acc[k] += __shfl_xor(acc[k], m, 64);
-  if (grp == 0) {
-#pragma unroll
-    for (int k = 0; k < 16; ++k) part[wid * D + c * 16 + k] = acc[k];
-  }
-  __syncthreads();
-  if (tid < D) {
-    float t[NWV];  // pairwise tree over the wavefronts' partial sums
-#pragma unroll
-    for (int i = 0; i < NWV; ++i) t[i] = part[i * D + tid];
-#pragma unroll
-    for (int st = 1; st < NWV; st *= 2)
-#pragma unroll
-      for (int i = 0; i < NWV; i += 2 * st) t[i] += t[i + st];
-    const float v = t[0];
-    const long row = bh / head_num;
-    const int head = (int)(bh % head_num);
-    new_v[row * ((long)head_num * D) + (long)head * D + tid] = (int8_t)float2int8(v, quant_scale);
-  }
+  const long row = bh / head_num;
+  const int head = (int)(bh % head_num);
+  decself_attend_row<D, NWV, UN>(q + bh * D, k_cache + bh * (long)max_step * D,
+                                 v_cache + bh * (long)max_step * D,
+                                 new_v + row * ((long)head_num * D) + (long)head * D, true, step_num,
+                                 attn_scale, dq, quant_scale, lds_f, threadIdx.x >> 6,
+                                 threadIdx.x & 63);
 }
 
 static int decself_check(long bh_total, int step_num, int max_step, int head_num, int d) {

@@ -116,11 +116,23 @@ struct EpiDecQkvI8 {
   const __half* bias;
   float alpha, dequant_scale, quant_scale;
   int hidden, head_num, dim_per_head, max_step, step_id;
-  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool) const {
+  // the 16 bias values of columns n .. n + 15: they do not depend on the product, so the
+  // decode-step kernel requests them with its first weights
+  struct Pre {
+    half8_t b0, b1;
+  };
+  __device__ __forceinline__ Pre prefetch(int n) const {
+    return Pre{*reinterpret_cast<const half8_t*>(bias + n),
+               *reinterpret_cast<const half8_t*>(bias + n + 8)};
+  }
+  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
+    store16_pre(m, n, N, c, full, prefetch(n));
+  }
+  __device__ __forceinline__ void store16_pre(long m, int n, int N, const v16i& c, bool,
+                                              const Pre& pre) const {
 #pragma clang fp contract(off)
     const int part = n / hidden, i = n - part * hidden;
-    const half8_t b0 = *reinterpret_cast<const half8_t*>(bias + n);
-    const half8_t b1 = *reinterpret_cast<const half8_t*>(bias + n + 8);
+    const half8_t b0 = pre.b0, b1 = pre.b1;
     int q[16];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
@@ -157,12 +169,22 @@ struct EpiEncdecQF16 {
   const __half* bias;
   float alpha, dequant_scale;
   int beam_size, head_num, dim_per_head;
-  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool) const {
+  struct Pre {  // the bias of columns n .. n + 15, requested ahead of the product
+    half8_t b0, b1;
+  };
+  __device__ __forceinline__ Pre prefetch(int n) const {
+    return Pre{*reinterpret_cast<const half8_t*>(bias + n),
+               *reinterpret_cast<const half8_t*>(bias + n + 8)};
+  }
+  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
+    store16_pre(m, n, N, c, full, prefetch(n));
+  }
+  __device__ __forceinline__ void store16_pre(long m, int n, int N, const v16i& c, bool,
+                                              const Pre& pre) const {
     const int head = n / dim_per_head, dim = n - head * dim_per_head;
     const long batch_id = m / beam_size, beam_id = m - batch_id * beam_size;
     __half* dst = new_q + ((batch_id * head_num + head) * beam_size + beam_id) * dim_per_head + dim;
-    const half8_t b0 = *reinterpret_cast<const half8_t*>(bias + n);
-    const half8_t b1 = *reinterpret_cast<const half8_t*>(bias + n + 8);
+    const half8_t b0 = pre.b0, b1 = pre.b1;
     half8_t lo, hi;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
@@ -316,6 +338,25 @@ struct EpiQkvF16 {
   }
   bool vec_ok(int) const { return true; }
   static const char* name() { return "EpiQkvF16"; }
+};
+
+// Epilogues with operands that can be requested before the product is known (decode-step
+// kernel): a bias slice kept in registers, or the table rows of the workgroup's columns in LDS.
+struct EpiNoPre {};
+template <typename Epi>
+struct epi_pre {
+  typedef EpiNoPre type;
+  static constexpr bool value = false;
+};
+template <>
+struct epi_pre<EpiDecQkvI8> {
+  typedef EpiDecQkvI8::Pre type;
+  static constexpr bool value = true;
+};
+template <>
+struct epi_pre<EpiEncdecQF16> {
+  typedef EpiEncdecQF16::Pre type;
+  static constexpr bool value = true;
 };
 
 // FULL: every 16-column group of the output exists and may be stored as a vector (N % 16
@@ -1031,6 +1072,8 @@ __global__ void __launch_bounds__(256)
 gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
                       int N, int K, int, int, bool vec_store, int ksplit) {
   __shared__ int red[4][MBLK][16][64];  // [wavefront][m block][register][lane]
+  constexpr bool kLut = std::is_same<Epi, EpiLutI8>::value;
+  __shared__ __align__(16) int8_t tab[kLut ? 32 * 256 : 16];  // table rows of the 32 columns
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, g = lane >> 5;
   // blockIdx.x = column block + (K range) * column blocks; range p stores to rows
@@ -1038,6 +1081,17 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   const int ncol = (int)gridDim.x / ksplit;
   const int part = (int)blockIdx.x / ncol;
   const int n0 = ((int)blockIdx.x % ncol) * 32;
+  // What the epilogue reads besides the product is requested first, so that it travels with
+  // the weights instead of after the last matrix instruction: the bias slice of the lane's 16
+  // columns, or 32 bytes per thread of the 32 table rows (columns past N clamped).
+  typename epi_pre<Epi>::type pre;
+  if constexpr (epi_pre<Epi>::value) pre = epi.prefetch(max(min(n0 + 16 * g, N - 16), 0));
+  uint4 tab0, tab1;
+  if constexpr (kLut) {
+    const int8_t* tp = epi_lut(epi) + (long)min(n0 + (tid >> 3), N - 1) * 256 + (tid & 7) * 32;
+    tab0 = *reinterpret_cast<const uint4*>(tp);
+    tab1 = *reinterpret_cast<const uint4*>(tp + 16);
+  }
   const int8_t* wp = W + (long)min(n0 + sigma(l32), N - 1) * K + g * 64;
   const int8_t* ap[MBLK];
 #pragma unroll
@@ -1081,6 +1135,10 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   for (int i = 0; i < MBLK; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) red[wave][i][r][lane] = acc[i][r];
+  if constexpr (kLut) {
+    *reinterpret_cast<uint4*>(tab + (tid >> 3) * 256 + (tid & 7) * 32) = tab0;
+    *reinterpret_cast<uint4*>(tab + (tid >> 3) * 256 + (tid & 7) * 32 + 16) = tab1;
+  }
   __syncthreads();
   if (wave < MBLK) {
     v16i c;
@@ -1090,8 +1148,123 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
              (red[2][wave][r][lane] + red[3][wave][r][lane]);
     const long m = wave * 32 + l32;
     const int n = n0 + 16 * g;
-    if (m < M && n < N)
-      epi.store16(m + (long)part * M, n, N, c, FULL ? true : (vec_store && n + 16 <= N));
+    if (m < M && n < N) {
+      const bool full = FULL ? true : (vec_store && n + 16 <= N);
+      if constexpr (kLut)
+        epi.store16_lds(m + (long)part * M, n, N, c, full, tab, 16 * g);
+      else if constexpr (epi_pre<Epi>::value)
+        epi.store16_pre(m + (long)part * M, n, N, c, full, pre);
+      else
+        epi.store16(m + (long)part * M, n, N, c, full);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Decode-step path on 16 x 16 x 64 products (K range of a workgroup a multiple of 256 bytes).
+// The 32 x 32 x 32 form above gives a lane one weight row, so a load instruction of a
+// wavefront touches 64 different 64-byte segments and uses 16 bytes of each: the address unit
+// of the compute unit, not memory, bounds it (measured: 3.4 us from the first instruction to
+// the last product of a 32 KB slab).  With 16 x 16 x 64 products the four lanes l, l + 16,
+// l + 32, l + 48 hold the four 16-byte quarters of one row's 64-byte K slice, so an
+// instruction reads 16 whole segments, and 16 activation rows -- one decoding batch -- fill
+// the product with nothing clamped.  A workgroup still owns 32 output columns (two 16-column
+// blocks) for all rows; wavefront w takes the w-th quarter of the workgroup's K range, four
+// slices per round, every load of a round requested before its first product; the partial
+// tiles meet in LDS, where the epilogue threads (one per row and column block) gather the 16
+// columns the epilogues expect.
+// ---------------------------------------------------------------------------------
+template <typename Epi, int MB, bool FULL>
+__global__ void __launch_bounds__(256)
+gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
+                        int N, int K, int kw, int, bool vec_store, int) {
+  __shared__ int red[4][MB][2][4][64];  // [wavefront][row block][column block][register][lane]
+  constexpr bool kLut = std::is_same<Epi, EpiLutI8>::value;
+  __shared__ __align__(16) int8_t tab[kLut ? 32 * 256 : 16];  // table rows of the 32 columns
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kq = lane >> 4;
+  // grid: x = column block, y = K range (plane of the output); kw = bytes of K per wavefront,
+  // a multiple of 64, from the host: a kernel of a few microseconds cannot afford integer
+  // divisions and kernel-argument loads that wait for one another before its first load
+  const int part = (int)blockIdx.y;
+  const int n0 = (int)blockIdx.x * 32;
+  // epilogue thread t: row t % (16 MB), column block t / (16 MB) (threads beyond 32 MB idle)
+  const int em = tid % (16 * MB), eblk = (tid / (16 * MB)) & 1;
+  // What the epilogue reads besides the product travels with the weights.
+  typename epi_pre<Epi>::type pre;
+  if constexpr (epi_pre<Epi>::value) pre = epi.prefetch(max(min(n0 + 16 * eblk, N - 16), 0));
+  uint4 tab0, tab1;
+  if constexpr (kLut) {
+    const int8_t* tp = epi_lut(epi) + (long)min(n0 + (tid >> 3), N - 1) * 256 + (tid & 7) * 32;
+    tab0 = *reinterpret_cast<const uint4*>(tp);
+    tab1 = *reinterpret_cast<const uint4*>(tp + 16);
+  }
+  const long kbase = ((long)part * 4 + wave) * kw + kq * 16;
+  const int8_t* wp[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) wp[b] = W + (long)min(n0 + 16 * b + l16, N - 1) * K + kbase;
+  const int8_t* ap[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i) ap[i] = A + (long)min(16 * i + l16, M - 1) * K + kbase;
+  v4i acc[MB][2];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) acc[i][b] = (v4i)0;
+  const int ns = kw / 64;
+  for (int s0 = 0; s0 < ns; s0 += 4) {
+    v4i wv[4][2], av[4][MB];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int off = min(s0 + u, ns - 1) * 64;  // clamped: the loads stay unconditional
+#pragma unroll
+      for (int b = 0; b < 2; ++b) wv[u][b] = *reinterpret_cast<const v4i*>(wp[b] + off);
+#pragma unroll
+      for (int i = 0; i < MB; ++i) av[u][i] = *reinterpret_cast<const v4i*>(ap[i] + off);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (s0 + u < ns) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+            acc[i][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[u][b], av[u][i], acc[i][b], 0, 0, 0);
+      }
+    }
+  }
+  // lane holds C[row 16 i + l16][column n0 + 16 b + 4 kq + r], r = 0..3
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][i][b][r][lane] = acc[i][b][r];
+  if constexpr (kLut) {
+    *reinterpret_cast<uint4*>(tab + (tid >> 3) * 256 + (tid & 7) * 32) = tab0;
+    *reinterpret_cast<uint4*>(tab + (tid >> 3) * 256 + (tid & 7) * 32 + 16) = tab1;
+  }
+  __syncthreads();
+  if (tid < 32 * MB) {
+    const int n = n0 + 16 * eblk;
+    if (em < M && n < N) {
+      v16i c;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int src = q * 16 + (em & 15);
+          c[4 * q + r] = (red[0][em >> 4][eblk][r][src] + red[1][em >> 4][eblk][r][src]) +
+                         (red[2][em >> 4][eblk][r][src] + red[3][em >> 4][eblk][r][src]);
+        }
+      const bool full = FULL ? true : (vec_store && n + 16 <= N);
+      if constexpr (kLut)
+        epi.store16_lds(em + (long)part * M, n, N, c, full, tab, 16 * eblk);
+      else if constexpr (epi_pre<Epi>::value)
+        epi.store16_pre(em + (long)part * M, n, N, c, full, pre);
+      else
+        epi.store16(em + (long)part * M, n, N, c, full);
+    }
   }
 }
 
@@ -1101,6 +1274,8 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
 static thread_local hipEvent_t g_ev_start = nullptr, g_ev_stop = nullptr;
 // switch for A/B measurements of the one-tile-per-workgroup kernel against the persistent ones
 static bool g_tile_kernel_enabled = true;
+// the same for the two decode-step kernels (tests compare them bit for bit)
+static bool g_skinny16_enabled = true;
 
 void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop) {
   g_ev_start = start;
@@ -1138,16 +1313,17 @@ static int raise_lds_limit(size_t smem) {
 template <auto Kern, typename Epi>
 static int launch(int grid, int threads, size_t smem, const int8_t* A, const int8_t* W, Epi epi,
                   int M, int N, int K, int tiles_m, int tiles_n, bool vec_store, hipStream_t s,
-                  int ksplit = 1) {
+                  int ksplit = 1, int grid_y = 1) {
   if (int rc = raise_lds_limit<Kern>(smem)) return rc;
   if (g_ev_start != nullptr) {
     // kernel-exact begin/end timestamps on the launch stream
     hipEvent_t e0 = g_ev_start, e1 = g_ev_stop;
     g_ev_start = g_ev_stop = nullptr;
-    hipExtLaunchKernelGGL(Kern, dim3(grid), dim3(threads), (unsigned)smem, s, e0, e1, 0, A, W, epi,
-                          M, N, K, tiles_m, tiles_n, vec_store, ksplit);
+    hipExtLaunchKernelGGL(Kern, dim3(grid, grid_y), dim3(threads), (unsigned)smem, s, e0, e1, 0, A,
+                          W, epi, M, N, K, tiles_m, tiles_n, vec_store, ksplit);
   } else {
-    Kern<<<grid, threads, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store, ksplit);
+    Kern<<<dim3(grid, grid_y), threads, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store,
+                                                   ksplit);
   }
   return lsh_check_launch("gemm_i8_kernel");
 }
@@ -1251,6 +1427,20 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   const bool full = vec_store && N % 16 == 0;  // no column tail: the lean instantiation
   if (M <= 64 && K % kBK == 0) {
     const int grid = ((N + 31) / 32) * ksplit;
+    if ((K / ksplit) % 256 == 0 && g_skinny16_enabled) {
+      // whole 64-byte slices for each of the four wavefronts: the 16 x 16 x 64 form
+#define LSH_SKINNY16(MB)                                                                       \
+  (full ? launch<gemm_i8_skinny16_kernel<Epi, MB, true>>(grid / ksplit, 256, 0, A, W, epi, M, N,  \
+                                                         K, K / ksplit / 4, 0, vec_store, s,     \
+                                                         ksplit, ksplit)                         \
+        : launch<gemm_i8_skinny16_kernel<Epi, MB, false>>(grid / ksplit, 256, 0, A, W, epi, M, N, \
+                                                          K, K / ksplit / 4, 0, vec_store, s,    \
+                                                          ksplit, ksplit))
+      if (M <= 16) return LSH_SKINNY16(1);
+      if (M <= 32) return LSH_SKINNY16(2);
+      return LSH_SKINNY16(4);
+#undef LSH_SKINNY16
+    }
     if (M <= 32) {
       if (full)
         return launch<gemm_i8_skinny_kernel<Epi, 1, true>>(grid, 256, 0, A, W, epi, M, N, K, 0, 0,
@@ -1343,7 +1533,15 @@ bool gemm_i8_enable_tile_kernel(bool on) {
   return prev;
 }
 
+bool gemm_i8_enable_skinny16_kernel(bool on) {
+  const bool prev = g_skinny16_enabled;
+  g_skinny16_enabled = on;
+  return prev;
+}
+
 std::string gemm_i8_kernel_name(int M, int N, int K, const char* epilogue) {
+  if (M <= 64 && K % 256 == 0 && g_skinny16_enabled)
+    return std::string("gemm_i8_skinny16_kernel<") + epilogue + ">";
   if (M <= 64 && K % kBK == 0) return std::string("gemm_i8_skinny_kernel<") + epilogue + ">";
   if (!stream_ok(M, N, K)) return std::string("gemm_i8_generic_kernel<") + epilogue + ">";
   const std::string e = epilogue ? epilogue : "";

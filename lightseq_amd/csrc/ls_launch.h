@@ -176,6 +176,17 @@ int gemm_i8_decself_qkv_i8o(const int8_t* A, const int8_t* W, const __half* qkv_
                             int8_t* new_k, int8_t* new_v, int step_token_num, int hidden, int K,
                             int head_num, int max_step, int step_id, float alpha,
                             float dequant_scale, float quant_scale, hipStream_t s);
+// gemm_i8_decself_qkv_i8o followed by decself_attention_i8 (step_num = step_id + 1) in one
+// launch, for heads of 64 dimensions (dec_qkv_attn_kernels.hip).  ctx must not alias x.
+bool decself_qkv_attention_supported(int rows, int hidden, int head_num, int max_step);
+bool decself_qkv_attention_enable(bool on);  // what the models do; returns the previous setting
+bool decself_qkv_attention_enabled();
+int decself_qkv_attention_i8(const int8_t* x, const int8_t* qkv_weight, const __half* qkv_bias,
+                             int8_t* new_q, int8_t* k_cache, int8_t* v_cache, int8_t* ctx,
+                             int rows, int hidden, int head_num, int max_step, int step_id,
+                             float alpha, float dequant_scale, float cache_quant_scale,
+                             float attn_scale, float cache_dequant_scale, float ctx_quant_scale,
+                             hipStream_t s);
 // Decode-step cross-attention query product with ker_arrange_encdec_q_i8I as its epilogue:
 // fp16 q [batch, heads, beam, d].
 int gemm_i8_encdec_q_f16(const int8_t* A, const int8_t* W, const __half* q_bias, __half* new_q,
@@ -198,6 +209,9 @@ void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop);
 // A/B switch: route large products to the persistent kernels instead of the one-tile-per-
 // workgroup kernel (on by default)
 bool gemm_i8_enable_tile_kernel(bool on);  // returns the previous setting
+// The same for the decode-step products (M <= 64): the 16 x 16 x 64 kernel (default, where a
+// workgroup's K range is a multiple of 256) or the 32 x 32 x 32 one; same bits.
+bool gemm_i8_enable_skinny16_kernel(bool on);
 bool bias_act_enable_lut_kernel(bool on);  // returns the previous setting
 // register-resident int8 MFMA loop (measurement aid): out needs workgroups * 256 ints; *ops
 // receives the integer operations of one launch

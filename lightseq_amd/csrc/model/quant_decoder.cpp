@@ -325,6 +325,18 @@ void QuantDecoder::self_attention() {
   const size_t mh = (size_t)M * H;
   TAP("self_ln_q", _buf_a.get(), mh);
   TAP("res_in", _cur_step_query.get(), mh * sizeof(__half));
+  const float attn_scale =
+      __half2float(__float2half_rn(sqrtf(1.f / (float)_tw._dim_per_head)));
+  // With taps set the two launches run, so that q and the caches are copied before the
+  // attention as the tap names promise; the bytes are the same either way.
+  if (!step_taps.any() && decself_qkv_attention_enabled() && _tw._dim_per_head == 64 &&
+      decself_qkv_attention_supported(M, H, _tw._head_num, _tw._max_step)) {
+    LSH_CALL(decself_qkv_attention_i8(_buf_a.get(), w.w_self_qkv.get(), w.b_self_qkv.get(),
+                                      _buf_q.get(), k_cache, v_cache, _buf_b.get(), M, H,
+                                      _tw._head_num, _tw._max_step, _cur_step,
+                                      c[0] * c[6] / (c[12] * Q), c[12] / Q, Q / c[18], attn_scale,
+                                      c[18] / Q, Q / c[7], _stream));
+  } else {
   // QKV product; its epilogue is ker_arrange_decself_qkv_i8I_i8O: q -> _buf_q, k / v -> slot
   // _cur_step of the caches (all three with the cache clip)
   if (_tw._dim_per_head % 16 == 0) {
@@ -344,11 +356,10 @@ void QuantDecoder::self_attention() {
   TAP("self_k_cache", k_cache, mh * _tw._max_step);
   TAP("self_v_cache", v_cache, mh * _tw._max_step);
   // int8 q.K -> softmax -> new value, one kernel
-  const float attn_scale =
-      __half2float(__float2half_rn(sqrtf(1.f / (float)_tw._dim_per_head)));
   LSH_CALL(decself_attention_i8(_buf_q.get(), k_cache, v_cache, _buf_b.get(), M * _tw._head_num,
                                 _cur_step + 1, _tw._max_step, _tw._head_num, _tw._dim_per_head,
                                 attn_scale, c[18] / Q, Q / c[7], _stream));
+  }
   TAP("self_ctx_q", _buf_b.get(), mh);
   LSH_CALL(gemm_i8_i8o(_buf_b.get(), w.w_self_out.get(), _buf_a.get(), M, H, H,
                        c[1] * c[7] / (c[13] * Q), _stream));

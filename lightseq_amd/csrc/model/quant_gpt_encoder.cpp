@@ -219,6 +219,15 @@ const int8_t* QuantGptEncoder::step_pass() {
                                              w.ln1_bias.get(), w.b_out.get(), Q / c[4], false));
     TAP("ln1_q", a, bh);
     TAP("res_in", _query.get(), bh * sizeof(__half));
+    // With taps set the two launches run, so that q and the caches are copied before the
+    // attention as the tap names promise.
+    if (!step_taps.any() && decself_qkv_attention_enabled() && _tw._dim_per_head == 64 &&
+        decself_qkv_attention_supported(B, H, _tw._head_num, _tw._max_step)) {
+      LSH_CALL(decself_qkv_attention_i8(a, w.w_qkv.get(), w.b_qkv.get(), _buf_q.get(), k_cache,
+                                        v_cache, b, B, H, _tw._head_num, _tw._max_step,
+                                        _batch_seq_len - 1, c[0] * c[4] / (c[8] * Q), c[8] / Q,
+                                        Q / c[11], _atten_scaler, c[11] / Q, Q / c[5], _stream));
+    } else {
     // QKV product; its epilogue is ker_arrange_decself_qkv_i8I_i8O: q -> _buf_q, k / v appended
     // to the caches at the token's position
     if (_tw._dim_per_head % 16 == 0) {
@@ -240,6 +249,7 @@ const int8_t* QuantGptEncoder::step_pass() {
                                   _batch_seq_len,
                                   _tw._max_step, _tw._head_num, _tw._dim_per_head, _atten_scaler,
                                   c[11] / Q, Q / c[5], _stream));
+    }
     TAP("ctx_q", b, bh);
     LSH_CALL(gemm_i8_i8o(b, w.w_out.get(), a, B, H, H, c[1] * c[5] / (c[9] * Q), _stream));
     TAP("out_q", a, bh);

@@ -560,6 +560,16 @@ def gemm_i8_decself_qkv_i8o(a, w, qkv_bias, new_q, new_k, new_v, step_token_num,
          quant_scale, current_stream())
 
 
+def decself_qkv_attention_i8(x, w, qkv_bias, new_q, k_cache, v_cache, ctx, rows, hidden, head_num,
+                             max_step, step_id, alpha, dequant_scale, cache_quant_scale, attn_scale,
+                             cache_dequant_scale, ctx_quant_scale):
+    """Decode-step QKV product, cache append and self attention of heads of 64 in one launch."""
+    _dev(x, w, qkv_bias, new_q, k_cache, v_cache, ctx)
+    call("lsh_decself_qkv_attention_i8_f16", ptr(x), ptr(w), ptr(qkv_bias), ptr(new_q), ptr(k_cache),
+         ptr(v_cache), ptr(ctx), rows, hidden, head_num, max_step, step_id, alpha, dequant_scale,
+         cache_quant_scale, attn_scale, cache_dequant_scale, ctx_quant_scale, current_stream())
+
+
 def gemm_i8_encdec_q(a, w, q_bias, new_q, step_token_num, hidden, k, beam_size, head_num, alpha,
                      dequant_scale):
     """Decode-step cross-attention query product with ker_arrange_encdec_q_i8I as its epilogue."""
@@ -568,10 +578,22 @@ def gemm_i8_encdec_q(a, w, q_bias, new_q, step_token_num, hidden, k, beam_size, 
          k, beam_size, head_num, alpha, dequant_scale, current_stream())
 
 
+def gemm_i8_decode_kernel_16x16(on):
+    """Route decode-step products (at most 64 rows) to the 16 x 16 x 64 kernel (default) or to
+    the 32 x 32 x 32 one; returns the previous setting."""
+    return bool(lib.load().lsh_gemm_i8_decode_kernel_16x16(int(bool(on))))
+
+
 def gemm_i8_tile_kernel(on):
     """Route large products to the one-tile-per-workgroup kernel (default) or to the persistent
     kernels; returns the previous setting."""
     return bool(lib.load().lsh_gemm_i8_tile_kernel(int(bool(on))))
+
+
+def decself_qkv_attention_in_models(on):
+    """Let the generation models fuse the decode-step QKV product with the self attention
+    (default) or keep the two launches; returns the previous setting."""
+    return bool(lib.load().lsh_decself_qkv_attention_in_models(int(bool(on))))
 
 
 def bias_act_lut_kernel(on):

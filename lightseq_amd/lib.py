@@ -52,12 +52,15 @@ _SIGNATURES = {
     "lsh_build_act_lut": (False, "pp" + "ifffi" + "s"),
     "lsh_gemm_i8_lut_i8o": (False, "pppp" + "iiif" + "s"),
     "lsh_gemm_i8_decself_qkv_i8o_f16": (False, "pppppp" + "iiiiii" + "fff" + "s"),
+    "lsh_decself_qkv_attention_i8_f16": (False, "ppppppp" + "iiiii" + "ffffff" + "s"),
     "lsh_gemm_i8_encdec_q_f16": (False, "pppp" + "iiiii" + "ff" + "s"),
     "lsh_gemm_i8_i32o_splitk": (False, "ppp" + "iiii" + "p" + "s"),
     "lsh_gemm_i8_preferred_ksplit": (False, "iii"),
     "lsh_layer_norm_row_kernel": (False, "i"),
     "lsh_gemm_i8_tile_kernel": (False, "i"),
+    "lsh_gemm_i8_decode_kernel_16x16": (False, "i"),
     "lsh_bias_act_lut_kernel": (False, "i"),
+    "lsh_decself_qkv_attention_in_models": (False, "i"),
     "lsh_mfma_i8_peak_probe": (False, "piips"),
     "lsh_tile_weight_16x64": (False, "ppiis"),
     "lsh_gemm_i8_residual_ln_i8O_f16": (False, "pp" + "f" + "ppppp" + "iii" + "ff" + "s" + "i"),

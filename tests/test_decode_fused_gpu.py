@@ -115,3 +115,73 @@ def test_cross_attention_q_product_equals_the_pair(rng, batch, beam, heads, d, K
     q1 = torch.full((batch, heads, beam, d), 3.0, dtype=torch.float16, device=DEV)
     _k().gemm_i8_encdec_q(to_dev(a), to_dev(w), to_dev(bias), q1, M, H, K, beam, heads, alpha, ds)
     np.testing.assert_array_equal(to_np(q1).view(np.uint16), to_np(q0).view(np.uint16))
+
+
+@pytest.mark.parametrize("M,heads,K,max_step,step", [
+    (16, 16, 1024, 700, 639),   # GPT-2-medium decode step near the end: 4 wavefronts per row
+    (16, 16, 1024, 700, 200),   # ... and where the stand-alone attention has the same group shape
+    (16, 16, 1024, 200, 100),
+    (64, 16, 1024, 66, 63),     # Transformer-big beam step: one wavefront per row
+    (64, 16, 1024, 66, 0),
+    (5, 8, 512, 40, 17),        # rows not a multiple of the row group, head count a multiple of 8
+    (3, 2, 128, 300, 130),      # few heads, ragged row group
+    (9, 4, 256, 90, 64),
+])
+def test_qkv_product_cache_append_and_attention_in_one_launch(rng, M, heads, K, max_step, step):
+    """lsh_decself_qkv_attention_i8_f16 == lsh_gemm_i8_decself_qkv_i8o_f16 followed by
+    lsh_decself_attention_i8: q codes and caches byte for byte; context codes byte for byte
+    where the group shapes agree (more than 64 and at most 256 cached steps), else within one
+    code on at most 0.1 % (another summation tree)."""
+    from conftest import assert_codes_close
+    d, H = 64, heads * 64
+    assert K == H
+    x = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(3 * H, K), dtype=np.int8)
+    bias = (rng.standard_normal(3 * H) * 0.4).astype(np.float16)
+    alpha = 2.5 / (np.sqrt(K) * 127)
+    ds, qs = 3.0 / 127, 127 / 3.5
+    attn_scale, cache_dq, ctx_qs = 0.125, 3.5 / 127, 127 / 2.0
+    fill = rng.integers(-127, 128, size=(2, M, heads, max_step, d), dtype=np.int8)
+    k = _k()
+    xd, wd, bd = to_dev(x), to_dev(w), to_dev(bias)
+
+    q0 = torch.zeros((M, H), dtype=torch.int8, device=DEV)
+    kv0 = to_dev(fill.copy())
+    ctx0 = torch.zeros((M, H), dtype=torch.int8, device=DEV)
+    k.gemm_i8_decself_qkv_i8o(xd, wd, bd, q0, kv0[0], kv0[1], M, H, K, heads, max_step, step, alpha, ds, qs)
+    k.decself_attention_i8(q0, kv0[0], kv0[1], ctx0, M * heads, step + 1, max_step, heads, d, attn_scale,
+                           cache_dq, ctx_qs)
+
+    q1 = torch.full((M, H), 5, dtype=torch.int8, device=DEV)
+    kv1 = to_dev(fill.copy())
+    ctx1 = torch.full((M, H), 7, dtype=torch.int8, device=DEV)
+    k.decself_qkv_attention_i8(xd, wd, bd, q1, kv1[0], kv1[1], ctx1, M, H, heads, max_step, step, alpha, ds,
+                               qs, attn_scale, cache_dq, ctx_qs)
+    np.testing.assert_array_equal(to_np(q1), to_np(q0))
+    np.testing.assert_array_equal(to_np(kv1), to_np(kv0))
+    if 64 < step + 1 <= 256:
+        np.testing.assert_array_equal(to_np(ctx1), to_np(ctx0))
+    else:
+        assert_codes_close(to_np(ctx1), to_np(ctx0))
+
+
+def test_qkv_product_and_attention_in_one_launch_rejects_what_it_does_not_cover():
+    from lightseq_amd.lib import LSHError
+    k = _k()
+
+    def call(M, heads, d, max_step, step):
+        H = heads * d
+        z = lambda *s: torch.zeros(s, dtype=torch.int8, device=DEV)  # noqa: E731
+        k.decself_qkv_attention_i8(z(M, H), z(3 * H, H), torch.zeros(3 * H, dtype=torch.float16, device=DEV),
+                                   z(M, H), z(M, heads, max_step, d), z(M, heads, max_step, d), z(M, H), M, H,
+                                   heads, max_step, step, 1e-3, 1e-2, 30.0, 0.125, 1e-2, 30.0)
+
+    call(4, 2, 64, 8, 3)  # covered
+    for bad in [(4, 2, 32, 8, 3),      # heads of 32: hidden != heads * 64
+                (4, 3, 64, 8, 3),      # hidden 192 is not a multiple of 128
+                (4, 32, 64, 8, 3),     # hidden 2048
+                (4, 2, 64, 8, 8),      # step outside the cache
+                (4, 2, 64, 5000, 3)]:  # cache longer than 4096
+        with pytest.raises(LSHError):
+            call(*bad)
+

@@ -222,6 +222,41 @@ def test_fused_qkv_arrange_rejects_small_heads(rng):
         k.gemm_i8_qkv_arrange(a, w, out, bias, 64, 8, 8, 16, 8, 1, 1.0, 1.0)
 
 
+@pytest.mark.parametrize("M,N,K,ksplit", [(16, 3072, 1024, 1), (16, 1024, 4096, 8), (64, 1024, 4096, 4),
+                                          (64, 32000, 1024, 1), (16, 50257, 1024, 1), (1, 48, 256, 1),
+                                          (17, 1000, 768, 1), (33, 40, 512, 2), (48, 4096, 1024, 1),
+                                          (5, 8, 2048, 2), (64, 1024, 4096, 16)])
+def test_decode_step_kernels_give_the_same_bytes(rng, M, N, K, ksplit):
+    """Products of at most 64 rows: the 16 x 16 x 64 kernel and the 32 x 32 x 32 kernel agree bit
+    for bit -- int32 planes, requantised codes, the table epilogue -- and with the exact product."""
+    k = _k()
+    a = rng.integers(-127, 128, size=(M, K), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(N, K), dtype=np.int8)
+    ad, wd = to_dev(a), to_dev(w)
+    alpha = 3.0 / (np.sqrt(K) * 127)
+    lut = to_dev(rng.integers(-127, 128, size=(N, 256), dtype=np.int8))
+    outs = []
+    prev = k.gemm_i8_decode_kernel_16x16(True)
+    try:
+        for on in (True, False):
+            k.gemm_i8_decode_kernel_16x16(on)
+            planes = torch.full((ksplit, M, N), 7, dtype=torch.int32, device=DEV)
+            assert k.gemm_i8_i32o_splitk(ad, wd, planes, M, N, K, ksplit) == ksplit
+            c8 = torch.full((M, N), 9, dtype=torch.int8, device=DEV)
+            k.gemm_i8_i8o(ad, wd, c8, M, N, K, alpha)
+            cl = torch.full((M, N), 9, dtype=torch.int8, device=DEV)
+            k.gemm_i8_lut_i8o(ad, wd, cl, lut, M, N, K, alpha)
+            outs.append((planes, c8, cl))
+    finally:
+        k.gemm_i8_decode_kernel_16x16(prev)
+    for x, y in zip(*outs):
+        assert torch.equal(x, y)
+    np.testing.assert_array_equal(to_np(outs[0][0]).astype(np.int64).sum(0), _exact_i32(a, w))
+    # the table epilogue is the table entry of the requantised code
+    codes = to_np(outs[0][1]).astype(np.int64) + 128
+    np.testing.assert_array_equal(to_np(outs[0][2]), np.take_along_axis(to_np(lut).T, codes, axis=0))
+
+
 @pytest.mark.parametrize("M,N,K,ksplit", [(4096, 768, 3072, 2), (16, 1024, 4096, 8), (64, 1024, 4096, 4),
                                           (300, 256, 1024, 4), (33, 96, 256, 2)])
 def test_split_k_planes_sum_to_the_product(rng, M, N, K, ksplit):
