@@ -207,10 +207,11 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
                        const int8_t* __restrict__ v_cache, int8_t* __restrict__ new_v,
                        int step_num, int max_step, int head_num, float attn_scale, float dq,
                        float quant_scale) {
-  extern __shared__ float lds_f[];
-  const long bh = blockIdx.x;
-  const long row = bh / head_num;
-  const int head = (int)(bh % head_num);
+  extern __shared__ __align__(16) float lds_f[];
+  // grid: x = head, y = row (no division before the first load)
+  const int head = (int)blockIdx.x;
+  const long row = blockIdx.y;
+  const long bh = row * head_num + head;
   decself_attend_row<D, NWV, UN>(q + bh * D, k_cache + bh * (long)max_step * D,
                                  v_cache + bh * (long)max_step * D,
                                  new_v + row * ((long)head_num * D) + (long)head * D, true, step_num,
@@ -262,26 +263,29 @@ int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v
   if (int rc = decself_check(batch_head_num, step_num, max_step, head_num, dim_per_head)) return rc;
   const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_cache) |
                          reinterpret_cast<uintptr_t>(v_cache)) & 15u) == 0;
-  if (aligned && (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128)) {
+  if (aligned && batch_head_num % head_num == 0 && batch_head_num / head_num <= 65535 &&
+      (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128)) {
     // 8 wavefronts once the cache is long (width buys loads in flight), 4 below.  The
     // choice depends on the step count only, never on the number of rows: the two widths
     // sum the values in different trees, and a row's result must not depend on its batch.
     // The loads in flight per lane (UN) follow the cache length too: unrolled rounds that
     // a short cache never fills are code to fetch and clamped loads to wait for.
     const bool wide = step_num > 256;
-    const size_t lds =
-        ((size_t)((step_num + 63) & ~63) + 16 + (wide ? 8 : 4) * dim_per_head) * sizeof(float);
+    const dim3 grid(head_num, batch_head_num / head_num);
 #define LSH_DECSELF(D)                                                                          \
   if (wide)                                                                                     \
-    decself_attn_wg_kernel<D, 8, 8><<<batch_head_num, 512, lds, s>>>(                           \
+    decself_attn_wg_kernel<D, 8, 8>                                                             \
+        <<<grid, 512, decself_group_floats<D, 8>(step_num) * sizeof(float), s>>>(               \
         q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
         quant_scale);                                                                           \
   else if (step_num > 128 * 64 / D)                                                             \
-    decself_attn_wg_kernel<D, 4, 4><<<batch_head_num, 256, lds, s>>>(                           \
+    decself_attn_wg_kernel<D, 4, 4>                                                             \
+        <<<grid, 256, decself_group_floats<D, 4>(step_num) * sizeof(float), s>>>(               \
         q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
         quant_scale);                                                                           \
   else                                                                                          \
-    decself_attn_wg_kernel<D, 4, 2><<<batch_head_num, 256, lds, s>>>(                           \
+    decself_attn_wg_kernel<D, 4, 2>                                                             \
+        <<<grid, 256, decself_group_floats<D, 4>(step_num) * sizeof(float), s>>>(               \
         q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
         quant_scale)
     if (dim_per_head == 32) { LSH_DECSELF(32); }
