@@ -16,6 +16,8 @@
 
 #include <hip/hip_ext.h>
 
+#include <type_traits>
+
 namespace lsh {
 
 enum LnMode {
@@ -477,76 +479,94 @@ __global__ void ln_rows_generic_kernel(const AccT* __restrict__ gemm_out, T* res
 }
 
 // One row per workgroup, 4 consecutive elements per lane (hidden <= 4 * blockDim.x, hidden
-// % 4 == 0), reductions across the wavefronts through LDS, the accumulator planes summed in
-// a rolled loop.  The code is a fifth of the 8-wide kernel's: a kernel's instructions are
-// fetched cold on every launch (about 0.35 us per KB measured), which is what a launch
-// over a few rows costs most.
+// % 4 == 0): the layer norm of the decode steps, where a launch lasts a few microseconds and
+// every dependent step inside it shows.  So: no integer division and no branch before the loads
+// (indices are clamped, not predicated, which also lets the kernel arguments arrive in one
+// batch), every load -- parameters and up to eight accumulator planes -- requested before the
+// first is used, sums over a wavefront by DPP permutations and lane reads instead of LDS
+// permutes, and one barrier per reduction.
+// Order of a row sum: (x0 + x1) + (x2 + x3) per lane; lanes of a quad, the quads of a row of
+// 16 lanes and the four rows of a wavefront pairwise; the wavefronts in ascending order.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  auto add_dpp = [](float x, auto ctrl) {
+    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                              0xf, 0xf, false);
+    return x + __builtin_bit_cast(float, r);
+  };
+  v = add_dpp(v, std::integral_constant<int, 0xB1>());   // quad_perm [1,0,3,2]: lane ^ 1
+  v = add_dpp(v, std::integral_constant<int, 0x4E>());   // quad_perm [2,3,0,1]: lane ^ 2
+  v = add_dpp(v, std::integral_constant<int, 0x141>());  // row_half_mirror: the other quad of 8
+  v = add_dpp(v, std::integral_constant<int, 0x140>());  // row_mirror: the other half of 16
+  const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+  const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+  const float s2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+  const float s3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+  return (s0 + s1) + (s2 + s3);
+}
+
 template <typename T, typename AccT, int MODE>
-__global__ void __launch_bounds__(1024)
+__global__ void __launch_bounds__(256)
 ln_row_wg_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
                  int8_t* __restrict__ out_q, const T* __restrict__ scale,
                  const T* __restrict__ bias, const T* __restrict__ residual_bias,
                  const T* __restrict__ colsum, int hidden, float dequant_scale,
-                 float quant_scale, int is_post_ln, int nparts, long part_stride, int tokens,
-                 int tpr) {
-  // `tpr` threads (a multiple of 64) per row, blockDim.x / tpr rows per workgroup
-  __shared__ float red[2][16];
+                 float quant_scale, int is_post_ln, int nparts, long part_stride) {
+  __shared__ float red[2][4];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wpr = tpr >> 6;                  // wavefronts per row
-  const int rib = threadIdx.x / tpr;         // row within the workgroup
-  const int row = blockIdx.x * (blockDim.x / tpr) + rib;
-  const int e = (threadIdx.x - rib * tpr) * 4;
-  const bool on = e < hidden && row < tokens;
-  const long base = (long)(row < tokens ? row : 0) * hidden;
-  auto row_total = [&](float v, float* r) {  // sum over the row's wavefronts
-    v = wave_sum(v);
+  const int wpr = (int)blockDim.x >> 6;  // wavefronts of the row
+  const int e0 = (int)threadIdx.x * 4;
+  const bool on = e0 < hidden;
+  const int e = on ? e0 : 0;  // lanes past the row load its first elements and drop them
+  const long base = (long)blockIdx.x * hidden;
+  auto row_total = [&](float v, float* r) {
+    v = wave_sum_dpp(v);
     if (lane == 0) r[wid] = v;
     __syncthreads();
-    float t = 0.f;
-    for (int i = 0; i < wpr; ++i) t += r[rib * wpr + i];
+    float t = r[0];
+    for (int i = 1; i < wpr; ++i) t += r[i];
     return t;
   };
-  float x[4] = {0.f, 0.f, 0.f, 0.f}, g[4], b[4], rb[4] = {0.f, 0.f, 0.f, 0.f};
-  if (on) {
-    ld4(scale, e, g);
-    ld4(bias, e, b);
-    if (MODE != kLnResOut && residual_bias != nullptr) ld4(residual_bias, e, rb);
-    float r[4];
-    ld4(residual, base + e, r);
-    if (MODE == kLnFirst) {
+  float g[4], b[4], rb[4] = {0.f, 0.f, 0.f, 0.f}, r[4], c[4] = {0.f, 0.f, 0.f, 0.f};
+  ld4(residual, base + e, r);
+  float a[4] = {0.f, 0.f, 0.f, 0.f};
+  if (MODE != kLnFirst) {
+    if constexpr (sizeof(AccT) == 4) {
+      // up to eight planes in flight together (integer sums: any order gives the same bits); a
+      // plane index beyond the last is clamped for the load and its value dropped
+      int4 m[8];
 #pragma unroll
-      for (int k = 0; k < 4; ++k) x[k] = TT<T>::safe(r[k]);
-    } else {
-      float a[4];
-      if constexpr (sizeof(AccT) == 4) {
-        int4 acc = *reinterpret_cast<const int4*>(gemm_out + base + e);
-        // four planes per round trip (integer sums: any order gives the same bits); a plane
-        // index beyond the last is clamped for the load and its value dropped
-        for (int p = 1; p < nparts; p += 4) {
-          int4 m[4];
+      for (int u = 0; u < 8; ++u)
+        m[u] = *reinterpret_cast<const int4*>(gemm_out + (long)min(u, nparts - 1) * part_stride +
+                                              base + e);
+      int4 acc = m[0];
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
-            m[u] = *reinterpret_cast<const int4*>(
-                gemm_out + (long)min(p + u, nparts - 1) * part_stride + base + e);
-#pragma unroll
-          for (int u = 0; u < 4; ++u)
-            if (p + u < nparts) {
-              acc.x += m[u].x; acc.y += m[u].y; acc.z += m[u].z; acc.w += m[u].w;
-            }
+      for (int u = 1; u < 8; ++u)
+        if (u < nparts) {
+          acc.x += m[u].x; acc.y += m[u].y; acc.z += m[u].z; acc.w += m[u].w;
         }
-        a[0] = (float)acc.x; a[1] = (float)acc.y; a[2] = (float)acc.z; a[3] = (float)acc.w;
-      } else {
-        ld4_acc(gemm_out, base + e, a);
+      for (int p = 8; p < nparts; ++p) {
+        const int4 t = *reinterpret_cast<const int4*>(gemm_out + (long)p * part_stride + base + e);
+        acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
       }
-#pragma unroll
-      for (int k = 0; k < 4; ++k) x[k] = a[k] * dequant_scale + TT<T>::safe(r[k]);
-      if (colsum != nullptr) {
-        float c[4];
-        ld4(colsum, e, c);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) x[k] += TT<T>::safe(c[k]);
-      }
+      a[0] = (float)acc.x; a[1] = (float)acc.y; a[2] = (float)acc.z; a[3] = (float)acc.w;
+    } else {
+      ld4_acc(gemm_out, base + e, a);
     }
+  }
+  ld4(scale, e, g);
+  ld4(bias, e, b);
+  if (MODE != kLnResOut && residual_bias != nullptr) ld4(residual_bias, e, rb);
+  if (MODE != kLnFirst && colsum != nullptr) ld4(colsum, e, c);
+  float x[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (MODE == kLnFirst) {
+      x[k] = TT<T>::safe(r[k]);
+    } else {
+      x[k] = a[k] * dequant_scale + TT<T>::safe(r[k]);
+      if (colsum != nullptr) x[k] += TT<T>::safe(c[k]);
+    }
+    if (!on) x[k] = 0.f;
   }
   const float mean = row_total((x[0] + x[1]) + (x[2] + x[3]), red[0]) / (float)hidden;
   float var = 0.f;
@@ -592,7 +612,6 @@ bool ln_set_few_rows(bool on) {
   g_ln_few_rows = on;
   return prev;
 }
-constexpr int kLnRowsPerWg = 1;
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -609,11 +628,10 @@ static int launch_ln(const AccT* gemm_out, T* residual, T* out_t, int8_t* out_q,
                       aligned16(scale) && aligned16(bias) && aligned16(residual_bias) &&
                       aligned16(colsum);
   if (vec_ok && hidden <= 1024 && g_ln_few_rows) {
-    const int tpr = ((hidden / 4 + 63) / 64) * 64;
-    const int rpb = kLnRowsPerWg * tpr <= 1024 ? kLnRowsPerWg : 1;
-    ln_row_wg_kernel<T, AccT, MODE><<<(tokens + rpb - 1) / rpb, rpb * tpr, 0, stream>>>(
+    const int tpr = ((hidden / 4 + 63) / 64) * 64;  // threads of a row: whole wavefronts
+    ln_row_wg_kernel<T, AccT, MODE><<<tokens, tpr, 0, stream>>>(
         gemm_out, residual, out_t, out_q, scale, bias, residual_bias, colsum, hidden,
-        dequant_scale, quant_scale, is_post_ln, nparts, part_stride, tokens, tpr);
+        dequant_scale, quant_scale, is_post_ln, nparts, part_stride);
     return lsh_check_launch("ln_row_wg_kernel");
   }
   if (vec_ok && hidden % 8 == 0) {
