@@ -573,6 +573,122 @@ encdec_attn_vec_kernel(const __half* __restrict__ q, const __half* __restrict__ 
   }
 }
 
+// Short sources (at most 16 loads of a wavefront cover the keys): one wavefront per (sentence,
+// head, beam) as above, laid out for a generation step that lasts a few microseconds.  D / 8
+// adjacent lanes share a key or value row (16-byte loads, a load instruction of the wavefront
+// reads whole rows back to back), keys and values are requested together before anything is
+// used, scores and probabilities stay in the registers of the lanes that use them, the sums
+// over lanes are DPP permutations and lane reads, and only the D partial context sums of the
+// wavefront's four rows of 16 lanes meet in LDS.  The rounding points are those of the
+// kernels above (score, probability and context element rounded to fp16); the sums run in
+// another order.
+template <int D, int UN>
+__global__ void __launch_bounds__(256)
+encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
+                         const __half* __restrict__ v, const int* __restrict__ pad_mask,
+                         __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale,
+                         int beam_size, int head_num, int seq_len, float alpha_h) {
+#pragma clang fp contract(off)
+  constexpr int CH = D / 8;     // lanes per row
+  constexpr int KPW = 64 / CH;  // rows per load instruction of the wavefront
+  __shared__ float part_all[4][4][D];
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  // grid: x = head, y = sentence, z = groups of 4 beams; wavefront = beam
+  const int head = (int)blockIdx.x, beam = (int)blockIdx.z * 4 + wid;
+  const long b = blockIdx.y;
+  const bool alive = beam < beam_size;
+  const int bm = alive ? beam : beam_size - 1;
+  const long bh = b * head_num + head;
+  const long w = bh * beam_size + bm;
+  const int c = lane % CH, grp = lane / CH;
+  const int* mask = pad_mask + b * seq_len;
+  const __half* kb = k + bh * (long)seq_len * D + c * 8;
+  const __half* vb = v + bh * (long)seq_len * D + c * 8;
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  union Row {
+    uint4 u;
+    h2 p[4];
+    __half h[8];
+  };
+  Row qv, kv[UN], vv[UN];
+  int mk[UN];
+  qv.u = *reinterpret_cast<const uint4*>(q + w * D + c * 8);
+#pragma unroll
+  for (int u = 0; u < UN; ++u) {
+    const int j = min(u * KPW + grp, seq_len - 1);  // clamped, not predicated
+    kv[u].u = *reinterpret_cast<const uint4*>(kb + (long)j * D);
+    mk[u] = mask[j];
+  }
+#pragma unroll
+  for (int u = 0; u < UN; ++u) {
+    const int j = min(u * KPW + grp, seq_len - 1);
+    vv[u].u = *reinterpret_cast<const uint4*>(vb + (long)j * D);
+  }
+  float val[UN];
+  float mx = kFloatInfNeg;
+#pragma unroll
+  for (int u = 0; u < UN; ++u) {
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_fdot2(qv.p[e], kv[u].p[e], acc, false);
+    // the CH partial dot products of the row
+    acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0xB1, 0xf, 0xf, false));
+    acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x4E, 0xf, 0xf, false));
+    if (CH >= 8)
+      acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x141, 0xf, 0xf, false));
+    if (CH >= 16)
+      acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x140, 0xf, 0xf, false));
+    const bool valid = u * KPW + grp < seq_len && !mk[u];
+    val[u] = TT<__half>::rnd(alpha_h * acc);
+    if (valid) mx = fmaxf(mx, val[u]);
+    else val[u] = kFloatInfNeg;
+  }
+  mx = row_ror_max<8>(row_ror_max<4>(row_ror_max<2>(row_ror_max<1>(mx))));
+  mx = fmaxf(fmaxf(lane_of(mx, 0), lane_of(mx, 16)), fmaxf(lane_of(mx, 32), lane_of(mx, 48)));
+  float sum = 0.f;
+#pragma unroll
+  for (int u = 0; u < UN; ++u) {
+    val[u] = val[u] > kFloatInfNeg ? __expf(val[u] - mx) : 0.f;
+    sum += val[u];
+  }
+  // every row once: lanes of one c, rotations by multiples of CH within a row of 16 lanes
+  if (CH <= 4) sum = row_ror_add<4>(sum);
+  if (CH <= 8) sum = row_ror_add<8>(sum);
+  sum = (lane_of(sum, 0) + lane_of(sum, 16)) + (lane_of(sum, 32) + lane_of(sum, 48));
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+  for (int u = 0; u < UN; ++u) {
+    const float p = TT<__half>::rnd(val[u] / sum);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(p, __half2float(vv[u].h[e]), acc[e]);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    if (CH <= 4) acc[e] = row_ror_add<4>(acc[e]);
+    if (CH <= 8) acc[e] = row_ror_add<8>(acc[e]);
+  }
+  float* part = &part_all[wid][0][0];
+  if ((lane & 15) < CH) {
+    float* pp = part + (lane >> 4) * D + c * 8;
+    *reinterpret_cast<float4*>(pp) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    *reinterpret_cast<float4*>(pp + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (!alive) return;
+  const long row = b * beam_size + beam;
+  for (int dd = lane; dd < D; dd += 64) {
+    const float t = (part[dd] + part[D + dd]) + (part[2 * D + dd] + part[3 * D + dd]);
+    const float cv = TT<__half>::rnd(t);
+    if (ctx) ctx[w * D + dd] = __float2half_rn(cv);
+    if (ctx_q)
+      ctx_q[row * ((long)head_num * D) + (long)head * D + dd] = (int8_t)float2int8(cv, quant_scale);
+  }
+}
+
 int encdec_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,
                          __half* ctx, int8_t* ctx_q, float quant_scale, int batch_size,
                          int beam_size, int head_num, int batch_seq_len, int dim_per_head,
@@ -587,6 +703,28 @@ int encdec_attention_f16(const __half* q, const __half* k, const __half* v, cons
   const size_t lds = (size_t)4 * ((batch_seq_len + 63) & ~63) * sizeof(float);
   const bool aligned = ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
                          reinterpret_cast<uintptr_t>(v)) & 15u) == 0;
+  if (aligned && batch_size <= 65535 && beam_size <= 4 * 65535 &&
+      (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128) &&
+      batch_seq_len <= 16 * (512 / dim_per_head)) {
+    // short sources: keys, values and probabilities in registers.  The choice follows the
+    // source length and the head size only, never the number of rows.
+    const dim3 grid(head_num, batch_size, (beam_size + 3) / 4);
+    const int kpw = 512 / dim_per_head;  // rows per load instruction of a wavefront
+    const int un = (batch_seq_len + kpw - 1) / kpw;
+#define LSH_ENCDEC_SHORT(D, UN)                                                                   \
+  encdec_attn_short_kernel<D, UN><<<grid, 256, 0, s>>>(q, k, v, pad_mask, ctx, ctx_q, quant_scale, \
+                                                       beam_size, head_num, batch_seq_len, alpha_h)
+#define LSH_ENCDEC_SHORT_D(D)                \
+  if (un <= 4) LSH_ENCDEC_SHORT(D, 4);       \
+  else if (un <= 8) LSH_ENCDEC_SHORT(D, 8);  \
+  else LSH_ENCDEC_SHORT(D, 16)
+    if (dim_per_head == 32) { LSH_ENCDEC_SHORT_D(32); }
+    else if (dim_per_head == 64) { LSH_ENCDEC_SHORT_D(64); }
+    else { LSH_ENCDEC_SHORT_D(128); }
+#undef LSH_ENCDEC_SHORT_D
+#undef LSH_ENCDEC_SHORT
+    return lsh_check_launch("encdec_attn_short_kernel");
+  }
   if (aligned && (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128)) {
 #define LSH_ENCDEC(D)                                                                           \
   encdec_attn_vec_kernel<D><<<(int)((waves + 3) / 4), 256, lds, s>>>(                           \
