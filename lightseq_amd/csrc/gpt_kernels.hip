@@ -8,6 +8,8 @@
 #include "ls_device.cuh"
 #include "ls_launch.h"
 
+#include <type_traits>
+
 namespace lsh {
 
 constexpr float kLogitThreshMin = -64.f;  // inference/kernels/transformerKernels.h:11
@@ -36,6 +38,38 @@ gpt_embedding_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__
   }
 }
 
+// The same for one position per sequence (a generation step): a workgroup per sequence, four
+// elements per lane, no division; it also counts the token into real_seq_len (what
+// gpt_count_tokens_kernel does in a launch of its own) and clears `zero_flag` when given, so a
+// step spends one launch here instead of three.  Same arithmetic, same bits.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gpt_embedding_step_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__ pos_emb,
+                          const int* __restrict__ token_id, T* __restrict__ output,
+                          int* real_seq_len, int* zero_flag, int padding_id, int pos,
+                          float dequant_scale, int hidden, int vocab) {
+#pragma clang fp contract(off)
+  const int b = blockIdx.x;
+  int tid = token_id[b];
+  const bool pad = tid == padding_id;
+  if (vocab > 0) tid = min(max(tid, 0), vocab - 1);  // never index outside the table
+  if (threadIdx.x == 0) {
+    if (!pad) real_seq_len[b] += 1;
+    if (zero_flag != nullptr && b == 0) zero_flag[0] = 0;
+  }
+  for (int i = threadIdx.x * 4; i < hidden; i += blockDim.x * 4) {
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
+    if (!pad) {
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(token_emb + (long)tid * hidden + i);
+      float p[4];
+      ld4(pos_emb, (long)pos * hidden + i, p);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = (float)unpack_i8(w, k) * dequant_scale + p[k];
+    }
+    st4(output, (long)b * hidden + i, o);
+  }
+}
+
 // real_seq_len[b] += non-padding tokens of row b (the reference counts with atomics)
 __global__ void __launch_bounds__(256)
 gpt_count_tokens_kernel(const int* __restrict__ token_id, int* real_seq_len, int padding_id,
@@ -53,12 +87,22 @@ template <typename T>
 int gpt_embedding_i8I(int batch_size, int batch_seq_len, int hidden_size, hipStream_t s,
                       const int8_t* token_emb, const T* pos_emb, const int* token_id, T* output,
                       int* real_seq_len, int padding_id, int pos_offset, float dequant_scale,
-                      int vocab_size, int max_step) {
+                      int vocab_size, int max_step, int* zero_flag) {
   if (!token_emb || !pos_emb || !token_id || !output || !real_seq_len || batch_size <= 0 ||
       batch_seq_len <= 0 || hidden_size <= 0)
     return lsh_fail(LSH_ERR_INVALID, "ker_gpt_embedding_i8I: bad arguments");
   if (pos_offset < 0 || (max_step > 0 && pos_offset + batch_seq_len > max_step))
     return lsh_fail(LSH_ERR_INVALID, "ker_gpt_embedding_i8I: position outside the table");
+  const bool aligned = ((reinterpret_cast<uintptr_t>(token_emb) | reinterpret_cast<uintptr_t>(pos_emb) |
+                         reinterpret_cast<uintptr_t>(output)) & 15u) == 0;
+  if (batch_seq_len == 1 && hidden_size % 4 == 0 && aligned) {
+    gpt_embedding_step_kernel<T><<<batch_size, 256, 0, s>>>(
+        token_emb, pos_emb, token_id, output, real_seq_len, zero_flag, padding_id, pos_offset,
+        dequant_scale, hidden_size, vocab_size);
+    return lsh_check_launch("gpt_embedding_step_kernel");
+  }
+  if (zero_flag != nullptr)
+    if (int rc = fill_i32(zero_flag, 0, 1, s)) return rc;
   gpt_embedding_kernel<T><<<batch_size * batch_seq_len, 256, 0, s>>>(
       token_emb, pos_emb, token_id, output, padding_id, pos_offset, dequant_scale, batch_seq_len,
       hidden_size, vocab_size);
@@ -68,9 +112,9 @@ int gpt_embedding_i8I(int batch_size, int batch_seq_len, int hidden_size, hipStr
   return lsh_check_launch("gpt_count_tokens_kernel");
 }
 template int gpt_embedding_i8I<float>(int, int, int, hipStream_t, const int8_t*, const float*,
-                                      const int*, float*, int*, int, int, float, int, int);
+                                      const int*, float*, int*, int, int, float, int, int, int*);
 template int gpt_embedding_i8I<__half>(int, int, int, hipStream_t, const int8_t*, const __half*,
-                                       const int*, __half*, int*, int, int, float, int, int);
+                                       const int*, __half*, int*, int, int, float, int, int, int*);
 
 // ---------------------------------------------------------------------------------
 // prompt pass: int8 QKV GEMM output [tokens, 3H] + bias -> requantised with the cache
@@ -275,39 +319,63 @@ template int arrange_qkv_with_cache_i8I_i8O<__half>(int, int, hipStream_t, const
 // arg-max runs on the int8 codes; ties go to the lowest token id (the reference lets
 // racing stores decide).
 // ---------------------------------------------------------------------------------
+// First maximum of a row of int8 logits (lowest id on ties), the same in every thread.  The row
+// is read in 16-byte pieces aligned to 16 bytes in memory (rows of an odd vocabulary start
+// anywhere), every piece of a thread requested before the first is scanned; a candidate is
+// the key (code + 128) << 20 | (2^20 - 1 - id), so the arg-max is one integer maximum: over a
+// wavefront by DPP permutations and lane reads, over the workgroup through LDS with one
+// barrier.  vocab <= 2^20.
 __device__ __forceinline__ int block_argmax_i8(const int8_t* __restrict__ lr, int vocab,
                                                int* red /*[32]*/) {
-  int best_c = -129, best_i = 0x7fffffff;
-  for (int v = threadIdx.x; v < vocab; v += blockDim.x) {
-    const int c = lr[v];
-    if (c > best_c) {  // ascending v per thread: the first maximum is kept
-      best_c = c;
-      best_i = v;
-    }
-  }
+  constexpr int kIdBits = 20, kIdMask = (1 << kIdBits) - 1;
+  const int a = (int)(reinterpret_cast<uintptr_t>(lr) & 15u);  // bytes of the first piece before the row
+  const int8_t* base = lr - a;
+  const int pieces = (vocab + a + 15) >> 4;
+  int key = 0;  // below every real key (code + 128 >= 1)
+  for (int p0 = 0; p0 < pieces; p0 += 4 * (int)blockDim.x) {
+    uint4 w[4];
 #pragma unroll
-  for (int m = 32; m > 0; m >>= 1) {
-    const int oc = __shfl_xor(best_c, m, 64), oi = __shfl_xor(best_i, m, 64);
-    if (oc > best_c || (oc == best_c && oi < best_i)) {
-      best_c = oc;
-      best_i = oi;
+    for (int u = 0; u < 4; ++u) {
+      // pieces past the row are clamped to the last one that lies inside it; a piece that
+      // straddles an end of the row is read byte by byte below
+      const int p = min(p0 + u * (int)blockDim.x + (int)threadIdx.x, pieces - 1);
+      const bool inside = p * 16 >= a && p * 16 + 16 <= vocab + a;
+      w[u] = inside ? *reinterpret_cast<const uint4*>(base + (long)p * 16) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int p = p0 + u * (int)blockDim.x + (int)threadIdx.x;
+      if (p < pieces) {
+        const int v0 = p * 16 - a;  // id of the piece's first byte
+        const bool inside = v0 >= 0 && v0 + 16 <= vocab;
+        const uint32_t ws[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int v = v0 + e;
+          int c;
+          if (inside) c = unpack_i8(ws[e >> 2], e & 3);
+          else if (v >= 0 && v < vocab) c = lr[v];
+          else continue;
+          key = max(key, ((c + 128) << kIdBits) | (kIdMask - v));
+        }
+      }
     }
   }
+  auto max_dpp = [](int x, auto ctrl) {
+    return max(x, __builtin_amdgcn_update_dpp(0, x, decltype(ctrl)::value, 0xf, 0xf, false));
+  };
+  key = max_dpp(key, std::integral_constant<int, 0xB1>());   // lane ^ 1
+  key = max_dpp(key, std::integral_constant<int, 0x4E>());   // lane ^ 2
+  key = max_dpp(key, std::integral_constant<int, 0x141>());  // the other quad of 8
+  key = max_dpp(key, std::integral_constant<int, 0x140>());  // the other half of 16
+  key = max(max(__builtin_amdgcn_readlane(key, 0), __builtin_amdgcn_readlane(key, 16)),
+            max(__builtin_amdgcn_readlane(key, 32), __builtin_amdgcn_readlane(key, 48)));
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  if (lane == 0) red[wid] = key;
   __syncthreads();
-  if (lane == 0) {
-    red[wid] = best_c;
-    red[16 + wid] = best_i;
-  }
-  __syncthreads();
-  best_c = red[0];
-  best_i = red[16];
-  for (int w2 = 1; w2 < nw; ++w2)
-    if (red[w2] > best_c || (red[w2] == best_c && red[16 + w2] < best_i)) {
-      best_c = red[w2];
-      best_i = red[16 + w2];
-    }
-  return best_i;
+  key = red[0];
+  for (int w2 = 1; w2 < nw; ++w2) key = max(key, red[w2]);
+  return kIdMask - (key & kIdMask);
 }
 
 // ker_topk_sample_i8I<1> (inference/kernels/gptKernels_int8.cc.cu:252-463): ids re-laid
@@ -353,6 +421,8 @@ int topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len, hipSt
                       "needs the reference's generator state");
     return lsh_fail(LSH_ERR_INVALID, "topk argument should be in [1,2,4,8,16,32]");
   }
+  if (vocab_size > (1 << 20))
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "ker_topk_sample_i8I: vocabulary above 2^20 ids");
   topk_sample_greedy_kernel<<<batch_size, 1024, 0, s>>>(logits, old_input_ids, new_input_ids,
                                                         vocab_size, batch_seq_len, logits_seq_len,
                                                         unfinished, eos_id);
@@ -384,6 +454,8 @@ int gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_siz
   if (!logits || !ids || !last_ids || !unfinished || batch_size <= 0 || vocab_size <= 0 ||
       cur_len <= 0 || cur_len >= max_step)
     return lsh_fail(LSH_ERR_INVALID, "gpt_greedy_step: bad arguments");
+  if (vocab_size > (1 << 20))
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "gpt_greedy_step: vocabulary above 2^20 ids");
   gpt_greedy_step_kernel<<<batch_size, 1024, 0, s>>>(logits, ids, last_ids, vocab_size, max_step,
                                                      cur_len, unfinished, eos_id);
   return lsh_check_launch("gpt_greedy_step_kernel");

@@ -311,7 +311,9 @@ template <typename T>
 int gpt_embedding_i8I(int batch_size, int batch_seq_len, int hidden_size, hipStream_t s,
                       const int8_t* token_emb, const T* pos_emb, const int* token_id, T* output,
                       int* real_seq_len, int padding_id, int pos_offset, float dequant_scale,
-                      int vocab_size, int max_step);
+                      int vocab_size, int max_step, int* zero_flag = nullptr);
+// zero_flag: when given, the int it points to is cleared by the same launch (a generation
+// step's "unfinished" flag)
 int gpt_arrange_qkv_prefill_f16(int batch_token_num, int hidden_size, hipStream_t s,
                                 const int8_t* ori_qkv, const __half* qkv_bias, __half* q_codes,
                                 __half* k_codes, __half* v_deq, int8_t* k_cache, int8_t* v_cache,

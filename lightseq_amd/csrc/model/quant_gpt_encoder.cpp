@@ -205,7 +205,7 @@ const int8_t* QuantGptEncoder::step_pass() {
   LSH_CALL(gpt_embedding_i8I<__half>(B, 1, H, _stream, _int8_emb.get(), _pos_emb.get(),
                                      _last_ids.get(), _query.get(), _real_seq_len.get(),
                                      _tw._padding_id, _batch_seq_len - 1, _src_emb_clip_max / Q,
-                                     _tw._src_vocab_size, _tw._max_step));
+                                     _tw._src_vocab_size, _tw._max_step, _unfinished.get()));
   int8_t *a = _buf_a.get(), *b = _buf_b.get();
   _tap_step = _steps_run;
   const size_t bh = (size_t)B * H;
@@ -268,7 +268,7 @@ const int8_t* QuantGptEncoder::step_pass() {
 #undef TAP
 
 // logits of the last position + greedy choice, enqueued only (:399-487)
-void QuantGptEncoder::enqueue_sampling(const int8_t* hidden) {
+void QuantGptEncoder::enqueue_sampling(const int8_t* hidden, bool clear_flag) {
   const int H = _tw._hidden_size, V = _tw._src_vocab_size, B = _batch_size;
   LSH_CALL(gemm_i8_i8o(hidden, _int8_emb.get(), _logits.get(), B, V, H,
                        _output_ln_clip_max * _src_emb_clip_max / (_logits_clip_max * _quant_range),
@@ -276,7 +276,8 @@ void QuantGptEncoder::enqueue_sampling(const int8_t* hidden) {
   if (_rec_logits && _steps_run < _rec_max_steps)
     CHECK_GPU_ERROR(hipMemcpyAsync(_rec_logits + (size_t)_steps_run * B * V, _logits.get(),
                                    (size_t)B * V, hipMemcpyDeviceToDevice, _stream));
-  LSH_CALL(fill_i32(_unfinished.get(), 0, 1, _stream));
+  // (after a cached step the flag was cleared by the step's embedding launch)
+  if (clear_flag) LSH_CALL(fill_i32(_unfinished.get(), 0, 1, _stream));
   LSH_CALL(gpt_greedy_step(_logits.get(), _ids.get(), _last_ids.get(), V, _tw._max_step,
                            _batch_seq_len, B, _unfinished.get(), _tw._eos_id, _stream));
 }
@@ -322,13 +323,13 @@ int QuantGptEncoder::run_one_sample(int batch_size, int batch_seq_len) {
                                    hipMemcpyDeviceToDevice, _stream));
   if (_batch_seq_len < _tw._max_step) {
     // (:347-353) after the prompt pass the run ends when nothing is unfinished
-    enqueue_sampling(_hid_last.get());
+    enqueue_sampling(_hid_last.get(), true);
     if (!(finish_token() == 0 || _batch_seq_len >= _batch_max_seq_len)) {
       while (_batch_seq_len < _batch_max_seq_len) {
         // the launches of a step depend on the batch size and the position only
         const uint64_t key = ((uint64_t)_batch_size << 32) | (uint32_t)_batch_seq_len;
         _graphs.run(key, _stream, _use_graphs && !_rec_logits && !step_taps.any(),
-                    [&] { enqueue_sampling(step_pass()); });
+                    [&] { enqueue_sampling(step_pass(), false); });
         int unfinished = finish_token();
         if (!unfinished && !_is_benchmark) break;
       }

@@ -57,7 +57,7 @@ class QuantGptEncoder {
   void prompt_pass(const int* ids);
   const int8_t* step_pass();
   void ffn_add_norm(int rows, int8_t* in, int8_t* tmp);
-  void enqueue_sampling(const int8_t* hidden);
+  void enqueue_sampling(const int8_t* hidden, bool clear_flag);
   int finish_token();
 
   const int _max_batch_size;
