@@ -13,6 +13,8 @@
 //    threshold never cuts into a row's best `beam_size`), without a global sort, a
 //    prefix scan or a device-to-host round trip.  Ties go to the lower candidate id.
 #include "ls_device.cuh"
+
+#include <type_traits>
 #include "ls_launch.h"
 
 #include <mutex>
@@ -582,8 +584,8 @@ beam_topk_reg_kernel(const int8_t* __restrict__ logits, const T* __restrict__ lo
                      int cur_step, int beam_size, int end_id) {
 #pragma clang fp contract(off)
   constexpr int NI = 32;
-  __shared__ float red[32];
-  __shared__ ScoreIdx wbest[16];
+  __shared__ float red_max[16], red_sum[16];
+  __shared__ unsigned long long wbest[2][16];  // per-wavefront best key, double-buffered by round
   const int row = blockIdx.x, t = threadIdx.x;
   const int lane = t & 63, wid = t >> 6;
   const int batch_id = row / beam_size, beam_id = row % beam_size;
@@ -630,49 +632,70 @@ beam_topk_reg_kernel(const int8_t* __restrict__ logits, const T* __restrict__ lo
 #pragma unroll
   for (int i = 0; i < NI; ++i)
     if (id_of(i) < vocab) tmax = fmaxf(tmax, lg[i]);
-  const float max_logit = block_max(tmax, red);
+  const float max_logit = block_max_dpp(tmax, red_max);
   float se = 0.f;
 #pragma unroll
   for (int i = 0; i < NI; ++i)
     if (id_of(i) < vocab) se += __expf(fmaxf(lg[i] - max_logit, kLogitThreshMin));
-  const float sum_exp = block_sum(se, red);
+  const float sum_exp = block_sum_dpp(se, red_sum);
   const float base = seq_probs[row] - logf(sum_exp) - max_logit;
 #pragma unroll
   for (int i = 0; i < NI; ++i) lg[i] = cand_score(lg[i], base, length_norm, batch_id);
-  // A thread keeps the first of its own candidates that comes after the last pick; a round
-  // is a block-wide arg-max over these, and only the thread that owned the pick looks
-  // through its registers again (every other thread's candidate still comes after it).
-  auto my_first_after = [&](const ScoreIdx& prev) {
-    ScoreIdx best;
-    best.s = -INFINITY;
-    best.i = kNoCand;
+  // A candidate is one 64-bit key: the score as an order-preserving integer above
+  // 2^31 - 1 - id, so "higher score first, lower id on ties" is an integer maximum.  A thread
+  // keeps the largest of its own keys that is below the last pick; a round is a block-wide
+  // maximum over these -- DPP permutations and lane reads inside a wavefront, one barrier
+  // and 16 LDS reads across the workgroup -- and only the thread that owned the pick looks
+  // through its registers again (every other thread's key is still below it).
+  auto key_of = [&](int i) -> unsigned long long {
+    const int id = id_of(i);
+    if (id >= vocab) return 0ull;
+    unsigned u = __builtin_bit_cast(unsigned, lg[i] + 0.f);  // -0 -> +0
+    u ^= (u >> 31) ? 0xffffffffu : 0x80000000u;
+    return ((unsigned long long)u << 32) | (unsigned)(0x7fffffff - id);
+  };
+  auto my_best_below = [&](unsigned long long bound) {
+    unsigned long long best = 0ull;
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
-      ScoreIdx c;
-      c.s = lg[i];
-      c.i = id_of(i);
-      if (c.i < vocab && before(prev, c) && before(c, best)) best = c;
+      const unsigned long long c = key_of(i);
+      if (c < bound && c > best) best = c;
     }
     return best;
   };
-  ScoreIdx prev;
-  prev.s = INFINITY;
-  prev.i = -1;
-  ScoreIdx mine = my_first_after(prev);
+  auto umax64 = [](unsigned long long a, unsigned long long b) { return a > b ? a : b; };
+  auto dpp64 = [](unsigned long long x, auto ctrl) {
+    const unsigned lo = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)x, decltype(ctrl)::value, 0xf, 0xf, false);
+    const unsigned hi = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)(x >> 32), decltype(ctrl)::value, 0xf, 0xf, false);
+    return ((unsigned long long)hi << 32) | lo;
+  };
+  auto lane64 = [](unsigned long long x, int l) {
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)x, l);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(x >> 32), l);
+    return ((unsigned long long)hi << 32) | lo;
+  };
+  unsigned long long mine = my_best_below(~0ull);
   for (int k = 0; k < beam_size; ++k) {
-    ScoreIdx best = wave_first(mine);
+    unsigned long long best = mine;
+    best = umax64(best, dpp64(best, std::integral_constant<int, kDppXor1>()));
+    best = umax64(best, dpp64(best, std::integral_constant<int, kDppXor2>()));
+    best = umax64(best, dpp64(best, std::integral_constant<int, kDppHalfMirror>()));
+    best = umax64(best, dpp64(best, std::integral_constant<int, kDppMirror>()));
+    best = umax64(umax64(lane64(best, 0), lane64(best, 16)), umax64(lane64(best, 32), lane64(best, 48)));
+    unsigned long long* wb = wbest[k & 1];
+    if (lane == 0) wb[wid] = best;
     __syncthreads();
-    if (lane == 0) wbest[wid] = best;
-    __syncthreads();
-    best = wbest[0];
-    for (int w2 = 1; w2 < 16; ++w2)
-      if (before(wbest[w2], best)) best = wbest[w2];
+    best = wb[0];
+#pragma unroll
+    for (int w2 = 1; w2 < 16; ++w2) best = umax64(best, wb[w2]);
     if (t == 0) {
-      os[k] = best.i == kNoCand ? -INFINITY : best.s;
-      oi[k] = best.i == kNoCand ? kNoCand : beam_id * vocab + best.i;
+      // key 0: no candidate left
+      unsigned u = (unsigned)(best >> 32);
+      u ^= (u >> 31) ? 0x80000000u : 0xffffffffu;
+      os[k] = best == 0ull ? -INFINITY : __builtin_bit_cast(float, u);
+      oi[k] = best == 0ull ? kNoCand : beam_id * vocab + (0x7fffffff - (int)(unsigned)best);
     }
-    prev = best;
-    if (best.i == mine.i && best.i != kNoCand) mine = my_first_after(prev);
+    if (best == mine && best != 0ull) mine = my_best_below(best);
   }
 }
 

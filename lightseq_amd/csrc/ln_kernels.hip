@@ -487,23 +487,6 @@ __global__ void ln_rows_generic_kernel(const AccT* __restrict__ gemm_out, T* res
 // permutes, and one barrier per reduction.
 // Order of a row sum: (x0 + x1) + (x2 + x3) per lane; lanes of a quad, the quads of a row of
 // 16 lanes and the four rows of a wavefront pairwise; the wavefronts in ascending order.
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-  auto add_dpp = [](float x, auto ctrl) {
-    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
-                                              0xf, 0xf, false);
-    return x + __builtin_bit_cast(float, r);
-  };
-  v = add_dpp(v, std::integral_constant<int, 0xB1>());   // quad_perm [1,0,3,2]: lane ^ 1
-  v = add_dpp(v, std::integral_constant<int, 0x4E>());   // quad_perm [2,3,0,1]: lane ^ 2
-  v = add_dpp(v, std::integral_constant<int, 0x141>());  // row_half_mirror: the other quad of 8
-  v = add_dpp(v, std::integral_constant<int, 0x140>());  // row_mirror: the other half of 16
-  const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
-  const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
-  const float s2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
-  const float s3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
-  return (s0 + s1) + (s2 + s3);
-}
-
 template <typename T, typename AccT, int MODE>
 __global__ void __launch_bounds__(256)
 ln_row_wg_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,

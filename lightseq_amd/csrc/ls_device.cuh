@@ -176,6 +176,56 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The same over DPP permutations and lane reads: no LDS permute instructions and a much
+// shorter dependent chain (quad, 8 lanes, 16 lanes, then the four rows of the wavefront
+// pairwise).  Another order of additions than wave_sum; every lane gets the result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane l of a row of 16 reads lane 7 - l of its half
+constexpr int kDppMirror = 0x140;      // ... lane 15 - l of its row
+__device__ __forceinline__ float lane_read(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v += dpp_f<kDppXor1>(v);
+  v += dpp_f<kDppXor2>(v);
+  v += dpp_f<kDppHalfMirror>(v);
+  v += dpp_f<kDppMirror>(v);
+  return (lane_read(v, 0) + lane_read(v, 16)) + (lane_read(v, 32) + lane_read(v, 48));
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+  v = fmaxf(v, dpp_f<kDppXor1>(v));
+  v = fmaxf(v, dpp_f<kDppXor2>(v));
+  v = fmaxf(v, dpp_f<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_f<kDppMirror>(v));
+  return fmaxf(fmaxf(lane_read(v, 0), lane_read(v, 16)), fmaxf(lane_read(v, 32), lane_read(v, 48)));
+}
+// Block-wide forms with one barrier: `red` (16 floats of LDS) must not be in use by an
+// earlier reduction that other wavefronts may still be reading (give each call its own).
+__device__ __forceinline__ float block_sum_dpp(float v, float* red) {
+  v = wave_sum_dpp(v);
+  const int nw = (blockDim.x + kWave - 1) >> 6;
+  if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = red[0];
+  for (int i = 1; i < nw; ++i) r += red[i];
+  return r;
+}
+__device__ __forceinline__ float block_max_dpp(float v, float* red) {
+  v = wave_max_dpp(v);
+  const int nw = (blockDim.x + kWave - 1) >> 6;
+  if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = red[0];
+  for (int i = 1; i < nw; ++i) r = fmaxf(r, red[i]);
+  return r;
+}
+
 // Block-wide reductions for blocks of up to 1024 threads (16 wavefronts).
 // `red` must point to at least 16 floats of LDS.  All threads get the result.
 __device__ __forceinline__ float block_sum(float v, float* red) {
