@@ -792,6 +792,10 @@ gemm_i8_tile_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, 
   static_assert((NST - 1) * PER < 64, "vmcnt range");
   static_assert(!LUT || (TM >= TN && TN % (4 * NWV) == 0), "table fits a freed stage");
   extern __shared__ __align__(16) int8_t smem[];
+  // the operand pointers are wanted in registers here, so that their kernel-argument load
+  // leaves with the one for the shape instead of after the tile arithmetic that needs the shape
+  // (the tile arithmetic below is made to wait for them)
+  asm volatile("" : "+s"(tiles_m) : "s"(A), "s"(W));
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WGN, wn = wave % WGN, l32 = lane & 31, g = lane >> 5;
   int tm, tn;
@@ -1181,6 +1185,7 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
   __shared__ int red[4][MB][2][4][64];  // [wavefront][row block][column block][register][lane]
   constexpr bool kLut = std::is_same<Epi, EpiLutI8>::value;
   __shared__ __align__(16) int8_t tab[kLut ? 32 * 256 : 16];  // table rows of the 32 columns
+  asm volatile("" ::"s"(A), "s"(W));  // one batch of kernel-argument loads, not two in a row
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kq = lane >> 4;
   // grid: x = column block, y = K range (plane of the output); kw = bytes of K per wavefront,
