@@ -74,11 +74,16 @@ def test_qkv_product_with_cache_append_rejects_bad_arguments(rng):
 
 
 @pytest.mark.parametrize("B,beam,heads,S,d", [(3, 4, 2, 37, 64), (2, 2, 3, 64, 32), (1, 4, 2, 130, 128),
-                                              (16, 4, 16, 64, 64)])
+                                              (16, 4, 16, 64, 64), (2, 2, 2, 200, 64), (2, 3, 2, 300, 32),
+                                              (1, 5, 2, 60, 128), (2, 1, 4, 128, 64)])
 def test_cross_attention_vector_kernel_equals_the_scalar_one(rng, B, beam, heads, S, d):
     """lsh_encdec_attention_f16 picks a vector-load kernel for 16-byte aligned operands and
-    head sizes 32 / 64 / 128; it sums in the same order as the general kernel, so a query
-    buffer shifted by 8 bytes (general kernel) gives the same context bits and codes."""
+    head sizes 32 / 64 / 128; for sources longer than 16 loads of a wavefront cover (8192 / d
+    keys) it sums in the same order as the general kernel, so a query buffer shifted by 8 bytes
+    (general kernel) gives the same context bits and codes.  Shorter sources run the kernel that
+    keeps keys, values and probabilities in registers and sums in another order: the same fp16
+    rounding points, context within one fp16 step of the magnitudes involved and codes within
+    +-1 on at most 0.5 % of the elements."""
     q = (rng.standard_normal((B, heads, beam, d)) * 0.7).astype(np.float16)
     k = (rng.standard_normal((B, heads, S, d)) * 0.7).astype(np.float16)
     v = (rng.standard_normal((B, heads, S, d)) * 0.7).astype(np.float16)
@@ -95,8 +100,14 @@ def test_cross_attention_vector_kernel_equals_the_scalar_one(rng, B, beam, heads
         ctx_q = torch.zeros((B * beam, heads * d), dtype=torch.int8, device=DEV)
         _k().encdec_attention(qd, to_dev(k), to_dev(v), to_dev(mask), ctx, ctx_q, qs, B, beam, heads, S, d)
         outs.append((to_np(ctx), to_np(ctx_q)))
-    np.testing.assert_array_equal(outs[0][0].view(np.uint16), outs[1][0].view(np.uint16))
-    np.testing.assert_array_equal(outs[0][1], outs[1][1])
+    if S > 16 * (512 // d):
+        np.testing.assert_array_equal(outs[0][0].view(np.uint16), outs[1][0].view(np.uint16))
+        np.testing.assert_array_equal(outs[0][1], outs[1][1])
+    else:
+        from conftest import assert_codes_close
+        np.testing.assert_allclose(outs[0][0].astype(np.float32), outs[1][0].astype(np.float32), atol=2e-3,
+                                   rtol=2e-3)
+        assert_codes_close(outs[0][1], outs[1][1], max_frac=5e-3)
 
 
 @pytest.mark.parametrize("batch,beam,heads,d,K", [(16, 4, 16, 64, 1024), (3, 2, 4, 32, 256), (2, 1, 2, 128, 384),
