@@ -1273,6 +1273,86 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
   }
 }
 
+// The same for outputs of thousands of columns (vocabulary logits), K <= 1024, no K split: with
+// 32 columns per workgroup such a product is a thousand workgroups that each wait for their
+// own memory round trip, several rounds of the chip; here a workgroup walks NPAIR pairs of
+// 16-column blocks with its activation fragments resident in registers (fetched once), the
+// weights of the next pair requested before the products of the current one, and the partial
+// tiles of consecutive pairs in alternating LDS buffers (one barrier per pair).
+template <typename Epi, int MB, int NPAIR>
+__global__ void __launch_bounds__(256)
+gemm_i8_skinny16_wide_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi,
+                             int M, int N, int K, int kw, int, bool vec_store, int) {
+  __shared__ int red[2][4][MB][2][4][64];
+  asm volatile("" ::"s"(A), "s"(W));
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, kq = lane >> 4;
+  const int n00 = (int)blockIdx.x * (32 * NPAIR);
+  const int em = tid % (16 * MB), eblk = (tid / (16 * MB)) & 1;
+  const long kbase = (long)wave * kw + kq * 16;
+  const int ns = kw / 64;  // 1 .. 4 slices per wavefront
+  v4i av[4][MB];
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+      av[u][i] = *reinterpret_cast<const v4i*>(A + (long)min(16 * i + l16, M - 1) * K + kbase +
+                                               min(u, ns - 1) * 64);
+  auto load_w = [&](int pair, v4i (&wv)[4][2]) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int8_t* wp = W + (long)min(n00 + 32 * pair + 16 * b + l16, N - 1) * K + kbase;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) wv[u][b] = *reinterpret_cast<const v4i*>(wp + min(u, ns - 1) * 64);
+    }
+  };
+  v4i wv[2][4][2];
+  load_w(0, wv[0]);
+#pragma unroll
+  for (int pair = 0; pair < NPAIR; ++pair) {
+    if (n00 + 32 * pair >= N) break;  // (uniform)
+    if (pair + 1 < NPAIR) load_w(pair + 1, wv[(pair + 1) & 1]);
+    v4i acc[MB][2];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) acc[i][b] = (v4i)0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (u < ns) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+            acc[i][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[pair & 1][u][b], av[u][i],
+                                                              acc[i][b], 0, 0, 0);
+      }
+    auto& rd = red[pair & 1];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) rd[wave][i][b][r][lane] = acc[i][b][r];
+    __syncthreads();
+    if (tid < 32 * MB) {
+      const int n = n00 + 32 * pair + 16 * eblk;
+      if (em < M && n < N) {
+        v16i c;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int src = q * 16 + (em & 15);
+            c[4 * q + r] = (rd[0][em >> 4][eblk][r][src] + rd[1][em >> 4][eblk][r][src]) +
+                           (rd[2][em >> 4][eblk][r][src] + rd[3][em >> 4][eblk][r][src]);
+          }
+        epi.store16(em, n, N, c, vec_store && n + 16 <= N);
+      }
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------
@@ -1432,6 +1512,25 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   const bool full = vec_store && N % 16 == 0;  // no column tail: the lean instantiation
   if (M <= 64 && K % kBK == 0) {
     const int grid = ((N + 31) / 32) * ksplit;
+    if constexpr (std::is_same<Epi, EpiI8>::value || std::is_same<Epi, EpiI32>::value) {
+      // thousands of columns: fewer, longer workgroups (one round of the chip)
+      if (ksplit == 1 && K % 256 == 0 && K <= 1024 && N >= 8192 && g_skinny16_enabled) {
+        const int kw = K / 4;
+#define LSH_WIDE(MB, NPAIR)                                                                    \
+  launch<gemm_i8_skinny16_wide_kernel<Epi, MB, NPAIR>>((N + 32 * NPAIR - 1) / (32 * NPAIR), 256, 0, \
+                                                       A, W, epi, M, N, K, kw, 0, vec_store, s)
+        // 128 columns per workgroup up to 32768 columns (<= 256 workgroups), 256 beyond
+        if (N <= 32768) {
+          if (M <= 16) return LSH_WIDE(1, 4);
+          if (M <= 32) return LSH_WIDE(2, 4);
+          return LSH_WIDE(4, 4);
+        }
+        if (M <= 16) return LSH_WIDE(1, 8);
+        if (M <= 32) return LSH_WIDE(2, 8);
+        return LSH_WIDE(4, 8);
+#undef LSH_WIDE
+      }
+    }
     if ((K / ksplit) % 256 == 0 && g_skinny16_enabled) {
       // whole 64-byte slices for each of the four wavefronts: the 16 x 16 x 64 form
 #define LSH_SKINNY16(MB)                                                                       \
