@@ -1193,6 +1193,9 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
   // divisions and kernel-argument loads that wait for one another before its first load
   const int part = (int)blockIdx.y;
   const int n0 = (int)blockIdx.x * 32;
+  // grid z: blocks of 16 MB rows (more than 32 rows run as two workgroups of 32 rows per column
+  // block: half the fragments and products in a row for each, the weights read twice from L2)
+  const int m0 = (int)blockIdx.z * (16 * MB);
   // epilogue thread t: row t % (16 MB), column block t / (16 MB) (threads beyond 32 MB idle)
   const int em = tid % (16 * MB), eblk = (tid / (16 * MB)) & 1;
   // What the epilogue reads besides the product travels with the weights.
@@ -1210,7 +1213,7 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
   for (int b = 0; b < 2; ++b) wp[b] = W + (long)min(n0 + 16 * b + l16, N - 1) * K + kbase;
   const int8_t* ap[MB];
 #pragma unroll
-  for (int i = 0; i < MB; ++i) ap[i] = A + (long)min(16 * i + l16, M - 1) * K + kbase;
+  for (int i = 0; i < MB; ++i) ap[i] = A + (long)min(m0 + 16 * i + l16, M - 1) * K + kbase;
   v4i acc[MB][2];
 #pragma unroll
   for (int i = 0; i < MB; ++i)
@@ -1252,7 +1255,7 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
   __syncthreads();
   if (tid < 32 * MB) {
     const int n = n0 + 16 * eblk;
-    if (em < M && n < N) {
+    if (m0 + em < M && n < N) {
       v16i c;
 #pragma unroll
       for (int q = 0; q < 4; ++q)
@@ -1264,11 +1267,11 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
         }
       const bool full = FULL ? true : (vec_store && n + 16 <= N);
       if constexpr (kLut)
-        epi.store16_lds(em + (long)part * M, n, N, c, full, tab, 16 * eblk);
+        epi.store16_lds(m0 + em + (long)part * M, n, N, c, full, tab, 16 * eblk);
       else if constexpr (epi_pre<Epi>::value)
-        epi.store16_pre(em + (long)part * M, n, N, c, full, pre);
+        epi.store16_pre(m0 + em + (long)part * M, n, N, c, full, pre);
       else
-        epi.store16(em + (long)part * M, n, N, c, full);
+        epi.store16(m0 + em + (long)part * M, n, N, c, full);
     }
   }
 }
@@ -1398,16 +1401,16 @@ static int raise_lds_limit(size_t smem) {
 template <auto Kern, typename Epi>
 static int launch(int grid, int threads, size_t smem, const int8_t* A, const int8_t* W, Epi epi,
                   int M, int N, int K, int tiles_m, int tiles_n, bool vec_store, hipStream_t s,
-                  int ksplit = 1, int grid_y = 1) {
+                  int ksplit = 1, int grid_y = 1, int grid_z = 1) {
   if (int rc = raise_lds_limit<Kern>(smem)) return rc;
   if (g_ev_start != nullptr) {
     // kernel-exact begin/end timestamps on the launch stream
     hipEvent_t e0 = g_ev_start, e1 = g_ev_stop;
     g_ev_start = g_ev_stop = nullptr;
-    hipExtLaunchKernelGGL(Kern, dim3(grid, grid_y), dim3(threads), (unsigned)smem, s, e0, e1, 0, A,
+    hipExtLaunchKernelGGL(Kern, dim3(grid, grid_y, grid_z), dim3(threads), (unsigned)smem, s, e0, e1, 0, A,
                           W, epi, M, N, K, tiles_m, tiles_n, vec_store, ksplit);
   } else {
-    Kern<<<dim3(grid, grid_y), threads, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store,
+    Kern<<<dim3(grid, grid_y, grid_z), threads, smem, s>>>(A, W, epi, M, N, K, tiles_m, tiles_n, vec_store,
                                                    ksplit);
   }
   return lsh_check_launch("gemm_i8_kernel");
@@ -1533,16 +1536,29 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
     }
     if ((K / ksplit) % 256 == 0 && g_skinny16_enabled) {
       // whole 64-byte slices for each of the four wavefronts: the 16 x 16 x 64 form
-#define LSH_SKINNY16(MB)                                                                       \
+#define LSH_SKINNY16(MB, GZ)                                                                   \
   (full ? launch<gemm_i8_skinny16_kernel<Epi, MB, true>>(grid / ksplit, 256, 0, A, W, epi, M, N,  \
                                                          K, K / ksplit / 4, 0, vec_store, s,     \
-                                                         ksplit, ksplit)                         \
+                                                         ksplit, ksplit, GZ)                     \
         : launch<gemm_i8_skinny16_kernel<Epi, MB, false>>(grid / ksplit, 256, 0, A, W, epi, M, N, \
                                                           K, K / ksplit / 4, 0, vec_store, s,    \
-                                                          ksplit, ksplit))
-      if (M <= 16) return LSH_SKINNY16(1);
-      if (M <= 32) return LSH_SKINNY16(2);
-      return LSH_SKINNY16(4);
+                                                          ksplit, ksplit, GZ))
+      // More than 16 rows: the 16-row blocks are dealt to as many workgroups per column block as
+      // one round of the chip holds (measured: a wavefront with one block's fragments and
+      // products in a row finishes sooner than one with two or four, and the weights read again
+      // come from L2).
+      const int blocks = (M + 15) / 16;  // 1 .. 4
+      if (blocks == 1) return LSH_SKINNY16(1, 1);
+      if (blocks == 2) {
+        if ((long)grid * 2 <= 256) return LSH_SKINNY16(1, 2);
+        return LSH_SKINNY16(2, 1);
+      }
+      if ((long)grid * blocks <= 256) {
+        if (blocks == 3) return LSH_SKINNY16(1, 3);
+        return LSH_SKINNY16(1, 4);
+      }
+      if ((long)grid * 2 <= 256) return LSH_SKINNY16(2, 2);
+      return LSH_SKINNY16(4, 1);
 #undef LSH_SKINNY16
     }
     if (M <= 32) {
