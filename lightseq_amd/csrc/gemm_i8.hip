@@ -1178,13 +1178,14 @@ gemm_i8_skinny_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
 // tiles meet in LDS, where the epilogue threads (one per row and column block) gather the 16
 // columns the epilogues expect.
 // ---------------------------------------------------------------------------------
-template <typename Epi, int MB, bool FULL>
+template <typename Epi, int MB, bool FULL, int NB = 2>
 __global__ void __launch_bounds__(256)
 gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
                         int N, int K, int kw, int, bool vec_store, int) {
-  __shared__ int red[4][MB][2][4][64];  // [wavefront][row block][column block][register][lane]
+  // NB 16-column blocks per workgroup: 2, or 1 where that still fits one round of the chip
+  __shared__ int red[4][MB][NB][4][64];  // [wavefront][row block][column block][register][lane]
   constexpr bool kLut = std::is_same<Epi, EpiLutI8>::value;
-  __shared__ __align__(16) int8_t tab[kLut ? 32 * 256 : 16];  // table rows of the 32 columns
+  __shared__ __align__(16) int8_t tab[kLut ? 16 * NB * 256 : 16];  // table rows of the columns
   asm volatile("" ::"s"(A), "s"(W));  // one batch of kernel-argument loads, not two in a row
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, kq = lane >> 4;
@@ -1192,41 +1193,41 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
   // a multiple of 64, from the host: a kernel of a few microseconds cannot afford integer
   // divisions and kernel-argument loads that wait for one another before its first load
   const int part = (int)blockIdx.y;
-  const int n0 = (int)blockIdx.x * 32;
+  const int n0 = (int)blockIdx.x * (16 * NB);
   // grid z: blocks of 16 MB rows (more than 32 rows run as two workgroups of 32 rows per column
   // block: half the fragments and products in a row for each, the weights read twice from L2)
   const int m0 = (int)blockIdx.z * (16 * MB);
   // epilogue thread t: row t % (16 MB), column block t / (16 MB) (threads beyond 32 MB idle)
-  const int em = tid % (16 * MB), eblk = (tid / (16 * MB)) & 1;
+  const int em = tid % (16 * MB), eblk = (tid / (16 * MB)) & (NB - 1);
   // What the epilogue reads besides the product travels with the weights.
   typename epi_pre<Epi>::type pre;
   if constexpr (epi_pre<Epi>::value) pre = epi.prefetch(max(min(n0 + 16 * eblk, N - 16), 0));
   uint4 tab0, tab1;
   if constexpr (kLut) {
-    const int8_t* tp = epi_lut(epi) + (long)min(n0 + (tid >> 3), N - 1) * 256 + (tid & 7) * 32;
+    const int8_t* tp = epi_lut(epi) + (long)min(n0 + ((tid >> 3) & (16 * NB - 1)), N - 1) * 256 + (tid & 7) * 32;
     tab0 = *reinterpret_cast<const uint4*>(tp);
     tab1 = *reinterpret_cast<const uint4*>(tp + 16);
   }
   const long kbase = ((long)part * 4 + wave) * kw + kq * 16;
-  const int8_t* wp[2];
+  const int8_t* wp[NB];
 #pragma unroll
-  for (int b = 0; b < 2; ++b) wp[b] = W + (long)min(n0 + 16 * b + l16, N - 1) * K + kbase;
+  for (int b = 0; b < NB; ++b) wp[b] = W + (long)min(n0 + 16 * b + l16, N - 1) * K + kbase;
   const int8_t* ap[MB];
 #pragma unroll
   for (int i = 0; i < MB; ++i) ap[i] = A + (long)min(m0 + 16 * i + l16, M - 1) * K + kbase;
-  v4i acc[MB][2];
+  v4i acc[MB][NB];
 #pragma unroll
   for (int i = 0; i < MB; ++i)
 #pragma unroll
-    for (int b = 0; b < 2; ++b) acc[i][b] = (v4i)0;
+    for (int b = 0; b < NB; ++b) acc[i][b] = (v4i)0;
   const int ns = kw / 64;
   for (int s0 = 0; s0 < ns; s0 += 4) {
-    v4i wv[4][2], av[4][MB];
+    v4i wv[4][NB], av[4][MB];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int off = min(s0 + u, ns - 1) * 64;  // clamped: the loads stay unconditional
 #pragma unroll
-      for (int b = 0; b < 2; ++b) wv[u][b] = *reinterpret_cast<const v4i*>(wp[b] + off);
+      for (int b = 0; b < NB; ++b) wv[u][b] = *reinterpret_cast<const v4i*>(wp[b] + off);
 #pragma unroll
       for (int i = 0; i < MB; ++i) av[u][i] = *reinterpret_cast<const v4i*>(ap[i] + off);
     }
@@ -1236,7 +1237,7 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
 #pragma unroll
         for (int i = 0; i < MB; ++i)
 #pragma unroll
-          for (int b = 0; b < 2; ++b)
+          for (int b = 0; b < NB; ++b)
             acc[i][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[u][b], av[u][i], acc[i][b], 0, 0, 0);
       }
     }
@@ -1245,15 +1246,17 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
 #pragma unroll
   for (int i = 0; i < MB; ++i)
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[wave][i][b][r][lane] = acc[i][b][r];
   if constexpr (kLut) {
-    *reinterpret_cast<uint4*>(tab + (tid >> 3) * 256 + (tid & 7) * 32) = tab0;
-    *reinterpret_cast<uint4*>(tab + (tid >> 3) * 256 + (tid & 7) * 32 + 16) = tab1;
+    if (tid < 128 * NB) {
+      *reinterpret_cast<uint4*>(tab + (tid >> 3) * 256 + (tid & 7) * 32) = tab0;
+      *reinterpret_cast<uint4*>(tab + (tid >> 3) * 256 + (tid & 7) * 32 + 16) = tab1;
+    }
   }
   __syncthreads();
-  if (tid < 32 * MB) {
+  if (tid < 16 * NB * MB) {
     const int n = n0 + 16 * eblk;
     if (m0 + em < M && n < N) {
       v16i c;
@@ -1536,13 +1539,17 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
     }
     if ((K / ksplit) % 256 == 0 && g_skinny16_enabled) {
       // whole 64-byte slices for each of the four wavefronts: the 16 x 16 x 64 form
-#define LSH_SKINNY16(MB, GZ)                                                                   \
-  (full ? launch<gemm_i8_skinny16_kernel<Epi, MB, true>>(grid / ksplit, 256, 0, A, W, epi, M, N,  \
-                                                         K, K / ksplit / 4, 0, vec_store, s,     \
-                                                         ksplit, ksplit, GZ)                     \
-        : launch<gemm_i8_skinny16_kernel<Epi, MB, false>>(grid / ksplit, 256, 0, A, W, epi, M, N, \
-                                                          K, K / ksplit / 4, 0, vec_store, s,    \
-                                                          ksplit, ksplit, GZ))
+#define LSH_SKINNY16(MB, GZ)                                                                    \
+  (full && (long)grid * 2 * (GZ) <= 256                                                          \
+       ? launch<gemm_i8_skinny16_kernel<Epi, MB, true, 1>>(((N + 15) / 16), 256, 0, A, W, epi, M, \
+                                                           N, K, K / ksplit / 4, 0, vec_store, s, \
+                                                           ksplit, ksplit, GZ)                   \
+   : full ? launch<gemm_i8_skinny16_kernel<Epi, MB, true>>(grid / ksplit, 256, 0, A, W, epi, M, N, \
+                                                           K, K / ksplit / 4, 0, vec_store, s,    \
+                                                           ksplit, ksplit, GZ)                    \
+          : launch<gemm_i8_skinny16_kernel<Epi, MB, false>>(grid / ksplit, 256, 0, A, W, epi, M,  \
+                                                            N, K, K / ksplit / 4, 0, vec_store,   \
+                                                            s, ksplit, ksplit, GZ))
       // More than 16 rows: the 16-row blocks are dealt to as many workgroups per column block as
       // one round of the chip holds (measured: a wavefront with one block's fragments and
       // products in a row finishes sooner than one with two or four, and the weights read again
