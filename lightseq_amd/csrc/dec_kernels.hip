@@ -219,6 +219,28 @@ decself_attn_wg_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ 
                                  threadIdx.x & 63);
 }
 
+// Short caches (one wavefront's loads cover them: at most 8 * 1024 / D steps): four (row, head)
+// pairs per workgroup, one wavefront each, so that a step's attention is one round of the
+// chip instead of four (1024 pairs at batch 16 x beam 4 x 16 heads).
+template <int D, int UN>
+__global__ void __launch_bounds__(256)
+decself_attn_pack_kernel(const int8_t* __restrict__ q, const int8_t* __restrict__ k_cache,
+                         const int8_t* __restrict__ v_cache, int8_t* __restrict__ new_v,
+                         long bh_total, int step_num, int max_step, float attn_scale, float dq,
+                         float quant_scale) {
+  extern __shared__ __align__(16) float lds_f[];
+  const int wave = threadIdx.x >> 6;
+  const long bh_raw = (long)blockIdx.x * 4 + wave;
+  const bool live = bh_raw < bh_total;
+  const long bh = live ? bh_raw : bh_total - 1;
+  // new_v is [rows, heads * D] and a pair's D codes sit at bh * D of it
+  decself_attend_row_once<D, 1, UN>(q + bh * D, k_cache + bh * (long)max_step * D,
+                                    v_cache + bh * (long)max_step * D, new_v + bh * D, live,
+                                    step_num, attn_scale, dq, quant_scale,
+                                    lds_f + wave * decself_group_floats<D, 1>(step_num), 0,
+                                    threadIdx.x & 63);
+}
+
 static int decself_check(long bh_total, int step_num, int max_step, int head_num, int d) {
   if (bh_total <= 0 || head_num <= 0 || d <= 0 || max_step <= 0)
     return lsh_fail(LSH_ERR_INVALID, "decoder self attention: bad shape");
@@ -265,26 +287,41 @@ int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v
                          reinterpret_cast<uintptr_t>(v_cache)) & 15u) == 0;
   if (aligned && batch_head_num % head_num == 0 && batch_head_num / head_num <= 65535 &&
       (dim_per_head == 32 || dim_per_head == 64 || dim_per_head == 128)) {
-    // 8 wavefronts once the cache is long (width buys loads in flight), 4 below.  The
-    // choice depends on the step count only, never on the number of rows: the two widths
-    // sum the values in different trees, and a row's result must not depend on its batch.
-    // The loads in flight per lane (UN) follow the cache length too: unrolled rounds that
-    // a short cache never fills are code to fetch and clamped loads to wait for.
+    // 8 wavefronts per (row, head) once the cache is long (width buys loads in flight), 4
+    // below, 1 (four pairs per workgroup) where one wavefront's loads cover the cache.  The
+    // choice depends on the step count only, never on the number of rows: the widths sum the
+    // values in different trees, and a row's result must not depend on its batch.  The loads
+    // in flight per lane (UN) follow the cache length too: unrolled rounds that a short cache
+    // never fills are code to fetch and clamped loads to wait for.
     const bool wide = step_num > 256;
     const dim3 grid(head_num, batch_head_num / head_num);
+    const int kpw = 1024 / dim_per_head;  // cached steps per load instruction of a wavefront
+    if (step_num <= 8 * kpw) {
+#define LSH_DECSELF_PACK(D)                                                                      \
+  if (step_num <= 4 * kpw)                                                                       \
+    decself_attn_pack_kernel<D, 4>                                                               \
+        <<<(batch_head_num + 3) / 4, 256, 4 * decself_group_floats<D, 1>(step_num) * sizeof(float), \
+           s>>>(q, k_cache, v_cache, new_v, batch_head_num, step_num, max_step, attn_scale,      \
+                dequant_scale, quant_scale);                                                     \
+  else                                                                                           \
+    decself_attn_pack_kernel<D, 8>                                                               \
+        <<<(batch_head_num + 3) / 4, 256, 4 * decself_group_floats<D, 1>(step_num) * sizeof(float), \
+           s>>>(q, k_cache, v_cache, new_v, batch_head_num, step_num, max_step, attn_scale,      \
+                dequant_scale, quant_scale)
+      if (dim_per_head == 32) { LSH_DECSELF_PACK(32); }
+      else if (dim_per_head == 64) { LSH_DECSELF_PACK(64); }
+      else { LSH_DECSELF_PACK(128); }
+#undef LSH_DECSELF_PACK
+      return lsh_check_launch("decself_attn_pack_kernel");
+    }
 #define LSH_DECSELF(D)                                                                          \
   if (wide)                                                                                     \
     decself_attn_wg_kernel<D, 8, 8>                                                             \
         <<<grid, 512, decself_group_floats<D, 8>(step_num) * sizeof(float), s>>>(               \
         q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
         quant_scale);                                                                           \
-  else if (step_num > 128 * 64 / D)                                                             \
+  else /* 8192 / D < step_num <= 256 */                                                         \
     decself_attn_wg_kernel<D, 4, 4>                                                             \
-        <<<grid, 256, decself_group_floats<D, 4>(step_num) * sizeof(float), s>>>(               \
-        q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
-        quant_scale);                                                                           \
-  else                                                                                          \
-    decself_attn_wg_kernel<D, 4, 2>                                                             \
         <<<grid, 256, decself_group_floats<D, 4>(step_num) * sizeof(float), s>>>(               \
         q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
         quant_scale)

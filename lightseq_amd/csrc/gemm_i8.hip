@@ -1700,7 +1700,11 @@ int gemm_i8_preferred_ksplit(int M, int N, int K) {
     return 1;
   }
   int ks = 1;
-  while (ks < 8 && items * ks * 2 <= (M <= 64 ? 256 : 512) && nch % (ks * 2) == 0 &&
+  // (four planes: with one 16-column block per workgroup that is a round of the chip at hidden
+  // 1024, and the layer norm that sums the planes has half as many to fetch as with eight --
+  // measured over whole generation steps: 2 % (GPT-2-medium) and 3 % (Transformer-big) faster
+  // than eight planes, two planes 3 % slower than four)
+  while (ks < 4 && items * ks * 2 <= (M <= 64 ? 256 : 512) && nch % (ks * 2) == 0 &&
          nch / (ks * 2) >= per_item_min)
     ks *= 2;
   return ks;
