@@ -299,7 +299,7 @@ int lsh_gemm_i8_decself_qkv_i8o_f16(const int8_t* A, const int8_t* W, const void
  * -> q codes to new_q [rows, hidden], k and v codes to slot step_id of the caches [rows,
  * head_num, max_step, 64] (the same bytes as the stand-alone product), then the attention of
  * every (row, head) over slots 0..step_id -> int8 context codes ctx [rows, hidden] (the same
- * bytes as the stand-alone attention for caches of more than 64 and at most 256 steps; with
+ * bytes as the stand-alone attention for caches of more than 128 and at most 256 steps; with
  * other lengths the value sums run in another tree and a code can differ by one next to a
  * rounding boundary).  alpha, dequant_scale, cache_quant_scale: the scales of the product;
  * attn_scale, cache_dequant_scale, ctx_quant_scale: those of the attention.  ctx must not alias

@@ -314,13 +314,23 @@ int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v
 #undef LSH_DECSELF_PACK
       return lsh_check_launch("decself_attn_pack_kernel");
     }
+    // loads per lane of the 8-wavefront form: as many as the cache needs (a slot beyond the cache
+    // is a clamped load and a dead row of arithmetic; the lanes' rows and the order of their
+    // sums do not depend on it, so neither do the bits)
+    const int un8 = (step_num + 8 * kpw - 1) / (8 * kpw);
+#define LSH_DECSELF_WIDE(D, UN)                                                                 \
+  decself_attn_wg_kernel<D, 8, UN>                                                              \
+      <<<grid, 512, decself_group_floats<D, 8>(step_num) * sizeof(float), s>>>(                 \
+          q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,  \
+          quant_scale)
 #define LSH_DECSELF(D)                                                                          \
-  if (wide)                                                                                     \
-    decself_attn_wg_kernel<D, 8, 8>                                                             \
-        <<<grid, 512, decself_group_floats<D, 8>(step_num) * sizeof(float), s>>>(               \
-        q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
-        quant_scale);                                                                           \
-  else /* 8192 / D < step_num <= 256 */                                                         \
+  if (wide) {                                                                                   \
+    if (un8 <= 3) LSH_DECSELF_WIDE(D, 3);                                                       \
+    else if (un8 == 4) LSH_DECSELF_WIDE(D, 4);                                                  \
+    else if (un8 == 5) LSH_DECSELF_WIDE(D, 5);                                                  \
+    else if (un8 == 6) LSH_DECSELF_WIDE(D, 6);                                                  \
+    else LSH_DECSELF_WIDE(D, 8);                                                                \
+  } else /* 8192 / D < step_num <= 256 */                                                         \
     decself_attn_wg_kernel<D, 4, 4>                                                             \
         <<<grid, 256, decself_group_floats<D, 4>(step_num) * sizeof(float), s>>>(               \
         q, k_cache, v_cache, new_v, step_num, max_step, head_num, attn_scale, dequant_scale,    \
@@ -329,6 +339,7 @@ int decself_attention_i8(const int8_t* q, const int8_t* k_cache, const int8_t* v
     else if (dim_per_head == 64) { LSH_DECSELF(64); }
     else { LSH_DECSELF(128); }
 #undef LSH_DECSELF
+#undef LSH_DECSELF_WIDE
     return lsh_check_launch("decself_attn_wg_kernel");
   }
   decself_attn_kernel<2><<<(batch_head_num + 3) / 4, 256, decself_lds(step_num), s>>>(

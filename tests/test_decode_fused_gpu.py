@@ -141,7 +141,7 @@ def test_cross_attention_q_product_equals_the_pair(rng, batch, beam, heads, d, K
 def test_qkv_product_cache_append_and_attention_in_one_launch(rng, M, heads, K, max_step, step):
     """lsh_decself_qkv_attention_i8_f16 == lsh_gemm_i8_decself_qkv_i8o_f16 followed by
     lsh_decself_attention_i8: q codes and caches byte for byte; context codes byte for byte
-    where the group shapes agree (more than 64 and at most 256 cached steps), else within one
+    where the group shapes agree (more than 128 and at most 256 cached steps), else within one
     code on at most 0.1 % (another summation tree)."""
     from conftest import assert_codes_close
     d, H = 64, heads * 64
@@ -170,7 +170,7 @@ def test_qkv_product_cache_append_and_attention_in_one_launch(rng, M, heads, K, 
                                qs, attn_scale, cache_dq, ctx_qs)
     np.testing.assert_array_equal(to_np(q1), to_np(q0))
     np.testing.assert_array_equal(to_np(kv1), to_np(kv0))
-    if 64 < step + 1 <= 256:
+    if 128 < step + 1 <= 256:
         np.testing.assert_array_equal(to_np(ctx1), to_np(ctx0))
     else:
         assert_codes_close(to_np(ctx1), to_np(ctx0))
