@@ -676,17 +676,38 @@ int lsh_ker_arrange_qkv_with_cache_i8I_i8O_f32(int batch_token_num, int hidden_s
                                                int dim_per_head, int head_num,
                                                float dequant_scale, float quant_scale,
                                                int in_col32);
-/* kernels/gptKernels_int8.h ker_topk_sample_i8I_launcher (gptKernels_int8.cc.cu:422-463).
- * k == 1 (greedy) only: k in {2,..,32} -> LSH_ERR_UNSUPPORTED (random sampling needs the
- * reference's curand state, passed here as an ignored pointer), other k ->
- * LSH_ERR_INVALID with the reference's message.  Ties at the maximum go to the lowest
- * token id (racing stores decide in the reference).  real_seq_len is unused, as in the
- * reference. */
+/* kernels/gptKernels_int8.h ker_topk_sample_i8I_launcher (gptKernels_int8.cc.cu:252-463) and
+ * ker_topp_sample_i8I_launcher (:465-660).  k == 1: greedy, ties at the maximum go to the lowest
+ * token id (racing stores decide in the reference), curandstate unused.  k in {2, 4, 8, 16, 32}
+ * and top-p: random sampling as the kernels act with 1024 threads per block (thread t owns the
+ * ids congruent to t modulo 1024; at most one candidate per thread at or above the rough k-th
+ * largest thread maximum / the nucleus threshold; softmax over the candidates; one uniform
+ * number picks the first thread whose cumulative probability reaches it).  Other k ->
+ * LSH_ERR_INVALID with the reference's message.  curandstate: in place of the reference's
+ * curandState array (seeded with clock(), so no stream of numbers is defined there), an array of
+ * lsh_rng_state_t, one per sequence, filled by lsh_rng_setup and advanced by every draw: the
+ * uniform number of a draw is word 0 of Philox4x32-10 (key = seed, counter = (draws, 0,
+ * sequence, 0)) mapped to (0, 1] as curand_uniform maps 32 bits.  Top-p: the reference reads an
+ * uninitialised threshold in all threads but one (:533-539); built is what it intends (the
+ * longest prefix of the descending thread maxima whose exp-sum stays within p of the total, at
+ * least the largest).  real_seq_len is unused, as in the reference.  vocab_size <= 2^20. */
+typedef struct lsh_rng_state {
+  uint64_t seed;
+  uint32_t sequence, draws;
+} lsh_rng_state_t;
+/* state[i] = {seed, i, 0} for i < n (replaces ker_curand_setup,
+ * kernels/transformerKernels.cc.cu:2270-2274); state 16-byte aligned device memory */
+int lsh_rng_setup(void* state, int n, uint64_t seed, lsh_stream_t stream);
 int lsh_ker_topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len,
                             int max_thread_per_block, lsh_stream_t stream, const int8_t* logits,
                             int* old_input_ids, int* new_input_ids, const int* real_seq_len,
                             int vocab_size, int k, int* unfinished, void* curandstate, int eos_id,
                             float dequant_scale, int in_col32);
+int lsh_ker_topp_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len,
+                            int max_thread_per_block, lsh_stream_t stream, const int8_t* logits,
+                            int* old_input_ids, int* new_input_ids, const int* real_seq_len,
+                            int vocab_size, float p, int* unfinished, void* curandstate,
+                            int eos_id, float dequant_scale, int in_col32);
 /* kernels/gptKernels_int8.h ker_ppl_i8I_launcher (gptKernels_int8.cc.cu:182-190). */
 int lsh_ker_ppl_i8I(int batch_size, int batch_seq_len, int max_thread_per_block,
                     lsh_stream_t stream, const int8_t* logits, const int* input_ids,
@@ -712,7 +733,10 @@ int lsh_ker_ppl_i8I_workspace(int batch_size, int batch_seq_len, lsh_stream_t st
  *    fp32 MFMA accumulators over code values are the exact int32 scores.  ctx
  *    ([batch, head, seq, d] fp16) and ctx_q ([batch*seq, hidden] int8) are each optional;
  *  - lsh_gpt_greedy_step = ker_topk_sample_i8I<1> on ids kept in place as
- *    [batch, max_step]: writes column cur_len, last_ids[batch] and the unfinished flag. */
+ *    [batch, max_step]: writes column cur_len, last_ids[batch] and the unfinished flag;
+ *  - lsh_gpt_sample_step = ker_topk_sample_i8I<k> (k in {2, 4, 8, 16, 32}) or, with k == 0,
+ *    ker_topp_sample_i8I with p, on the same in-place ids; state as for
+ *    lsh_ker_topk_sample_i8I. */
 int lsh_gpt_arrange_qkv_prefill_f16(int batch_token_num, int hidden_size, lsh_stream_t stream,
                                     const int8_t* ori_qkv, const void* qkv_bias, void* q_codes,
                                     void* k_codes, void* v_deq, int8_t* k_cache, int8_t* v_cache,
@@ -726,6 +750,9 @@ int lsh_gpt_prefill_attention_f16(const void* q_codes, const void* k_codes, cons
 int lsh_gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size,
                         int max_step, int cur_len, int batch_size, int* unfinished, int eos_id,
                         lsh_stream_t stream);
+int lsh_gpt_sample_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size,
+                        int max_step, int cur_len, int batch_size, int* unfinished, int eos_id,
+                        int k, float p, float dequant_scale, void* state, lsh_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -114,6 +114,14 @@ int ls_model_get_steps_run(ls_model* model, int* steps);
 int ls_model_set_graph_mode(ls_model* model, int on);
 int ls_model_get_graph_stats(ls_model* model, int* captured, long long* replayed);
 
+/* QuantGpt with sampling_method topk (topk > 1) or topp: restart the per-sequence generator
+ * states of the sampling steps (sequence i of a batch draws from Philox4x32-10 keyed with `seed`,
+ * counter (draw, 0, i, 0)).  A model starts with seed 0, so two runs of one model file give the
+ * same tokens; the reference seeds its cuRAND states with clock()
+ * (kernels/transformerKernels.cc.cu:2270-2274, model/quant_gpt_encoder.cc.cu:66-71) and defines
+ * no stream of numbers.  No counterpart in the reference. */
+int ls_model_set_seed(ls_model* model, unsigned long long seed);
+
 #ifdef __cplusplus
 }
 #endif

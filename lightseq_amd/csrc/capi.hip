@@ -731,12 +731,27 @@ int lsh_ker_topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_le
                             float dequant_scale, int in_col32) {
   (void)max_thread_per_block;
   (void)real_seq_len;
-  (void)curandstate;
   if (int rc = no_col32(in_col32, 0, "ker_topk_sample_i8I")) return rc;
   if (!(dequant_scale > 0.f))
     return lsh_fail(LSH_ERR_INVALID, "ker_topk_sample_i8I: dequant_scale must be positive");
   return topk_sample_i8I(batch_size, batch_seq_len, logits_seq_len, HS(stream), logits,
-                         old_input_ids, new_input_ids, vocab_size, k, unfinished, eos_id);
+                         old_input_ids, new_input_ids, vocab_size, k, unfinished, eos_id,
+                         curandstate, dequant_scale);
+}
+int lsh_ker_topp_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len,
+                            int max_thread_per_block, lsh_stream_t stream, const int8_t* logits,
+                            int* old_input_ids, int* new_input_ids, const int* real_seq_len,
+                            int vocab_size, float p, int* unfinished, void* curandstate,
+                            int eos_id, float dequant_scale, int in_col32) {
+  (void)max_thread_per_block;
+  (void)real_seq_len;
+  if (int rc = no_col32(in_col32, 0, "ker_topp_sample_i8I")) return rc;
+  return topp_sample_i8I(batch_size, batch_seq_len, logits_seq_len, HS(stream), logits,
+                         old_input_ids, new_input_ids, vocab_size, p, unfinished, curandstate,
+                         eos_id, dequant_scale);
+}
+int lsh_rng_setup(void* state, int n, uint64_t seed, lsh_stream_t stream) {
+  return sample_state_setup(state, n, seed, HS(stream));
 }
 int lsh_ker_ppl_i8I(int batch_size, int batch_seq_len, int max_thread_per_block,
                     lsh_stream_t stream, const int8_t* logits, const int* input_ids,
@@ -778,6 +793,12 @@ int lsh_gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab
                         lsh_stream_t stream) {
   return gpt_greedy_step(logits, ids, last_ids, vocab_size, max_step, cur_len, batch_size,
                          unfinished, eos_id, HS(stream));
+}
+int lsh_gpt_sample_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size,
+                        int max_step, int cur_len, int batch_size, int* unfinished, int eos_id,
+                        int k, float p, float dequant_scale, void* state, lsh_stream_t stream) {
+  return gpt_sample_step(logits, ids, last_ids, vocab_size, max_step, cur_len, batch_size,
+                         unfinished, eos_id, k, p, dequant_scale, state, HS(stream));
 }
 
 }  // extern "C"

@@ -8,6 +8,7 @@
 #include "ls_device.cuh"
 #include "ls_launch.h"
 
+#include <string>
 #include <type_traits>
 
 namespace lsh {
@@ -408,17 +409,23 @@ __global__ void topk_sample_tail_kernel(int* old_input_ids, const int* __restric
     old_input_ids[(long)batch * seq_len + b] = new_input_ids[(long)b * (seq_len + 1) + seq_len];
 }
 
+static int sample_ids(int batch_size, int batch_seq_len, int logits_seq_len, hipStream_t s,
+                      const int8_t* logits, int* old_input_ids, int* new_input_ids, int vocab_size,
+                      int k, float p, int* unfinished, void* state, int eos_id,
+                      float dequant_scale, const char* who);
+
 int topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len, hipStream_t s,
                     const int8_t* logits, int* old_input_ids, int* new_input_ids,
-                    int vocab_size, int k, int* unfinished, int eos_id) {
+                    int vocab_size, int k, int* unfinished, int eos_id, void* state,
+                    float dequant_scale) {
   if (!logits || !old_input_ids || !new_input_ids || !unfinished || batch_size <= 0 ||
       batch_seq_len <= 0 || logits_seq_len <= 0 || vocab_size <= 0)
     return lsh_fail(LSH_ERR_INVALID, "ker_topk_sample_i8I: bad arguments");
   if (k != 1) {
     if (k == 2 || k == 4 || k == 8 || k == 16 || k == 32)
-      return lsh_fail(LSH_ERR_UNSUPPORTED,
-                      "ker_topk_sample_i8I: only topk = 1 (greedy) is provided; random sampling "
-                      "needs the reference's generator state");
+      return sample_ids(batch_size, batch_seq_len, logits_seq_len, s, logits, old_input_ids,
+                        new_input_ids, vocab_size, k, 0.f, unfinished, state, eos_id,
+                        dequant_scale, "ker_topk_sample_i8I");
     return lsh_fail(LSH_ERR_INVALID, "topk argument should be in [1,2,4,8,16,32]");
   }
   if (vocab_size > (1 << 20))
@@ -459,6 +466,304 @@ int gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_siz
   gpt_greedy_step_kernel<<<batch_size, 1024, 0, s>>>(logits, ids, last_ids, vocab_size, max_step,
                                                      cur_len, unfinished, eos_id);
   return lsh_check_launch("gpt_greedy_step_kernel");
+}
+
+// ---------------------------------------------------------------------------------
+// random sampling: ker_topk_sample_i8I<k>, k > 1 (inference/kernels/gptKernels_int8.cc.cu:252-
+// 420) and ker_topp_sample_i8I (:465-640) as they act with the 1024 threads per block the model
+// launches them with: thread t owns the vocabulary ids congruent to t modulo 1024 (a class),
+// the candidate set holds at most one id per class -- the first one of the largest
+// exp(max(logit - max, -64)) among the class's ids at or above a threshold -- and one uniform
+// number picks the first class, in thread order, whose cumulative probability reaches it.
+// Top-k: the threshold is the rough k-th largest class maximum (kernels/common.h:118-137:
+// maxima of the 32 warps of 32 threads, maximum over the warps that agree modulo k, minimum
+// over the k groups).  Top-p: the reference compares every thread's prefix sum with a threshold
+// that only its last thread assigns (:533-539), which defines nothing; built here is what it
+// intends: class maxima in descending order, exps, inclusive prefix, and the threshold is the
+// smallest maximum whose prefix stays within p of the total (at least the largest).
+// The dequantisation code * scale (scale > 0) is monotone, so maxima, thresholds and the order
+// of candidates run on the int8 codes; exps and probabilities are float as in the reference.
+// The uniform numbers: the reference draws them from a cuRAND state seeded with clock()
+// (kernels/transformerKernels.cc.cu:2270-2274); here they are Philox4x32-10 words (key = seed,
+// counter = (draw, 0, row, 0), word 0) mapped to (0, 1] as curand_uniform maps 32 bits, with
+// the state {seed, row, draws} per sequence in device memory, advanced by the kernel.
+// ---------------------------------------------------------------------------------
+struct alignas(16) SampleState {
+  unsigned long long seed;
+  unsigned int row, draws;
+};
+static_assert(sizeof(SampleState) == 16, "lsh_rng_state_t is 16 bytes");
+
+__device__ __forceinline__ uint32_t philox4x32_10_word0(uint32_t c0, uint32_t c1, uint32_t c2,
+                                                        uint32_t c3, uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const unsigned long long p0 = 0xD2511F53ull * c0, p1 = 0xCD9E8D57ull * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1;
+    c3 = (uint32_t)p0;
+    c0 = n0;
+    c2 = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+
+__global__ void sample_state_setup_kernel(SampleState* st, int n, unsigned long long seed) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) st[i] = SampleState{seed, (unsigned)i, 0u};
+}
+
+int sample_state_setup(void* state, int n, unsigned long long seed, hipStream_t s) {
+  if (!state || n <= 0 || (reinterpret_cast<uintptr_t>(state) & 15u) != 0)
+    return lsh_fail(LSH_ERR_INVALID, "rng_setup: needs a 16-byte aligned state array");
+  sample_state_setup_kernel<<<(n + 255) / 256, 256, 0, s>>>(static_cast<SampleState*>(state), n,
+                                                            seed);
+  return lsh_check_launch("sample_state_setup_kernel");
+}
+
+constexpr int kSampleThreads = 1024;
+constexpr int kSampleIdBits = 20, kSampleIdMask = (1 << kSampleIdBits) - 1;
+
+struct SampleShared {
+  int cls[kSampleThreads];   // class maxima (codes; -129 = empty), then candidate keys
+  float pf[kSampleThreads];  // exps of the 257 code values (top-p), then wavefront prefix totals
+  int hist[260];             // classes per maximum code (top-p)
+  float red[16];
+  int thr, tok;
+  float x;
+};
+
+// The 16 consecutive ids a thread reads per piece belong to 16 classes that do not change from
+// piece to piece (16 * 1024 is a multiple of 1024), so a thread reduces in registers and
+// touches LDS 16 times at the end.  f(e, v, c): slot e of the thread, id v, code c.
+template <typename F>
+__device__ __forceinline__ void sample_scan_row(const int8_t* __restrict__ lr, int vocab, F f) {
+  const int a = (int)(reinterpret_cast<uintptr_t>(lr) & 15u);
+  const int8_t* base = lr - a;
+  const int pieces = (vocab + a + 15) >> 4;
+  for (int p = threadIdx.x; p < pieces; p += kSampleThreads) {
+    const int v0 = p * 16 - a;
+    if (v0 >= 0 && v0 + 16 <= vocab) {
+      const uint4 w = *reinterpret_cast<const uint4*>(base + (long)p * 16);
+      const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int e = 0; e < 16; ++e) f(e, v0 + e, unpack_i8(ws[e >> 2], e & 3));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+        if (v0 + e >= 0 && v0 + e < vocab) f(e, v0 + e, (int)lr[v0 + e]);
+    }
+  }
+}
+
+// One row; every thread returns the sampled id.  k > 1: top-k, k == 0: top-p with p.
+__device__ int sample_row(const int8_t* __restrict__ lr, int vocab, int k, float p, float scale,
+                          SampleState* st, SampleShared& sh) {
+  const int t = threadIdx.x;
+  const int a = (int)(reinterpret_cast<uintptr_t>(lr) & 15u);
+  const int cls0 = (16 * t - a) & (kSampleThreads - 1);  // class of the thread's slot 0
+  sh.cls[t] = -129;
+  if (t < 260) sh.hist[t] = 0;
+  if (t == 0) {
+    const SampleState s = *st;
+    const uint32_t w = philox4x32_10_word0(s.draws, 0u, s.row, 0u, (uint32_t)s.seed,
+                                           (uint32_t)(s.seed >> 32));
+    sh.x = (float)w * 2.3283064365386963e-10f + 1.1641532182693481e-10f;  // (0, 1]
+    st->draws = s.draws + 1;
+  }
+  __syncthreads();
+  {
+    int m[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) m[e] = -129;
+    sample_scan_row(lr, vocab, [&](int e, int, int c) { m[e] = max(m[e], c); });
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+      if (m[e] > -129) atomicMax(&sh.cls[(cls0 + e) & (kSampleThreads - 1)], m[e]);
+  }
+  __syncthreads();
+  const int cm = sh.cls[t];
+  const int gmax = (int)block_max((float)cm, sh.red);
+  const float mx = (float)gmax * scale;
+  if (k > 0) {
+    // rough k-th largest class maximum
+    if (t < 32) {
+      int w = sh.cls[32 * t];
+      for (int l = 1; l < 32; ++l) w = max(w, sh.cls[32 * t + l]);
+      sh.hist[t] = w;
+    }
+    __syncthreads();
+    if (t == 0) {
+      int best = 127;
+      for (int g = 0; g < k; ++g) {
+        int w = sh.hist[g];
+        for (int j = g + k; j < 32; j += k) w = max(w, sh.hist[j]);
+        best = min(best, w);
+      }
+      sh.thr = best;
+    }
+  } else {
+    // classes per maximum code, exp of every code, then one thread walks the codes downwards
+    atomicAdd(&sh.hist[cm + 129], 1);
+    if (t < 257)
+      sh.pf[t] = expf(fmaxf((float)(t - 129) * scale - mx, kLogitThreshMin));  // t = code + 129
+    __syncthreads();
+    if (t == 0) {
+      // an empty class holds -inf in the reference: exp(-64) each
+      float total = (float)sh.hist[0] * expf(kLogitThreshMin);
+      for (int c = gmax; c >= -128; --c) total += (float)sh.hist[c + 129] * sh.pf[c + 129];
+      const float limit = p * total;
+      float pre = 0.f;
+      int thr = gmax;
+      for (int c = gmax; c >= -128; --c) {
+        const int n = sh.hist[c + 129];
+        if (n == 0) continue;
+        if (pre + sh.pf[c + 129] > limit) break;
+        thr = c;
+        pre += (float)n * sh.pf[c + 129];
+      }
+      sh.thr = thr;
+    }
+  }
+  __syncthreads();
+  const int thr = sh.thr;
+  sh.cls[t] = 0;  // candidate keys: (rank << 20) | (2^20 - 1 - id); 0 = none
+  __syncthreads();
+  {
+    // rank: 1 where the exp is clamped (all such ids tie: the first one wins), code + 130 else
+    int key[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) key[e] = 0;
+    sample_scan_row(lr, vocab, [&](int e, int v, int c) {
+      if (c >= thr) {
+        const bool clamped = (float)c * scale - mx < kLogitThreshMin;
+        key[e] = max(key[e], ((clamped ? 1 : c + 130) << kSampleIdBits) | (kSampleIdMask - v));
+      }
+    });
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+      if (key[e] != 0) atomicMax(&sh.cls[(cls0 + e) & (kSampleThreads - 1)], key[e]);
+  }
+  __syncthreads();
+  const int key = sh.cls[t];
+  const int rank = key >> kSampleIdBits;
+  const int my_id = key == 0 ? vocab : kSampleIdMask - (key & kSampleIdMask);
+  const float ex = key == 0 ? 0.f
+                            : expf(rank == 1 ? kLogitThreshMin
+                                             : fmaxf((float)(rank - 130) * scale - mx, kLogitThreshMin));
+  const float prob = ex / block_sum(ex, sh.red);
+  // inclusive prefix in thread order: within the wavefront, then the totals of the wavefronts before
+  float pre = prob;
+  const int lane = t & 63, wid = t >> 6;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const float up = __shfl_up(pre, d);
+    if (lane >= d) pre += up;
+  }
+  __syncthreads();
+  if (lane == 63) sh.pf[wid] = pre;
+  __syncthreads();
+  for (int w = 0; w < wid; ++w) pre += sh.pf[w];
+  const float x = sh.x;
+  int pick = kSampleThreads - (int)block_max((float)(x > pre ? 0 : kSampleThreads - t), sh.red);
+  if (pick == kSampleThreads) {
+    // rounding left the last prefix below x: the lowest thread of the largest probability
+    const float pmax = block_max(prob, sh.red);
+    pick = kSampleThreads - (int)block_max((float)(prob == pmax ? kSampleThreads - t : 0), sh.red);
+  }
+  if (t == pick) sh.tok = my_id;
+  __syncthreads();
+  return sh.tok;
+}
+
+// ker_topk_sample_i8I<k> / ker_topp_sample_i8I: ids re-laid out from [batch, seq_len] to
+// [batch, seq_len + 1] (the sampled ids behind the old array by topk_sample_tail_kernel)
+__global__ void __launch_bounds__(kSampleThreads)
+sample_ids_kernel(const int8_t* __restrict__ logits, int* old_input_ids,
+                  int* __restrict__ new_input_ids, int vocab, int seq_len, int logits_seq_len,
+                  int* unfinished, int eos_id, int k, float p, float scale, SampleState* st) {
+  __shared__ SampleShared sh;
+  const int b = blockIdx.x;
+  const bool ended = old_input_ids[(long)b * seq_len + seq_len - 1] == eos_id;
+  for (int t = threadIdx.x; t < seq_len; t += blockDim.x)
+    new_input_ids[(long)b * (seq_len + 1) + t] = old_input_ids[(long)b * seq_len + t];
+  int tok = eos_id;
+  if (!ended)
+    tok = sample_row(logits + ((long)b * logits_seq_len + logits_seq_len - 1) * vocab, vocab, k, p,
+                     scale, st + b, sh);
+  if (threadIdx.x == 0) {
+    if (!ended && tok != eos_id) unfinished[0] = 1;
+    new_input_ids[(long)b * (seq_len + 1) + seq_len] = tok;
+  }
+}
+
+static int sample_ids(int batch_size, int batch_seq_len, int logits_seq_len, hipStream_t s,
+                      const int8_t* logits, int* old_input_ids, int* new_input_ids, int vocab_size,
+                      int k, float p, int* unfinished, void* state, int eos_id,
+                      float dequant_scale, const char* who) {
+  if (!state || (reinterpret_cast<uintptr_t>(state) & 15u) != 0)
+    return lsh_fail(LSH_ERR_INVALID, (std::string(who) + ": random sampling needs the generator "
+                                                         "state array (lsh_rng_setup)").c_str());
+  if (!(dequant_scale > 0.f))
+    return lsh_fail(LSH_ERR_INVALID, (std::string(who) + ": dequant_scale must be positive").c_str());
+  if (vocab_size > (1 << kSampleIdBits))
+    return lsh_fail(LSH_ERR_UNSUPPORTED, (std::string(who) + ": vocabulary above 2^20 ids").c_str());
+  sample_ids_kernel<<<batch_size, kSampleThreads, 0, s>>>(
+      logits, old_input_ids, new_input_ids, vocab_size, batch_seq_len, logits_seq_len, unfinished,
+      eos_id, k, p, dequant_scale, static_cast<SampleState*>(state));
+  if (int rc = lsh_check_launch("sample_ids_kernel")) return rc;
+  topk_sample_tail_kernel<<<(batch_size + 255) / 256, 256, 0, s>>>(old_input_ids, new_input_ids,
+                                                                   batch_size, batch_seq_len);
+  return lsh_check_launch("topk_sample_tail_kernel");
+}
+
+int topp_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len, hipStream_t s,
+                    const int8_t* logits, int* old_input_ids, int* new_input_ids, int vocab_size,
+                    float p, int* unfinished, void* state, int eos_id, float dequant_scale) {
+  if (!logits || !old_input_ids || !new_input_ids || !unfinished || batch_size <= 0 ||
+      batch_seq_len <= 0 || logits_seq_len <= 0 || vocab_size <= 0 || !(p > 0.f) || p > 1.f)
+    return lsh_fail(LSH_ERR_INVALID, "ker_topp_sample_i8I: bad arguments");
+  return sample_ids(batch_size, batch_seq_len, logits_seq_len, s, logits, old_input_ids,
+                    new_input_ids, vocab_size, 0, p, unfinished, state, eos_id, dequant_scale,
+                    "ker_topp_sample_i8I");
+}
+
+// the model's step with random sampling: as gpt_greedy_step_kernel
+__global__ void __launch_bounds__(kSampleThreads)
+gpt_sample_step_kernel(const int8_t* __restrict__ logits, int* ids, int* __restrict__ last_ids,
+                       int vocab, int max_step, int cur_len, int* unfinished, int eos_id, int k,
+                       float p, float scale, SampleState* st) {
+  __shared__ SampleShared sh;
+  const int b = blockIdx.x;
+  const bool ended = ids[(long)b * max_step + cur_len - 1] == eos_id;
+  int tok = eos_id;
+  if (!ended) tok = sample_row(logits + (long)b * vocab, vocab, k, p, scale, st + b, sh);
+  if (threadIdx.x == 0) {
+    if (!ended && tok != eos_id) unfinished[0] = 1;
+    ids[(long)b * max_step + cur_len] = tok;
+    last_ids[b] = tok;
+  }
+}
+
+int gpt_sample_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size, int max_step,
+                    int cur_len, int batch_size, int* unfinished, int eos_id, int k, float p,
+                    float dequant_scale, void* state, hipStream_t s) {
+  if (!logits || !ids || !last_ids || !unfinished || !state || batch_size <= 0 ||
+      vocab_size <= 0 || cur_len <= 0 || cur_len >= max_step || !(dequant_scale > 0.f) ||
+      (reinterpret_cast<uintptr_t>(state) & 15u) != 0)
+    return lsh_fail(LSH_ERR_INVALID, "gpt_sample_step: bad arguments");
+  if (k != 0 && k != 2 && k != 4 && k != 8 && k != 16 && k != 32)
+    return lsh_fail(LSH_ERR_INVALID, "topk argument should be in [1,2,4,8,16,32]");
+  if (k == 0 && (!(p > 0.f) || p > 1.f))
+    return lsh_fail(LSH_ERR_INVALID, "gpt_sample_step: topp outside (0, 1]");
+  if (vocab_size > (1 << kSampleIdBits))
+    return lsh_fail(LSH_ERR_UNSUPPORTED, "gpt_sample_step: vocabulary above 2^20 ids");
+  gpt_sample_step_kernel<<<batch_size, kSampleThreads, 0, s>>>(
+      logits, ids, last_ids, vocab_size, max_step, cur_len, unfinished, eos_id, k, p,
+      dequant_scale, static_cast<SampleState*>(state));
+  return lsh_check_launch("gpt_sample_step_kernel");
 }
 
 // ---------------------------------------------------------------------------------

@@ -335,9 +335,21 @@ int arrange_qkv_with_cache_i8I_i8O(int batch_token_num, int hidden_size, hipStre
                                    int8_t* new_k, const int8_t* k_cache, int8_t* new_v,
                                    const int8_t* v_cache, int batch_seq_len, int dim_per_head,
                                    int head_num, float dequant_scale, float quant_scale);
+// k == 1: greedy (state unused); k in {2, 4, 8, 16, 32}: random sampling with the generator
+// states `state` (16 bytes per sequence, sample_state_setup)
 int topk_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len, hipStream_t s,
                     const int8_t* logits, int* old_input_ids, int* new_input_ids,
-                    int vocab_size, int k, int* unfinished, int eos_id);
+                    int vocab_size, int k, int* unfinished, int eos_id, void* state,
+                    float dequant_scale);
+int topp_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len, hipStream_t s,
+                    const int8_t* logits, int* old_input_ids, int* new_input_ids, int vocab_size,
+                    float p, int* unfinished, void* state, int eos_id, float dequant_scale);
+// generator states of n sequences: {seed, sequence index, draws made = 0}
+int sample_state_setup(void* state, int n, unsigned long long seed, hipStream_t s);
+// the model's step with random sampling (k in {2,..,32}: top-k; k == 0: top-p with p)
+int gpt_sample_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size, int max_step,
+                    int cur_len, int batch_size, int* unfinished, int eos_id, int k, float p,
+                    float dequant_scale, void* state, hipStream_t s);
 int gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size, int max_step,
                     int cur_len, int batch_size, int* unfinished, int eos_id, hipStream_t s);
 int ppl_i8I(int batch_size, int batch_seq_len, hipStream_t s, const int8_t* logits,

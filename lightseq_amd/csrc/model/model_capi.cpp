@@ -294,6 +294,13 @@ int ls_model_set_graph_mode(ls_model* model, int on) {
                        "graph mode applies to the generation steps of QuantTransformer and QuantGpt");
 }
 
+int ls_model_set_seed(ls_model* model, unsigned long long seed) {
+  NEED_MODEL(model);
+  if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get()))
+    return guarded([&] { qg->encoder()->set_seed(seed); });
+  return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "a seed applies to the random sampling of QuantGpt");
+}
+
 int ls_model_get_graph_stats(ls_model* model, int* captured, long long* replayed) {
   NEED_MODEL(model);
   if (!captured || !replayed) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");

@@ -37,12 +37,13 @@ std::string QuantGptEncoder::check() {
   const std::string& m = _tw._sampling_method;
   if (m != "topk" && m != "topp" && m != "ppl")
     return std::string("unsupported sampling_method: ") + m;
-  if (_tw._topk <= 0) return "topk must be positive";
-  if (m == "topp" || (m == "topk" && _tw._topk != 1))
-    return "random sampling is not available in this build: the model file asks for sampling_method " +
-           m + " with topk = " + std::to_string(_tw._topk) + ", topp = " + std::to_string(_tw._topp) +
-           " (a file that sets no topk gets the format's default, 4); export it with topk = 1 "
-           "(greedy) or sampling_method ppl";
+  if (m == "topk" && _tw._topk != 1 && _tw._topk != 2 && _tw._topk != 4 && _tw._topk != 8 &&
+      _tw._topk != 16 && _tw._topk != 32)
+    return "topk argument should be in [1,2,4,8,16,32], the model file has topk = " +
+           std::to_string(_tw._topk);
+  if (m == "topp" && (!(_tw._topp > 0.f) || _tw._topp > 1.f))
+    return "topp must lie in (0, 1], the model file has topp = " + std::to_string(_tw._topp);
+  if (_tw._src_vocab_size > (1 << 20)) return "violate vocab_size <= 2^20 (sampling kernels)";
   if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)
     return "violate hidden_size % 16 = 0 and inner_size % 16 = 0 (int8 MFMA GEMM)";
   if (_tw._dim_per_head != 32 && _tw._dim_per_head != 64 && _tw._dim_per_head != 128)
@@ -61,6 +62,8 @@ void QuantGptEncoder::init_buffer() {
   _ids.alloc(tokens);
   _last_ids.alloc(_max_batch_size);
   _unfinished.alloc(1);
+  _sample_state.alloc(2 * (size_t)_max_batch_size);  // 16 bytes per sequence
+  set_seed(0);
   CHECK_GPU_ERROR(hipHostMalloc(reinterpret_cast<void**>(&_h_unfinished), sizeof(int)));
   *_h_unfinished = 0;
   _query.alloc((size_t)_max_batch_dim);
@@ -278,8 +281,22 @@ void QuantGptEncoder::enqueue_sampling(const int8_t* hidden, bool clear_flag) {
                                    (size_t)B * V, hipMemcpyDeviceToDevice, _stream));
   // (after a cached step the flag was cleared by the step's embedding launch)
   if (clear_flag) LSH_CALL(fill_i32(_unfinished.get(), 0, 1, _stream));
-  LSH_CALL(gpt_greedy_step(_logits.get(), _ids.get(), _last_ids.get(), V, _tw._max_step,
-                           _batch_seq_len, B, _unfinished.get(), _tw._eos_id, _stream));
+  const bool topp = _tw._sampling_method == "topp";
+  if (!topp && _tw._topk == 1) {
+    LSH_CALL(gpt_greedy_step(_logits.get(), _ids.get(), _last_ids.get(), V, _tw._max_step,
+                             _batch_seq_len, B, _unfinished.get(), _tw._eos_id, _stream));
+  } else {
+    // ker_topk_sample_i8I<k> / ker_topp_sample_i8I (:405-430, :448-473)
+    LSH_CALL(gpt_sample_step(_logits.get(), _ids.get(), _last_ids.get(), V, _tw._max_step,
+                             _batch_seq_len, B, _unfinished.get(), _tw._eos_id,
+                             topp ? 0 : _tw._topk, _tw._topp, _logits_clip_max / _quant_range,
+                             _sample_state.get(), _stream));
+  }
+}
+
+// Restart the generator states of the random-sampling steps: sequence i draws from (seed, i).
+void QuantGptEncoder::set_seed(unsigned long long seed) {
+  LSH_CALL(sample_state_setup(_sample_state.get(), _max_batch_size, seed, _stream));
 }
 
 // host side of a sampled token: counters and the unfinished flag (one word back from the device)

@@ -33,6 +33,9 @@ class QuantGptEncoder {
   void run_one_infer(int batch_size, int batch_seq_len);  // perplexity
   int run_one_sample(int batch_size, int batch_seq_len);  // returns the sampled length
   void benchmark_mode(bool is_benchmark) { _is_benchmark = is_benchmark; }
+  // Random sampling (topk > 1, topp): restart the per-sequence generator states from `seed`
+  // (0 at load; the reference seeds its cuRAND states with clock()).
+  void set_seed(unsigned long long seed);
 
   // Optional record for parity checks: the last-position int8 logits of every sampling
   // step, [max_steps, batch, vocab] (device pointer owned by the caller).
@@ -80,6 +83,7 @@ class QuantGptEncoder {
   int _rec_max_steps = 0;
 
   DeviceBuffer<int> _real_seq_len, _ids, _last_ids, _unfinished;
+  DeviceBuffer<long long> _sample_state;  // lsh_rng_state_t [max_batch_size]
   DeviceBuffer<__half> _query, _qkv_buf;  // q codes | k codes | v, each max_batch_dim
   DeviceBuffer<int8_t> _buf_a, _buf_b, _buf_q, _hid_last, _logits;
   DeviceBuffer<int32_t> _int32_ffn_out_buf;

@@ -58,6 +58,7 @@ def _bind():
         "ls_model_set_step_record": [_P, _P, _P, _I],
         "ls_model_get_steps_run": [_P, ip],
         "ls_model_set_graph_mode": [_P, _I],
+        "ls_model_set_seed": [_P, ctypes.c_uint64],
         "ls_model_get_graph_stats": [_P, ip, ctypes.POINTER(ctypes.c_longlong)],
     }
     for name, argtypes in sigs.items():
@@ -176,6 +177,10 @@ class LSModel:
     def graph_mode(self, flag):
         """QuantTransformer / QuantGpt: replay generation steps as HIP graphs."""
         self._call("ls_model_set_graph_mode", self._h, int(bool(flag)))
+
+    def set_seed(self, seed):
+        """QuantGpt with random sampling (topk > 1, topp): restart the generator states."""
+        self._call("ls_model_set_seed", self._h, int(seed) & 0xFFFFFFFFFFFFFFFF)
 
     def graph_stats(self):
         """(graphs captured, steps replayed) so far."""

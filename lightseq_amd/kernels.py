@@ -494,6 +494,25 @@ def ker_topk_sample_i8I_launcher(batch_size, batch_seq_len, logits_seq_len, max_
          eos_id, dequant_scale, int(in_col32))
 
 
+def ker_topp_sample_i8I_launcher(batch_size, batch_seq_len, logits_seq_len, max_thread_per_block,
+                                 logits, old_input_ids, new_input_ids, real_seq_len, vocab_size, p,
+                                 unfinished, curandstate, eos_id, dequant_scale, in_col32=False):
+    _dev(logits, old_input_ids, new_input_ids, unfinished, curandstate)
+    call("lsh_ker_topp_sample_i8I", batch_size, batch_seq_len, logits_seq_len,
+         max_thread_per_block, current_stream(), ptr(logits), ptr(old_input_ids),
+         ptr(new_input_ids), ptr(real_seq_len), vocab_size, p, ptr(unfinished), ptr(curandstate),
+         eos_id, dequant_scale, int(in_col32))
+
+
+def rng_setup(batch_size, seed, device="cuda"):
+    """Generator states of ``batch_size`` sequences for the random-sampling launchers (in place
+    of the reference's curandState array): an int64 tensor [batch_size, 2] holding
+    ``lsh_rng_state_t`` records {seed, sequence, draws}."""
+    state = torch.zeros((batch_size, 2), dtype=torch.int64, device=device)
+    call("lsh_rng_setup", ptr(state), batch_size, int(seed) & 0xFFFFFFFFFFFFFFFF, current_stream())
+    return state
+
+
 def ker_ppl_i8I_launcher(batch_size, batch_seq_len, max_thread_per_block, logits, input_ids,
                          real_seq_len, ppl, vocab_size, dequant_scale, in_col32=False):
     _dev(logits, input_ids, real_seq_len, ppl)
@@ -537,7 +556,16 @@ def gpt_greedy_step(logits, ids, last_ids, vocab_size, max_step, cur_len, batch_
          cur_len, batch_size, ptr(unfinished), eos_id, current_stream())
 
 
-__all__ = [n for n in dir() if n.startswith(("launch_", "ker_", "gemm_", "encself_", "quantize_", "gpt_",
+def gpt_sample_step(logits, ids, last_ids, vocab_size, max_step, cur_len, batch_size, unfinished,
+                    eos_id, k, p, dequant_scale, state):
+    """The model's step with random sampling: top-k for k in {2, 4, 8, 16, 32}, top-p for k == 0."""
+    _dev(logits, ids, last_ids, unfinished, state)
+    call("lsh_gpt_sample_step", ptr(logits), ptr(ids), ptr(last_ids), vocab_size, max_step,
+         cur_len, batch_size, ptr(unfinished), eos_id, k, p, dequant_scale, ptr(state),
+         current_stream())
+
+
+__all__ = [n for n in dir() if n.startswith(("launch_", "ker_", "gemm_", "rng_", "encself_", "quantize_", "gpt_",
                                              "decself_", "encdec_", "select_beam_", "beam_",
                                              "refresh_", "length_norm"))]
 _ = lib  # re-exported for callers that want lib.LSHError

@@ -25,10 +25,10 @@ class LSHError(RuntimeError):
 
 
 _P, _I, _F, _L = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_long
-_CODES = {"p": _P, "s": _P, "i": _I, "f": _F, "l": _L, "c": ctypes.c_char_p}
+_CODES = {"p": _P, "s": _P, "i": _I, "f": _F, "l": _L, "c": ctypes.c_char_p, "Q": ctypes.c_uint64}
 
 # name -> (has _f16/_f32 variants, argument codes).  p pointer, s stream, i int, f float,
-# l int64_t, c C string
+# l int64_t, Q uint64_t, c C string
 _SIGNATURES = {
     "lsh_launch_quantize_tensor": (True, "ppiifsi"),
     "lsh_launch_dequantize_tensor": (True, "ppiifsi"),
@@ -104,6 +104,9 @@ _SIGNATURES = {
     "lsh_gpt_arrange_qkv_prefill_f16": (False, "iis" + "ppppppp" + "iiii" + "ff"),
     "lsh_gpt_prefill_attention_f16": (False, "pppppp" + "ff" + "iiii" + "s"),
     "lsh_gpt_greedy_step": (False, "ppp" + "iiii" + "p" + "i" + "s"),
+    "lsh_gpt_sample_step": (False, "ppp" + "iiii" + "p" + "i" + "iff" + "p" + "s"),
+    "lsh_ker_topp_sample_i8I": (False, "iiiis" + "pppp" + "if" + "pp" + "ifi"),
+    "lsh_rng_setup": (False, "piQs"),
     # operator launchers of the csrc layer path (include/lightseq_ops.h)
     "lsh_launch_quantize": (True, "ppppp" + "ii" + "s"),
     "lsh_launch_quantize_2d": (True, "ppppp" + "iii" + "s" + "i"),

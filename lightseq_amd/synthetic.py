@@ -316,7 +316,7 @@ def make_quant_gpt(cfg, seed=0, ln_noise=0.02, w_std=None):
             "ffn_first_output_clip_max": proj, "self_qkv_bias_out_clip_max": proj,
         })
     conf = {"head_num": cfg["head_num"], "src_padding_id": cfg["padding_id"],
-            "sampling_method": cfg.get("sampling_method", "topk"), "topp": 0.75,
+            "sampling_method": cfg.get("sampling_method", "topk"), "topp": cfg.get("topp", 0.75),
             "topk": cfg.get("topk", 1), "eos_id": cfg["eos_id"],
             "extra_decode_length": cfg["extra_decode_length"]}
     return {"src_embedding": emb, "encoder_stack": layers, "model_conf": conf}

@@ -36,6 +36,8 @@ def _code(arg):
         return "f"
     if arg.startswith("int64_t"):
         return "l"
+    if arg.startswith("uint64_t") or arg.startswith("unsigned long long"):
+        return "Q"
     if arg.startswith("int"):
         return "i"
     raise AssertionError("unhandled parameter type: %r" % arg)
