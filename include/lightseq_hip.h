@@ -600,6 +600,29 @@ int lsh_beam_search_step_i8I_f32(const int8_t* logits, const void* logit_bias, f
                                  float dequant_scale, int vocab_size, int max_step,
                                  float length_norm, int cur_step, int batch_size, int beam_size,
                                  int end_id, lsh_stream_t stream);
+/* The same step with a second workspace, with which the per-row top-k -- bound by vector
+ * instructions, one workgroup per row on one compute unit -- is dealt to ceil(vocab_size / 8192)
+ * workgroups per row (each computes the row's statistics and the proposals of its part; the
+ * merge reads them all).  lsh_beam_search_step_workspace: bytes the shape needs, 0
+ * when it does not use one (vocab_size <= 8192, > 32768 or not a multiple of 16).  With a null,
+ * short or misaligned (8 bytes) workspace the step runs as lsh_beam_search_step_i8I.  Same
+ * beams and ids; the log-sum-exp of a row is added in another order (a last-place difference
+ * of the scores).  What QuantTransformer runs.  No counterpart in the reference. */
+int64_t lsh_beam_search_step_workspace(int batch_size, int beam_size, int vocab_size);
+int lsh_beam_search_step_ws_i8I_f16(const int8_t* logits, const void* logit_bias, float* seq_probs,
+                                    float* seq_score, const int* old_alive_seq,
+                                    int* new_alive_seq, float* top_score, int* top_idx,
+                                    int* parent, int* num_finished, float dequant_scale,
+                                    int vocab_size, int max_step, float length_norm, int cur_step,
+                                    int batch_size, int beam_size, int end_id, void* workspace,
+                                    int64_t workspace_bytes, lsh_stream_t stream);
+int lsh_beam_search_step_ws_i8I_f32(const int8_t* logits, const void* logit_bias, float* seq_probs,
+                                    float* seq_score, const int* old_alive_seq,
+                                    int* new_alive_seq, float* top_score, int* top_idx,
+                                    int* parent, int* num_finished, float dequant_scale,
+                                    int vocab_size, int max_step, float length_norm, int cur_step,
+                                    int batch_size, int beam_size, int end_id, void* workspace,
+                                    int64_t workspace_bytes, lsh_stream_t stream);
 /* lsh_beam_search_step_i8I_f16 for callers that cannot allocate device memory (code
  * under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  No
  * counterpart in the reference.  The proposal workspace (top_score / top_idx) is a

@@ -699,6 +699,151 @@ beam_topk_reg_kernel(const int8_t* __restrict__ logits, const T* __restrict__ lo
   }
 }
 
+// The per-row top-k dealt to P workgroups per row (vocabularies of up to 32 * 1024 ids, VEC
+// layout): beam_topk_reg_kernel is bound by vector instructions -- a row's 32 K logits cost
+// about 45 instructions each and one workgroup keeps them all on one compute unit, 64 rows on
+// 64 of the 256 -- so a row's ids are cut into P <= 4 parts of at most 8192 and the top-k runs
+// as rows x P workgroups of 512 threads (16 ids per thread and part).  Every workgroup of a row
+// computes the row's maximum and sum of exponentials itself, from all of the row (the one-pass
+// sums of beam_topk_reg_kernel in another order; a separate statistics launch ahead of it cost
+// more than the repeated arithmetic), then the scores of its own part's ids and the part's
+// best beam_size by the same 64-bit keys.
+// The merge then reads P * beam_size proposals per row instead of beam_size: a row's best
+// beam_size by (score, id) are among the union of its parts' best beam_size by (score, id), so
+// the beams chosen are the same.
+template <typename T>
+__device__ __forceinline__ void beam_part_load(const int8_t* __restrict__ lr,
+                                               const T* __restrict__ logit_bias, int lo, int hi,
+                                               float dq, float (&lg)[16]) {
+#pragma clang fp contract(off)
+  // thread t owns ids lo + 16 t .. + 15: 512 threads, one 16-byte piece each (two wavefronts
+  // per SIMD take turns; with 32 ids per thread and one wavefront per SIMD every dependent
+  // instruction waits out its latency and the kernel takes twice as long)
+  const int v0 = lo + 16 * (int)threadIdx.x;
+  if (v0 < hi) {
+    const uint4 w = *reinterpret_cast<const uint4*>(lr + v0);
+    float b[16];
+    ld4(logit_bias, v0, *reinterpret_cast<float(*)[4]>(b));
+    ld4(logit_bias, v0 + 4, *reinterpret_cast<float(*)[4]>(b + 4));
+    ld4(logit_bias, v0 + 8, *reinterpret_cast<float(*)[4]>(b + 8));
+    ld4(logit_bias, v0 + 12, *reinterpret_cast<float(*)[4]>(b + 12));
+    const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int e = 0; e < 16; ++e) lg[e] = (float)unpack_i8(ws[e >> 2], e & 3) * dq + b[e];
+  } else {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) lg[e] = 0.f;
+  }
+}
+
+constexpr int kBeamPartIds = 8192;  // ids of a part, at most (a multiple of 16: parts stay aligned)
+
+template <typename T>
+__global__ void __launch_bounds__(512)
+beam_topk_part_kernel(const int8_t* __restrict__ logits, const T* __restrict__ logit_bias,
+                      const float* __restrict__ seq_probs, const float* __restrict__ seq_score,
+                      const int* __restrict__ alive_seq, float dq, float* __restrict__ top_score,
+                      int* __restrict__ top_idx, int vocab, int max_step, float length_norm,
+                      int cur_step, int beam_size, int end_id) {
+#pragma clang fp contract(off)
+  __shared__ unsigned long long wbest[2][8];
+  __shared__ float red_max[16], red_sum[16];
+  const int part = blockIdx.x, row = blockIdx.y, P = gridDim.x, t = threadIdx.x;
+  const int lane = t & 63, wid = t >> 6;
+  const int batch_id = row / beam_size, beam_id = row % beam_size;
+  float* os = top_score + ((long)row * P + part) * beam_size;
+  int* oi = top_idx + ((long)row * P + part) * beam_size;
+  if (cur_step != 0 && alive_seq[(long)row * max_step + cur_step] == end_id) {
+    // a finished beam proposes itself once (part 0, slot 0)
+    if (t < beam_size) {
+      const bool self = part == 0 && t == 0;
+      os[t] = self ? seq_score[row] : -INFINITY;
+      oi[t] = self ? end_id + beam_id * vocab : kNoCand;
+    }
+    return;
+  }
+  const int lo = part * kBeamPartIds, hi = min(lo + kBeamPartIds, vocab);
+  // the row's maximum and sum of exponentials: every workgroup of the row reads all of it (the
+  // other parts' logits come from L2), so no workgroup waits for another
+  float all[4][16];
+#pragma unroll
+  for (int p = 0; p < 4; ++p)
+    beam_part_load(logits + (long)row * vocab, logit_bias, p * kBeamPartIds,
+                   min((p + 1) * kBeamPartIds, vocab), dq, all[p]);
+  float tmax = kFloatInfNeg;
+#pragma unroll
+  for (int p = 0; p < 4; ++p)
+    if (p * kBeamPartIds + 16 * t < vocab) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, all[p][i]);
+    }
+  const float max_logit = block_max_dpp(tmax, red_max);
+  float se = 0.f;
+#pragma unroll
+  for (int p = 0; p < 4; ++p)
+    if (p * kBeamPartIds + 16 * t < vocab) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) se += __expf(fmaxf(all[p][i] - max_logit, kLogitThreshMin));
+    }
+  const float sum_exp = block_sum_dpp(se, red_sum);
+  float lg[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    lg[i] = part == 0 ? all[0][i] : part == 1 ? all[1][i] : part == 2 ? all[2][i] : all[3][i];
+  const float base = seq_probs[row] - logf(sum_exp) - max_logit;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) lg[i] = cand_score(lg[i], base, length_norm, batch_id);
+  auto id_of = [&](int i) { return lo + 16 * t + i; };
+  auto key_of = [&](int i) -> unsigned long long {
+    const int id = id_of(i);
+    if (id >= hi) return 0ull;
+    unsigned u = __builtin_bit_cast(unsigned, lg[i] + 0.f);  // -0 -> +0
+    u ^= (u >> 31) ? 0xffffffffu : 0x80000000u;
+    return ((unsigned long long)u << 32) | (unsigned)(0x7fffffff - id);
+  };
+  auto my_best_below = [&](unsigned long long bound) {
+    unsigned long long best = 0ull;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const unsigned long long c = key_of(i);
+      if (c < bound && c > best) best = c;
+    }
+    return best;
+  };
+  auto umax64 = [](unsigned long long a, unsigned long long b) { return a > b ? a : b; };
+  auto dpp64 = [](unsigned long long x, auto ctrl) {
+    const unsigned l = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)x, decltype(ctrl)::value, 0xf, 0xf, false);
+    const unsigned h = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)(x >> 32), decltype(ctrl)::value, 0xf, 0xf, false);
+    return ((unsigned long long)h << 32) | l;
+  };
+  auto lane64 = [](unsigned long long x, int l) {
+    const unsigned lo32 = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)x, l);
+    const unsigned hi32 = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(x >> 32), l);
+    return ((unsigned long long)hi32 << 32) | lo32;
+  };
+  unsigned long long mine = my_best_below(~0ull);
+  for (int k = 0; k < beam_size; ++k) {
+    unsigned long long best = mine;
+    best = umax64(best, dpp64(best, std::integral_constant<int, kDppXor1>()));
+    best = umax64(best, dpp64(best, std::integral_constant<int, kDppXor2>()));
+    best = umax64(best, dpp64(best, std::integral_constant<int, kDppHalfMirror>()));
+    best = umax64(best, dpp64(best, std::integral_constant<int, kDppMirror>()));
+    best = umax64(umax64(lane64(best, 0), lane64(best, 16)), umax64(lane64(best, 32), lane64(best, 48)));
+    unsigned long long* wb = wbest[k & 1];
+    if (lane == 0) wb[wid] = best;
+    __syncthreads();
+    best = umax64(umax64(umax64(wb[0], wb[1]), umax64(wb[2], wb[3])),
+                  umax64(umax64(wb[4], wb[5]), umax64(wb[6], wb[7])));
+    if (t == 0) {
+      unsigned u = (unsigned)(best >> 32);
+      u ^= (u >> 31) ? 0x80000000u : 0xffffffffu;
+      os[k] = best == 0ull ? -INFINITY : __builtin_bit_cast(float, u);
+      oi[k] = best == 0ull ? kNoCand : beam_id * vocab + (0x7fffffff - (int)(unsigned)best);
+    }
+    if (best == mine && best != 0ull) mine = my_best_below(best);
+  }
+}
+
 // beam_merge_kernel: one block, one wavefront per sentence (sentences are dealt to the
 // wavefronts round-robin).  Picks the sentence's best `beam_size` of its
 // beam_size * beam_size proposals in (score descending, candidate id ascending) order
@@ -711,52 +856,162 @@ beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ t
                   float* __restrict__ seq_probs, float* __restrict__ seq_score,
                   int* __restrict__ parent, int* __restrict__ num_finished, int batch,
                   int beam_size, int vocab, int max_step, int cur_step, float length_norm,
-                  int end_id) {
+                  int end_id, int parts) {
 #pragma clang fp contract(off)
   __shared__ int fin_cnt[16];
+  __shared__ int seq_lds[16][512];  // a sentence's old sequences (beam_size * max_step <= 512)
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int nw = blockDim.x >> 6;
-  const int ncand = beam_size * beam_size;  // <= 1024
+  const int ncand = beam_size * beam_size * parts;  // proposals of a sentence
   int finished = 0;
-  for (int b = wid; b < batch; b += nw) {
-    const float* cs = top_score + (long)b * ncand;
-    const int* ci = top_idx + (long)b * ncand;
-    ScoreIdx prev;
-    prev.s = INFINITY;
-    prev.i = -1;
-    for (int j = 0; j < beam_size; ++j) {
-      ScoreIdx best;
-      best.s = -INFINITY;
-      best.i = kNoCand;
-      for (int c = lane; c < ncand; c += 64) {
-        ScoreIdx x;
-        x.s = cs[c];
-        x.i = ci[c];
-        if (x.i != kNoCand && before(prev, x) && before(x, best)) best = x;
+  // applies one pick (ker_refresh_result): the new sequence, then probability or score
+  auto apply = [&](int b, int j, float score, int idx) {
+    // a sentence always has at least beam_size proposals; guard the indices anyway
+    const int ori = idx == kNoCand ? end_id : idx;
+    int can_beam = ori / vocab;
+    const int can_vocab = ori % vocab;
+    if (can_beam >= beam_size) can_beam = 0;
+    const int* from = old_alive_seq + ((long)b * beam_size + can_beam) * max_step;
+    int* to = new_alive_seq + ((long)b * beam_size + j) * max_step;
+    for (int t = lane; t < max_step; t += 64)
+      to[t] = t > cur_step + 1 ? end_id : (t == cur_step + 1 ? can_vocab : from[t]);
+    if (lane == 0) {
+      if (can_vocab != end_id) {
+        seq_probs[b * beam_size + j] = (score - (float)b * kMinLogProb) / length_norm;
+        parent[b * beam_size + j] = can_beam;
+      } else {
+        seq_score[b * beam_size + j] = score;
+        parent[b * beam_size + j] = -1;
+        ++finished;
       }
-      best = wave_first(best);
-      prev = best;
-      // a sentence always has at least beam_size proposals; guard the indices anyway
-      const int ori = best.i == kNoCand ? end_id : best.i;
-      int can_beam = ori / vocab;
-      const int can_vocab = ori % vocab;
-      if (can_beam >= beam_size) can_beam = 0;
-      const int* from = old_alive_seq + ((long)b * beam_size + can_beam) * max_step;
-      int* to = new_alive_seq + ((long)b * beam_size + j) * max_step;
-      for (int t = lane; t < max_step; t += 64)
-        to[t] = t > cur_step + 1 ? end_id : (t == cur_step + 1 ? can_vocab : from[t]);
-      if (lane == 0) {
-        if (can_vocab != end_id) {
-          seq_probs[b * beam_size + j] = (best.s - (float)b * kMinLogProb) / length_norm;
+    }
+  };
+  if (ncand <= 256) {
+    // up to four proposals per lane, held in registers as 64-bit keys (score as an
+    // order-preserving integer above 2^31 - 1 - id: "higher score first, lower id on ties" is
+    // an integer maximum); the picks are made first, without touching memory, then applied
+    auto dpp64 = [](unsigned long long x, auto ctrl) {
+      const unsigned l = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)x, decltype(ctrl)::value, 0xf, 0xf, false);
+      const unsigned h = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)(x >> 32), decltype(ctrl)::value, 0xf, 0xf, false);
+      return ((unsigned long long)h << 32) | l;
+    };
+    auto lane64 = [](unsigned long long x, int l) {
+      const unsigned lo32 = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)x, l);
+      const unsigned hi32 = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(x >> 32), l);
+      return ((unsigned long long)hi32 << 32) | lo32;
+    };
+    auto umax64 = [](unsigned long long a, unsigned long long b) { return a > b ? a : b; };
+    const int total = beam_size * max_step;
+    const bool staged = total <= 512;
+    for (int b = wid; b < batch; b += nw) {
+      const float* cs = top_score + (long)b * ncand;
+      const int* ci = top_idx + (long)b * ncand;
+      // the sentence's old sequences are requested together with the proposals and parked in
+      // LDS: the new sequences then cost no second trip to memory after the picks are known
+      int olds[8];
+      if (staged) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          olds[u] = old_alive_seq[(long)b * total + min(lane + 64 * u, total - 1)];
+      }
+      unsigned long long key[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int c = min(lane + 64 * q, ncand - 1);
+        const float sc = cs[c];
+        const int id = ci[c];
+        unsigned u = __builtin_bit_cast(unsigned, sc + 0.f);
+        u ^= (u >> 31) ? 0xffffffffu : 0x80000000u;
+        key[q] = (lane + 64 * q < ncand && id != kNoCand)
+                     ? (((unsigned long long)u << 32) | (unsigned)(0x7fffffff - id)) : 0ull;
+      }
+      unsigned long long bound = ~0ull, won = 0ull;  // lane j keeps pick j
+      for (int j = 0; j < beam_size; ++j) {
+        unsigned long long best = 0ull;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (key[q] < bound && key[q] > best) best = key[q];
+        best = umax64(best, dpp64(best, std::integral_constant<int, kDppXor1>()));
+        best = umax64(best, dpp64(best, std::integral_constant<int, kDppXor2>()));
+        best = umax64(best, dpp64(best, std::integral_constant<int, kDppHalfMirror>()));
+        best = umax64(best, dpp64(best, std::integral_constant<int, kDppMirror>()));
+        best = umax64(umax64(lane64(best, 0), lane64(best, 16)), umax64(lane64(best, 32), lane64(best, 48)));
+        if (lane == j) won = best;
+        bound = best;  // 0 once nothing is left: no key lies below it
+      }
+      if (staged) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) seq_lds[wid][lane + 64 * u] = olds[u];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+      // the picks applied (ker_refresh_result): all new sequences of the sentence in one
+      // flat loop, four independent elements per lane, then probabilities and scores
+      for (int x0 = 0; x0 < total; x0 += 256) {
+        int val[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int x = min(x0 + 64 * u + lane, total - 1);
+          const int j = x / max_step, t = x - j * max_step;
+          const unsigned long long k = __shfl(won, j);
+          const int ori = k == 0ull ? end_id : 0x7fffffff - (int)(unsigned)k;
+          int can_beam = ori / vocab;
+          const int can_vocab = ori - can_beam * vocab;
+          if (can_beam >= beam_size) can_beam = 0;
+          const int from = staged ? seq_lds[wid][can_beam * max_step + t]
+                                  : old_alive_seq[((long)b * beam_size + can_beam) * max_step + t];
+          val[u] = t > cur_step + 1 ? end_id : (t == cur_step + 1 ? can_vocab : from);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int x = x0 + 64 * u + lane;
+          if (x < total) new_alive_seq[(long)b * beam_size * max_step + x] = val[u];
+        }
+      }
+      if (lane < beam_size) {
+        const int j = lane;
+        const unsigned long long k = won;
+        unsigned u = (unsigned)(k >> 32);
+        u ^= (u >> 31) ? 0x80000000u : 0xffffffffu;
+        const float score = k == 0ull ? -INFINITY : __builtin_bit_cast(float, u);
+        const int ori = k == 0ull ? end_id : 0x7fffffff - (int)(unsigned)k;
+        if (ori % vocab != end_id) {
+          int can_beam = ori / vocab;
+          if (can_beam >= beam_size) can_beam = 0;
+          seq_probs[b * beam_size + j] = (score - (float)b * kMinLogProb) / length_norm;
           parent[b * beam_size + j] = can_beam;
         } else {
-          seq_score[b * beam_size + j] = best.s;
+          seq_score[b * beam_size + j] = score;
           parent[b * beam_size + j] = -1;
           ++finished;
         }
       }
     }
+  } else {
+    for (int b = wid; b < batch; b += nw) {
+      const float* cs = top_score + (long)b * ncand;
+      const int* ci = top_idx + (long)b * ncand;
+      ScoreIdx prev;
+      prev.s = INFINITY;
+      prev.i = -1;
+      for (int j = 0; j < beam_size; ++j) {
+        ScoreIdx best;
+        best.s = -INFINITY;
+        best.i = kNoCand;
+        for (int c = lane; c < ncand; c += 64) {
+          ScoreIdx x;
+          x.s = cs[c];
+          x.i = ci[c];
+          if (x.i != kNoCand && before(prev, x) && before(x, best)) best = x;
+        }
+        best = wave_first(best);
+        prev = best;
+        apply(b, j, best.s, best.i);
+      }
+    }
   }
+  for (int d = 32; d > 0; d >>= 1) finished += __shfl_xor(finished, d);  // lanes count their own picks
   if (lane == 0) fin_cnt[wid] = finished;
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -766,12 +1021,24 @@ beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ t
   }
 }
 
+// 4-byte words of the optional second workspace with which the per-row top-k is dealt to
+// several workgroups per row (0: the shape does not use one): per (row, part) beam_size
+// proposals (score, id).
+size_t beam_search_step_workspace_words(int batch_size, int beam_size, int vocab_size) {
+  if (batch_size <= 0 || beam_size <= 0 || vocab_size <= kBeamPartIds || vocab_size > 32 * 1024 ||
+      vocab_size % 16 != 0)
+    return 0;
+  const size_t parts = (size_t)(vocab_size + kBeamPartIds - 1) / kBeamPartIds;
+  return (size_t)batch_size * beam_size * parts * 2 * (size_t)beam_size;
+}
+
 template <typename T>
 int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_probs,
                          float* seq_score, const int* old_alive_seq, int* new_alive_seq,
                          float* top_score, int* top_idx, int* parent, int* num_finished,
                          float dequant_scale, int vocab_size, int max_step, float length_norm,
-                         int cur_step, int batch_size, int beam_size, int end_id, hipStream_t s) {
+                         int cur_step, int batch_size, int beam_size, int end_id, hipStream_t s,
+                         float* part_ws, size_t part_ws_words) {
   if (!logits || !logit_bias || !seq_probs || !seq_score || !old_alive_seq || !new_alive_seq ||
       !top_score || !top_idx || !parent || !num_finished || vocab_size <= 0 || batch_size <= 0 ||
       max_step <= 0 || cur_step < 0 || cur_step + 1 >= max_step)
@@ -785,7 +1052,22 @@ int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_p
   const bool vec = vocab_size % 16 == 0 &&
                    ((reinterpret_cast<uintptr_t>(logits) | reinterpret_cast<uintptr_t>(logit_bias)) &
                     15u) == 0;
-  if (vocab_size <= 32 * 1024 && vec)
+  const int rows = batch_size * beam_size;
+  const size_t need = beam_search_step_workspace_words(batch_size, beam_size, vocab_size);
+  int parts = 1;
+  if (vec && part_ws != nullptr && need != 0 && part_ws_words >= need && rows <= 65535 &&
+      (reinterpret_cast<uintptr_t>(part_ws) & 7u) == 0) {
+    // the row's ids dealt to several workgroups
+    parts = (vocab_size + kBeamPartIds - 1) / kBeamPartIds;
+    float* p_score = part_ws;
+    int* p_idx = reinterpret_cast<int*>(p_score + (size_t)rows * parts * beam_size);
+    beam_topk_part_kernel<T><<<dim3(parts, rows), 512, 0, s>>>(
+        logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, p_score, p_idx,
+        vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+    if (int rc = lsh_check_launch("beam_topk_part_kernel")) return rc;
+    top_score = p_score;
+    top_idx = p_idx;
+  } else if (vocab_size <= 32 * 1024 && vec)
     beam_topk_reg_kernel<T, true><<<batch_size * beam_size, 1024, 0, s>>>(
         logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score,
         top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
@@ -801,15 +1083,15 @@ int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_p
   beam_merge_kernel<<<1, 1024, 0, s>>>(top_score, top_idx, old_alive_seq, new_alive_seq,
                                        seq_probs, seq_score, parent, num_finished, batch_size,
                                        beam_size, vocab_size, max_step, cur_step, length_norm,
-                                       end_id);
+                                       end_id, parts);
   return lsh_check_launch("beam_merge_kernel");
 }
 template int beam_search_step_i8I<float>(const int8_t*, const float*, float*, float*, const int*,
                                          int*, float*, int*, int*, int*, float, int, int, float,
-                                         int, int, int, int, hipStream_t);
+                                         int, int, int, int, hipStream_t, float*, size_t);
 template int beam_search_step_i8I<__half>(const int8_t*, const __half*, float*, float*, const int*,
                                           int*, float*, int*, int*, int*, float, int, int, float,
-                                          int, int, int, int, hipStream_t);
+                                          int, int, int, int, hipStream_t, float*, size_t);
 
 // ---------------------------------------------------------------------------------
 // The search step for callers that cannot allocate device memory (code under HIP graph
@@ -864,7 +1146,7 @@ int beam_search_step_noalloc_i8I_f16(const int8_t* logits, const __half* logit_b
   return beam_search_step_i8I<__half>(logits, logit_bias, seq_probs, seq_score, old_alive_seq,
                                       new_alive_seq, top_score, top_idx, parent, num_finished,
                                       dequant_scale, vocab_size, max_step, length_norm, cur_step,
-                                      batch_size, beam_size, end_id, s);
+                                      batch_size, beam_size, end_id, s, nullptr, 0);
 }
 
 }  // namespace lsh

@@ -647,6 +647,26 @@ int lsh_ker_write_topk_result(const int* alive_seq, float* seq_score, int* res_s
 LSH_BEAM_STEP(lsh_beam_search_step_i8I_f16, __half, H)
 LSH_BEAM_STEP(lsh_beam_search_step_i8I_f32, float, F)
 #undef LSH_BEAM_STEP
+int64_t lsh_beam_search_step_workspace(int batch_size, int beam_size, int vocab_size) {
+  return (int64_t)beam_search_step_workspace_words(batch_size, beam_size, vocab_size) * 4;
+}
+#define LSH_BEAM_STEP_WS(NAME, TY, CAST_C)                                                     \
+  int NAME(const int8_t* logits, const void* logit_bias, float* seq_probs, float* seq_score,   \
+           const int* old_alive_seq, int* new_alive_seq, float* top_score, int* top_idx,       \
+           int* parent, int* num_finished, float dequant_scale, int vocab_size, int max_step,  \
+           float length_norm_v, int cur_step, int batch_size, int beam_size, int end_id,       \
+           void* workspace, int64_t workspace_bytes, lsh_stream_t stream) {                    \
+    if (workspace_bytes < 0) return lsh_fail(LSH_ERR_INVALID, #NAME ": negative workspace");   \
+    return beam_search_step_i8I<TY>(logits, CAST_C(logit_bias), seq_probs, seq_score,          \
+                                    old_alive_seq, new_alive_seq, top_score, top_idx, parent,  \
+                                    num_finished, dequant_scale, vocab_size, max_step,         \
+                                    length_norm_v, cur_step, batch_size, beam_size, end_id,    \
+                                    HS(stream), static_cast<float*>(workspace),                \
+                                    (size_t)workspace_bytes / 4);                              \
+  }
+LSH_BEAM_STEP_WS(lsh_beam_search_step_ws_i8I_f16, __half, H)
+LSH_BEAM_STEP_WS(lsh_beam_search_step_ws_i8I_f32, float, F)
+#undef LSH_BEAM_STEP_WS
 
 int lsh_beam_search_step_noalloc_i8I_f16(const int8_t* logits, const void* logit_bias,
                                          float* seq_probs, float* seq_score,

@@ -68,6 +68,13 @@ struct EpiI32 {
         if (n + i < N) p[i] = c[i];
     }
   }
+  // one element (the decode-step kernels give every thread one element of a 16 x 16 block)
+  struct Pre1 {};
+  __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
+  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1, const int8_t*,
+                                         int) const {
+    C[m * N + n] = acc;
+  }
   bool vec_ok(int N) const { return N % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
   static const char* name() { return "EpiI32"; }
 };
@@ -99,6 +106,12 @@ struct EpiI8 {
 #pragma unroll
     for (int i = 0; i < 16; ++i) q[i] = requant_acc(c[i], alpha);
     store16_i8(C + m * N + n, n, N, q, full);
+  }
+  struct Pre1 {};
+  __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
+  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1, const int8_t*,
+                                         int) const {
+    C[m * N + n] = (int8_t)requant_acc_fast(acc, alpha);
   }
   bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
   static const char* name() { return "EpiI8"; }
@@ -156,6 +169,27 @@ struct EpiDecQkvI8 {
     *reinterpret_cast<uint4*>(dst) = o;
     (void)N;
   }
+  // one element; its bias value is requested with the first weights
+  struct Pre1 {
+    __half b;
+  };
+  __device__ __forceinline__ Pre1 prefetch1(int n) const { return Pre1{bias[n]}; }
+  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1 pre, const int8_t*,
+                                         int) const {
+#pragma clang fp contract(off)
+    // the 16 columns of a block share part and head (dim_per_head % 16 == 0): divisions on the
+    // block's first column, which is the same in every lane
+    const int nb = __builtin_amdgcn_readfirstlane(n & ~15);
+    const int part = nb / hidden, ib = nb - part * hidden;
+    const int head = ib / dim_per_head, dim = ib - head * dim_per_head + (n & 15);
+    const float val = (float)requant_acc_fast(acc, alpha) * dequant_scale + __half2float(pre.b);
+    const int q = float2int8(val, quant_scale);
+    int8_t* dst = part == 0 ? new_q + m * hidden + ib + (n & 15)
+                            : (part == 1 ? new_k : new_v) +
+                                  ((m * head_num + head) * max_step + step_id) * dim_per_head + dim;
+    *dst = (int8_t)q;
+    (void)N;
+  }
   bool vec_ok(int) const { return true; }
   static const char* name() { return "EpiDecQkvI8"; }
 };
@@ -195,6 +229,20 @@ struct EpiEncdecQF16 {
     }
     *reinterpret_cast<half8_t*>(dst) = lo;
     *reinterpret_cast<half8_t*>(dst + 8) = hi;
+    (void)N;
+  }
+  struct Pre1 {
+    __half b;
+  };
+  __device__ __forceinline__ Pre1 prefetch1(int n) const { return Pre1{bias[n]}; }
+  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1 pre, const int8_t*,
+                                         int) const {
+    const int nb = __builtin_amdgcn_readfirstlane(n & ~15);
+    const int head = nb / dim_per_head, dim = nb - head * dim_per_head + (n & 15);
+    const long batch_id = m / beam_size, beam_id = m - batch_id * beam_size;
+    new_q[((batch_id * head_num + head) * beam_size + beam_id) * dim_per_head + dim] =
+        __float2half_rn(dequant_add_bias_h(requant_acc_fast(acc, alpha), dequant_scale,
+                                           __half2float(pre.b)));
     (void)N;
   }
   bool vec_ok(int) const { return true; }
@@ -288,6 +336,14 @@ struct EpiLutI8 {
       q[i] = tab[(n_local + i) * 256 + requant_acc_fast(c[i], alpha) + 128];
     store16_i8(C + m * N + n, n, N, q, full);
   }
+  // one element, the table rows of the workgroup's columns staged in LDS (n_local: the
+  // element's column among them)
+  struct Pre1 {};
+  __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
+  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1, const int8_t* tab,
+                                         int n_local) const {
+    C[m * N + n] = tab[n_local * 256 + requant_acc_fast(acc, alpha) + 128];
+  }
   bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
   static const char* name() { return "EpiLutI8"; }
 };
@@ -343,6 +399,11 @@ struct EpiQkvF16 {
 // Epilogues with operands that can be requested before the product is known (decode-step
 // kernel): a bias slice kept in registers, or the table rows of the workgroup's columns in LDS.
 struct EpiNoPre {};
+// epilogues that can store one element at a time (what the decode-step kernels use)
+template <typename Epi, typename = void>
+struct has_store1 : std::false_type {};
+template <typename Epi>
+struct has_store1<Epi, std::void_t<typename Epi::Pre1>> : std::true_type {};
 template <typename Epi>
 struct epi_pre {
   typedef EpiNoPre type;
@@ -1200,8 +1261,16 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
   // epilogue thread t: row t % (16 MB), column block t / (16 MB) (threads beyond 32 MB idle)
   const int em = tid % (16 * MB), eblk = (tid / (16 * MB)) & (NB - 1);
   // What the epilogue reads besides the product travels with the weights.
+  constexpr bool kOne = has_store1<Epi>::value;  // every thread stores one element per block
+  const int ecol = tid & 15, erow = tid >> 4;    // ... element (erow, ecol) of a 16 x 16 block
   typename epi_pre<Epi>::type pre;
-  if constexpr (epi_pre<Epi>::value) pre = epi.prefetch(max(min(n0 + 16 * eblk, N - 16), 0));
+  typename std::conditional<kOne, Epi, EpiI32>::type::Pre1 pre1[NB];
+  if constexpr (kOne) {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) pre1[b] = epi.prefetch1(min(n0 + 16 * b + ecol, N - 1));
+  } else if constexpr (epi_pre<Epi>::value) {
+    pre = epi.prefetch(max(min(n0 + 16 * eblk, N - 16), 0));
+  }
   uint4 tab0, tab1;
   if constexpr (kLut) {
     const int8_t* tp = epi_lut(epi) + (long)min(n0 + ((tid >> 3) & (16 * NB - 1)), N - 1) * 256 + (tid & 7) * 32;
@@ -1256,7 +1325,24 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
     }
   }
   __syncthreads();
-  if (tid < 16 * NB * MB) {
+  if constexpr (kOne) {
+    // A wavefront that walks 16 columns of a row in a row of instructions runs as long as the
+    // rest of the kernel: the instructions of one wavefront, not the memory, bound a launch of
+    // this size.  So every thread finishes one element of each 16 x 16 block: four LDS reads,
+    // three adds, the epilogue of one value, one store; 16 lanes write 16 neighbouring columns.
+    const int src = (ecol >> 2) * 16 + erow, r = ecol & 3;  // lane and register that held it
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const int m = m0 + 16 * i + erow, n = n0 + 16 * b + ecol;
+        if (m < M && n < N) {
+          const int acc = (red[0][i][b][r][src] + red[1][i][b][r][src]) +
+                          (red[2][i][b][r][src] + red[3][i][b][r][src]);
+          epi.store1(m + (long)part * M, n, N, acc, pre1[b], tab, 16 * b + ecol);
+        }
+      }
+  } else if (tid < 16 * NB * MB) {
     const int n = n0 + 16 * eblk;
     if (m0 + em < M && n < N) {
       v16i c;

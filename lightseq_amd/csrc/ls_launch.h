@@ -297,7 +297,11 @@ int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_p
                          float* seq_score, const int* old_alive_seq, int* new_alive_seq,
                          float* top_score, int* top_idx, int* parent, int* num_finished,
                          float dequant_scale, int vocab_size, int max_step, float length_norm,
-                         int cur_step, int batch_size, int beam_size, int end_id, hipStream_t s);
+                         int cur_step, int batch_size, int beam_size, int end_id, hipStream_t s,
+                         float* part_ws = nullptr, size_t part_ws_words = 0);
+// 4-byte words of the optional workspace `part_ws` with which the per-row top-k of the step is
+// dealt to several workgroups per row (0: this shape runs one workgroup per row either way)
+size_t beam_search_step_workspace_words(int batch_size, int beam_size, int vocab_size);
 // the same step with its proposal workspace in a static device array (allocates nothing)
 int beam_search_step_noalloc_i8I_f16(const int8_t* logits, const __half* logit_bias,
                                      float* seq_probs, float* seq_score, const int* old_alive_seq,

@@ -104,6 +104,9 @@ void QuantDecoder::init_buffer() {
   if (!_p_d_alive_seq_score) _p_d_alive_seq_score = _alive_seq_score_own.get();
   _top_score.alloc(rows * beam);
   _top_idx.alloc(rows * beam);
+  // the per-row top-k dealt to several workgroups per row, where the vocabulary allows
+  if (const size_t words = beam_search_step_workspace_words(_max_batch_size, beam, _tw._trg_vocab_size))
+    _topk_part_ws.alloc(words);
   _parent.alloc(rows);
   _num_finished.alloc(1);
   CHECK_GPU_ERROR(hipHostMalloc(reinterpret_cast<void**>(&_h_num_finished), sizeof(int)));
@@ -464,7 +467,8 @@ void QuantDecoder::beam_search() {
       _logits.get(), _logit_bias.get(), _alive_seq_probs.get(), _p_d_alive_seq_score, alive,
       alive_new, _top_score.get(), _top_idx.get(), _parent.get(), _num_finished.get(),
       _logits_clip_max / _quant_range, _tw._trg_vocab_size, _tw._max_step,
-      _h_length_norm[_cur_step], _cur_step, _batch_size, _tw._beam_size, _tw._end_id, _stream));
+      _h_length_norm[_cur_step], _cur_step, _batch_size, _tw._beam_size, _tw._end_id, _stream,
+      _topk_part_ws.get(), _topk_part_ws.size()));
   if (_rec_alive && _cur_step < _rec_max_steps)
     CHECK_GPU_ERROR(hipMemcpyAsync(
         _rec_alive + (size_t)_cur_step * _step_token_num * _tw._max_step, alive_new,

@@ -96,7 +96,7 @@ class QuantDecoder {
   int _cache_cur = 0;
   DeviceBuffer<int> _alive_seq[2];
   int _alive_cur = 0;
-  DeviceBuffer<float> _alive_seq_probs, _alive_seq_score_own, _top_score;
+  DeviceBuffer<float> _alive_seq_probs, _alive_seq_score_own, _top_score, _topk_part_ws;
   DeviceBuffer<int> _top_idx, _parent, _num_finished;
   // weights
   DeviceBuffer<int8_t> _int8_trg_emb;  // [vocab, H]: embedding rows and logits kernel

@@ -7,6 +7,8 @@ stream, ``max_thread_per_block`` is accepted and ignored (the HIP kernels choose
 their own launch shape) and COL32 flags must stay False.  The storage type T is
 taken from the dtype of the T-typed tensors (float16 / float32).
 """
+import ctypes
+
 import torch
 
 from . import lib
@@ -423,6 +425,29 @@ def beam_search_step_i8I(logits, logit_bias, seq_probs, seq_score, old_alive_seq
          ptr(seq_probs), ptr(seq_score), ptr(old_alive_seq), ptr(new_alive_seq), ptr(top_score),
          ptr(top_idx), ptr(parent), ptr(num_finished), dequant_scale, vocab_size, max_step,
          length_norm_value, cur_step, batch_size, beam_size, end_id, current_stream())
+
+
+def beam_search_step_workspace(batch_size, beam_size, vocab_size):
+    """Bytes of the optional second workspace of :func:`beam_search_step_ws_i8I` (0: unused)."""
+    f = lib.load().lsh_beam_search_step_workspace
+    f.restype = ctypes.c_int64
+    return int(f(int(batch_size), int(beam_size), int(vocab_size)))
+
+
+def beam_search_step_ws_i8I(logits, logit_bias, seq_probs, seq_score, old_alive_seq, new_alive_seq,
+                            top_score, top_idx, parent, num_finished, dequant_scale, vocab_size,
+                            max_step, length_norm_value, cur_step, batch_size, beam_size, end_id,
+                            workspace):
+    """:func:`beam_search_step_i8I` with the per-row top-k dealt to several workgroups per row
+    (``workspace``: a tensor of :func:`beam_search_step_workspace` bytes, or None)."""
+    _dev(logits, logit_bias, seq_probs, seq_score, old_alive_seq, new_alive_seq, top_score,
+         top_idx, parent, num_finished, workspace)
+    nbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    call("lsh_beam_search_step_ws_i8I" + _suffix(logit_bias), ptr(logits), ptr(logit_bias),
+         ptr(seq_probs), ptr(seq_score), ptr(old_alive_seq), ptr(new_alive_seq), ptr(top_score),
+         ptr(top_idx), ptr(parent), ptr(num_finished), dequant_scale, vocab_size, max_step,
+         length_norm_value, cur_step, batch_size, beam_size, end_id, ptr(workspace), nbytes,
+         current_stream())
 
 
 def beam_search_step_noalloc_i8I(logits, logit_bias, seq_probs, seq_score, old_alive_seq,

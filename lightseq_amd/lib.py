@@ -91,6 +91,7 @@ _SIGNATURES = {
     "lsh_ker_write_trg_tokenid_neg_penalty": (False, "ppp" + "iiiiii" + "s"),
     "lsh_ker_write_topk_result": (False, "ppp" + "iiiiii" + "s"),
     "lsh_beam_search_step_i8I": (True, "pppppppppp" + "f" + "ii" + "f" + "iiii" + "s"),
+    "lsh_beam_search_step_ws_i8I": (True, "pppppppppp" + "f" + "ii" + "f" + "iiii" + "pl" + "s"),
     "lsh_beam_search_step_noalloc_i8I_f16": (False, "pppppppp" + "f" + "ii" + "f" + "iiii" + "s"),
     "lsh_refresh_cache_by_parent_i8": (False, "iis" + "ppppp" + "l" + "iiiii"),
     # GPT path

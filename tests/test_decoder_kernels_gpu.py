@@ -391,6 +391,60 @@ def test_beam_search_step(oracle, rng, dtype, tie_bias, batch, beam, vocab, max_
     np.testing.assert_array_equal(to_np(vn), wv)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tie_bias", [False, True])
+@pytest.mark.parametrize("batch,beam,vocab,cur_step", [(2, 8, 32000, 17), (16, 4, 32000, 9), (2, 4, 32768, 2),
+                                                       (3, 2, 8208, 0), (1, 32, 16384, 4), (2, 4, 9000 - 8, 3),
+                                                       (2, 4, 5008, 3), (1, 4, 40000, 2)])
+def test_beam_search_step_with_the_rows_dealt_to_several_workgroups(oracle, rng, dtype, tie_bias, batch,
+                                                                     beam, vocab, cur_step):
+    """lsh_beam_search_step_ws_i8I picks the beams the reference pipeline picks and the beams of
+    lsh_beam_search_step_i8I (vocabularies of 8208 .. 32768 ids run the split kernels, the last
+    two cases fall back), finished beams included."""
+    end_id, max_step = 3, 24
+    logits, bias, probs, score, alive, _ = _beam_state(rng, batch, beam, vocab, max_step, cur_step,
+                                                       end_id, dtype, tie_bias=tie_bias)
+    logits[::2, end_id] = 100
+    rows = batch * beam
+    dq = 2.5 / 127
+    ln = oracle.length_norm(cur_step + 1, 0.6)
+    s_idx, s_sc, s_num, w_alive, w_probs, w_score, w_fin = _oracle_step(
+        oracle, logits, bias, probs, score, alive, dq, ln, cur_step, beam, end_id, vocab)
+    nbytes = _k().beam_search_step_workspace(batch, beam, vocab)
+    assert (nbytes > 0) == (8192 < vocab <= 32768 and vocab % 16 == 0)
+    if nbytes:
+        assert nbytes == rows * -(-vocab // 8192) * 2 * beam * 4
+    out = []
+    for ws in (torch.zeros(max(nbytes, 8) // 4, dtype=torch.float32, device=DEV), None):
+        new_alive = torch.zeros(rows, max_step, dtype=torch.int32, device=DEV)
+        p_d, s_d = to_dev(probs), to_dev(score)
+        top_s = torch.zeros(rows * beam, dtype=torch.float32, device=DEV)
+        top_i = torch.zeros(rows * beam, dtype=torch.int32, device=DEV)
+        parent = torch.full((rows,), -7, dtype=torch.int32, device=DEV)
+        fin = torch.zeros(1, dtype=torch.int32, device=DEV)
+        _k().beam_search_step_ws_i8I(to_dev(logits), to_dev(bias), p_d, s_d, to_dev(alive), new_alive,
+                                     top_s, top_i, parent, fin, dq, vocab, max_step, ln, cur_step, batch,
+                                     beam, end_id, ws)
+        out.append((to_np(new_alive), to_np(parent), int(to_np(fin)[0]), to_np(p_d), to_np(s_d)))
+    (a_alive, a_parent, a_fin, a_p, a_s), (b_alive, b_parent, b_fin, b_p, b_s) = out
+    np.testing.assert_array_equal(a_alive, w_alive)
+    assert a_fin == w_fin
+    picks = np.stack([s_idx[s_num[1 + b * beam] + np.arange(beam)] for b in range(batch)])
+    want_parent = np.where(picks % vocab == end_id, -1, picks // vocab).reshape(-1)
+    np.testing.assert_array_equal(a_parent, want_parent)
+    live = want_parent >= 0
+    np.testing.assert_allclose(a_p[live], w_probs[live], rtol=2e-6, atol=2e-4)
+    np.testing.assert_allclose(a_s[~live], w_score[~live], rtol=2e-6, atol=2e-4)
+    np.testing.assert_array_equal(a_p[~live], probs[~live])
+    np.testing.assert_array_equal(a_s[live], score[live])
+    # against the one-workgroup-per-row step: same sequences, parents, count; scores to the last place
+    np.testing.assert_array_equal(a_alive, b_alive)
+    np.testing.assert_array_equal(a_parent, b_parent)
+    assert a_fin == b_fin
+    np.testing.assert_allclose(a_p, b_p, rtol=1e-6, atol=1e-5)
+    np.testing.assert_allclose(a_s, b_s, rtol=1e-6, atol=1e-5)
+
+
 @pytest.mark.parametrize("batch,beam,max_step,out_len", [(3, 4, 16, 9), (8, 4, 32, 31), (2, 1, 8, 1),
                                                          (5, 8, 16, 15)])
 def test_output_writers(oracle, rng, batch, beam, max_step, out_len):
