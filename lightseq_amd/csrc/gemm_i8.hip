@@ -117,6 +117,17 @@ struct EpiI8 {
   static const char* name() { return "EpiI8"; }
 };
 
+// n / d for 0 <= n < 2^24, d > 0, with inv = 1.0f / d from the host: the float product is
+// within one of the quotient, the remainder decides.  A handful of instructions where the
+// integer division is about forty -- in kernels whose length is their instruction count.
+__device__ __forceinline__ int div_by(int n, int d, float inv) {
+  int q = (int)((float)n * inv);
+  const int r = n - q * d;
+  if (r >= d) ++q;
+  if (r < 0) --q;
+  return q;
+}
+
 // Decode-step QKV product followed by ker_arrange_decself_qkv_i8I_i8O
 // (inference/kernels/transformerKernels_int8.cc.cu:1432-1513; call sites
 // model/quant_decoder.cc.cu:660-674, model/quant_gpt_encoder.cc.cu:640-653): the int8 code
@@ -129,6 +140,7 @@ struct EpiDecQkvI8 {
   const __half* bias;
   float alpha, dequant_scale, quant_scale;
   int hidden, head_num, dim_per_head, max_step, step_id;
+  float inv_hidden, inv_dim;  // 1 / hidden, 1 / dim_per_head (for store1)
   // the 16 bias values of columns n .. n + 15: they do not depend on the product, so the
   // decode-step kernel requests them with its first weights
   struct Pre {
@@ -180,8 +192,8 @@ struct EpiDecQkvI8 {
     // the 16 columns of a block share part and head (dim_per_head % 16 == 0): divisions on the
     // block's first column, which is the same in every lane
     const int nb = __builtin_amdgcn_readfirstlane(n & ~15);
-    const int part = nb / hidden, ib = nb - part * hidden;
-    const int head = ib / dim_per_head, dim = ib - head * dim_per_head + (n & 15);
+    const int part = div_by(nb, hidden, inv_hidden), ib = nb - part * hidden;
+    const int head = div_by(ib, dim_per_head, inv_dim), dim = ib - head * dim_per_head + (n & 15);
     const float val = (float)requant_acc_fast(acc, alpha) * dequant_scale + __half2float(pre.b);
     const int q = float2int8(val, quant_scale);
     int8_t* dst = part == 0 ? new_q + m * hidden + ib + (n & 15)
@@ -203,6 +215,7 @@ struct EpiEncdecQF16 {
   const __half* bias;
   float alpha, dequant_scale;
   int beam_size, head_num, dim_per_head;
+  float inv_beam, inv_dim;  // 1 / beam_size, 1 / dim_per_head (for store1)
   struct Pre {  // the bias of columns n .. n + 15, requested ahead of the product
     half8_t b0, b1;
   };
@@ -238,9 +251,9 @@ struct EpiEncdecQF16 {
   __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1 pre, const int8_t*,
                                          int) const {
     const int nb = __builtin_amdgcn_readfirstlane(n & ~15);
-    const int head = nb / dim_per_head, dim = nb - head * dim_per_head + (n & 15);
-    const long batch_id = m / beam_size, beam_id = m - batch_id * beam_size;
-    new_q[((batch_id * head_num + head) * beam_size + beam_id) * dim_per_head + dim] =
+    const int head = div_by(nb, dim_per_head, inv_dim), dim = nb - head * dim_per_head + (n & 15);
+    const int batch_id = div_by((int)m, beam_size, inv_beam), beam_id = (int)m - batch_id * beam_size;
+    new_q[(((long)batch_id * head_num + head) * beam_size + beam_id) * dim_per_head + dim] =
         __float2half_rn(dequant_add_bias_h(requant_acc_fast(acc, alpha), dequant_scale,
                                            __half2float(pre.b)));
     (void)N;
@@ -1427,7 +1440,23 @@ gemm_i8_skinny16_wide_kernel(const int8_t* __restrict__ A, const int8_t* __restr
 #pragma unroll
         for (int r = 0; r < 4; ++r) rd[wave][i][b][r][lane] = acc[i][b][r];
     __syncthreads();
-    if (tid < 32 * MB) {
+    if constexpr (has_store1<Epi>::value && MB <= 2) {
+      // one element per thread and 16 x 16 block (see gemm_i8_skinny16_kernel; with 64 rows
+      // that is eight elements per thread and pair, no shorter than 16 in half the threads)
+      const int ecol = tid & 15, erow = tid >> 4;
+      const int src = (ecol >> 2) * 16 + erow, r = ecol & 3;
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const int m = 16 * i + erow, n = n00 + 32 * pair + 16 * b + ecol;
+          if (m < M && n < N) {
+            const int acc1 = (rd[0][i][b][r][src] + rd[1][i][b][r][src]) +
+                             (rd[2][i][b][r][src] + rd[3][i][b][r][src]);
+            epi.store1(m, n, N, acc1, typename Epi::Pre1{}, nullptr, 0);
+          }
+        }
+    } else if (tid < 32 * MB) {
       const int n = n00 + 32 * pair + 16 * eblk;
       if (em < M && n < N) {
         v16i c;
@@ -1882,7 +1911,8 @@ int gemm_i8_decself_qkv_i8o(const int8_t* A, const int8_t* W, const __half* qkv_
                     "int8 gemm (decoder qkv): needs dim_per_head % 16 == 0 and aligned outputs");
   return dispatch(A, W,
                   EpiDecQkvI8{new_q, new_k, new_v, qkv_bias, alpha, dequant_scale, quant_scale,
-                              hidden, head_num, d, max_step, step_id},
+                              hidden, head_num, d, max_step, step_id, 1.0f / (float)hidden,
+                              1.0f / (float)d},
                   step_token_num, 3 * hidden, K, s);
 }
 
@@ -1897,7 +1927,9 @@ int gemm_i8_encdec_q_f16(const int8_t* A, const int8_t* W, const __half* q_bias,
       ((reinterpret_cast<uintptr_t>(q_bias) | reinterpret_cast<uintptr_t>(new_q)) & 15u) != 0)
     return lsh_fail(LSH_ERR_UNSUPPORTED,
                     "int8 gemm (cross-attention q): needs dim_per_head % 16 == 0 and aligned output");
-  return dispatch(A, W, EpiEncdecQF16{new_q, q_bias, alpha, dequant_scale, beam_size, head_num, d},
+  return dispatch(A, W,
+                  EpiEncdecQF16{new_q, q_bias, alpha, dequant_scale, beam_size, head_num, d,
+                                1.0f / (float)beam_size, 1.0f / (float)d},
                   step_token_num, hidden, K, s);
 }
 

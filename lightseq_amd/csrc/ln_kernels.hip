@@ -482,7 +482,7 @@ __global__ void ln_rows_generic_kernel(const AccT* __restrict__ gemm_out, T* res
 // % 4 == 0): the layer norm of the decode steps, where a launch lasts a few microseconds and
 // every dependent step inside it shows.  So: no integer division and no branch before the loads
 // (indices are clamped, not predicated, which also lets the kernel arguments arrive in one
-// batch), every load -- parameters and up to eight accumulator planes -- requested before the
+// batch), every load -- parameters and up to four accumulator planes -- requested before the
 // first is used, sums over a wavefront by DPP permutations and lane reads instead of LDS
 // permutes, and one barrier per reduction.
 // Order of a row sum: (x0 + x1) + (x2 + x3) per lane; lanes of a quad, the quads of a row of
@@ -505,41 +505,65 @@ ln_row_wg_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
     v = wave_sum_dpp(v);
     if (lane == 0) r[wid] = v;
     __syncthreads();
+    // ascending order, without a loop (wpr <= 4)
     float t = r[0];
-    for (int i = 1; i < wpr; ++i) t += r[i];
+    const float r1 = r[1], r2 = r[2], r3 = r[3];
+    if (wpr > 1) t += r1;
+    if (wpr > 2) t += r2;
+    if (wpr > 3) t += r3;
     return t;
   };
   float g[4], b[4], rb[4] = {0.f, 0.f, 0.f, 0.f}, r[4], c[4] = {0.f, 0.f, 0.f, 0.f};
   ld4(residual, base + e, r);
+  // every load of the kernel is requested before the first value is used (the parameters
+  // before the accumulator planes, whose sums wait for them); optional operands through a
+  // pointer that is always valid, dropped afterwards: a load inside a branch is followed by
+  // its wait, one memory round trip after the other
+  const bool has_rb = MODE != kLnResOut && residual_bias != nullptr;
+  const bool has_cs = MODE != kLnFirst && colsum != nullptr;
+  auto g_raw = ld4_raw(scale, e), b_raw = ld4_raw(bias, e);
+  auto rb_raw = ld4_raw(has_rb ? residual_bias : scale, e);
+  auto c_raw = ld4_raw(has_cs ? colsum : scale, e);
   float a[4] = {0.f, 0.f, 0.f, 0.f};
   if (MODE != kLnFirst) {
     if constexpr (sizeof(AccT) == 4) {
-      // up to eight planes in flight together (integer sums: any order gives the same bits); a
-      // plane index beyond the last is clamped for the load and its value dropped
-      int4 m[8];
+      // up to four planes in flight together (what the decode-step products write; integer
+      // sums: any order gives the same bits); a plane index beyond the last is clamped for the
+      // load and its value dropped
+      int4 m[4];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < 4; ++u)
         m[u] = *reinterpret_cast<const int4*>(gemm_out + (long)min(u, nparts - 1) * part_stride +
                                               base + e);
+      pin4(g_raw, b_raw, rb_raw, c_raw);  // (requested ahead of the planes: they are here first)
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        asm volatile("" : "+v"(m[u].x), "+v"(m[u].y), "+v"(m[u].z), "+v"(m[u].w));
       int4 acc = m[0];
 #pragma unroll
-      for (int u = 1; u < 8; ++u)
-        if (u < nparts) {
-          acc.x += m[u].x; acc.y += m[u].y; acc.z += m[u].z; acc.w += m[u].w;
-        }
-      for (int p = 8; p < nparts; ++p) {
+      for (int u = 1; u < 4; ++u) {
+        const bool on_u = u < nparts;
+        acc.x += on_u ? m[u].x : 0; acc.y += on_u ? m[u].y : 0;
+        acc.z += on_u ? m[u].z : 0; acc.w += on_u ? m[u].w : 0;
+      }
+      for (int p = 4; p < nparts; ++p) {
         const int4 t = *reinterpret_cast<const int4*>(gemm_out + (long)p * part_stride + base + e);
         acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
       }
       a[0] = (float)acc.x; a[1] = (float)acc.y; a[2] = (float)acc.z; a[3] = (float)acc.w;
     } else {
       ld4_acc(gemm_out, base + e, a);
+      pin4(g_raw, b_raw, rb_raw, c_raw);
     }
+  } else {
+    pin4(g_raw, b_raw, rb_raw, c_raw);
   }
-  ld4(scale, e, g);
-  ld4(bias, e, b);
-  if (MODE != kLnResOut && residual_bias != nullptr) ld4(residual_bias, e, rb);
-  if (MODE != kLnFirst && colsum != nullptr) ld4(colsum, e, c);
+  cvt4(g_raw, g);
+  cvt4(b_raw, b);
+  cvt4(rb_raw, rb);
+  cvt4(c_raw, c);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) rb[k] = has_rb ? rb[k] : 0.f;
   float x[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {

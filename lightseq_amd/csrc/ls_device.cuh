@@ -154,6 +154,36 @@ __device__ __forceinline__ void ld4(const __half* p, long i, float (&o)[4]) {
 #pragma unroll
   for (int k = 0; k < 4; ++k) o[k] = __half2float(t.v[k]);
 }
+// Four consecutive T as raw words, to be converted after pin4(): between the two the caller
+// requests whatever else it loads.  pin4() makes the words opaque to the compiler, which
+// otherwise sinks a load whose values are used under a condition into that branch, where it
+// is followed by its wait -- one memory round trip after the other.
+struct Raw4F { float4 v; };
+struct Raw4H { uint2 v; };
+__device__ __forceinline__ Raw4F ld4_raw(const float* p, long i) {
+  return Raw4F{*reinterpret_cast<const float4*>(p + i)};
+}
+__device__ __forceinline__ Raw4H ld4_raw(const __half* p, long i) {
+  return Raw4H{*reinterpret_cast<const uint2*>(p + i)};
+}
+__device__ __forceinline__ void pin4(Raw4F& a, Raw4F& b, Raw4F& c, Raw4F& d) {
+  asm volatile("" : "+v"(a.v.x), "+v"(a.v.y), "+v"(a.v.z), "+v"(a.v.w), "+v"(b.v.x), "+v"(b.v.y),
+               "+v"(b.v.z), "+v"(b.v.w), "+v"(c.v.x), "+v"(c.v.y), "+v"(c.v.z), "+v"(c.v.w),
+               "+v"(d.v.x), "+v"(d.v.y), "+v"(d.v.z), "+v"(d.v.w));
+}
+__device__ __forceinline__ void pin4(Raw4H& a, Raw4H& b, Raw4H& c, Raw4H& d) {
+  asm volatile("" : "+v"(a.v.x), "+v"(a.v.y), "+v"(b.v.x), "+v"(b.v.y), "+v"(c.v.x), "+v"(c.v.y),
+               "+v"(d.v.x), "+v"(d.v.y));
+}
+__device__ __forceinline__ void cvt4(const Raw4F& r, float (&o)[4]) {
+  o[0] = r.v.x; o[1] = r.v.y; o[2] = r.v.z; o[3] = r.v.w;
+}
+__device__ __forceinline__ void cvt4(const Raw4H& r, float (&o)[4]) {
+  half4_t t;
+  __builtin_memcpy(&t, &r.v, sizeof(t));
+#pragma unroll
+  for (int k = 0; k < 4; ++k) o[k] = __half2float(t.v[k]);
+}
 __device__ __forceinline__ void st4(float* p, long i, const float (&o)[4]) {
   *reinterpret_cast<float4*>(p + i) = make_float4(o[0], o[1], o[2], o[3]);
 }
