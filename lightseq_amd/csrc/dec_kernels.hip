@@ -672,6 +672,9 @@ encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict_
     const int j = min(u * KPW + grp, seq_len - 1);
     vv[u].u = *reinterpret_cast<const uint4*>(vb + (long)j * D);
   }
+  // every load is requested before the first product: left alone the scheduler moves half of
+  // the value loads behind the soft-max, a second trip to memory in a kernel of one
+  __builtin_amdgcn_sched_barrier(0);
   float val[UN];
   float mx = kFloatInfNeg;
 #pragma unroll

@@ -170,6 +170,58 @@ __device__ __forceinline__ void st8(__half* p, long i, const float (&o)[8]) {
   for (int k = 0; k < 8; ++k) t.v[k] = __float2half_rn(o[k]);
   *reinterpret_cast<half8_t*>(p + i) = t;
 }
+// Eight consecutive elements as raw words (converted after every load of the row has been
+// requested) and the statement that makes the words opaque to the compiler, which otherwise
+// sinks a load into the branch that uses its values, where it is followed by its wait.
+struct Raw8F { float4 a, b; };
+struct Raw8H { uint4 a; };
+struct Raw8I { int4 a, b; };
+struct Raw8C { uint2 a; };
+__device__ __forceinline__ Raw8F ld8_raw(const float* p, long i) {
+  return Raw8F{*reinterpret_cast<const float4*>(p + i), *reinterpret_cast<const float4*>(p + i + 4)};
+}
+__device__ __forceinline__ Raw8H ld8_raw(const __half* p, long i) {
+  return Raw8H{*reinterpret_cast<const uint4*>(p + i)};
+}
+__device__ __forceinline__ Raw8I ld8_raw(const int32_t* p, long i) {
+  return Raw8I{*reinterpret_cast<const int4*>(p + i), *reinterpret_cast<const int4*>(p + i + 4)};
+}
+__device__ __forceinline__ Raw8C ld8_raw(const int8_t* p, long i) {
+  return Raw8C{*reinterpret_cast<const uint2*>(p + i)};
+}
+__device__ __forceinline__ void pin8(Raw8F& r) {
+  asm volatile("" : "+v"(r.a.x), "+v"(r.a.y), "+v"(r.a.z), "+v"(r.a.w), "+v"(r.b.x), "+v"(r.b.y),
+               "+v"(r.b.z), "+v"(r.b.w));
+}
+__device__ __forceinline__ void pin8(Raw8H& r) {
+  asm volatile("" : "+v"(r.a.x), "+v"(r.a.y), "+v"(r.a.z), "+v"(r.a.w));
+}
+__device__ __forceinline__ void pin8(Raw8I& r) {
+  asm volatile("" : "+v"(r.a.x), "+v"(r.a.y), "+v"(r.a.z), "+v"(r.a.w), "+v"(r.b.x), "+v"(r.b.y),
+               "+v"(r.b.z), "+v"(r.b.w));
+}
+__device__ __forceinline__ void pin8(Raw8C& r) { asm volatile("" : "+v"(r.a.x), "+v"(r.a.y)); }
+__device__ __forceinline__ void cvt8(const Raw8F& r, float (&o)[8]) {
+  o[0] = r.a.x; o[1] = r.a.y; o[2] = r.a.z; o[3] = r.a.w;
+  o[4] = r.b.x; o[5] = r.b.y; o[6] = r.b.z; o[7] = r.b.w;
+}
+__device__ __forceinline__ void cvt8(const Raw8H& r, float (&o)[8]) {
+  half8_t t;
+  __builtin_memcpy(&t, &r.a, sizeof(t));
+#pragma unroll
+  for (int k = 0; k < 8; ++k) o[k] = __half2float(t.v[k]);
+}
+__device__ __forceinline__ void cvt8(const Raw8I& r, int (&o)[8]) {
+  o[0] = r.a.x; o[1] = r.a.y; o[2] = r.a.z; o[3] = r.a.w;
+  o[4] = r.b.x; o[5] = r.b.y; o[6] = r.b.z; o[7] = r.b.w;
+}
+__device__ __forceinline__ void cvt8(const Raw8C& r, float (&o)[8]) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    o[k] = (float)unpack_i8(r.a.x, k);
+    o[4 + k] = (float)unpack_i8(r.a.y, k);
+  }
+}
 template <int LPR>
 __device__ __forceinline__ float row_sum(float v) {
 #pragma unroll
@@ -192,34 +244,57 @@ ln_rows8_row(int row, bool live, int sub, const AccT* __restrict__ gemm_out, T* 
   const long base = (long)(live ? row : 0) * hidden;
 
   float x[ITER][8];
-  // scale, bias and residual bias travel with the first round of loads, so the kernel has
-  // one global-memory round trip before its reductions and none after
-  float gs[ITER][8], bs[ITER][8], rbs[ITER][8];
+  // Every load of the row -- parameters, residual, accumulator, column sums -- is requested
+  // before the first value is used: no branch around a load (columns beyond the row and rows
+  // beyond the tensor are clamped, optional operands read through a pointer that is always
+  // valid, and what they bring is dropped), a scheduling barrier after the last request, and
+  // only then the statements that make the values visible to the arithmetic.  Written with
+  // conditions around the loads, the compiler put each load next to its use: six to nine
+  // memory round trips in a row instead of one.
+  const bool has_rb = MODE != kLnResOut && residual_bias != nullptr;
+  const bool has_cs = MODE != kLnFirst && colsum != nullptr;
+  const bool own_res = !(sizeof(T) == 2 && pre_res != nullptr);
+  const T* rbp = has_rb ? residual_bias : scale;
+  const T* csp = has_cs ? colsum : scale;
+  decltype(ld8_raw(scale, 0)) g_raw[ITER], b_raw[ITER], rb_raw[ITER], cs_raw[ITER], r_raw[ITER];
+  decltype(ld8_raw(gemm_out, 0)) a_raw[ITER];
 #pragma unroll
   for (int it = 0; it < ITER; ++it) {
-    const int e = (it * LPR + sub) * 8;
-    if (e < hidden) {
-      ld8(scale, e, gs[it]);
-      ld8(bias, e, bs[it]);
-      if (MODE != kLnResOut && residual_bias != nullptr) {
-        ld8(residual_bias, e, rbs[it]);
-      } else {
-#pragma unroll
-        for (int k = 0; k < 8; ++k) rbs[it][k] = 0.f;
-      }
-    }
+    const int e = min((it * LPR + sub) * 8, hidden - 8);
+    g_raw[it] = ld8_raw(scale, e);
+    b_raw[it] = ld8_raw(bias, e);
+    rb_raw[it] = ld8_raw(rbp, e);
+    cs_raw[it] = ld8_raw(csp, e);
+    r_raw[it] = ld8_raw(own_res ? residual + base + e : scale, 0);
+    if (MODE != kLnFirst) a_raw[it] = ld8_raw(gemm_out, base + e);
   }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int it = 0; it < ITER; ++it) {
+    pin8(g_raw[it]);
+    pin8(b_raw[it]);
+    pin8(rb_raw[it]);
+    pin8(cs_raw[it]);
+    pin8(r_raw[it]);
+    if (MODE != kLnFirst) pin8(a_raw[it]);
+  }
+  float gs[ITER][8], bs[ITER][8], rbs[ITER][8];
   float sum = 0.f;
 #pragma unroll
   for (int it = 0; it < ITER; ++it) {
     const int e = (it * LPR + sub) * 8;
+    cvt8(g_raw[it], gs[it]);
+    cvt8(b_raw[it], bs[it]);
+    cvt8(rb_raw[it], rbs[it]);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) rbs[it][k] = has_rb ? rbs[it][k] : 0.f;
     if (e < hidden && live) {
       float r[8];
-      if (sizeof(T) == 2 && pre_res != nullptr) {
+      if (own_res) {
+        cvt8(r_raw[it], r);
+      } else {
 #pragma unroll
         for (int k = 0; k < 8; ++k) r[k] = __half2float(pre_res[it].v[k]);
-      } else {
-        ld8(residual, base + e, r);
       }
       if (MODE == kLnFirst) {
 #pragma unroll
@@ -230,7 +305,7 @@ ln_rows8_row(int row, bool live, int sub, const AccT* __restrict__ gemm_out, T* 
           // further planes in a rolled loop: launches of a few rows, where the planes come
           // from, use the row kernel, and this one stays small
           int acc[8];
-          ld8_acc(gemm_out, base + e, acc);
+          cvt8(a_raw[it], acc);
           for (int p = 1; p < nparts; ++p) {
             int more[8];
             ld8_acc(gemm_out + p * part_stride, base + e, more);
@@ -240,13 +315,13 @@ ln_rows8_row(int row, bool live, int sub, const AccT* __restrict__ gemm_out, T* 
 #pragma unroll
           for (int k = 0; k < 8; ++k) a[k] = (float)acc[k];
         } else {
-          ld8_acc(gemm_out, base + e, a);
+          cvt8(a_raw[it], a);
         }
 #pragma unroll
         for (int k = 0; k < 8; ++k) x[it][k] = a[k] * dequant_scale + TT<T>::safe(r[k]);
-        if (colsum != nullptr) {
+        if (has_cs) {
           float c[8];
-          ld8(colsum, e, c);
+          cvt8(cs_raw[it], c);
 #pragma unroll
           for (int k = 0; k < 8; ++k) x[it][k] += TT<T>::safe(c[k]);
         }
