@@ -320,46 +320,49 @@ template int arrange_qkv_with_cache_i8I_i8O<__half>(int, int, hipStream_t, const
 // arg-max runs on the int8 codes; ties go to the lowest token id (the reference lets
 // racing stores decide).
 // ---------------------------------------------------------------------------------
-// First maximum of a row of int8 logits (lowest id on ties), the same in every thread.  The row
-// is read in 16-byte pieces aligned to 16 bytes in memory (rows of an odd vocabulary start
-// anywhere), every piece of a thread requested before the first is scanned; a candidate is
-// the key (code + 128) << 20 | (2^20 - 1 - id), so the arg-max is one integer maximum: over a
-// wavefront by DPP permutations and lane reads, over the workgroup through LDS with one
-// barrier.  vocab <= 2^20.
+// First maximum of a row of int8 logits (lowest id on ties), the same in every thread.  A
+// candidate is the key (code + 128) << 20 | (2^20 - 1 - id), so the arg-max is one integer
+// maximum: over a wavefront by DPP permutations and lane reads, over the workgroup through LDS
+// with one barrier.  vocab <= 2^20.
+// The row starts anywhere (an odd vocabulary), so it is read as the 16-byte pieces that lie
+// wholly inside it -- four per thread requested together, the index clamped instead of the load
+// predicated -- plus at most 15 bytes before and 15 after them, one per thread of the first
+// wavefront.  No branch sits between the loads and none around them: per element it is one
+// bit-field extract, one shift-add and one maximum (the kernel's length is its instruction
+// count; the byte-by-byte handling of partial pieces this replaces was 3000 instructions).
 __device__ __forceinline__ int block_argmax_i8(const int8_t* __restrict__ lr, int vocab,
                                                int* red /*[32]*/) {
   constexpr int kIdBits = 20, kIdMask = (1 << kIdBits) - 1;
-  const int a = (int)(reinterpret_cast<uintptr_t>(lr) & 15u);  // bytes of the first piece before the row
-  const int8_t* base = lr - a;
-  const int pieces = (vocab + a + 15) >> 4;
-  int key = 0;  // below every real key (code + 128 >= 1)
-  for (int p0 = 0; p0 < pieces; p0 += 4 * (int)blockDim.x) {
+  const int t = threadIdx.x;
+  const int a = (int)(reinterpret_cast<uintptr_t>(lr) & 15u);
+  const int head = min((16 - a) & 15, vocab);  // elements before the first aligned piece
+  const int8_t* body = lr + head;              // 16-byte aligned
+  const int nfull = (vocab - head) >> 4;       // whole pieces inside the row
+  const int tail0 = head + (nfull << 4);       // first element behind them
+  // head (threads 0..15) and tail (threads 16..31) elements, one byte each
+  const int ev = t < 16 ? t : tail0 + (t - 16);
+  const bool eon = t < 16 ? t < head : (t < 32 && ev < vocab);
+  const int ec = lr[eon ? ev : 0];
+  int key = eon ? (((ec + 128) << kIdBits) | (kIdMask - ev)) : 0;  // 0: below every real key
+  for (int p0 = 0; p0 < nfull; p0 += 4 * (int)blockDim.x) {
     uint4 w[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      // pieces past the row are clamped to the last one that lies inside it; a piece that
-      // straddles an end of the row is read byte by byte below
-      const int p = min(p0 + u * (int)blockDim.x + (int)threadIdx.x, pieces - 1);
-      const bool inside = p * 16 >= a && p * 16 + 16 <= vocab + a;
-      w[u] = inside ? *reinterpret_cast<const uint4*>(base + (long)p * 16) : make_uint4(0, 0, 0, 0);
-    }
+    for (int u = 0; u < 4; ++u)
+      w[u] = *reinterpret_cast<const uint4*>(
+          body + (long)min(p0 + u * (int)blockDim.x + t, nfull - 1) * 16);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int p = p0 + u * (int)blockDim.x + (int)threadIdx.x;
-      if (p < pieces) {
-        const int v0 = p * 16 - a;  // id of the piece's first byte
-        const bool inside = v0 >= 0 && v0 + 16 <= vocab;
-        const uint32_t ws[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+      const int p = p0 + u * (int)blockDim.x + t;
+      const int base = kIdMask - (head + p * 16);  // id part of the piece's first element
+      const uint32_t ws[4] = {w[u].x ^ 0x80808080u, w[u].y ^ 0x80808080u, w[u].z ^ 0x80808080u,
+                              w[u].w ^ 0x80808080u};  // code + 128 in every byte
+      int kp = 0;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int v = v0 + e;
-          int c;
-          if (inside) c = unpack_i8(ws[e >> 2], e & 3);
-          else if (v >= 0 && v < vocab) c = lr[v];
-          else continue;
-          key = max(key, ((c + 128) << kIdBits) | (kIdMask - v));
-        }
+      for (int e = 0; e < 16; ++e) {
+        const int c = (int)__builtin_amdgcn_ubfe(ws[e >> 2], 8 * (e & 3), 8);
+        kp = max(kp, (c << kIdBits) + (base - e));
       }
+      key = p < nfull ? max(key, kp) : key;
     }
   }
   auto max_dpp = [](int x, auto ctrl) {
