@@ -71,9 +71,13 @@ struct EpiI32 {
   // one element (the decode-step kernels give every thread one element of a 16 x 16 block)
   struct Pre1 {};
   __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
-  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1, const int8_t*,
+  struct Blk1 {
+    int n;
+  };
+  __device__ __forceinline__ Blk1 block1(int n) const { return Blk1{n}; }
+  __device__ __forceinline__ void store1(long m, Blk1 blk, int N, int acc, Pre1, const int8_t*,
                                          int) const {
-    C[m * N + n] = acc;
+    C[m * N + blk.n] = acc;
   }
   bool vec_ok(int N) const { return N % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
   static const char* name() { return "EpiI32"; }
@@ -109,9 +113,13 @@ struct EpiI8 {
   }
   struct Pre1 {};
   __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
-  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1, const int8_t*,
+  struct Blk1 {
+    int n;
+  };
+  __device__ __forceinline__ Blk1 block1(int n) const { return Blk1{n}; }
+  __device__ __forceinline__ void store1(long m, Blk1 blk, int N, int acc, Pre1, const int8_t*,
                                          int) const {
-    C[m * N + n] = (int8_t)requant_acc_fast(acc, alpha);
+    C[m * N + blk.n] = (int8_t)requant_acc_fast(acc, alpha);
   }
   bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
   static const char* name() { return "EpiI8"; }
@@ -186,20 +194,29 @@ struct EpiDecQkvI8 {
     __half b;
   };
   __device__ __forceinline__ Pre1 prefetch1(int n) const { return Pre1{bias[n]}; }
-  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1 pre, const int8_t*,
-                                         int) const {
-#pragma clang fp contract(off)
-    // the 16 columns of a block share part and head (dim_per_head % 16 == 0): divisions on the
-    // block's first column, which is the same in every lane
+  // what the elements of one column share: the 16 columns of a block lie in one part and one
+  // head (dim_per_head % 16 == 0), so the divisions run on the block's first column, the same
+  // in every lane, once per block; an element's address is base + row * row_stride + add.
+  // 32-bit offsets: this form serves the decode-step kernels only (at most 64 rows; the
+  // launcher refuses caches of 2^31 bytes and more for them)
+  struct Blk1 {
+    int8_t* base;
+    int row_stride, add;
+  };
+  __device__ __forceinline__ Blk1 block1(int n) const {
     const int nb = __builtin_amdgcn_readfirstlane(n & ~15);
     const int part = div_by(nb, hidden, inv_hidden), ib = nb - part * hidden;
     const int head = div_by(ib, dim_per_head, inv_dim), dim = ib - head * dim_per_head + (n & 15);
+    if (part == 0) return Blk1{new_q, hidden, ib + (n & 15)};
+    return Blk1{part == 1 ? new_k : new_v, head_num * max_step * dim_per_head,
+                (head * max_step + step_id) * dim_per_head + dim};
+  }
+  __device__ __forceinline__ void store1(long m, Blk1 blk, int N, int acc, Pre1 pre,
+                                         const int8_t*, int) const {
+#pragma clang fp contract(off)
     const float val = (float)requant_acc_fast(acc, alpha) * dequant_scale + __half2float(pre.b);
-    const int q = float2int8(val, quant_scale);
-    int8_t* dst = part == 0 ? new_q + m * hidden + ib + (n & 15)
-                            : (part == 1 ? new_k : new_v) +
-                                  ((m * head_num + head) * max_step + step_id) * dim_per_head + dim;
-    *dst = (int8_t)q;
+    blk.base[(unsigned)((int)m * blk.row_stride + blk.add)] =
+        (int8_t)float2int8(val, quant_scale);
     (void)N;
   }
   bool vec_ok(int) const { return true; }
@@ -248,12 +265,18 @@ struct EpiEncdecQF16 {
     __half b;
   };
   __device__ __forceinline__ Pre1 prefetch1(int n) const { return Pre1{bias[n]}; }
-  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1 pre, const int8_t*,
-                                         int) const {
+  struct Blk1 {
+    int add;  // the column's share of the offset: head * beam_size * dim_per_head + dim
+  };
+  __device__ __forceinline__ Blk1 block1(int n) const {
     const int nb = __builtin_amdgcn_readfirstlane(n & ~15);
     const int head = div_by(nb, dim_per_head, inv_dim), dim = nb - head * dim_per_head + (n & 15);
+    return Blk1{head * beam_size * dim_per_head + dim};
+  }
+  __device__ __forceinline__ void store1(long m, Blk1 blk, int N, int acc, Pre1 pre,
+                                         const int8_t*, int) const {
     const int batch_id = div_by((int)m, beam_size, inv_beam), beam_id = (int)m - batch_id * beam_size;
-    new_q[(((long)batch_id * head_num + head) * beam_size + beam_id) * dim_per_head + dim] =
+    new_q[(unsigned)((batch_id * head_num * beam_size + beam_id) * dim_per_head + blk.add)] =
         __float2half_rn(dequant_add_bias_h(requant_acc_fast(acc, alpha), dequant_scale,
                                            __half2float(pre.b)));
     (void)N;
@@ -353,9 +376,13 @@ struct EpiLutI8 {
   // element's column among them)
   struct Pre1 {};
   __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
-  __device__ __forceinline__ void store1(long m, int n, int N, int acc, Pre1, const int8_t* tab,
-                                         int n_local) const {
-    C[m * N + n] = tab[n_local * 256 + requant_acc_fast(acc, alpha) + 128];
+  struct Blk1 {
+    int n;
+  };
+  __device__ __forceinline__ Blk1 block1(int n) const { return Blk1{n}; }
+  __device__ __forceinline__ void store1(long m, Blk1 blk, int N, int acc, Pre1,
+                                         const int8_t* tab, int n_local) const {
+    C[m * N + blk.n] = tab[n_local * 256 + requant_acc_fast(acc, alpha) + 128];
   }
   bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
   static const char* name() { return "EpiLutI8"; }
@@ -1345,16 +1372,19 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
     // three adds, the epilogue of one value, one store; 16 lanes write 16 neighbouring columns.
     const int src = (ecol >> 2) * 16 + erow, r = ecol & 3;  // lane and register that held it
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
+    for (int b = 0; b < NB; ++b) {
+      const int n = n0 + 16 * b + ecol;
+      const auto blk = epi.block1(min(n, N - 1));  // what the elements of the column share
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        const int m = m0 + 16 * i + erow, n = n0 + 16 * b + ecol;
+      for (int i = 0; i < MB; ++i) {
+        const int m = m0 + 16 * i + erow;
         if (m < M && n < N) {
           const int acc = (red[0][i][b][r][src] + red[1][i][b][r][src]) +
                           (red[2][i][b][r][src] + red[3][i][b][r][src]);
-          epi.store1(m + (long)part * M, n, N, acc, pre1[b], tab, 16 * b + ecol);
+          epi.store1(m + (long)part * M, blk, N, acc, pre1[b], tab, 16 * b + ecol);
         }
       }
+    }
   } else if (tid < 16 * NB * MB) {
     const int n = n0 + 16 * eblk;
     if (m0 + em < M && n < N) {
@@ -1446,16 +1476,19 @@ gemm_i8_skinny16_wide_kernel(const int8_t* __restrict__ A, const int8_t* __restr
       const int ecol = tid & 15, erow = tid >> 4;
       const int src = (ecol >> 2) * 16 + erow, r = ecol & 3;
 #pragma unroll
-      for (int i = 0; i < MB; ++i)
+      for (int b = 0; b < 2; ++b) {
+        const int n = n00 + 32 * pair + 16 * b + ecol;
+        const auto blk = epi.block1(min(n, N - 1));
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          const int m = 16 * i + erow, n = n00 + 32 * pair + 16 * b + ecol;
+        for (int i = 0; i < MB; ++i) {
+          const int m = 16 * i + erow;
           if (m < M && n < N) {
             const int acc1 = (rd[0][i][b][r][src] + rd[1][i][b][r][src]) +
                              (rd[2][i][b][r][src] + rd[3][i][b][r][src]);
-            epi.store1(m, n, N, acc1, typename Epi::Pre1{}, nullptr, 0);
+            epi.store1(m, blk, N, acc1, typename Epi::Pre1{}, nullptr, 0);
           }
         }
+      }
     } else if (tid < 32 * MB) {
       const int n = n00 + 32 * pair + 16 * eblk;
       if (em < M && n < N) {
@@ -1909,6 +1942,9 @@ int gemm_i8_decself_qkv_i8o(const int8_t* A, const int8_t* W, const __half* qkv_
         reinterpret_cast<uintptr_t>(new_k) | reinterpret_cast<uintptr_t>(new_v)) & 15u) != 0)
     return lsh_fail(LSH_ERR_UNSUPPORTED,
                     "int8 gemm (decoder qkv): needs dim_per_head % 16 == 0 and aligned outputs");
+  if (step_token_num <= 64 && (long)step_token_num * hidden * max_step >= (1L << 31))
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "int8 gemm (decoder qkv): a cache of 2^31 bytes or more at 64 rows or fewer");
   return dispatch(A, W,
                   EpiDecQkvI8{new_q, new_k, new_v, qkv_bias, alpha, dequant_scale, quant_scale,
                               hidden, head_num, d, max_step, step_id, 1.0f / (float)hidden,
