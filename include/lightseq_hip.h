@@ -318,6 +318,20 @@ int lsh_decself_qkv_attention_i8_f16(const int8_t* x, const int8_t* qkv_weight,
  * generation runs the single launch is no faster than the pair (the projection of a head is
  * too little work to hide its weight stream).  No counterpart in the reference. */
 int lsh_decself_qkv_attention_in_models(int on);
+/* lsh_launch_dec_emb_i8I_vocab_major_f16 followed by lsh_ker_norm_layer_resual_i8O_f16 with the
+ * row kernel selected (lsh_layer_norm_row_kernel(1)) as one launch, for the first layer of a
+ * decode step (model/quant_decoder.cc.cu:570-580 + :620-633): tokens [rows, max_step] (column
+ * `step` is read), token_emb int8 [vocab, hidden], pos_emb fp16 [max_step, hidden]; residual
+ * [rows, hidden] receives what the layer norm leaves there (embedding, or the normalised row
+ * when is_post_ln, + residual_bias), out_q the int8 codes.  The same bytes as the pair.
+ * hidden % 4 == 0, hidden <= 1024, 16-byte aligned operands (LSH_ERR_UNSUPPORTED otherwise).
+ * No counterpart in the reference. */
+int lsh_dec_emb_norm_layer_i8O_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,
+                                   void* residual, int8_t* out_q, const void* scale,
+                                   const void* bias, const void* residual_bias, int rows,
+                                   int hidden, int vocab_size, int step, int max_step,
+                                   float dequant_scale, int scaled, float quant_scale,
+                                   int is_post_ln, lsh_stream_t stream);
 /* Decode-step cross-attention query product with ker_arrange_encdec_q_i8I
  * (kernels/transformerKernels_int8.cc.cu:1596-1645; call site model/quant_decoder.cc.cu:745-760)
  * as its epilogue: A [step_token_num, k] x W [hidden, k] -> int8 code (alpha) ->

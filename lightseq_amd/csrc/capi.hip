@@ -104,6 +104,17 @@ int lsh_launch_dequantize_tensor_f32(const int32_t* input, void* output, int bat
                                   dequant_scale, HS(stream));
 }
 
+int lsh_dec_emb_norm_layer_i8O_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,
+                                   void* residual, int8_t* out_q, const void* scale,
+                                   const void* bias, const void* residual_bias, int rows,
+                                   int hidden, int vocab_size, int step, int max_step,
+                                   float dequant_scale, int scaled, float quant_scale,
+                                   int is_post_ln, lsh_stream_t stream) {
+  return dec_emb_norm_layer_i8O<__half>(token_emb, H(pos_emb), tokens, HM(residual), out_q, H(scale),
+                                        H(bias), H(residual_bias), rows, hidden, vocab_size, step,
+                                        max_step, dequant_scale, scaled != 0, quant_scale,
+                                        is_post_ln != 0, HS(stream));
+}
 // ---- LayerNorm family --------------------------------------------------------------
 int lsh_layer_norm_row_kernel(int on) { return ln_set_few_rows(on != 0) ? 1 : 0; }
 int lsh_gemm_i8_tile_kernel(int on) { return gemm_i8_enable_tile_kernel(on != 0) ? 1 : 0; }

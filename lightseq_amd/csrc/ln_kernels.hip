@@ -553,6 +553,59 @@ __global__ void ln_rows_generic_kernel(const AccT* __restrict__ gemm_out, T* res
   }
 }
 
+// What follows the row's values in the workgroup-per-row kernels: mean, variance, the
+// normalised row, its int8 codes and the new residual stream.  x: the lane's four values (0
+// beyond the row), on: the lane holds elements of the row.
+template <typename T, int MODE>
+__device__ __forceinline__ void
+ln_row_wg_finish(const float (&x)[4], bool on, int e, long base, const float (&g)[4],
+                 const float (&b)[4], const float (&rb)[4], T* residual, T* out_t,
+                 int8_t* __restrict__ out_q, int hidden, float quant_scale, int is_post_ln,
+                 float (*red)[4]) {
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wpr = (int)blockDim.x >> 6;  // wavefronts of the row
+  auto row_total = [&](float v, float* r) {
+    v = wave_sum_dpp(v);
+    if (lane == 0) r[wid] = v;
+    __syncthreads();
+    // ascending order, without a loop (wpr <= 4)
+    float t = r[0];
+    const float r1 = r[1], r2 = r[2], r3 = r[3];
+    if (wpr > 1) t += r1;
+    if (wpr > 2) t += r2;
+    if (wpr > 3) t += r3;
+    return t;
+  };
+  const float mean = row_total((x[0] + x[1]) + (x[2] + x[3]), red[0]) / (float)hidden;
+  float var = 0.f;
+  if (on) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float t = x[k] - mean;
+      var += t * t;
+    }
+  }
+  const float rstd = rsqrtf(row_total(var, red[1]) / (float)hidden + kLnEpsilon);
+  if (!on) return;
+  float o[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) o[k] = (x[k] - mean) * rstd * TT<T>::safe(g[k]) + TT<T>::safe(b[k]);
+  if (MODE == kLnResOut) {
+    st4(out_t, base + e, o);
+  } else {
+    *reinterpret_cast<uint32_t*>(out_q + base + e) =
+        pack4_i8(float2int8(o[0], quant_scale), float2int8(o[1], quant_scale),
+                 float2int8(o[2], quant_scale), float2int8(o[3], quant_scale));
+    float w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float keep = is_post_ln ? o[k] : x[k];
+      w[k] = (MODE == kLnFirst) ? keep + rb[k] : TT<T>::rnd(keep) + rb[k];
+    }
+    st4(residual, base + e, w);
+  }
+}
+
 // One row per workgroup, 4 consecutive elements per lane (hidden <= 4 * blockDim.x, hidden
 // % 4 == 0): the layer norm of the decode steps, where a launch lasts a few microseconds and
 // every dependent step inside it shows.  So: no integer division and no branch before the loads
@@ -570,24 +623,10 @@ ln_row_wg_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
                  const T* __restrict__ colsum, int hidden, float dequant_scale,
                  float quant_scale, int is_post_ln, int nparts, long part_stride) {
   __shared__ float red[2][4];
-  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wpr = (int)blockDim.x >> 6;  // wavefronts of the row
   const int e0 = (int)threadIdx.x * 4;
   const bool on = e0 < hidden;
   const int e = on ? e0 : 0;  // lanes past the row load its first elements and drop them
   const long base = (long)blockIdx.x * hidden;
-  auto row_total = [&](float v, float* r) {
-    v = wave_sum_dpp(v);
-    if (lane == 0) r[wid] = v;
-    __syncthreads();
-    // ascending order, without a loop (wpr <= 4)
-    float t = r[0];
-    const float r1 = r[1], r2 = r[2], r3 = r[3];
-    if (wpr > 1) t += r1;
-    if (wpr > 2) t += r2;
-    if (wpr > 3) t += r3;
-    return t;
-  };
   float g[4], b[4], rb[4] = {0.f, 0.f, 0.f, 0.f}, r[4], c[4] = {0.f, 0.f, 0.f, 0.f};
   ld4(residual, base + e, r);
   // every load of the kernel is requested before the first value is used (the parameters
@@ -650,34 +689,8 @@ ln_row_wg_kernel(const AccT* __restrict__ gemm_out, T* residual, T* out_t,
     }
     if (!on) x[k] = 0.f;
   }
-  const float mean = row_total((x[0] + x[1]) + (x[2] + x[3]), red[0]) / (float)hidden;
-  float var = 0.f;
-  if (on) {
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const float t = x[k] - mean;
-      var += t * t;
-    }
-  }
-  const float rstd = rsqrtf(row_total(var, red[1]) / (float)hidden + kLnEpsilon);
-  if (!on) return;
-  float o[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) o[k] = (x[k] - mean) * rstd * TT<T>::safe(g[k]) + TT<T>::safe(b[k]);
-  if (MODE == kLnResOut) {
-    st4(out_t, base + e, o);
-  } else {
-    *reinterpret_cast<uint32_t*>(out_q + base + e) =
-        pack4_i8(float2int8(o[0], quant_scale), float2int8(o[1], quant_scale),
-                 float2int8(o[2], quant_scale), float2int8(o[3], quant_scale));
-    float w[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const float keep = is_post_ln ? o[k] : x[k];
-      w[k] = (MODE == kLnFirst) ? keep + rb[k] : TT<T>::rnd(keep) + rb[k];
-    }
-    st4(residual, base + e, w);
-  }
+  ln_row_wg_finish<T, MODE>(x, on, e, base, g, b, rb, residual, out_t, out_q, hidden, quant_scale,
+                            is_post_ln, red);
 }
 
 // The workgroup-per-row kernel is chosen by the caller, never by the row count: the two
@@ -696,6 +709,83 @@ bool ln_set_few_rows(bool on) {
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// The decoder's target embedding (inference/kernels/embKernels_int8.cc.cu:158-200) and the first
+// layer norm of the stack (ker_norm_layer_resual_i8O) in one launch, for the decode steps: a
+// row's embedding -- int8 table row (vocabulary-major) * scale + position row, rounded to the
+// storage type as the stand-alone kernel stores it -- is the row the layer norm reads, so the
+// bytes are those of launch_dec_emb_i8I followed by ker_norm_layer_resual_i8O with the row
+// kernel.  The token id is one dependent load ahead of the table row; the parameters travel
+// meanwhile.
+template <typename T>
+__global__ void __launch_bounds__(256)
+dec_emb_ln_row_wg_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__ pos_emb,
+                         const int* __restrict__ tokens, T* residual,
+                         int8_t* __restrict__ out_q, const T* __restrict__ scale,
+                         const T* __restrict__ bias, const T* __restrict__ residual_bias,
+                         int hidden, int vocab, int step, int max_step, float emb_scale,
+                         float quant_scale, int is_post_ln) {
+#pragma clang fp contract(off)
+  __shared__ float red[2][4];
+  const int e0 = (int)threadIdx.x * 4;
+  const bool on = e0 < hidden;
+  const int e = on ? e0 : 0;
+  const long base = (long)blockIdx.x * hidden;
+  int token = tokens[(long)blockIdx.x * max_step + step];
+  const bool has_rb = residual_bias != nullptr;
+  auto g_raw = ld4_raw(scale, e), b_raw = ld4_raw(bias, e);
+  auto rb_raw = ld4_raw(has_rb ? residual_bias : scale, e);
+  auto p_raw = ld4_raw(pos_emb, (long)step * hidden + e);
+  token = min(max(token, 0), vocab - 1);  // never index outside the table
+  const uint32_t ew = *reinterpret_cast<const uint32_t*>(token_emb + (long)token * hidden + e);
+  pin4(g_raw, b_raw, rb_raw, p_raw);
+  float g[4], b[4], rb[4], pos[4], x[4];
+  cvt4(g_raw, g);
+  cvt4(b_raw, b);
+  cvt4(rb_raw, rb);
+  cvt4(p_raw, pos);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    rb[k] = has_rb ? rb[k] : 0.f;
+    const float v = (float)unpack_i8(ew, k) * emb_scale + pos[k];
+    x[k] = on ? TT<T>::safe(TT<T>::rnd(v)) : 0.f;
+  }
+  ln_row_wg_finish<T, kLnFirst>(x, on, e, base, g, b, rb, residual, nullptr, out_q, hidden,
+                                quant_scale, is_post_ln, red);
+}
+
+template <typename T>
+int dec_emb_norm_layer_i8O(const int8_t* token_emb, const T* pos_emb, const int* tokens,
+                           T* residual, int8_t* out_q, const T* scale, const T* bias,
+                           const T* residual_bias, int rows, int hidden, int vocab, int step,
+                           int max_step, float dequant_scale, bool scaled, float quant_scale,
+                           bool is_post_ln, hipStream_t s) {
+  if (!token_emb || !pos_emb || !tokens || !residual || !out_q || !scale || !bias || rows <= 0 ||
+      hidden <= 0 || vocab <= 0 || max_step <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "dec_emb_norm_layer_i8O: bad arguments");
+  if (step < 0 || step >= max_step) return lsh_fail(LSH_ERR_INVALID, "violate step < max_step");
+  if (hidden % 4 != 0 || hidden > 1024 || !aligned16(token_emb) || !aligned16(pos_emb) ||
+      !aligned16(residual) || !aligned16(out_q) || !aligned16(scale) || !aligned16(bias) ||
+      !aligned16(residual_bias))
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "dec_emb_norm_layer_i8O: needs hidden % 4 == 0, hidden <= 1024, aligned operands");
+  float emb_scale = dequant_scale;
+  if (scaled) emb_scale *= sqrtf((float)hidden);
+  const int tpr = ((hidden / 4 + 63) / 64) * 64;
+  dec_emb_ln_row_wg_kernel<T><<<rows, tpr, 0, s>>>(token_emb, pos_emb, tokens, residual, out_q,
+                                                   scale, bias, residual_bias, hidden, vocab, step,
+                                                   max_step, emb_scale, quant_scale,
+                                                   is_post_ln ? 1 : 0);
+  return lsh_check_launch("dec_emb_ln_row_wg_kernel");
+}
+template int dec_emb_norm_layer_i8O<__half>(const int8_t*, const __half*, const int*, __half*,
+                                            int8_t*, const __half*, const __half*, const __half*,
+                                            int, int, int, int, int, float, bool, float, bool,
+                                            hipStream_t);
+template int dec_emb_norm_layer_i8O<float>(const int8_t*, const float*, const int*, float*,
+                                           int8_t*, const float*, const float*, const float*, int,
+                                           int, int, int, int, float, bool, float, bool,
+                                           hipStream_t);
 
 template <typename T, typename AccT, int MODE>
 static int launch_ln(const AccT* gemm_out, T* residual, T* out_t, int8_t* out_q, const T* scale,

@@ -54,6 +54,15 @@ template <typename T>
 int norm_layer_resual_i8O(int token_num, int hidden_size, hipStream_t stream, T* input,
                           int8_t* output, const T* scale, const T* bias, const T* residual_bias,
                           float quant_scale, bool is_post_ln);
+// launch_dec_emb_i8I (vocabulary-major table) followed by norm_layer_resual_i8O under an
+// LnFewRowsScope, in one launch: residual receives what the layer norm leaves there, out_q its
+// int8 codes.  hidden % 4 == 0, hidden <= 1024.
+template <typename T>
+int dec_emb_norm_layer_i8O(const int8_t* token_emb, const T* pos_emb, const int* tokens,
+                           T* residual, int8_t* out_q, const T* scale, const T* bias,
+                           const T* residual_bias, int rows, int hidden, int vocab, int step,
+                           int max_step, float dequant_scale, bool scaled, float quant_scale,
+                           bool is_post_ln, hipStream_t s);
 template <typename T, typename AccT>
 int residual_bias_ln_i8O(const AccT* input, const T* scale, const T* bias, const T* residual_bias,
                          int8_t* output, T* residual, int batch_tokens, int hidden_size,

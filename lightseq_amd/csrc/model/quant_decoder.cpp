@@ -305,7 +305,13 @@ void QuantDecoder::enqueue_step() {
 //   the layer, after the first, the second and the last layer norm
 #define TAP(name, ptr, bytes) step_taps.copy(_layer_id, _cur_step, name, ptr, bytes, _stream)
 
+// hidden sizes the fused embedding + first layer norm covers
+bool QuantDecoder::emb_ln_fused() const {
+  return _tw._hidden_size % 4 == 0 && _tw._hidden_size <= 1024;
+}
+
 void QuantDecoder::embedding() {
+  if (emb_ln_fused()) return;  // done by the first layer's launch
   LSH_CALL(dec_emb_i8I<__half>(_int8_trg_emb.get(), _pos_emb.get(), _alive_seq[_alive_cur].get(),
                                _cur_step_query.get(), _batch_size, _tw._beam_size,
                                _tw._hidden_size, _tw._trg_vocab_size, _cur_step, _tw._max_step,
@@ -321,9 +327,18 @@ void QuantDecoder::self_attention() {
   int8_t* v_cache = _self_v_cache[_cache_cur].get() + (size_t)_layer_id * _layer_size_self_k;
 
   if (_layer_id == 0) {
-    LSH_CALL(norm_layer_resual_i8O<__half>(M, H, _stream, _cur_step_query.get(), _buf_a.get(),
-                                           w.self_ln_scale.get(), w.self_ln_bias.get(),
-                                           w.b_self_out.get(), Q / c[6], _tw._is_post_ln));
+    if (emb_ln_fused()) {
+      // the step's embedding and the first layer norm in one launch (the bytes of the pair)
+      LSH_CALL(dec_emb_norm_layer_i8O<__half>(
+          _int8_trg_emb.get(), _pos_emb.get(), _alive_seq[_alive_cur].get(),
+          _cur_step_query.get(), _buf_a.get(), w.self_ln_scale.get(), w.self_ln_bias.get(),
+          w.b_self_out.get(), M, H, _tw._trg_vocab_size, _cur_step, _tw._max_step,
+          _trg_emb_clip_max / _quant_range, true, Q / c[6], _tw._is_post_ln, _stream));
+    } else {
+      LSH_CALL(norm_layer_resual_i8O<__half>(M, H, _stream, _cur_step_query.get(), _buf_a.get(),
+                                             w.self_ln_scale.get(), w.self_ln_bias.get(),
+                                             w.b_self_out.get(), Q / c[6], _tw._is_post_ln));
+    }
   }
   const size_t mh = (size_t)M * H;
   TAP("self_ln_q", _buf_a.get(), mh);

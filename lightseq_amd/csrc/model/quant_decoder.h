@@ -60,6 +60,7 @@ class QuantDecoder {
   void project_encoder_output();
   bool run_step();
   void embedding();
+  bool emb_ln_fused() const;
   void self_attention();
   void encdec_attention();
   void ffn_add_norm();

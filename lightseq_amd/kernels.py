@@ -637,6 +637,18 @@ def gemm_i8_decode_kernel_16x16(on):
     return bool(lib.load().lsh_gemm_i8_decode_kernel_16x16(int(bool(on))))
 
 
+def dec_emb_norm_layer_i8O(token_emb, pos_emb, tokens, residual, out_q, scale, bias, residual_bias,
+                           rows, hidden, vocab_size, step, max_step, dequant_scale, scaled,
+                           quant_scale, is_post_ln):
+    """Decode step, first layer: target embedding (vocabulary-major int8 table) and the first layer
+    norm of the stack in one launch (fp16)."""
+    _dev(token_emb, pos_emb, tokens, residual, out_q, scale, bias, residual_bias)
+    call("lsh_dec_emb_norm_layer_i8O_f16", ptr(token_emb), ptr(pos_emb), ptr(tokens), ptr(residual),
+         ptr(out_q), ptr(scale), ptr(bias), ptr(residual_bias), rows, hidden, vocab_size, step,
+         max_step, dequant_scale, int(bool(scaled)), quant_scale, int(bool(is_post_ln)),
+         current_stream())
+
+
 def gemm_i8_tile_kernel(on):
     """Route large products to the one-tile-per-workgroup kernel (default) or to the persistent
     kernels; returns the previous setting."""

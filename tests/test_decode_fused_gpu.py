@@ -196,3 +196,41 @@ def test_qkv_product_and_attention_in_one_launch_rejects_what_it_does_not_cover(
         with pytest.raises(LSHError):
             call(*bad)
 
+
+
+@pytest.mark.parametrize("rows,hidden,vocab,step,post_ln,with_rb", [(64, 1024, 32000, 17, True, True),
+                                                                      (16, 512, 1000, 0, False, True),
+                                                                      (5, 768, 333, 3, True, True),
+                                                                      (3, 132, 50, 6, False, True)])
+def test_target_embedding_and_first_layer_norm_in_one_launch(rng, rows, hidden, vocab, step, post_ln, with_rb):
+    """lsh_dec_emb_norm_layer_i8O_f16 == lsh_launch_dec_emb_i8I_vocab_major_f16 followed by
+    lsh_ker_norm_layer_resual_i8O_f16 with the row kernel: codes and residual stream byte for
+    byte (ids outside the table are clamped by both)."""
+    k = _k()
+    max_step = 9 + step
+    emb = to_dev(rng.integers(-127, 128, size=(vocab, hidden), dtype=np.int8))
+    pos = to_dev((rng.standard_normal((max_step, hidden)) * 0.5).astype(np.float16))
+    tokens = rng.integers(0, vocab, size=(rows, max_step), dtype=np.int32)
+    tokens[0, step] = vocab + 7  # outside the table
+    tokens = to_dev(tokens)
+    g = to_dev((1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16))
+    b = to_dev((0.1 * rng.standard_normal(hidden)).astype(np.float16))
+    rb = to_dev((0.1 * rng.standard_normal(hidden)).astype(np.float16)) if with_rb else None
+    dq, qs = 0.6 / 127, 127 / 3.0
+
+    res0 = torch.zeros((rows, hidden), dtype=torch.float16, device=DEV)
+    q0 = torch.zeros((rows, hidden), dtype=torch.int8, device=DEV)
+    prev = k.layer_norm_row_kernel(True)
+    try:
+        k.launch_dec_emb_i8I(emb, pos, tokens, None, None, res0, rows, 1, hidden, vocab, step, max_step, 0,
+                             dq, True, vocab_major=True)
+        k.ker_norm_layer_resual_i8O_launcher(rows, hidden, res0, q0, g, b, rb, 1024, qs, post_ln)
+    finally:
+        k.layer_norm_row_kernel(prev)
+
+    res1 = torch.full((rows, hidden), 3.0, dtype=torch.float16, device=DEV)
+    q1 = torch.full((rows, hidden), 9, dtype=torch.int8, device=DEV)
+    k.dec_emb_norm_layer_i8O(emb, pos, tokens, res1, q1, g, b, rb, rows, hidden, vocab, step, max_step, dq,
+                             True, qs, post_ln)
+    np.testing.assert_array_equal(to_np(q1), to_np(q0))
+    np.testing.assert_array_equal(to_np(res1).view(np.uint16), to_np(res0).view(np.uint16))
