@@ -946,27 +946,20 @@ beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ t
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       }
-      // the picks applied (ker_refresh_result): all new sequences of the sentence in one
-      // flat loop, four independent elements per lane, then probabilities and scores
-      for (int x0 = 0; x0 < total; x0 += 256) {
-        int val[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int x = min(x0 + 64 * u + lane, total - 1);
-          const int j = x / max_step, t = x - j * max_step;
-          const unsigned long long k = __shfl(won, j);
-          const int ori = k == 0ull ? end_id : 0x7fffffff - (int)(unsigned)k;
-          int can_beam = ori / vocab;
-          const int can_vocab = ori - can_beam * vocab;
-          if (can_beam >= beam_size) can_beam = 0;
-          const int from = staged ? seq_lds[wid][can_beam * max_step + t]
-                                  : old_alive_seq[((long)b * beam_size + can_beam) * max_step + t];
-          val[u] = t > cur_step + 1 ? end_id : (t == cur_step + 1 ? can_vocab : from);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int x = x0 + 64 * u + lane;
-          if (x < total) new_alive_seq[(long)b * beam_size * max_step + x] = val[u];
+      // the picks applied (ker_refresh_result): beam by beam, with the pick, its source beam and
+      // its token in scalar registers (one division per beam, none per element), the old
+      // sequence read from LDS; then probabilities and scores, a lane per beam
+      for (int j = 0; j < beam_size; ++j) {
+        const unsigned long long k = lane64(won, j);
+        const int ori = k == 0ull ? end_id : 0x7fffffff - (int)(unsigned)k;
+        int can_beam = ori / vocab;
+        const int can_vocab = ori - can_beam * vocab;
+        if (can_beam >= beam_size) can_beam = 0;
+        const int* from = old_alive_seq + ((long)b * beam_size + can_beam) * max_step;
+        int* to = new_alive_seq + ((long)b * beam_size + j) * max_step;
+        for (int t = lane; t < max_step; t += 64) {
+          const int old = staged ? seq_lds[wid][can_beam * max_step + t] : from[t];
+          to[t] = t > cur_step + 1 ? end_id : (t == cur_step + 1 ? can_vocab : old);
         }
       }
       if (lane < beam_size) {
