@@ -520,8 +520,10 @@ beam_topk_kernel(const int8_t* __restrict__ logits, const T* __restrict__ logit_
                  const float* __restrict__ seq_probs, const float* __restrict__ seq_score,
                  const int* __restrict__ alive_seq, float dq, float* __restrict__ top_score,
                  int* __restrict__ top_idx, int vocab, int max_step, float length_norm,
-                 int cur_step, int beam_size, int end_id) {
+                 int cur_step, int beam_size, int end_id, int* __restrict__ num_finished) {
 #pragma clang fp contract(off)
+  // the merge that follows adds its finished beams to the count: it starts at zero
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *num_finished = 0;
   __shared__ float red[1024 + 32];
   __shared__ ScoreIdx wbest[16];
   const int row = blockIdx.x, t = threadIdx.x;
@@ -581,8 +583,10 @@ beam_topk_reg_kernel(const int8_t* __restrict__ logits, const T* __restrict__ lo
                      const float* __restrict__ seq_probs, const float* __restrict__ seq_score,
                      const int* __restrict__ alive_seq, float dq, float* __restrict__ top_score,
                      int* __restrict__ top_idx, int vocab, int max_step, float length_norm,
-                     int cur_step, int beam_size, int end_id) {
+                     int cur_step, int beam_size, int end_id, int* __restrict__ num_finished) {
 #pragma clang fp contract(off)
+  // the merge that follows adds its finished beams to the count: it starts at zero
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *num_finished = 0;
   constexpr int NI = 32;
   __shared__ float red_max[16], red_sum[16];
   __shared__ unsigned long long wbest[2][16];  // per-wavefront best key, double-buffered by round
@@ -744,8 +748,10 @@ beam_topk_part_kernel(const int8_t* __restrict__ logits, const T* __restrict__ l
                       const float* __restrict__ seq_probs, const float* __restrict__ seq_score,
                       const int* __restrict__ alive_seq, float dq, float* __restrict__ top_score,
                       int* __restrict__ top_idx, int vocab, int max_step, float length_norm,
-                      int cur_step, int beam_size, int end_id) {
+                      int cur_step, int beam_size, int end_id, int* __restrict__ num_finished) {
 #pragma clang fp contract(off)
+  // the merge that follows adds its finished beams to the count: it starts at zero
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *num_finished = 0;
   __shared__ unsigned long long wbest[2][8];
   __shared__ float red_max[16], red_sum[16];
   const int part = blockIdx.x, row = blockIdx.y, P = gridDim.x, t = threadIdx.x;
@@ -844,13 +850,14 @@ beam_topk_part_kernel(const int8_t* __restrict__ logits, const T* __restrict__ l
   }
 }
 
-// beam_merge_kernel: one block, one wavefront per sentence (sentences are dealt to the
-// wavefronts round-robin).  Picks the sentence's best `beam_size` of its
-// beam_size * beam_size proposals in (score descending, candidate id ascending) order
+// beam_merge_kernel: one workgroup of one wavefront per sentence (more than 1024 sentences are
+// dealt round-robin).  Picks the sentence's best `beam_size` of its
+// beam_size * beam_size * parts proposals in (score descending, candidate id ascending) order
 // and applies ker_refresh_result to them (inference/kernels/transformerKernels.cc.cu:
 // 1398-1463): new sequences, summed log-probabilities of live beams, scores of
-// finished ones, the finished count, plus the parent table for the cache reorder.
-__global__ void __launch_bounds__(1024)
+// finished ones, the finished count (added to *num_finished, which the top-k kernel ahead of
+// it cleared), plus the parent table for the cache reorder.
+__global__ void __launch_bounds__(64)
 beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ top_idx,
                   const int* __restrict__ old_alive_seq, int* __restrict__ new_alive_seq,
                   float* __restrict__ seq_probs, float* __restrict__ seq_score,
@@ -858,10 +865,11 @@ beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ t
                   int beam_size, int vocab, int max_step, int cur_step, float length_norm,
                   int end_id, int parts) {
 #pragma clang fp contract(off)
-  __shared__ int fin_cnt[16];
-  __shared__ int seq_lds[16][512];  // a sentence's old sequences (beam_size * max_step <= 512)
-  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
-  const int nw = blockDim.x >> 6;
+  // grid: a workgroup of one wavefront per sentence (16 sentences as the 16 wavefronts of one
+  // workgroup took turns on one compute unit's SIMDs: four times the time per instruction)
+  __shared__ int seq_lds[1][512];  // the sentence's old sequences (beam_size * max_step <= 512)
+  const int lane = threadIdx.x & 63, wid = 0;
+  const int nw = gridDim.x;
   const int ncand = beam_size * beam_size * parts;  // proposals of a sentence
   int finished = 0;
   // applies one pick (ker_refresh_result): the new sequence, then probability or score
@@ -903,7 +911,7 @@ beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ t
     auto umax64 = [](unsigned long long a, unsigned long long b) { return a > b ? a : b; };
     const int total = beam_size * max_step;
     const bool staged = total <= 512;
-    for (int b = wid; b < batch; b += nw) {
+    for (int b = blockIdx.x; b < batch; b += nw) {
       const float* cs = top_score + (long)b * ncand;
       const int* ci = top_idx + (long)b * ncand;
       // the sentence's old sequences are requested together with the proposals and parked in
@@ -982,7 +990,7 @@ beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ t
       }
     }
   } else {
-    for (int b = wid; b < batch; b += nw) {
+    for (int b = blockIdx.x; b < batch; b += nw) {
       const float* cs = top_score + (long)b * ncand;
       const int* ci = top_idx + (long)b * ncand;
       ScoreIdx prev;
@@ -1005,13 +1013,7 @@ beam_merge_kernel(const float* __restrict__ top_score, const int* __restrict__ t
     }
   }
   for (int d = 32; d > 0; d >>= 1) finished += __shfl_xor(finished, d);  // lanes count their own picks
-  if (lane == 0) fin_cnt[wid] = finished;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int tot = 0;
-    for (int w2 = 0; w2 < nw; ++w2) tot += fin_cnt[w2];
-    *num_finished = tot;
-  }
+  if (lane == 0 && finished != 0) atomicAdd(num_finished, finished);  // cleared by the top-k kernel
 }
 
 // 4-byte words of the optional second workspace with which the per-row top-k is dealt to
@@ -1056,24 +1058,24 @@ int beam_search_step_i8I(const int8_t* logits, const T* logit_bias, float* seq_p
     int* p_idx = reinterpret_cast<int*>(p_score + (size_t)rows * parts * beam_size);
     beam_topk_part_kernel<T><<<dim3(parts, rows), 512, 0, s>>>(
         logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, p_score, p_idx,
-        vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+        vocab_size, max_step, length_norm, cur_step, beam_size, end_id, num_finished);
     if (int rc = lsh_check_launch("beam_topk_part_kernel")) return rc;
     top_score = p_score;
     top_idx = p_idx;
   } else if (vocab_size <= 32 * 1024 && vec)
     beam_topk_reg_kernel<T, true><<<batch_size * beam_size, 1024, 0, s>>>(
         logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score,
-        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id, num_finished);
   else if (vocab_size <= 32 * 1024)
     beam_topk_reg_kernel<T, false><<<batch_size * beam_size, 1024, 0, s>>>(
         logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score,
-        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id, num_finished);
   else
     beam_topk_kernel<T><<<batch_size * beam_size, 1024, 0, s>>>(
         logits, logit_bias, seq_probs, seq_score, old_alive_seq, dequant_scale, top_score,
-        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id);
+        top_idx, vocab_size, max_step, length_norm, cur_step, beam_size, end_id, num_finished);
   if (int rc = lsh_check_launch("beam_topk_kernel")) return rc;
-  beam_merge_kernel<<<1, 1024, 0, s>>>(top_score, top_idx, old_alive_seq, new_alive_seq,
+  beam_merge_kernel<<<batch_size < 1024 ? batch_size : 1024, 64, 0, s>>>(top_score, top_idx, old_alive_seq, new_alive_seq,
                                        seq_probs, seq_score, parent, num_finished, batch_size,
                                        beam_size, vocab_size, max_step, cur_step, length_norm,
                                        end_id, parts);
