@@ -1340,8 +1340,18 @@ gemm_i8_skinny16_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__
 #pragma unroll
       for (int i = 0; i < MB; ++i) av[u][i] = *reinterpret_cast<const v4i*>(ap[i] + off);
     }
+    // Every load of the round stays ahead of its first product: a slice whose products are
+    // conditional (a K range of fewer than four slices) had its loads moved into that branch by
+    // the compiler, behind the wait for the others -- a second trip to memory in a kernel of
+    // one.  The scheduling barrier keeps the requests together, the empty statements keep the
+    // fragments live whatever the branch does.
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
+#pragma unroll
+      for (int b = 0; b < NB; ++b) asm volatile("" : "+v"(wv[u][b]));
+#pragma unroll
+      for (int i = 0; i < MB; ++i) asm volatile("" : "+v"(av[u][i]));
       if (s0 + u < ns) {
 #pragma unroll
         for (int i = 0; i < MB; ++i)
@@ -1452,8 +1462,15 @@ gemm_i8_skinny16_wide_kernel(const int8_t* __restrict__ A, const int8_t* __restr
     for (int i = 0; i < MB; ++i)
 #pragma unroll
       for (int b = 0; b < 2; ++b) acc[i][b] = (v4i)0;
+    __builtin_amdgcn_sched_barrier(0);  // (the requests stay ahead of the products, see above)
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < 4; ++u) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) asm volatile("" : "+v"(wv[pair & 1][u][b]));
+      if (pair == 0) {
+#pragma unroll
+        for (int i = 0; i < MB; ++i) asm volatile("" : "+v"(av[u][i]));
+      }
       if (u < ns) {
 #pragma unroll
         for (int i = 0; i < MB; ++i)
@@ -1462,6 +1479,7 @@ gemm_i8_skinny16_wide_kernel(const int8_t* __restrict__ A, const int8_t* __restr
             acc[i][b] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[pair & 1][u][b], av[u][i],
                                                               acc[i][b], 0, 0, 0);
       }
+    }
     auto& rd = red[pair & 1];
 #pragma unroll
     for (int i = 0; i < MB; ++i)
