@@ -201,24 +201,25 @@ __device__ __forceinline__ float byte_to_float(uint32_t w) {
 }
 
 template <int D, int NWV, int UN>
-__device__ __forceinline__ void decself_attend_row_once(const int8_t* q, const int8_t* kb,
-                                                        const int8_t* vb, int8_t* out, bool live,
-                                                        int step_num, float attn_scale, float dq,
-                                                        float quant_scale, float* lds, int wid,
-                                                        int lane) {
-#pragma clang fp contract(off)
-  constexpr int CH = D / 16;    // lanes per cache row
-  constexpr int KPW = 64 / CH;  // rows per wavefront per load
-  float* red_max = lds;         // [NWV]
-  float* red_sum = lds + 16;    // [NWV]
-  float* part = lds + 32;       // [NWV * 4][D] value sums per row of 16 lanes
+__device__ __forceinline__ void decself_attend_row_once_body(uint4 qv, const uint4 (&kv)[UN],
+                                                             const uint4 (&vv)[UN], int8_t* out,
+                                                             bool live, int step_num,
+                                                             float attn_scale, float dq,
+                                                             float quant_scale, float* lds, int wid,
+                                                             int lane);
+
+// The cache rows of a lane for the register-resident form: lane (grp, c) of wavefront wid holds
+// bytes [16 c, 16 c + 16) of rows (u NWV + wid) KPW + grp, u < UN (clamped to the last row,
+// not predicated: unconditional loads stay back to back).
+template <int D, int NWV, int UN>
+__device__ __forceinline__ void decself_attend_load_rows(const int8_t* kb, const int8_t* vb,
+                                                         int step_num, int wid, int lane,
+                                                         uint4 (&kv)[UN], uint4 (&vv)[UN]) {
+  constexpr int CH = D / 16, KPW = 64 / CH;
   const int c = lane % CH, grp = lane / CH;
-  const uint4 qv = *reinterpret_cast<const uint4*>(q + c * 16);
-  uint4 kv[UN], vv[UN];
 #pragma unroll
   for (int u = 0; u < UN; ++u) {
     const int j = (u * NWV + wid) * KPW + grp;
-    // clamped instead of predicated: unconditional loads stay back to back
     kv[u] = *reinterpret_cast<const uint4*>(kb + (long)min(j, step_num - 1) * D + c * 16);
   }
 #pragma unroll
@@ -226,6 +227,38 @@ __device__ __forceinline__ void decself_attend_row_once(const int8_t* q, const i
     const int j = (u * NWV + wid) * KPW + grp;
     vv[u] = *reinterpret_cast<const uint4*>(vb + (long)min(j, step_num - 1) * D + c * 16);
   }
+}
+
+template <int D, int NWV, int UN>
+__device__ __forceinline__ void decself_attend_row_once(const int8_t* q, const int8_t* kb,
+                                                        const int8_t* vb, int8_t* out, bool live,
+                                                        int step_num, float attn_scale, float dq,
+                                                        float quant_scale, float* lds, int wid,
+                                                        int lane) {
+  constexpr int CH = D / 16;
+  const uint4 qv = *reinterpret_cast<const uint4*>(q + (lane % CH) * 16);
+  uint4 kv[UN], vv[UN];
+  decself_attend_load_rows<D, NWV, UN>(kb, vb, step_num, wid, lane, kv, vv);
+  decself_attend_row_once_body<D, NWV, UN>(qv, kv, vv, out, live, step_num, attn_scale, dq,
+                                           quant_scale, lds, wid, lane);
+}
+
+// What follows the loads: scores, soft-max, value sums, the context codes.  The fused
+// projection + attention kernel requests the rows before its product and enters here.
+template <int D, int NWV, int UN>
+__device__ __forceinline__ void decself_attend_row_once_body(uint4 qv, const uint4 (&kv)[UN],
+                                                             const uint4 (&vv)[UN], int8_t* out,
+                                                             bool live, int step_num,
+                                                             float attn_scale, float dq,
+                                                             float quant_scale, float* lds, int wid,
+                                                             int lane) {
+#pragma clang fp contract(off)
+  constexpr int CH = D / 16;    // lanes per cache row
+  constexpr int KPW = 64 / CH;  // rows per wavefront per load
+  float* red_max = lds;         // [NWV]
+  float* red_sum = lds + 16;    // [NWV]
+  float* part = lds + 32;       // [NWV * 4][D] value sums per row of 16 lanes
+  const int c = lane % CH, grp = lane / CH;
   // scores of the lane's rows (every lane of a row group ends with the row's score)
   float val[UN];
   float mx = kFloatInfNeg;

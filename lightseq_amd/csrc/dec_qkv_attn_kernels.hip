@@ -145,6 +145,136 @@ decself_qkv_attn_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__
   }
 }
 
+// The same for caches of 257 to 1024 steps (one row and one head per workgroup, the eight
+// wavefronts of the stand-alone attention over such a cache): the two streams of the pair --
+// the head's weights and the row's cache -- are requested together at the start.  The cache
+// rows do not depend on the projection except the one the step appends, so every lane loads
+// its rows first (the appended row's slot holds old bytes), the product and its epilogue run
+// while they travel, the epilogue leaves the new q, k and v codes in LDS as well as in memory,
+// and the lane that owns the appended row takes it from there before it enters the attention
+// body of the stand-alone kernel (decself_attend_row_once_body: the same bits).
+template <int UN>
+__global__ void __launch_bounds__(512)
+decself_qkv_attn_early_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ W,
+                              const __half* __restrict__ bias, int8_t* new_q, int8_t* k_cache,
+                              int8_t* v_cache, int8_t* __restrict__ ctx, int rows, int hidden,
+                              int head_num, int max_step, int step_id, float alpha,
+                              float dequant_scale, float cache_quant_scale, float attn_scale,
+                              float cache_dequant_scale, float ctx_quant_scale) {
+  constexpr int D = kDqaD, COLS = kDqaCols, NWV = 8;
+  constexpr int CH = D / 16, KPW = 64 / CH;
+  extern __shared__ float lds_f[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int head, row;
+  if ((head_num & 7) == 0) {
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3, hp = head_num >> 3;
+    head = xcd + 8 * (j % hp);
+    row = j / hp;
+  } else {
+    head = blockIdx.x % head_num;
+    row = blockIdx.x / head_num;
+  }
+  const int step_num = step_id + 1;
+  const long gfl = decself_group_floats<D, NWV>(step_num);
+  int32_t* partial = reinterpret_cast<int32_t*>(lds_f + gfl);              // [2][COLS]
+  int8_t* fresh = reinterpret_cast<int8_t*>(partial + 2 * COLS);           // q | k | v codes, [COLS]
+  const long bh = (long)row * head_num + head;
+  const int8_t* kb = k_cache + bh * (long)max_step * D;
+  const int8_t* vb = v_cache + bh * (long)max_step * D;
+
+  // ---- 0. the row's cache: requested before anything else ----
+  uint4 kv[UN], vv[UN];
+  decself_attend_load_rows<D, NWV, UN>(kb, vb, step_num, wave, lane, kv, vv);
+  // (and the bias of the element this thread finishes in the epilogue)
+  const __half bias_h = bias[(long)(min(tid, COLS - 1) >> 6) * hidden + head * D + (tid & 63)];
+
+  // ---- 1. product: wavefront (kpart = wave & 1, blk0 = wave >> 1) owns K half kpart of the
+  //         16-column blocks blk0, blk0 + 4, blk0 + 8 (matrix row 0 is the row) ----
+  {
+    const int kpart = wave & 1, blk0 = wave >> 1;
+    const int KH = hidden >> 7;  // 64-byte K slices per half (<= 8)
+    const int kq = lane >> 4;
+    const int8_t* xp = x + (long)row * hidden + (kpart * KH) * 64 + kq * 16;
+    dqa_v4i xf[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) xf[s] = *reinterpret_cast<const dqa_v4i*>(xp + min(s, KH - 1) * 64);
+    const int8_t* wp[3];
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+      const int n = (blk0 + 4 * t) * 16 + (lane & 15);  // column of the head's q | k | v
+      wp[t] = W + ((long)(n >> 6) * hidden + head * D + (n & 63)) * hidden + (kpart * KH) * 64 +
+              kq * 16;
+    }
+    dqa_v4i w[3][8], acc[3];
+#pragma unroll
+    for (int t = 0; t < 3; ++t)
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        w[t][s] = *reinterpret_cast<const dqa_v4i*>(wp[t] + min(s, KH - 1) * 64);
+    __builtin_amdgcn_sched_barrier(0);  // every request of the kernel is out before a product
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+      acc[t] = (dqa_v4i)0;
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        asm volatile("" : "+v"(w[t][s]));
+        if (t == 0) asm volatile("" : "+v"(xf[s]));
+        if (s < KH) acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[t][s], xf[s], acc[t], 0, 0, 0);
+      }
+    }
+    // lane holds C[row lane % 16][block * 16 + 4 * (lane / 16) + 0..3]; row 0 is the row
+    if ((lane & 15) == 0) {
+#pragma unroll
+      for (int t = 0; t < 3; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          partial[kpart * COLS + (blk0 + 4 * t) * 16 + 4 * kq + i] = acc[t][i];
+    }
+  }
+  __syncthreads();
+
+  // ---- 2. epilogue of the stand-alone product, one element per thread: q to new_q, k and v
+  //         to slot step_id of the caches, and all three to LDS ----
+  if (tid < COLS) {
+#pragma clang fp contract(off)
+    const int n = tid;
+    const int sum = partial[n] + partial[COLS + n];
+    const int part = n >> 6, dd = n & 63;
+    const float b = __half2float(bias_h);
+    const float val = (float)requant_acc(sum, alpha) * dequant_scale + b;
+    const int8_t code = (int8_t)float2int8(val, cache_quant_scale);
+    fresh[n] = code;
+    if (part == 0) {
+      new_q[(long)row * hidden + head * D + dd] = code;
+    } else {
+      int8_t* cache = part == 1 ? k_cache : v_cache;
+      cache[(bh * max_step + step_id) * D + dd] = code;
+    }
+  }
+  __syncthreads();
+
+  // ---- 3. attention: the lane that holds the appended row takes it from LDS ----
+  {
+    const int c = lane % CH, grp = lane / CH;
+    const uint4 qv = *reinterpret_cast<const uint4*>(fresh + c * 16);
+    const uint4 nk = *reinterpret_cast<const uint4*>(fresh + D + c * 16);
+    const uint4 nv = *reinterpret_cast<const uint4*>(fresh + 2 * D + c * 16);
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int j = (u * NWV + wave) * KPW + grp;
+      // rows beyond the cache were clamped to the appended one; they are masked in the body,
+      // but take the new bytes all the same
+      if (j >= step_id) {
+        kv[u] = nk;
+        vv[u] = nv;
+      }
+    }
+    decself_attend_row_once_body<D, NWV, UN>(qv, kv, vv, ctx + (long)row * hidden + head * D,
+                                             true, step_num, attn_scale, cache_dequant_scale,
+                                             ctx_quant_scale, lds_f, wave, lane);
+  }
+}
+
 bool decself_qkv_attention_enable(bool on) { return g_dqa_enabled.exchange(on); }
 bool decself_qkv_attention_enabled() { return g_dqa_enabled.load(std::memory_order_relaxed); }
 
@@ -189,10 +319,28 @@ int decself_qkv_attention_i8(const int8_t* x, const int8_t* qkv_weight, const __
         step_id, alpha, dequant_scale, cache_quant_scale, attn_scale, cache_dequant_scale,         \
         ctx_quant_scale);                                                                          \
   } while (0)
+#define LSH_DQA_EARLY(UN)                                                                          \
+  do {                                                                                             \
+    const size_t lds = (size_t)decself_group_floats<kDqaD, 8>(step_num) * sizeof(float) +          \
+                       (size_t)2 * kDqaCols * sizeof(int32_t) + kDqaCols;                          \
+    decself_qkv_attn_early_kernel<UN><<<rows * head_num, 512, lds, s>>>(                           \
+        x, qkv_weight, qkv_bias, new_q, k_cache, v_cache, ctx, rows, hidden, head_num, max_step,   \
+        step_id, alpha, dequant_scale, cache_quant_scale, attn_scale, cache_dequant_scale,         \
+        ctx_quant_scale);                                                                          \
+  } while (0)
   if (step_num <= 64) LSH_DQA(1, 4, 8);
   else if (step_num <= 128) LSH_DQA(4, 2, 2);
   else if (step_num <= 256) LSH_DQA(4, 4, 2);
-  else LSH_DQA(8, 8, 1);
+  else if (step_num <= 1024) {
+    // the group shape and loads per lane of the stand-alone attention at this length
+    const int un8 = (step_num + 127) / 128;
+    if (un8 <= 3) LSH_DQA_EARLY(3);
+    else if (un8 == 4) LSH_DQA_EARLY(4);
+    else if (un8 == 5) LSH_DQA_EARLY(5);
+    else if (un8 == 6) LSH_DQA_EARLY(6);
+    else LSH_DQA_EARLY(8);
+  } else LSH_DQA(8, 8, 1);
+#undef LSH_DQA_EARLY
 #undef LSH_DQA
   return lsh_check_launch("decself_qkv_attn_kernel");
 }
