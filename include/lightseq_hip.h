@@ -332,6 +332,21 @@ int lsh_dec_emb_norm_layer_i8O_f16(const int8_t* token_emb, const void* pos_emb,
                                    int hidden, int vocab_size, int step, int max_step,
                                    float dequant_scale, int scaled, float quant_scale,
                                    int is_post_ln, lsh_stream_t stream);
+/* lsh_launch_gpt_embedding_i8I_f16 for one position per sequence (batch_seq_len 1, pos_offset
+ * `pos`) followed by lsh_ker_norm_layer_resual_i8O_f16 with the row kernel selected, as one
+ * launch: the first layer of a cached GPT generation step (model/quant_gpt_encoder.cc.cu:363-377
+ * + :215-225).  token_id [batch] (a padding token embeds to zeros and is not counted),
+ * real_seq_len [batch] += 1 per counted token, zero_flag (may be NULL) cleared; residual
+ * [batch, hidden] and out_q as lsh_dec_emb_norm_layer_i8O_f16.  The same bytes as the pair.
+ * hidden % 4 == 0, hidden <= 1024, 16-byte aligned operands (LSH_ERR_UNSUPPORTED otherwise).
+ * No counterpart in the reference. */
+int lsh_gpt_emb_step_norm_layer_i8O_f16(const int8_t* token_emb, const void* pos_emb,
+                                        const int* token_id, void* residual, int8_t* out_q,
+                                        const void* scale, const void* bias,
+                                        const void* residual_bias, int* real_seq_len,
+                                        int* zero_flag, int batch_size, int hidden, int vocab_size,
+                                        int padding_id, int pos, int max_step, float dequant_scale,
+                                        float quant_scale, int is_post_ln, lsh_stream_t stream);
 /* Decode-step cross-attention query product with ker_arrange_encdec_q_i8I
  * (kernels/transformerKernels_int8.cc.cu:1596-1645; call site model/quant_decoder.cc.cu:745-760)
  * as its epilogue: A [step_token_num, k] x W [hidden, k] -> int8 code (alpha) ->

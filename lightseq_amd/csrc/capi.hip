@@ -115,6 +115,18 @@ int lsh_dec_emb_norm_layer_i8O_f16(const int8_t* token_emb, const void* pos_emb,
                                         max_step, dequant_scale, scaled != 0, quant_scale,
                                         is_post_ln != 0, HS(stream));
 }
+int lsh_gpt_emb_step_norm_layer_i8O_f16(const int8_t* token_emb, const void* pos_emb,
+                                        const int* token_id, void* residual, int8_t* out_q,
+                                        const void* scale, const void* bias,
+                                        const void* residual_bias, int* real_seq_len,
+                                        int* zero_flag, int batch_size, int hidden, int vocab_size,
+                                        int padding_id, int pos, int max_step, float dequant_scale,
+                                        float quant_scale, int is_post_ln, lsh_stream_t stream) {
+  return gpt_emb_step_norm_layer_i8O<__half>(
+      token_emb, H(pos_emb), token_id, HM(residual), out_q, H(scale), H(bias), H(residual_bias),
+      real_seq_len, zero_flag, batch_size, hidden, vocab_size, padding_id, pos, max_step,
+      dequant_scale, quant_scale, is_post_ln != 0, HS(stream));
+}
 // ---- LayerNorm family --------------------------------------------------------------
 int lsh_layer_norm_row_kernel(int on) { return ln_set_few_rows(on != 0) ? 1 : 0; }
 int lsh_gemm_i8_tile_kernel(int on) { return gemm_i8_enable_tile_kernel(on != 0) ? 1 : 0; }

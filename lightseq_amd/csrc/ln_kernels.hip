@@ -787,6 +787,84 @@ template int dec_emb_norm_layer_i8O<float>(const int8_t*, const float*, const in
                                            int, int, int, int, float, bool, float, bool,
                                            hipStream_t);
 
+// The same for a generation step of the GPT model: the embedding of one token per sequence at
+// position `pos` (a padding token gives zeros), the token counted into real_seq_len and
+// zero_flag cleared as gpt_embedding_step_kernel does, then the first layer's layer norm.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gpt_emb_ln_row_wg_kernel(const int8_t* __restrict__ token_emb, const T* __restrict__ pos_emb,
+                         const int* __restrict__ token_id, T* residual,
+                         int8_t* __restrict__ out_q, const T* __restrict__ scale,
+                         const T* __restrict__ bias, const T* __restrict__ residual_bias,
+                         int* real_seq_len, int* zero_flag, int padding_id, int hidden, int vocab,
+                         int pos, float emb_scale, float quant_scale, int is_post_ln) {
+#pragma clang fp contract(off)
+  __shared__ float red[2][4];
+  const int e0 = (int)threadIdx.x * 4;
+  const bool on = e0 < hidden;
+  const int e = on ? e0 : 0;
+  const long base = (long)blockIdx.x * hidden;
+  int token = token_id[blockIdx.x];
+  const bool has_rb = residual_bias != nullptr;
+  auto g_raw = ld4_raw(scale, e), b_raw = ld4_raw(bias, e);
+  auto rb_raw = ld4_raw(has_rb ? residual_bias : scale, e);
+  auto p_raw = ld4_raw(pos_emb, (long)pos * hidden + e);
+  const bool pad = token == padding_id;
+  token = min(max(token, 0), vocab - 1);  // never index outside the table
+  const uint32_t ew = *reinterpret_cast<const uint32_t*>(token_emb + (long)token * hidden + e);
+  if (threadIdx.x == 0) {
+    if (!pad) real_seq_len[blockIdx.x] += 1;
+    if (zero_flag != nullptr && blockIdx.x == 0) zero_flag[0] = 0;
+  }
+  pin4(g_raw, b_raw, rb_raw, p_raw);
+  float g[4], b[4], rb[4], pe[4], x[4];
+  cvt4(g_raw, g);
+  cvt4(b_raw, b);
+  cvt4(rb_raw, rb);
+  cvt4(p_raw, pe);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    rb[k] = has_rb ? rb[k] : 0.f;
+    const float v = pad ? 0.f : (float)unpack_i8(ew, k) * emb_scale + pe[k];
+    x[k] = on ? TT<T>::safe(TT<T>::rnd(v)) : 0.f;
+  }
+  ln_row_wg_finish<T, kLnFirst>(x, on, e, base, g, b, rb, residual, nullptr, out_q, hidden,
+                                quant_scale, is_post_ln, red);
+}
+
+template <typename T>
+int gpt_emb_step_norm_layer_i8O(const int8_t* token_emb, const T* pos_emb, const int* token_id,
+                                T* residual, int8_t* out_q, const T* scale, const T* bias,
+                                const T* residual_bias, int* real_seq_len, int* zero_flag,
+                                int batch_size, int hidden, int vocab, int padding_id, int pos,
+                                int max_step, float dequant_scale, float quant_scale,
+                                bool is_post_ln, hipStream_t s) {
+  if (!token_emb || !pos_emb || !token_id || !residual || !out_q || !scale || !bias ||
+      !real_seq_len || batch_size <= 0 || hidden <= 0 || vocab <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "gpt_emb_step_norm_layer_i8O: bad arguments");
+  if (pos < 0 || pos >= max_step)
+    return lsh_fail(LSH_ERR_INVALID, "gpt_emb_step_norm_layer_i8O: position outside the table");
+  if (hidden % 4 != 0 || hidden > 1024 || !aligned16(token_emb) || !aligned16(pos_emb) ||
+      !aligned16(residual) || !aligned16(out_q) || !aligned16(scale) || !aligned16(bias) ||
+      !aligned16(residual_bias))
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "gpt_emb_step_norm_layer_i8O: needs hidden % 4 == 0, hidden <= 1024, aligned "
+                    "operands");
+  const int tpr = ((hidden / 4 + 63) / 64) * 64;
+  gpt_emb_ln_row_wg_kernel<T><<<batch_size, tpr, 0, s>>>(
+      token_emb, pos_emb, token_id, residual, out_q, scale, bias, residual_bias, real_seq_len,
+      zero_flag, padding_id, hidden, vocab, pos, dequant_scale, quant_scale, is_post_ln ? 1 : 0);
+  return lsh_check_launch("gpt_emb_ln_row_wg_kernel");
+}
+template int gpt_emb_step_norm_layer_i8O<__half>(const int8_t*, const __half*, const int*,
+                                                 __half*, int8_t*, const __half*, const __half*,
+                                                 const __half*, int*, int*, int, int, int, int,
+                                                 int, int, float, float, bool, hipStream_t);
+template int gpt_emb_step_norm_layer_i8O<float>(const int8_t*, const float*, const int*, float*,
+                                                int8_t*, const float*, const float*, const float*,
+                                                int*, int*, int, int, int, int, int, int, float,
+                                                float, bool, hipStream_t);
+
 template <typename T, typename AccT, int MODE>
 static int launch_ln(const AccT* gemm_out, T* residual, T* out_t, int8_t* out_q, const T* scale,
                      const T* bias, const T* residual_bias, const T* colsum, int tokens,

@@ -58,6 +58,13 @@ int norm_layer_resual_i8O(int token_num, int hidden_size, hipStream_t stream, T*
 // LnFewRowsScope, in one launch: residual receives what the layer norm leaves there, out_q its
 // int8 codes.  hidden % 4 == 0, hidden <= 1024.
 template <typename T>
+int gpt_emb_step_norm_layer_i8O(const int8_t* token_emb, const T* pos_emb, const int* token_id,
+                                T* residual, int8_t* out_q, const T* scale, const T* bias,
+                                const T* residual_bias, int* real_seq_len, int* zero_flag,
+                                int batch_size, int hidden, int vocab, int padding_id, int pos,
+                                int max_step, float dequant_scale, float quant_scale,
+                                bool is_post_ln, hipStream_t s);
+template <typename T>
 int dec_emb_norm_layer_i8O(const int8_t* token_emb, const T* pos_emb, const int* tokens,
                            T* residual, int8_t* out_q, const T* scale, const T* bias,
                            const T* residual_bias, int rows, int hidden, int vocab, int step,

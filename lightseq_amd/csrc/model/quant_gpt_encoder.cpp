@@ -205,19 +205,31 @@ const int8_t* QuantGptEncoder::step_pass() {
   LnFewRowsScope few_rows;  // every step of every batch size: layer norms by the row kernel
   const int H = _tw._hidden_size, B = _batch_size;
   const float Q = _quant_range;
-  LSH_CALL(gpt_embedding_i8I<__half>(B, 1, H, _stream, _int8_emb.get(), _pos_emb.get(),
-                                     _last_ids.get(), _query.get(), _real_seq_len.get(),
-                                     _tw._padding_id, _batch_seq_len - 1, _src_emb_clip_max / Q,
-                                     _tw._src_vocab_size, _tw._max_step, _unfinished.get()));
   int8_t *a = _buf_a.get(), *b = _buf_b.get();
   _tap_step = _steps_run;
+  // the step's embedding and the first layer norm are one launch where the row kernel covers
+  // the width (the same bytes); with taps set the two launches run
+  const bool emb_ln_fused = !step_taps.any() && H % 4 == 0 && H <= 1024 && _tw._n_enc_layer > 0;
+  if (emb_ln_fused) {
+    const Layer& w0 = _layers[0];
+    LSH_CALL(gpt_emb_step_norm_layer_i8O<__half>(
+        _int8_emb.get(), _pos_emb.get(), _last_ids.get(), _query.get(), a, w0.ln1_scale.get(),
+        w0.ln1_bias.get(), w0.b_out.get(), _real_seq_len.get(), _unfinished.get(), B, H,
+        _tw._src_vocab_size, _tw._padding_id, _batch_seq_len - 1, _tw._max_step,
+        _src_emb_clip_max / Q, Q / _enc_clip_max[4], false, _stream));
+  } else {
+    LSH_CALL(gpt_embedding_i8I<__half>(B, 1, H, _stream, _int8_emb.get(), _pos_emb.get(),
+                                       _last_ids.get(), _query.get(), _real_seq_len.get(),
+                                       _tw._padding_id, _batch_seq_len - 1, _src_emb_clip_max / Q,
+                                       _tw._src_vocab_size, _tw._max_step, _unfinished.get()));
+  }
   const size_t bh = (size_t)B * H;
   for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
     const Layer& w = _layers[_layer_id];
     const float* c = &_enc_clip_max[_layer_id * 12];
     int8_t* k_cache = _self_k_cache.get() + (size_t)_layer_id * _max_batch_dim;
     int8_t* v_cache = _self_v_cache.get() + (size_t)_layer_id * _max_batch_dim;
-    if (_layer_id == 0)
+    if (_layer_id == 0 && !emb_ln_fused)
       LSH_CALL(norm_layer_resual_i8O<__half>(B, H, _stream, _query.get(), a, w.ln1_scale.get(),
                                              w.ln1_bias.get(), w.b_out.get(), Q / c[4], false));
     TAP("ln1_q", a, bh);

@@ -649,6 +649,20 @@ def dec_emb_norm_layer_i8O(token_emb, pos_emb, tokens, residual, out_q, scale, b
          current_stream())
 
 
+def gpt_emb_step_norm_layer_i8O(token_emb, pos_emb, token_id, residual, out_q, scale, bias,
+                                residual_bias, real_seq_len, zero_flag, batch_size, hidden,
+                                vocab_size, padding_id, pos, max_step, dequant_scale, quant_scale,
+                                is_post_ln):
+    """Cached GPT generation step, first layer: the step's token embedding (with the token count
+    and the flag clear of the embedding launch) and the first layer norm in one launch (fp16)."""
+    _dev(token_emb, pos_emb, token_id, residual, out_q, scale, bias, residual_bias, real_seq_len,
+         zero_flag)
+    call("lsh_gpt_emb_step_norm_layer_i8O_f16", ptr(token_emb), ptr(pos_emb), ptr(token_id),
+         ptr(residual), ptr(out_q), ptr(scale), ptr(bias), ptr(residual_bias), ptr(real_seq_len),
+         ptr(zero_flag), batch_size, hidden, vocab_size, padding_id, pos, max_step, dequant_scale,
+         quant_scale, int(bool(is_post_ln)), current_stream())
+
+
 def gemm_i8_tile_kernel(on):
     """Route large products to the one-tile-per-workgroup kernel (default) or to the persistent
     kernels; returns the previous setting."""

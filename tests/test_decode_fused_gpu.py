@@ -241,3 +241,51 @@ def test_target_embedding_and_first_layer_norm_in_one_launch(rng, rows, hidden, 
                              True, qs, post_ln)
     np.testing.assert_array_equal(to_np(q1), to_np(q0))
     np.testing.assert_array_equal(to_np(res1).view(np.uint16), to_np(res0).view(np.uint16))
+
+
+@pytest.mark.parametrize("batch,hidden,vocab,pos,post_ln", [(16, 1024, 50257, 512, False), (5, 768, 333, 0, True),
+                                                          (3, 132, 50, 6, False)])
+def test_gpt_step_embedding_and_first_layer_norm_in_one_launch(rng, batch, hidden, vocab, pos, post_ln):
+    """lsh_gpt_emb_step_norm_layer_i8O_f16 == lsh_ker_gpt_embedding_i8I_f16 (one position per
+    sequence) followed by lsh_ker_norm_layer_resual_i8O_f16 with the row kernel: codes, residual
+    stream and token counts byte for byte; a padding token embeds to zeros and is not counted;
+    the flag word is cleared."""
+    from lightseq_amd.lib import LSHError
+    k = _k()
+    max_step = pos + 4
+    pad = vocab - 1
+    emb = to_dev(rng.integers(-127, 128, size=(vocab, hidden), dtype=np.int8))
+    pe = to_dev((rng.standard_normal((max_step, hidden)) * 0.5).astype(np.float16))
+    ids = rng.integers(0, vocab - 1, size=(batch,), dtype=np.int32)
+    ids[1] = pad
+    ids = to_dev(ids)
+    g = to_dev((1 + 0.1 * rng.standard_normal(hidden)).astype(np.float16))
+    b = to_dev((0.1 * rng.standard_normal(hidden)).astype(np.float16))
+    rb = to_dev((0.1 * rng.standard_normal(hidden)).astype(np.float16))
+    dq, qs = 0.6 / 127, 127 / 3.0
+    lens = rng.integers(1, 40, size=(batch,), dtype=np.int32)
+
+    res0 = torch.zeros((batch, hidden), dtype=torch.float16, device=DEV)
+    q0 = torch.zeros((batch, hidden), dtype=torch.int8, device=DEV)
+    len0 = to_dev(lens.copy())
+    prev = k.layer_norm_row_kernel(True)
+    try:
+        k.ker_gpt_embedding_i8I_launcher(batch, 1, hidden, emb, pe, ids, res0, len0, pad, pos, dq)
+        k.ker_norm_layer_resual_i8O_launcher(batch, hidden, res0, q0, g, b, rb, 1024, qs, post_ln)
+    finally:
+        k.layer_norm_row_kernel(prev)
+
+    res1 = torch.full((batch, hidden), 3.0, dtype=torch.float16, device=DEV)
+    q1 = torch.full((batch, hidden), 9, dtype=torch.int8, device=DEV)
+    len1 = to_dev(lens.copy())
+    flag = torch.full((1,), 5, dtype=torch.int32, device=DEV)
+    k.gpt_emb_step_norm_layer_i8O(emb, pe, ids, res1, q1, g, b, rb, len1, flag, batch, hidden, vocab, pad, pos,
+                                  max_step, dq, qs, post_ln)
+    np.testing.assert_array_equal(to_np(q1), to_np(q0))
+    np.testing.assert_array_equal(to_np(res1).view(np.uint16), to_np(res0).view(np.uint16))
+    np.testing.assert_array_equal(to_np(len1), to_np(len0))
+    assert to_np(len1)[1] == lens[1] and to_np(len1)[0] == lens[0] + 1
+    assert int(to_np(flag)[0]) == 0
+    with pytest.raises(LSHError):  # position outside the table
+        k.gpt_emb_step_norm_layer_i8O(emb, pe, ids, res1, q1, g, b, rb, len1, flag, batch, hidden, vocab, pad,
+                                      max_step, max_step, dq, qs, post_ln)
