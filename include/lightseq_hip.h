@@ -347,6 +347,17 @@ int lsh_gpt_emb_step_norm_layer_i8O_f16(const int8_t* token_emb, const void* pos
                                         int* zero_flag, int batch_size, int hidden, int vocab_size,
                                         int padding_id, int pos, int max_step, float dequant_scale,
                                         float quant_scale, int is_post_ln, lsh_stream_t stream);
+/* lsh_gemm_i8_encdec_q_f16 followed by lsh_encdec_attention_f16 (int8 context only) as one
+ * launch (model/quant_decoder.cc.cu:745-800): x int8 [batch * beam, hidden], q_weight
+ * [hidden, hidden], k / v fp16 [batch, head, batch_seq_len, 64], ctx_q int8 [batch * beam,
+ * hidden] (must not overlap x).  The same bytes as the pair; the fp16 query is not stored.
+ * Heads of 64, hidden <= 1024, at most 4 beams, batch_seq_len <= 128, 16-byte aligned operands
+ * (LSH_ERR_UNSUPPORTED otherwise).  No counterpart in the reference. */
+int lsh_encdec_q_attention_f16(const int8_t* x, const int8_t* q_weight, const void* q_bias,
+                               const void* k, const void* v, const int* pad_mask, int8_t* ctx_q,
+                               float quant_scale, int batch_size, int beam_size, int head_num,
+                               int batch_seq_len, int hidden, float alpha, float dequant_scale,
+                               lsh_stream_t stream);
 /* Decode-step cross-attention query product with ker_arrange_encdec_q_i8I
  * (kernels/transformerKernels_int8.cc.cu:1596-1645; call site model/quant_decoder.cc.cu:745-760)
  * as its epilogue: A [step_token_num, k] x W [hidden, k] -> int8 code (alpha) ->

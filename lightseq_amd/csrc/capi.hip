@@ -418,6 +418,15 @@ int lsh_gemm_i8_encdec_q_f16(const int8_t* A, const int8_t* W, const void* q_bia
   return gemm_i8_encdec_q_f16(A, W, H(q_bias), HM(new_q), step_token_num, hidden, k, beam_size,
                               head_num, alpha, dequant_scale, HS(stream));
 }
+int lsh_encdec_q_attention_f16(const int8_t* x, const int8_t* q_weight, const void* q_bias,
+                               const void* k, const void* v, const int* pad_mask, int8_t* ctx_q,
+                               float quant_scale, int batch_size, int beam_size, int head_num,
+                               int batch_seq_len, int hidden, float alpha, float dequant_scale,
+                               lsh_stream_t stream) {
+  return encdec_q_attention_f16(x, q_weight, H(q_bias), H(k), H(v), pad_mask, ctx_q, quant_scale,
+                                batch_size, beam_size, head_num, batch_seq_len, hidden, alpha,
+                                dequant_scale, HS(stream));
+}
 int lsh_gemm_i8_lut_i8o(const int8_t* A, const int8_t* W, int8_t* C, const int8_t* lut, int m,
                         int n, int k, float alpha, lsh_stream_t stream) {
   return gemm_i8_lut_i8o(A, W, C, lut, m, n, k, alpha, HS(stream));

@@ -630,16 +630,34 @@ encdec_attn_vec_kernel(const __half* __restrict__ q, const __half* __restrict__ 
 // wavefront's four rows of 16 lanes meet in LDS.  The rounding points are those of the
 // kernels above (score, probability and context element rounded to fp16); the sums run in
 // another order.
-template <int D, int UN>
+//
+// QPROD: the query is not read but made here, by the product that precedes the attention in a
+// decoder layer (x int8 [rows, hidden] times the head's D rows of W [hidden, hidden], the
+// epilogue of gemm_i8_encdec_q_f16: the same fp16 values).  D = 64, at most 4 beams, hidden a
+// multiple of 64 up to 1024: wavefront w multiplies columns 16 w .. 16 w + 15 of the head for
+// the sentence's beams (v_mfma_i32_16x16x64_i8, weights as the row operand, fragments straight
+// from memory), the values meet in LDS, and wavefront b goes on with beam b.  Keys, values and
+// mask are requested before the weights, so the two streams travel together.
+struct EncdecQProd {
+  const int8_t* x;
+  const int8_t* W;
+  const __half* bias;
+  int hidden;
+  float alpha, dequant_scale;
+};
+
+template <int D, int UN, bool QPROD = false>
 __global__ void __launch_bounds__(256)
 encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
                          const __half* __restrict__ v, const int* __restrict__ pad_mask,
                          __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale,
-                         int beam_size, int head_num, int seq_len, float alpha_h) {
+                         int beam_size, int head_num, int seq_len, float alpha_h,
+                         EncdecQProd qp = EncdecQProd{}) {
 #pragma clang fp contract(off)
   constexpr int CH = D / 8;     // lanes per row
   constexpr int KPW = 64 / CH;  // rows per load instruction of the wavefront
   __shared__ float part_all[4][4][D];
+  __shared__ __align__(16) __half q_lds[QPROD ? 4 * D : 8];
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   // grid: x = head, y = sentence, z = groups of 4 beams; wavefront = beam
   const int head = (int)blockIdx.x, beam = (int)blockIdx.z * 4 + wid;
@@ -660,7 +678,7 @@ encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict_
   };
   Row qv, kv[UN], vv[UN];
   int mk[UN];
-  qv.u = *reinterpret_cast<const uint4*>(q + w * D + c * 8);
+  if (!QPROD) qv.u = *reinterpret_cast<const uint4*>(q + w * D + c * 8);
 #pragma unroll
   for (int u = 0; u < UN; ++u) {
     const int j = min(u * KPW + grp, seq_len - 1);  // clamped, not predicated
@@ -671,6 +689,44 @@ encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict_
   for (int u = 0; u < UN; ++u) {
     const int j = min(u * KPW + grp, seq_len - 1);
     vv[u].u = *reinterpret_cast<const uint4*>(vb + (long)j * D);
+  }
+  if constexpr (QPROD) {
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    const int KS = qp.hidden >> 6;  // 64-byte K slices (<= 16)
+    const int m = lane & 15, kq = lane >> 4;
+    // matrix row m: beam m of the sentence (rows beyond the beams repeat the last one)
+    const int8_t* xp = qp.x + (b * beam_size + min(m, beam_size - 1)) * (long)qp.hidden + kq * 16;
+    // the row operand: column 16 wid + m of the head
+    const int8_t* wp = qp.W + ((long)head * D + wid * 16 + m) * (long)qp.hidden + kq * 16;
+    const uint2 braw = *reinterpret_cast<const uint2*>(qp.bias + head * D + wid * 16 + 4 * kq);
+    v4i xf[16], wf[16];
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) wf[sl] = *reinterpret_cast<const v4i*>(wp + min(sl, KS - 1) * 64);
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) xf[sl] = *reinterpret_cast<const v4i*>(xp + min(sl, KS - 1) * 64);
+    __builtin_amdgcn_sched_barrier(0);  // every request of the kernel is out before a product
+    v4i acc = (v4i)0;
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) {
+      asm volatile("" : "+v"(wf[sl]));
+      asm volatile("" : "+v"(xf[sl]));
+      if (sl < KS) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[sl], xf[sl], acc, 0, 0, 0);
+    }
+    // lane holds the product of beam m with columns 16 wid + 4 kq + 0..3 of the head
+    if (m < beam_size) {
+      union {
+        uint2 u;
+        __half h[4];
+      } bb, out;
+      bb.u = braw;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        out.h[i] = __float2half_rn(dequant_add_bias_h(requant_acc(acc[i], qp.alpha),
+                                                      qp.dequant_scale, __half2float(bb.h[i])));
+      *reinterpret_cast<uint2*>(q_lds + m * D + wid * 16 + 4 * kq) = out.u;
+    }
+    __syncthreads();
+    qv.u = *reinterpret_cast<const uint4*>(q_lds + bm * D + c * 8);
   }
   // every load is requested before the first product: left alone the scheduler moves half of
   // the value loads behind the soft-max, a second trip to memory in a kernel of one
@@ -738,6 +794,47 @@ encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict_
     if (ctx_q)
       ctx_q[row * ((long)head_num * D) + (long)head * D + dd] = (int8_t)float2int8(cv, quant_scale);
   }
+}
+
+// The query product of a decoder layer and its cross attention as one launch, where the short
+// kernel covers the shape: the fp16 query never leaves the compute unit.  ctx_q must not
+// overlap x (other workgroups still read the rows).
+bool encdec_q_attention_supported(int beam_size, int head_num, int hidden, int batch_seq_len) {
+  return beam_size >= 1 && beam_size <= 4 && head_num > 0 && hidden == head_num * 64 &&
+         hidden <= 1024 && batch_seq_len >= 1 && batch_seq_len <= 16 * 8;
+}
+
+int encdec_q_attention_f16(const int8_t* x, const int8_t* q_weight, const __half* q_bias,
+                           const __half* k, const __half* v, const int* pad_mask, int8_t* ctx_q,
+                           float quant_scale, int batch_size, int beam_size, int head_num,
+                           int batch_seq_len, int hidden, float alpha, float dequant_scale,
+                           hipStream_t s) {
+  if (!x || !q_weight || !q_bias || !k || !v || !pad_mask || !ctx_q || batch_size <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "encdec_q_attention: bad arguments");
+  if (!encdec_q_attention_supported(beam_size, head_num, hidden, batch_seq_len) ||
+      batch_size > 65535 ||
+      ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(q_weight) |
+        reinterpret_cast<uintptr_t>(q_bias) | reinterpret_cast<uintptr_t>(k) |
+        reinterpret_cast<uintptr_t>(v)) & 15u) != 0)
+    return lsh_fail(LSH_ERR_UNSUPPORTED,
+                    "encdec_q_attention: needs heads of 64, hidden <= 1024, at most 4 beams, a "
+                    "source of at most 128 tokens, 16-byte aligned operands");
+  const long rows = (long)batch_size * beam_size;
+  if (x < ctx_q + rows * hidden && ctx_q < x + rows * hidden)
+    return lsh_fail(LSH_ERR_INVALID, "encdec_q_attention: ctx_q overlaps x");
+  const float alpha_h = __half2float(__float2half_rn(sqrtf(1.f / 64.f)));
+  const dim3 grid(head_num, batch_size, 1);
+  const EncdecQProd qp{x, q_weight, q_bias, hidden, alpha, dequant_scale};
+  const int un = (batch_seq_len + 7) / 8;
+#define LSH_ENCDEC_Q(UN)                                                                     \
+  encdec_attn_short_kernel<64, UN, true><<<grid, 256, 0, s>>>(                               \
+      nullptr, k, v, pad_mask, nullptr, ctx_q, quant_scale, beam_size, head_num, batch_seq_len, \
+      alpha_h, qp)
+  if (un <= 4) LSH_ENCDEC_Q(4);
+  else if (un <= 8) LSH_ENCDEC_Q(8);
+  else LSH_ENCDEC_Q(16);
+#undef LSH_ENCDEC_Q
+  return lsh_check_launch("encdec_attn_short_kernel<q product>");
 }
 
 int encdec_attention_f16(const __half* q, const __half* k, const __half* v, const int* pad_mask,

@@ -276,6 +276,12 @@ int encdec_attention_f16(const __half* q, const __half* k, const __half* v, cons
                          __half* ctx, int8_t* ctx_q, float quant_scale, int batch_size,
                          int beam_size, int head_num, int batch_seq_len, int dim_per_head,
                          hipStream_t s);
+bool encdec_q_attention_supported(int beam_size, int head_num, int hidden, int batch_seq_len);
+int encdec_q_attention_f16(const int8_t* x, const int8_t* q_weight, const __half* q_bias,
+                           const __half* k, const __half* v, const int* pad_mask, int8_t* ctx_q,
+                           float quant_scale, int batch_size, int beam_size, int head_num,
+                           int batch_seq_len, int hidden, float alpha, float dequant_scale,
+                           hipStream_t s);
 
 // ---- beam search (beam_kernels.hip) -------------------------------------------------------
 template <typename T>

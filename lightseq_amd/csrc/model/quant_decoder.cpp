@@ -396,6 +396,26 @@ void QuantDecoder::encdec_attention() {
   const float* c = &_dec_clip_max[_layer_id * 19];
   const float Q = _quant_range;
 
+  const size_t mh = (size_t)M * H;
+  // Short sources, heads of 64: the q product and the attention are one launch (the same
+  // bytes; the context goes to the second part of _buf_a because other workgroups still read
+  // the rows of _buf_b).  With taps set the launches below run.
+  if (!step_taps.any() && _tw._dim_per_head == 64 &&
+      encdec_q_attention_supported(_tw._beam_size, _tw._head_num, H, _batch_seq_len)) {
+    int8_t* ctx_q = _buf_a.get() + mh;
+    LSH_CALL(encdec_q_attention_f16(
+        _buf_b.get(), w.w_encdec_q.get(), w.b_encdec_q.get(),
+        _encdec_k.get() + (size_t)_layer_id * _layer_size_encdec_k,
+        _encdec_v.get() + (size_t)_layer_id * _layer_size_encdec_k, _p_d_padding_mask, ctx_q,
+        Q / c[9], _batch_size, _tw._beam_size, _tw._head_num, _batch_seq_len, H,
+        c[2] * c[8] / (c[14] * Q), c[14] / Q, _stream));
+    LSH_CALL(gemm_i8_i8o(ctx_q, w.w_encdec_out.get(), _buf_a.get(), M, H, H,
+                         c[3] * c[9] / (c[15] * Q), _stream));
+    LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(
+        _buf_a.get(), w.ffn_ln_scale.get(), w.ffn_ln_bias.get(), w.b_ffn2.get(), _buf_b.get(),
+        _cur_step_query.get(), M, H, c[15] / Q, Q / c[10], _stream, _tw._is_post_ln, nullptr)));
+    return;
+  }
   // q product; its epilogue is ker_arrange_encdec_q_i8I (fp16 q [batch, heads, beam, d])
   if (_tw._dim_per_head % 16 == 0) {
     LSH_CALL(gemm_i8_encdec_q_f16(_buf_b.get(), w.w_encdec_q.get(), w.b_encdec_q.get(),
@@ -408,7 +428,6 @@ void QuantDecoder::encdec_attention() {
                                           _query_buf1.get(), _tw._beam_size, _tw._dim_per_head,
                                           _tw._head_num, c[14] / Q));
   }
-  const size_t mh = (size_t)M * H;
   TAP("encdec_q", _query_buf1.get(), mh * sizeof(__half));
   TAP("encdec_k", _encdec_k.get() + (size_t)_layer_id * _layer_size_encdec_k,
       (size_t)_batch_token_num * H * sizeof(__half));

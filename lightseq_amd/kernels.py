@@ -631,6 +631,16 @@ def gemm_i8_encdec_q(a, w, q_bias, new_q, step_token_num, hidden, k, beam_size, 
          k, beam_size, head_num, alpha, dequant_scale, current_stream())
 
 
+def encdec_q_attention(x, q_weight, q_bias, k, v, pad_mask, ctx_q, quant_scale, batch_size, beam_size,
+                       head_num, batch_seq_len, hidden, alpha, dequant_scale):
+    """Decode step: cross-attention query product and the attention itself in one launch (heads
+    of 64, short sources); the bytes of gemm_i8_encdec_q + encdec_attention."""
+    _dev(x, q_weight, q_bias, k, v, pad_mask, ctx_q)
+    call("lsh_encdec_q_attention_f16", ptr(x), ptr(q_weight), ptr(q_bias), ptr(k), ptr(v),
+         ptr(pad_mask), ptr(ctx_q), quant_scale, batch_size, beam_size, head_num, batch_seq_len,
+         hidden, alpha, dequant_scale, current_stream())
+
+
 def gemm_i8_decode_kernel_16x16(on):
     """Route decode-step products (at most 64 rows) to the 16 x 16 x 64 kernel (default) or to
     the 32 x 32 x 32 one; returns the previous setting."""

@@ -53,6 +53,7 @@ _SIGNATURES = {
     "lsh_gemm_i8_lut_i8o": (False, "pppp" + "iiif" + "s"),
     "lsh_gemm_i8_decself_qkv_i8o_f16": (False, "pppppp" + "iiiiii" + "fff" + "s"),
     "lsh_decself_qkv_attention_i8_f16": (False, "ppppppp" + "iiiii" + "ffffff" + "s"),
+    "lsh_encdec_q_attention_f16": (False, "ppppppp" + "f" + "iiiii" + "ff" + "s"),
     "lsh_gemm_i8_encdec_q_f16": (False, "pppp" + "iiiii" + "ff" + "s"),
     "lsh_gpt_emb_step_norm_layer_i8O_f16": (False, "pppppppppp" + "iiiiii" + "ffi" + "s"),
     "lsh_dec_emb_norm_layer_i8O_f16": (False, "pppppppp" + "iiiii" + "fifi" + "s"),

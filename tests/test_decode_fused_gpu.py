@@ -289,3 +289,42 @@ def test_gpt_step_embedding_and_first_layer_norm_in_one_launch(rng, batch, hidde
     with pytest.raises(LSHError):  # position outside the table
         k.gpt_emb_step_norm_layer_i8O(emb, pe, ids, res1, q1, g, b, rb, len1, flag, batch, hidden, vocab, pad,
                                       max_step, max_step, dq, qs, post_ln)
+
+
+@pytest.mark.parametrize("batch,beam,heads,S", [(16, 4, 16, 64), (3, 2, 4, 37), (2, 1, 2, 128), (5, 3, 8, 9),
+                                                (2, 4, 16, 100)])
+def test_cross_attention_q_product_and_attention_in_one_launch(rng, batch, beam, heads, S):
+    """lsh_encdec_q_attention_f16 == lsh_gemm_i8_encdec_q_f16 followed by lsh_encdec_attention_f16:
+    the int8 context byte for byte (padded source positions included); what it does not cover
+    is refused."""
+    from lightseq_amd.lib import LSHError
+    k = _k()
+    d = 64
+    M, H = batch * beam, heads * d
+    x = to_dev(rng.integers(-127, 128, size=(M, H), dtype=np.int8))
+    w = to_dev(rng.integers(-127, 128, size=(H, H), dtype=np.int8))
+    bias = to_dev((rng.standard_normal(H) * 0.4).astype(np.float16))
+    alpha, ds = 2.5 / (np.sqrt(H) * 127), 3.0 / 127
+    kk = to_dev((rng.standard_normal((batch, heads, S, d)) * 0.7).astype(np.float16))
+    vv = to_dev((rng.standard_normal((batch, heads, S, d)) * 0.7).astype(np.float16))
+    mask = np.zeros((batch, S), dtype=np.int32)
+    for b in range(batch):
+        mask[b, S - int(rng.integers(0, max(1, S // 2))):] = 1
+    mask[0, :] = 0
+    mask = to_dev(mask)
+    qs = 127 / 1.5
+
+    q0 = torch.zeros((batch, heads, beam, d), dtype=torch.float16, device=DEV)
+    ctx0 = torch.zeros((M, H), dtype=torch.int8, device=DEV)
+    k.gemm_i8_encdec_q(x, w, bias, q0, M, H, H, beam, heads, alpha, ds)
+    k.encdec_attention(q0, kk, vv, mask, None, ctx0, qs, batch, beam, heads, S, d)
+    ctx1 = torch.full((M, H), 7, dtype=torch.int8, device=DEV)
+    k.encdec_q_attention(x, w, bias, kk, vv, mask, ctx1, qs, batch, beam, heads, S, H, alpha, ds)
+    np.testing.assert_array_equal(to_np(ctx1), to_np(ctx0))
+
+    with pytest.raises(LSHError):  # the context over the input rows
+        k.encdec_q_attention(x, w, bias, kk, vv, mask, x, qs, batch, beam, heads, S, H, alpha, ds)
+    with pytest.raises(LSHError):  # more than four beams
+        k.encdec_q_attention(x, w, bias, kk, vv, mask, ctx1, qs, 1, 5, heads, S, H, alpha, ds)
+    with pytest.raises(LSHError):  # a source beyond the short kernel
+        k.encdec_q_attention(x, w, bias, kk, vv, mask, ctx1, qs, batch, beam, heads, 129, H, alpha, ds)
