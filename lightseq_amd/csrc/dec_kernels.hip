@@ -634,10 +634,12 @@ encdec_attn_vec_kernel(const __half* __restrict__ q, const __half* __restrict__ 
 // QPROD: the query is not read but made here, by the product that precedes the attention in a
 // decoder layer (x int8 [rows, hidden] times the head's D rows of W [hidden, hidden], the
 // epilogue of gemm_i8_encdec_q_f16: the same fp16 values).  D = 64, at most 4 beams, hidden a
-// multiple of 64 up to 1024: wavefront w multiplies columns 16 w .. 16 w + 15 of the head for
-// the sentence's beams (v_mfma_i32_16x16x64_i8, weights as the row operand, fragments straight
-// from memory), the values meet in LDS, and wavefront b goes on with beam b.  Keys, values and
-// mask are requested before the weights, so the two streams travel together.
+// multiple of 64 up to 1024, eight wavefronts: wavefront 4 + w multiplies columns 16 w ..
+// 16 w + 15 of the head for the sentence's beams (v_mfma_i32_16x16x64_i8, weights as the row
+// operand, fragments straight from memory) and leaves the values in LDS, while wavefront b
+// requests the keys, values and mask of beam b; after the barrier the product wavefronts are
+// done and wavefront b goes on with beam b.  Two short instruction streams side by side
+// instead of one long one, and the two memory streams travel together.
 struct EncdecQProd {
   const int8_t* x;
   const int8_t* W;
@@ -647,7 +649,7 @@ struct EncdecQProd {
 };
 
 template <int D, int UN, bool QPROD = false>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(QPROD ? 512 : 256)
 encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict__ k,
                          const __half* __restrict__ v, const int* __restrict__ pad_mask,
                          __half* __restrict__ ctx, int8_t* __restrict__ ctx_q, float quant_scale,
@@ -676,6 +678,47 @@ encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict_
     h2 p[4];
     __half h[8];
   };
+  if constexpr (QPROD) {
+    if (wid >= 4) {  // the product wavefronts
+      const int pw = wid - 4;
+      typedef int v4i __attribute__((ext_vector_type(4)));
+      const int KS = qp.hidden >> 6;  // 64-byte K slices (<= 16)
+      const int m = lane & 15, kq = lane >> 4;
+      // matrix row m: beam m of the sentence (rows beyond the beams repeat the last one)
+      const int8_t* xp = qp.x + (b * beam_size + min(m, beam_size - 1)) * (long)qp.hidden + kq * 16;
+      // the row operand: column 16 pw + m of the head
+      const int8_t* wp = qp.W + ((long)head * D + pw * 16 + m) * (long)qp.hidden + kq * 16;
+      const uint2 braw = *reinterpret_cast<const uint2*>(qp.bias + head * D + pw * 16 + 4 * kq);
+      v4i xf[16], wf[16];
+#pragma unroll
+      for (int sl = 0; sl < 16; ++sl) wf[sl] = *reinterpret_cast<const v4i*>(wp + min(sl, KS - 1) * 64);
+#pragma unroll
+      for (int sl = 0; sl < 16; ++sl) xf[sl] = *reinterpret_cast<const v4i*>(xp + min(sl, KS - 1) * 64);
+      __builtin_amdgcn_sched_barrier(0);  // every request of the kernel is out before a product
+      v4i acc = (v4i)0;
+#pragma unroll
+      for (int sl = 0; sl < 16; ++sl) {
+        asm volatile("" : "+v"(wf[sl]));
+        asm volatile("" : "+v"(xf[sl]));
+        if (sl < KS) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[sl], xf[sl], acc, 0, 0, 0);
+      }
+      // lane holds the product of beam m with columns 16 pw + 4 kq + 0..3 of the head
+      if (m < beam_size) {
+        union {
+          uint2 u;
+          __half h[4];
+        } bb, out;
+        bb.u = braw;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          out.h[i] = __float2half_rn(dequant_add_bias_h(requant_acc(acc[i], qp.alpha),
+                                                        qp.dequant_scale, __half2float(bb.h[i])));
+        *reinterpret_cast<uint2*>(q_lds + m * D + pw * 16 + 4 * kq) = out.u;
+      }
+      __syncthreads();
+      return;
+    }
+  }
   Row qv, kv[UN], vv[UN];
   int mk[UN];
   if (!QPROD) qv.u = *reinterpret_cast<const uint4*>(q + w * D + c * 8);
@@ -691,40 +734,6 @@ encdec_attn_short_kernel(const __half* __restrict__ q, const __half* __restrict_
     vv[u].u = *reinterpret_cast<const uint4*>(vb + (long)j * D);
   }
   if constexpr (QPROD) {
-    typedef int v4i __attribute__((ext_vector_type(4)));
-    const int KS = qp.hidden >> 6;  // 64-byte K slices (<= 16)
-    const int m = lane & 15, kq = lane >> 4;
-    // matrix row m: beam m of the sentence (rows beyond the beams repeat the last one)
-    const int8_t* xp = qp.x + (b * beam_size + min(m, beam_size - 1)) * (long)qp.hidden + kq * 16;
-    // the row operand: column 16 wid + m of the head
-    const int8_t* wp = qp.W + ((long)head * D + wid * 16 + m) * (long)qp.hidden + kq * 16;
-    const uint2 braw = *reinterpret_cast<const uint2*>(qp.bias + head * D + wid * 16 + 4 * kq);
-    v4i xf[16], wf[16];
-#pragma unroll
-    for (int sl = 0; sl < 16; ++sl) wf[sl] = *reinterpret_cast<const v4i*>(wp + min(sl, KS - 1) * 64);
-#pragma unroll
-    for (int sl = 0; sl < 16; ++sl) xf[sl] = *reinterpret_cast<const v4i*>(xp + min(sl, KS - 1) * 64);
-    __builtin_amdgcn_sched_barrier(0);  // every request of the kernel is out before a product
-    v4i acc = (v4i)0;
-#pragma unroll
-    for (int sl = 0; sl < 16; ++sl) {
-      asm volatile("" : "+v"(wf[sl]));
-      asm volatile("" : "+v"(xf[sl]));
-      if (sl < KS) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[sl], xf[sl], acc, 0, 0, 0);
-    }
-    // lane holds the product of beam m with columns 16 wid + 4 kq + 0..3 of the head
-    if (m < beam_size) {
-      union {
-        uint2 u;
-        __half h[4];
-      } bb, out;
-      bb.u = braw;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        out.h[i] = __float2half_rn(dequant_add_bias_h(requant_acc(acc[i], qp.alpha),
-                                                      qp.dequant_scale, __half2float(bb.h[i])));
-      *reinterpret_cast<uint2*>(q_lds + m * D + wid * 16 + 4 * kq) = out.u;
-    }
     __syncthreads();
     qv.u = *reinterpret_cast<const uint4*>(q_lds + bm * D + c * 8);
   }
@@ -827,7 +836,7 @@ int encdec_q_attention_f16(const int8_t* x, const int8_t* q_weight, const __half
   const EncdecQProd qp{x, q_weight, q_bias, hidden, alpha, dequant_scale};
   const int un = (batch_seq_len + 7) / 8;
 #define LSH_ENCDEC_Q(UN)                                                                     \
-  encdec_attn_short_kernel<64, UN, true><<<grid, 256, 0, s>>>(                               \
+  encdec_attn_short_kernel<64, UN, true><<<grid, 512, 0, s>>>(                               \
       nullptr, k, v, pad_mask, nullptr, ctx_q, quant_scale, beam_size, head_num, batch_seq_len, \
       alpha_h, qp)
   if (un <= 4) LSH_ENCDEC_Q(4);
