@@ -771,6 +771,62 @@ int lsh_ker_topp_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_le
                             int* old_input_ids, int* new_input_ids, const int* real_seq_len,
                             int vocab_size, float p, int* unfinished, void* curandstate,
                             int eos_id, float dequant_scale, int in_col32);
+/* kernels/transformerKernels_int8.h:123-143 ker_topk_sample_i8I_launcher and
+ * ker_topp_sample_i8I_launcher of the encoder-decoder model (bodies
+ * transformerKernels_int8.cc.cu:1908-2290; called by QuantDecoder::sample and
+ * ::topk_greedy_search, model/quant_decoder.cc.cu:952-998, 1101-1130).  Against the GPT
+ * launchers above: a logit is code * dequant_scale + logit_bias[id], the ids live in place in
+ * old_input_ids [batch_size, max_step] (column batch_seq_len receives the token; a row whose
+ * last token is eos_id gets another eos_id and does not touch the flag), new_input_ids is
+ * unused as in the reference.  The fourth-to-last pointer is the "unfinished" word (the
+ * reference's header calls it all_finished for top-k): set to 1 when a sampled token is not
+ * eos_id; the caller clears it.  k == 1: the first id of the largest logit (a race decides in
+ * the reference), curandstate may be null.  Random numbers and the top-p nucleus: as for
+ * lsh_ker_topk_sample_i8I above.  The reference's top-p also adds the bias of every id of a
+ * thread into that thread's maximum (:2136-2137); built is the maximum of the biased logits. */
+int lsh_ker_topk_sample_i8I_dec_f16(int batch_size, int batch_seq_len, int max_step,
+                                    int logits_seq_len, int max_thread_per_block,
+                                    lsh_stream_t stream, const int8_t* logits,
+                                    const void* logit_bias, int* old_input_ids,
+                                    int* new_input_ids, int vocab_size, int k, int* all_finished,
+                                    void* curandstate, int eos_id, float dequant_scale,
+                                    int in_col32);
+int lsh_ker_topk_sample_i8I_dec_f32(int batch_size, int batch_seq_len, int max_step,
+                                    int logits_seq_len, int max_thread_per_block,
+                                    lsh_stream_t stream, const int8_t* logits,
+                                    const void* logit_bias, int* old_input_ids,
+                                    int* new_input_ids, int vocab_size, int k, int* all_finished,
+                                    void* curandstate, int eos_id, float dequant_scale,
+                                    int in_col32);
+int lsh_ker_topp_sample_i8I_dec_f16(int batch_size, int batch_seq_len, int max_step,
+                                    int logits_seq_len, int max_thread_per_block,
+                                    lsh_stream_t stream, const int8_t* logits,
+                                    const void* logit_bias, int* old_input_ids,
+                                    int* new_input_ids, int vocab_size, float p, int* unfinished,
+                                    void* curandstate, int eos_id, float dequant_scale,
+                                    int in_col32);
+int lsh_ker_topp_sample_i8I_dec_f32(int batch_size, int batch_seq_len, int max_step,
+                                    int logits_seq_len, int max_thread_per_block,
+                                    lsh_stream_t stream, const int8_t* logits,
+                                    const void* logit_bias, int* old_input_ids,
+                                    int* new_input_ids, int vocab_size, float p, int* unfinished,
+                                    void* curandstate, int eos_id, float dequant_scale,
+                                    int in_col32);
+/* kernels/gptKernels_int8.h:57-61 ker_attention_mask_weights_i32I_launcher
+ * (gptKernels_int8.cc.cu:815-853): soft-max of the int32 scores of the last dst_seq_len query
+ * positions over src_seq_len <= 1024 keys, query i seeing keys 0 .. i + src_seq_len -
+ * dst_seq_len; correlation int32 and output T, both [batch_size, head_num * dst_seq_len,
+ * src_seq_len]; rows of queries at or beyond real_seq_len[batch] are left untouched. */
+int lsh_ker_attention_mask_weights_i32I_f16(int batch_size, int dst_seq_len, int src_seq_len,
+                                            int head_num, lsh_stream_t stream,
+                                            const int32_t* correlation, void* output,
+                                            const int* real_seq_len, float attn_scale,
+                                            float dequant_scale);
+int lsh_ker_attention_mask_weights_i32I_f32(int batch_size, int dst_seq_len, int src_seq_len,
+                                            int head_num, lsh_stream_t stream,
+                                            const int32_t* correlation, void* output,
+                                            const int* real_seq_len, float attn_scale,
+                                            float dequant_scale);
 /* kernels/gptKernels_int8.h ker_ppl_i8I_launcher (gptKernels_int8.cc.cu:182-190). */
 int lsh_ker_ppl_i8I(int batch_size, int batch_seq_len, int max_thread_per_block,
                     lsh_stream_t stream, const int8_t* logits, const int* input_ids,

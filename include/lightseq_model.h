@@ -114,7 +114,8 @@ int ls_model_get_steps_run(ls_model* model, int* steps);
 int ls_model_set_graph_mode(ls_model* model, int on);
 int ls_model_get_graph_stats(ls_model* model, int* captured, long long* replayed);
 
-/* QuantGpt with sampling_method topk (topk > 1) or topp: restart the per-sequence generator
+/* QuantGpt with sampling_method topk (topk > 1) or topp, QuantTransformer with sampling_method
+ * topk or topp (model/quant_decoder.cc.cu:952-998): restart the per-sequence generator
  * states of the sampling steps (sequence i of a batch draws from Philox4x32-10 keyed with `seed`,
  * counter (draw, 0, i, 0)).  A model starts with seed 0, so two runs of one model file give the
  * same tokens; the reference seeds its cuRAND states with clock()

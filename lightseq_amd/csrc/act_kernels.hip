@@ -134,7 +134,11 @@ bias_act_lut_kernel(const int8_t* in, int8_t* out, const T* __restrict__ bias, i
 }
 
 static std::atomic<bool> g_act_lut_enabled{true};
-bool bias_act_enable_lut_kernel(bool on) { return g_act_lut_enabled.exchange(on); }
+bool bias_act_enable_lut_kernel(bool on) {
+  const bool prev = g_act_lut_enabled.exchange(on);
+  if (prev != on) route_epoch_bump();
+  return prev;
+}
 
 template <typename T, int ACT>
 static int launch_bias_act(int tokens, hipStream_t s, const int8_t* input, int8_t* output,

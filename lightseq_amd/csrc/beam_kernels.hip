@@ -477,7 +477,11 @@ int write_topk_result(const int* alive_seq, float* seq_score, int* res_seq, int 
                       int max_step, int beam_size, int end_id, int rows, int out_len,
                       hipStream_t s) {
   (void)vocab_size;
-  if (int rc = write_check(alive_seq, seq_score, res_seq, rows, max_step, beam_size, out_len,
+  // the last output column is the end token whatever the sequence holds, so a sampling run that
+  // used every step (out_len == max_step; the reference reads one element past the row there)
+  // stays inside the row
+  if (int rc = write_check(alive_seq, seq_score, res_seq, rows, max_step, beam_size,
+                           out_len == max_step ? out_len - 1 : out_len,
                            "ker_write_topk_result: bad arguments"))
     return rc;
   write_topk_result_kernel<<<rows, 256, 0, s>>>(alive_seq, seq_score, res_seq, max_step,

@@ -802,6 +802,45 @@ int lsh_ker_topp_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_le
                          old_input_ids, new_input_ids, vocab_size, p, unfinished, curandstate,
                          eos_id, dequant_scale);
 }
+#define LSH_DEC_SAMPLE(SUF, T)                                                                  \
+  int lsh_ker_topk_sample_i8I_dec_##SUF(                                                        \
+      int batch_size, int batch_seq_len, int max_step, int logits_seq_len,                      \
+      int max_thread_per_block, lsh_stream_t stream, const int8_t* logits,                      \
+      const void* logit_bias, int* old_input_ids, int* new_input_ids, int vocab_size, int k,    \
+      int* all_finished, void* curandstate, int eos_id, float dequant_scale, int in_col32) {    \
+    (void)max_thread_per_block;                                                                 \
+    (void)new_input_ids;                                                                        \
+    if (int rc = no_col32(in_col32, 0, "ker_topk_sample_i8I")) return rc;                       \
+    return dec_topk_sample_i8I<T>(batch_size, batch_seq_len, max_step, logits_seq_len,          \
+                                  HS(stream), logits, static_cast<const T*>(logit_bias),        \
+                                  old_input_ids, vocab_size, k, all_finished, curandstate,      \
+                                  eos_id, dequant_scale);                                       \
+  }                                                                                             \
+  int lsh_ker_topp_sample_i8I_dec_##SUF(                                                        \
+      int batch_size, int batch_seq_len, int max_step, int logits_seq_len,                      \
+      int max_thread_per_block, lsh_stream_t stream, const int8_t* logits,                      \
+      const void* logit_bias, int* old_input_ids, int* new_input_ids, int vocab_size, float p,  \
+      int* unfinished, void* curandstate, int eos_id, float dequant_scale, int in_col32) {      \
+    (void)max_thread_per_block;                                                                 \
+    (void)new_input_ids;                                                                        \
+    if (int rc = no_col32(in_col32, 0, "ker_topp_sample_i8I")) return rc;                       \
+    return dec_topp_sample_i8I<T>(batch_size, batch_seq_len, max_step, logits_seq_len,          \
+                                  HS(stream), logits, static_cast<const T*>(logit_bias),        \
+                                  old_input_ids, vocab_size, p, unfinished, curandstate,        \
+                                  eos_id, dequant_scale);                                       \
+  }                                                                                             \
+  int lsh_ker_attention_mask_weights_i32I_##SUF(                                                \
+      int batch_size, int dst_seq_len, int src_seq_len, int head_num, lsh_stream_t stream,      \
+      const int32_t* correlation, void* output, const int* real_seq_len, float attn_scale,      \
+      float dequant_scale) {                                                                    \
+    return attention_mask_weights_i32I<T>(batch_size, dst_seq_len, src_seq_len, head_num,       \
+                                          HS(stream), correlation, static_cast<T*>(output),     \
+                                          real_seq_len, attn_scale, dequant_scale);             \
+  }
+LSH_DEC_SAMPLE(f16, __half)
+LSH_DEC_SAMPLE(f32, float)
+#undef LSH_DEC_SAMPLE
+
 int lsh_rng_setup(void* state, int n, uint64_t seed, lsh_stream_t stream) {
   return sample_state_setup(state, n, seed, HS(stream));
 }

@@ -275,7 +275,11 @@ decself_qkv_attn_early_kernel(const int8_t* __restrict__ x, const int8_t* __rest
   }
 }
 
-bool decself_qkv_attention_enable(bool on) { return g_dqa_enabled.exchange(on); }
+bool decself_qkv_attention_enable(bool on) {
+  const bool prev = g_dqa_enabled.exchange(on);
+  if (prev != on) route_epoch_bump();
+  return prev;
+}
 bool decself_qkv_attention_enabled() { return g_dqa_enabled.load(std::memory_order_relaxed); }
 
 bool decself_qkv_attention_supported(int rows, int hidden, int head_num, int max_step) {

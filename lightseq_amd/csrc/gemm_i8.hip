@@ -40,6 +40,7 @@
 
 #include <hip/hip_ext.h>
 
+#include <atomic>
 #include <cstdlib>
 #include <mutex>
 #include <string>
@@ -1530,9 +1531,13 @@ gemm_i8_skinny16_wide_kernel(const int8_t* __restrict__ A, const int8_t* __restr
 // ---------------------------------------------------------------------------------
 static thread_local hipEvent_t g_ev_start = nullptr, g_ev_stop = nullptr;
 // switch for A/B measurements of the one-tile-per-workgroup kernel against the persistent ones
-static bool g_tile_kernel_enabled = true;
+static std::atomic<bool> g_tile_kernel_enabled{true};
 // the same for the two decode-step kernels (tests compare them bit for bit)
-static bool g_skinny16_enabled = true;
+static std::atomic<bool> g_skinny16_enabled{true};
+static std::atomic<unsigned long> g_route_epoch{0};
+
+unsigned long route_epoch() { return g_route_epoch.load(std::memory_order_acquire); }
+void route_epoch_bump() { g_route_epoch.fetch_add(1, std::memory_order_acq_rel); }
 
 void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop) {
   g_ev_start = start;
@@ -1821,14 +1826,14 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
 }
 
 bool gemm_i8_enable_tile_kernel(bool on) {
-  const bool prev = g_tile_kernel_enabled;
-  g_tile_kernel_enabled = on;
+  const bool prev = g_tile_kernel_enabled.exchange(on);
+  if (prev != on) route_epoch_bump();
   return prev;
 }
 
 bool gemm_i8_enable_skinny16_kernel(bool on) {
-  const bool prev = g_skinny16_enabled;
-  g_skinny16_enabled = on;
+  const bool prev = g_skinny16_enabled.exchange(on);
+  if (prev != on) route_epoch_bump();
   return prev;
 }
 

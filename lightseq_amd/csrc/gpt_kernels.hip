@@ -7,6 +7,7 @@
 // where the reference re-lays out (copies) every cache and the whole id matrix per step.
 #include "ls_device.cuh"
 #include "ls_launch.h"
+#include "sample_common.h"
 
 #include <string>
 #include <type_traits>
@@ -224,6 +225,65 @@ template int correlation_softmax_gpt_i32I<float>(int, int, int, hipStream_t, con
                                                  float*, const int*, float, float);
 template int correlation_softmax_gpt_i32I<__half>(int, int, int, hipStream_t, const int32_t*,
                                                   __half*, const int*, float, float);
+
+// ---------------------------------------------------------------------------------
+// ker_attention_mask_weights_i32I (inference/kernels/gptKernels_int8.cc.cu:815-853): the
+// soft-max of the last dst_seq_len query positions of a sequence over src_seq_len keys, each
+// query seeing the keys up to its own position.  correlation / output [batch, head_num *
+// dst_seq_len, src_seq_len]; a query at or beyond its sequence's real length leaves its output
+// row untouched, as the reference's early return does.  The reference runs one thread per key
+// (src_seq_len <= 1024); here a wavefront takes a row.
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+attention_mask_weights_i32I_kernel(const int32_t* __restrict__ corr, T* __restrict__ out,
+                                   const int* __restrict__ real_seq_len, long rows,
+                                   int rows_per_batch, int dst_seq_len, int src_seq_len,
+                                   float attn_scale, float dq) {
+#pragma clang fp contract(off)
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int b = (int)(row / rows_per_batch);
+  const int qpos = (int)(row % dst_seq_len) + src_seq_len - dst_seq_len;
+  if (qpos >= real_seq_len[b]) return;
+  const int32_t* c = corr + row * src_seq_len;
+  T* o = out + row * src_seq_len;
+  float mx = kFloatInfNeg;
+  for (int j = lane; j <= qpos && j < src_seq_len; j += 64)
+    mx = fmaxf(mx, (float)c[j] * attn_scale * dq * dq);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int j = lane; j <= qpos && j < src_seq_len; j += 64)
+    sum += expf(fmaxf(kLogitThreshMin, (float)c[j] * attn_scale * dq * dq - mx));
+  sum = wave_sum(sum);
+  for (int j = lane; j < src_seq_len; j += 64) {
+    const float e =
+        j <= qpos ? expf(fmaxf(kLogitThreshMin, (float)c[j] * attn_scale * dq * dq - mx)) : 0.f;
+    TT<T>::st(o, j, e / (sum + 1e-12f));  // epsilon: inference/kernels/transformerKernels.h:13
+  }
+}
+
+template <typename T>
+int attention_mask_weights_i32I(int batch_size, int dst_seq_len, int src_seq_len, int head_num,
+                                hipStream_t s, const int32_t* correlation, T* output,
+                                const int* real_seq_len, float attn_scale, float dequant_scale) {
+  if (!correlation || !output || !real_seq_len || batch_size <= 0 || dst_seq_len <= 0 ||
+      src_seq_len < dst_seq_len || head_num <= 0)
+    return lsh_fail(LSH_ERR_INVALID, "ker_attention_mask_weights_i32I: bad arguments");
+  if (src_seq_len > 1024)  // the reference launches src_seq_len threads per block
+    return lsh_fail(LSH_ERR_INVALID, "ker_attention_mask_weights_i32I: src_seq_len above 1024");
+  const int rows_per_batch = head_num * dst_seq_len;
+  const long rows = (long)batch_size * rows_per_batch;
+  attention_mask_weights_i32I_kernel<T><<<(int)((rows + 3) / 4), 256, 0, s>>>(
+      correlation, output, real_seq_len, rows, rows_per_batch, dst_seq_len, src_seq_len,
+      attn_scale, dequant_scale);
+  return lsh_check_launch("attention_mask_weights_i32I_kernel");
+}
+template int attention_mask_weights_i32I<float>(int, int, int, int, hipStream_t, const int32_t*,
+                                                float*, const int*, float, float);
+template int attention_mask_weights_i32I<__half>(int, int, int, int, hipStream_t, const int32_t*,
+                                                 __half*, const int*, float, float);
 
 // batched int8 q.K^T of the prompt pass (inference/model/quant_gpt_encoder.cc.cu:498-505)
 // for callers of the unfused launchers: scores[bh, i, j] = sum_d q[bh,i,d] * k[bh,j,d]
@@ -491,28 +551,6 @@ int gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_siz
 // counter = (draw, 0, row, 0), word 0) mapped to (0, 1] as curand_uniform maps 32 bits, with
 // the state {seed, row, draws} per sequence in device memory, advanced by the kernel.
 // ---------------------------------------------------------------------------------
-struct alignas(16) SampleState {
-  unsigned long long seed;
-  unsigned int row, draws;
-};
-static_assert(sizeof(SampleState) == 16, "lsh_rng_state_t is 16 bytes");
-
-__device__ __forceinline__ uint32_t philox4x32_10_word0(uint32_t c0, uint32_t c1, uint32_t c2,
-                                                        uint32_t c3, uint32_t k0, uint32_t k1) {
-#pragma unroll
-  for (int r = 0; r < 10; ++r) {
-    const unsigned long long p0 = 0xD2511F53ull * c0, p1 = 0xCD9E8D57ull * c2;
-    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
-    c1 = (uint32_t)p1;
-    c3 = (uint32_t)p0;
-    c0 = n0;
-    c2 = n2;
-    k0 += 0x9E3779B9u;
-    k1 += 0xBB67AE85u;
-  }
-  return c0;
-}
-
 __global__ void sample_state_setup_kernel(SampleState* st, int n, unsigned long long seed) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) st[i] = SampleState{seed, (unsigned)i, 0u};
@@ -525,18 +563,6 @@ int sample_state_setup(void* state, int n, unsigned long long seed, hipStream_t 
                                                             seed);
   return lsh_check_launch("sample_state_setup_kernel");
 }
-
-constexpr int kSampleThreads = 1024;
-constexpr int kSampleIdBits = 20, kSampleIdMask = (1 << kSampleIdBits) - 1;
-
-struct SampleShared {
-  int cls[kSampleThreads];   // class maxima (codes; -129 = empty), then candidate keys
-  float pf[kSampleThreads];  // exps of the 257 code values (top-p), then wavefront prefix totals
-  int hist[260];             // classes per maximum code (top-p)
-  float red[16];
-  int thr, tok;
-  float x;
-};
 
 // The 16 consecutive ids a thread reads per piece belong to 16 classes that do not change from
 // piece to piece (16 * 1024 is a multiple of 1024), so a thread reduces in registers and
@@ -569,13 +595,7 @@ __device__ int sample_row(const int8_t* __restrict__ lr, int vocab, int k, float
   const int cls0 = (16 * t - a) & (kSampleThreads - 1);  // class of the thread's slot 0
   sh.cls[t] = -129;
   if (t < 260) sh.hist[t] = 0;
-  if (t == 0) {
-    const SampleState s = *st;
-    const uint32_t w = philox4x32_10_word0(s.draws, 0u, s.row, 0u, (uint32_t)s.seed,
-                                           (uint32_t)(s.seed >> 32));
-    sh.x = (float)w * 2.3283064365386963e-10f + 1.1641532182693481e-10f;  // (0, 1]
-    st->draws = s.draws + 1;
-  }
+  if (t == 0) sh.x = sample_draw_uniform(st);
   __syncthreads();
   {
     int m[16];
@@ -656,29 +676,7 @@ __device__ int sample_row(const int8_t* __restrict__ lr, int vocab, int k, float
   const float ex = key == 0 ? 0.f
                             : expf(rank == 1 ? kLogitThreshMin
                                              : fmaxf((float)(rank - 130) * scale - mx, kLogitThreshMin));
-  const float prob = ex / block_sum(ex, sh.red);
-  // inclusive prefix in thread order: within the wavefront, then the totals of the wavefronts before
-  float pre = prob;
-  const int lane = t & 63, wid = t >> 6;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const float up = __shfl_up(pre, d);
-    if (lane >= d) pre += up;
-  }
-  __syncthreads();
-  if (lane == 63) sh.pf[wid] = pre;
-  __syncthreads();
-  for (int w = 0; w < wid; ++w) pre += sh.pf[w];
-  const float x = sh.x;
-  int pick = kSampleThreads - (int)block_max((float)(x > pre ? 0 : kSampleThreads - t), sh.red);
-  if (pick == kSampleThreads) {
-    // rounding left the last prefix below x: the lowest thread of the largest probability
-    const float pmax = block_max(prob, sh.red);
-    pick = kSampleThreads - (int)block_max((float)(prob == pmax ? kSampleThreads - t : 0), sh.red);
-  }
-  if (t == pick) sh.tok = my_id;
-  __syncthreads();
-  return sh.tok;
+  return sample_pick(ex, my_id, sh);
 }
 
 // ker_topk_sample_i8I<k> / ker_topp_sample_i8I: ids re-laid out from [batch, seq_len] to

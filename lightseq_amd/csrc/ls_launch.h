@@ -222,6 +222,12 @@ const char* gemm_i8_act_epilogue_name(int act);
 // The next int8 GEMM launched from this thread records kernel-exact begin / end
 // timestamps into the two events (hipExtLaunchKernelGGL), then the hook clears itself.
 void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop);
+// Counts the changes of the process-wide route switches below (tile kernel, decode-step
+// kernel, fused decode attention, activation table kernel).  Whoever keeps launches recorded
+// (the models' step graphs) compares it with the value it recorded under and drops what it
+// holds when a switch has moved since.
+unsigned long route_epoch();
+void route_epoch_bump();
 // A/B switch: route large products to the persistent kernels instead of the one-tile-per-
 // workgroup kernel (on by default)
 bool gemm_i8_enable_tile_kernel(bool on);  // returns the previous setting
@@ -372,6 +378,24 @@ int topp_sample_i8I(int batch_size, int batch_seq_len, int logits_seq_len, hipSt
                     float p, int* unfinished, void* state, int eos_id, float dequant_scale);
 // generator states of n sequences: {seed, sequence index, draws made = 0}
 int sample_state_setup(void* state, int n, unsigned long long seed, hipStream_t s);
+// ker_attention_mask_weights_i32I_launcher (inference/kernels/gptKernels_int8.h:57-61)
+template <typename T>
+int attention_mask_weights_i32I(int batch_size, int dst_seq_len, int src_seq_len, int head_num,
+                                hipStream_t s, const int32_t* correlation, T* output,
+                                const int* real_seq_len, float attn_scale, float dequant_scale);
+// Encoder-decoder sampling (sample_kernels.hip): ker_topk_sample_i8I_launcher /
+// ker_topp_sample_i8I_launcher of inference/kernels/transformerKernels_int8.h:123-143; ids
+// [rows, max_step] in place, column batch_seq_len receives the token; k == 1 needs no state.
+template <typename T>
+int dec_topk_sample_i8I(int batch_size, int batch_seq_len, int max_step, int logits_seq_len,
+                        hipStream_t s, const int8_t* logits, const T* logit_bias, int* ids,
+                        int vocab_size, int k, int* unfinished, void* state, int eos_id,
+                        float dequant_scale);
+template <typename T>
+int dec_topp_sample_i8I(int batch_size, int batch_seq_len, int max_step, int logits_seq_len,
+                        hipStream_t s, const int8_t* logits, const T* logit_bias, int* ids,
+                        int vocab_size, float p, int* unfinished, void* state, int eos_id,
+                        float dequant_scale);
 // the model's step with random sampling (k in {2,..,32}: top-k; k == 0: top-p with p)
 int gpt_sample_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size, int max_step,
                     int cur_len, int batch_size, int* unfinished, int eos_id, int k, float p,

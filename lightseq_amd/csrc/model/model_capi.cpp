@@ -298,7 +298,10 @@ int ls_model_set_seed(ls_model* model, unsigned long long seed) {
   NEED_MODEL(model);
   if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get()))
     return guarded([&] { qg->encoder()->set_seed(seed); });
-  return lsh::lsh_fail(LSH_ERR_UNSUPPORTED, "a seed applies to the random sampling of QuantGpt");
+  if (QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get()))
+    return guarded([&] { qt->decoder()->set_seed(seed); });
+  return lsh::lsh_fail(LSH_ERR_UNSUPPORTED,
+                       "a seed applies to the random sampling of QuantGpt and QuantTransformer");
 }
 
 int ls_model_get_graph_stats(ls_model* model, int* captured, long long* replayed) {

@@ -7,8 +7,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
-#include <stdexcept>
+#include <list>
 #include <map>
+#include <stdexcept>
 #include <string>
 #include <unordered_map>
 #include <unordered_set>
@@ -117,10 +118,14 @@ class StepTaps {
 
 // HIP graphs of a generation step.  A step is a fixed sequence of launches whose arguments
 // depend only on the shapes of the call and on the position of the step, so the sequence
-// enqueued for one key is the sequence for every later call with that key.
+// enqueued for one key is the sequence for every later call with that key -- as long as the
+// process-wide route switches stand as they stood at the capture (route_epoch(); a change drops
+// every graph held) and the body bakes in no pointer that a caller can replace.
 //   first time a key is seen   the step runs eagerly (kernel attributes get set, nothing is kept)
 //   second time                the step is captured from the stream, instantiated and launched
 //   later                      one hipGraphLaunch
+// At most kMaxGraphs executables are kept, the least recently launched one is destroyed first.
+// A key whose capture or instantiation fails runs eagerly from then on.
 // The body may only enqueue kernels and device-to-device copies on the stream: no memset nodes
 // (they replay wrongly on this platform), no synchronisation, no host reads.
 class StepGraphs {
@@ -130,12 +135,16 @@ class StepGraphs {
   StepGraphs& operator=(const StepGraphs&) = delete;
   ~StepGraphs() { clear(); }
   void clear() {
-    for (auto& kv : execs_) (void)hipGraphExecDestroy(kv.second);
+    for (auto& kv : execs_) (void)hipGraphExecDestroy(kv.second.exec);
     execs_.clear();
+    lru_.clear();
     seen_.clear();
+    eager_only_.clear();
   }
   int captured() const { return captured_; }
   long replayed() const { return replayed_; }
+  size_t held() const { return execs_.size(); }
+  static constexpr size_t kMaxGraphs = 512;
 
   template <typename Body>
   void run(uint64_t key, hipStream_t stream, bool enabled, Body&& body) {
@@ -143,19 +152,56 @@ class StepGraphs {
       body();
       return;
     }
+    const unsigned long epoch = lsh::route_epoch();
+    if (epoch != epoch_) {
+      clear();
+      epoch_ = epoch;
+    }
     auto it = execs_.find(key);
     if (it != execs_.end()) {
-      CHECK_GPU_ERROR(hipGraphLaunch(it->second, stream));
+      lru_.splice(lru_.begin(), lru_, it->second.pos);
+      CHECK_GPU_ERROR(hipGraphLaunch(it->second.exec, stream));
       ++replayed_;
       return;
     }
-    if (seen_.insert(key).second) {  // first encounter
+    if (eager_only_.count(key) || seen_.insert(key).second) {  // failed before / first encounter
       body();
       return;
     }
-    if (execs_.size() >= kMaxGraphs) clear_execs();
+    hipGraphExec_t exec = capture(stream, body);
+    if (!exec) {  // the platform refused: the step still has to run
+      eager_only_.insert(key);
+      body();
+      return;
+    }
+    while (execs_.size() >= kMaxGraphs) {
+      const uint64_t old = lru_.back();
+      lru_.pop_back();
+      auto o = execs_.find(old);
+      (void)hipGraphExecDestroy(o->second.exec);
+      execs_.erase(o);
+    }
+    lru_.push_front(key);
+    execs_[key] = Held{exec, lru_.begin()};
+    ++captured_;
+    CHECK_GPU_ERROR(hipGraphLaunch(exec, stream));
+    ++replayed_;
+  }
+
+ private:
+  struct Held {
+    hipGraphExec_t exec;
+    std::list<uint64_t>::iterator pos;
+  };
+  // Records the body; null when the capture or the instantiation fails (nothing has run then).
+  // An exception of the body itself (a launcher that rejects its arguments) propagates.
+  template <typename Body>
+  hipGraphExec_t capture(hipStream_t stream, Body&& body) {
+    if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
     hipGraph_t graph = nullptr;
-    CHECK_GPU_ERROR(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
     try {
       body();
     } catch (...) {
@@ -163,25 +209,24 @@ class StepGraphs {
       if (graph) (void)hipGraphDestroy(graph);
       throw;
     }
-    CHECK_GPU_ERROR(hipStreamEndCapture(stream, &graph));
+    if (hipStreamEndCapture(stream, &graph) != hipSuccess || !graph) {
+      (void)hipGetLastError();
+      if (graph) (void)hipGraphDestroy(graph);
+      return nullptr;
+    }
     hipGraphExec_t exec = nullptr;
-    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
-    CHECK_GPU_ERROR(e);
-    execs_[key] = exec;
-    ++captured_;
-    CHECK_GPU_ERROR(hipGraphLaunch(exec, stream));
-    ++replayed_;
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    return exec;
   }
-
- private:
-  void clear_execs() {
-    for (auto& kv : execs_) (void)hipGraphExecDestroy(kv.second);
-    execs_.clear();
-  }
-  static constexpr size_t kMaxGraphs = 4096;
-  std::unordered_map<uint64_t, hipGraphExec_t> execs_;
-  std::unordered_set<uint64_t> seen_;
+  std::unordered_map<uint64_t, Held> execs_;
+  std::list<uint64_t> lru_;  // most recently launched first
+  std::unordered_set<uint64_t> seen_, eager_only_;
+  unsigned long epoch_ = 0;
   int captured_ = 0;
   long replayed_ = 0;
 };

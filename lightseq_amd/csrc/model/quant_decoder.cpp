@@ -56,9 +56,13 @@ std::string QuantDecoder::check() {
   const std::string& m = _tw._sampling_method;
   if (m != "beam_search" && m != "topk" && m != "topp" && m != "topk_greedy")
     return std::string("unsupported sampling_method: ") + m;
-  if (m != "beam_search")
-    return "sampling_method " + m + " (topk = " + std::to_string(_tw._topk) + ", topp = " +
-           std::to_string(_tw._topp) + ") is not available in this build (beam_search only)";
+  // (inference/model/quant_decoder.cc.cu:392-397)
+  if (m == "topk" || m == "topp") _output_topk = false;
+  if (m == "topk_greedy") _output_topk = true;
+  if (m == "topk" && _tw._topk != 1 && _tw._topk != 2 && _tw._topk != 4 && _tw._topk != 8 &&
+      _tw._topk != 16 && _tw._topk != 32)
+    return "topk argument should be in [1,2,4,8,16,32]";
+  if (m == "topp" && (!(_tw._topp > 0.f) || _tw._topp > 1.f)) return "topp outside (0, 1]";
   if (_tw._diverse_lambda != 0.f) return "diverse beam search is not available in this build";
   if (_tw._max_step > 1024) return "max_step should not greater than 1024";
   if (_tw._hidden_size % 16 != 0 || _tw._inner_size % 16 != 0)
@@ -109,6 +113,9 @@ void QuantDecoder::init_buffer() {
     _topk_part_ws.alloc(words);
   _parent.alloc(rows);
   _num_finished.alloc(1);
+  _sample_unfinished.alloc(1);
+  _sample_state.alloc(rows * 2);
+  set_seed(0);
   CHECK_GPU_ERROR(hipHostMalloc(reinterpret_cast<void**>(&_h_num_finished), sizeof(int)));
   *_h_num_finished = 0;
   CHECK_GPU_ERROR(hipStreamSynchronize(_stream));  // start_id_vec dies below
@@ -190,6 +197,16 @@ void QuantDecoder::init_buffer() {
   }
 }
 
+void QuantDecoder::set_seed(unsigned long long seed) {
+  LSH_CALL(sample_state_setup(_sample_state.get(), (int)(_sample_state.size() / 2), seed, _stream));
+}
+
+// "topk_greedy" opens with one beam-search step, which gives every beam of a sentence another
+// first token (inference/model/quant_decoder.cc.cu:1101-1106)
+bool QuantDecoder::step_runs_beam_search() const {
+  return !_is_sampling || (_tw._sampling_method == "topk_greedy" && _cur_step == 0);
+}
+
 void QuantDecoder::run_one_infer(int batch_size, int batch_seq_len) {
   if (batch_size > _max_batch_size)
     throw std::runtime_error("batch size of input greater than max_batch_size");
@@ -204,6 +221,16 @@ void QuantDecoder::run_one_infer(int batch_size, int batch_seq_len) {
   _step_token_num = batch_size * _tw._beam_size;
   _batch_max_decode_length =
       std::min(_tw._max_step, batch_seq_len + _tw._extra_decode_length) - 1;
+  // (:429-434)
+  _is_sampling = _tw._sampling_method == "topk" || _tw._sampling_method == "topp" ||
+                 _tw._sampling_method == "topk_greedy";
+  if (_is_sampling) {
+    _batch_max_decode_length = _tw._max_step;
+    // nothing writes the scores of a sampled sequence; the reference returns its buffer as
+    // allocated, here every call returns zeros
+    CHECK_GPU_ERROR(hipMemsetAsync(_alive_seq_score_own.get(), 0, sizeof(float) * _step_token_num,
+                                   _stream));
+  }
   _steps_run = 0;
   // every call starts from the same halves of the double-buffered sequences and caches (column
   // 0 of both sequence buffers holds the start token; everything else is rewritten as the
@@ -223,8 +250,14 @@ void QuantDecoder::run_one_infer(int batch_size, int batch_seq_len) {
   }
 
   /* ---step3. output the decoding result--- */
+  // The steps keep the scores of finished beams in the decoder's own buffer: a step may be a
+  // recorded graph, and the caller may hand over another output buffer between two calls.
+  if (_p_d_alive_seq_score != _alive_seq_score_own.get())
+    CHECK_GPU_ERROR(hipMemcpyAsync(_p_d_alive_seq_score, _alive_seq_score_own.get(),
+                                   sizeof(float) * _step_token_num, hipMemcpyDeviceToDevice,
+                                   _stream));
   int* alive = _alive_seq[_alive_cur].get();
-  if (_output_topk) {
+  if (_output_topk || _is_sampling) {
     if (_cur_step == _batch_max_decode_length) _cur_step -= 1;
     LSH_CALL(write_topk_result(alive, _p_d_alive_seq_score, _p_d_result, _tw._trg_vocab_size,
                                _tw._max_step, _tw._beam_size, _tw._end_id, _step_token_num,
@@ -255,13 +288,24 @@ void QuantDecoder::project_encoder_output() {
 }
 
 bool QuantDecoder::run_step() {
+  const bool search = step_runs_beam_search();
   // The launches of a step depend on the shapes of the call, the step index and which of the
-  // two sequence / cache buffers is current: one graph per such key.
+  // two sequence / cache buffers is current: one graph per such key.  A sampling step clears
+  // its flag with a memset and runs eagerly.
   const uint64_t key = ((uint64_t)_batch_size << 40) | ((uint64_t)_batch_seq_len << 24) |
                        ((uint64_t)_cur_step << 8) | (uint64_t)(_alive_cur << 1 | _cache_cur);
-  _graphs.run(key, _stream, _use_graphs && !_rec_logits && !_rec_alive && !step_taps.any(),
+  _graphs.run(key, _stream,
+              _use_graphs && !_is_sampling && !_rec_logits && !_rec_alive && !step_taps.any(),
               [&] { enqueue_step(); });
   ++_steps_run;
+  if (!search) {
+    // (:979-984, 1126-1131) the sequences stay in their buffer, the caches are not reordered
+    if (_is_benchmark) return false;
+    CHECK_GPU_ERROR(hipMemcpyAsync(_h_num_finished, _sample_unfinished.get(), sizeof(int),
+                                   hipMemcpyDeviceToHost, _stream));
+    CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+    return *_h_num_finished != 1;
+  }
   _alive_cur ^= 1;
   if (_cur_step > 0) _cache_cur ^= 1;
   if (!_is_benchmark) {
@@ -293,7 +337,10 @@ void QuantDecoder::enqueue_step() {
     CHECK_GPU_ERROR(hipMemcpyAsync(
         _rec_logits + (size_t)_cur_step * _step_token_num * _tw._trg_vocab_size, _logits.get(),
         (size_t)_step_token_num * _tw._trg_vocab_size, hipMemcpyDeviceToDevice, _stream));
-  beam_search();
+  if (step_runs_beam_search())
+    beam_search();
+  else
+    sample_tokens();
 }
 
 // Step taps (debug): name -> what is copied, of layer step_taps' layer at its step.
@@ -494,11 +541,35 @@ void QuantDecoder::ffn_add_norm() {
 
 #undef TAP
 
+// QuantDecoder::sample and ::topk_greedy_search after its first step
+// (inference/model/quant_decoder.cc.cu:952-984, 1108-1131): one token per row, in place
+void QuantDecoder::sample_tokens() {
+  int* alive = _alive_seq[_alive_cur].get();
+  CHECK_GPU_ERROR(hipMemsetAsync(_sample_unfinished.get(), 0, sizeof(int), _stream));
+  const float dq = _logits_clip_max / _quant_range;
+  if (_tw._sampling_method == "topp") {
+    LSH_CALL(dec_topp_sample_i8I<__half>(_step_token_num, _cur_step + 1, _tw._max_step, 1, _stream,
+                                         _logits.get(), _logit_bias.get(), alive,
+                                         _tw._trg_vocab_size, _tw._topp, _sample_unfinished.get(),
+                                         _sample_state.get(), _tw._end_id, dq));
+  } else {
+    const int k = _tw._sampling_method == "topk" ? _tw._topk : 1;
+    LSH_CALL(dec_topk_sample_i8I<__half>(_step_token_num, _cur_step + 1, _tw._max_step, 1, _stream,
+                                         _logits.get(), _logit_bias.get(), alive,
+                                         _tw._trg_vocab_size, k, _sample_unfinished.get(),
+                                         _sample_state.get(), _tw._end_id, dq));
+  }
+  if (_rec_alive && _cur_step < _rec_max_steps)
+    CHECK_GPU_ERROR(hipMemcpyAsync(
+        _rec_alive + (size_t)_cur_step * _step_token_num * _tw._max_step, alive,
+        (size_t)_step_token_num * _tw._max_step * sizeof(int), hipMemcpyDeviceToDevice, _stream));
+}
+
 void QuantDecoder::beam_search() {
   int* alive = _alive_seq[_alive_cur].get();
   int* alive_new = _alive_seq[_alive_cur ^ 1].get();
   LSH_CALL(beam_search_step_i8I<__half>(
-      _logits.get(), _logit_bias.get(), _alive_seq_probs.get(), _p_d_alive_seq_score, alive,
+      _logits.get(), _logit_bias.get(), _alive_seq_probs.get(), _alive_seq_score_own.get(), alive,
       alive_new, _top_score.get(), _top_idx.get(), _parent.get(), _num_finished.get(),
       _logits_clip_max / _quant_range, _tw._trg_vocab_size, _tw._max_step,
       _h_length_norm[_cur_step], _cur_step, _batch_size, _tw._beam_size, _tw._end_id, _stream,

@@ -31,6 +31,9 @@ class QuantDecoder {
   std::string check();
   void run_one_infer(int batch_size, int batch_seq_len);
   void benchmark_mode(bool is_benchmark) { _is_benchmark = is_benchmark; }
+  // Restart the generator states of the sampling methods ("topk", "topp"): row i draws from
+  // (seed, i).  Seed 0 at load.
+  void set_seed(unsigned long long seed);
 
   // Optional per-step records for parity checks (device pointers owned by the caller):
   // logits [max_steps, batch*beam, vocab] int8 and the sequences after each step
@@ -66,6 +69,8 @@ class QuantDecoder {
   void ffn_add_norm();
   void enqueue_step();
   void beam_search();
+  void sample_tokens();
+  bool step_runs_beam_search() const;
 
   const int _max_batch_size;
   QuantTransformerWeight& _tw;
@@ -81,7 +86,8 @@ class QuantDecoder {
   int _batch_max_decode_length = 0, _layer_id = 0, _steps_run = 0;
   long _layer_size_encdec_k, _layer_size_self_k;
   std::vector<float> _h_alive_seq_probs, _h_length_norm;
-  int* _h_num_finished = nullptr;  // pinned
+  int* _h_num_finished = nullptr;  // pinned; also receives the unfinished word of a sampling step
+  bool _is_sampling = false;
 
   int8_t* _rec_logits = nullptr;
   int* _rec_alive = nullptr;
@@ -99,6 +105,8 @@ class QuantDecoder {
   int _alive_cur = 0;
   DeviceBuffer<float> _alive_seq_probs, _alive_seq_score_own, _top_score, _topk_part_ws;
   DeviceBuffer<int> _top_idx, _parent, _num_finished;
+  DeviceBuffer<int> _sample_unfinished;           // the flag of a sampling step
+  DeviceBuffer<unsigned long long> _sample_state;  // lsh_rng_state_t per row (16 bytes each)
   // weights
   DeviceBuffer<int8_t> _int8_trg_emb;  // [vocab, H]: embedding rows and logits kernel
   DeviceBuffer<__half> _pos_emb, _out_ln_scale, _out_ln_bias, _kv_kernel /*[n_layer*2*H, H]*/,

@@ -529,6 +529,41 @@ def ker_topp_sample_i8I_launcher(batch_size, batch_seq_len, logits_seq_len, max_
          eos_id, dequant_scale, int(in_col32))
 
 
+def ker_topk_sample_i8I_dec_launcher(batch_size, batch_seq_len, max_step, logits_seq_len,
+                                     max_thread_per_block, logits, logit_bias, old_input_ids,
+                                     new_input_ids, vocab_size, k, all_finished, curandstate,
+                                     eos_id, dequant_scale, in_col32=False):
+    """Encoder-decoder ``ker_topk_sample_i8I_launcher`` (transformerKernels_int8.h:123-132): ids in
+    place in ``old_input_ids`` [batch, max_step]; ``curandstate`` may be None for k == 1."""
+    _dev(logits, logit_bias, old_input_ids, all_finished)
+    call("lsh_ker_topk_sample_i8I_dec" + _suffix(logit_bias), batch_size, batch_seq_len, max_step,
+         logits_seq_len, max_thread_per_block, current_stream(), ptr(logits), ptr(logit_bias),
+         ptr(old_input_ids), ptr(new_input_ids), vocab_size, k, ptr(all_finished),
+         ptr(curandstate), eos_id, dequant_scale, int(in_col32))
+
+
+def ker_topp_sample_i8I_dec_launcher(batch_size, batch_seq_len, max_step, logits_seq_len,
+                                     max_thread_per_block, logits, logit_bias, old_input_ids,
+                                     new_input_ids, vocab_size, p, unfinished, curandstate, eos_id,
+                                     dequant_scale, in_col32=False):
+    """Encoder-decoder ``ker_topp_sample_i8I_launcher`` (transformerKernels_int8.h:134-143)."""
+    _dev(logits, logit_bias, old_input_ids, unfinished, curandstate)
+    call("lsh_ker_topp_sample_i8I_dec" + _suffix(logit_bias), batch_size, batch_seq_len, max_step,
+         logits_seq_len, max_thread_per_block, current_stream(), ptr(logits), ptr(logit_bias),
+         ptr(old_input_ids), ptr(new_input_ids), vocab_size, p, ptr(unfinished), ptr(curandstate),
+         eos_id, dequant_scale, int(in_col32))
+
+
+def ker_attention_mask_weights_i32I_launcher(batch_size, dst_seq_len, src_seq_len, head_num,
+                                             correlation, output, real_seq_len, attn_scale,
+                                             dequant_scale):
+    """``ker_attention_mask_weights_i32I_launcher`` (gptKernels_int8.h:57-61)."""
+    _dev(correlation, output, real_seq_len)
+    call("lsh_ker_attention_mask_weights_i32I" + _suffix(output), batch_size, dst_seq_len,
+         src_seq_len, head_num, current_stream(), ptr(correlation), ptr(output), ptr(real_seq_len),
+         attn_scale, dequant_scale)
+
+
 def rng_setup(batch_size, seed, device="cuda"):
     """Generator states of ``batch_size`` sequences for the random-sampling launchers (in place
     of the reference's curandState array): an int64 tensor [batch_size, 2] holding

@@ -111,6 +111,9 @@ _SIGNATURES = {
     "lsh_gpt_sample_step": (False, "ppp" + "iiii" + "p" + "i" + "iff" + "p" + "s"),
     "lsh_ker_topp_sample_i8I": (False, "iiiis" + "pppp" + "if" + "pp" + "ifi"),
     "lsh_rng_setup": (False, "piQs"),
+    "lsh_ker_topk_sample_i8I_dec": (True, "iiiiis" + "pppp" + "ii" + "pp" + "ifi"),
+    "lsh_ker_topp_sample_i8I_dec": (True, "iiiiis" + "pppp" + "if" + "pp" + "ifi"),
+    "lsh_ker_attention_mask_weights_i32I": (True, "iiiis" + "ppp" + "ff"),
     # operator launchers of the csrc layer path (include/lightseq_ops.h)
     "lsh_launch_quantize": (True, "ppppp" + "ii" + "s"),
     "lsh_launch_quantize_2d": (True, "ppppp" + "iii" + "s" + "i"),

@@ -236,7 +236,8 @@ def make_quant_transformer(cfg, seed=0, ln_noise=0.02, eos_bias=None, w_std=None
             "extra_decode_length": cfg["extra_decode_length"],
             "length_penalty": cfg["length_penalty"], "src_padding_id": cfg["padding_id"],
             "trg_start_id": cfg["start_id"], "diverse_lambda": 0.0,
-            "sampling_method": cfg.get("sampling_method", "beam_search"), "topp": 0.75, "topk": 1,
+            "sampling_method": cfg.get("sampling_method", "beam_search"),
+            "topp": cfg.get("topp", 0.75), "topk": cfg.get("topk", 1),
             "trg_end_id": cfg["end_id"], "is_post_ln": cfg["is_post_ln"],
             "no_scale_embedding": False, "use_gelu": cfg["use_gelu"], "multilg_type": 0}
     return {"src_embedding": src_emb, "encoder_stack": enc_layers, "trg_embedding": trg_emb,

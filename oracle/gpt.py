@@ -46,6 +46,20 @@ def correlation_softmax_gpt_i32I(correlation, real_seq_len, head_num, attn_scale
     return out
 
 
+def attention_mask_weights_i32I(correlation, real_seq_len, head_num, dst_seq_len, attn_scale,
+                                dequant_scale, out):
+    """correlation [batch, head * dst_seq_len, src_seq_len] int32; ``out`` (same shape, float16
+    or float32) is updated in place: rows of queries beyond the real length keep their values."""
+    correlation = _c_arr(correlation, np.int32)
+    rsl = _c_arr(real_seq_len, np.int32)
+    batch, rows, src = correlation.shape
+    assert rows == head_num * dst_seq_len and out.shape == correlation.shape
+    assert out.flags["C_CONTIGUOUS"]
+    _lib.lso_attention_mask_weights_i32I(_p(correlation), _p(out), _p(rsl), batch, dst_seq_len, src,
+                                         head_num, _fl(attn_scale), _fl(dequant_scale), _f16(out))
+    return out
+
+
 def arrange_qkv_with_cache_i8I_i8O(ori_qkv, qkv_bias, k_cache, v_cache, dequant_scale, quant_scale):
     """ori_qkv [batch, 3H]; caches [batch, head, seq_len-1, d].  Returns (new_q
     [batch, head, 1, d], new_k, new_v [batch, head, seq_len, d])."""

@@ -375,6 +375,11 @@ void lso_gpt_scores_i8(const int8_t* q, const int8_t* k, int32_t* scores,
 
 /* kernels/gptKernels_int8.cc.cu:192-250.  Rows of padded queries are written as
  * zeros (the reference leaves them untouched). */
+/* ker_attention_mask_weights_i32I (gptKernels_int8.cc.cu:815-843) */
+void lso_attention_mask_weights_i32I(const int32_t* correlation, void* output,
+                                     const int* real_seq_len, int batch, int dst_seq_len,
+                                     int src_seq_len, int head_num, float attn_scale,
+                                     float dequant_scale, int f16);
 void lso_correlation_softmax_gpt_i32I(const int32_t* correlation, void* output,
                                       const int* real_seq_len, int batch,
                                       int seq_len, int head_num, float attn_scale,

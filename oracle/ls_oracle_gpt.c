@@ -94,6 +94,43 @@ void lso_correlation_softmax_gpt_i32I(const int32_t* correlation, void* output,
   }
 }
 
+/* ker_attention_mask_weights_i32I (inference/kernels/gptKernels_int8.cc.cu:815-843): the last
+ * dst_seq_len queries over src_seq_len keys; correlation / output [batch, head_num *
+ * dst_seq_len, src_seq_len].  Rows of queries at or beyond the real length stay untouched
+ * (the kernel returns before its store, :820-823). */
+void lso_attention_mask_weights_i32I(const int32_t* correlation, void* output,
+                                     const int* real_seq_len, int batch, int dst_seq_len,
+                                     int src_seq_len, int head_num, float attn_scale,
+                                     float dequant_scale, int f16) {
+  const long rows_per_batch = (long)head_num * dst_seq_len;
+#pragma omp parallel for schedule(static)
+  for (long r = 0; r < (long)batch * rows_per_batch; ++r) {
+    int b = (int)(r / rows_per_batch);
+    int qpos = (int)(r % dst_seq_len) + src_seq_len - dst_seq_len; /* (:819) */
+    if (qpos >= real_seq_len[b]) continue;
+    long base = r * src_seq_len;
+    float mx = kFloatInfNeg;
+    for (int j = 0; j < src_seq_len && j <= qpos; ++j) { /* (:824-827) mask = j > qpos */
+      float val = (float)correlation[base + j] * attn_scale * dequant_scale * dequant_scale;
+      mx = fmaxf(mx, val);
+    }
+    double sum = 0.0;
+    for (int j = 0; j < src_seq_len && j <= qpos; ++j) {
+      float val = (float)correlation[base + j] * attn_scale * dequant_scale * dequant_scale;
+      sum += (double)expf(fmaxf(kLogitThreshMin, val - mx)); /* (:837) */
+    }
+    float fsum = (float)sum;
+    for (int j = 0; j < src_seq_len; ++j) {
+      float e = 0.f;
+      if (j <= qpos) {
+        float val = (float)correlation[base + j] * attn_scale * dequant_scale * dequant_scale;
+        e = expf(fmaxf(kLogitThreshMin, val - mx));
+      }
+      stT(output, base + j, e / (fsum + 1e-12f), f16); /* (:843), epsilon transformerKernels.h:13 */
+    }
+  }
+}
+
 void lso_arrange_qkv_with_cache_i8I_i8O(const int8_t* ori_qkv, const void* qkv_bias,
                                         int8_t* new_q, int8_t* new_k,
                                         const int8_t* k_cache, int8_t* new_v,

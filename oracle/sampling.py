@@ -137,3 +137,119 @@ def topp_sample_row(codes, p, dequant_scale, x):
     ts, ids, es = _candidates(codes, thr, dequant_scale)
     tok, amb = _choose(ts, ids, es, x)
     return tok, amb or amb0, ids, es / es.sum()
+
+
+# ---------------------------------------------------------------------------------------------
+# Encoder-decoder model: ker_topk_sample_i8I<k> / ker_topp_sample_i8I of
+# inference/kernels/transformerKernels_int8.cc.cu:1908-2290.  A logit is
+# float(code) * dequant_scale + logit_bias[id] (:1945-1947), so everything runs on float32
+# logits; the class structure, the candidate rule and the choice are those above.
+#
+# Not defined by the reference, fixed here (parity unpinned):
+# * whether the compiler fuses the product and the sum of a logit: rounded separately here;
+# * k == 1: every thread holding the maximum stores its id (:2047-2049, a race): the first id;
+# * top-p: the class maximum is formed as fmaxf(m, code * scale) + bias inside the loop over the
+#   class's ids (:2136-2137), which adds up the bias of every id; restated is the maximum of the
+#   biased logits, and the intended nucleus as for the GPT kernel.
+# ---------------------------------------------------------------------------------------------
+def biased_logits(codes, bias, dequant_scale):
+    """float32 logits of one row: the product and the sum rounded separately."""
+    prod = (np.asarray(codes, np.int8).astype(np.float32) * np.float32(dequant_scale)).astype(np.float32)
+    return (prod + np.asarray(bias).astype(np.float32)).astype(np.float32)
+
+
+def _class_max_f(logit):
+    """Per-class maximum logit (class t: ids t, t + 1024, ...); -inf = empty class."""
+    cm = np.full(THREADS, -np.inf, np.float32)
+    for t in range(min(THREADS, len(logit))):
+        cm[t] = logit[t::THREADS].max()
+    return cm
+
+
+def rough_kth_value(class_max, k):
+    """kernels/common.h:118-137 on float class maxima."""
+    warp = class_max.reshape(32, 32).max(axis=1)
+    return np.float32(min(warp[g::k].max() for g in range(k)))
+
+
+def _candidates_f(logit, thr):
+    """Step 2 (:1969-1990, :2185-2204): per class, among the ids whose logit reaches the
+    threshold, the first one with the largest exp(max(logit - max, thresh_min))."""
+    mx = logit.max()
+    ex = np.exp(np.maximum(logit - mx, np.float32(LOGIT_THRESH_MIN)).astype(np.float32)).astype(np.float32)
+    ts, ids, es = [], [], []
+    for t in range(min(THREADS, len(logit))):
+        idx = np.arange(t, len(logit), THREADS)
+        ok = logit[idx] >= thr
+        if not ok.any():
+            continue
+        cand = idx[ok]
+        j = int(np.argmax(ex[cand]))
+        ts.append(t)
+        ids.append(int(cand[j]))
+        es.append(float(ex[cand[j]]))
+    return np.array(ts), np.array(ids), np.array(es, np.float64)
+
+
+def dec_greedy_row(codes, bias, dequant_scale):
+    """k == 1: the first id of the largest logit."""
+    return int(np.argmax(biased_logits(codes, bias, dequant_scale)))
+
+
+def dec_topk_sample_row(codes, bias, k, dequant_scale, x):
+    """One row of the decoder's ``ker_topk_sample_i8I<k>``, k in {2, 4, 8, 16, 32}: (token id,
+    ambiguous, candidate ids, candidate probabilities)."""
+    logit = biased_logits(codes, bias, dequant_scale)
+    kth = rough_kth_value(_class_max_f(logit), k)
+    ts, ids, es = _candidates_f(logit, kth)
+    tok, amb = _choose(ts, ids, es, x)
+    return tok, amb, ids, es / es.sum()
+
+
+def dec_topp_threshold(class_max, p):
+    """The smallest class maximum inside the nucleus: (value, ambiguous)."""
+    srt = np.sort(class_max[np.isfinite(class_max)])[::-1]
+    ex = np.exp(np.maximum(srt - srt[0], np.float32(LOGIT_THRESH_MIN)).astype(np.float32)).astype(np.float64)
+    total = ex.sum() + (THREADS - len(srt)) * float(np.exp(np.float32(LOGIT_THRESH_MIN)))
+    pre = np.cumsum(ex)
+    inside = np.nonzero(pre <= p * total)[0]
+    amb = bool(np.any(np.abs(pre - p * total) < AMBIGUOUS * total))
+    return (np.float32(srt[inside[-1]]) if len(inside) else np.float32(srt[0])), amb
+
+
+def dec_topp_sample_row(codes, bias, p, dequant_scale, x):
+    """One row of the decoder's ``ker_topp_sample_i8I``."""
+    logit = biased_logits(codes, bias, dequant_scale)
+    thr, amb0 = dec_topp_threshold(_class_max_f(logit), p)
+    ts, ids, es = _candidates_f(logit, thr)
+    tok, amb = _choose(ts, ids, es, x)
+    return tok, amb or amb0, ids, es / es.sum()
+
+
+def dec_sample_step(logits, bias, ids, cur_len, eos_id, dequant_scale, k=0, p=0.0, seed=0, draws=None):
+    """One step of QuantDecoder::sample / ::topk_greedy_search
+    (inference/model/quant_decoder.cc.cu:952-998, 1101-1130) on ids [rows, max_step] in place:
+    a row whose last token is ``eos_id`` gets another one and draws nothing; otherwise column
+    ``cur_len`` receives the token.  ``draws`` [rows] counts the uniform numbers used per row
+    (updated).  Returns (unfinished flag, list of rows whose draw was ambiguous)."""
+    rows = ids.shape[0]
+    unfinished, ambiguous = 0, []
+    for b in range(rows):
+        if cur_len > 1 and ids[b, cur_len - 1] == eos_id:
+            ids[b, cur_len] = eos_id
+            continue
+        if k == 1:
+            tok = dec_greedy_row(logits[b], bias, dequant_scale)
+        else:
+            x = uniform_of_draw(seed, b, int(draws[b]))
+            draws[b] += 1
+            if k > 1:
+                tok, amb, _, _ = dec_topk_sample_row(logits[b], bias, k, dequant_scale, x)
+            else:
+                tok, amb, _, _ = dec_topp_sample_row(logits[b], bias, p, dequant_scale, x)
+            if amb:
+                ambiguous.append(b)
+        ids[b, cur_len] = tok
+        if tok != eos_id:
+            unfinished = 1
+    return unfinished, ambiguous

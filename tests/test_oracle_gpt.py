@@ -52,6 +52,37 @@ def test_scores_and_causal_softmax(rng):
 
 
 @pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("dst,src", [(1, 7), (4, 9), (6, 6)])
+def test_attention_mask_weights(rng, dtype, dst, src):
+    """The last `dst` queries over `src` keys against scipy's soft-max in float64 with the mask
+    written independently (key j visible to query i iff j <= i + src - dst); queries at or
+    beyond the real length keep what the output buffer held."""
+    batch, heads = 3, 2
+    corr = rng.integers(-40000, 40000, size=(batch, heads * dst, src)).astype(np.int32)
+    rsl = np.array([src, max(src - dst + 1, 1), src - 1], np.int32)
+    attn_scale, dq = np.float32(0.125), np.float32(2.0 / 127)
+    out = np.full(corr.shape, 7.0, dtype)
+    _og().attention_mask_weights_i32I(corr, rsl, heads, dst, attn_scale, dq, out)
+    x = corr.astype(np.float64) * float(attn_scale) * float(dq) * float(dq)
+    qpos = (np.arange(heads * dst) % dst) + src - dst
+    visible = np.arange(src)[None, :] <= qpos[:, None]
+    want = softmax(np.where(visible[None], x, -np.inf), axis=-1)
+    assert (qpos < rsl[0]).all() and not (qpos < rsl[2]).all()
+    for b in range(batch):
+        live = qpos < rsl[b]
+        tol = 2e-3 if dtype == np.float16 else 1e-6
+        np.testing.assert_allclose(out[b][live].astype(np.float64), want[b][live], atol=tol)
+        assert np.all(out[b][live][~visible[live]] == 0)
+        assert np.all(out[b][~live] == 7.0)
+    # a dropped scale factor or a shifted mask fails: one-hot rows where one key dominates
+    corr2 = np.zeros((1, dst, src), np.int32)
+    corr2[0, :, 0] = 30_000_000
+    out2 = np.zeros(corr2.shape, np.float32)
+    _og().attention_mask_weights_i32I(corr2, np.array([src], np.int32), 1, dst, attn_scale, dq, out2)
+    np.testing.assert_allclose(out2[0, :, 0], 1.0, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
 def test_arrange_qkv_with_cache(rng, dtype):
     batch, heads, old_len, d = 2, 3, 4, 8
     H = heads * d

@@ -123,3 +123,97 @@ def test_topp_keeps_the_largest_when_it_alone_exceeds_p():
     codes[77] = 120
     tok, amb, ids, probs = S.topp_sample_row(codes, 0.3, 0.2, 0.9)
     assert ids.tolist() == [77] and tok == 77
+
+
+# ---- encoder-decoder form: logit = code * scale + bias[id] ---------------------------------
+def _row(rng, V, spread=35):
+    return np.clip(rng.standard_normal(V) * spread, -127, 127).astype(np.int8)
+
+
+@pytest.mark.parametrize("k", [2, 4, 32])
+def test_decoder_topk_reduces_to_the_code_form_without_bias(k):
+    """With a zero bias the float route must give what the int8-code route gives (the two are
+    written separately: float thresholds and comparisons here, integer ones there)."""
+    rng = np.random.default_rng(30 + k)
+    V, scale = 4000, 0.07
+    codes = _row(rng, V)
+    for x in [0.01, 0.37, 0.99]:
+        a = S.dec_topk_sample_row(codes, np.zeros(V, np.float16), k, scale, x)
+        b = S.topk_sample_row(codes, k, scale, x)
+        assert a[0] == b[0] and a[2].tolist() == b[2].tolist()
+        np.testing.assert_allclose(a[3], b[3], rtol=1e-6)
+
+
+@pytest.mark.parametrize("p", [0.1, 0.6, 1.0])
+def test_decoder_topp_reduces_to_the_code_form_without_bias(p):
+    rng = np.random.default_rng(int(p * 10))
+    V, scale = 6000, 0.12
+    codes = _row(rng, V)
+    a = S.dec_topp_sample_row(codes, np.zeros(V, np.float32), p, scale, 0.41)
+    b = S.topp_sample_row(codes, p, scale, 0.41)
+    assert a[0] == b[0] and a[2].tolist() == b[2].tolist()
+    np.testing.assert_allclose(a[3], b[3], rtol=1e-6)
+
+
+def test_decoder_bias_enters_the_threshold_the_candidates_and_the_probabilities():
+    """Brute force in float64 with a bias large enough to reorder the ids: a route that dropped
+    the bias anywhere (class maxima, threshold test, exps) gives other candidates or weights."""
+    rng = np.random.default_rng(5)
+    V, scale, k = 3000, 0.05, 8
+    codes = _row(rng, V, 20)
+    bias = (rng.standard_normal(V) * 3).astype(np.float16)
+    logit = codes.astype(np.float64) * np.float64(np.float32(scale)) + bias.astype(np.float64)
+    tok, _, ids, probs = S.dec_topk_sample_row(codes, bias, k, scale, 0.5)
+    cmax = np.array([logit[t::1024].max() for t in range(1024)])
+    warp = cmax.reshape(32, 32).max(axis=1)
+    kth = min(warp[g::k].max() for g in range(k))
+    want = [int(np.arange(t, V, 1024)[np.argmax(logit[t::1024])]) for t in range(1024)
+            if cmax[t] >= kth - 1e-6]
+    assert sorted(ids.tolist()) == sorted(want) and len(want) >= k
+    np.testing.assert_allclose(probs, softmax(logit[ids]), rtol=2e-4)
+    assert sorted(ids.tolist()) != sorted(S.topk_sample_row(codes, k, scale, 0.5)[2].tolist())
+    # greedy: the bias decides
+    bias2 = np.zeros(V, np.float32)
+    bias2[1234] = 100.0
+    assert S.dec_greedy_row(codes, bias2, scale) == 1234
+    assert S.dec_greedy_row(np.zeros(V, np.int8), np.zeros(V, np.float32), scale) == 0  # first of ties
+
+
+def test_decoder_topp_nucleus_by_brute_force_with_bias():
+    rng = np.random.default_rng(8)
+    V, scale, p = 5000, 0.1, 0.5
+    codes = _row(rng, V, 25)
+    bias = (rng.standard_normal(V) * 2).astype(np.float32)
+    logit = S.biased_logits(codes, bias, scale).astype(np.float64)
+    cm = np.array([logit[t::1024].max() for t in range(1024)])
+    srt = np.sort(cm)[::-1]
+    ex = np.exp(np.maximum(srt - srt[0], -64.0))
+    pre, total, want = 0.0, ex.sum(), srt[0]
+    for v, e in zip(srt, ex):
+        pre += e
+        if pre > p * total:
+            break
+        want = v
+    thr, _ = S.dec_topp_threshold(S._class_max_f(logit.astype(np.float32)), p)
+    assert abs(float(thr) - want) < 1e-6
+    tok, _, ids, probs = S.dec_topp_sample_row(codes, bias, p, scale, 0.77)
+    assert (logit[ids] >= want - 1e-6).all() and tok in ids and abs(probs.sum() - 1) < 1e-9
+
+
+def test_decoder_step_keeps_ended_rows_and_reports_the_flag():
+    rng = np.random.default_rng(2)
+    V, eos, max_step = 2000, 7, 6
+    logits = np.stack([_row(rng, V) for _ in range(3)])
+    bias = np.zeros(V, np.float16)
+    ids = np.full((3, max_step), 1, np.int32)
+    ids[1, 2] = eos
+    draws = np.zeros(3, np.int64)
+    unf, _ = S.dec_sample_step(logits, bias, ids, 3, eos, 0.1, k=4, seed=11, draws=draws)
+    assert ids[1, 3] == eos and draws.tolist() == [1, 0, 1] and unf == 1
+    assert ids[0, 3] == S.dec_topk_sample_row(logits[0], bias, 4, 0.1, S.uniform_of_draw(11, 0, 0))[0]
+    # every row picks the end token: nothing unfinished
+    bias_eos = np.zeros(V, np.float32)
+    bias_eos[eos] = 1000.0
+    ids2 = np.full((3, max_step), 1, np.int32)
+    unf, _ = S.dec_sample_step(logits, bias_eos, ids2, 1, eos, 0.1, k=1)
+    assert unf == 0 and (ids2[:, 1] == eos).all()

@@ -186,3 +186,124 @@ def test_quant_gpt_with_random_sampling(tmp_path, method, topk, topp):
                 checked += 1
     assert checked >= steps
 
+
+
+# ---- encoder-decoder launchers: logit = code * scale + bias[id], ids in place ---------------
+def _dec_case(rng, batch, vocab, max_step, cur_len, eos, bias_dtype, spread=30):
+    logits = _logits(rng, batch, vocab, spread)
+    bias = (rng.standard_normal(vocab) * 2).astype(bias_dtype)
+    ids = rng.integers(eos + 1, vocab, size=(batch, max_step), dtype=np.int32)
+    return logits, bias, ids
+
+
+@pytest.mark.parametrize("bias_dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("vocab,k", [(1000, 1), (32000, 1), (1024, 2), (5000, 4), (32000, 8), (2077, 32)])
+def test_decoder_topk_sampling_launcher_against_the_oracle(rng, vocab, k, bias_dtype):
+    kk = _k()
+    batch, max_step, cur_len, eos, scale, seed = 6, 9, 4, 2, 0.09, 40 + k
+    logits, bias, ids = _dec_case(rng, batch, vocab, max_step, cur_len, eos, bias_dtype)
+    ids[2, cur_len - 1] = eos          # an ended row: another end token, no draw, no flag
+    if k == 1:
+        logits[4, :] = 5               # ties at the maximum go to the first id (bias breaks none)
+        bias_tie = bias.copy()
+        bias_tie[:] = 0
+    state = kk.rng_setup(batch, seed)
+    d_ids, d_unf = to_dev(ids), torch.zeros(1, dtype=torch.int32, device=DEV)
+    want = ids.copy()
+    draws = np.zeros(batch, np.int64)
+    for step in range(2):
+        cl = cur_len + step
+        kk.ker_topk_sample_i8I_dec_launcher(batch, cl, max_step, 1, 1024, to_dev(logits), to_dev(bias),
+                                            d_ids, None, vocab, k, d_unf, None if k == 1 else state,
+                                            eos, scale)
+        got = to_np(d_ids)
+        unf, amb = S.dec_sample_step(logits, bias, want, cl, eos, scale, k=k, seed=seed, draws=draws)
+        for b in range(batch):
+            if b in amb:
+                want[b, cl] = got[b, cl]   # a draw at a boundary of the distribution: either side
+        np.testing.assert_array_equal(got, want, err_msg="step %d" % step)
+        assert int(to_np(d_unf)[0]) == unf == 1
+    if k > 1:
+        st = to_np(state).view(np.uint32).reshape(batch, 4)
+        assert st[:, 3].tolist() == [2, 2, 0, 2, 2, 2]
+    else:
+        d2 = to_dev(ids)
+        kk.ker_topk_sample_i8I_dec_launcher(batch, cur_len, max_step, 1, 1024, to_dev(logits),
+                                            to_dev(bias_tie), d2, None, vocab, 1, d_unf, None, eos, scale)
+        assert int(to_np(d2)[4, cur_len]) == 0
+
+
+@pytest.mark.parametrize("vocab,p", [(900, 0.5), (1024, 0.9), (32000, 0.75), (7001, 1.0), (4096, 0.01)])
+def test_decoder_topp_sampling_launcher_against_the_oracle(rng, vocab, p):
+    kk = _k()
+    batch, max_step, cur_len, eos, scale, seed = 5, 6, 1, 2, 0.12, 5
+    logits, bias, ids = _dec_case(rng, batch, vocab, max_step, cur_len, eos, np.float16, spread=25)
+    logits[0, 11] = 127
+    bias[11] = 3.0                     # a row with a dominant id
+    ids[3, 0] = eos                    # cur_len == 1: the start column never ends a row (:1917)
+    state = kk.rng_setup(batch, seed)
+    d_ids, d_unf = to_dev(ids), torch.zeros(1, dtype=torch.int32, device=DEV)
+    kk.ker_topp_sample_i8I_dec_launcher(batch, cur_len, max_step, 1, 1024, to_dev(logits), to_dev(bias),
+                                        d_ids, None, vocab, p, d_unf, state, eos, scale)
+    got = to_np(d_ids)
+    np.testing.assert_array_equal(got[:, :cur_len], ids[:, :cur_len])
+    np.testing.assert_array_equal(got[:, cur_len + 1:], ids[:, cur_len + 1:])
+    for b in range(batch):
+        tok, amb, cand, _ = S.dec_topp_sample_row(logits[b], bias, p, scale, S.uniform_of_draw(seed, b, 0))
+        if not amb:
+            assert got[b, cur_len] in cand and got[b, cur_len] == tok, b
+
+
+def test_decoder_sampling_uses_the_last_logits_row_of_a_sequence(rng):
+    kk = _k()
+    batch, lsl, vocab, max_step, eos, scale = 3, 4, 3000, 5, 1, 0.1
+    logits = _logits(rng, batch * lsl, vocab)
+    bias = np.zeros(vocab, np.float32)
+    ids = np.full((batch, max_step), 7, np.int32)
+    d_ids, d_unf = to_dev(ids), torch.zeros(1, dtype=torch.int32, device=DEV)
+    kk.ker_topk_sample_i8I_dec_launcher(batch, 2, max_step, lsl, 1024, to_dev(logits), to_dev(bias),
+                                        d_ids, None, vocab, 1, d_unf, None, eos, scale)
+    got = to_np(d_ids)
+    for b in range(batch):
+        assert got[b, 2] == int(np.argmax(logits[(b + 1) * lsl - 1]))
+
+
+def test_decoder_sampling_launchers_reject_bad_arguments():
+    from lightseq_amd.lib import LSHError
+    kk = _k()
+    z8 = torch.zeros(64, dtype=torch.int8, device=DEV)
+    zi = torch.zeros(64, dtype=torch.int32, device=DEV)
+    zb = torch.zeros(16, dtype=torch.float16, device=DEV)
+    st = kk.rng_setup(2, 1)
+    with pytest.raises(LSHError, match=r"\[1,2,4,8,16,32\]"):
+        kk.ker_topk_sample_i8I_dec_launcher(2, 2, 8, 1, 1024, z8, zb, zi, None, 16, 3, zi, st, 1, 0.1)
+    with pytest.raises(LSHError, match="generator state"):
+        kk.ker_topk_sample_i8I_dec_launcher(2, 2, 8, 1, 1024, z8, zb, zi, None, 16, 4, zi, None, 1, 0.1)
+    with pytest.raises(LSHError, match="topp"):
+        kk.ker_topp_sample_i8I_dec_launcher(2, 2, 8, 1, 1024, z8, zb, zi, None, 16, 1.5, zi, st, 1, 0.1)
+    with pytest.raises(LSHError):   # the column to write lies outside the row
+        kk.ker_topk_sample_i8I_dec_launcher(2, 8, 8, 1, 1024, z8, zb, zi, None, 16, 1, zi, None, 1, 0.1)
+    with pytest.raises(LSHError, match="COL32|col32"):
+        kk.ker_topk_sample_i8I_dec_launcher(2, 2, 8, 1, 1024, z8, zb, zi, None, 16, 1, zi, None, 1, 0.1,
+                                            in_col32=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("dst,src", [(1, 640), (5, 9), (16, 16), (3, 1024)])
+def test_attention_mask_weights_launcher(rng, dtype, dst, src):
+    from oracle import gpt as og
+    kk = _k()
+    batch, heads = 3, 4
+    corr = rng.integers(-30000, 30000, size=(batch, heads * dst, src)).astype(np.int32)
+    rsl = np.array([src, max(src - dst + 1, 1), src - 1], np.int32)
+    attn_scale, dq = 0.125, 2.0 / 127
+    npdt = np.float16 if dtype == torch.float16 else np.float32
+    want = np.full(corr.shape, 3.0, npdt)
+    og.attention_mask_weights_i32I(corr, rsl, heads, dst, attn_scale, dq, want)
+    out = torch.full(corr.shape, 3.0, dtype=dtype, device=DEV)
+    kk.ker_attention_mask_weights_i32I_launcher(batch, dst, src, heads, to_dev(corr), out, to_dev(rsl),
+                                                attn_scale, dq)
+    got = to_np(out).astype(np.float32)
+    tol = 1e-3 if dtype == torch.float16 else 2e-6   # float sums run in another order
+    np.testing.assert_allclose(got, want.astype(np.float32), atol=tol)
+    np.testing.assert_array_equal(got == 3.0, want.astype(np.float32) == 3.0)  # untouched rows

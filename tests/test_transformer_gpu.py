@@ -224,11 +224,13 @@ def test_interface_and_errors(tmp_path):
     model.close()
     with pytest.raises(LSHError, match="failed"):
         LSModel("QuantTransformer", os.path.join(str(tmp_path), "missing.pb"), 2)
-    bad = dict(cfg, sampling_method="topp")
-    path2 = os.path.join(str(tmp_path), "topp.pb")
-    synthetic.write_quant_transformer(path2, bad, seed=1)
-    with pytest.raises(LSHError, match="sampling_method"):
-        LSModel("QuantTransformer", path2, 2)
+    for bad, what in [(dict(cfg, sampling_method="nucleus"), "sampling_method"),
+                      (dict(cfg, sampling_method="topk", topk=3), r"\[1,2,4,8,16,32\]"),
+                      (dict(cfg, sampling_method="topp", topp=0.0), "topp")]:
+        path2 = os.path.join(str(tmp_path), "bad.pb")
+        synthetic.write_quant_transformer(path2, bad, seed=1)
+        with pytest.raises(LSHError, match=what):
+            LSModel("QuantTransformer", path2, 2)
 
 
 def test_transformer_big_shape(oracle, tmp_path):
@@ -497,3 +499,120 @@ def test_graph_replay_of_the_steps_equals_eager(tmp_path, benchmark):
     model.graph_mode(False)
     np.testing.assert_array_equal(model.infer(ids)[0], want)
     model.close()
+
+
+def test_graph_replay_follows_a_replaced_output_buffer_and_route_switches(tmp_path):
+    """A caller may hand the model another `target_scores` buffer between two calls, and a
+    process-wide kernel switch may move after the steps were recorded: the replayed steps must
+    write where the eager steps would and run what the eager steps would."""
+    from lightseq_amd import kernels, synthetic
+    from lightseq_amd.inference import QuantTransformer
+    cfg = synthetic.transformer_config("tiny")
+    sigma = 0.02 * np.sqrt(cfg["hidden"])
+    path, _ = _make(tmp_path, cfg, 9, eos_bias=2.0 * sigma, w_std=0.2)
+    ids = _src_ids(cfg, 3, 10, 4)
+    model = QuantTransformer(path, 4)
+    want_tok, want_score = model.infer(ids)
+    model.graph_mode(True)
+    for _ in range(2):  # seen, captured
+        model.infer(ids)
+    first = model._d_outputs[1]
+    second = torch.full_like(first, 777.0)
+    model.set_output_ptr(1, second.data_ptr())
+    model._d_outputs[1] = second
+    first.fill_(-555.0)
+    torch.cuda.synchronize()
+    tok, score = model.infer(ids)
+    np.testing.assert_array_equal(tok, want_tok)
+    np.testing.assert_array_equal(score, want_score)
+    assert float(first.max()) == -555.0, "a replayed step wrote into the replaced buffer"
+    captured, _ = model.graph_stats()
+    assert captured >= 1
+    # a route switch after the capture drops the recorded steps
+    prev = kernels.gemm_i8_decode_kernel_16x16(False)
+    try:
+        tok, score = model.infer(ids)      # first sight under the new routes: eager
+        np.testing.assert_array_equal(tok, want_tok)
+        tok, score = model.infer(ids)      # captured again
+        np.testing.assert_array_equal(tok, want_tok)
+        np.testing.assert_array_equal(score, want_score)
+        assert model.graph_stats()[0] > captured
+    finally:
+        kernels.gemm_i8_decode_kernel_16x16(prev)
+    model.graph_mode(False)
+    model.close()
+
+
+@pytest.mark.parametrize("method,topk,topp,benchmark", [("topk", 4, 0.75, False), ("topk", 1, 0.75, False),
+                                                        ("topp", 1, 0.6, False), ("topk_greedy", 1, 0.75, False),
+                                                        ("topk", 8, 0.75, True)])
+def test_quant_transformer_sampling_methods(tmp_path, method, topk, topp, benchmark):
+    """QuantDecoder::sample / ::topk_greedy_search (model/quant_decoder.cc.cu:952-998, 1101-1130)
+    stage-conditionally: every token is what the sampling restatement gives for the step's
+    recorded logits, the shared bias and the (seed, row, draw) number; the run stops when no row
+    sampled anything but the end token; the same seed gives the same tokens."""
+    from lightseq_amd import synthetic
+    from lightseq_amd.inference import QuantTransformer
+    from oracle import sampling as S
+    cfg = synthetic.transformer_config("tiny")
+    cfg.update(sampling_method=method, topk=topk, topp=topp)
+    sigma = 0.02 * np.sqrt(cfg["hidden"])
+    path, msg = _make(tmp_path, cfg, 21, eos_bias=3.0 * sigma, w_std=0.2)
+    beam = cfg["beam_size"] if method == "topk_greedy" else 1   # (pywrapper/quant_transformer.cc:29-31)
+    batch = 3
+    rows = batch * beam
+    ids = _src_ids(cfg, batch, 9, 3)
+    model = QuantTransformer(path, batch)
+    assert model.get_output_max_shape(0) == [batch, beam, cfg["max_step"]]
+    model.benchmark_mode(benchmark)
+    first, _ = model.infer(ids)                       # seed 0 at load
+    model.set_seed(0)
+    rec_l = torch.zeros(cfg["max_step"], rows, cfg["trg_vocab"], dtype=torch.int8, device=DEV)
+    rec_a = torch.zeros(cfg["max_step"], rows, cfg["max_step"], dtype=torch.int32, device=DEV)
+    model.set_step_record(rec_l, rec_a, cfg["max_step"])
+    tokens, scores = model.infer(ids)
+    steps = model.steps_run()
+    np.testing.assert_array_equal(tokens, first)
+    model.set_step_record(None, None, 0)
+    model.set_seed(77)
+    other, _ = model.infer(ids)
+    model.close()
+    assert tokens.shape[:2] == (batch, beam) and scores.shape == (batch, beam)
+    if benchmark:
+        assert steps == cfg["max_step"] - 1
+    logits, alive = rec_l.cpu().numpy()[:steps], rec_a.cpu().numpy()[:steps]
+    te = msg["trg_embedding"]
+    bias = np.asarray(te["shared_bias"], np.float32).astype(np.float16)
+    scale = float(te["logits_clip_max"]) / 127.0
+    end, start = cfg["end_id"], cfg["start_id"]
+    k = topk if method == "topk" else (0 if method == "topp" else 1)
+    want = np.full((rows, cfg["max_step"]), start, np.int32)
+    draws = np.zeros(rows, np.int64)
+    checked = 0
+    for s in range(steps):
+        if method == "topk_greedy" and s == 0:
+            want = alive[0].copy()                    # the opening beam-search step (tested elsewhere)
+            for b in range(batch):                    # gives the beams of a sentence different tokens
+                assert len(set(want[b * beam:(b + 1) * beam, 1].tolist())) == beam
+            continue
+        unf, amb = S.dec_sample_step(logits[s], bias, want, s + 1, end, scale, k=k, p=topp, seed=0,
+                                     draws=draws)
+        for r in amb:
+            want[r, s + 1] = alive[s][r, s + 1]
+        np.testing.assert_array_equal(alive[s][:, :s + 2], want[:, :s + 2], err_msg="step %d" % s)
+        checked += rows - len(amb)
+        if not benchmark:
+            assert (unf == 0) == (s == steps - 1) or s == cfg["max_step"] - 2, (s, steps, unf)
+    assert checked >= steps
+    # ker_write_topk_result (kernels/transformerKernels.cc.cu:1803-1812): the sequences without
+    # the start token, the last column forced to the end token; scores are zeros here
+    out_len = tokens.shape[2]
+    # stopped early at step s: s + 1 = steps columns; every step used: max_step columns
+    assert out_len == (cfg["max_step"] if steps == cfg["max_step"] - 1 and
+                       (benchmark or unf == 1) else steps)
+    got = tokens.reshape(rows, out_len)
+    np.testing.assert_array_equal(got[:, :out_len - 1], want[:, 1:out_len])
+    assert (got[:, out_len - 1] == end).all()
+    np.testing.assert_array_equal(scores, np.zeros_like(scores))
+    if method != "topk_greedy" and k != 1:
+        assert other.shape[0] == batch  # another seed runs; its tokens may or may not differ
