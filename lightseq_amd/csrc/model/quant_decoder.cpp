@@ -226,8 +226,8 @@ void QuantDecoder::run_one_infer(int batch_size, int batch_seq_len) {
                  _tw._sampling_method == "topk_greedy";
   if (_is_sampling) {
     _batch_max_decode_length = _tw._max_step;
-    // nothing writes the scores of a sampled sequence; the reference returns its buffer as
-    // allocated, here every call returns zeros
+    // nothing writes the scores of a sampled sequence; the reference hands its buffer to the
+    // result writer as allocated, here every call starts it from zeros
     CHECK_GPU_ERROR(hipMemsetAsync(_alive_seq_score_own.get(), 0, sizeof(float) * _step_token_num,
                                    _stream));
   }
