@@ -38,8 +38,10 @@ launch against that.
 
 ``--workload transformer_big`` and ``--workload gpt2_medium`` time the two generation
 workloads (beam-search translation, greedy GPT generation) through ``QuantTransformer`` /
-``QuantGpt`` in benchmark mode and report generated tokens/s; they print a line of the
-same form without the GEMM roofline.
+``QuantGpt`` in benchmark mode: generated tokens/s over whole ``Infer()`` calls, the time of a
+decode step between HIP events on the model's stream, its launches, a roofline block (one step's
+algorithmic HBM bytes -- weights, cached keys and values, logits -- against 8 TB/s) and the CPU
+oracle on a few steps of the same width.  The default line carries both under ``generation``.
 """
 import argparse
 import json
@@ -499,71 +501,175 @@ def bench_bert(args):
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, msg, ids)
         out["cpu_baseline"]["torch_cpu"] = torch_cpu_baseline(cfg, ids)
+    if not args.no_generation:
+        # the two generation workloads, each a few whole Infer() calls (their own lines with
+        # --workload): decode-step time against the HBM roofline, the oracle beside it
+        out["generation"] = {w: bench_generation(w, steps=3, warmup=1, graphs=False,
+                                                 with_cpu=not args.no_cpu_baseline)
+                             for w in ("transformer_big", "gpt2_medium")}
     return out
 
 
-def bench_generation(args):
-    """Transformer-big beam search (batch 16 x beam 4, source 64, 64 steps) or
-    GPT-2-medium greedy generation (batch 16, prompt 512, 128 new tokens)."""
+def _generation_setup(workload):
+    """Model file, token ids and the shape figures of one generation workload."""
     import numpy as np
-    import torch
-    from lightseq_amd import inference, synthetic
+    from lightseq_amd import synthetic
     tmp = tempfile.mkdtemp(prefix="ls_bench_")
-    if args.workload == "transformer_big":
+    if workload == "transformer_big":
         cfg = synthetic.transformer_config("transformer_big")
         src_len, steps_wanted, batch = 64, 64, 16
         # decoding runs min(max_step, src + extra) - 2 steps
         cfg.update(max_step=128, extra_decode_length=steps_wanted + 2 - src_len)
         path = os.path.join(tmp, "quant_transformer_big.pb")
-        synthetic.write_quant_transformer(path, cfg, seed=0)
+        msg = synthetic.write_quant_transformer(path, cfg, seed=0)
         ids, _ = synthetic.make_token_ids(dict(vocab=cfg["src_vocab"], padding_id=0), batch, src_len,
                                           seed=0, min_len=src_len)
-        model = inference.QuantTransformer(path, batch)
-        entry = "QuantTransformer / LSModel::Infer"
         desc = ("Transformer-big-shaped int8 encoder-decoder, beam search: hidden 1024, 16 heads, "
                 "FFN 4096 ReLU, 6+6 layers, batch 16 x beam 4, source length 64, 64 decode steps, "
                 "vocab 32000, random-init weights")
+        return dict(cfg=cfg, msg=msg, path=path, ids=ids, batch=batch, src_len=src_len, desc=desc,
+                    cls="QuantTransformer")
+    cfg = synthetic.gpt_config("gpt2_medium")
+    src_len, batch = 512, 16
+    path = os.path.join(tmp, "quant_gpt2_medium.pb")
+    msg = synthetic.write_quant_gpt(path, cfg, seed=0)
+    ids = np.random.default_rng(0).integers(0, cfg["vocab"] - 1, size=(batch, src_len), dtype=np.int32)
+    desc = ("GPT-2-medium-shaped int8 decoder-only generation: 24 layers, hidden 1024, 16 heads, "
+            "FFN 4096 GELU, pre-LN, vocab 50257, batch 16, prompt 512, 128 generated tokens, "
+            "greedy, random-init weights")
+    return dict(cfg=cfg, msg=msg, path=path, ids=ids, batch=batch, src_len=src_len, desc=desc,
+                cls="QuantGpt")
+
+
+def _step_bytes(workload, cfg, batch, src_len, loop_steps):
+    """Algorithmic HBM bytes of one decode step, averaged over the steps of the loop: every int8
+    weight once, the cached keys and values the step's attention reads, the logits written and
+    read once.  (The reference also copies the whole self-attention cache every step; no
+    algorithm needs that and it is not counted.)"""
+    H, I = cfg["hidden"], cfg["inner"]
+    if workload == "transformer_big":
+        L, V, rows = cfg["n_dec_layer"], cfg["trg_vocab"], batch * cfg["beam_size"]
+        weights = L * (6 * H * H + 2 * H * I) + V * H
+        avg_len = (loop_steps + 1) / 2.0                 # step t reads t + 1 cached positions
+        cache = L * rows * 2 * H * avg_len               # int8 self-attention keys and values
+        cross = L * batch * src_len * H * 2 * 2          # fp16 cross keys and values, once per sentence
     else:
-        cfg = synthetic.gpt_config("gpt2_medium")
-        src_len, steps_wanted, batch = 512, 128, 16
-        path = os.path.join(tmp, "quant_gpt2_medium.pb")
-        synthetic.write_quant_gpt(path, cfg, seed=0)
-        rng = np.random.default_rng(0)
-        ids = rng.integers(0, cfg["vocab"] - 1, size=(batch, src_len), dtype=np.int32)
-        model = inference.QuantGpt(path, batch)
-        entry = "QuantGpt / LSModel::Infer"
-        desc = ("GPT-2-medium-shaped int8 decoder-only generation: 24 layers, hidden 1024, 16 heads, "
-                "FFN 4096 GELU, pre-LN, vocab 50257, batch 16, prompt 512, 128 generated tokens, "
-                "greedy, random-init weights")
-    os.remove(path)
+        L, V, rows = cfg["n_layer"], cfg["vocab"], batch
+        weights = L * 12 * H * H + V * H
+        avg_len = src_len + 1 + (loop_steps + 1) / 2.0   # the first loop step reads prompt + 2 positions
+        cache = L * rows * 2 * H * avg_len
+        cross = 0
+    logits = 2 * rows * V
+    return {"weights": int(weights), "self_attention_cache": int(cache), "cross_attention_kv": int(cross),
+            "logits": int(logits), "total": int(weights + cache + cross + logits)}
+
+
+def _generation_cpu_baseline(workload, setup):
+    """The C oracle on a bounded sample of the workload: the full width, depth and batch, a few
+    decode steps.  Two runs that differ only in the number of steps; their difference prices a
+    step without the encoder / prompt pass."""
+    import numpy as np
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    cfg, msg, batch = setup["cfg"], setup["msg"], setup["batch"]
+    few, more = 2, 6
+    t_all = time.perf_counter()
+    if workload == "transformer_big":
+        from oracle import oracle
+        from oracle.model_io import oracle_transformer_weights_from_message
+        enc_w, dec_w = oracle_transformer_weights_from_message(msg, cfg, np.float16)
+        ids = setup["ids"]
+        enc_out, mask, _ = oracle.quant_bert_encoder(enc_w, ids)
+        times, ran = [], []
+        for n in (few, more):
+            w = dict(dec_w, extra_decode_length=n + 2 - ids.shape[1])
+            t0 = time.perf_counter()
+            r = oracle.quant_decoder(w, enc_out, mask, is_benchmark=True)
+            times.append(time.perf_counter() - t0)
+            ran.append(r["steps_run"])
+        what = "batch %d x beam %d, source %d" % (batch, cfg["beam_size"], ids.shape[1])
+    else:
+        from oracle import gpt
+        w0 = gpt.gpt_weights_from_message(msg, cfg, np.float16)
+        prompt = 32
+        ids = setup["ids"][:, :prompt]
+        times, ran = [], []
+        for n in (few, more):
+            w = dict(w0, extra_decode_length=n + 1)     # the prompt pass gives one token, the loop n
+            t0 = time.perf_counter()
+            r = gpt.quant_gpt_sample(w, ids, is_benchmark=True)
+            times.append(time.perf_counter() - t0)
+            ran.append(r["steps_run"])
+        what = "batch %d, prompt cut to %d tokens (a step is priced by its weights)" % (batch, prompt)
+    if ran[1] <= ran[0]:  # every sequence ended on its first token: nothing to price
+        return {"value": None, "unit": "generated tokens/s (decode steps only)", "cores": cores,
+                "kind": "port", "sample": "%s: the runs stopped after %s steps" % (what, ran)}
+    per_step = (times[1] - times[0]) / (ran[1] - ran[0])
+    return {"value": batch / per_step, "unit": "generated tokens/s (decode steps only)", "cores": cores,
+            "kind": "port", "s_per_decode_step": per_step,
+            "sample": "%s, full width and depth: runs of %d and %d decode steps, a step = their "
+                      "difference / %d; %.1f s of CPU work" % (what, ran[0], ran[1], ran[1] - ran[0],
+                                                               time.perf_counter() - t_all)}
+
+
+def bench_generation(workload, steps, warmup, graphs=False, with_cpu=True):
+    """Transformer-big beam search (batch 16 x beam 4, source 64, 64 steps) or
+    GPT-2-medium greedy generation (batch 16, prompt 512, 128 new tokens): whole Infer() calls."""
+    import numpy as np
+    import torch
+    from lightseq_amd import inference
+    setup = _generation_setup(workload)
+    cfg, batch, src_len, ids = setup["cfg"], setup["batch"], setup["src_len"], setup["ids"]
+    model = getattr(inference, setup["cls"])(setup["path"], batch)
+    os.remove(setup["path"])
     model.benchmark_mode(True)
-    model.graph_mode(args.graphs)
     model._upload(ids)
-    if args.graphs:
-        for _ in range(2):  # first call: keys seen; second: graphs captured
-            model.infer_device()
-    for _ in range(args.warmup):
+    # launches of one step: the nodes of a captured step graph (two calls: keys seen, then captured)
+    model.graph_mode(True)
+    for _ in range(2):
+        model.infer_device()
+    launches = model.graph_nodes()
+    model.graph_mode(bool(graphs))
+    for _ in range(warmup):
         model.infer_device()
     torch.cuda.synchronize()
+    prep, loop, nloop = [], [], 0
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         model.infer_device()
+        a, b, nloop = model.phase_times()
+        prep.append(a)
+        loop.append(b)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     steps_run = model.steps_run()
     model.close()
-    gen_tokens = batch * steps_run
-    return {
-        "metric": "generated tokens/sec (%s)" % args.workload,
-        "value": gen_tokens * args.steps / dt, "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": 1e3 * dt / args.steps, "higher_is_better": True, "scaling": "weak",
+    ms_step = float(np.mean(loop)) / max(1, nloop)
+    nbytes = _step_bytes(workload, cfg, batch, src_len, nloop)
+    gbs = nbytes["total"] / (ms_step * 1e-3) / 1e9
+    out = {
+        "metric": "generated tokens/sec (%s)" % workload,
+        "value": batch * steps_run * steps / dt, "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": 1e3 * dt / steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "int8", "data": "synthetic",
-        "config": {"workload": desc, "batch": batch, "source_len": src_len,
-                   "decode_steps": steps_run, "ms_per_decode_step": 1e3 * dt / args.steps / steps_run,
-                   "hip_graph_steps": bool(args.graphs), "entry_point": entry},
-        "roofline": None,
+        "config": {"workload": setup["desc"], "batch": batch, "source_len": src_len,
+                   "generated_tokens_per_sequence": steps_run, "loop_steps": nloop,
+                   "ms_before_the_step_loop": float(np.mean(prep)),
+                   "ms_per_decode_step": ms_step, "launches_per_step": launches,
+                   "us_per_launch": 1e3 * ms_step / max(1, launches),
+                   "hip_graph_steps": bool(graphs),
+                   "entry_point": setup["cls"] + " / LSModel::Infer",
+                   "how": "wall clock around %d Infer() calls (value, ms_per_step); HIP events on the "
+                          "model's stream around the step loop (ms_per_decode_step)" % steps},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "one decode step (%d dependent launches)" % launches,
+                     "algorithmic_bytes_per_step": nbytes,
+                     "launch_floor_frac": None},
     }
+    if with_cpu:
+        out["cpu_baseline"] = _generation_cpu_baseline(workload, setup)
+    return out
 
 
 def main():
@@ -576,6 +682,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fused", action="store_true",
                     help="skip the stand-alone timing of the fused kernels")
+    ap.add_argument("--no-generation", action="store_true",
+                    help="default workload: skip the two generation workloads of the `generation` block")
     ap.add_argument("--graphs", action="store_true",
                     help="generation workloads: replay the steps as HIP graphs (ls_model_set_graph_mode)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -602,8 +710,12 @@ def main():
         for _ in range(3):
             torch.add(src, 1, out=dst)
         torch.cuda.synchronize()
-    out = bench_bert(args) if bert else bench_generation(args)
+    out = bench_bert(args) if bert else bench_generation(args.workload, args.steps, args.warmup,
+                                                         args.graphs, not args.no_cpu_baseline)
     print(json.dumps(out))
+    sys.stdout.flush()
+    # nothing may outlive the command: no helper thread or OpenMP team keeps the interpreter alive
+    os._exit(0)
 
 
 if __name__ == "__main__":

@@ -102,6 +102,11 @@ int ls_model_set_tap_step(ls_model* model, int step);
  * NULL).  ls_model_get_steps_run gives the number of steps the last Infer() ran. */
 int ls_model_set_step_record(ls_model* model, int8_t* logits, int* alive_seq, int max_steps);
 int ls_model_get_steps_run(ls_model* model, int* steps);
+/* Measurement aid without counterpart in the reference, QuantTransformer and QuantGpt: GPU time
+ * of the last Infer() between HIP events on the model's stream -- prepare_ms: before the step
+ * loop (QuantTransformer: the K/V projection of the encoder output; QuantGpt: the prompt pass
+ * and the first token), steps_ms: the step loop, steps: the steps it ran. */
+int ls_model_get_phase_times(ls_model* model, float* prepare_ms, float* steps_ms, int* steps);
 /* No counterpart in the reference (its step loops launch kernel by kernel:
  * model/quant_decoder.cc.cu:446-454, quant_gpt_encoder.cc.cu:361-389).  QuantTransformer and
  * QuantGpt: when on, every generation step -- embedding, the layer stack, the logits GEMM, the
@@ -113,6 +118,8 @@ int ls_model_get_steps_run(ls_model* model, int* steps);
  * ls_model_get_graph_stats: graphs captured so far, steps replayed so far. */
 int ls_model_set_graph_mode(ls_model* model, int on);
 int ls_model_get_graph_stats(ls_model* model, int* captured, long long* replayed);
+/* nodes (kernel launches and copies) of the step graph captured last: the launches of one step */
+int ls_model_get_graph_nodes(ls_model* model, int* nodes);
 
 /* QuantGpt with sampling_method topk (topk > 1) or topp, QuantTransformer with sampling_method
  * topk or topp (model/quant_decoder.cc.cu:952-998): restart the per-sequence generator

@@ -321,6 +321,38 @@ int ls_model_get_graph_stats(ls_model* model, int* captured, long long* replayed
                        "graph mode applies to the generation steps of QuantTransformer and QuantGpt");
 }
 
+int ls_model_get_graph_nodes(ls_model* model, int* nodes) {
+  NEED_MODEL(model);
+  if (!nodes) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");
+  if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get())) {
+    *nodes = qg->encoder()->graph_nodes();
+    return LSH_OK;
+  }
+  if (QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get())) {
+    *nodes = qt->decoder()->graph_nodes();
+    return LSH_OK;
+  }
+  return lsh::lsh_fail(LSH_ERR_UNSUPPORTED,
+                       "graph mode applies to the generation steps of QuantTransformer and QuantGpt");
+}
+
+int ls_model_get_phase_times(ls_model* model, float* prepare_ms, float* steps_ms, int* steps) {
+  NEED_MODEL(model);
+  if (!prepare_ms || !steps_ms || !steps) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");
+  const lightseq::hip::PhaseEvents* ph = nullptr;
+  if (QuantGpt* qg = dynamic_cast<QuantGpt*>(model->impl.get())) ph = &qg->encoder()->phases();
+  if (QuantTransformer* qt = dynamic_cast<QuantTransformer*>(model->impl.get()))
+    ph = &qt->decoder()->phases();
+  if (!ph)
+    return lsh::lsh_fail(LSH_ERR_UNSUPPORTED,
+                         "phase times exist for the generation models QuantTransformer and QuantGpt");
+  bool have = false;
+  const int rc = guarded([&] { have = ph->times(prepare_ms, steps_ms, steps); });
+  if (rc != LSH_OK) return rc;
+  if (!have) return lsh::lsh_fail(LSH_ERR_INVALID, "no generation run has completed yet");
+  return LSH_OK;
+}
+
 int ls_model_get_steps_run(ls_model* model, int* steps) {
   NEED_MODEL(model);
   if (!steps) return lsh::lsh_fail(LSH_ERR_INVALID, "null pointer");

@@ -89,6 +89,38 @@ class StreamOwner {
   hipStream_t s_ = nullptr;
 };
 
+// Three HIP events on the model's stream per Infer() of a generation model: entry, start of the
+// step loop, end of the step loop.  times() is valid once the stream has been synchronised.
+class PhaseEvents {
+ public:
+  PhaseEvents() = default;
+  PhaseEvents(const PhaseEvents&) = delete;
+  PhaseEvents& operator=(const PhaseEvents&) = delete;
+  ~PhaseEvents() {
+    for (hipEvent_t e : ev_)
+      if (e) (void)hipEventDestroy(e);
+  }
+  void mark(int i, hipStream_t s) {
+    if (!ev_[i]) CHECK_GPU_ERROR(hipEventCreate(&ev_[i]));
+    CHECK_GPU_ERROR(hipEventRecord(ev_[i], s));
+    if (i == 0) loop_steps_ = 0;
+    marked_ |= 1 << i;
+  }
+  void set_loop_steps(int n) { loop_steps_ = n; }
+  // milliseconds before the step loop and inside it, steps the loop ran; false before a run
+  bool times(float* prepare_ms, float* steps_ms, int* steps) const {
+    if (marked_ != 7) return false;
+    CHECK_GPU_ERROR(hipEventElapsedTime(prepare_ms, ev_[0], ev_[1]));
+    CHECK_GPU_ERROR(hipEventElapsedTime(steps_ms, ev_[1], ev_[2]));
+    *steps = loop_steps_;
+    return true;
+  }
+
+ private:
+  hipEvent_t ev_[3] = {nullptr, nullptr, nullptr};
+  int marked_ = 0, loop_steps_ = 0;
+};
+
 // Debug taps of a generation step (parity bisection): device-to-device copies of named
 // intermediates of decoder layer `layer` at step `step` into buffers the caller owns.  A name
 // registered with a null pointer is forgotten.  A layer < 0 at the copy site means "any".
@@ -144,6 +176,7 @@ class StepGraphs {
   int captured() const { return captured_; }
   long replayed() const { return replayed_; }
   size_t held() const { return execs_.size(); }
+  int last_graph_nodes() const { return last_nodes_; }  // launches of the step captured last
   static constexpr size_t kMaxGraphs = 512;
 
   template <typename Body>
@@ -214,6 +247,8 @@ class StepGraphs {
       if (graph) (void)hipGraphDestroy(graph);
       return nullptr;
     }
+    size_t nodes = 0;
+    if (hipGraphGetNodes(graph, nullptr, &nodes) == hipSuccess) last_nodes_ = (int)nodes;
     hipGraphExec_t exec = nullptr;
     const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
@@ -227,7 +262,7 @@ class StepGraphs {
   std::list<uint64_t> lru_;  // most recently launched first
   std::unordered_set<uint64_t> seen_, eager_only_;
   unsigned long epoch_ = 0;
-  int captured_ = 0;
+  int captured_ = 0, last_nodes_ = 0;
   long replayed_ = 0;
 };
 

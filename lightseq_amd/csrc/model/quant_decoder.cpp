@@ -238,16 +238,20 @@ void QuantDecoder::run_one_infer(int batch_size, int batch_seq_len) {
   _alive_cur = 0;
   _cache_cur = 0;
 
+  _phases.mark(0, _stream);
   project_encoder_output();
   CHECK_GPU_ERROR(hipMemcpyAsync(_alive_seq_probs.get(), _h_alive_seq_probs.data(),
                                  sizeof(float) * _step_token_num, hipMemcpyHostToDevice,
                                  _stream));
 
   /* ---step2. autoregressive decoding--- */
+  _phases.mark(1, _stream);
   for (_cur_step = 0; _cur_step < _batch_max_decode_length - 1; _cur_step++) {
     bool early_stop = run_step();
     if (!_is_benchmark && early_stop) break;
   }
+  _phases.mark(2, _stream);
+  _phases.set_loop_steps(_steps_run);
 
   /* ---step3. output the decoding result--- */
   // The steps keep the scores of finished beams in the decoder's own buffer: a step may be a

@@ -44,6 +44,8 @@ class QuantDecoder {
     _rec_max_steps = max_steps;
   }
   int steps_run() const { return _steps_run; }
+  // event times of the last run_one_infer: the K/V projection of the encoder output, the steps
+  const PhaseEvents& phases() const { return _phases; }
   // Replay decoding steps through HIP graphs, one per (batch, source length, step, buffer
   // parity): see StepGraphs.  Off while a step record is set.
   void graph_mode(bool on) { _use_graphs = on; }
@@ -51,6 +53,7 @@ class QuantDecoder {
   StepTaps step_taps;
   int graphs_captured() const { return _graphs.captured(); }
   long graphs_replayed() const { return _graphs.replayed(); }
+  int graph_nodes() const { return _graphs.last_graph_nodes(); }
 
   const int* _p_d_padding_mask;
   const __half* _p_d_encoder_output;
@@ -81,6 +84,7 @@ class QuantDecoder {
   bool _is_benchmark = false;
   bool _use_graphs = false;
   StepGraphs _graphs;
+  PhaseEvents _phases;
 
   int _batch_size = 0, _batch_seq_len = 0, _batch_token_num = 0, _step_token_num = 0;
   int _batch_max_decode_length = 0, _layer_id = 0, _steps_run = 0;

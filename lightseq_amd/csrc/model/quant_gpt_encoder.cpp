@@ -340,6 +340,7 @@ int QuantGptEncoder::run_one_sample(int batch_size, int batch_seq_len) {
   _steps_run = 0;
   const int H = _tw._hidden_size;
 
+  _phases.mark(0, _stream);
   // ids [batch, max_step] <- prompt
   CHECK_GPU_ERROR(hipMemcpy2DAsync(_ids.get(), sizeof(int) * _tw._max_step, _p_d_token_id,
                                    sizeof(int) * batch_seq_len, sizeof(int) * batch_seq_len,
@@ -350,11 +351,15 @@ int QuantGptEncoder::run_one_sample(int batch_size, int batch_seq_len) {
                                    _buf_a.get() + (size_t)(batch_seq_len - 1) * H,
                                    (size_t)batch_seq_len * H, H, batch_size,
                                    hipMemcpyDeviceToDevice, _stream));
+  int loop_steps = 0;
   if (_batch_seq_len < _tw._max_step) {
     // (:347-353) after the prompt pass the run ends when nothing is unfinished
     enqueue_sampling(_hid_last.get(), true);
-    if (!(finish_token() == 0 || _batch_seq_len >= _batch_max_seq_len)) {
+    const bool go_on = !(finish_token() == 0 || _batch_seq_len >= _batch_max_seq_len);
+    _phases.mark(1, _stream);
+    if (go_on) {
       while (_batch_seq_len < _batch_max_seq_len) {
+        ++loop_steps;
         // the launches of a step depend on the batch size and the position only
         const uint64_t key = ((uint64_t)_batch_size << 32) | (uint32_t)_batch_seq_len;
         _graphs.run(key, _stream, _use_graphs && !_rec_logits && !step_taps.any(),
@@ -363,7 +368,11 @@ int QuantGptEncoder::run_one_sample(int batch_size, int batch_seq_len) {
         if (!unfinished && !_is_benchmark) break;
       }
     }
+  } else {
+    _phases.mark(1, _stream);
   }
+  _phases.mark(2, _stream);
+  _phases.set_loop_steps(loop_steps);
   CHECK_GPU_ERROR(hipMemcpy2DAsync(_p_d_sample_id, sizeof(int) * _batch_seq_len, _ids.get(),
                                    sizeof(int) * _tw._max_step, sizeof(int) * _batch_seq_len,
                                    batch_size, hipMemcpyDeviceToDevice, _stream));

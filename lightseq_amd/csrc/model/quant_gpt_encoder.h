@@ -44,6 +44,8 @@ class QuantGptEncoder {
     _rec_max_steps = max_steps;
   }
   int steps_run() const { return _steps_run; }
+  // event times of the last run_one_sample: the prompt pass with the first token, the cached steps
+  const PhaseEvents& phases() const { return _phases; }
   // Replay the cached steps through HIP graphs, one per (batch size, position): see StepGraphs.
   // Off while a step record is set.
   void graph_mode(bool on) { _use_graphs = on; }
@@ -51,6 +53,7 @@ class QuantGptEncoder {
   StepTaps step_taps;
   int graphs_captured() const { return _graphs.captured(); }
   long graphs_replayed() const { return _graphs.replayed(); }
+  int graph_nodes() const { return _graphs.last_graph_nodes(); }
 
   const int* _p_d_token_id;
   float* _p_d_ppl;
@@ -76,6 +79,7 @@ class QuantGptEncoder {
 
   int _batch_size = 0, _batch_seq_len = 0, _batch_token_num = 0, _batch_max_seq_len = 0;
   int _layer_id = 0, _steps_run = 0;
+  PhaseEvents _phases;
   long _max_batch_dim;
   int* _h_unfinished = nullptr;  // pinned
   int8_t* _rec_logits = nullptr;

@@ -55,11 +55,13 @@ def _bind():
         "ls_model_set_tap_step": [_P, _I],
         "ls_model_set_profiling": [_P, _I],
         "ls_model_get_profile": [_P, ctypes.c_char_p, _I],
+        "ls_model_get_phase_times": [_P, _P, _P, _P],
         "ls_model_set_step_record": [_P, _P, _P, _I],
         "ls_model_get_steps_run": [_P, ip],
         "ls_model_set_graph_mode": [_P, _I],
         "ls_model_set_seed": [_P, ctypes.c_uint64],
         "ls_model_get_graph_stats": [_P, ip, ctypes.POINTER(ctypes.c_longlong)],
+        "ls_model_get_graph_nodes": [_P, ip],
     }
     for name, argtypes in sigs.items():
         fn = getattr(L, name)
@@ -174,6 +176,14 @@ class LSModel:
         self._call("ls_model_get_profile", self._h, buf, 8192)
         return json.loads(buf.value.decode())
 
+    def phase_times(self):
+        """Generation models: (milliseconds before the step loop, milliseconds inside it, steps
+        the loop ran) of the last ``Infer()``, between HIP events on the model's stream."""
+        a, b, n = ctypes.c_float(0), ctypes.c_float(0), ctypes.c_int(0)
+        self._call("ls_model_get_phase_times", self._h, ctypes.byref(a), ctypes.byref(b),
+                   ctypes.byref(n))
+        return a.value, b.value, n.value
+
     def graph_mode(self, flag):
         """QuantTransformer / QuantGpt: replay generation steps as HIP graphs."""
         self._call("ls_model_set_graph_mode", self._h, int(bool(flag)))
@@ -181,6 +191,10 @@ class LSModel:
     def set_seed(self, seed):
         """QuantGpt with random sampling (topk > 1, topp): restart the generator states."""
         self._call("ls_model_set_seed", self._h, int(seed) & 0xFFFFFFFFFFFFFFFF)
+
+    def graph_nodes(self):
+        """Launches of one generation step: the nodes of the step graph captured last."""
+        return self._int("ls_model_get_graph_nodes")
 
     def graph_stats(self):
         """(graphs captured, steps replayed) so far."""

@@ -527,6 +527,9 @@ def test_graph_replay_of_the_steps_equals_eager(tmp_path, benchmark):
     model.set_step_record(rec, cfg["max_step"])
     np.testing.assert_array_equal(model.sample(ids), want)
     assert model.graph_stats()[1] == replayed
+    assert model.graph_nodes() >= 7 * cfg["n_layer"]
+    prepare_ms, steps_ms, loop_steps = model.phase_times()
+    assert loop_steps == model.steps_run() - 1 and steps_ms > 0 and prepare_ms > 0
     model.graph_mode(False)
     model.set_step_record(None, 0)
     np.testing.assert_array_equal(model.sample(ids), want)

@@ -496,6 +496,10 @@ def test_graph_replay_of_the_steps_equals_eager(tmp_path, benchmark):
             np.testing.assert_array_equal(model.infer(other)[0], want_other)
     captured, replayed = model.graph_stats()
     assert captured >= 1 and replayed >= 3 * captured, (captured, replayed)
+    # measurement aids: the launches of a step and the event times around the step loop
+    assert model.graph_nodes() >= 10 * cfg["n_dec_layer"]
+    prepare_ms, steps_ms, loop_steps = model.phase_times()
+    assert loop_steps == model.steps_run() and steps_ms > 0 and prepare_ms > 0
     model.graph_mode(False)
     np.testing.assert_array_equal(model.infer(ids)[0], want)
     model.close()
