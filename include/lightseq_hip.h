@@ -275,6 +275,35 @@ int lsh_gemm_i8_residual_ln_i8O_f16(const int8_t* A, const int8_t* w_tiled, floa
                                     int8_t* output, void* residual, int batch_tokens,
                                     int hidden_size, int k, float dequant_scale, float quant_scale,
                                     lsh_stream_t stream, int is_post_ln);
+/* The feed-forward half of an encoder layer as one launch, no counterpart in the reference
+ * (it replaces three launches of model/quant_bert_encoder.cc.cu:414-520 and leaves their bytes):
+ *   act = lut1[ requant(x W1^T, alpha1) ]       int8 [m, inner]   (lsh_gemm_i8_lut_i8o)
+ *   acc = act W2^T                              int32 [m, hidden] (lsh_gemm_i8_i32o)
+ *   final_ln == 0: lsh_ker_residual_bias_ln_i32I_i8O_f16(acc, scale, bias, residual_bias, out_q,
+ *                  residual, ..., is_post_ln, colsum);
+ *   final_ln != 0: lsh_ker_residual_bias_ln_i32I_f16(acc, scale, bias, residual, out_t, ...,
+ *                  colsum) (out_t may alias residual; residual_bias and out_q unused).
+ * The token rows are dealt to the GPU's 8 XCDs; the 32 workgroups of an XCD wait for one another
+ * between the three phases through the L2 they share.  Needs a GPU of 256 compute units that
+ * each hold a workgroup of the kernel (otherwise LSH_ERR_UNSUPPORTED), hidden and inner
+ * multiples of 128, hidden <= 1024, m >= 8.
+ * sync: lsh_ffn_segment_sync_words() uint32 words of device memory that the caller zeroes
+ * once; *launches: the caller's count of launches that used `sync` (starts at 0, advanced by
+ * the call).  Every wait inside the kernel is bounded by spin_limit polls (about a microsecond
+ * each): if the workgroups cannot all become resident -- another kernel of this kind running
+ * at the same time -- the kernel gives up, sets sync[words - 1] (bit 0: a wait gave up, bit 1:
+ * a workgroup found itself on another XCD than its index says) and ends; the outputs are then
+ * undefined, and `sync` and *launches must be zeroed before the next call.  Calls that overlap
+ * on one GPU must not share `sync`. */
+size_t lsh_ffn_segment_sync_words(void);
+int lsh_ffn_segment_supported(int m, int hidden, int inner);
+int lsh_ffn_segment_i8_f16(const int8_t* x, const int8_t* w1, const int8_t* lut1, float alpha1,
+                           int8_t* act, const int8_t* w2, int32_t* acc, void* residual, void* out_t,
+                           int8_t* out_q, const void* scale, const void* bias,
+                           const void* residual_bias, const void* colsum, int m, int hidden,
+                           int inner, float dequant_scale, float quant_scale, int is_post_ln,
+                           int final_ln, uint32_t* sync, uint32_t* launches, int spin_limit,
+                           lsh_stream_t stream);
 /* Measurement aid, no counterpart in the reference: one launch of `workgroups` x 4 wavefronts
  * that issue nothing but independent int8 MFMAs (v_mfma_i32_32x32x32_i8) on register-resident
  * operands, `iters` x 8 each.  out: workgroups * 256 ints (checksums, so that nothing is

@@ -146,6 +146,22 @@ int lsh_gemm_i8_residual_ln_i8O_f16(const int8_t* A, const int8_t* w_tiled, floa
                                          output, HM(residual), batch_tokens, hidden_size, k,
                                          dequant_scale, quant_scale, HS(stream), is_post_ln != 0);
 }
+size_t lsh_ffn_segment_sync_words(void) { return ffn_segment_sync_words(); }
+int lsh_ffn_segment_supported(int m, int hidden, int inner) {
+  return ffn_segment_supported(m, hidden, inner) ? 1 : 0;
+}
+int lsh_ffn_segment_i8_f16(const int8_t* x, const int8_t* w1, const int8_t* lut1, float alpha1,
+                           int8_t* act, const int8_t* w2, int32_t* acc, void* residual, void* out_t,
+                           int8_t* out_q, const void* scale, const void* bias,
+                           const void* residual_bias, const void* colsum, int m, int hidden,
+                           int inner, float dequant_scale, float quant_scale, int is_post_ln,
+                           int final_ln, uint32_t* sync, uint32_t* launches, int spin_limit,
+                           lsh_stream_t stream) {
+  return ffn_segment_i8(x, w1, lut1, alpha1, act, w2, acc, HM(residual), HM(out_t), out_q, H(scale),
+                        H(bias), H(residual_bias), H(colsum), m, hidden, inner, dequant_scale,
+                        quant_scale, is_post_ln != 0, final_ln != 0, sync, launches, spin_limit,
+                        HS(stream));
+}
 int lsh_mfma_i8_peak_probe(int* out, int workgroups, int iters, double* ops, lsh_stream_t stream) {
   return mfma_i8_peak_probe(out, workgroups, iters, ops, HS(stream));
 }

@@ -37,6 +37,7 @@
 #include "ls_device.cuh"
 #include "ls_launch.h"
 #include "tile_common.cuh"
+#include "gemm_tile.cuh"
 
 #include <hip/hip_ext.h>
 
@@ -49,82 +50,6 @@
 namespace lsh {
 
 constexpr int kBM = 128, kBN = 128;
-
-// ---------------------------------------------------------------------------------
-// Epilogues.  store16(m, n, N, c, full): c[0..15] are C[m, n .. n+15]; `full` means all
-// 16 columns exist and the vector path may be used.
-// ---------------------------------------------------------------------------------
-struct EpiI32 {
-  int32_t* C;
-  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
-    int32_t* p = C + m * N + n;
-    if (full) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        *reinterpret_cast<int4*>(p + 4 * q) =
-            make_int4(c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (n + i < N) p[i] = c[i];
-    }
-  }
-  // one element (the decode-step kernels give every thread one element of a 16 x 16 block)
-  struct Pre1 {};
-  __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
-  struct Blk1 {
-    int n;
-  };
-  __device__ __forceinline__ Blk1 block1(int n) const { return Blk1{n}; }
-  __device__ __forceinline__ void store1(long m, Blk1 blk, int N, int acc, Pre1, const int8_t*,
-                                         int) const {
-    C[m * N + blk.n] = acc;
-  }
-  bool vec_ok(int N) const { return N % 4 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
-  static const char* name() { return "EpiI32"; }
-};
-
-__device__ __forceinline__ void store16_i8(int8_t* p, int n, int N, const int (&q)[16], bool full) {
-  if (full) {
-    uint4 o;
-    o.x = pack4_i8(q[0], q[1], q[2], q[3]);
-    o.y = pack4_i8(q[4], q[5], q[6], q[7]);
-    o.z = pack4_i8(q[8], q[9], q[10], q[11]);
-    o.w = pack4_i8(q[12], q[13], q[14], q[15]);
-    *reinterpret_cast<uint4*>(p) = o;
-  } else {
-#pragma unroll
-    for (int i = 0; i < 16; ++i)
-      if (n + i < N) p[i] = (int8_t)q[i];
-  }
-}
-
-struct EpiI8 {
-  int8_t* C;
-  float alpha;
-  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
-    if (full) {
-      *reinterpret_cast<uint4*>(C + m * N + n) = requant16_packed(c, alpha);
-      return;
-    }
-    int q[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) q[i] = requant_acc(c[i], alpha);
-    store16_i8(C + m * N + n, n, N, q, full);
-  }
-  struct Pre1 {};
-  __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
-  struct Blk1 {
-    int n;
-  };
-  __device__ __forceinline__ Blk1 block1(int n) const { return Blk1{n}; }
-  __device__ __forceinline__ void store1(long m, Blk1 blk, int N, int acc, Pre1, const int8_t*,
-                                         int) const {
-    C[m * N + blk.n] = (int8_t)requant_acc_fast(acc, alpha);
-  }
-  bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
-  static const char* name() { return "EpiI8"; }
-};
 
 // n / d for 0 <= n < 2^24, d > 0, with inv = 1.0f / d from the host: the float product is
 // within one of the quotient, the remainder decides.  A handful of instructions where the
@@ -341,57 +266,6 @@ struct EpiActI8 {
   }
   static const char* name() { return ACT == kActGelu ? "EpiGeluI8" : "EpiReluI8"; }
 };
-
-// The same epilogue through a table.  After the requantisation an element is one of 255
-// codes, and what follows (dequantise, add the column's bias, activation, requantise)
-// depends only on that code and the column: table[n][code + 128], N x 256 bytes built once
-// per weight matrix by build_act_lut with the very device function EpiActI8 evaluates, so
-// the result is bit-identical.  The bias + GELU arithmetic costs ~35 vector instructions per
-// element -- more than the matrix cores spend on a K = 768 product -- while the lookup is
-// one byte load per element from a table that stays in L2 (768 KB for N = 3072); the lanes
-// of one load instruction read two table rows, i.e. a handful of cache lines.
-struct EpiLutI8 {
-  int8_t* C;
-  const int8_t* lut;
-  float alpha;
-  __device__ __forceinline__ void store16(long m, int n, int N, const v16i& c, bool full) const {
-    int q[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int col = n + i < N ? n + i : N - 1;
-      q[i] = lut[(long)col * 256 + requant_acc(c[i], alpha) + 128];
-    }
-    store16_i8(C + m * N + n, n, N, q, full);
-  }
-  // the same with the table rows of the tile's columns staged in LDS (`tab`: 256 bytes per
-  // column, first row = the tile's first column; n_local = n - first column)
-  __device__ __forceinline__ void store16_lds(long m, int n, int N, const v16i& c, bool full,
-                                              const int8_t* tab, int n_local) const {
-    int q[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i)
-      q[i] = tab[(n_local + i) * 256 + requant_acc_fast(c[i], alpha) + 128];
-    store16_i8(C + m * N + n, n, N, q, full);
-  }
-  // one element, the table rows of the workgroup's columns staged in LDS (n_local: the
-  // element's column among them)
-  struct Pre1 {};
-  __device__ __forceinline__ Pre1 prefetch1(int) const { return Pre1{}; }
-  struct Blk1 {
-    int n;
-  };
-  __device__ __forceinline__ Blk1 block1(int n) const { return Blk1{n}; }
-  __device__ __forceinline__ void store1(long m, Blk1 blk, int N, int acc, Pre1,
-                                         const int8_t* tab, int n_local) const {
-    C[m * N + blk.n] = tab[n_local * 256 + requant_acc_fast(acc, alpha) + 128];
-  }
-  bool vec_ok(int N) const { return N % 16 == 0 && (reinterpret_cast<uintptr_t>(C) & 15u) == 0; }
-  static const char* name() { return "EpiLutI8"; }
-};
-
-template <typename Epi>
-__device__ __forceinline__ const int8_t* epi_lut(const Epi&) { return nullptr; }
-__device__ __forceinline__ const int8_t* epi_lut(const EpiLutI8& e) { return e.lut; }
 
 template <int ACT>
 __global__ void __launch_bounds__(256)
@@ -884,179 +758,15 @@ template <typename Epi, int WGM, int WGN, int MB, int NB, int NST>
 __global__ void __launch_bounds__(64 * WGM * WGN)
 gemm_i8_tile_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W, Epi epi, int M,
                     int N, int K, int tiles_m, int tiles_n, bool, int) {
-  constexpr bool LUT = std::is_same<Epi, EpiLutI8>::value;
-  constexpr int NWV = WGM * WGN;
-  constexpr int TM = WGM * MB * 32, TN = WGN * NB * 32;
-  constexpr int STAGE = (TM + TN) * kBK;
-  constexpr int NA = TM / 8 / NWV, NW = TN / 8 / NWV, PER = NA + NW;  // 1-KB loads per wavefront
-  constexpr int NTAB = TN / 4 / NWV;  // table loads per wavefront
-  static_assert(TM % (8 * NWV) == 0 && TN % (8 * NWV) == 0, "stage rows split over the wavefronts");
-  static_assert((NST - 1) * PER < 64, "vmcnt range");
-  static_assert(!LUT || (TM >= TN && TN % (4 * NWV) == 0), "table fits a freed stage");
   extern __shared__ __align__(16) int8_t smem[];
   // the operand pointers are wanted in registers here, so that their kernel-argument load
   // leaves with the one for the shape instead of after the tile arithmetic that needs the shape
   // (the tile arithmetic below is made to wait for them)
   asm volatile("" : "+s"(tiles_m) : "s"(A), "s"(W));
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave / WGN, wn = wave % WGN, l32 = lane & 31, g = lane >> 5;
+  constexpr int TM = WGM * MB * 32;
   int tm, tn;
   tile_of(blockIdx.x, tiles_m * tiles_n, tiles_m, tiles_n, tm, tn);
-  const int nk = K / kBK;
-
-  uint32_t a_src[NA], w_src[NW];
-#pragma unroll
-  for (int i = 0; i < NA; ++i) {
-    const int row = (wave + NWV * i) * 8 + (lane >> 3);
-    const int c = (lane & 7) ^ key_act(row);
-    a_src[i] = (uint32_t)min(tm * TM + row, M - 1) * (uint32_t)K + c * 16;
-  }
-#pragma unroll
-  for (int i = 0; i < NW; ++i) {
-    const int row = (wave + NWV * i) * 8 + (lane >> 3);
-    const int c = (lane & 7) ^ key_wgt(row);
-    w_src[i] = (uint32_t)min(tn * TN + row, N - 1) * (uint32_t)K + c * 16;
-  }
-  const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
-  auto dma1 = [&](const int8_t* base, uint32_t voff, uint32_t lds) {
-    lds = __builtin_amdgcn_readfirstlane(lds);
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff),
-                 "s"(base)
-                 : "memory");
-  };
-  auto issue = [&](int kt, int slot) {  // K step kt into ring slot `slot`
-    const uint32_t base = lds0 + slot * STAGE;
-#pragma unroll
-    for (int i = 0; i < NA; ++i) dma1(A + kt * kBK, a_src[i], base + (wave + NWV * i) * 1024);
-#pragma unroll
-    for (int i = 0; i < NW; ++i)
-      dma1(W + kt * kBK, w_src[i], base + TM * kBK + (wave + NWV * i) * 1024);
-  };
-  // LDS byte offset of this lane's fragment chunk for K slice 0; slice ks is at (offset ^ (ks << 5)):
-  // chunk index 2 * ks + g, swizzled by the row key, and 2 * ks only touches bits 1-2 of it
-  int a_base[MB], w_base[NB];
-#pragma unroll
-  for (int i = 0; i < MB; ++i) {
-    const int row = wm * (MB * 32) + i * 32 + l32;
-    a_base[i] = row * kBK + ((g ^ key_act(row)) << 4);
-  }
-#pragma unroll
-  for (int j = 0; j < NB; ++j) {
-    const int row = wn * (NB * 32) + j * 32 + sigma(l32);
-    w_base[j] = TM * kBK + row * kBK + ((g ^ key_wgt(row)) << 4);
-  }
-  struct Frag {
-    v4i a[MB], w[NB];
-  };
-  auto load_frag = [&](Frag& f, const int8_t* stage, int ks) {
-#pragma unroll
-    for (int i = 0; i < MB; ++i)
-      f.a[i] = *reinterpret_cast<const v4i*>(stage + (a_base[i] ^ (ks << 5)));
-#pragma unroll
-    for (int j = 0; j < NB; ++j)
-      f.w[j] = *reinterpret_cast<const v4i*>(stage + (w_base[j] ^ (ks << 5)));
-  };
-  v16i acc[MB][NB];
-#pragma unroll
-  for (int i = 0; i < MB; ++i)
-#pragma unroll
-    for (int j = 0; j < NB; ++j) acc[i][j] = (v16i)0;
-  auto mma = [&](const Frag& f) {
-#pragma unroll
-    for (int i = 0; i < MB; ++i)
-#pragma unroll
-      for (int j = 0; j < NB; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[j], f.a[i], acc[i][j], 0, 0, 0);
-  };
-  // issue order of one slice: an LDS read of the next slice after each of the first MFMAs
-  auto pattern = [&]() {
-#pragma unroll
-    for (int q = 0; q < MB + NB; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    if (MB * NB > MB + NB) __builtin_amdgcn_sched_group_barrier(0x008, MB * NB - (MB + NB), 0);
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  Frag f[2];
-  auto slices = [&](const int8_t* stage) {  // slices 1..3 read, slices 0..2 multiplied
-#pragma unroll
-    for (int ks = 1; ks < 4; ++ks) {
-      load_frag(f[ks & 1], stage, ks);
-      mma(f[(ks - 1) & 1]);
-      pattern();
-    }
-  };
-
-#pragma unroll
-  for (int s = 0; s < NST; ++s) issue(s, s);
-  wait_vmcnt<(NST - 1) * PER>();
-  __builtin_amdgcn_s_barrier();
-  load_frag(f[0], smem, 0);
-  int slot = 0;
-  // steady state: a step ends by refilling its own slot with step kt + NST
-  for (int kt = 0; kt < nk - NST; ++kt) {
-    slices(smem + slot * STAGE);
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront has read all of the stage
-    wait_vmcnt<(NST - 2) * PER>();       // its own loads of step kt + 1 have landed ...
-    __builtin_amdgcn_s_barrier();        // ... and everyone's; everyone is done with step kt
-    issue(kt + NST, slot);
-    __builtin_amdgcn_sched_barrier(0);
-    if (++slot == NST) slot = 0;
-    load_frag(f[0], smem + slot * STAGE, 0);
-    mma(f[1]);
-    pattern();
-  }
-  // drain: NST - 1 steps without a refill, then the last step
-  int tab_slot = 0;
-#pragma unroll
-  for (int t = 0; t < NST - 1; ++t) {
-    slices(smem + slot * STAGE);
-    __builtin_amdgcn_s_waitcnt(0xC07F);
-    if (NST - 2 - t == 0) wait_vmcnt<0>();
-    else if (NST - 2 - t == 1) wait_vmcnt<PER>();
-    else wait_vmcnt<2 * PER>();
-    __builtin_amdgcn_s_barrier();
-    if (LUT && t == NST - 2) {
-      // the slot of the second-to-last step is free: the tile's table rows go there
-      tab_slot = slot;
-      const long first = (long)tn * TN * 256, last = (long)N * 256 - 16;
-#pragma unroll
-      for (int i = 0; i < NTAB; ++i) {
-        const int q = wave + NWV * i;
-        const long off = min(first + q * 1024 + lane * 16, last);  // rows beyond N: never stored
-        dma1(reinterpret_cast<const int8_t*>(epi_lut(epi)), (uint32_t)off,
-             lds0 + slot * STAGE + q * 1024);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (++slot == NST) slot = 0;
-    load_frag(f[0], smem + slot * STAGE, 0);
-    mma(f[1]);
-    pattern();
-  }
-  slices(smem + slot * STAGE);
-  mma(f[1]);
-  if (LUT) {
-    wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-  }
-  const int8_t* tab = smem + tab_slot * STAGE;
-#pragma unroll
-  for (int i = 0; i < MB; ++i) {
-    const long m = (long)tm * TM + wm * (MB * 32) + i * 32 + l32;
-    if (m < M) {
-#pragma unroll
-      for (int j = 0; j < NB; ++j) {
-        const int nl = wn * (NB * 32) + j * 32 + 16 * g;
-        const int n = tn * TN + nl;
-        if (n < N) {
-          if constexpr (LUT) epi.store16_lds(m, n, N, acc[i][j], true, tab, nl);
-          else epi.store16(m, n, N, acc[i][j], true);
-        }
-      }
-    }
-  }
+  tile_gemm<Epi, WGM, WGN, MB, NB, NST>(A, W, epi, tm * TM, M, N, K, tn, smem);
 }
 
 // ---------------------------------------------------------------------------------

@@ -239,6 +239,20 @@ bool bias_act_enable_lut_kernel(bool on);  // returns the previous setting
 // receives the integer operations of one launch
 int mfma_i8_peak_probe(int* out, int workgroups, int iters, double* ops, hipStream_t s);
 
+// ---- feed-forward segment of an encoder layer in one launch (xcd_ffn_kernels.hip) ----------
+// FFN1 with the tabulated epilogue -> FFN2 -> dequantise + residual (+ colsum) + layer norm
+// (+ quantise), the rows dealt to the 8 XCDs whose workgroups synchronise through their L2.
+// Same bytes as gemm_i8_lut_i8o + gemm_i8_i32o + residual_bias_ln_i8O / residual_bias_ln_i32I.
+bool ffn_segment_supported(int M, int H, int I);
+size_t ffn_segment_sync_words();  // unsigned words of device memory behind `sync`
+int ffn_segment_i8(const int8_t* x, const int8_t* w1, const int8_t* lut1, float alpha1, int8_t* act,
+                   const int8_t* w2, int32_t* acc, __half* residual, __half* out_t, int8_t* out_q,
+                   const __half* scale, const __half* bias, const __half* residual_bias,
+                   const __half* colsum, int M, int H, int I, float dequant_scale,
+                   float quant_scale, bool is_post_ln, bool final_ln, unsigned* sync,
+                   unsigned* launches, int spin_limit, hipStream_t s);
+void ffn_segment_time_next_launch(hipEvent_t start, hipEvent_t stop);
+
 // ---- fp16 MFMA GEMM (gemm_f16.hip) ------------------------------------------------------
 int gemm_f16_nt(const __half* A, const __half* W, __half* C, int M, int N, int K, hipStream_t s);
 // StridedBatchGemm<T>::Forward (ops/includes/strided_batch_gemm.h:45-57); op: 0 = N, 1 = T

@@ -754,3 +754,42 @@ def gemm_i8_lut_i8o(a, w, c, lut, m, n, k, alpha):
     """int8-output GEMM whose epilogue is the table built by :func:`build_act_lut`."""
     _dev(a, w, c, lut)
     call("lsh_gemm_i8_lut_i8o", ptr(a), ptr(w), ptr(c), ptr(lut), m, n, k, alpha, current_stream())
+
+
+class FfnSegmentSync:
+    """Barrier counters, error word and launch count of ``ffn_segment_i8`` (one per caller)."""
+
+    def __init__(self, device="cuda"):
+        import ctypes as _c
+        L = lib.load()
+        L.lsh_ffn_segment_sync_words.restype = _c.c_size_t
+        L.lsh_ffn_segment_sync_words.argtypes = []
+        self.words = int(L.lsh_ffn_segment_sync_words())
+        self.sync = torch.zeros(self.words, dtype=torch.int32, device=device)
+        self.launches = _c.c_uint32(0)
+
+    def error(self):
+        """The error word after the stream has drained (0 = every wait was met)."""
+        return int(self.sync[-1].item()) & 0xFFFFFFFF
+
+    def reset(self):
+        self.sync.zero_()
+        self.launches.value = 0
+
+
+def ffn_segment_supported(m, hidden, inner):
+    return bool(lib.load().lsh_ffn_segment_supported(int(m), int(hidden), int(inner)))
+
+
+def ffn_segment_i8(x, w1, lut1, alpha1, act, w2, acc, residual, out_t, out_q, scale, bias,
+                   residual_bias, colsum, m, hidden, inner, dequant_scale, quant_scale, is_post_ln,
+                   final_ln, sync, spin_limit=1 << 15):
+    """FFN1 (tabulated epilogue) -> FFN2 -> layer norm of an encoder layer in one launch; ``sync``:
+    a :class:`FfnSegmentSync`."""
+    import ctypes as _c
+    _dev(x, w1, lut1, act, w2, acc, residual, out_t, out_q, scale, bias, residual_bias, colsum)
+    call("lsh_ffn_segment_i8_f16", ptr(x), ptr(w1), ptr(lut1), alpha1, ptr(act), ptr(w2), ptr(acc),
+         ptr(residual), ptr(out_t), ptr(out_q), ptr(scale), ptr(bias), ptr(residual_bias),
+         ptr(colsum), m, hidden, inner, dequant_scale, quant_scale, int(bool(is_post_ln)),
+         int(bool(final_ln)), ptr(sync.sync), _c.addressof(sync.launches), int(spin_limit),
+         current_stream())

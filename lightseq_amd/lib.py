@@ -65,6 +65,9 @@ _SIGNATURES = {
     "lsh_bias_act_lut_kernel": (False, "i"),
     "lsh_decself_qkv_attention_in_models": (False, "i"),
     "lsh_mfma_i8_peak_probe": (False, "piips"),
+    "lsh_ffn_segment_supported": (False, "iii"),
+    "lsh_ffn_segment_i8_f16": (False, "ppp" + "f" + "ppp" + "ppp" + "pppp" + "iii" + "ff" + "ii" + "pp" +
+                               "i" + "s"),
     "lsh_tile_weight_16x64": (False, "ppiis"),
     "lsh_gemm_i8_residual_ln_i8O_f16": (False, "pp" + "f" + "ppppp" + "iii" + "ff" + "s" + "i"),
     "lsh_ker_residual_bias_ln_planes_i32I_i8O_f16": (False, "p" + "il" + "ppppp" + "iiff" + "s" +

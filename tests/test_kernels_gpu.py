@@ -321,6 +321,34 @@ def test_qkv_projection_and_attention_in_one_kernel(rng, B, S, h):
     assert to_np(got).any()
 
 
+@pytest.mark.parametrize("B,S,h,lens", [(4, 128, 4, [128, 97, 33, 1]), (3, 50, 4, [50, 17, 32]),
+                                        (8, 128, 12, [128, 64, 65, 96, 32, 31, 100, 5])])
+def test_qkv_projection_and_attention_against_the_oracle(oracle, rng, B, S, h, lens):
+    """lsh_qkv_attention_i8 against the oracle's chain (int8 GEMM -> arrange + dequantise ->
+    scores -> masked soft-max -> context -> merge + quantise; transformerKernels.cc.cu:1119-1172
+    for the mask) on right-padded sequences of ragged lengths: valid rows to the int8 bar, rows
+    of padded queries exactly zero."""
+    d = 64
+    H = h * d
+    x = rng.integers(-127, 128, size=(B * S, H), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(3 * H, H), dtype=np.int8)
+    bias = _randT(rng, (3 * H,), np.float16, 0.3)
+    mask = (np.arange(S)[None, :] >= np.asarray(lens)[:, None]).astype(np.int32)
+    alpha = 127.0 / (127 * 127 * np.sqrt(H) / 3.0)
+    ds, qs = 1.4 / 127, 127 / 0.9
+    codes = oracle.gemm_i8_i8(x, w, alpha)
+    qkv = oracle.arrange_encself_qkv_i8I(codes, bias, B, S, h, ds)
+    probs = oracle.correlation_softmax_encself(oracle.attn_scores(qkv[0], qkv[1], np.sqrt(1.0 / d)), mask)
+    want = oracle.arrange_atten_output_i8O(oracle.attn_context(probs, qkv[2]), qs)
+    got = torch.full((B * S, H), 9, dtype=torch.int8, device=DEV)
+    _k().qkv_attention_i8(to_dev(x), to_dev(w), to_dev(bias), to_dev(mask), got, alpha, ds, qs, B, S, h, d)
+    got = to_np(got)
+    valid = (mask == 0).reshape(-1)
+    assert_codes_close(got[valid], want[valid], max_frac=5e-3, what="context codes")
+    assert np.abs(got[valid]).mean() > 5
+    assert not got[~valid].any(), "rows of padded queries must be zero"
+
+
 def test_qkv_projection_and_attention_in_one_kernel_rejects_other_shapes(rng):
     import lightseq_amd.lib as L
     for B, S, h, d in [(2, 128, 4, 32), (2, 129, 4, 64), (2, 64, 2, 64), (2, 64, 3, 64)]:

@@ -71,13 +71,23 @@ def _oracle_weights(msg, cfg):
     return model_io.oracle_transformer_weights_from_message(msg, cfg, np.float16)
 
 
+# mean, 99.9th percentile and maximum of |GPU - oracle| over the valid positions of the encoder
+# output (fp16), both sides free-running
+ENC_DRIFT = (5e-4, 2e-2, 4e-2)   # observed at Transformer-big width, 2 layers: 1.5e-4, 1.1e-2, 2.2e-2
+
+
 def _check_against_oracle(oracle, msg, cfg, ids, gpu, max_logit_mismatch):
     enc_w, dec_w = _oracle_weights(msg, cfg)
     # encoder stage: the fp16 hidden states (layer outputs, tolerance of the path: 2e-2)
     want_enc, mask, _ = oracle.quant_bert_encoder(enc_w, ids)
     valid = mask == 0
     err = np.abs(gpu["enc_out"].astype(np.float32) - want_enc.astype(np.float32))[valid]
-    assert err.max() <= 2e-2 or np.mean(err > 2e-2) < 2e-3, err.max()
+    # the free-running encoder stack against the oracle's own run: the path's 2e-2 holds per layer
+    # on equal inputs; over a stack a flipped code moves a few outputs further (three numbers)
+    print("encoder drift: mean %.2e, 99.9th percentile %.2e, max %.2e" %
+          (err.mean(), np.quantile(err, 0.999), err.max()))
+    assert err.mean() <= ENC_DRIFT[0] and np.quantile(err, 0.999) <= ENC_DRIFT[1] and \
+        err.max() <= ENC_DRIFT[2], (err.mean(), np.quantile(err, 0.999), err.max())
 
     # decoder, conditioned on the GPU's encoder output and logits
     r = oracle.quant_decoder(dec_w, gpu["enc_out"], mask, forced_logits=gpu["logits"], record=True)
