@@ -451,6 +451,8 @@ def bench_bert(args):
         k["ms"] += site["total_ms"]
         k["launches"] += site["launches"]
         ops = 2.0 * site["m"] * site["n"] * site["k"]
+        if site["kernel"] == "ffn_segment_kernel":
+            ops *= 2.0  # FFN1 and FFN2 in one launch: the same number of operations each
         if site["kernel"] == "qkv_attn_kernel":
             # the launch also holds the layer's attention: 4 B h S^2 d fp16 flops, counted
             # twice because the fp16 MFMA peak is half the int8 peak this is priced against
@@ -468,15 +470,18 @@ def bench_bert(args):
                                      "compute unit (lsh_mfma_i8_peak_probe)",
                 "ops_counted": ("2*M*N*K int8 operations of the product" +
                                 (" + 2 x the 4*B*h*S^2*d fp16 flops of the attention in the same launch"
-                                 if name == "qkv_attn_kernel" else "")),
+                                 if name == "qkv_attn_kernel" else "") +
+                                (", FFN1 and FFN2 both (one launch; the layer norm in it adds none)"
+                                 if name == "ffn_segment_kernel" else "")),
                 "traffic": _profiled_traffic(name, dom_site),
                 "traffic_source": "profiles/" + TRAFFIC_SUMMARY, "kernel": name,
                 "sites": dom["sites"], "avg_launch_us": avg_ms * 1e3,
                 "gemm_sites": {s["site"]: {"kernel": s["kernel"], "mnk": [s["m"], s["n"], s["k"]],
                                            "avg_us": 1e3 * s["total_ms"] / max(1, s["launches"]),
-                                           "tops": 2.0 * s["m"] * s["n"] * s["k"] * s["launches"]
+                                           "tops": (2.0 if s["kernel"] == "ffn_segment_kernel" else 1.0)
+                                           * 2.0 * s["m"] * s["n"] * s["k"] * s["launches"]
                                            / max(1e-12, s["total_ms"] * 1e-3) / 1e12}
-                               for s in prof}}
+                               for s in prof if s["launches"] > 0}}
     out = {
         "metric": "int8 tokens/sec BERT-base b32 s128; int8 GEMM % MFMA-i8 peak; fused GB/s",
         "value": tokens_per_s, "unit": "tokens/s",
@@ -507,6 +512,66 @@ def bench_bert(args):
         out["generation"] = {w: bench_generation(w, steps=3, warmup=1, graphs=False,
                                                  with_cpu=not args.no_cpu_baseline)
                              for w in ("transformer_big", "gpt2_medium")}
+    return out
+
+
+def bench_ffn_segment(args):
+    """A/B of the feed-forward half of a layer as one launch (rows dealt to the XCDs, XCD-local
+    barriers; ``lsh_ffn_segment_i8_f16``) against its three launches, inside the BERT workload:
+    step times of both routes, the event-timed launch, and the per-workgroup clock stamps at the
+    kernel's phase boundaries."""
+    import numpy as np
+    import torch
+    from lightseq_amd import inference, kernels as K, synthetic
+    cfg = synthetic.bert_config("bert_base")
+    path = _write_model(cfg)
+    ids, _ = synthetic.make_token_ids(cfg, BATCH, SEQ, seed=0, min_len=32)
+    model = inference.QuantBert(path, BATCH)
+    os.remove(path)
+    model._upload(ids)
+    out = {"workload": "BERT-base b32 x s128, 12 layers", "ms_per_step": {}, "launch_us": {}}
+    prev = K.ffn_segment_in_models(False)
+    try:
+        for rnd in range(3):
+            for on in (True, False):
+                K.ffn_segment_in_models(on)
+                for _ in range(args.warmup):
+                    model.infer_device()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    model.infer_device()
+                torch.cuda.synchronize()
+                out["ms_per_step"].setdefault("segment" if on else "three launches", []).append(
+                    1e3 * (time.perf_counter() - t0) / args.steps)
+        for on in (True, False):
+            K.ffn_segment_in_models(on)
+            model.set_profiling(True)
+            for _ in range(args.steps):
+                model.infer_device()
+            prof = model.get_profile()
+            model.set_profiling(False)
+            out["launch_us"]["segment" if on else "three launches (the layer norm is not event-timed)"] = {
+                p["site"]: {"kernel": p["kernel"], "avg_us": 1e3 * p["total_ms"] / p["launches"]}
+                for p in prof if p["launches"] and p["site"] in ("ffn1", "ffn2")}
+        K.ffn_segment_in_models(True)
+        st = torch.zeros(256, 8, dtype=torch.int64, device="cuda:0")
+        K.ffn_segment_stamps(st)
+        runs = []
+        for _ in range(20):
+            model.infer_device()   # the stamps of the last layer's launch remain
+            runs.append(st.cpu().numpy().copy())
+        K.ffn_segment_stamps(None)
+    finally:
+        K.ffn_segment_in_models(prev)
+    model.close()
+    a = np.stack(runs).astype(np.float64) * 0.01  # 100 MHz clock -> microseconds
+    names = ["start", "FFN1 done", "past barrier 1", "FFN2 done", "past barrier 2", "layer norm done"]
+    d = np.diff(a, axis=2)
+    out["phase_us (mean over the 256 workgroups; mean over launches of the slowest workgroup)"] = {
+        "%s -> %s" % (names[i], names[i + 1]): [float(d[:, :, i].mean()), float(d[:, :, i].max(axis=1).mean())]
+        for i in range(5)}
+    out["first start -> last end, in-kernel, us"] = float((a[:, :, 5].max(axis=1) - a[:, :, 0].min(axis=1)).mean())
     return out
 
 
@@ -684,6 +749,8 @@ def main():
                     help="skip the stand-alone timing of the fused kernels")
     ap.add_argument("--no-generation", action="store_true",
                     help="default workload: skip the two generation workloads of the `generation` block")
+    ap.add_argument("--ffn-segment", action="store_true",
+                    help="A/B and phase stamps of the one-launch feed-forward segment (not the headline line)")
     ap.add_argument("--graphs", action="store_true",
                     help="generation workloads: replay the steps as HIP graphs (ls_model_set_graph_mode)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -710,6 +777,10 @@ def main():
         for _ in range(3):
             torch.add(src, 1, out=dst)
         torch.cuda.synchronize()
+    if args.ffn_segment:
+        print(json.dumps(bench_ffn_segment(args)))
+        sys.stdout.flush()
+        os._exit(0)
     out = bench_bert(args) if bert else bench_generation(args.workload, args.steps, args.warmup,
                                                          args.graphs, not args.no_cpu_baseline)
     print(json.dumps(out))

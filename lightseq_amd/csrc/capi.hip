@@ -146,6 +146,11 @@ int lsh_gemm_i8_residual_ln_i8O_f16(const int8_t* A, const int8_t* w_tiled, floa
                                          output, HM(residual), batch_tokens, hidden_size, k,
                                          dequant_scale, quant_scale, HS(stream), is_post_ln != 0);
 }
+int lsh_ffn_segment_in_models(int on) { return ffn_segment_enable(on != 0) ? 1 : 0; }
+int lsh_ffn_segment_stamps(uint64_t* dev) {
+  ffn_segment_stamps(reinterpret_cast<unsigned long long*>(dev));
+  return LSH_OK;
+}
 size_t lsh_ffn_segment_sync_words(void) { return ffn_segment_sync_words(); }
 int lsh_ffn_segment_supported(int m, int hidden, int inner) {
   return ffn_segment_supported(m, hidden, inner) ? 1 : 0;

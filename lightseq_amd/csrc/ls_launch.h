@@ -252,6 +252,14 @@ int ffn_segment_i8(const int8_t* x, const int8_t* w1, const int8_t* lut1, float 
                    float quant_scale, bool is_post_ln, bool final_ln, unsigned* sync,
                    unsigned* launches, int spin_limit, hipStream_t s);
 void ffn_segment_time_next_launch(hipEvent_t start, hipEvent_t stop);
+void ffn_segment_stamps(unsigned long long* dev);  // 256 x 8 clock values per launch, or null
+// what the models do (off by default: measured no faster than the three launches; returns the
+// previous setting), and the process-wide
+// claim that keeps two models from running the segment kernel at the same time
+bool ffn_segment_enable(bool on);
+bool ffn_segment_enabled();
+bool ffn_segment_claim(const void* who);
+void ffn_segment_release(const void* who);
 
 // ---- fp16 MFMA GEMM (gemm_f16.hip) ------------------------------------------------------
 int gemm_f16_nt(const __half* A, const __half* W, __half* C, int M, int N, int K, hipStream_t s);

@@ -7,6 +7,9 @@
 namespace lightseq {
 namespace hip {
 
+// polls (about a microsecond each) after which a wait inside the feed-forward segment gives up
+static const int kSegmentSpinLimit = 1 << 15;
+
 using namespace lsh;
 
 QuantBertEncoder::QuantBertEncoder(int max_batch_size, const int* p_d_token_id,
@@ -48,6 +51,10 @@ void QuantBertEncoder::init_buffer() {
   // room for the accumulator planes of a split-K second FFN product (up to 4 at encoder
   // sizes, up to 8 for the few rows of a decode step)
   _int32_ffn_out_buf.alloc(std::max((size_t)tokens * H * 4, (size_t)64 * H * 8));
+  _seg_sync.alloc(ffn_segment_sync_words());
+  CHECK_GPU_ERROR(hipMemsetAsync(_seg_sync.get(), 0, _seg_sync.size() * sizeof(unsigned), _stream));
+  CHECK_GPU_ERROR(hipHostMalloc(reinterpret_cast<void**>(&_h_seg_error), sizeof(unsigned)));
+  *_h_seg_error = 0;
 
   _int8_emb = upload_kernel(_tw.token_embedding, _tw._src_vocab_size, H, false, _stream);
   _pos_emb = upload_half(_tw.position_embedding, _stream);
@@ -117,11 +124,14 @@ void QuantBertEncoder::prof_begin(int site, int m, int n, int k, const char* epi
   if (!_profiling) return;
   const bool fused_ln = std::string(epilogue) == "fused_ln";
   const bool fused_qa = std::string(epilogue) == "fused_qkv_attn";
+  const bool segment = std::string(epilogue) == "ffn_segment";
   SiteProfile& p = _profile[site];
-  if (p.m != m || p.n != n || p.k != k || p.kernel.empty()) {
+  if (p.m != m || p.n != n || p.k != k || p.kernel.empty() || p.route != epilogue) {
     p.m = m; p.n = n; p.k = k;
+    p.route = epilogue;
     p.kernel = fused_ln   ? "gemm_ln_rows16_kernel"
                : fused_qa ? "qkv_attn_kernel"
+               : segment  ? "ffn_segment_kernel"
                           : gemm_i8_kernel_name(m, n, k, epilogue);
   }
   Pending pe;
@@ -137,6 +147,7 @@ void QuantBertEncoder::prof_begin(int site, int m, int n, int k, const char* epi
   // the launcher records the kernel's own begin / end timestamps into the events
   if (fused_ln) gemm_ln_time_next_launch(pe.e0, pe.e1);
   else if (fused_qa) qkv_attention_time_next_launch(pe.e0, pe.e1);
+  else if (segment) ffn_segment_time_next_launch(pe.e0, pe.e1);
   else gemm_i8_time_next_launch(pe.e0, pe.e1);
   _pending.push_back(pe);
 }
@@ -151,6 +162,26 @@ void QuantBertEncoder::collect_profile() {
     _event_pool.push_back(pe.e1);
   }
   _pending.clear();
+}
+
+QuantBertEncoder::~QuantBertEncoder() {
+  ffn_segment_release(this);
+  if (_h_seg_error) (void)hipHostFree(_h_seg_error);
+}
+
+bool QuantBertEncoder::finish_infer() {
+  if (!_seg_active) return false;
+  _seg_active = false;
+  ffn_segment_release(this);
+  if (*_h_seg_error == 0) return false;
+  // a wait inside the segment kernel gave up: its outputs are undefined.  Clear the counters,
+  // leave that route, and let the caller run the batch again on the three launches.
+  CHECK_GPU_ERROR(hipMemsetAsync(_seg_sync.get(), 0, _seg_sync.size() * sizeof(unsigned), _stream));
+  CHECK_GPU_ERROR(hipStreamSynchronize(_stream));
+  _seg_launches = 0;
+  *_h_seg_error = 0;
+  _seg_off = true;
+  return true;
 }
 
 void QuantBertEncoder::tap(int8_t* dst, const int8_t* src, size_t n) {
@@ -172,10 +203,16 @@ void QuantBertEncoder::run_one_infer(int batch_size, int batch_seq_len) {
                                _p_d_padding_mask, _tw._padding_id, batch_size, batch_seq_len,
                                _tw._hidden_size, _stream, _src_emb_clip_max / _quant_range,
                                _tw._scale_embedding, _tw._src_vocab_size));
+  _seg_active = _fuse && !_seg_off && ffn_segment_enabled() && _seg_sync.get() != nullptr &&
+                ffn_segment_supported(_batch_token_num, _tw._hidden_size, _tw._inner_size) &&
+                ffn_segment_claim(this);
   for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
     self_attention();
     ffn_add_norm();
   }
+  if (_seg_active)
+    CHECK_GPU_ERROR(hipMemcpyAsync(_h_seg_error, _seg_sync.get() + _seg_sync.size() - 1,
+                                   sizeof(unsigned), hipMemcpyDeviceToHost, _stream));
 }
 
 void QuantBertEncoder::self_attention() {
@@ -267,6 +304,32 @@ void QuantBertEncoder::ffn_add_norm() {
   const float* c = &_enc_clip_max[_layer_id * _tw._clip_stride];
   const float Q = _quant_range;
 
+  const float dequant_scale =
+      _tw._use_gelu ? c[3] * c[7] / (Q * Q) : c[3] * c[7] / (2 * Q * Q);
+  const __half* colsum = w.ffn2_colsum.get();  // nullptr for GELU models
+  const bool last = _layer_id == _tw._n_enc_layer - 1;
+  const bool tapped = taps.tap_layer == _layer_id && (taps.ffn1_q || taps.ffn2_acc || taps.res_ffn);
+  if (_seg_active && !tapped) {
+    // FFN1 + table, FFN2 and the layer norm in one launch (the bytes of the three launches
+    // below).  Reads _int8_ffn_in_buf, leaves the activation codes in _int8_ffn_out_buf and the
+    // next layer's input codes in _int8_ffn_in_buf.
+    prof_begin(2, M, I, H, "ffn_segment");
+    const Layer* nx = last ? nullptr : &_layers[_layer_id + 1];
+    const float clip_next = last ? 1.f : _enc_clip_max[(_layer_id + 1) * _tw._clip_stride + 4];
+    // the last phase writes the next layer's codes over the rows the first phase read: rows
+    // belong to one XCD, whose workgroups have all left the first phase by then
+    LSH_CALL(ffn_segment_i8(
+        _int8_ffn_in_buf.get(), w.w_ffn1.get(), w.ffn1_act_lut.get(), c[2] * c[6] / (c[10] * Q),
+        _int8_ffn_out_buf.get(), w.w_ffn2.get(), _int32_ffn_out_buf.get(), _p_d_output,
+        last ? _p_d_output : nullptr, last ? nullptr : _int8_ffn_in_buf.get(),
+        last ? _final_ln_scale.get() : nx->ln1_scale.get(),
+        last ? _final_ln_bias.get() : nx->ln1_bias.get(), last ? nullptr : nx->b_out.get(), colsum,
+        M, H, I, dequant_scale, last ? 0.f : Q / clip_next, _tw._is_post_ln, last, _seg_sync.get(),
+        &_seg_launches, kSegmentSpinLimit, _stream));
+    tap(taps.act_q, _int8_ffn_out_buf.get(), (size_t)M * I);
+    return;
+  }
+
   // FFN1 -> int8 code -> dequant + bias + activation + requant.  Fused into the GEMM
   // epilogue unless the int8 GEMM output is tapped; both routes give the same bits.
   // The fused GEMM reads _int8_ffn_in_buf and must not overwrite it: it writes to
@@ -314,10 +377,7 @@ void QuantBertEncoder::ffn_add_norm() {
   if (taps.res_ffn && taps.tap_layer == _layer_id)
     CHECK_GPU_ERROR(hipMemcpyAsync(taps.res_ffn, _p_d_output, (size_t)M * H * sizeof(__half),
                                    hipMemcpyDeviceToDevice, _stream));
-  const float dequant_scale =
-      _tw._use_gelu ? c[3] * c[7] / (Q * Q) : c[3] * c[7] / (2 * Q * Q);
-  const __half* colsum = w.ffn2_colsum.get();  // nullptr for GELU models
-  if (_layer_id == _tw._n_enc_layer - 1) {
+  if (last) {
     LSH_CALL(residual_bias_ln_i32I<__half>(_int32_ffn_out_buf.get(), _final_ln_scale.get(),
                                            _final_ln_bias.get(), _p_d_output, _p_d_output, M, H,
                                            dequant_scale, _stream, colsum, nparts, part_stride));

@@ -21,9 +21,13 @@ class QuantBertEncoder {
  public:
   QuantBertEncoder(int max_batch_size, const int* p_d_token_id, int* p_d_padding_mask,
                    __half* p_d_output, const QuantBertWeight& tw, hipStream_t stream);
+  ~QuantBertEncoder();
   void init_buffer();
   std::string check();
   void run_one_infer(int batch_size, int batch_seq_len);
+  // After the stream has been synchronised: true when the run has to be repeated (a kernel that
+  // waits for workgroups of its own launch gave up; the encoder has switched that route off).
+  bool finish_infer();
 
   // Debug taps (all optional, device pointers owned by the caller): copies of the
   // intermediates of layer `tap_layer`, for parity bisection.
@@ -40,7 +44,7 @@ class QuantBertEncoder {
   // Per-GEMM-site timing with HIP events on the model's stream (off by default).
   // collect_profile() must be called after the stream has been synchronised.
   struct SiteProfile {
-    std::string site, kernel;
+    std::string site, kernel, route;
     int m = 0, n = 0, k = 0;
     long launches = 0;
     double total_ms = 0.0;
@@ -67,6 +71,12 @@ class QuantBertEncoder {
   struct Pending { int site; hipEvent_t e0, e1; };
   std::vector<Pending> _pending;
   std::vector<hipEvent_t> _event_pool;
+  // the feed-forward half of a layer as one launch (xcd_ffn_kernels.hip)
+  DeviceBuffer<unsigned> _seg_sync;
+  unsigned _seg_launches = 0;
+  unsigned* _h_seg_error = nullptr;  // pinned copy of the error word
+  bool _seg_active = false;          // this run holds the process-wide claim
+  bool _seg_off = false;             // switched off after a launch that gave up
 
   const int _max_batch_size;
   const QuantBertWeight& _tw;

@@ -55,6 +55,12 @@ void QuantTransformer::Infer() {
                                    hipMemcpyDeviceToDevice, stream_));
   decoder_->run_one_infer(batch_size, seq_len);
   CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+  if (encoder_->finish_infer()) {  // an encoder route gave up and was switched off: once more
+    encoder_->run_one_infer(batch_size, seq_len);
+    decoder_->run_one_infer(batch_size, seq_len);
+    CHECK_GPU_ERROR(hipStreamSynchronize(stream_));
+    encoder_->finish_infer();
+  }
   encoder_->collect_profile();
   int output_seq_len = decoder_->_cur_step + 1;
   int output_k = decoder_->_output_topk ? tw_._beam_size : 1;

@@ -30,6 +30,7 @@
 
 #include <hip/hip_ext.h>
 
+#include <atomic>
 #include <mutex>
 
 namespace lsh {
@@ -89,6 +90,8 @@ struct FfnSegmentArgs {
   float alpha1, dequant_scale, quant_scale;
   int M, H, I, rows_per_xcd, is_post_ln, spin_limit;
   unsigned base;          // what the counters held before this launch
+  unsigned launch;        // launches before this one
+  unsigned long long* stamps;  // measurement aid: [256][8] 100 MHz clock values, or null
 };
 
 template <int LPR, int ITER, bool FINAL>
@@ -98,9 +101,26 @@ ffn_segment_kernel(const FfnSegmentArgs a) {
   __shared__ int s_go;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  if (xcd_hw_id() != (unsigned)xcd && tid == 0) XcdL2Mem::fetch_or(a.error, kXcdErrMapping);
+  // The dispatcher deals consecutive workgroups to consecutive XCDs, starting wherever the
+  // previous kernel of the queue left off: the XCD is read from the hardware, and blockIdx / 8
+  // numbers its workgroups.  That every (XCD, slot) pair is taken exactly once is checked: the
+  // workgroup flips its bit of the XCD's mask (word 1 of the counter line, all bits equal
+  // between launches) and must find it as the launch count says.
+  const int xcd = (int)xcd_hw_id() & 7, slot = blockIdx.x >> 3;
+  auto stamp = [&](int i) {
+    if (a.stamps != nullptr && tid == 0) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      a.stamps[blockIdx.x * 8 + i] = __builtin_amdgcn_s_memrealtime();
+    }
+  };
+  stamp(0);
   unsigned* counter = a.counters + xcd * kXcdCounterStride;
+  bool slot_taken = false;
+  if (tid == 0) {
+    const unsigned old = __hip_atomic_fetch_xor(counter + 1, 1u << slot, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+    slot_taken = ((old >> slot) & 1u) != (a.launch & 1u);
+  }
   const int row_lo = min(xcd * a.rows_per_xcd, a.M), row_hi = min(row_lo + a.rows_per_xcd, a.M);
   const int rows = row_hi - row_lo;
 
@@ -115,7 +135,10 @@ ffn_segment_kernel(const FfnSegmentArgs a) {
       __syncthreads();  // the epilogue has read its table: the ring may be refilled
     }
   }
+  if (slot_taken) XcdL2Mem::fetch_or(a.error, kXcdErrMapping);
+  stamp(1);
   if (!xcd_barrier(counter, a.base + kSegSlots, a.error, a.spin_limit, &s_go)) return;
+  stamp(2);
 
   // ---- phase 2: FFN2, 128 x 96 tiles on wavefronts 0-3 ----
   {
@@ -133,7 +156,9 @@ ffn_segment_kernel(const FfnSegmentArgs a) {
       __syncthreads();
     }
   }
+  stamp(3);
   if (!xcd_barrier(counter, a.base + 2 * kSegSlots, a.error, a.spin_limit, &s_go)) return;
+  stamp(4);
 
   // ---- phase 3: LayerNorm, groups of RPI rows ----
   {
@@ -170,6 +195,7 @@ ffn_segment_kernel(const FfnSegmentArgs a) {
       __syncthreads();
     }
   }
+  stamp(5);
 }
 
 // ---------------------------------------------------------------------------------
@@ -180,6 +206,33 @@ void ffn_segment_time_next_launch(hipEvent_t start, hipEvent_t stop) {
   g_seg_ev_start = start;
   g_seg_ev_stop = stop;
 }
+
+// At most one holder of the segment kernel per process at a time: two launches of it that were
+// each partly resident would wait for workgroups that the other one keeps off the compute units
+// (both would give up after their poll limit; this keeps it from happening between the models
+// of one process).
+static std::atomic<const void*> g_segment_owner{nullptr};
+static std::atomic<bool> g_segment_enabled{false};
+bool ffn_segment_claim(const void* who) {
+  const void* expected = nullptr;
+  return g_segment_owner.compare_exchange_strong(expected, who) || expected == who;
+}
+void ffn_segment_release(const void* who) {
+  const void* expected = who;
+  g_segment_owner.compare_exchange_strong(expected, nullptr);
+}
+bool ffn_segment_enable(bool on) {
+  const bool prev = g_segment_enabled.exchange(on);
+  if (prev != on) route_epoch_bump();
+  return prev;
+}
+bool ffn_segment_enabled() { return g_segment_enabled.load(std::memory_order_relaxed); }
+
+// Measurement aid: device memory for 256 x 8 clock values (100 MHz) that the next launches fill
+// per workgroup -- 0 start, 1 FFN1 done, 2 past the first barrier, 3 FFN2 done, 4 past the second
+// barrier, 5 layer norm done; null switches it off.
+static std::atomic<unsigned long long*> g_segment_stamps{nullptr};
+void ffn_segment_stamps(unsigned long long* dev) { g_segment_stamps.store(dev); }
 
 size_t ffn_segment_sync_words() { return (size_t)kXcdCount * kXcdCounterStride + 1; }
 
@@ -277,6 +330,8 @@ int ffn_segment_i8(const int8_t* x, const int8_t* w1, const int8_t* lut1, float 
   a.is_post_ln = is_post_ln ? 1 : 0;
   a.spin_limit = spin_limit;
   a.base = *launches * 2u * kSegSlots;
+  a.launch = *launches;
+  a.stamps = g_segment_stamps.load();
   *launches += 1;
 #define LSH_SEG(LPR, IT) \
   (final_ln ? launch_segment<LPR, IT, true>(a, s) : launch_segment<LPR, IT, false>(a, s))

@@ -21,9 +21,10 @@
 //    every 64 polls) and returns false once it is set.  A caller that gets false leaves the
 //    kernel at once -- every wavefront of the workgroup, through a flag in LDS -- so a kernel
 //    whose workgroups could not all become resident ends instead of spinning.
-//  * Which workgroups form an XCD: workgroup b runs on XCD b % 8.  That is how the dispatcher
-//    deals workgroups out on this part; each workgroup checks it against the hardware's XCC_ID
-//    register and sets kXcdErrMapping otherwise (stale data would be read, not a hang).
+//  * Which workgroups form an XCD is read from the hardware (the XCC_ID register); the kernel
+//    that uses the barrier has to make sure that every XCD holds exactly `expected` of its
+//    workgroups -- too few and the waiters give up (kXcdErrTimeout), too many and a round
+//    would complete early, so a workgroup that finds its place taken sets kXcdErrMapping.
 #pragma once
 
 #ifndef LSH_XCD_FN
@@ -33,7 +34,7 @@
 namespace lsh {
 
 constexpr unsigned kXcdErrTimeout = 1u;  // a wait gave up
-constexpr unsigned kXcdErrMapping = 2u;  // a workgroup does not run on XCD blockIdx % 8
+constexpr unsigned kXcdErrMapping = 2u;  // two workgroups took the same place of an XCD
 constexpr int kXcdCount = 8;
 constexpr int kXcdCounterStride = 32;  // unsigned words between two XCDs' counters (128 bytes)
 

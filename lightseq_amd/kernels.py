@@ -777,6 +777,20 @@ class FfnSegmentSync:
         self.launches.value = 0
 
 
+def ffn_segment_in_models(on):
+    """Let the encoder models run the feed-forward half of a layer as one launch, or as three
+    (default); returns the previous setting."""
+    return bool(lib.load().lsh_ffn_segment_in_models(int(bool(on))))
+
+
+def ffn_segment_stamps(buf):
+    """Measurement aid: an int64 tensor [256, 8] that every following launch of the segment
+    kernel fills with per-workgroup clock values (100 MHz) at its phase boundaries; None: off."""
+    if buf is not None and (buf.dtype != torch.int64 or buf.numel() < 256 * 8 or not buf.is_cuda):
+        raise ValueError("stamps: an int64 GPU tensor of 256 x 8 values")
+    call("lsh_ffn_segment_stamps", ptr(buf))
+
+
 def ffn_segment_supported(m, hidden, inner):
     return bool(lib.load().lsh_ffn_segment_supported(int(m), int(hidden), int(inner)))
 

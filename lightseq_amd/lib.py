@@ -66,6 +66,8 @@ _SIGNATURES = {
     "lsh_decself_qkv_attention_in_models": (False, "i"),
     "lsh_mfma_i8_peak_probe": (False, "piips"),
     "lsh_ffn_segment_supported": (False, "iii"),
+    "lsh_ffn_segment_in_models": (False, "i"),
+    "lsh_ffn_segment_stamps": (False, "p"),
     "lsh_ffn_segment_i8_f16": (False, "ppp" + "f" + "ppp" + "ppp" + "pppp" + "iii" + "ff" + "ii" + "pp" +
                                "i" + "s"),
     "lsh_tile_weight_16x64": (False, "ppiis"),

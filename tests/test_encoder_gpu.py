@@ -326,6 +326,35 @@ def test_bert_base_free_running_drift_against_the_oracle(tmp_path, oracle):
     assert diff.mean() <= 3e-2 and np.quantile(diff, 0.999) <= 0.12 and diff.max() <= 0.2
 
 
+@pytest.mark.parametrize("preset,kw,B,S", [("bert_base", dict(n_layer=3, vocab=2000, max_step=128), 32, 128),
+                                            ("bert_base", dict(n_layer=2, vocab=2000, max_step=128), 5, 77),
+                                            ("tiny", dict(), 4, 24)])
+def test_feed_forward_segment_route_leaves_the_same_bytes(tmp_path, preset, kw, B, S):
+    """The layers run with their feed-forward half as one launch (XCD-local barriers) give the
+    output of the three launches, byte for byte; the route is taken where the shape is covered
+    and two runs in a row work (the barrier counters go on)."""
+    from lightseq_amd import inference, kernels, synthetic
+    cfg, msg, path = _build(tmp_path, preset, 6, **kw)
+    ids, lens = synthetic.make_token_ids(cfg, B, S, seed=6, min_len=max(1, S // 4))
+    model = inference.QuantBert(path, B)
+    want = model.infer_fp16(ids)
+    prev = kernels.ffn_segment_in_models(True)
+    try:
+        model.set_profiling(True)
+        got = [model.infer_fp16(ids) for _ in range(3)]
+        prof = model.get_profile()
+        model.set_profiling(False)
+    finally:
+        kernels.ffn_segment_in_models(prev)
+    for g in got:
+        np.testing.assert_array_equal(g, want)
+    names = {p["site"]: p["kernel"] for p in prof if p["launches"]}
+    if kernels.ffn_segment_supported(B * S, cfg["hidden"], cfg["inner"]):
+        assert names.get("ffn1") == "ffn_segment_kernel" and "ffn2" not in names, names
+    np.testing.assert_array_equal(model.infer_fp16(ids), want)   # and back on the three launches
+    model.close()
+
+
 def test_bert_base_full_stack_properties(tmp_path):
     """The benchmark workload itself (12 layers, b32 x s128): size-independent
     properties.  A sequence's output does not depend on what else is in the batch

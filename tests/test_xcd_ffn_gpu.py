@@ -136,15 +136,22 @@ def test_segment_gives_up_when_its_workgroups_cannot_all_arrive():
     z8 = lambda *s: torch.zeros(s, dtype=torch.int8, device=DEV)
     f16 = lambda *s: torch.ones(s, dtype=torch.float16, device=DEV)
     sync = k.FfnSegmentSync()
-    sync.launches.value = 5            # targets start at 5 * 64 while the counters stand at zero
+    sync.launches.value = 6            # targets start at 6 * 64 while the counters stand at zero
     res = f16(M, H)
     k.ffn_segment_i8(z8(M, H), z8(I, H), z8(I, 256), 1e-3, z8(M, I), z8(H, I),
                      torch.zeros((M, H), dtype=torch.int32, device=DEV), res, None, z8(M, H), f16(H),
                      f16(H), f16(H), None, M, H, I, 1e-3, 10.0, True, False, sync, spin_limit=200)
     torch.cuda.synchronize()
-    assert sync.error() & 1
+    assert sync.error() == 1
     sync.reset()
     assert sync.error() == 0
+    # a launch count of the wrong parity looks like places taken twice: the other error bit
+    sync.launches.value = 1
+    k.ffn_segment_i8(z8(M, H), z8(I, H), z8(I, 256), 1e-3, z8(M, I), z8(H, I),
+                     torch.zeros((M, H), dtype=torch.int32, device=DEV), res, None, z8(M, H), f16(H),
+                     f16(H), f16(H), None, M, H, I, 1e-3, 10.0, True, False, sync, spin_limit=200)
+    torch.cuda.synchronize()
+    assert sync.error() & 2
 
 
 def test_segment_rejects_what_it_does_not_cover():
