@@ -210,6 +210,27 @@ int lsh_qkv_attention_i8_f16(const int8_t* x, const int8_t* qkv_weight, const vo
                              int batch_seq_len, int head_num, int dim_per_head,
                              lsh_stream_t stream);
 
+/* The same launch with a plan made from the padding mask (no counterpart in the reference).
+ * The context of a padded query is zero whatever its q is, and a padded key contributes exactly
+ * nothing (kernels/transformerKernels.cc.cu:1119-1172), so a workgroup leaves out the 32-token
+ * blocks of its sequence that hold nothing but padding -- in the product, in the conversion and
+ * in the attention -- and the plan deals the (sequence, head) pairs out longest sequence first,
+ * so that the compute units that hold two workgroups hold a long and a short one.  Bytes: those
+ * of lsh_qkv_attention_i8_f16 on the rows of tokens that are not padding, zeros on the others
+ * (there the unplanned launch leaves zeros too).  plan: batch_size * head_num ints of device
+ * memory, written by lsh_qkv_attention_plan, valid for launches with that mask, batch_size,
+ * batch_seq_len and head_num; batch_size <= 1024. */
+int lsh_qkv_attention_plan(const int* src_padding_mask, int* plan, int batch_size,
+                           int batch_seq_len, int head_num, lsh_stream_t stream);
+/* whether the encoder models make and use a plan (default) -- an A/B switch; returns the
+ * previous setting */
+int lsh_qkv_attention_plan_in_models(int on);
+int lsh_qkv_attention_planned_i8_f16(const int8_t* x, const int8_t* qkv_weight, const void* qkv_bias,
+                                     const int* src_padding_mask, const int* plan, int8_t* ctx_q,
+                                     float requant_alpha, float dequant_scale, float quant_scale,
+                                     int batch_size, int batch_seq_len, int head_num,
+                                     int dim_per_head, lsh_stream_t stream);
+
 /* ---- embedding ------------------------------------------------------------------------ */
 /* kernels/embKernels_int8.h:7-13 */
 int lsh_launch_enc_emb_i8I_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,

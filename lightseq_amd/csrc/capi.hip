@@ -370,6 +370,22 @@ int lsh_qkv_attention_i8_f16(const int8_t* x, const int8_t* qkv_weight, const vo
                           dim_per_head, HS(stream));
 }
 
+int lsh_qkv_attention_plan_in_models(int on) { return qkv_attention_plan_enable(on != 0) ? 1 : 0; }
+int lsh_qkv_attention_plan(const int* src_padding_mask, int* plan, int batch_size,
+                           int batch_seq_len, int head_num, lsh_stream_t stream) {
+  return qkv_attention_plan(src_padding_mask, plan, batch_size, batch_seq_len, head_num, HS(stream));
+}
+int lsh_qkv_attention_planned_i8_f16(const int8_t* x, const int8_t* qkv_weight, const void* qkv_bias,
+                                     const int* src_padding_mask, const int* plan, int8_t* ctx_q,
+                                     float requant_alpha, float dequant_scale, float quant_scale,
+                                     int batch_size, int batch_seq_len, int head_num,
+                                     int dim_per_head, lsh_stream_t stream) {
+  if (!plan) return lsh_fail(LSH_ERR_INVALID, "qkv_attention_planned_i8: null plan");
+  return qkv_attention_i8(x, qkv_weight, H(qkv_bias), src_padding_mask, ctx_q, requant_alpha,
+                          dequant_scale, quant_scale, batch_size, batch_seq_len, head_num,
+                          dim_per_head, HS(stream), plan);
+}
+
 // ---- embedding ----------------------------------------------------------------------------------
 int lsh_launch_enc_emb_i8I_f16(const int8_t* token_emb, const void* pos_emb, const int* tokens,
                                void* output, int* pad_mask, int pad_id, int batch_size,

@@ -161,7 +161,16 @@ void qkv_attention_time_next_launch(hipEvent_t start, hipEvent_t stop);
 int qkv_attention_i8(const int8_t* x, const int8_t* qkv_weight, const __half* qkv_bias,
                      const int* pad_mask, int8_t* ctx_q, float requant_alpha, float dequant_scale,
                      float quant_scale, int batch, int seq_len, int head_num, int dim_per_head,
-                     hipStream_t s);
+                     hipStream_t s, const int* plan = nullptr);
+// The plan of such launches (batch * head_num ints, made once per padding mask): workgroups take
+// their (sequence, head) pairs longest sequence first, paired on a compute unit with the
+// shortest, and leave out the 32-token blocks that hold nothing but padding.  Same bytes on
+// the rows of tokens that are not padding, zeros on the others.
+bool qkv_attention_plan_supported(int batch, int seq_len, int head_num);
+bool qkv_attention_plan_enable(bool on);  // what the models do (default on); returns the previous setting
+bool qkv_attention_plan_enabled();
+int qkv_attention_plan(const int* pad_mask, int* plan, int batch, int seq_len, int head_num,
+                       hipStream_t s);
 
 // ---- int8 MFMA GEMM (gemm_i8.hip) -----------------------------------------------------
 // C[M,N] = A[M,K] * W[N,K]^T, both operands K-contiguous.

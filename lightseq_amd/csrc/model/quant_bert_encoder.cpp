@@ -51,6 +51,7 @@ void QuantBertEncoder::init_buffer() {
   // room for the accumulator planes of a split-K second FFN product (up to 4 at encoder
   // sizes, up to 8 for the few rows of a decode step)
   _int32_ffn_out_buf.alloc(std::max((size_t)tokens * H * 4, (size_t)64 * H * 8));
+  _qa_plan.alloc((size_t)_max_batch_size * _tw._head_num);
   _seg_sync.alloc(ffn_segment_sync_words());
   CHECK_GPU_ERROR(hipMemsetAsync(_seg_sync.get(), 0, _seg_sync.size() * sizeof(unsigned), _stream));
   CHECK_GPU_ERROR(hipHostMalloc(reinterpret_cast<void**>(&_h_seg_error), sizeof(unsigned)));
@@ -203,6 +204,15 @@ void QuantBertEncoder::run_one_infer(int batch_size, int batch_seq_len) {
                                _p_d_padding_mask, _tw._padding_id, batch_size, batch_seq_len,
                                _tw._hidden_size, _stream, _src_emb_clip_max / _quant_range,
                                _tw._scale_embedding, _tw._src_vocab_size));
+  // one plan for the fused QKV + attention launches of all layers: the padding mask is theirs all
+  _qa_plan_cur = nullptr;
+  if (_fuse && qkv_attention_plan_enabled() &&
+      qkv_attention_fused_supported(batch_size, batch_seq_len, _tw._head_num, _tw._dim_per_head) &&
+      qkv_attention_plan_supported(batch_size, batch_seq_len, _tw._head_num)) {
+    LSH_CALL(qkv_attention_plan(_p_d_padding_mask, _qa_plan.get(), batch_size, batch_seq_len,
+                                _tw._head_num, _stream));
+    _qa_plan_cur = _qa_plan.get();
+  }
   _seg_active = _fuse && !_seg_off && ffn_segment_enabled() && _seg_sync.get() != nullptr &&
                 ffn_segment_supported(_batch_token_num, _tw._hidden_size, _tw._inner_size) &&
                 ffn_segment_claim(this);
@@ -244,7 +254,7 @@ void QuantBertEncoder::self_attention() {
     LSH_CALL(qkv_attention_i8(_int8_ffn_in_buf.get(), w.w_qkv.get(), w.b_qkv.get(),
                               _p_d_padding_mask, _int8_ffn_out_buf.get(), c[0] * c[4] / (c[8] * Q),
                               c[8] / Q, Q / c[5], _batch_size, _batch_seq_len, _tw._head_num, dph,
-                              _stream));
+                              _stream, _qa_plan_cur));
     std::swap(_int8_ffn_in_buf, _int8_ffn_out_buf);
   } else {
     prof_begin(0, M, 3 * H, H, "EpiI8");

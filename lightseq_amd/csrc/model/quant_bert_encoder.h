@@ -92,6 +92,8 @@ class QuantBertEncoder {
   DeviceBuffer<__half> _qkv_buf;  // q | k | v, each max_batch_dim
   DeviceBuffer<int8_t> _int8_ffn_in_buf, _int8_ffn_out_buf;
   DeviceBuffer<int32_t> _int32_ffn_out_buf;
+  DeviceBuffer<int> _qa_plan;      // plan of the fused QKV + attention launches of a call
+  const int* _qa_plan_cur = nullptr;  // ... when this call has one
   // weights
   DeviceBuffer<int8_t> _int8_emb;                       // [vocab, H]
   DeviceBuffer<__half> _pos_emb, _final_ln_scale, _final_ln_bias;

@@ -158,50 +158,52 @@ __device__ __forceinline__ uint32_t float2int8_pack4(float x0, float x1, float x
 // (padk0) and 64 + g * 32 + l32 (padk1)), which the conversion to fp16 turns into -inf as
 // the mask would; all other scores receive +0.
 //
+// NKB: how many blocks of 32 keys exist (keys from NKB * 32 on are padding and are not looked
+// at: a masked key's probability is exactly zero, so leaving its block out changes nothing).
 // qreg[ks]: d = ks * 16 + g * 8 .. + 8 of the lane's query.  q_pad: the query is padding (its
 // context is zero).  out_h / out_q: where the D context values of the lane's query go (fp16 /
 // int8 codes), or null; nothing is stored when `live` is false.
 constexpr int attn_kstr(int D) { return D + 8; }  // halfs per K row in LDS
 constexpr int kAttnVstr = 128 + 4;                // halfs per V^T row in LDS
 
-template <int D>
+template <int D, int NKB = 4>
 __device__ __forceinline__ void attend_block128(const _Float16* Ks, const _Float16* Vt,
                                                 const v8h (&qreg)[D / 16], bool padk0, bool padk1,
                                                 bool q_pad, bool live, float alpha,
                                                 float quant_scale, __half* out_h, int8_t* out_q,
                                                 int l32, int g) {
   constexpr int KSTR = attn_kstr(D), VSTR = kAttnVstr;
-  v16f sc[4];
+  v16f sc[NKB];
   {
-    v8h kf[4][D / 16];
+    v8h kf[NKB][D / 16];
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb)
+    for (int sb = 0; sb < NKB; ++sb)
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks)
         kf[sb][ks] = *reinterpret_cast<const v8h*>(&Ks[(sb * 32 + l32) * KSTR + ks * 16 + g * 8]);
-    v8h bx = (v8h)(_Float16)0, ax[4];
+    v8h bx = (v8h)(_Float16)0, ax[NKB];
     bx[0] = (_Float16)65504.f;
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb) {
+    for (int sb = 0; sb < NKB; ++sb) {
       ax[sb] = (v8h)(_Float16)0;
       ax[sb][0] = (g == (sb & 1) && (sb < 2 ? padk0 : padk1)) ? (_Float16)-65504.f : (_Float16)0;
     }
     __builtin_amdgcn_sched_barrier(0);
-    v16f c[4];
+    v16f c[NKB];
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb)
+    for (int sb = 0; sb < NKB; ++sb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) c[sb][i] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ++ks)
 #pragma unroll
-      for (int sb = 0; sb < 4; ++sb)
+      for (int sb = 0; sb < NKB; ++sb)
         c[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[sb][ks], qreg[ks], c[sb], 0, 0, 0);
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb)
+    for (int sb = 0; sb < NKB; ++sb)
       c[sb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ax[sb], bx, c[sb], 0, 0, 0);
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb)
+    for (int sb = 0; sb < NKB; ++sb)
 #pragma unroll
       for (int i = 0; i < 16; ++i) sc[sb][i] = round_h(alpha * c[sb][i]);
   }
@@ -209,7 +211,7 @@ __device__ __forceinline__ void attend_block128(const _Float16* Ks, const _Float
   // row maximum, exponentials (kept for the second pass) and their sum
   float m = kFloatInfNeg;
 #pragma unroll
-  for (int sb = 0; sb < 4; ++sb)
+  for (int sb = 0; sb < NKB; ++sb)
 #pragma unroll
     for (int i = 0; i < 16; ++i) m = fmaxf(m, sc[sb][i]);
   m = fmaxf(m, __shfl_xor(m, 32, 64));
@@ -217,7 +219,7 @@ __device__ __forceinline__ void attend_block128(const _Float16* Ks, const _Float
   const float nm = -mref * 1.44269504088896340736f;
   float sum = 0.f;
 #pragma unroll
-  for (int sb = 0; sb < 4; ++sb)
+  for (int sb = 0; sb < NKB; ++sb)
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       // exp(s - m) as 2^(s * log2(e) - m * log2(e)): one multiply-add and the exp2 instruction
@@ -238,9 +240,9 @@ __device__ __forceinline__ void attend_block128(const _Float16* Ks, const _Float
   for (int db = 0; db < D / 32; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-  v4h vf[4][2][D / 32][2];
+  v4h vf[NKB][2][D / 32][2];
 #pragma unroll
-  for (int sb = 0; sb < 4; ++sb)
+  for (int sb = 0; sb < NKB; ++sb)
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -251,7 +253,7 @@ __device__ __forceinline__ void attend_block128(const _Float16* Ks, const _Float
       }
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int sb = 0; sb < 4; ++sb) {
+  for (int sb = 0; sb < NKB; ++sb) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       v8h pb;

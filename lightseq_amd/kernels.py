@@ -648,6 +648,31 @@ def gemm_i8_decself_qkv_i8o(a, w, qkv_bias, new_q, new_k, new_v, step_token_num,
          quant_scale, current_stream())
 
 
+def qkv_attention_plan(src_padding_mask, batch, seq_len, head_num):
+    """The plan of ``qkv_attention_i8`` launches with this padding mask: an int32 tensor
+    [batch * head_num]."""
+    _dev(src_padding_mask)
+    plan = torch.zeros(batch * head_num, dtype=torch.int32, device=src_padding_mask.device)
+    call("lsh_qkv_attention_plan", ptr(src_padding_mask), ptr(plan), batch, seq_len, head_num,
+         current_stream())
+    return plan
+
+
+def qkv_attention_plan_in_models(on):
+    """Let the encoder models plan their fused QKV + attention launches from the padding mask
+    (default) or not; returns the previous setting."""
+    return bool(lib.load().lsh_qkv_attention_plan_in_models(int(bool(on))))
+
+
+def qkv_attention_planned_i8(x, qkv_weight, qkv_bias, src_padding_mask, plan, ctx_q, requant_alpha,
+                             dequant_scale, quant_scale, batch, seq_len, head_num, dim_per_head):
+    """``qkv_attention_i8`` that skips the blocks of padding and takes the pairs in the plan's order."""
+    _dev(x, qkv_weight, qkv_bias, src_padding_mask, plan, ctx_q)
+    call("lsh_qkv_attention_planned_i8_f16", ptr(x), ptr(qkv_weight), ptr(qkv_bias),
+         ptr(src_padding_mask), ptr(plan), ptr(ctx_q), requant_alpha, dequant_scale, quant_scale,
+         batch, seq_len, head_num, dim_per_head, current_stream())
+
+
 def decself_qkv_attention_i8(x, w, qkv_bias, new_q, k_cache, v_cache, ctx, rows, hidden, head_num,
                              max_step, step_id, alpha, dequant_scale, cache_quant_scale, attn_scale,
                              cache_dequant_scale, ctx_quant_scale):

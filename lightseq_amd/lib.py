@@ -45,6 +45,9 @@ _SIGNATURES = {
     "lsh_encself_attention_f16": (False, "pppppp" + "fiiiis"),
     "lsh_encself_attention_i8qkv_f16": (False, "ppfppp" + "fiiiis"),
     "lsh_qkv_attention_i8_f16": (False, "ppppp" + "fff" + "iiiis"),
+    "lsh_qkv_attention_plan": (False, "pp" + "iii" + "s"),
+    "lsh_qkv_attention_plan_in_models": (False, "i"),
+    "lsh_qkv_attention_planned_i8_f16": (False, "pppppp" + "fff" + "iiiis"),
     "lsh_launch_enc_emb_i8I": (True, "ppppp" + "iiiispp" + "ifi"),
     "lsh_launch_scaled_colsum": (True, "ppiifs"),
     "lsh_gemm_i8_i32o": (False, "pppiiis"),

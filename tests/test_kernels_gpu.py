@@ -349,6 +349,52 @@ def test_qkv_projection_and_attention_against_the_oracle(oracle, rng, B, S, h, l
     assert not got[~valid].any(), "rows of padded queries must be zero"
 
 
+@pytest.mark.parametrize("B,S,h,lens", [(32, 128, 12, None), (8, 128, 4, [128, 1, 32, 33, 64, 65, 96, 97]),
+                                        (16, 100, 4, None), (5, 128, 4, [0, 128, 77, 31, 100]),
+                                        (24, 40, 8, None), (3, 128, 2 * 2, [128, 128, 128])])
+def test_planned_qkv_attention_leaves_the_same_bytes(oracle, rng, B, S, h, lens):
+    """With a plan (pairs dealt longest sequence first, blocks of nothing but padding left out)
+    the launch gives the bytes of the unplanned one everywhere -- rows of padded queries are
+    zero on both -- for right-padded sequences of every block count, a sequence of padding only,
+    and a mask with padding in the middle; and the oracle's chain on the valid rows."""
+    d = 64
+    H = h * d
+    x = rng.integers(-127, 128, size=(B * S, H), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(3 * H, H), dtype=np.int8)
+    bias = _randT(rng, (3 * H,), np.float16, 0.3)
+    if lens is None:
+        lens = rng.integers(max(1, S // 4), S + 1, size=B)
+    lens = np.minimum(np.asarray(lens), S)
+    mask = (np.arange(S)[None, :] >= lens[:, None]).astype(np.int32)
+    if B >= 8:
+        mask[3, 5:9] = 1      # padding inside a sequence: masked keys, zeroed queries, blocks kept
+    alpha = 127.0 / (127 * 127 * np.sqrt(H) / 3.0)
+    ds, qs = 1.4 / 127, 127 / 0.9
+    xd, wd, bd, md = to_dev(x), to_dev(w), to_dev(bias), to_dev(mask)
+    want = torch.full((B * S, H), 7, dtype=torch.int8, device=DEV)
+    _k().qkv_attention_i8(xd, wd, bd, md, want, alpha, ds, qs, B, S, h, d)
+    plan = _k().qkv_attention_plan(md, B, S, h)
+    got = torch.full((B * S, H), 9, dtype=torch.int8, device=DEV)
+    _k().qkv_attention_planned_i8(xd, wd, bd, md, plan, got, alpha, ds, qs, B, S, h, d)
+    np.testing.assert_array_equal(to_np(got), to_np(want))
+    # the plan is a permutation of the (sequence, head) pairs with the right block counts
+    p = to_np(plan)
+    pairs = sorted((int(v) & 0xffff, (int(v) >> 16) & 0xfff) for v in p)
+    assert pairs == [(b, hh) for b in range(B) for hh in range(h)]
+    eff = np.array([0 if not (mask[b] == 0).any() else int(np.nonzero(mask[b] == 0)[0][-1]) + 1 for b in range(B)])
+    for v in p:
+        assert (int(v) >> 28) & 7 == (eff[int(v) & 0xffff] + 31) // 32
+    # against the oracle on the rows of valid queries
+    codes = oracle.gemm_i8_i8(x, w, alpha)
+    qkv = oracle.arrange_encself_qkv_i8I(codes, bias, B, S, h, ds)
+    probs = oracle.correlation_softmax_encself(oracle.attn_scores(qkv[0], qkv[1], np.sqrt(1.0 / d)), mask)
+    ref = oracle.arrange_atten_output_i8O(oracle.attn_context(probs, qkv[2]), qs)
+    valid = (mask == 0).reshape(-1)
+    if valid.any():
+        assert_codes_close(to_np(got)[valid], ref[valid], max_frac=5e-3, what="context codes")
+    assert not to_np(got)[~valid].any()
+
+
 def test_qkv_projection_and_attention_in_one_kernel_rejects_other_shapes(rng):
     import lightseq_amd.lib as L
     for B, S, h, d in [(2, 128, 4, 32), (2, 129, 4, 64), (2, 64, 2, 64), (2, 64, 3, 64)]:
