@@ -256,11 +256,15 @@ def gemm_microbench(reps=40):
         c8 = torch.zeros(M, N, dtype=torch.int8, device=dev)
         ops = 2.0 * M * N * Kd
         alpha = clip_in * clip_w / (clip_out * 127)
+        lut = torch.zeros((N, 256), dtype=torch.int8, device=dev)
+        K.build_act_lut(lut, bias, N, clip_out / 127, 127 / clip_act, clip_act, 0)
         cases = {
             "int32 out": lambda: K.gemm_i8_i32o(a, w, c32, M, N, Kd),
             "int8 out (requantising epilogue)": lambda: K.gemm_i8_i8o(a, w, c8, M, N, Kd, alpha),
             "int8 out, bias+GELU+requant fused": lambda: K.gemm_i8_bias_gelu_i8o(
                 a, w, c8, bias, M, N, Kd, alpha, clip_out / 127, 127 / clip_act),
+            "int8 out, bias+GELU+requant fused through the per-column table (what the models run; "
+            "same bytes)": lambda: K.gemm_i8_lut_i8o(a, w, c8, lut, M, N, Kd, alpha),
         }
         res = {}
         for name, fn in cases.items():

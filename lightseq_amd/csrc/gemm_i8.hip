@@ -339,10 +339,37 @@ struct epi_pre<EpiEncdecQF16> {
 // == 0 and the epilogue's alignment holds), so the scalar tail path is not even compiled:
 // a kernel's instructions are fetched cold on every launch, and code that is never run
 // still sits between the lines that are.
+// int32 output keeps a lane's accumulators along the rows (the activation fragment is the first
+// MFMA operand): register k of lane (l32, g) is row 8 (k / 4) + 4 g + k % 4 of column sigma(l32)
+// of its 32 x 32 block, and a store instruction writes two whole 128-byte lines.
+template <typename Epi>
+constexpr bool rows_in_regs = std::is_same<Epi, EpiI32>::value;
+
+template <typename Epi>
+__device__ __forceinline__ v16i mfma_i8_tile(const v4i& w, const v4i& a, const v16i& c) {
+  if constexpr (rows_in_regs<Epi>) return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, w, c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_i32_32x32x32_i8(w, a, c, 0, 0, 0);
+}
+
 template <typename Epi, int MB, int NB, bool FULL = false>
 __device__ __forceinline__ void store_tile_acc(const Epi& epi, const v16i (&acc)[MB][NB], int m0,
                                                int n0, int wm, int wn, int l32, int g, int M, int N,
                                                bool vec_store, long m_off = 0) {
+  if constexpr (rows_in_regs<Epi>) {
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int n = n0 + wn * (NB * 32) + j * 32 + sigma(l32);
+        int32_t* cp = epi.C + n;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          const long m = m0 + wm * (MB * 32) + i * 32 + 8 * (k >> 2) + 4 * g + (k & 3);
+          if (m < M && n < N) cp[(m + m_off) * N] = acc[i][j][k];
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < MB; ++i) {
     const long m = m0 + wm * (MB * 32) + i * 32 + l32;
@@ -527,7 +554,7 @@ gemm_i8_stream_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ W
   auto mma = [&](const Frag& f) {
 #pragma unroll
     for (int i = 0; i < 2; ++i)
-      acc[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w, f.a[i], acc[i][0], 0, 0, 0);
+      acc[i][0] = mfma_i8_tile<Epi>(f.w, f.a[i], acc[i][0]);
   };
 
   if (my_tiles > 0) set_src(0);
@@ -723,8 +750,7 @@ gemm_i8_stream128_kernel(const int8_t* __restrict__ A, const int8_t* __restrict_
         for (int i = 0; i < 2; ++i)
 #pragma unroll
           for (int jj = 0; jj < 2; ++jj)
-            acc[i][jj] =
-                __builtin_amdgcn_mfma_i32_32x32x32_i8(av[ks][jj], bv[ks][i], acc[i][jj], 0, 0, 0);
+            acc[i][jj] = mfma_i8_tile<Epi>(av[ks][jj], bv[ks][i], acc[i][jj]);
       st ^= 1;
     }
     store_tile_acc<Epi, 2, 2, FULL>(epi, acc, tm * kBM, tn * kBN, wm, wn, l32, g, M, N, vec_store,
@@ -860,7 +886,7 @@ gemm_i8_generic_kernel(const int8_t* __restrict__ A, const int8_t* __restrict__ 
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[j], bv[i], acc[i][j], 0, 0, 0);
+          acc[i][j] = mfma_i8_tile<Epi>(av[j], bv[i], acc[i][j]);
     }
     if (kt + 1 < nk) {
       int8_t* nxt = smem + (cur ^ 1) * kStage;

@@ -161,6 +161,10 @@ __device__ __forceinline__ void tile_gemm(const int8_t* __restrict__ A,
                                           const int8_t* __restrict__ W, const Epi& epi, int row0,
                                           int row_end, int N, int K, int tn, int8_t* smem) {
   constexpr bool LUT = std::is_same<Epi, EpiLutI8>::value;
+  // The operand order of the MFMA decides what a lane's 16 accumulators are: weight rows first,
+  // 16 adjacent columns of one output row (one 16-byte store of int8 codes); activations first,
+  // 16 rows of one column -- the layout for int32 output, whose stores then cover whole lines.
+  constexpr bool ROWS_IN_REGS = std::is_same<Epi, EpiI32>::value;
   constexpr int NWV = WGM * WGN;
   constexpr int TM = WGM * MB * 32, TN = WGN * NB * 32;
   constexpr int STAGE = (TM + TN) * kBK;
@@ -246,7 +250,9 @@ __device__ __forceinline__ void tile_gemm(const int8_t* __restrict__ A,
     for (int i = 0; i < MB; ++i)
 #pragma unroll
       for (int j = 0; j < NB; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[j], f.a[i], acc[i][j], 0, 0, 0);
+        acc[i][j] = ROWS_IN_REGS
+                        ? __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a[i], f.w[j], acc[i][j], 0, 0, 0)
+                        : __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[j], f.a[i], acc[i][j], 0, 0, 0);
   };
   // issue order of one slice: an LDS read of the next slice after each of the first MFMAs
   auto pattern = [&]() {
@@ -320,6 +326,24 @@ __device__ __forceinline__ void tile_gemm(const int8_t* __restrict__ A,
   if (LUT) {
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
+  }
+  if constexpr (ROWS_IN_REGS) {
+    // int32 output: a lane holds column sigma(l32) of its block and the rows 8 (k / 4) + 4 g +
+    // k % 4 in register k, so a store instruction writes two whole 128-byte lines (32 lanes, 32
+    // adjacent columns of one row each)
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int n = tn * TN + wn * (NB * 32) + j * 32 + sigma(l32);
+        int32_t* cp = epi.C + n;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+          const long m = (long)row0 + wm * (MB * 32) + i * 32 + 8 * (k >> 2) + 4 * g + (k & 3);
+          if (m < row_end && n < N) cp[m * N] = acc[i][j][k];
+        }
+      }
+    return;
   }
   const int8_t* tab = smem + tab_slot * STAGE;
 #pragma unroll
