@@ -1280,6 +1280,23 @@ void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop) {
   g_ev_stop = stop;
 }
 
+// Compute units of the current device (256 on MI355X), read once per device: the choices below
+// reason in rounds of the chip -- one, two or three resident workgroups per compute unit.
+static int cu_count() {
+  static std::mutex mu;
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  std::lock_guard<std::mutex> lock(mu);
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 static bool stream_ok(int M, int N, int K) {
   if (K % kBK != 0) return false;
   const unsigned long long lim = 0xffffffffull;
@@ -1334,8 +1351,10 @@ static int launch(int grid, int threads, size_t smem, const int8_t* A, const int
 // 4096 x 2304 x 768: 15.8 and 15.3).
 static bool narrow_pays(int M, int N, int K, int ksplit) {
   const long wide_items = (long)((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) * ksplit;
-  const long rounds_wide = (wide_items + 511) / 512, half_rounds_narrow = (2 * wide_items + 511) / 512;
-  return K / ksplit / kBK >= 12 || wide_items < 256 || half_rounds_narrow < 2 * rounds_wide;
+  const long cus = cu_count(), res2 = 2 * cus;  // two resident workgroups per compute unit
+  const long rounds_wide = (wide_items + res2 - 1) / res2,
+             half_rounds_narrow = (2 * wide_items + res2 - 1) / res2;
+  return K / ksplit / kBK >= 12 || wide_items < cus || half_rounds_narrow < 2 * rounds_wide;
 }
 
 // Epilogues that run the 128x128 form of the fast path: every one that reads memory (tables,
@@ -1370,13 +1389,14 @@ struct TileChoice {
 // the persistent kernels.
 static TileChoice choose_tile(int M, int N, int K) {
   TileChoice best{kTileNone, 0, 0};
+  const long cus = cu_count();
   if (K % kBK != 0 || K / kBK < 3 || M < 1024) return best;
   if (N < 1024) {
     // narrow outputs (N = hidden size): 128 x 96 tiles on 4 wavefronts (32 x 96 each) when they
     // give about one tile per compute unit; measured 4096 x 768 x 768 5.8 us against 9.5 us and
     // 4096 x 768 x 3072 (int32 out) 18.3 us against 20.1 us for the persistent kernels
     const long tiles = (long)((M + 127) / 128) * ((N + 95) / 96);
-    if (N % 96 == 0 && tiles >= 192 && tiles <= 256) best = TileChoice{kTile128x96, 128, 96};
+    if (N % 96 == 0 && tiles >= cus * 3 / 4 && tiles <= cus) best = TileChoice{kTile128x96, 128, 96};
     return best;
   }
   const struct {
@@ -1386,10 +1406,10 @@ static TileChoice choose_tile(int M, int N, int K) {
   double best_cost = 0;
   for (const auto& c : cand) {
     const long tiles = (long)((M + c.tm - 1) / c.tm) * ((N + c.tn - 1) / c.tn);
-    if (tiles < 128) continue;
-    const long rounds = (tiles + 255) / 256;
-    const long last = tiles - (rounds - 1) * 256;
-    if (last < 144) continue;
+    if (tiles < cus / 2) continue;
+    const long rounds = (tiles + cus - 1) / cus;
+    const long last = tiles - (rounds - 1) * cus;
+    if (last < cus * 9 / 16) continue;
     // wasted columns / rows of partial tiles count through the padded area
     const double area = (double)c.tm * c.tn;
     const double cost = rounds * area * (1.0 + 48.0 * (c.tm + c.tn) / area);
@@ -1423,6 +1443,7 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   if ((long)tiles_m * tiles_n * ksplit >= (1L << 24))
     return lsh_fail(LSH_ERR_UNSUPPORTED, "int8 gemm: more than 2^24 output tiles");
   const bool full = vec_store && N % 16 == 0;  // no column tail: the lean instantiation
+  const long cus = cu_count();
   if (M <= 64 && K % kBK == 0) {
     const int grid = ((N + 31) / 32) * ksplit;
     if constexpr (std::is_same<Epi, EpiI8>::value || std::is_same<Epi, EpiI32>::value) {
@@ -1432,8 +1453,9 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
 #define LSH_WIDE(MB, NPAIR)                                                                    \
   launch<gemm_i8_skinny16_wide_kernel<Epi, MB, NPAIR>>((N + 32 * NPAIR - 1) / (32 * NPAIR), 256, 0, \
                                                        A, W, epi, M, N, K, kw, 0, vec_store, s)
-        // 128 columns per workgroup up to 32768 columns (<= 256 workgroups), 256 beyond
-        if (N <= 32768) {
+        // 128 columns per workgroup while that is one round of the chip (32768 columns on 256
+        // compute units), 256 beyond
+        if (N <= 128 * cus) {
           if (M <= 16) return LSH_WIDE(1, 4);
           if (M <= 32) return LSH_WIDE(2, 4);
           return LSH_WIDE(4, 4);
@@ -1447,7 +1469,7 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
     if ((K / ksplit) % 256 == 0 && g_skinny16_enabled) {
       // whole 64-byte slices for each of the four wavefronts: the 16 x 16 x 64 form
 #define LSH_SKINNY16(MB, GZ)                                                                    \
-  (full && (long)grid * 2 * (GZ) <= 256                                                          \
+  (full && (long)grid * 2 * (GZ) <= cus                                                          \
        ? launch<gemm_i8_skinny16_kernel<Epi, MB, true, 1>>(((N + 15) / 16), 256, 0, A, W, epi, M, \
                                                            N, K, K / ksplit / 4, 0, vec_store, s, \
                                                            ksplit, ksplit, GZ)                   \
@@ -1464,14 +1486,14 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
       const int blocks = (M + 15) / 16;  // 1 .. 4
       if (blocks == 1) return LSH_SKINNY16(1, 1);
       if (blocks == 2) {
-        if ((long)grid * 2 <= 256) return LSH_SKINNY16(1, 2);
+        if ((long)grid * 2 <= cus) return LSH_SKINNY16(1, 2);
         return LSH_SKINNY16(2, 1);
       }
-      if ((long)grid * blocks <= 256) {
+      if ((long)grid * blocks <= cus) {
         if (blocks == 3) return LSH_SKINNY16(1, 3);
         return LSH_SKINNY16(1, 4);
       }
-      if ((long)grid * 2 <= 256) return LSH_SKINNY16(2, 2);
+      if ((long)grid * 2 <= cus) return LSH_SKINNY16(2, 2);
       return LSH_SKINNY16(4, 1);
 #undef LSH_SKINNY16
     }
@@ -1523,10 +1545,10 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
       const int items = tiles_m * tn64;
       const size_t lds = 2 * kStreamStageBytes + (size_t)kSBN * 256;
       if (full)
-        return launch<gemm_i8_stream_kernel<Epi, true, 2, true>>(items < 512 ? items : 512, 256, lds,
+        return launch<gemm_i8_stream_kernel<Epi, true, 2, true>>(items < 2 * cus ? items : (int)(2 * cus), 256, lds,
                                                                  A, W, epi, M, N, K, tiles_m, tn64,
                                                                  vec_store, s, 1);
-      return launch<gemm_i8_stream_kernel<Epi, false, 2, true>>(items < 512 ? items : 512, 256, lds,
+      return launch<gemm_i8_stream_kernel<Epi, false, 2, true>>(items < 2 * cus ? items : (int)(2 * cus), 256, lds,
                                                                 A, W, epi, M, N, K, tiles_m, tn64,
                                                                 vec_store, s, 1);
     }
@@ -1534,7 +1556,7 @@ static int dispatch(const int8_t* A, const int8_t* W, Epi epi, int M, int N, int
   if (stream) {
     const int items = tiles * ksplit;
     // resident workgroups per compute unit: 2 (64 or 72 KB of LDS each) or 3 (48 KB)
-    const int cap = narrow && !deep ? 768 : 512;
+    const int cap = (int)(narrow && !deep ? 3 * cus : 2 * cus);
     const int grid = items < cap ? items : cap;
     if (!narrow) {
       if (full)
@@ -1611,7 +1633,7 @@ int gemm_i8_preferred_ksplit(int M, int N, int K) {
   // 1024, and the layer norm that sums the planes has half as many to fetch as with eight --
   // measured over whole generation steps: 2 % (GPT-2-medium) and 3 % (Transformer-big) faster
   // than eight planes, two planes 3 % slower than four)
-  while (ks < 4 && items * ks * 2 <= (M <= 64 ? 256 : 512) && nch % (ks * 2) == 0 &&
+  while (ks < 4 && items * ks * 2 <= cu_count() && nch % (ks * 2) == 0 &&
          nch / (ks * 2) >= per_item_min)
     ks *= 2;
   return ks;
