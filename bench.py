@@ -753,6 +753,17 @@ def bench_generation(workload, steps, warmup, graphs=False, with_cpu=True):
     return out
 
 
+def _leave():
+    """Nothing may outlive the command: no helper thread or OpenMP team keeps the interpreter alive.  Under a
+    profiler (rocprofv3 exports ROCP* variables) the process ends the ordinary way instead: the tool writes its
+    files from exit handlers that os._exit would skip."""
+    sys.stdout.flush()
+    sys.stderr.flush()
+    if any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ):
+        return
+    os._exit(0)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -795,14 +806,12 @@ def main():
         torch.cuda.synchronize()
     if args.ffn_segment:
         print(json.dumps(bench_ffn_segment(args)))
-        sys.stdout.flush()
-        os._exit(0)
+        _leave()
+        return
     out = bench_bert(args) if bert else bench_generation(args.workload, args.steps, args.warmup,
                                                          args.graphs, not args.no_cpu_baseline)
     print(json.dumps(out))
-    sys.stdout.flush()
-    # nothing may outlive the command: no helper thread or OpenMP team keeps the interpreter alive
-    os._exit(0)
+    _leave()
 
 
 if __name__ == "__main__":
