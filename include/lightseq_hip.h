@@ -926,6 +926,35 @@ int lsh_gpt_prefill_attention_f16(const void* q_codes, const void* k_codes, cons
                                   float quant_scale, float dequant_scale, int batch_size,
                                   int batch_seq_len, int head_num, int dim_per_head,
                                   lsh_stream_t stream);
+/* The same two stages on int8 codes end to end (no counterpart in the reference; what QuantGpt
+ * runs for heads of 64 and prompts of at most 1024 tokens -- lsh_gpt_prefill_i8_supported):
+ *  - lsh_gpt_arrange_qkv_prefill_i8 = ker_arrange_encself_qkv_i8I_i8O_launcher
+ *    (model/quant_gpt_encoder.cc.cu:489-496) writing the requantised q codes
+ *    [batch, head, seq, d] and the k / v codes straight into the caches
+ *    [batch, head, max_step, d]; nothing is written as fp16.  hidden % 128 == 0, head size 16,
+ *    32, 64 or a multiple of 128;
+ *  - lsh_gpt_prefill_attention_i8 = the q.K^T GEMM on the codes (int32 scores, bit for bit),
+ *    ker_correlation_softmax_gpt_i32I, the P.V GEMM over values half(code / v_quant_scale) (what
+ *    the arrange kernel of the reference stores as dequantised v) and
+ *    ker_arrange_atten_output_i8O (:498-530) in one causal kernel that reads the q codes and
+ *    the caches; ctx_q [batch * seq, hidden] int8; queries at or beyond real_seq_len give
+ *    zeros.  dequant_scale dequantises q and k codes (scores = int32 * attn_scale *
+ *    dequant_scale^2). */
+int lsh_gpt_prefill_i8_supported(int batch_seq_len, int head_num, int dim_per_head);
+/* Process-wide switch: QuantGpt's prompt pass on the int8 codes where the shape is covered
+ * (default) or through the fp16-storage pair above; returns the previous setting.  The two
+ * routes give the same bytes. */
+int lsh_gpt_prefill_on_codes_in_models(int on);
+int lsh_gpt_arrange_qkv_prefill_i8(int batch_token_num, int hidden_size, lsh_stream_t stream,
+                                   const int8_t* ori_qkv, const void* qkv_bias, int8_t* q_codes,
+                                   int8_t* k_cache, int8_t* v_cache, int batch_seq_len,
+                                   int dim_per_head, int head_num, int max_step,
+                                   float dequant_scale, float quant_scale);
+int lsh_gpt_prefill_attention_i8(const int8_t* q_codes, const int8_t* k_cache,
+                                 const int8_t* v_cache, const int* real_seq_len, int8_t* ctx_q,
+                                 float quant_scale, float dequant_scale, float v_quant_scale,
+                                 int batch_size, int batch_seq_len, int head_num, int dim_per_head,
+                                 int max_step, lsh_stream_t stream);
 int lsh_gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size,
                         int max_step, int cur_len, int batch_size, int* unfinished, int eos_id,
                         lsh_stream_t stream);

@@ -7,6 +7,8 @@
 #include "ls_device.cuh"
 #include "ls_launch.h"
 
+#include <type_traits>
+
 namespace lsh {
 
 __device__ __forceinline__ void unpack8(uint2 w, float (&o)[8]) {
@@ -107,6 +109,63 @@ arrange_qkv_kernel(const int8_t* __restrict__ ori, const T* __restrict__ bias,
   }
 }
 
+// The fp16 form for whole sequences: a workgroup owns one 128-byte column group (128 / d heads)
+// of one part (q, k or v) of one sequence and walks its tokens, 32 rows per pass, 16 codes per
+// thread.  What it writes is contiguous per head -- seq_len * d halfs -- instead of one
+// 128-byte piece per head and token scattered over the three tensors, and the bias slice is
+// loaded once.  Same arithmetic per element as the kernel above.
+template <int UNR>
+__global__ void __launch_bounds__(256)
+arrange_qkv_heads_kernel(const int8_t* __restrict__ ori, const __half* __restrict__ bias,
+                         __half* __restrict__ new_qkv, long max_batch_dim, int seq_len, int d,
+                         int head_num, int groups, float ds) {
+  const int hidden = d * head_num;
+  const int grp = blockIdx.x % groups, which = (blockIdx.x / groups) % 3;
+  const int b = blockIdx.x / (groups * 3);
+  const int row = threadIdx.x >> 3, seg = threadIdx.x & 7;
+  const int col = grp * 128 + seg * 16;  // first of this thread's 16 columns inside the part
+  const int head = col / d, dim = col % d;
+  float bv[16];
+  {
+    float lo[8], hi[8];
+    ld8(bias, (long)which * hidden + col, lo);
+    ld8(bias, (long)which * hidden + col + 8, hi);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      bv[k] = lo[k];
+      bv[8 + k] = hi[k];
+    }
+  }
+  const int8_t* src = ori + ((long)b * seq_len * 3 + which) * hidden + col;
+  __half* dst = new_qkv + max_batch_dim * which + ((long)b * head_num + head) * seq_len * d + dim;
+  for (int s0 = row; s0 < seq_len; s0 += 32 * UNR) {
+    uint4 w[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int s = min(s0 + 32 * u, seq_len - 1);
+      w[u] = *reinterpret_cast<const uint4*>(src + (long)s * 3 * hidden);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int s = s0 + 32 * u;
+      if (s >= seq_len) break;
+      const uint32_t wi[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+      float x[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k)
+        x[k] = dequant_add_bias_h(unpack_i8(wi[k >> 2], k & 3), ds, bv[k]);
+      float lo[8], hi[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        lo[k] = x[k];
+        hi[k] = x[8 + k];
+      }
+      st8(dst, (long)s * d, lo);
+      st8(dst, (long)s * d + 8, hi);
+    }
+  }
+}
+
 static int grid_for(long items) {
   long g = (items + 255) / 256;
   const long cap = 256L * 16;
@@ -126,6 +185,22 @@ int arrange_encself_qkv_i8I(int batch_token_num, int hidden_size, hipStream_t s,
   const long total = (long)batch_token_num * 3 * hidden_size;
   const bool vec = dim_per_head % 8 == 0 && max_batch_dim % 8 == 0 && al16(ori_qkv) &&
                    al16(qkv_bias) && al16(new_qkv);
+  if constexpr (std::is_same<T, __half>::value) {
+    const int batch = batch_token_num / batch_seq_len;
+    if (vec && hidden_size % 128 == 0 && dim_per_head % 16 == 0 && 128 % dim_per_head == 0 &&
+        batch_seq_len >= 32 && (long)batch * 3 * (hidden_size / 128) < (1L << 30)) {
+      const int groups = hidden_size / 128;
+      if (batch_seq_len > 64)
+        arrange_qkv_heads_kernel<4><<<batch * 3 * groups, 256, 0, s>>>(
+            ori_qkv, qkv_bias, new_qkv, max_batch_dim, batch_seq_len, dim_per_head, head_num,
+            groups, dequant_scale);
+      else
+        arrange_qkv_heads_kernel<2><<<batch * 3 * groups, 256, 0, s>>>(
+            ori_qkv, qkv_bias, new_qkv, max_batch_dim, batch_seq_len, dim_per_head, head_num,
+            groups, dequant_scale);
+      return lsh_check_launch("arrange_qkv_heads_kernel");
+    }
+  }
   if (vec)
     arrange_qkv_kernel<T, 8, false><<<grid_for(total / 8), 256, 0, s>>>(
         ori_qkv, qkv_bias, new_qkv, nullptr, nullptr, nullptr, nullptr, max_batch_dim, total / 8,

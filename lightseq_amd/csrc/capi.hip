@@ -916,6 +916,28 @@ int lsh_gpt_prefill_attention_f16(const void* q_codes, const void* k_codes, cons
                                    quant_scale, dequant_scale, batch_size, batch_seq_len,
                                    head_num, dim_per_head, HS(stream));
 }
+int lsh_gpt_prefill_on_codes_in_models(int on) { return gpt_prefill_i8_enable(on != 0) ? 1 : 0; }
+int lsh_gpt_prefill_i8_supported(int batch_seq_len, int head_num, int dim_per_head) {
+  return gpt_prefill_i8_supported(batch_seq_len, head_num, dim_per_head) ? 1 : 0;
+}
+int lsh_gpt_arrange_qkv_prefill_i8(int batch_token_num, int hidden_size, lsh_stream_t stream,
+                                   const int8_t* ori_qkv, const void* qkv_bias, int8_t* q_codes,
+                                   int8_t* k_cache, int8_t* v_cache, int batch_seq_len,
+                                   int dim_per_head, int head_num, int max_step,
+                                   float dequant_scale, float quant_scale) {
+  return gpt_arrange_qkv_prefill_i8(batch_token_num, hidden_size, HS(stream), ori_qkv, H(qkv_bias),
+                                    q_codes, k_cache, v_cache, batch_seq_len, dim_per_head,
+                                    head_num, max_step, dequant_scale, quant_scale);
+}
+int lsh_gpt_prefill_attention_i8(const int8_t* q_codes, const int8_t* k_cache,
+                                 const int8_t* v_cache, const int* real_seq_len, int8_t* ctx_q,
+                                 float quant_scale, float dequant_scale, float v_quant_scale,
+                                 int batch_size, int batch_seq_len, int head_num, int dim_per_head,
+                                 int max_step, lsh_stream_t stream) {
+  return gpt_prefill_attention_i8(q_codes, k_cache, v_cache, real_seq_len, ctx_q, quant_scale,
+                                  dequant_scale, v_quant_scale, batch_size, batch_seq_len, head_num,
+                                  dim_per_head, max_step, HS(stream));
+}
 int lsh_gpt_greedy_step(const int8_t* logits, int* ids, int* last_ids, int vocab_size,
                         int max_step, int cur_len, int batch_size, int* unfinished, int eos_id,
                         lsh_stream_t stream) {

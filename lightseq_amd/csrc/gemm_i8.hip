@@ -1282,7 +1282,7 @@ void gemm_i8_time_next_launch(hipEvent_t start, hipEvent_t stop) {
 
 // Compute units of the current device (256 on MI355X), read once per device: the choices below
 // reason in rounds of the chip -- one, two or three resident workgroups per compute unit.
-static int cu_count() {
+int cu_count() {
   static std::mutex mu;
   static int cached[64] = {};
   int dev = 0;

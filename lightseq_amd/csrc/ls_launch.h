@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include <cmath>
+#include <mutex>
 #include <string>
 
 #include "../../include/lightseq_hip.h"
@@ -386,6 +387,22 @@ int gpt_prefill_attention_f16(const __half* q_codes, const __half* k_codes, cons
                               const int* real_seq_len, __half* ctx, int8_t* ctx_q,
                               float quant_scale, float dequant_scale, int batch, int seq_len,
                               int head_num, int dim_per_head, hipStream_t s);
+// the prompt pass on int8 codes end to end (gpt_prefill_kernels.hip): heads of 64, at most 1024
+// tokens for the attention
+bool gpt_prefill_i8_supported(int seq_len, int head_num, int dim_per_head);
+// what QuantGpt's prompt pass does where the shape is covered (default: on); returns the
+// previous setting
+bool gpt_prefill_i8_enable(bool on);
+bool gpt_prefill_i8_enabled();
+int gpt_arrange_qkv_prefill_i8(int batch_token_num, int hidden_size, hipStream_t s,
+                               const int8_t* ori_qkv, const __half* qkv_bias, int8_t* q_codes,
+                               int8_t* k_cache, int8_t* v_cache, int batch_seq_len,
+                               int dim_per_head, int head_num, int max_step, float dequant_scale,
+                               float quant_scale);
+int gpt_prefill_attention_i8(const int8_t* q_codes, const int8_t* k_cache, const int8_t* v_cache,
+                             const int* real_seq_len, int8_t* ctx_q, float quant_scale,
+                             float dequant_scale, float v_quant_scale, int batch, int seq_len,
+                             int head_num, int dim_per_head, int max_step, hipStream_t s);
 template <typename T>
 int correlation_softmax_gpt_i32I(int batch_size, int batch_seq_len, int head_num, hipStream_t s,
                                  const int32_t* correlation, T* output, const int* real_seq_len,
@@ -505,6 +522,9 @@ int layer_cross_attention_f16(const __half* q, const __half* k, const __half* v,
                               hipStream_t s);
 
 // inference/kernels/transformerKernels.h:137-140
+// compute units of the current device, read once per device (gemm_i8.hip)
+int cu_count();
+
 inline float length_norm(int length, float alpha) {
   if (alpha < 0.f) return 1.f / length;
   return std::pow((5.f + length) / 6.f, -alpha);

@@ -176,6 +176,9 @@ void QuantGptEncoder::prompt_pass(const int* ids) {
   __half* qc = _qkv_buf.get();
   __half* kc = qc + _max_batch_dim;
   __half* vd = kc + _max_batch_dim;
+  const bool on_codes =
+      gpt_prefill_i8_enabled() && H % 128 == 0 &&
+      gpt_prefill_i8_supported(_batch_seq_len, _tw._head_num, _tw._dim_per_head);
   for (_layer_id = 0; _layer_id < _tw._n_enc_layer; _layer_id++) {
     const Layer& w = _layers[_layer_id];
     const float* c = &_enc_clip_max[_layer_id * 12];
@@ -183,14 +186,26 @@ void QuantGptEncoder::prompt_pass(const int* ids) {
       LSH_CALL(norm_layer_resual_i8O<__half>(M, H, _stream, _query.get(), a, w.ln1_scale.get(),
                                              w.ln1_bias.get(), w.b_out.get(), Q / c[4], false));
     LSH_CALL(gemm_i8_i8o(a, w.w_qkv.get(), b, M, 3 * H, H, c[0] * c[4] / (c[8] * Q), _stream));
-    LSH_CALL(gpt_arrange_qkv_prefill_f16(
-        M, H, _stream, b, w.b_qkv.get(), qc, kc, vd,
-        _self_k_cache.get() + (size_t)_layer_id * _max_batch_dim,
-        _self_v_cache.get() + (size_t)_layer_id * _max_batch_dim, _batch_seq_len,
-        _tw._dim_per_head, _tw._head_num, _tw._max_step, c[8] / Q, Q / c[11]));
-    LSH_CALL(gpt_prefill_attention_f16(qc, kc, vd, _real_seq_len.get(), nullptr, a, Q / c[5],
-                                       c[11] / Q, _batch_size, _batch_seq_len, _tw._head_num,
-                                       _tw._dim_per_head, _stream));
+    int8_t* k_cache = _self_k_cache.get() + (size_t)_layer_id * _max_batch_dim;
+    int8_t* v_cache = _self_v_cache.get() + (size_t)_layer_id * _max_batch_dim;
+    if (on_codes) {
+      // int8 end to end: q codes and the caches are all the arrange stage writes, and the
+      // attention reads them
+      int8_t* q8 = reinterpret_cast<int8_t*>(qc);
+      LSH_CALL(gpt_arrange_qkv_prefill_i8(M, H, _stream, b, w.b_qkv.get(), q8, k_cache, v_cache,
+                                          _batch_seq_len, _tw._dim_per_head, _tw._head_num,
+                                          _tw._max_step, c[8] / Q, Q / c[11]));
+      LSH_CALL(gpt_prefill_attention_i8(q8, k_cache, v_cache, _real_seq_len.get(), a, Q / c[5],
+                                        c[11] / Q, Q / c[11], _batch_size, _batch_seq_len,
+                                        _tw._head_num, _tw._dim_per_head, _tw._max_step, _stream));
+    } else {
+      LSH_CALL(gpt_arrange_qkv_prefill_f16(M, H, _stream, b, w.b_qkv.get(), qc, kc, vd, k_cache,
+                                           v_cache, _batch_seq_len, _tw._dim_per_head,
+                                           _tw._head_num, _tw._max_step, c[8] / Q, Q / c[11]));
+      LSH_CALL(gpt_prefill_attention_f16(qc, kc, vd, _real_seq_len.get(), nullptr, a, Q / c[5],
+                                         c[11] / Q, _batch_size, _batch_seq_len, _tw._head_num,
+                                         _tw._dim_per_head, _stream));
+    }
     LSH_CALL(gemm_i8_i8o(a, w.w_out.get(), b, M, H, H, c[1] * c[5] / (c[9] * Q), _stream));
     LSH_CALL((residual_bias_ln_i8O<__half, int8_t>(b, w.ln2_scale.get(), w.ln2_bias.get(),
                                                    w.b_ffn2.get(), a, _query.get(), M, H,

@@ -609,6 +609,38 @@ def gpt_prefill_attention(q_codes, k_codes, v, real_seq_len, ctx, ctx_q, quant_s
          dim_per_head, current_stream())
 
 
+def gpt_prefill_i8_supported(batch_seq_len, head_num, dim_per_head):
+    return bool(lib.load().lsh_gpt_prefill_i8_supported(int(batch_seq_len), int(head_num),
+                                                        int(dim_per_head)))
+
+
+def gpt_prefill_on_codes_in_models(on):
+    """Switch QuantGpt's prompt pass between the int8-code kernels (default) and the fp16-storage
+    pair; returns the previous setting."""
+    return bool(lib.load().lsh_gpt_prefill_on_codes_in_models(int(bool(on))))
+
+
+def gpt_arrange_qkv_prefill_i8(batch_token_num, hidden_size, ori_qkv, qkv_bias, q_codes, k_cache,
+                               v_cache, batch_seq_len, dim_per_head, head_num, max_step,
+                               dequant_scale, quant_scale):
+    """ker_arrange_encself_qkv_i8I_i8O of the prompt pass with int8 outputs only: q codes
+    [batch, head, seq, d], k / v codes into the caches [batch, head, max_step, d]."""
+    _dev(ori_qkv, qkv_bias, q_codes, k_cache, v_cache)
+    call("lsh_gpt_arrange_qkv_prefill_i8", batch_token_num, hidden_size, current_stream(),
+         ptr(ori_qkv), ptr(qkv_bias), ptr(q_codes), ptr(k_cache), ptr(v_cache), batch_seq_len,
+         dim_per_head, head_num, max_step, dequant_scale, quant_scale)
+
+
+def gpt_prefill_attention_i8(q_codes, k_cache, v_cache, real_seq_len, ctx_q, quant_scale,
+                             dequant_scale, v_quant_scale, batch_size, batch_seq_len, head_num,
+                             dim_per_head, max_step):
+    """Causal prompt attention of the int8 GPT path on the q codes and the caches."""
+    _dev(q_codes, k_cache, v_cache, real_seq_len, ctx_q)
+    call("lsh_gpt_prefill_attention_i8", ptr(q_codes), ptr(k_cache), ptr(v_cache),
+         ptr(real_seq_len), ptr(ctx_q), quant_scale, dequant_scale, v_quant_scale, batch_size,
+         batch_seq_len, head_num, dim_per_head, max_step, current_stream())
+
+
 def gpt_greedy_step(logits, ids, last_ids, vocab_size, max_step, cur_len, batch_size, unfinished,
                     eos_id):
     _dev(logits, ids, last_ids, unfinished)

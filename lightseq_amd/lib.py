@@ -115,6 +115,10 @@ _SIGNATURES = {
     "lsh_ker_ppl_i8I_workspace": (False, "iis" + "pppp" + "if" + "p"),
     "lsh_gpt_arrange_qkv_prefill_f16": (False, "iis" + "ppppppp" + "iiii" + "ff"),
     "lsh_gpt_prefill_attention_f16": (False, "pppppp" + "ff" + "iiii" + "s"),
+    "lsh_gpt_prefill_i8_supported": (False, "iii"),
+    "lsh_gpt_prefill_on_codes_in_models": (False, "i"),
+    "lsh_gpt_arrange_qkv_prefill_i8": (False, "iis" + "ppppp" + "iiii" + "ff"),
+    "lsh_gpt_prefill_attention_i8": (False, "ppppp" + "fff" + "iiiii" + "s"),
     "lsh_gpt_greedy_step": (False, "ppp" + "iiii" + "p" + "i" + "s"),
     "lsh_gpt_sample_step": (False, "ppp" + "iiii" + "p" + "i" + "iff" + "p" + "s"),
     "lsh_ker_topp_sample_i8I": (False, "iiiis" + "pppp" + "if" + "pp" + "ifi"),

@@ -206,6 +206,78 @@ def test_prefill_attention_fused(oracle, rng, batch, heads, seq, d, max_step):
         assert not to_np(ctx_q).reshape(batch, seq, H)[b, rsl[b]:].any()
 
 
+@pytest.mark.parametrize("batch,heads,seq,max_step", [(2, 2, 9, 16), (2, 16, 130, 160), (1, 4, 64, 64),
+                                                      (3, 2, 200, 256), (2, 4, 512, 640),
+                                                      (1, 2, 1000, 1024), (3, 4, 384, 384)])
+def test_prefill_attention_on_codes(oracle, rng, batch, heads, seq, max_step):
+    """gpt_arrange_qkv_prefill_i8 + gpt_prefill_attention_i8 (int8 codes end to end, what the
+    model runs for heads of 64) == the reference's unfused chain, ragged real lengths included;
+    and the same context codes as the fp16-storage pair."""
+    d = 64
+    H, M, bh = heads * d, batch * seq, batch * heads
+    ori = _codes(rng, (M, 3 * H))
+    bias = (rng.standard_normal(3 * H) * 0.5).astype(np.float16)
+    dq_in, qs_cache = 3.0 / 127, 127 / 3.2
+    rsl = rng.integers(max(1, seq // 2), seq + 1, size=batch).astype(np.int32)
+    rsl[0] = seq
+    q8, k8, v8, dv = oracle.arrange_encself_qkv_i8I_i8O(ori, bias, batch, seq, heads, dq_in, qs_cache)
+    sc = _og().gpt_scores_i8(q8.reshape(bh, seq, d), k8.reshape(bh, seq, d))
+    attn_scale = float(np.float16(np.sqrt(1.0 / d)))
+    pr = _og().correlation_softmax_gpt_i32I(sc, rsl, heads, attn_scale, 1.0 / qs_cache, np.float16)
+    ctx = oracle.attn_context(pr, dv)
+    qs_out = 127 / 1.6
+    want_q = oracle.arrange_atten_output_i8O(ctx.reshape(batch, heads, seq, d), qs_out)
+
+    k = _k()
+    assert k.gpt_prefill_i8_supported(seq, heads, d)
+    assert not k.gpt_prefill_i8_supported(seq, heads, 32)
+    assert not k.gpt_prefill_i8_supported(1025, heads, d)
+    qc = torch.full((batch, heads, seq, d), 7, dtype=torch.int8, device=DEV)
+    kcache = torch.zeros(batch, heads, max_step, d, dtype=torch.int8, device=DEV)
+    vcache = torch.zeros_like(kcache)
+    orid, biasd, rsld = to_dev(ori), to_dev(bias), to_dev(rsl)
+    k.gpt_arrange_qkv_prefill_i8(M, H, orid, biasd, qc, kcache, vcache, seq, d, heads, max_step,
+                                 dq_in, qs_cache)
+    np.testing.assert_array_equal(to_np(qc), q8)
+    np.testing.assert_array_equal(to_np(kcache)[:, :, :seq], k8)
+    np.testing.assert_array_equal(to_np(vcache)[:, :, :seq], v8)
+    assert not to_np(kcache)[:, :, seq:].any() and not to_np(vcache)[:, :, seq:].any()
+
+    ctx_q = torch.full((M, H), 5, dtype=torch.int8, device=DEV)
+    k.gpt_prefill_attention_i8(qc, kcache, vcache, rsld, ctx_q, qs_out, 1.0 / qs_cache, qs_cache,
+                               batch, seq, heads, d, max_step)
+    got = to_np(ctx_q)
+    assert_codes_close(got, want_q.reshape(M, H), max_frac=5e-3, what="gpt ctx_q (codes)")
+    for b in range(batch):  # padded queries give zeros
+        assert not got.reshape(batch, seq, H)[b, rsl[b]:].any()
+
+    # the fp16-storage pair on the same input: same score integers, same rounding points
+    qf = torch.zeros(batch, heads, seq, d, dtype=torch.float16, device=DEV)
+    kf, vf = torch.zeros_like(qf), torch.zeros_like(qf)
+    kc2, vc2 = torch.zeros_like(kcache), torch.zeros_like(vcache)
+    k.gpt_arrange_qkv_prefill(M, H, orid, biasd, qf, kf, vf, kc2, vc2, seq, d, heads, max_step,
+                              dq_in, qs_cache)
+    assert torch.equal(kc2, kcache) and torch.equal(vc2, vcache)
+    ctx_q2 = torch.zeros(M, H, dtype=torch.int8, device=DEV)
+    k.gpt_prefill_attention(qf, kf, vf, rsld, None, ctx_q2, qs_out, 1.0 / qs_cache, batch, seq,
+                            heads, d)
+    assert torch.equal(ctx_q2, ctx_q)
+
+
+def test_prefill_on_codes_rejects_what_it_does_not_cover(rng):
+    k = _k()
+    q = torch.zeros(1, 2, 16, 32, dtype=torch.int8, device=DEV)
+    c = torch.zeros(1, 2, 16, 32, dtype=torch.int8, device=DEV)
+    out = torch.zeros(16, 64, dtype=torch.int8, device=DEV)
+    rsl = torch.full((1,), 16, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="heads of 64"):
+        k.gpt_prefill_attention_i8(q, c, c, rsl, out, 1.0, 1.0, 1.0, 1, 16, 2, 32, 16)
+    ori = torch.zeros(16, 3 * 72, dtype=torch.int8, device=DEV)
+    bias = torch.zeros(3 * 72, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        k.gpt_arrange_qkv_prefill_i8(16, 72, ori, bias, q, c, c, 16, 24, 3, 16, 1.0, 1.0)
+
+
 # --------------------------------------------------------------------------- #
 # model
 # --------------------------------------------------------------------------- #

@@ -151,7 +151,7 @@ def test_bias_gelu(oracle, rng, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape", [(4096, 3072), (1024, 64), (1500, 192), (5000, 1088), (2049, 320), (3000, 1280), (16500, 256), (20000, 64)])
+@pytest.mark.parametrize("shape", [(4096, 3072), (1024, 64), (1500, 192), (5000, 1088), (2049, 320), (3000, 1280), (16500, 256), (20000, 64), (16384, 3072), (40001, 128)])
 def test_bias_gelu_tabulated_equals_evaluated(oracle, rng, dtype, shape):
     """With 1024 rows or more the kernel looks the codes up in per-column tables built in LDS:
     the same bytes as evaluating every element (all 256 input codes occur, -128 included), in
@@ -196,7 +196,8 @@ def test_bias_relu(oracle, rng, dtype, narrow, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("B,S,h,d", [(3, 17, 12, 64), (2, 5, 4, 6), (1, 128, 8, 64)])
+@pytest.mark.parametrize("B,S,h,d", [(3, 17, 12, 64), (2, 5, 4, 6), (1, 128, 8, 64), (3, 128, 12, 64), (2, 50, 8, 32),
+                                     (2, 100, 3, 128), (5, 33, 6, 64), (2, 300, 4, 64)])
 def test_arrange_encself_qkv(oracle, rng, dtype, B, S, h, d):
     H = h * d
     ori = rng.integers(-127, 128, size=(B * S, 3 * H), dtype=np.int8)
