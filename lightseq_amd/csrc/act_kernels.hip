@@ -8,7 +8,7 @@
 // the 256 codes of each column once per workgroup in LDS and to look every element up
 // (bias_act_lut_kernel) than to evaluate the function per element -- the table entries come
 // from the same routine, so the bytes are the same.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
 
 #include <atomic>

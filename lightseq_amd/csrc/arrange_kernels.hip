@@ -4,7 +4,7 @@
 //
 // Replaces inference/kernels/transformerKernels_int8.cc.cu:1080-1393 and
 // inference/kernels/embKernels_int8.cc.cu:13-155.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
 
 #include <type_traits>

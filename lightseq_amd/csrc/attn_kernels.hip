@@ -10,9 +10,9 @@
 // and inference/kernels/transformerKernels.cc.cu:1119-1172.
 #include <type_traits>
 
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
-#include "tile_common.cuh"
+#include "tile_common.h"
 
 namespace lsh {
 

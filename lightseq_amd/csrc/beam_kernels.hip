@@ -12,7 +12,7 @@
 //    sentence's best `beam_size` is among its row's best `beam_size`, and the rough
 //    threshold never cuts into a row's best `beam_size`), without a global sort, a
 //    prefix scan or a device-to-host round trip.  Ties go to the lower candidate id.
-#include "ls_device.cuh"
+#include "ls_device.h"
 
 #include <type_traits>
 #include "ls_launch.h"

@@ -2,7 +2,7 @@
 // dispatch on the storage type.  No kernel code lives here.
 #include <string>
 
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
 
 namespace lsh {

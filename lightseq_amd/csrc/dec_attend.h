@@ -10,7 +10,7 @@
 // (inference/kernels/transformerKernels_int8.cc.cu:1515-1594 with the q.K product of
 // model/quant_decoder.cc.cu:679-685 in front.)
 #pragma once
-#include "ls_device.cuh"
+#include "ls_device.h"
 
 namespace lsh {
 

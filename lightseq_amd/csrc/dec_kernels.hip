@@ -6,8 +6,8 @@
 // rows, not tiling.  A wavefront owns one (row, head) pair in the attention kernels;
 // all cross-lane traffic is wave reductions, and sums run in a fixed order so that a
 // step is reproducible bit for bit.
-#include "dec_attend.cuh"
-#include "ls_device.cuh"
+#include "dec_attend.h"
+#include "ls_device.h"
 #include "ls_launch.h"
 
 namespace lsh {

@@ -20,8 +20,8 @@
 // With the group shape of the stand-alone kernel (NWV = 4) the context codes are the same
 // bytes as the pair's; with one wavefront per row (short caches, many rows) the value sums
 // run in another tree and a code can differ by one next to a rounding boundary.
-#include "dec_attend.cuh"
-#include "ls_device.cuh"
+#include "dec_attend.h"
+#include "ls_device.h"
 #include "ls_launch.h"
 
 #include <atomic>

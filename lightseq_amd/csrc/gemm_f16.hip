@@ -7,7 +7,7 @@
 // wavefront a 64 x 32 slice of it, and the MFMA operands are loaded straight from
 // global memory (one 16-byte row fragment per lane and k-step; rows beyond the
 // matrix are clamped for the loads and masked for the stores).
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
 
 namespace lsh {

@@ -34,10 +34,10 @@
 // that consecutive accumulator registers of a lane run along N, and the W rows fed to
 // the MFMA are permuted (sigma) so that the 16 accumulators of a lane are 16 adjacent
 // columns of C: one 16-byte store for int8 output, two for fp16.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
-#include "tile_common.cuh"
-#include "gemm_tile.cuh"
+#include "tile_common.h"
+#include "gemm_tile.h"
 
 #include <hip/hip_ext.h>
 

@@ -2,8 +2,8 @@
 // run a product as one phase of a longer launch (xcd_ffn_kernels.hip): the plain int32, the
 // requantising and the tabulated epilogue, and the K loop of one large output tile.
 #pragma once
-#include "ls_device.cuh"
-#include "tile_common.cuh"
+#include "ls_device.h"
+#include "tile_common.h"
 
 #include <type_traits>
 

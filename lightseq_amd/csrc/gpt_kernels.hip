@@ -5,7 +5,7 @@
 // The model keeps keys and values in caches of fixed stride [batch, head, max_step, d]
 // and token ids in [batch, max_step]: a generation step appends one column in place,
 // where the reference re-lays out (copies) every cache and the whole id matrix per step.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
 #include "sample_common.h"
 

@@ -22,9 +22,9 @@
 // reference: probability -> fp16, context -> fp16 -> int8; the quotient exp / sum is the
 // correctly rounded one (see encself_attn_kernel).  Workgroups of the last query blocks (most key
 // blocks) are launched first.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
-#include "tile_common.cuh"
+#include "tile_common.h"
 
 #include <atomic>
 #include <mutex>

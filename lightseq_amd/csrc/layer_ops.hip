@@ -7,7 +7,7 @@
 // layer's parameter blob), so no kernel needs a host copy of them.  Row kernels
 // (layer norm, softmax) give one 64-lane wavefront to a row and reduce with cross-lane
 // shuffles.  Dropout ratios must be 0 (inference); the mask outputs are still written.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
 
 namespace lsh {

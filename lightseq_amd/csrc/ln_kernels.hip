@@ -11,9 +11,9 @@
 //  * ln_rows_kernel (any hidden): one wavefront per row, 4 elements per lane per step.
 //
 // Replaces inference/kernels/transformerKernels_int8.cc.cu:149-863.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
-#include "ln_rows8.cuh"
+#include "ln_rows8.h"
 
 #include <hip/hip_ext.h>
 

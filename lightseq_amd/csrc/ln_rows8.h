@@ -4,7 +4,7 @@
 // segment (xcd_ffn_kernels.hip).  Replaces inference/kernels/transformerKernels_int8.cc.cu:
 // 149-863.
 #pragma once
-#include "ls_device.cuh"
+#include "ls_device.h"
 
 namespace lsh {
 

@@ -1,6 +1,6 @@
 #include "quant_gpt_encoder.h"
 
-#include "../ls_device.cuh"
+#include "../ls_device.h"
 
 #include <algorithm>
 

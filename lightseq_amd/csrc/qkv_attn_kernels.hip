@@ -16,9 +16,9 @@
 //     values transposed;
 //  3. the attention of one block of keys (attend_block128), context written as int8 codes.
 // Results are byte-identical to the chain of stand-alone kernels.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
-#include "tile_common.cuh"
+#include "tile_common.h"
 
 #include <hip/hip_ext.h>
 

@@ -4,7 +4,7 @@
 // Replaces inference/kernels/transformerKernels_int8.cc.cu:29-147,
 // inference/model/cublas_helper.cc:502-605 (quantize_weight + layout transform)
 // and inference/kernels/transformerKernels.cc.cu:18-80.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
 
 namespace lsh {

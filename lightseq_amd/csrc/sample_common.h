@@ -6,7 +6,7 @@
 // transformerKernels_int8.cc.cu:1908-2290).
 #pragma once
 
-#include "ls_device.cuh"
+#include "ls_device.h"
 
 namespace lsh {
 

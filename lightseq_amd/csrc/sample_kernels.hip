@@ -23,7 +23,7 @@
 //            (larger maximum, or equal maximum and lower thread).
 // The product and the sum of a logit are rounded separately (no FMA contraction), so that a
 // logit has one value wherever it is formed.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
 #include "sample_common.h"
 

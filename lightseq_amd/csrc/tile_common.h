@@ -3,7 +3,7 @@
 // requantising pack, int8 -> fp16 dequantisation, and the attention of one block of up to
 // 128 keys held in LDS.
 #pragma once
-#include "ls_device.cuh"
+#include "ls_device.h"
 
 namespace lsh {
 

@@ -20,10 +20,10 @@
 //   3. LayerNorm of groups of 16 (8) rows: the int32 rows come into LDS past the vector cache,
 //      then the row routine of the stand-alone kernel runs on them.
 // A wait that gives up (xcd_sync.h) ends the kernel; the host then sees the error word.
-#include "ls_device.cuh"
+#include "ls_device.h"
 #include "ls_launch.h"
-#include "gemm_tile.cuh"
-#include "ln_rows8.cuh"
+#include "gemm_tile.h"
+#include "ln_rows8.h"
 
 #define LSH_XCD_FN __device__ __forceinline__
 #include "xcd_sync.h"
