@@ -151,7 +151,7 @@ def test_bias_gelu(oracle, rng, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape", [(4096, 3072), (1024, 64), (1500, 192), (5000, 1088), (2049, 320), (3000, 1280), (16500, 256), (20000, 64), (16384, 3072), (40001, 128)])
+@pytest.mark.parametrize("shape", [(4096, 3072), (1024, 64), (1500, 192), (5000, 1088), (2049, 320), (3000, 1280), (16500, 256), (20000, 64), (16384, 3072), (40001, 128), (20011, 1024), (16500, 512)])
 def test_bias_gelu_tabulated_equals_evaluated(oracle, rng, dtype, shape):
     """With 1024 rows or more the kernel looks the codes up in per-column tables built in LDS:
     the same bytes as evaluating every element (all 256 input codes occur, -128 included), in
